@@ -1,0 +1,173 @@
+// Device-side building blocks shared by every gfx950 kernel in this library:
+// 128-bit vector I/O for fp32 and bf16 storage, the bf16 rounding rule, and
+// wave64 / workgroup sum reductions built on DPP and ds_swizzle.
+//
+// All arithmetic is fp32 with contraction disabled at compile time
+// (-ffp-contract=off): every multiply and add rounds separately, which is what
+// the numpy CPU kernels of the reference do (backend.py:376-487, 1097-1126).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace agrad {
+
+constexpr int kWave = 64;
+
+typedef uint16_t bf16_t;  // raw bfloat16 storage bits
+
+// fp32 -> bf16, round to nearest even; Inf kept; NaN keeps its high half with
+// the quiet bit forced (reference rule: utils.py:20-27, metal_ops.metal:12010-12041).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    uint32_t rounded = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    uint32_t special = (u >> 16) | ((u & 0x007fffffu) ? 0x0040u : 0u);
+    return ((u & 0x7f800000u) == 0x7f800000u) ? special : rounded;
+}
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) {
+    return __uint_as_float(b << 16);
+}
+
+// ---------------------------------------------------------------------------
+// Vector I/O.  VecIO<T, V> moves V consecutive elements between memory and an
+// fp32 register array.  (float,4) and (bf16,8) are one 128-bit access.
+// ---------------------------------------------------------------------------
+template <typename T, int V> struct VecIO;
+
+template <> struct VecIO<float, 4> {
+    static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+        float4 t = *reinterpret_cast<const float4*>(p);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    }
+    static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
+        float4 t; t.x = v[0]; t.y = v[1]; t.z = v[2]; t.w = v[3];
+        *reinterpret_cast<float4*>(p) = t;
+    }
+};
+
+template <> struct VecIO<float, 1> {
+    static __device__ __forceinline__ void load(const float* p, float (&v)[1]) { v[0] = *p; }
+    static __device__ __forceinline__ void store(float* p, const float (&v)[1]) { *p = v[0]; }
+};
+
+template <> struct VecIO<bf16_t, 8> {
+    static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
+        uint4 t = *reinterpret_cast<const uint4*>(p);
+        uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i]     = __uint_as_float(w[i] << 16);
+            v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    }
+    static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[8]) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            w[i] = f32_to_bf16_bits(v[2 * i]) | (f32_to_bf16_bits(v[2 * i + 1]) << 16);
+        uint4 t; t.x = w[0]; t.y = w[1]; t.z = w[2]; t.w = w[3];
+        *reinterpret_cast<uint4*>(p) = t;
+    }
+};
+
+template <> struct VecIO<bf16_t, 1> {
+    static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[1]) {
+        v[0] = bf16_bits_to_f32(*p);
+    }
+    static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[1]) {
+        *p = (bf16_t)f32_to_bf16_bits(v[0]);
+    }
+};
+
+// Widest vector a dtype supports (16 bytes).
+template <typename T> struct WideVec;
+template <> struct WideVec<float>  { static constexpr int value = 4; };
+template <> struct WideVec<bf16_t> { static constexpr int value = 8; };
+
+// ---------------------------------------------------------------------------
+// Cross-lane sums.  A wave64 is four DPP rows of 16 lanes: quad_perm and the
+// row mirrors fold a row without touching LDS, ds_swizzle folds row pairs, and
+// two readlanes fold the two 32-lane halves into a wave-uniform value.
+// Every lane of the wave must be active when these are called.
+// ---------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
+constexpr int kDppQuadXor1      = 0xB1;   // quad_perm:[1,0,3,2]
+constexpr int kDppQuadXor2      = 0x4E;   // quad_perm:[2,3,0,1]
+constexpr int kDppRowHalfMirror = 0x141;
+constexpr int kDppRowMirror     = 0x140;
+constexpr int kSwizzleXor16     = 0x401F; // bit mode: and 0x1f, or 0, xor 0x10
+
+__device__ __forceinline__ float wave_sum(float v) {
+    v = v + dpp_move<kDppQuadXor1>(v);
+    v = v + dpp_move<kDppQuadXor2>(v);
+    v = v + dpp_move<kDppRowHalfMirror>(v);
+    v = v + dpp_move<kDppRowMirror>(v);
+    v = v + __builtin_bit_cast(
+                float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), kSwizzleXor16));
+    float lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+    float hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+    return lo + hi;
+}
+
+// Two independent sums folded together so their DPP chains interleave.
+__device__ __forceinline__ void wave_sum2(float& a, float& b) {
+    a = a + dpp_move<kDppQuadXor1>(a);       b = b + dpp_move<kDppQuadXor1>(b);
+    a = a + dpp_move<kDppQuadXor2>(a);       b = b + dpp_move<kDppQuadXor2>(b);
+    a = a + dpp_move<kDppRowHalfMirror>(a);  b = b + dpp_move<kDppRowHalfMirror>(b);
+    a = a + dpp_move<kDppRowMirror>(a);      b = b + dpp_move<kDppRowMirror>(b);
+    a = a + __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, a), kSwizzleXor16));
+    b = b + __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, b), kSwizzleXor16));
+    float a0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, a), 0));
+    float a1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, a), 32));
+    float b0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, b), 0));
+    float b1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, b), 32));
+    a = a0 + a1;
+    b = b0 + b1;
+}
+
+// Sum over the TPR threads that share one row.  TPR == 64: pure DPP.  TPR > 64:
+// each wave's total is staged in LDS and every thread adds the staged totals in
+// wave order.  `slot` selects one of a few LDS lines so that consecutive
+// reductions need only one barrier each (a slot is 2*TPR/64 floats; rotate at
+// least two slots).  Callers with TPR > 64 run exactly one row per workgroup, so
+// the barrier is reached by the whole workgroup.
+template <int TPR>
+__device__ __forceinline__ float row_sum(float v, float* lds, int slot) {
+    v = wave_sum(v);
+    if constexpr (TPR > kWave) {
+        constexpr int NW = TPR / kWave;
+        float* line = lds + slot * 2 * NW;
+        if ((threadIdx.x & (kWave - 1)) == 0) line[threadIdx.x / kWave] = v;
+        __syncthreads();
+        float t = line[0];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) t = t + line[w];
+        v = t;
+    }
+    return v;
+}
+
+template <int TPR>
+__device__ __forceinline__ void row_sum2(float& a, float& b, float* lds, int slot) {
+    wave_sum2(a, b);
+    if constexpr (TPR > kWave) {
+        constexpr int NW = TPR / kWave;
+        float* line = lds + slot * 2 * NW;
+        if ((threadIdx.x & (kWave - 1)) == 0) {
+            line[threadIdx.x / kWave] = a;
+            line[NW + threadIdx.x / kWave] = b;
+        }
+        __syncthreads();
+        float ta = line[0], tb = line[NW];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) { ta = ta + line[w]; tb = tb + line[NW + w]; }
+        a = ta; b = tb;
+    }
+}
+
+}  // namespace agrad

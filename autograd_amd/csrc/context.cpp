@@ -1,0 +1,579 @@
+// C ABI of libautograd_hip.so: context, memory, passes, the typed entry points
+// and the name-based dispatcher that plays the role of
+// MetalContext.dispatch_with_args_3d (metal_ext.mm:559-590).
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "launch.hpp"
+
+struct agrad_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipEvent_t ev_start = nullptr, ev_stop = nullptr;
+    int* err_flag = nullptr;               // device word set by kernels that see a bad token id
+    uint64_t total_mem = 0;
+    std::mutex mu;
+    std::map<uint64_t, uint64_t> allocs;   // base address -> bytes
+};
+
+namespace agrad {
+
+static thread_local std::string g_last_error;
+
+int set_error(int code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return code;
+}
+
+int check_hip(hipError_t e, const char* what) {
+    if (e == hipSuccess) return AGRAD_OK;
+    return set_error(AGRAD_EHIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+namespace {
+
+struct DeviceGuard {
+    explicit DeviceGuard(agrad_ctx* c) { (void)hipSetDevice(c->device); }
+};
+
+// Resolve (buffer id, byte offset) to a device address and check that `need`
+// bytes from there lie inside one allocation made through this context.
+int resolve(agrad_ctx* ctx, uint64_t id, uint64_t off, uint64_t need, const char* what, void** out) {
+    if (id == 0) {
+        *out = nullptr;
+        return need == 0 ? AGRAD_OK : set_error(AGRAD_EINVAL, "%s: null buffer", what);
+    }
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    auto it = ctx->allocs.upper_bound(id);
+    if (it == ctx->allocs.begin()) return set_error(AGRAD_EINVAL, "%s: buffer id 0x%llx is not an allocation of this context", what, (unsigned long long)id);
+    --it;
+    const uint64_t base = it->first, size = it->second;
+    if (id < base || id >= base + size)
+        return set_error(AGRAD_EINVAL, "%s: buffer id 0x%llx is not an allocation of this context", what, (unsigned long long)id);
+    const uint64_t begin = (id - base) + off;
+    if (begin > size || need > size - begin)
+        return set_error(AGRAD_EINVAL, "%s: range [%llu, +%llu) outside a %llu-byte buffer", what,
+                         (unsigned long long)begin, (unsigned long long)need, (unsigned long long)size);
+    *out = reinterpret_cast<void*>(id + off);
+    return AGRAD_OK;
+}
+
+int finish_stream(agrad_ctx* ctx) {
+    if (int rc = check_hip(hipStreamSynchronize(ctx->stream), "stream synchronize")) return rc;
+    int flag = 0;
+    if (int rc = check_hip(hipMemcpy(&flag, ctx->err_flag, sizeof(int), hipMemcpyDeviceToHost), "error flag read")) return rc;
+    if (flag != 0) {
+        (void)hipMemset(ctx->err_flag, 0, sizeof(int));
+        return set_error(AGRAD_EINDEX, "token id out of range in an embedding kernel");
+    }
+    return AGRAD_OK;
+}
+
+// ---- name-based dispatch table ------------------------------------------------
+struct Operand {
+    void* p;
+};
+struct Call {
+    agrad_ctx* ctx;
+    const uint64_t* ids;
+    const uint64_t* offs;
+    int nbuf;
+    const uint32_t* a;
+    int nargs;
+};
+typedef int (*Handler)(const Call&);
+struct Entry {
+    const char* name;
+    int nbuf, nargs;
+    const char* signature;
+    Handler fn;
+};
+
+inline uint64_t u64(const uint32_t* a, int lo) { return (uint64_t)a[lo] | ((uint64_t)a[lo + 1] << 32); }
+inline float f32(uint32_t bits) { float f; std::memcpy(&f, &bits, 4); return f; }
+inline bool dtype_ok(uint32_t d) { return d == AGRAD_F32 || d == AGRAD_BF16; }
+
+#define RESOLVE(i, need, var)                                                             \
+    void* var = nullptr;                                                                  \
+    if (int rc_ = resolve(c.ctx, c.ids[i], c.offs[i], (need), #var, &var)) return rc_;
+#define RESOLVE_IF(cond, i, need, var)                                                    \
+    void* var = nullptr;                                                                  \
+    if (cond) { if (int rc_ = resolve(c.ctx, c.ids[i], c.offs[i], (need), #var, &var)) return rc_; }
+#define NEED_DTYPE(d) if (!dtype_ok(d)) return set_error(AGRAD_EINVAL, "unknown dtype %u", (unsigned)(d));
+
+int h_fill(const Call& c) {
+    const uint64_t n = u64(c.a, 1);
+    RESOLVE(0, n * 4, out)
+    return launch_fill(c.ctx->stream, out, c.a[0], 4, n);
+}
+int h_fill2(const Call& c) {
+    const uint32_t itemsize = c.a[1];
+    if (itemsize != 1 && itemsize != 2 && itemsize != 4) return set_error(AGRAD_EINVAL, "fill: itemsize %u", itemsize);
+    const uint64_t n = u64(c.a, 2);
+    RESOLVE(0, n * itemsize, out)
+    return launch_fill(c.ctx->stream, out, c.a[0], (int)itemsize, n);
+}
+int h_copy(const Call& c) {
+    const uint64_t n = u64(c.a, 0);
+    RESOLVE(0, n, src) RESOLVE(1, n, dst)
+    return launch_copy(c.ctx->stream, src, dst, n);
+}
+int h_add_fwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t n = u64(c.a, 1), bytes = n * dtype_size(c.a[0]);
+    RESOLVE(0, bytes, x) RESOLVE(1, bytes, y) RESOLVE(2, bytes, out)
+    return launch_add(c.ctx->stream, c.a[0], x, y, out, n);
+}
+int h_add_bwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t n = u64(c.a, 2), bytes = n * dtype_size(c.a[0]);
+    RESOLVE(0, bytes, src) RESOLVE(1, bytes, dst)
+    return launch_accumulate(c.ctx->stream, c.a[0], src, dst, n, c.a[1]);
+}
+int h_cast_down(const Call& c) {
+    const uint64_t n = u64(c.a, 1);
+    RESOLVE(0, n * 4, src) RESOLVE(1, n * 2, dst)
+    return launch_cast_f32_bf16(c.ctx->stream, src, dst, n, c.a[0] != 0);
+}
+int h_cast_up(const Call& c) {
+    const uint64_t n = u64(c.a, 0);
+    RESOLVE(0, n * 2, src) RESOLVE(1, n * 4, dst)
+    return launch_cast_bf16_f32(c.ctx->stream, src, dst, n);
+}
+
+// buffers x, residual, gamma, beta, h, y | args dtype, rows, C, eps_bits, present
+template <int KIND>
+int h_norm_fwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t rows = c.a[1];
+    const uint32_t C = c.a[2], present = c.a[4];
+    const uint64_t act = rows * C * dtype_size(c.a[0]), par = (uint64_t)C * 4;
+    RESOLVE(0, act, x)
+    RESOLVE_IF(present & 2u, 1, act, res)
+    RESOLVE_IF(present & 4u, 2, par, gamma)
+    RESOLVE_IF(present & 8u, 3, par, beta)
+    RESOLVE_IF(present & 16u, 4, act, h)
+    RESOLVE(5, act, y)
+    return launch_norm_fwd(c.ctx->stream, KIND, c.a[0], x, res, (const float*)gamma, (const float*)beta,
+                           h, y, rows, C, f32(c.a[3]));
+}
+
+// buffers x, dy, gamma, dres, dx, dx2, dgamma, dbeta, workspace
+// args dtype, rows, C, eps_bits, flags, present, ws_bytes lo, hi
+template <int KIND>
+int h_norm_bwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t rows = c.a[1];
+    const uint32_t C = c.a[2], flags = c.a[4], present = c.a[5];
+    const uint64_t ws_bytes = u64(c.a, 6);
+    const uint64_t act = rows * C * dtype_size(c.a[0]), par = (uint64_t)C * 4;
+    RESOLVE(0, act, x) RESOLVE(1, act, dy)
+    RESOLVE_IF(present & 4u, 2, par, gamma)
+    RESOLVE_IF(present & 8u, 3, act, dres)
+    RESOLVE_IF(present & 16u, 4, act, dx)
+    RESOLVE_IF(present & 32u, 5, act, dx2)
+    RESOLVE_IF(present & 64u, 6, par, dgamma)
+    RESOLVE_IF(present & 128u, 7, par, dbeta)
+    RESOLVE_IF(present & 256u, 8, ws_bytes, ws)
+    return launch_norm_bwd(c.ctx->stream, KIND, c.a[0], x, dy, (const float*)gamma, dres, dx, dx2,
+                           (float*)dgamma, (float*)dbeta, ws, ws ? ws_bytes : 0, rows, C, f32(c.a[3]), flags);
+}
+
+// buffers x, y | args dtype, n lo, hi
+template <int WHICH>
+int h_act_fwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t n = u64(c.a, 1), bytes = n * dtype_size(c.a[0]);
+    RESOLVE(0, bytes, x) RESOLVE(1, bytes, y)
+    return WHICH == 0 ? launch_gelu_fwd(c.ctx->stream, c.a[0], x, y, n)
+                      : launch_relu2_fwd(c.ctx->stream, c.a[0], x, y, n);
+}
+// buffers dy, x, dx (the reference's order, backend.py:2951-2955) | args dtype, flags, n lo, hi
+template <int WHICH>
+int h_act_bwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t n = u64(c.a, 2), bytes = n * dtype_size(c.a[0]);
+    RESOLVE(0, bytes, dy) RESOLVE(1, bytes, x) RESOLVE(2, bytes, dx)
+    return WHICH == 0 ? launch_gelu_bwd(c.ctx->stream, c.a[0], x, dy, dx, n, c.a[1])
+                      : launch_relu2_bwd(c.ctx->stream, c.a[0], x, dy, dx, n, c.a[1]);
+}
+// buffers gu, h | args dtype, rows, H
+int h_swiglu_fwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t rows = c.a[1], hb = rows * c.a[2] * dtype_size(c.a[0]);
+    RESOLVE(0, 2 * hb, gu) RESOLVE(1, hb, h)
+    return launch_swiglu_fwd(c.ctx->stream, c.a[0], gu, h, rows, c.a[2]);
+}
+// buffers gu, dh, dgu | args dtype, rows, H, flags
+int h_swiglu_bwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t rows = c.a[1], hb = rows * c.a[2] * dtype_size(c.a[0]);
+    RESOLVE(0, 2 * hb, gu) RESOLVE(1, hb, dh) RESOLVE(2, 2 * hb, dgu)
+    return launch_swiglu_bwd(c.ctx->stream, c.a[0], gu, dh, dgu, rows, c.a[2], c.a[3]);
+}
+// buffers q, k, cos, sin | args dtype, B, T, H, HKV, D, hf_sign, backward, present
+int h_rope(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint32_t B = c.a[1], T = c.a[2], H = c.a[3], HKV = c.a[4], D = c.a[5], present = c.a[8];
+    const uint64_t tok = (uint64_t)B * T, es = dtype_size(c.a[0]);
+    RESOLVE(0, tok * H * D * es, q)
+    RESOLVE_IF(present & 2u, 1, tok * HKV * D * es, k)
+    RESOLVE(2, (uint64_t)T * (D / 2) * 4, cs) RESOLVE(3, (uint64_t)T * (D / 2) * 4, sn)
+    return launch_rope(c.ctx->stream, c.a[0], q, k, (const float*)cs, (const float*)sn, B, T, H, HKV, D,
+                       c.a[6] ? 1 : -1, c.a[7] != 0);
+}
+// buffers ids, W, out | args dtype, N, C, V
+int h_gather_fwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t N = c.a[1], es = dtype_size(c.a[0]);
+    const uint32_t C = c.a[2], V = c.a[3];
+    RESOLVE(0, N * 4, ids) RESOLVE(1, (uint64_t)V * C * es, W) RESOLVE(2, N * C * es, out)
+    return launch_gather_fwd(c.ctx->stream, c.a[0], (const int32_t*)ids, W, nullptr, out, N, 1, C, V, c.ctx->err_flag);
+}
+// buffers ids, W, wpe, out | args dtype, N, T, C, V
+int h_embed_sum_fwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t N = c.a[1], es = dtype_size(c.a[0]);
+    const uint32_t T = c.a[2], C = c.a[3], V = c.a[4];
+    RESOLVE(0, N * 4, ids) RESOLVE(1, (uint64_t)V * C * es, W) RESOLVE(2, (uint64_t)T * C * es, wpe)
+    RESOLVE(3, N * C * es, out)
+    return launch_gather_fwd(c.ctx->stream, c.a[0], (const int32_t*)ids, W, wpe, out, N, T, C, V, c.ctx->err_flag);
+}
+// buffers ids, dY, dW, workspace | args dtype, N, C, V, flags, ws_bytes lo, hi
+int h_gather_bwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t N = c.a[1], es = dtype_size(c.a[0]), ws_bytes = u64(c.a, 5);
+    const uint32_t C = c.a[2], V = c.a[3];
+    RESOLVE(0, N * 4, ids) RESOLVE(1, N * C * es, dY) RESOLVE(2, (uint64_t)V * C * es, dW)
+    RESOLVE(3, ws_bytes, ws)
+    return launch_embedding_bwd(c.ctx->stream, c.a[0], (const int32_t*)ids, dY, dW, ws, ws_bytes, N, C, V,
+                                c.a[4], c.ctx->err_flag);
+}
+// buffers dY, dwpe | args dtype, B, T, C, flags
+int h_pos_grad(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t es = dtype_size(c.a[0]), tc = (uint64_t)c.a[2] * c.a[3] * es;
+    RESOLVE(0, tc * c.a[1], dY) RESOLVE(1, tc, dwpe)
+    return launch_pos_embedding_bwd(c.ctx->stream, c.a[0], dY, dwpe, c.a[1], c.a[2], c.a[3], c.a[4]);
+}
+
+const Entry kTable[] = {
+    {"fill_scalar_kernel", 1, 3, "out | bits, n_lo, n_hi", h_fill},
+    {"fill_scalar_kernel2", 1, 4, "out | bits, itemsize, n_lo, n_hi", h_fill2},
+    {"copy_kernel", 2, 2, "src, dst | nbytes_lo, nbytes_hi", h_copy},
+    {"add_residual_forward", 3, 3, "x, y, out | dtype, n_lo, n_hi", h_add_fwd},
+    {"add_residual_backward", 2, 4, "g, dst | dtype, flags, n_lo, n_hi", h_add_bwd},
+    {"fp32_to_bf16", 2, 3, "src, dst | accumulate, n_lo, n_hi", h_cast_down},
+    {"bf16_to_fp32", 2, 2, "src, dst | n_lo, n_hi", h_cast_up},
+    {"layernorm_forward", 6, 5, "x, residual, gamma, beta, h, y | dtype, rows, C, eps_bits, present_mask", h_norm_fwd<AGRAD_NORM_LAYER>},
+    {"rmsnorm_forward", 6, 5, "x, residual, gamma, beta, h, y | dtype, rows, C, eps_bits, present_mask", h_norm_fwd<AGRAD_NORM_RMS>},
+    {"layernorm_backward_kernel", 9, 8, "x, dy, gamma, dres, dx, dx2, dgamma, dbeta, workspace | dtype, rows, C, eps_bits, flags, present_mask, ws_lo, ws_hi", h_norm_bwd<AGRAD_NORM_LAYER>},
+    {"rmsnorm_backward", 9, 8, "x, dy, gamma, dres, dx, dx2, dgamma, dbeta, workspace | dtype, rows, C, eps_bits, flags, present_mask, ws_lo, ws_hi", h_norm_bwd<AGRAD_NORM_RMS>},
+    {"gelu_forward_kernel", 2, 3, "x, y | dtype, n_lo, n_hi", h_act_fwd<0>},
+    {"gelu_backward_kernel", 3, 4, "dy, x, dx | dtype, flags, n_lo, n_hi", h_act_bwd<0>},
+    {"relu2_forward_kernel", 2, 3, "x, y | dtype, n_lo, n_hi", h_act_fwd<1>},
+    {"relu2_backward_kernel", 3, 4, "dy, x, dx | dtype, flags, n_lo, n_hi", h_act_bwd<1>},
+    {"swiglu_forward_kernel", 2, 3, "gu, h | dtype, rows, H", h_swiglu_fwd},
+    {"swiglu_backward_kernel", 3, 4, "gu, dh, dgu | dtype, rows, H, flags", h_swiglu_bwd},
+    {"rope_qk_inplace", 4, 9, "q, k, cos, sin | dtype, B, T, H, HKV, D, hf_sign, backward, present_mask", h_rope},
+    {"gather_forward_kernel", 3, 4, "ids, W, out | dtype, N, C, V", h_gather_fwd},
+    {"embedding_sum_forward", 4, 5, "ids, W, wpe, out | dtype, N, T, C, V", h_embed_sum_fwd},
+    {"gather_backward_kernel", 4, 7, "ids, dY, dW, workspace | dtype, N, C, V, flags, ws_lo, ws_hi", h_gather_bwd},
+    {"pos_emb_grad", 2, 5, "dY, dwpe | dtype, B, T, C, flags", h_pos_grad},
+};
+constexpr int kTableSize = (int)(sizeof(kTable) / sizeof(kTable[0]));
+
+const Entry* find_entry(const char* name) {
+    if (name == nullptr) return nullptr;
+    for (int i = 0; i < kTableSize; ++i)
+        if (std::strcmp(kTable[i].name, name) == 0) return &kTable[i];
+    return nullptr;
+}
+
+}  // namespace
+}  // namespace agrad
+
+using namespace agrad;
+
+#define CTX_OR_FAIL(ctx) \
+    if ((ctx) == nullptr) return set_error(AGRAD_EINVAL, "null context"); \
+    DeviceGuard guard_(ctx);
+
+extern "C" {
+
+const char* agrad_last_error(void) { return g_last_error.c_str(); }
+
+int agrad_device_count(int* count) {
+    if (count == nullptr) return set_error(AGRAD_EINVAL, "null count");
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess) { *count = 0; return check_hip(e, "hipGetDeviceCount"); }
+    *count = n;
+    return AGRAD_OK;
+}
+
+int agrad_ctx_create(int device, agrad_ctx** out) {
+    if (out == nullptr) return set_error(AGRAD_EINVAL, "null out pointer");
+    *out = nullptr;
+    int n = 0;
+    if (int rc = check_hip(hipGetDeviceCount(&n), "hipGetDeviceCount")) return rc;
+    if (device < 0 || device >= n) return set_error(AGRAD_EINVAL, "device %d out of range (%d visible)", device, n);
+    if (int rc = check_hip(hipSetDevice(device), "hipSetDevice")) return rc;
+    hipDeviceProp_t prop;
+    if (int rc = check_hip(hipGetDeviceProperties(&prop, device), "hipGetDeviceProperties")) return rc;
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return set_error(AGRAD_EHIP, "device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
+    agrad_ctx* c = new agrad_ctx();
+    c->device = device;
+    c->total_mem = prop.totalGlobalMem;
+    hipError_t e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
+    if (e == hipSuccess) e = hipEventCreate(&c->ev_start);
+    if (e == hipSuccess) e = hipEventCreate(&c->ev_stop);
+    if (e == hipSuccess) e = hipMalloc((void**)&c->err_flag, 256);
+    if (e == hipSuccess) e = hipMemset(c->err_flag, 0, 256);
+    if (e != hipSuccess) {
+        agrad_ctx_destroy(c);
+        return check_hip(e, "context setup");
+    }
+    *out = c;
+    return AGRAD_OK;
+}
+
+int agrad_ctx_destroy(agrad_ctx* ctx) {
+    if (ctx == nullptr) return AGRAD_OK;
+    (void)hipSetDevice(ctx->device);
+    if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    for (auto& kv : ctx->allocs) (void)hipFree(reinterpret_cast<void*>(kv.first));
+    if (ctx->err_flag) (void)hipFree(ctx->err_flag);
+    if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
+    if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
+    if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return AGRAD_OK;
+}
+
+int agrad_max_buffer_length(agrad_ctx* ctx, uint64_t* bytes) {
+    CTX_OR_FAIL(ctx)
+    if (bytes == nullptr) return set_error(AGRAD_EINVAL, "null out pointer");
+    *bytes = ctx->total_mem;
+    return AGRAD_OK;
+}
+
+int agrad_alloc(agrad_ctx* ctx, uint64_t bytes, uint64_t* buffer_id) {
+    CTX_OR_FAIL(ctx)
+    if (buffer_id == nullptr) return set_error(AGRAD_EINVAL, "null out pointer");
+    *buffer_id = 0;
+    void* p = nullptr;
+    const uint64_t want = bytes ? bytes : 1;
+    if (int rc = check_hip(hipMalloc(&p, want), "hipMalloc")) return rc;
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    ctx->allocs[reinterpret_cast<uint64_t>(p)] = want;
+    *buffer_id = reinterpret_cast<uint64_t>(p);
+    return AGRAD_OK;
+}
+
+int agrad_free(agrad_ctx* ctx, uint64_t buffer_id) {
+    CTX_OR_FAIL(ctx)
+    {
+        std::lock_guard<std::mutex> lock(ctx->mu);
+        auto it = ctx->allocs.find(buffer_id);
+        if (it == ctx->allocs.end()) return set_error(AGRAD_EINVAL, "free: 0x%llx is not a live buffer id", (unsigned long long)buffer_id);
+        ctx->allocs.erase(it);
+    }
+    if (int rc = check_hip(hipStreamSynchronize(ctx->stream), "stream synchronize")) return rc;
+    return check_hip(hipFree(reinterpret_cast<void*>(buffer_id)), "hipFree");
+}
+
+int agrad_begin_pass(agrad_ctx* ctx) {
+    CTX_OR_FAIL(ctx)
+    return AGRAD_OK;  // kernels are enqueued eagerly on the in-order stream
+}
+
+int agrad_end_pass(agrad_ctx* ctx) {
+    CTX_OR_FAIL(ctx)
+    return finish_stream(ctx);
+}
+
+int agrad_synchronize(agrad_ctx* ctx) {
+    CTX_OR_FAIL(ctx)
+    return finish_stream(ctx);
+}
+
+int agrad_copy_from_host(agrad_ctx* ctx, uint64_t buffer_id, uint64_t offset, const void* src, uint64_t nbytes) {
+    CTX_OR_FAIL(ctx)
+    if (nbytes == 0) return AGRAD_OK;
+    if (src == nullptr) return set_error(AGRAD_EINVAL, "copy_from_host: null source");
+    void* dst = nullptr;
+    if (int rc = resolve(ctx, buffer_id, offset, nbytes, "copy_from_host", &dst)) return rc;
+    if (int rc = check_hip(hipMemcpyAsync(dst, src, nbytes, hipMemcpyHostToDevice, ctx->stream), "hipMemcpyAsync H2D")) return rc;
+    return check_hip(hipStreamSynchronize(ctx->stream), "stream synchronize");
+}
+
+int agrad_copy_to_host(agrad_ctx* ctx, uint64_t buffer_id, uint64_t offset, void* dst, uint64_t nbytes) {
+    CTX_OR_FAIL(ctx)
+    if (nbytes == 0) return AGRAD_OK;
+    if (dst == nullptr) return set_error(AGRAD_EINVAL, "copy_to_host: null destination");
+    void* src = nullptr;
+    if (int rc = resolve(ctx, buffer_id, offset, nbytes, "copy_to_host", &src)) return rc;
+    if (int rc = check_hip(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToHost, ctx->stream), "hipMemcpyAsync D2H")) return rc;
+    return check_hip(hipStreamSynchronize(ctx->stream), "stream synchronize");
+}
+
+int agrad_fill(agrad_ctx* ctx, uint64_t buffer_id, uint64_t offset, uint32_t bits, int itemsize, uint64_t n) {
+    CTX_OR_FAIL(ctx)
+    if (itemsize != 1 && itemsize != 2 && itemsize != 4) return set_error(AGRAD_EINVAL, "fill: itemsize %d not in {1, 2, 4}", itemsize);
+    void* dst = nullptr;
+    if (int rc = resolve(ctx, buffer_id, offset, n * (uint64_t)itemsize, "fill", &dst)) return rc;
+    return launch_fill(ctx->stream, dst, bits, itemsize, n);
+}
+
+int agrad_stream(agrad_ctx* ctx, void** stream) {
+    CTX_OR_FAIL(ctx)
+    if (stream == nullptr) return set_error(AGRAD_EINVAL, "null out pointer");
+    *stream = (void*)ctx->stream;
+    return AGRAD_OK;
+}
+
+int agrad_timer_start(agrad_ctx* ctx) {
+    CTX_OR_FAIL(ctx)
+    return check_hip(hipEventRecord(ctx->ev_start, ctx->stream), "hipEventRecord");
+}
+
+int agrad_timer_stop(agrad_ctx* ctx, float* elapsed_ms) {
+    CTX_OR_FAIL(ctx)
+    if (elapsed_ms == nullptr) return set_error(AGRAD_EINVAL, "null out pointer");
+    if (int rc = check_hip(hipEventRecord(ctx->ev_stop, ctx->stream), "hipEventRecord")) return rc;
+    if (int rc = check_hip(hipEventSynchronize(ctx->ev_stop), "hipEventSynchronize")) return rc;
+    return check_hip(hipEventElapsedTime(elapsed_ms, ctx->ev_start, ctx->ev_stop), "hipEventElapsedTime");
+}
+
+int agrad_dispatch(agrad_ctx* ctx, const char* name, const uint64_t* buffer_ids, const uint64_t* offsets,
+                   int n_buffers, const uint32_t* args, int n_args,
+                   uint64_t gx, uint64_t gy, uint64_t gz, uint64_t tg) {
+    (void)gx; (void)gy; (void)gz; (void)tg;
+    CTX_OR_FAIL(ctx)
+    const Entry* e = find_entry(name);
+    if (e == nullptr) return set_error(AGRAD_ENOKERNEL, "no kernel named '%s'", name ? name : "(null)");
+    if (n_buffers != e->nbuf || n_args != e->nargs)
+        return set_error(AGRAD_EINVAL, "%s expects %d buffers and %d args (%s), got %d and %d", e->name,
+                         e->nbuf, e->nargs, e->signature, n_buffers, n_args);
+    if ((n_buffers > 0 && (buffer_ids == nullptr || offsets == nullptr)) || (n_args > 0 && args == nullptr))
+        return set_error(AGRAD_EINVAL, "%s: null argument list", e->name);
+    Call c{ctx, buffer_ids, offsets, n_buffers, args, n_args};
+    return e->fn(c);
+}
+
+int agrad_kernel_count(void) { return kTableSize; }
+const char* agrad_kernel_name(int index) { return (index >= 0 && index < kTableSize) ? kTable[index].name : nullptr; }
+const char* agrad_kernel_signature(const char* name) {
+    const Entry* e = find_entry(name);
+    return e ? e->signature : nullptr;
+}
+
+// ---- typed entry points --------------------------------------------------------
+
+int agrad_add_forward(agrad_ctx* ctx, int dtype, const void* x, const void* y, void* out, uint64_t n) {
+    CTX_OR_FAIL(ctx)
+    return launch_add(ctx->stream, dtype, x, y, out, n);
+}
+int agrad_grad_accumulate(agrad_ctx* ctx, int dtype, const void* src, void* dst, uint64_t n, uint32_t flags) {
+    CTX_OR_FAIL(ctx)
+    return launch_accumulate(ctx->stream, dtype, src, dst, n, flags);
+}
+int agrad_cast_f32_to_bf16(agrad_ctx* ctx, const void* src, void* dst, uint64_t n, int accumulate) {
+    CTX_OR_FAIL(ctx)
+    return launch_cast_f32_bf16(ctx->stream, src, dst, n, accumulate);
+}
+int agrad_cast_bf16_to_f32(agrad_ctx* ctx, const void* src, void* dst, uint64_t n) {
+    CTX_OR_FAIL(ctx)
+    return launch_cast_bf16_f32(ctx->stream, src, dst, n);
+}
+int agrad_copy(agrad_ctx* ctx, const void* src, void* dst, uint64_t nbytes) {
+    CTX_OR_FAIL(ctx)
+    return launch_copy(ctx->stream, src, dst, nbytes);
+}
+
+int agrad_norm_forward(agrad_ctx* ctx, int kind, int dtype, const void* x, const void* residual,
+                       const float* gamma, const float* beta, void* h_out, void* y,
+                       uint64_t rows, uint32_t C, float eps) {
+    CTX_OR_FAIL(ctx)
+    return launch_norm_fwd(ctx->stream, kind, dtype, x, residual, gamma, beta, h_out, y, rows, C, eps);
+}
+uint64_t agrad_norm_backward_workspace_bytes(uint64_t rows, uint32_t C, int dtype) {
+    return norm_bwd_workspace_bytes(rows, C, dtype);
+}
+int agrad_norm_backward(agrad_ctx* ctx, int kind, int dtype, const void* x, const void* dy,
+                        const float* gamma, const void* dres_in, void* dx, void* dx2,
+                        float* dgamma, float* dbeta, void* workspace, uint64_t workspace_bytes,
+                        uint64_t rows, uint32_t C, float eps, uint32_t flags) {
+    CTX_OR_FAIL(ctx)
+    return launch_norm_bwd(ctx->stream, kind, dtype, x, dy, gamma, dres_in, dx, dx2, dgamma, dbeta,
+                           workspace, workspace_bytes, rows, C, eps, flags);
+}
+
+int agrad_gelu_forward(agrad_ctx* ctx, int dtype, const void* x, void* y, uint64_t n) {
+    CTX_OR_FAIL(ctx)
+    return launch_gelu_fwd(ctx->stream, dtype, x, y, n);
+}
+int agrad_gelu_backward(agrad_ctx* ctx, int dtype, const void* x, const void* dy, void* dx, uint64_t n, uint32_t flags) {
+    CTX_OR_FAIL(ctx)
+    return launch_gelu_bwd(ctx->stream, dtype, x, dy, dx, n, flags);
+}
+int agrad_relu2_forward(agrad_ctx* ctx, int dtype, const void* x, void* y, uint64_t n) {
+    CTX_OR_FAIL(ctx)
+    return launch_relu2_fwd(ctx->stream, dtype, x, y, n);
+}
+int agrad_relu2_backward(agrad_ctx* ctx, int dtype, const void* x, const void* dy, void* dx, uint64_t n, uint32_t flags) {
+    CTX_OR_FAIL(ctx)
+    return launch_relu2_bwd(ctx->stream, dtype, x, dy, dx, n, flags);
+}
+int agrad_swiglu_forward(agrad_ctx* ctx, int dtype, const void* gu, void* h, uint64_t rows, uint32_t H) {
+    CTX_OR_FAIL(ctx)
+    return launch_swiglu_fwd(ctx->stream, dtype, gu, h, rows, H);
+}
+int agrad_swiglu_backward(agrad_ctx* ctx, int dtype, const void* gu, const void* dh, void* dgu,
+                          uint64_t rows, uint32_t H, uint32_t flags) {
+    CTX_OR_FAIL(ctx)
+    return launch_swiglu_bwd(ctx->stream, dtype, gu, dh, dgu, rows, H, flags);
+}
+
+int agrad_rope_qk(agrad_ctx* ctx, int dtype, void* q, void* k, const float* cos_table, const float* sin_table,
+                  uint32_t B, uint32_t T, uint32_t H, uint32_t HKV, uint32_t D, int rope_sign, int backward) {
+    CTX_OR_FAIL(ctx)
+    return launch_rope(ctx->stream, dtype, q, k, cos_table, sin_table, B, T, H, HKV, D, rope_sign, backward);
+}
+
+int agrad_gather_forward(agrad_ctx* ctx, int dtype, const int32_t* ids, const void* W, const void* wpe,
+                         void* out, uint64_t N, uint32_t T, uint32_t C, uint32_t V) {
+    CTX_OR_FAIL(ctx)
+    return launch_gather_fwd(ctx->stream, dtype, ids, W, wpe, out, N, T, C, V, ctx->err_flag);
+}
+uint64_t agrad_embedding_backward_workspace_bytes(uint64_t N, uint32_t C, uint32_t V, int dtype) {
+    return embedding_bwd_workspace_bytes(N, C, V, dtype);
+}
+int agrad_embedding_backward(agrad_ctx* ctx, int dtype, const int32_t* ids, const void* dY, void* dW,
+                             void* workspace, uint64_t workspace_bytes, uint64_t N, uint32_t C,
+                             uint32_t V, uint32_t flags) {
+    CTX_OR_FAIL(ctx)
+    return launch_embedding_bwd(ctx->stream, dtype, ids, dY, dW, workspace, workspace_bytes, N, C, V,
+                                flags, ctx->err_flag);
+}
+int agrad_pos_embedding_backward(agrad_ctx* ctx, int dtype, const void* dY, void* dwpe, uint32_t B,
+                                 uint32_t T, uint32_t C, uint32_t flags) {
+    CTX_OR_FAIL(ctx)
+    return launch_pos_embedding_bwd(ctx->stream, dtype, dY, dwpe, B, T, C, flags);
+}
+
+}  // extern "C"

@@ -1,0 +1,471 @@
+// Token / position embedding: gather forward and the deterministic gradient.
+//
+// Forward  out[n,:] = W[ids[n],:] (+ wpe[n % T,:]) is a row copy with 128-bit
+// accesses (cpu_gather_forward, backend.py:525-529).
+//
+// Backward dW[ids[n],:] += dY[n,:] (np.add.at, backend.py:531-538) is done
+// without float atomics:
+//   1. keys = ids, values = row numbers; stable LSD radix sort by key, so each
+//      token's rows form one run of the sorted order, in ascending row order;
+//   2. the sorted order is cut into chunks of L positions, one workgroup each;
+//      a workgroup sums every run inside its chunk in order (fp32) and stores
+//      it straight to dW when the run lies wholly inside the chunk;
+//   3. a run that crosses a chunk edge leaves fp32 partial rows in a carry
+//      buffer; a second kernel adds the partial rows of such a run in chunk
+//      order and stores the total.
+// Every sum has a fixed order, so the result is run-to-run identical, and runs
+// inside one chunk are bit-identical to the sequential CPU sum.
+#include "common.hpp"
+#include "launch.hpp"
+
+#include <cstring>
+
+#include <rocprim/device/device_radix_sort.hpp>
+
+namespace agrad {
+
+namespace {
+
+constexpr int kGatherBlock = 256;
+constexpr int kBatch = 8;          // rows a thread keeps in flight in the segmented sum
+constexpr uint32_t kMaxChunks = 2048;
+
+inline uint64_t align256(uint64_t v) { return (v + 255) & ~255ull; }
+
+// ---------------------------------------------------------------------------
+// forward
+// ---------------------------------------------------------------------------
+template <typename T, int VEC, int UNROLL>
+__global__ void __launch_bounds__(kGatherBlock)
+gather_fwd_kernel(const int32_t* __restrict__ ids, const T* __restrict__ W, const T* __restrict__ wpe,
+                  T* __restrict__ out, uint32_t total, uint32_t CV, uint32_t C, uint32_t T_len,
+                  uint32_t V, int* err_flag) {
+    const uint32_t first = blockIdx.x * (kGatherBlock * UNROLL) + threadIdx.x;
+    float v[UNROLL][VEC], p[UNROLL][VEC];
+    bool ok[UNROLL];
+    uint64_t dst[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        const uint32_t idx = first + u * kGatherBlock;
+        ok[u] = false;
+        if (idx < total) {
+            const uint32_t row = idx / CV;
+            const uint32_t col = (idx - row * CV) * VEC;
+            const int32_t tok = ids[row];
+            dst[u] = (uint64_t)row * C + col;
+            if (tok >= 0 && (uint32_t)tok < V) {
+                ok[u] = true;
+                VecIO<T, VEC>::load(W + (uint64_t)tok * C + col, v[u]);
+                if (wpe != nullptr) VecIO<T, VEC>::load(wpe + (uint64_t)(row % T_len) * C + col, p[u]);
+            } else if (col == 0) {
+                *err_flag = 1;
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        if (ok[u]) {
+            if (wpe != nullptr) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) v[u][k] = v[u][k] + p[u][k];
+            }
+            VecIO<T, VEC>::store(out + dst[u], v[u]);
+        }
+    }
+}
+
+// Bit-exact variant of the plain gather for bf16 / fp32: moves raw 16-byte
+// words, so NaN payloads and -0.0 survive untouched.
+template <int UNROLL>
+__global__ void __launch_bounds__(kGatherBlock)
+gather_rows16_kernel(const int32_t* __restrict__ ids, const uint4* __restrict__ W,
+                     uint4* __restrict__ out, uint32_t total, uint32_t CV, uint32_t V, int* err_flag) {
+    const uint32_t first = blockIdx.x * (kGatherBlock * UNROLL) + threadIdx.x;
+    uint4 v[UNROLL];
+    bool ok[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        const uint32_t idx = first + u * kGatherBlock;
+        ok[u] = false;
+        if (idx < total) {
+            const uint32_t row = idx / CV;
+            const uint32_t cv = idx - row * CV;
+            const int32_t tok = ids[row];
+            if (tok >= 0 && (uint32_t)tok < V) {
+                ok[u] = true;
+                v[u] = W[(uint64_t)tok * CV + cv];
+            } else if (cv == 0) {
+                *err_flag = 1;
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        const uint32_t idx = first + u * kGatherBlock;
+        if (ok[u]) out[idx] = v[u];
+    }
+}
+
+// scalar raw-bits gather (any C, any alignment)
+template <typename U>
+__global__ void __launch_bounds__(kGatherBlock)
+gather_scalar_kernel(const int32_t* __restrict__ ids, const U* __restrict__ W, const U* __restrict__ wpe,
+                     U* __restrict__ out, uint64_t total, uint32_t C, uint32_t T_len, uint32_t V,
+                     int* err_flag) {
+    const uint64_t idx = (uint64_t)blockIdx.x * kGatherBlock + threadIdx.x;
+    if (idx >= total) return;
+    const uint64_t row = idx / C;
+    const uint32_t col = (uint32_t)(idx - row * C);
+    const int32_t tok = ids[row];
+    if (tok < 0 || (uint32_t)tok >= V) {
+        if (col == 0) *err_flag = 1;
+        return;
+    }
+    if (wpe == nullptr) {
+        out[idx] = W[(uint64_t)tok * C + col];
+    } else {
+        float a[1], b[1];
+        VecIO<U, 1>::load(W + (uint64_t)tok * C + col, a);
+        VecIO<U, 1>::load(wpe + (row % T_len) * C + col, b);
+        a[0] = a[0] + b[0];
+        VecIO<U, 1>::store(out + idx, a);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// backward
+// ---------------------------------------------------------------------------
+// keys[i] = ids[i] (out-of-range ids become the sentinel V and are skipped
+// later), vals[i] = i
+__global__ void __launch_bounds__(256)
+emb_prepare_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ keys,
+                   uint32_t* __restrict__ vals, uint32_t N, uint32_t V, int* err_flag) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= N) return;
+    const int32_t t = ids[i];
+    const bool bad = t < 0 || (uint32_t)t >= V;
+    if (bad) *err_flag = 1;
+    keys[i] = bad ? V : (uint32_t)t;
+    vals[i] = i;
+}
+
+struct ChunkEdges {
+    uint32_t start, end;
+    bool open_left, open_right, single;
+};
+
+__device__ __forceinline__ ChunkEdges chunk_edges(const uint32_t* tok_s, uint32_t chunk, uint32_t L, uint32_t N) {
+    ChunkEdges e;
+    e.start = chunk * L;
+    e.end = e.start + L < N ? e.start + L : N;
+    const uint32_t first_tok = tok_s[e.start];
+    const uint32_t last_tok = tok_s[e.end - 1];
+    e.open_left = e.start > 0 && tok_s[e.start - 1] == first_tok;
+    e.open_right = e.end < N && tok_s[e.end] == last_tok;
+    e.single = first_tok == last_tok;
+    return e;
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void store_grad_row(T* dW, uint64_t off, const float (&acc)[VEC], bool accumulate) {
+    float o[VEC];
+    if (accumulate) {
+        VecIO<T, VEC>::load(dW + off, o);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) o[k] = o[k] + acc[k];
+    } else {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) o[k] = acc[k];
+    }
+    VecIO<T, VEC>::store(dW + off, o);
+}
+
+// One workgroup per chunk of L sorted positions; thread j owns column vectors
+// j, j + blockDim, ...  Control flow depends only on the (uniform) token run
+// structure, so a workgroup never diverges except on the column mask.
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+emb_segment_sum_kernel(const uint32_t* __restrict__ tok_s, const uint32_t* __restrict__ row_s,
+                       const T* __restrict__ dY, T* dW, float* __restrict__ carry_head,
+                       float* __restrict__ carry_tail, uint32_t N, uint32_t C, uint32_t CV,
+                       uint32_t V, uint32_t L, int accumulate) {
+    const ChunkEdges e = chunk_edges(tok_s, blockIdx.x, L, N);
+    for (uint32_t cv = threadIdx.x; cv < CV; cv += blockDim.x) {
+        const uint32_t col = cv * VEC;
+        float acc[VEC];
+        uint32_t cur = tok_s[e.start];
+        bool run_is_first = true;
+        bool have = false;
+        for (uint32_t p0 = e.start; p0 < e.end; p0 += kBatch) {
+            float v[kBatch][VEC];
+            uint32_t tk[kBatch];
+#pragma unroll
+            for (int b = 0; b < kBatch; ++b) {
+                const uint32_t p = p0 + b;
+                if (p < e.end) {
+                    tk[b] = tok_s[p];
+                    VecIO<T, VEC>::load(dY + (uint64_t)row_s[p] * C + col, v[b]);
+                }
+            }
+#pragma unroll
+            for (int b = 0; b < kBatch; ++b) {
+                const uint32_t p = p0 + b;
+                if (p < e.end) {
+                    if (have && tk[b] == cur) {
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + v[b][k];
+                    } else {
+                        if (have && cur < V) {
+                            // the finished run cannot touch the chunk's right edge
+                            if (run_is_first && e.open_left) {
+#pragma unroll
+                                for (int k = 0; k < VEC; ++k)
+                                    carry_head[(uint64_t)blockIdx.x * C + col + k] = acc[k];
+                            } else {
+                                store_grad_row<T, VEC>(dW, (uint64_t)cur * C + col, acc, accumulate != 0);
+                            }
+                        }
+                        if (have) run_is_first = false;
+                        cur = tk[b];
+                        have = true;
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) acc[k] = v[b][k];
+                    }
+                }
+            }
+        }
+        // the last run ends at the chunk's right edge
+        if (have && cur < V) {
+            if (run_is_first && e.open_left) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) carry_head[(uint64_t)blockIdx.x * C + col + k] = acc[k];
+            } else if (e.open_right) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) carry_tail[(uint64_t)blockIdx.x * C + col + k] = acc[k];
+            } else {
+                store_grad_row<T, VEC>(dW, (uint64_t)cur * C + col, acc, accumulate != 0);
+            }
+        }
+    }
+}
+
+// A run that crosses chunk edges starts as the tail partial of its first chunk
+// and continues as head partials of the following chunks.  The workgroup of the
+// first chunk adds them in chunk order and stores the token's row.
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+emb_carry_fix_kernel(const uint32_t* __restrict__ tok_s, T* dW, const float* __restrict__ carry_head,
+                     const float* __restrict__ carry_tail, uint32_t N, uint32_t C, uint32_t CV,
+                     uint32_t V, uint32_t L, uint32_t chunks, int accumulate) {
+    const ChunkEdges e = chunk_edges(tok_s, blockIdx.x, L, N);
+    const bool origin = e.open_right && !(e.single && e.open_left);
+    if (!origin) return;
+    const uint32_t tok = tok_s[e.end - 1];
+    if (tok >= V) return;
+    // number of following chunks the run reaches into
+    uint32_t last = blockIdx.x + 1;
+    while (last < chunks) {
+        const ChunkEdges f = chunk_edges(tok_s, last, L, N);
+        if (!(f.single && f.open_right)) break;
+        ++last;
+    }
+    if (last >= chunks) last = chunks - 1;
+    for (uint32_t cv = threadIdx.x; cv < CV; cv += blockDim.x) {
+        const uint32_t col = cv * VEC;
+        float acc[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc[k] = carry_tail[(uint64_t)blockIdx.x * C + col + k];
+        for (uint32_t c = blockIdx.x + 1; c <= last; ++c) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + carry_head[(uint64_t)c * C + col + k];
+        }
+        store_grad_row<T, VEC>(dW, (uint64_t)tok * C + col, acc, accumulate != 0);
+    }
+}
+
+// dwpe[t, c] (+)= sum_b dY[b, t, c], b ascending
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+pos_grad_kernel(const T* __restrict__ dY, T* dwpe, uint32_t B, uint64_t TCV, uint64_t TC, int accumulate) {
+    const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= TCV) return;
+    const uint64_t off = idx * VEC;
+    float acc[VEC];
+    VecIO<T, VEC>::load(dY + off, acc);
+    for (uint32_t b = 1; b < B; ++b) {
+        float v[VEC];
+        VecIO<T, VEC>::load(dY + (uint64_t)b * TC + off, v);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + v[k];
+    }
+    store_grad_row<T, VEC>(dwpe, off, acc, accumulate != 0);
+}
+
+struct EmbPlan {
+    uint32_t L, chunks;
+    uint64_t off_keys_in, off_keys_out, off_vals_in, off_vals_out, off_temp, temp_bytes, off_head,
+        off_tail, total;
+};
+
+int plan_embedding(uint64_t N, uint32_t C, uint32_t V, EmbPlan* p) {
+    uint32_t per = (uint32_t)((N + (uint64_t)kBatch * kMaxChunks - 1) / ((uint64_t)kBatch * kMaxChunks));
+    if (per == 0) per = 1;
+    p->L = kBatch * per;
+    p->chunks = (uint32_t)((N + p->L - 1) / p->L);
+    size_t temp = 0;
+    uint32_t* nil = nullptr;
+    int bits = 1;
+    while ((1ull << bits) <= V) ++bits;  // keys run up to the sentinel V
+    hipError_t err = rocprim::radix_sort_pairs(nullptr, temp, nil, nil, nil, nil, (size_t)N, 0u,
+                                               (unsigned)bits, (hipStream_t)0, false);
+    if (err != hipSuccess) return check_hip(err, "radix sort temp-size query");
+    uint64_t o = 0;
+    p->off_keys_in = o;  o += align256(N * 4);
+    p->off_keys_out = o; o += align256(N * 4);
+    p->off_vals_in = o;  o += align256(N * 4);
+    p->off_vals_out = o; o += align256(N * 4);
+    p->off_temp = o;     o += align256(temp);
+    p->temp_bytes = temp;
+    p->off_head = o;     o += align256((uint64_t)p->chunks * C * 4);
+    p->off_tail = o;     o += align256((uint64_t)p->chunks * C * 4);
+    p->total = o;
+    return AGRAD_OK;
+}
+
+template <typename T>
+int embedding_bwd_typed(hipStream_t s, const EmbPlan& p, const int32_t* ids, const T* dY, T* dW,
+                        uint8_t* ws, uint32_t N, uint32_t C, uint32_t V, uint32_t flags, int* err_flag) {
+    uint32_t* keys_in = (uint32_t*)(ws + p.off_keys_in);
+    uint32_t* keys_out = (uint32_t*)(ws + p.off_keys_out);
+    uint32_t* vals_in = (uint32_t*)(ws + p.off_vals_in);
+    uint32_t* vals_out = (uint32_t*)(ws + p.off_vals_out);
+    float* head = (float*)(ws + p.off_head);
+    float* tail = (float*)(ws + p.off_tail);
+
+    hipLaunchKernelGGL(emb_prepare_kernel, dim3((N + 255) / 256), dim3(256), 0, s, ids, keys_in, vals_in, N, V, err_flag);
+    int bits = 1;
+    while ((1ull << bits) <= V) ++bits;
+    size_t temp = p.temp_bytes;
+    hipError_t err = rocprim::radix_sort_pairs(ws + p.off_temp, temp, keys_in, keys_out, vals_in, vals_out,
+                                               (size_t)N, 0u, (unsigned)bits, s, false);
+    if (err != hipSuccess) return check_hip(err, "radix sort");
+
+    const int acc = (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0;
+    constexpr int WIDE = WideVec<T>::value;
+    const bool wide = C % WIDE == 0 && aligned16(dY) && aligned16(dW);
+    if (wide) {
+        const uint32_t CV = C / WIDE;
+        uint32_t block = ((CV + 63) / 64) * 64;
+        if (block > 256) block = 256;
+        hipLaunchKernelGGL((emb_segment_sum_kernel<T, WIDE>), dim3(p.chunks), dim3(block), 0, s, keys_out,
+                           vals_out, dY, dW, head, tail, N, C, CV, V, p.L, acc);
+        hipLaunchKernelGGL((emb_carry_fix_kernel<T, WIDE>), dim3(p.chunks), dim3(block), 0, s, keys_out, dW,
+                           head, tail, N, C, CV, V, p.L, p.chunks, acc);
+    } else {
+        uint32_t block = ((C + 63) / 64) * 64;
+        if (block > 256) block = 256;
+        hipLaunchKernelGGL((emb_segment_sum_kernel<T, 1>), dim3(p.chunks), dim3(block), 0, s, keys_out,
+                           vals_out, dY, dW, head, tail, N, C, C, V, p.L, acc);
+        hipLaunchKernelGGL((emb_carry_fix_kernel<T, 1>), dim3(p.chunks), dim3(block), 0, s, keys_out, dW,
+                           head, tail, N, C, C, V, p.L, p.chunks, acc);
+    }
+    return check_hip(hipGetLastError(), "embedding backward launch");
+}
+
+}  // namespace
+
+int launch_gather_fwd(hipStream_t s, int dtype, const int32_t* ids, const void* W, const void* wpe,
+                      void* out, uint64_t N, uint32_t T, uint32_t C, uint32_t V, int* err_flag) {
+    if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "gather: unknown dtype %d", dtype);
+    if (N == 0 || C == 0) return AGRAD_OK;
+    if (ids == nullptr || W == nullptr || out == nullptr) return set_error(AGRAD_EINVAL, "gather: null operand");
+    if (wpe != nullptr && T == 0) return set_error(AGRAD_EINVAL, "gather: position table needs T > 0");
+    if (T == 0) T = 1;
+    const uint32_t esz = dtype_size(dtype);
+    const uint32_t per16 = 16 / esz;
+    const bool wide = C % per16 == 0 && aligned16(W) && aligned16(out) && (!wpe || aligned16(wpe));
+    const uint64_t total_vec = wide ? N * (C / per16) : 0;
+    if (wide && total_vec < 0xffff0000ull) {
+        const uint32_t CV = C / per16;
+        const uint32_t total = (uint32_t)total_vec;
+        constexpr int UNROLL = 4;
+        const uint32_t grid = (total + kGatherBlock * UNROLL - 1) / (kGatherBlock * UNROLL);
+        if (wpe == nullptr) {
+            hipLaunchKernelGGL((gather_rows16_kernel<UNROLL>), dim3(grid), dim3(kGatherBlock), 0, s, ids,
+                               (const uint4*)W, (uint4*)out, total, CV, V, err_flag);
+        } else if (dtype == AGRAD_F32) {
+            hipLaunchKernelGGL((gather_fwd_kernel<float, 4, UNROLL>), dim3(grid), dim3(kGatherBlock), 0, s, ids,
+                               (const float*)W, (const float*)wpe, (float*)out, total, CV, C, T, V, err_flag);
+        } else {
+            hipLaunchKernelGGL((gather_fwd_kernel<bf16_t, 8, 2>), dim3((total + kGatherBlock * 2 - 1) / (kGatherBlock * 2)),
+                               dim3(kGatherBlock), 0, s, ids, (const bf16_t*)W, (const bf16_t*)wpe,
+                               (bf16_t*)out, total, CV, C, T, V, err_flag);
+        }
+    } else {
+        const uint64_t total = N * C;
+        const uint64_t grid = (total + kGatherBlock - 1) / kGatherBlock;
+        if (grid > 0x7fffffffull) return set_error(AGRAD_EINVAL, "gather: output too large");
+        if (dtype == AGRAD_F32)
+            hipLaunchKernelGGL((gather_scalar_kernel<float>), dim3((uint32_t)grid), dim3(kGatherBlock), 0, s, ids,
+                               (const float*)W, (const float*)wpe, (float*)out, total, C, T, V, err_flag);
+        else
+            hipLaunchKernelGGL((gather_scalar_kernel<bf16_t>), dim3((uint32_t)grid), dim3(kGatherBlock), 0, s, ids,
+                               (const bf16_t*)W, (const bf16_t*)wpe, (bf16_t*)out, total, C, T, V, err_flag);
+    }
+    return check_hip(hipGetLastError(), "gather launch");
+}
+
+uint64_t embedding_bwd_workspace_bytes(uint64_t N, uint32_t C, uint32_t V, int dtype) {
+    (void)dtype;
+    if (N == 0 || C == 0) return 0;
+    EmbPlan p;
+    if (plan_embedding(N, C, V, &p) != AGRAD_OK) return 0;
+    return p.total;
+}
+
+int launch_embedding_bwd(hipStream_t s, int dtype, const int32_t* ids, const void* dY, void* dW,
+                         void* workspace, uint64_t workspace_bytes, uint64_t N, uint32_t C,
+                         uint32_t V, uint32_t flags, int* err_flag) {
+    if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "embedding backward: unknown dtype %d", dtype);
+    if (N == 0 || C == 0) return AGRAD_OK;
+    if (ids == nullptr || dY == nullptr || dW == nullptr) return set_error(AGRAD_EINVAL, "embedding backward: null operand");
+    if (N >= 0x7fffffffull) return set_error(AGRAD_EINVAL, "embedding backward: too many rows");
+    if (V == 0 || V >= 0x7fffffffu) return set_error(AGRAD_EINVAL, "embedding backward: bad vocabulary size %u", V);
+    EmbPlan p;
+    if (int rc = plan_embedding(N, C, V, &p)) return rc;
+    if (workspace == nullptr || workspace_bytes < p.total)
+        return set_error(AGRAD_EWORKSPACE, "embedding backward: workspace %llu < %llu bytes",
+                         (unsigned long long)workspace_bytes, (unsigned long long)p.total);
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
+        return set_error(AGRAD_EINVAL, "embedding backward: workspace must be 256-byte aligned");
+    if (dtype == AGRAD_F32)
+        return embedding_bwd_typed<float>(s, p, ids, (const float*)dY, (float*)dW, (uint8_t*)workspace,
+                                          (uint32_t)N, C, V, flags, err_flag);
+    return embedding_bwd_typed<bf16_t>(s, p, ids, (const bf16_t*)dY, (bf16_t*)dW, (uint8_t*)workspace,
+                                       (uint32_t)N, C, V, flags, err_flag);
+}
+
+int launch_pos_embedding_bwd(hipStream_t s, int dtype, const void* dY, void* dwpe, uint32_t B,
+                             uint32_t T, uint32_t C, uint32_t flags) {
+    if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "position grad: unknown dtype %d", dtype);
+    if (B == 0 || T == 0 || C == 0) return AGRAD_OK;
+    if (dY == nullptr || dwpe == nullptr) return set_error(AGRAD_EINVAL, "position grad: null operand");
+    const int acc = (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0;
+    const uint64_t TC = (uint64_t)T * C;
+    const uint32_t per16 = 16 / dtype_size(dtype);
+    const bool wide = TC % per16 == 0 && aligned16(dY) && aligned16(dwpe) &&
+                      ((TC * dtype_size(dtype)) % 16 == 0);
+    const uint64_t n = wide ? TC / per16 : TC;
+    const uint64_t grid = (n + 255) / 256;
+    if (grid > 0x7fffffffull) return set_error(AGRAD_EINVAL, "position grad: table too large");
+    if (dtype == AGRAD_F32) {
+        if (wide) hipLaunchKernelGGL((pos_grad_kernel<float, 4>), dim3((uint32_t)grid), dim3(256), 0, s, (const float*)dY, (float*)dwpe, B, n, TC, acc);
+        else hipLaunchKernelGGL((pos_grad_kernel<float, 1>), dim3((uint32_t)grid), dim3(256), 0, s, (const float*)dY, (float*)dwpe, B, n, TC, acc);
+    } else {
+        if (wide) hipLaunchKernelGGL((pos_grad_kernel<bf16_t, 8>), dim3((uint32_t)grid), dim3(256), 0, s, (const bf16_t*)dY, (bf16_t*)dwpe, B, n, TC, acc);
+        else hipLaunchKernelGGL((pos_grad_kernel<bf16_t, 1>), dim3((uint32_t)grid), dim3(256), 0, s, (const bf16_t*)dY, (bf16_t*)dwpe, B, n, TC, acc);
+    }
+    return check_hip(hipGetLastError(), "position grad launch");
+}
+
+}  // namespace agrad

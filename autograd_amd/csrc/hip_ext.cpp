@@ -1,0 +1,171 @@
+// pybind11 module `hip_ext`: the HIP counterpart of the reference's `metal_ext`
+// (metal_ext.mm:770-796).  HipContext exposes the same method names the Python
+// host layer calls on MetalContext and forwards each one to the C ABI of
+// libautograd_hip.so; no kernel code lives here.
+#include <pybind11/numpy.h>
+#include <pybind11/pybind11.h>
+#include <pybind11/stl.h>
+
+#include <cstring>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../include/autograd_hip.h"
+
+namespace py = pybind11;
+
+namespace {
+
+void raise_for(int rc) {
+    if (rc == AGRAD_OK) return;
+    const std::string msg = agrad_last_error();
+    switch (rc) {
+        case AGRAD_EINDEX: throw py::index_error(msg);
+        case AGRAD_EINVAL: throw py::value_error(msg);
+        case AGRAD_EWORKSPACE: throw py::value_error(msg);
+        default: throw std::runtime_error(msg);
+    }
+}
+
+uint32_t float_bits(float f) {
+    uint32_t u;
+    std::memcpy(&u, &f, 4);
+    return u;
+}
+
+class HipContext {
+public:
+    explicit HipContext(int device = 0) { raise_for(agrad_ctx_create(device, &ctx_)); }
+    ~HipContext() { agrad_ctx_destroy(ctx_); }
+    HipContext(const HipContext&) = delete;
+    HipContext& operator=(const HipContext&) = delete;
+
+    uint64_t max_buffer_length() {
+        uint64_t v = 0;
+        raise_for(agrad_max_buffer_length(ctx_, &v));
+        return v;
+    }
+    uint64_t alloc(uint64_t bytes) {
+        uint64_t id = 0;
+        raise_for(agrad_alloc(ctx_, bytes, &id));
+        return id;
+    }
+    void free(uint64_t id) { raise_for(agrad_free(ctx_, id)); }
+    void begin_pass() { raise_for(agrad_begin_pass(ctx_)); }
+    void end_pass() {
+        py::gil_scoped_release nogil;
+        int rc = agrad_end_pass(ctx_);
+        py::gil_scoped_acquire gil;
+        raise_for(rc);
+    }
+    void synchronize() {
+        py::gil_scoped_release nogil;
+        int rc = agrad_synchronize(ctx_);
+        py::gil_scoped_acquire gil;
+        raise_for(rc);
+    }
+    // GPU time between the two calls, in the spirit of begin/end_pass_profiled
+    // (metal_ext.mm:215-286): returns {"gpu_ms": ...}.
+    void begin_pass_profiled() { raise_for(agrad_timer_start(ctx_)); }
+    py::dict end_pass_profiled() {
+        float ms = 0.0f;
+        raise_for(agrad_timer_stop(ctx_, &ms));
+        raise_for(agrad_end_pass(ctx_));
+        py::dict d;
+        d["gpu_ms"] = ms;
+        return d;
+    }
+
+    void dispatch_with_args_3d(const std::string& name, const std::vector<uint64_t>& ids,
+                               const std::vector<uint64_t>& offs, const std::vector<uint32_t>& args,
+                               uint64_t gx, uint64_t gy, uint64_t gz, uint64_t tg) {
+        if (ids.size() != offs.size()) throw py::value_error("buffer_ids and offsets differ in length");
+        raise_for(agrad_dispatch(ctx_, name.c_str(), ids.data(), offs.data(), (int)ids.size(), args.data(),
+                                 (int)args.size(), gx, gy, gz, tg));
+    }
+
+    void fill_scalar(const std::string& name, const std::vector<uint64_t>& ids,
+                     const std::vector<uint64_t>& offs, float value, uint64_t n) {
+        (void)name;
+        if (ids.size() != 1 || offs.size() != 1) throw py::value_error("fill_scalar takes one buffer");
+        raise_for(agrad_fill(ctx_, ids[0], offs[0], float_bits(value), 4, n));
+    }
+    void fill_scalar2(const std::string& name, const std::vector<uint64_t>& ids,
+                      const std::vector<uint64_t>& offs, uint32_t bits, int itemsize, uint64_t n) {
+        (void)name;
+        if (ids.size() != 1 || offs.size() != 1) throw py::value_error("fill_scalar2 takes one buffer");
+        raise_for(agrad_fill(ctx_, ids[0], offs[0], bits, itemsize, n));
+    }
+
+    // Any C-contiguous array; bytes are copied as they are.
+    void copy_from_host(uint64_t id, uint64_t off, py::array host) {
+        py::array c = py::array::ensure(host, py::array::c_style);
+        if (!c) throw py::value_error("copy_from_host needs an array");
+        raise_for(agrad_copy_from_host(ctx_, id, off, c.data(), (uint64_t)c.nbytes()));
+    }
+    py::array copy_to_host(uint64_t id, uint64_t off, const std::vector<py::ssize_t>& shape,
+                           const std::string& dtype) {
+        py::array out(py::dtype(dtype), shape);
+        raise_for(agrad_copy_to_host(ctx_, id, off, out.mutable_data(), (uint64_t)out.nbytes()));
+        return out;
+    }
+
+    uint64_t norm_backward_workspace_bytes(uint64_t rows, uint32_t C, int dtype) {
+        return agrad_norm_backward_workspace_bytes(rows, C, dtype);
+    }
+    uint64_t embedding_backward_workspace_bytes(uint64_t N, uint32_t C, uint32_t V, int dtype) {
+        return agrad_embedding_backward_workspace_bytes(N, C, V, dtype);
+    }
+    std::vector<std::string> kernel_names() {
+        std::vector<std::string> v;
+        for (int i = 0; i < agrad_kernel_count(); ++i) v.push_back(agrad_kernel_name(i));
+        return v;
+    }
+    py::object kernel_signature(const std::string& name) {
+        const char* s = agrad_kernel_signature(name.c_str());
+        if (s == nullptr) return py::none();
+        return py::str(s);
+    }
+    // agrad_ctx* as an integer, for callers that bind the C ABI with ctypes
+    uint64_t handle() { return reinterpret_cast<uint64_t>(ctx_); }
+
+private:
+    agrad_ctx* ctx_ = nullptr;
+};
+
+}  // namespace
+
+PYBIND11_MODULE(hip_ext, m) {
+    m.doc() = "MI355X (gfx950) native context for the autograd fused layer-op path";
+    m.attr("F32") = (int)AGRAD_F32;
+    m.attr("BF16") = (int)AGRAD_BF16;
+    m.attr("ACC_INPUT_GRAD") = (unsigned)AGRAD_ACC_INPUT_GRAD;
+    m.attr("ACC_PARAM_GRAD") = (unsigned)AGRAD_ACC_PARAM_GRAD;
+    m.def("device_count", [] {
+        int n = 0;
+        agrad_device_count(&n);
+        return n;
+    });
+    py::class_<HipContext>(m, "HipContext")
+        .def(py::init<int>(), py::arg("device") = 0)
+        .def("max_buffer_length", &HipContext::max_buffer_length)
+        .def("alloc", &HipContext::alloc)
+        .def("free", &HipContext::free)
+        .def("begin_pass", &HipContext::begin_pass)
+        .def("end_pass", &HipContext::end_pass)
+        .def("begin_pass_profiled", &HipContext::begin_pass_profiled)
+        .def("end_pass_profiled", &HipContext::end_pass_profiled)
+        .def("dispatch_with_args_3d", &HipContext::dispatch_with_args_3d)
+        .def("fill_scalar", &HipContext::fill_scalar)
+        .def("fill_scalar2", &HipContext::fill_scalar2)
+        .def("copy_from_host", &HipContext::copy_from_host)
+        .def("copy_to_host", &HipContext::copy_to_host, py::arg("buffer_id"), py::arg("offset"),
+             py::arg("shape"), py::arg("dtype") = "float32")
+        .def("norm_backward_workspace_bytes", &HipContext::norm_backward_workspace_bytes)
+        .def("embedding_backward_workspace_bytes", &HipContext::embedding_backward_workspace_bytes)
+        .def("kernel_names", &HipContext::kernel_names)
+        .def("kernel_signature", &HipContext::kernel_signature)
+        .def("handle", &HipContext::handle)
+        .def("synchronize", &HipContext::synchronize);
+}

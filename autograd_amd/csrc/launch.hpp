@@ -1,0 +1,63 @@
+// Host-side launchers, one per op family.  Each validates shapes and alignment,
+// picks the launch geometry, and enqueues on the given stream.  They return an
+// AGRAD_* status and record a message with set_error on failure.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/autograd_hip.h"
+
+namespace agrad {
+
+int set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+int check_hip(hipError_t e, const char* what);
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline uint32_t dtype_size(int dtype) { return dtype == AGRAD_BF16 ? 2u : 4u; }
+
+// Upper bound on the number of row-partials the norm backward keeps per column.
+uint32_t norm_bwd_max_blocks();
+
+// memops.hip
+int launch_fill(hipStream_t s, void* dst, uint32_t bits, int itemsize, uint64_t n);
+int launch_copy(hipStream_t s, const void* src, void* dst, uint64_t nbytes);
+int launch_add(hipStream_t s, int dtype, const void* x, const void* y, void* out, uint64_t n);
+int launch_accumulate(hipStream_t s, int dtype, const void* src, void* dst, uint64_t n, uint32_t flags);
+int launch_cast_f32_bf16(hipStream_t s, const void* src, void* dst, uint64_t n, int accumulate);
+int launch_cast_bf16_f32(hipStream_t s, const void* src, void* dst, uint64_t n);
+
+// norm.hip
+uint64_t norm_bwd_workspace_bytes(uint64_t rows, uint32_t C, int dtype);
+int launch_norm_fwd(hipStream_t s, int kind, int dtype, const void* x, const void* residual,
+                    const float* gamma, const float* beta, void* h_out, void* y,
+                    uint64_t rows, uint32_t C, float eps);
+int launch_norm_bwd(hipStream_t s, int kind, int dtype, const void* x, const void* dy,
+                    const float* gamma, const void* dres_in, void* dx, void* dx2,
+                    float* dgamma, float* dbeta, void* workspace, uint64_t workspace_bytes,
+                    uint64_t rows, uint32_t C, float eps, uint32_t flags);
+
+// activation.hip
+int launch_gelu_fwd(hipStream_t s, int dtype, const void* x, void* y, uint64_t n);
+int launch_gelu_bwd(hipStream_t s, int dtype, const void* x, const void* dy, void* dx, uint64_t n, uint32_t flags);
+int launch_relu2_fwd(hipStream_t s, int dtype, const void* x, void* y, uint64_t n);
+int launch_relu2_bwd(hipStream_t s, int dtype, const void* x, const void* dy, void* dx, uint64_t n, uint32_t flags);
+int launch_swiglu_fwd(hipStream_t s, int dtype, const void* gu, void* h, uint64_t rows, uint32_t H);
+int launch_swiglu_bwd(hipStream_t s, int dtype, const void* gu, const void* dh, void* dgu,
+                      uint64_t rows, uint32_t H, uint32_t flags);
+
+// rope.hip
+int launch_rope(hipStream_t s, int dtype, void* q, void* k, const float* cos_t, const float* sin_t,
+                uint32_t B, uint32_t T, uint32_t H, uint32_t HKV, uint32_t D, int sign, int backward);
+
+// embedding.hip
+int launch_gather_fwd(hipStream_t s, int dtype, const int32_t* ids, const void* W, const void* wpe,
+                      void* out, uint64_t N, uint32_t T, uint32_t C, uint32_t V, int* err_flag);
+uint64_t embedding_bwd_workspace_bytes(uint64_t N, uint32_t C, uint32_t V, int dtype);
+int launch_embedding_bwd(hipStream_t s, int dtype, const int32_t* ids, const void* dY, void* dW,
+                         void* workspace, uint64_t workspace_bytes, uint64_t N, uint32_t C,
+                         uint32_t V, uint32_t flags, int* err_flag);
+int launch_pos_embedding_bwd(hipStream_t s, int dtype, const void* dY, void* dwpe, uint32_t B,
+                             uint32_t T, uint32_t C, uint32_t flags);
+
+}  // namespace agrad

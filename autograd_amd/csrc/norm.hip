@@ -1,0 +1,715 @@
+// LayerNorm / RMSNorm forward and backward for gfx950, with the residual add
+// fused in (forward: h = x + r is normalised and optionally stored; backward:
+// the incoming residual gradient is added to dx in the same pass).
+//
+// Row mapping.  A row of C elements is owned by TPR threads:
+//   TPR = 64   one wavefront per row, four rows per 256-thread workgroup,
+//              cross-lane sums by DPP / ds_swizzle only            (C <= 1024)
+//   TPR = 256  one workgroup per row, wave totals staged through LDS (C <= 4096)
+//   TPR = 1024 same with 16 waves                                   (C <= 16384)
+// Each thread keeps its NV 128-bit vectors of the row in registers, so a row is
+// read from HBM exactly once per pass; the two-pass mean / variance of the
+// reference (backend.py:416-433) runs on registers.
+//
+// Backward keeps per-column partial sums of dgamma / dbeta in registers while a
+// workgroup walks its rows (grid-stride), writes one partial row per workgroup
+// to a workspace, and a second small kernel folds the partial rows in fixed
+// order: no atomics, run-to-run deterministic.
+//
+// Arithmetic order follows the reference CPU kernels: LayerNorm
+// backend.py:416-487, RMSNorm backend.py:1097-1108, 1228-1251, 1737-1745,
+// 1990-2011.  Rows that are unaligned or have C % vector != 0 take a scalar
+// workgroup-per-row kernel with the same arithmetic.
+#include "common.hpp"
+#include "launch.hpp"
+
+#include <cstdlib>
+
+namespace agrad {
+
+namespace {
+
+constexpr int kMaxEPT = 16;  // elements of a row a thread may keep in registers
+
+template <typename T>
+struct NormFwdArgs {
+    const T* x; const T* res; const float* gamma; const float* beta; T* h; T* y;
+    uint64_t rows; uint32_t C; float eps; int kind;
+};
+
+template <typename T>
+struct NormBwdArgs {
+    const T* x; const T* dy; const float* gamma; const T* dres; T* dx; T* dx2;
+    float* pgamma; float* pbeta;
+    uint64_t rows; uint32_t C; float eps; int kind; uint32_t flags;
+};
+
+// gamma / beta are fp32 whatever the activation type: VEC of them is one or two
+// 128-bit loads.
+template <int VEC>
+__device__ __forceinline__ void load_param(const float* p, float (&v)[VEC]) {
+    if constexpr (VEC == 1) {
+        v[0] = p[0];
+    } else {
+#pragma unroll
+        for (int j = 0; j < VEC / 4; ++j) {
+            const float4 t = *reinterpret_cast<const float4*>(p + 4 * j);
+            v[4 * j] = t.x; v[4 * j + 1] = t.y; v[4 * j + 2] = t.z; v[4 * j + 3] = t.w;
+        }
+    }
+}
+
+// Rotating LDS slot for consecutive row reductions (three slots: a slot is
+// rewritten only after two later barriers).
+struct SlotRing {
+    int cur = 0;
+    __device__ __forceinline__ int next() { const int s = cur; cur = cur == 2 ? 0 : cur + 1; return s; }
+};
+
+template <typename T> __device__ __forceinline__ float round_through(float v);
+template <> __device__ __forceinline__ float round_through<float>(float v) { return v; }
+template <> __device__ __forceinline__ float round_through<bf16_t>(float v) {
+    return bf16_bits_to_f32(f32_to_bf16_bits(v));
+}
+
+// ----------------------------------------------------------------------------
+// forward, register-resident row
+// ----------------------------------------------------------------------------
+template <typename T, int VEC, int NV, int TPR>
+__global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
+norm_fwd_kernel(const NormFwdArgs<T> a) {
+    constexpr int BLOCK = TPR > 256 ? TPR : 256;
+    constexpr int RPB = BLOCK / TPR;
+    __shared__ float lds[3 * 2 * (TPR / kWave)];
+
+    const int sub = threadIdx.x / TPR;
+    const int lane = threadIdx.x % TPR;
+    const uint64_t row = (uint64_t)blockIdx.x * RPB + sub;
+    if (row >= a.rows) return;  // whole waves only (TPR is a multiple of 64); RPB == 1 never exits
+    const uint32_t C = a.C;
+    const uint64_t base = row * C;
+
+    float v[NV][VEC];
+    bool on[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
+        on[i] = col < C;
+        if (on[i]) {
+            VecIO<T, VEC>::load(a.x + base + col, v[i]);
+        } else {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) v[i][k] = 0.0f;
+        }
+    }
+    if (a.res != nullptr) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            if (on[i]) {
+                const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
+                float r[VEC];
+                VecIO<T, VEC>::load(a.res + base + col, r);
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) v[i][k] = round_through<T>(v[i][k] + r[k]);
+                if (a.h != nullptr) VecIO<T, VEC>::store(a.h + base + col, v[i]);
+            }
+        }
+    }
+
+    const float fC = (float)C;
+    float scale;  // 1 / sqrt(var + eps)  or  1 / sqrt(mean(x^2) + eps)
+    if (a.kind == AGRAD_NORM_LAYER) {
+        float s = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) s = s + v[i][k];
+        const float mean = row_sum<TPR>(s, lds, 0) / fC;
+        float q = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                const float d = on[i] ? (v[i][k] - mean) : 0.0f;
+                v[i][k] = d;
+                q = q + d * d;
+            }
+        const float var = row_sum<TPR>(q, lds, 1) / fC;
+        scale = 1.0f / sqrtf(var + a.eps);
+    } else {
+        float q = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) q = q + v[i][k] * v[i][k];
+        const float ms = row_sum<TPR>(q, lds, 0) / fC;
+        scale = 1.0f / sqrtf(ms + a.eps);
+    }
+
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        if (on[i]) {
+            const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
+            float o[VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) o[k] = v[i][k] * scale;
+            if (a.gamma != nullptr) {
+                float w[VEC];
+                load_param<VEC>(a.gamma + col, w);
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) o[k] = o[k] * w[k];
+            }
+            if (a.beta != nullptr) {
+                float w[VEC];
+                load_param<VEC>(a.beta + col, w);
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) o[k] = o[k] + w[k];
+            }
+            VecIO<T, VEC>::store(a.y + base + col, o);
+        }
+    }
+}
+
+// ----------------------------------------------------------------------------
+// backward, register-resident row, dgamma / dbeta partials per workgroup
+// ----------------------------------------------------------------------------
+template <typename T, int VEC, int NV, int TPR>
+__global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
+norm_bwd_kernel(const NormBwdArgs<T> a) {
+    constexpr int BLOCK = TPR > 256 ? TPR : 256;
+    constexpr int RPB = BLOCK / TPR;
+    __shared__ float lds[3 * 2 * (TPR / kWave)];
+    extern __shared__ float comb[];  // (RPB - 1) * C floats when RPB > 1
+
+    const int sub = threadIdx.x / TPR;
+    const int lane = threadIdx.x % TPR;
+    const uint32_t C = a.C;
+    const float fC = (float)C;
+    const bool is_ln = a.kind == AGRAD_NORM_LAYER;
+    const bool want_pg = a.pgamma != nullptr;
+    const bool want_pb = a.pbeta != nullptr;
+    const bool acc = (a.flags & AGRAD_ACC_INPUT_GRAD) != 0;
+
+    bool on[NV];
+    float gam[NV][VEC], pg[NV][VEC], pb[NV][VEC];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
+        on[i] = col < C;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            gam[i][k] = 1.0f;
+            pg[i][k] = 0.0f;
+            pb[i][k] = 0.0f;
+        }
+        if (on[i] && a.gamma != nullptr) load_param<VEC>(a.gamma + col, gam[i]);
+    }
+    SlotRing ring;
+
+    for (uint64_t row = (uint64_t)blockIdx.x * RPB + sub; row < a.rows;
+         row += (uint64_t)gridDim.x * RPB) {
+        const uint64_t base = row * C;
+        float xv[NV][VEC], g[NV][VEC];
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
+            if (on[i]) {
+                VecIO<T, VEC>::load(a.x + base + col, xv[i]);
+                VecIO<T, VEC>::load(a.dy + base + col, g[i]);
+            } else {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) { xv[i][k] = 0.0f; g[i][k] = 0.0f; }
+            }
+        }
+
+        // recompute the row statistics; xv becomes x_hat
+        float scale;
+        if (is_ln) {
+            float s = 0.0f;
+#pragma unroll
+            for (int i = 0; i < NV; ++i)
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) s = s + xv[i][k];
+            const float mean = row_sum<TPR>(s, lds, ring.next()) / fC;
+            float q = 0.0f;
+#pragma unroll
+            for (int i = 0; i < NV; ++i)
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    const float d = on[i] ? (xv[i][k] - mean) : 0.0f;
+                    xv[i][k] = d;
+                    q = q + d * d;
+                }
+            const float var = row_sum<TPR>(q, lds, ring.next()) / fC;
+            scale = 1.0f / sqrtf(var + a.eps);
+        } else {
+            float q = 0.0f;
+#pragma unroll
+            for (int i = 0; i < NV; ++i)
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) q = q + xv[i][k] * xv[i][k];
+            const float ms = row_sum<TPR>(q, lds, ring.next()) / fC;
+            scale = 1.0f / sqrtf(ms + a.eps);
+        }
+
+        float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                const float xh = xv[i][k] * scale;
+                xv[i][k] = xh;
+                if (want_pg) pg[i][k] = pg[i][k] + g[i][k] * xh;
+                if (want_pb) pb[i][k] = pb[i][k] + g[i][k];
+                const float dyg = g[i][k] * gam[i][k];
+                g[i][k] = dyg;
+                s1 = s1 + dyg;
+                s2 = s2 + dyg * xh;
+            }
+
+        if (a.dx != nullptr) {
+            float c1 = 0.0f, c2;
+            if (is_ln) {
+                row_sum2<TPR>(s1, s2, lds, ring.next());
+                c1 = (s1 / fC) * scale;
+                c2 = (s2 / fC) * scale;
+            } else {
+                c2 = row_sum<TPR>(s2, lds, ring.next()) / fC;
+            }
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                if (on[i]) {
+                    const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
+                    float t[VEC];
+                    if (is_ln) {
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) {
+                            float u = g[i][k] * scale;
+                            u = u - c1;
+                            t[k] = u - xv[i][k] * c2;
+                        }
+                    } else {
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k)
+                            t[k] = (g[i][k] - xv[i][k] * c2) * scale;
+                    }
+                    if (acc) {
+                        float old[VEC];
+                        VecIO<T, VEC>::load(a.dx + base + col, old);
+                        if (a.dres != nullptr) {
+                            float r[VEC];
+                            VecIO<T, VEC>::load(a.dres + base + col, r);
+#pragma unroll
+                            for (int k = 0; k < VEC; ++k) old[k] = old[k] + r[k];
+                        }
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) t[k] = old[k] + t[k];
+                    } else if (a.dres != nullptr) {
+                        float r[VEC];
+                        VecIO<T, VEC>::load(a.dres + base + col, r);
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) t[k] = r[k] + t[k];
+                    }
+                    VecIO<T, VEC>::store(a.dx + base + col, t);
+                    if (a.dx2 != nullptr) VecIO<T, VEC>::store(a.dx2 + base + col, t);
+                }
+            }
+        }
+    }
+
+    // one partial row per workgroup
+    if (want_pg || want_pb) {
+        if constexpr (RPB > 1) {
+#pragma unroll 1
+            for (int pass = 0; pass < 2; ++pass) {
+                float* out = pass == 0 ? a.pgamma : a.pbeta;
+                if (out == nullptr) continue;  // uniform over the workgroup
+                if (sub > 0) {
+#pragma unroll
+                    for (int i = 0; i < NV; ++i)
+                        if (on[i]) {
+                            const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
+#pragma unroll
+                            for (int k = 0; k < VEC; ++k)
+                                comb[(uint32_t)(sub - 1) * C + col + k] = pass == 0 ? pg[i][k] : pb[i][k];
+                        }
+                }
+                __syncthreads();
+                if (sub == 0) {
+#pragma unroll
+                    for (int i = 0; i < NV; ++i)
+                        if (on[i]) {
+                            const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
+#pragma unroll
+                            for (int k = 0; k < VEC; ++k) {
+                                float t = pass == 0 ? pg[i][k] : pb[i][k];
+                                for (int w = 0; w < RPB - 1; ++w) t = t + comb[(uint32_t)w * C + col + k];
+                                out[(uint64_t)blockIdx.x * C + col + k] = t;
+                            }
+                        }
+                }
+                __syncthreads();
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NV; ++i)
+                if (on[i]) {
+                    const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) {
+                        if (want_pg) a.pgamma[(uint64_t)blockIdx.x * C + col + k] = pg[i][k];
+                        if (want_pb) a.pbeta[(uint64_t)blockIdx.x * C + col + k] = pb[i][k];
+                    }
+                }
+        }
+    }
+}
+
+// out[c] (+)= sum_p partial[p, c], p ascending inside each of 8 interleaved
+// row groups, the 8 group sums added in group order.
+__global__ void __launch_bounds__(256)
+colsum_finalize_kernel(const float* __restrict__ partial, uint32_t P, uint32_t C,
+                       float* __restrict__ out, int accumulate) {
+    __shared__ float tile[8][33];
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+    const uint32_t col = blockIdx.x * 32 + tx;
+    float s = 0.0f;
+    if (col < C)
+        for (uint32_t p = ty; p < P; p += 8) s = s + partial[(uint64_t)p * C + col];
+    tile[ty][tx] = s;
+    __syncthreads();
+    if (ty == 0 && col < C) {
+        float t = tile[0][tx];
+#pragma unroll
+        for (int j = 1; j < 8; ++j) t = t + tile[j][tx];
+        out[col] = accumulate ? (out[col] + t) : t;
+    }
+}
+
+// ----------------------------------------------------------------------------
+// scalar fallbacks: any C, any alignment; one 256-thread workgroup per row,
+// the row is re-read from memory for each pass.
+// ----------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ float ld1(const T* p) { float v[1]; VecIO<T, 1>::load(p, v); return v[0]; }
+template <typename T>
+__device__ __forceinline__ void st1(T* p, float f) { float v[1] = {f}; VecIO<T, 1>::store(p, v); }
+
+template <typename T>
+__device__ __forceinline__ float generic_row_value(const NormFwdArgs<T>& a, uint64_t idx) {
+    float v = ld1(a.x + idx);
+    if (a.res != nullptr) v = round_through<T>(v + ld1(a.res + idx));
+    return v;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) norm_fwd_generic_kernel(const NormFwdArgs<T> a) {
+    __shared__ float lds[3 * 2 * 4];
+    const uint32_t C = a.C;
+    const float fC = (float)C;
+    const uint64_t base = (uint64_t)blockIdx.x * C;
+    float mean = 0.0f, scale;
+    if (a.kind == AGRAD_NORM_LAYER) {
+        float s = 0.0f;
+        for (uint32_t c = threadIdx.x; c < C; c += 256) s = s + generic_row_value(a, base + c);
+        mean = row_sum<256>(s, lds, 0) / fC;
+        float q = 0.0f;
+        for (uint32_t c = threadIdx.x; c < C; c += 256) {
+            const float d = generic_row_value(a, base + c) - mean;
+            q = q + d * d;
+        }
+        scale = 1.0f / sqrtf(row_sum<256>(q, lds, 1) / fC + a.eps);
+    } else {
+        float q = 0.0f;
+        for (uint32_t c = threadIdx.x; c < C; c += 256) {
+            const float v = generic_row_value(a, base + c);
+            q = q + v * v;
+        }
+        scale = 1.0f / sqrtf(row_sum<256>(q, lds, 0) / fC + a.eps);
+    }
+    for (uint32_t c = threadIdx.x; c < C; c += 256) {
+        const float v = generic_row_value(a, base + c);
+        if (a.res != nullptr && a.h != nullptr) st1(a.h + base + c, v);
+        float o = (v - mean) * scale;
+        if (a.gamma != nullptr) o = o * a.gamma[c];
+        if (a.beta != nullptr) o = o + a.beta[c];
+        st1(a.y + base + c, o);
+    }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) norm_bwd_generic_kernel(const NormBwdArgs<T> a) {
+    __shared__ float lds[3 * 2 * 4];
+    const uint32_t C = a.C;
+    const float fC = (float)C;
+    const bool is_ln = a.kind == AGRAD_NORM_LAYER;
+    const bool acc = (a.flags & AGRAD_ACC_INPUT_GRAD) != 0;
+    bool first = true;
+    SlotRing ring;
+    for (uint64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
+        const uint64_t base = row * C;
+        float mean = 0.0f, scale;
+        if (is_ln) {
+            float s = 0.0f;
+            for (uint32_t c = threadIdx.x; c < C; c += 256) s = s + ld1(a.x + base + c);
+            mean = row_sum<256>(s, lds, ring.next()) / fC;
+            float q = 0.0f;
+            for (uint32_t c = threadIdx.x; c < C; c += 256) {
+                const float d = ld1(a.x + base + c) - mean;
+                q = q + d * d;
+            }
+            scale = 1.0f / sqrtf(row_sum<256>(q, lds, ring.next()) / fC + a.eps);
+        } else {
+            float q = 0.0f;
+            for (uint32_t c = threadIdx.x; c < C; c += 256) {
+                const float v = ld1(a.x + base + c);
+                q = q + v * v;
+            }
+            scale = 1.0f / sqrtf(row_sum<256>(q, lds, ring.next()) / fC + a.eps);
+        }
+        float s1 = 0.0f, s2 = 0.0f;
+        for (uint32_t c = threadIdx.x; c < C; c += 256) {
+            const float xh = (ld1(a.x + base + c) - mean) * scale;
+            const float g = ld1(a.dy + base + c);
+            // each thread owns its columns of this workgroup's partial row
+            if (a.pgamma != nullptr) {
+                float* p = a.pgamma + (uint64_t)blockIdx.x * C + c;
+                *p = first ? (g * xh) : (*p + g * xh);
+            }
+            if (a.pbeta != nullptr) {
+                float* p = a.pbeta + (uint64_t)blockIdx.x * C + c;
+                *p = first ? g : (*p + g);
+            }
+            const float dyg = g * (a.gamma != nullptr ? a.gamma[c] : 1.0f);
+            s1 = s1 + dyg;
+            s2 = s2 + dyg * xh;
+        }
+        first = false;
+        if (a.dx != nullptr) {
+            row_sum2<256>(s1, s2, lds, ring.next());
+            const float c1 = (s1 / fC) * scale;
+            const float c2 = is_ln ? (s2 / fC) * scale : (s2 / fC);
+            for (uint32_t c = threadIdx.x; c < C; c += 256) {
+                const float xh = (ld1(a.x + base + c) - mean) * scale;
+                const float dyg = ld1(a.dy + base + c) * (a.gamma != nullptr ? a.gamma[c] : 1.0f);
+                float t;
+                if (is_ln) {
+                    t = dyg * scale;
+                    t = t - c1;
+                    t = t - xh * c2;
+                } else {
+                    t = (dyg - xh * c2) * scale;
+                }
+                if (acc) {
+                    float old = ld1(a.dx + base + c);
+                    if (a.dres != nullptr) old = old + ld1(a.dres + base + c);
+                    t = old + t;
+                } else if (a.dres != nullptr) {
+                    t = ld1(a.dres + base + c) + t;
+                }
+                st1(a.dx + base + c, t);
+                if (a.dx2 != nullptr) st1(a.dx2 + base + c, t);
+            }
+        }
+    }
+}
+
+// ----------------------------------------------------------------------------
+// geometry
+// ----------------------------------------------------------------------------
+struct NormPlan {
+    bool generic;
+    int tpr;  // 64, 256, 1024
+    int nv;   // vectors per thread
+    int rpb;  // rows per workgroup
+};
+
+NormPlan plan_norm(uint32_t C, int dtype, bool aligned) {
+    const int vec = dtype == AGRAD_BF16 ? 8 : 4;
+    NormPlan p{true, 256, 0, 1};
+    if (!aligned || C % vec != 0) return p;
+    const int tprs[3] = {64, 256, 1024};
+    for (int t : tprs) {
+        if (C <= (uint32_t)t * kMaxEPT) {
+            p.generic = false;
+            p.tpr = t;
+            p.nv = (int)((C + (uint32_t)t * vec - 1) / ((uint32_t)t * vec));
+            p.rpb = t == 64 ? 4 : 1;
+            return p;
+        }
+    }
+    return p;
+}
+
+uint32_t bwd_blocks(const NormPlan& p, uint64_t rows) {
+    const uint64_t want = (rows + p.rpb - 1) / p.rpb;
+    const uint64_t cap = norm_bwd_max_blocks();
+    return (uint32_t)(want < cap ? (want ? want : 1) : cap);
+}
+
+template <typename T, int VEC, int TPR>
+int fwd_pick_nv(hipStream_t s, const NormPlan& p, const NormFwdArgs<T>& a) {
+    constexpr int BLOCK = TPR > 256 ? TPR : 256;
+    const uint32_t grid = (uint32_t)((a.rows + p.rpb - 1) / p.rpb);
+    switch (p.nv) {
+#define AGRAD_CASE(N)                                                                  \
+    case N:                                                                            \
+        if constexpr (N * VEC <= kMaxEPT) {                                            \
+            hipLaunchKernelGGL((norm_fwd_kernel<T, VEC, N, TPR>), dim3(grid), dim3(BLOCK), 0, s, a); \
+            return AGRAD_OK;                                                           \
+        }                                                                              \
+        break;
+        AGRAD_CASE(1) AGRAD_CASE(2) AGRAD_CASE(3) AGRAD_CASE(4)
+#undef AGRAD_CASE
+    }
+    return set_error(AGRAD_EINVAL, "norm forward: no kernel for nv=%d", p.nv);
+}
+
+template <typename T, int VEC, int TPR>
+int bwd_pick_nv(hipStream_t s, const NormPlan& p, const NormBwdArgs<T>& a, uint32_t grid) {
+    constexpr int BLOCK = TPR > 256 ? TPR : 256;
+    const size_t dyn = p.rpb > 1 ? (size_t)(p.rpb - 1) * a.C * sizeof(float) : 0;
+    switch (p.nv) {
+#define AGRAD_CASE(N)                                                                  \
+    case N:                                                                            \
+        if constexpr (N * VEC <= kMaxEPT) {                                            \
+            hipLaunchKernelGGL((norm_bwd_kernel<T, VEC, N, TPR>), dim3(grid), dim3(BLOCK), dyn, s, a); \
+            return AGRAD_OK;                                                           \
+        }                                                                              \
+        break;
+        AGRAD_CASE(1) AGRAD_CASE(2) AGRAD_CASE(3) AGRAD_CASE(4)
+#undef AGRAD_CASE
+    }
+    return set_error(AGRAD_EINVAL, "norm backward: no kernel for nv=%d", p.nv);
+}
+
+template <typename T>
+int norm_fwd_typed(hipStream_t s, const NormPlan& p, const NormFwdArgs<T>& a) {
+    constexpr int VEC = WideVec<T>::value;
+    if (p.generic) {
+        hipLaunchKernelGGL((norm_fwd_generic_kernel<T>), dim3((uint32_t)a.rows), dim3(256), 0, s, a);
+        return AGRAD_OK;
+    }
+    switch (p.tpr) {
+        case 64: return fwd_pick_nv<T, VEC, 64>(s, p, a);
+        case 256: return fwd_pick_nv<T, VEC, 256>(s, p, a);
+        default: return fwd_pick_nv<T, VEC, 1024>(s, p, a);
+    }
+}
+
+template <typename T>
+int norm_bwd_typed(hipStream_t s, const NormPlan& p, const NormBwdArgs<T>& a, uint32_t grid) {
+    constexpr int VEC = WideVec<T>::value;
+    if (p.generic) {
+        hipLaunchKernelGGL((norm_bwd_generic_kernel<T>), dim3(grid), dim3(256), 0, s, a);
+        return AGRAD_OK;
+    }
+    switch (p.tpr) {
+        case 64: return bwd_pick_nv<T, VEC, 64>(s, p, a, grid);
+        case 256: return bwd_pick_nv<T, VEC, 256>(s, p, a, grid);
+        default: return bwd_pick_nv<T, VEC, 1024>(s, p, a, grid);
+    }
+}
+
+}  // namespace
+
+uint32_t norm_bwd_max_blocks() {
+    static const uint32_t value = [] {
+        const char* e = std::getenv("AGRAD_NORM_BWD_BLOCKS");
+        long v = e ? std::atol(e) : 0;
+        return (uint32_t)(v > 0 && v <= 65536 ? v : 1024);
+    }();
+    return value;
+}
+
+uint64_t norm_bwd_workspace_bytes(uint64_t rows, uint32_t C, int dtype) {
+    // sized for the larger of the vector and the scalar geometry
+    NormPlan vecp = plan_norm(C, dtype, true);
+    NormPlan genp{true, 256, 0, 1};
+    uint64_t blocks = bwd_blocks(genp, rows);
+    if (!vecp.generic) {
+        const uint64_t b = bwd_blocks(vecp, rows);
+        if (b > blocks) blocks = b;
+    }
+    return 2ull * blocks * C * sizeof(float);
+}
+
+int launch_norm_fwd(hipStream_t s, int kind, int dtype, const void* x, const void* residual,
+                    const float* gamma, const float* beta, void* h_out, void* y,
+                    uint64_t rows, uint32_t C, float eps) {
+    if (kind != AGRAD_NORM_LAYER && kind != AGRAD_NORM_RMS)
+        return set_error(AGRAD_EINVAL, "norm forward: unknown kind %d", kind);
+    if (dtype != AGRAD_F32 && dtype != AGRAD_BF16)
+        return set_error(AGRAD_EINVAL, "norm forward: unknown dtype %d", dtype);
+    if (rows == 0 || C == 0) return AGRAD_OK;
+    if (x == nullptr || y == nullptr) return set_error(AGRAD_EINVAL, "norm forward: null x or y");
+    if (rows > 0x7fffffffull) return set_error(AGRAD_EINVAL, "norm forward: too many rows");
+    const bool aligned = aligned16(x) && aligned16(y) && (!residual || aligned16(residual)) &&
+                         (!h_out || aligned16(h_out)) && (!gamma || aligned16(gamma)) &&
+                         (!beta || aligned16(beta));
+    const NormPlan p = plan_norm(C, dtype, aligned);
+    if (dtype == AGRAD_F32) {
+        NormFwdArgs<float> a{(const float*)x, (const float*)residual, gamma, beta, (float*)h_out,
+                             (float*)y, rows, C, eps, kind};
+        return norm_fwd_typed<float>(s, p, a);
+    }
+    NormFwdArgs<bf16_t> a{(const bf16_t*)x, (const bf16_t*)residual, gamma, beta, (bf16_t*)h_out,
+                          (bf16_t*)y, rows, C, eps, kind};
+    return norm_fwd_typed<bf16_t>(s, p, a);
+}
+
+int launch_norm_bwd(hipStream_t s, int kind, int dtype, const void* x, const void* dy,
+                    const float* gamma, const void* dres_in, void* dx, void* dx2,
+                    float* dgamma, float* dbeta, void* workspace, uint64_t workspace_bytes,
+                    uint64_t rows, uint32_t C, float eps, uint32_t flags) {
+    if (kind != AGRAD_NORM_LAYER && kind != AGRAD_NORM_RMS)
+        return set_error(AGRAD_EINVAL, "norm backward: unknown kind %d", kind);
+    if (dtype != AGRAD_F32 && dtype != AGRAD_BF16)
+        return set_error(AGRAD_EINVAL, "norm backward: unknown dtype %d", dtype);
+    if (C == 0) return AGRAD_OK;
+    if (x == nullptr || dy == nullptr) return set_error(AGRAD_EINVAL, "norm backward: null x or dy");
+    if (dx == nullptr && dx2 != nullptr) return set_error(AGRAD_EINVAL, "norm backward: dx2 without dx");
+    if (dx == nullptr && dgamma == nullptr && dbeta == nullptr) return AGRAD_OK;
+    if (rows > 0x7fffffffull) return set_error(AGRAD_EINVAL, "norm backward: too many rows");
+    const bool aligned = aligned16(x) && aligned16(dy) && (!dres_in || aligned16(dres_in)) &&
+                         (!dx || aligned16(dx)) && (!dx2 || aligned16(dx2)) &&
+                         (!gamma || aligned16(gamma));
+    const NormPlan p = plan_norm(C, dtype, aligned);
+    const uint32_t grid = bwd_blocks(p, rows);
+    const bool want_params = dgamma != nullptr || dbeta != nullptr;
+    float* pg = nullptr;
+    float* pb = nullptr;
+    if (want_params) {
+        const uint64_t need = 2ull * grid * C * sizeof(float);
+        if (workspace == nullptr || workspace_bytes < need)
+            return set_error(AGRAD_EWORKSPACE, "norm backward: workspace %llu < %llu bytes",
+                             (unsigned long long)workspace_bytes, (unsigned long long)need);
+        if (dgamma) pg = (float*)workspace;
+        if (dbeta) pb = (float*)workspace + (uint64_t)grid * C;
+    }
+    int rc = AGRAD_OK;
+    if (rows > 0) {
+        if (dtype == AGRAD_F32) {
+            NormBwdArgs<float> a{(const float*)x, (const float*)dy, gamma, (const float*)dres_in,
+                                 (float*)dx, (float*)dx2, pg, pb, rows, C, eps, kind, flags};
+            rc = norm_bwd_typed<float>(s, p, a, grid);
+        } else {
+            NormBwdArgs<bf16_t> a{(const bf16_t*)x, (const bf16_t*)dy, gamma, (const bf16_t*)dres_in,
+                                  (bf16_t*)dx, (bf16_t*)dx2, pg, pb, rows, C, eps, kind, flags};
+            rc = norm_bwd_typed<bf16_t>(s, p, a, grid);
+        }
+        if (rc != AGRAD_OK) return rc;
+    }
+    if (want_params) {
+        const int accp = (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0;
+        const uint32_t P = rows > 0 ? grid : 0;
+        const uint32_t fgrid = (C + 31) / 32;
+        if (dgamma)
+            hipLaunchKernelGGL(colsum_finalize_kernel, dim3(fgrid), dim3(256), 0, s, pg, P, C, dgamma, accp);
+        if (dbeta)
+            hipLaunchKernelGGL(colsum_finalize_kernel, dim3(fgrid), dim3(256), 0, s, pb, P, C, dbeta, accp);
+    }
+    return check_hip(hipGetLastError(), "norm backward launch");
+}
+
+}  // namespace agrad

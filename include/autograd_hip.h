@@ -1,0 +1,192 @@
+/*
+ * autograd_hip.h -- C ABI of libautograd_hip.so: the MI355X (gfx950) native layer
+ * that takes the place of the reference's Metal extension for the fused
+ * layer-op path (norms, activations, rotary, embedding gather / grad).
+ *
+ * Everything crosses the boundary as plain pointers, sizes and 32-bit words.
+ * Device buffers are addressed the way the reference addresses Metal buffers:
+ * an opaque buffer id (here: the device address returned by agrad_alloc) plus a
+ * byte offset (storage.py:66-90).  All work is enqueued on the context's single
+ * in-order HIP stream; agrad_end_pass / agrad_synchronize block until it drains
+ * (metal_ext.mm:202-213, 763-767).
+ *
+ * Every function returns AGRAD_OK (0) or a negative AGRAD_E* code; the message
+ * of the last failure on the calling thread is agrad_last_error().
+ */
+#ifndef AUTOGRAD_HIP_H
+#define AUTOGRAD_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct agrad_ctx agrad_ctx;
+
+enum {
+    AGRAD_OK = 0,
+    AGRAD_EINVAL = -1,      /* bad argument, shape or alignment            */
+    AGRAD_EHIP = -2,        /* a HIP runtime call failed                   */
+    AGRAD_ENOKERNEL = -3,   /* agrad_dispatch: unknown kernel name         */
+    AGRAD_EINDEX = -4,      /* a token id outside [0, V) was seen on device */
+    AGRAD_EWORKSPACE = -5   /* workspace too small                         */
+};
+
+/* Storage type of the large operands.  Arithmetic is always fp32.            */
+enum { AGRAD_F32 = 0, AGRAD_BF16 = 1 };
+
+/* Norm flavour.                                                              */
+enum { AGRAD_NORM_LAYER = 0, AGRAD_NORM_RMS = 1 };
+
+/* Flag bits for backward entry points.                                       */
+enum {
+    AGRAD_ACC_INPUT_GRAD = 1u, /* dx += ... (CPU semantics, backend.py:414,477-487); else dx = ... */
+    AGRAD_ACC_PARAM_GRAD = 2u  /* dgamma/dbeta/dW += ...; else =                                   */
+};
+
+/* ---- context, memory, passes --------------------------------------------
+ * Replaces MetalContext() / alloc / free / max_buffer_length / begin_pass /
+ * end_pass / synchronize / copy_* / fill_scalar* (metal_ext.mm:33-213, 444-510,
+ * 723-767). */
+const char* agrad_last_error(void);
+int agrad_device_count(int* count);
+int agrad_ctx_create(int device, agrad_ctx** out);
+int agrad_ctx_destroy(agrad_ctx* ctx);
+int agrad_max_buffer_length(agrad_ctx* ctx, uint64_t* bytes);
+int agrad_alloc(agrad_ctx* ctx, uint64_t bytes, uint64_t* buffer_id);
+int agrad_free(agrad_ctx* ctx, uint64_t buffer_id);
+int agrad_begin_pass(agrad_ctx* ctx);
+/* Blocks until the stream drains; returns AGRAD_EINDEX if any kernel since the
+ * last check saw an out-of-range token id (numpy raises IndexError there,
+ * backend.py:525-538). */
+int agrad_end_pass(agrad_ctx* ctx);
+int agrad_synchronize(agrad_ctx* ctx);
+int agrad_copy_from_host(agrad_ctx* ctx, uint64_t buffer_id, uint64_t offset,
+                         const void* src, uint64_t nbytes);
+int agrad_copy_to_host(agrad_ctx* ctx, uint64_t buffer_id, uint64_t offset,
+                       void* dst, uint64_t nbytes);
+/* fill n items of itemsize 1, 2 or 4 bytes with the low bits of `bits`
+ * (fill_scalar_kernel / fill_scalar_kernel2, metal_ops.metal:122-144). */
+int agrad_fill(agrad_ctx* ctx, uint64_t buffer_id, uint64_t offset,
+               uint32_t bits, int itemsize, uint64_t n);
+/* The HIP stream of the context as a hipStream_t cast to void*.              */
+int agrad_stream(agrad_ctx* ctx, void** stream);
+/* Event timing on the context's stream (the role of begin_pass_profiled /
+ * end_pass_profiled, metal_ext.mm:215-286): elapsed GPU ms between the two. */
+int agrad_timer_start(agrad_ctx* ctx);
+int agrad_timer_stop(agrad_ctx* ctx, float* elapsed_ms);
+
+/* ---- name-based launch ----------------------------------------------------
+ * Replaces MetalContext.dispatch_with_args_3d (metal_ext.mm:559-590): a kernel
+ * name, parallel lists of buffer ids and byte offsets, and uint32 arguments
+ * (floats travel as their bit pattern, backend.py:2916).  The launch geometry
+ * is chosen here from the shape arguments; gx/gy/gz/tg are accepted so call
+ * sites keep the reference's signature, and are ignored.  Unknown names fail
+ * with AGRAD_ENOKERNEL (the reference silently binds a nil pipeline,
+ * metal_ext.mm:567).  Kernel names and their operand lists are given by
+ * agrad_kernel_signature. */
+int agrad_dispatch(agrad_ctx* ctx, const char* name,
+                   const uint64_t* buffer_ids, const uint64_t* offsets, int n_buffers,
+                   const uint32_t* args, int n_args,
+                   uint64_t gx, uint64_t gy, uint64_t gz, uint64_t tg);
+int agrad_kernel_count(void);
+const char* agrad_kernel_name(int index);
+/* Human-readable "buffers | args" description of a kernel, or NULL.          */
+const char* agrad_kernel_signature(const char* name);
+
+/* ---- typed entry points (device addresses, already offset) ----------------
+ * `dtype` is the storage type of activations / gradients / embedding tables;
+ * gamma, beta, dgamma, dbeta, cos, sin are always fp32; ids are int32.       */
+
+/* out[i] = x[i] + y[i]  (cpu_add_forward, backend.py:74-76; add_residual_forward,
+ * metal_ops.metal:161-181). */
+int agrad_add_forward(agrad_ctx* ctx, int dtype, const void* x, const void* y, void* out, uint64_t n);
+/* dst[i] (+)= src[i]  (same-shape branch of cpu_add_backward, backend.py:78-105). */
+int agrad_grad_accumulate(agrad_ctx* ctx, int dtype, const void* src, void* dst, uint64_t n, uint32_t flags);
+/* dst_bf16[i] = rne(src_f32[i]) (+ dst if accumulate) (fp32_to_bf16, metal_ops.metal:12010-12041). */
+int agrad_cast_f32_to_bf16(agrad_ctx* ctx, const void* src, void* dst, uint64_t n, int accumulate);
+int agrad_cast_bf16_to_f32(agrad_ctx* ctx, const void* src, void* dst, uint64_t n);
+/* plain device copy kernel; the calibration kernel for bandwidth and counters. */
+int agrad_copy(agrad_ctx* ctx, const void* src, void* dst, uint64_t nbytes);
+
+/* LayerNorm / RMSNorm forward over rows of width C.
+ *   residual != NULL: h = x + residual is normalised; h is stored to h_out if non-NULL.
+ *   gamma / beta may be NULL (weightless RMSNorm, backend.py:1097-1105).
+ * LayerNorm: cpu_layernorm_forward (backend.py:416-433), layernorm_forward
+ * (metal_ops.metal:3539-3649).  RMSNorm: backend.py:1097-1108, 1737-1745;
+ * rmsnorm_forward / rmsnorm_weighted_forward (metal_ops.metal:3412-3537). */
+int agrad_norm_forward(agrad_ctx* ctx, int kind, int dtype,
+                       const void* x, const void* residual,
+                       const float* gamma, const float* beta,
+                       void* h_out, void* y,
+                       uint64_t rows, uint32_t C, float eps);
+
+/* Bytes of workspace agrad_norm_backward needs for the column reductions.    */
+uint64_t agrad_norm_backward_workspace_bytes(uint64_t rows, uint32_t C, int dtype);
+/* Norm backward.  x is the tensor that was normalised (h when a residual was
+ * fused).  dx = [dx if ACC_INPUT_GRAD] + [dres_in] + dnorm; dx2 (optional)
+ * receives the same values (the second operand of a fused residual add).
+ * dgamma / dbeta (optional) are reduced over rows in two deterministic stages.
+ * cpu_layernorm_backward (backend.py:435-487); RMSNorm slices backend.py:1228-1251,
+ * 1990-2011; rmsnorm_backward's fused residual_grad (metal_ops.metal:8107-8257). */
+int agrad_norm_backward(agrad_ctx* ctx, int kind, int dtype,
+                        const void* x, const void* dy, const float* gamma,
+                        const void* dres_in, void* dx, void* dx2,
+                        float* dgamma, float* dbeta,
+                        void* workspace, uint64_t workspace_bytes,
+                        uint64_t rows, uint32_t C, float eps, uint32_t flags);
+
+/* tanh-GELU (cpu_gelu_forward / backward, backend.py:376-414).               */
+int agrad_gelu_forward(agrad_ctx* ctx, int dtype, const void* x, void* y, uint64_t n);
+int agrad_gelu_backward(agrad_ctx* ctx, int dtype, const void* x, const void* dy, void* dx, uint64_t n, uint32_t flags);
+/* ReLU^2: y = max(x,0)^2, dx = 2 max(x,0) dy.  No counterpart in the reference. */
+int agrad_relu2_forward(agrad_ctx* ctx, int dtype, const void* x, void* y, uint64_t n);
+int agrad_relu2_backward(agrad_ctx* ctx, int dtype, const void* x, const void* dy, void* dx, uint64_t n, uint32_t flags);
+/* SwiGLU on gu[rows, 2H] (gate = first H columns, up = last H): h = silu(g)*u.
+ * Backward writes dgu[rows, 2H] = [dg | du]; dgu may alias gu (in place).
+ * backend.py:1113-1126, 1178-1217; swiglu_forward_kernel /
+ * swiglu_backward_inplace_kernel (metal_ops.metal:3808-4017). */
+int agrad_swiglu_forward(agrad_ctx* ctx, int dtype, const void* gu, void* h, uint64_t rows, uint32_t H);
+int agrad_swiglu_backward(agrad_ctx* ctx, int dtype, const void* gu, const void* dh, void* dgu,
+                          uint64_t rows, uint32_t H, uint32_t flags);
+
+/* Split-half rotary embedding applied in place to q[B,T,H,D] and k[B,T,HKV,D]
+ * (k may be NULL) with fp32 tables cos/sin[T, D/2]:
+ *   lo' = lo*c - s*(hi*sin),  hi' = hi*c + s*(lo*sin),  s = rope_sign (+1 HF, -1 nanochat);
+ * backward != 0 applies the transpose (s negated).
+ * apply_rope_np / apply_rope_backward_np (backend.py:1382-1417), GQA loops
+ * (backend.py:1755-1782, 1937-1958); rope_qk_inplace / gqa_rope_inplace
+ * (metal_ops.metal:7423-7491, 11732-11747). */
+int agrad_rope_qk(agrad_ctx* ctx, int dtype, void* q, void* k,
+                  const float* cos_table, const float* sin_table,
+                  uint32_t B, uint32_t T, uint32_t H, uint32_t HKV, uint32_t D,
+                  int rope_sign, int backward);
+
+/* out[n,:] = W[ids[n],:] (+ wpe[n % T,:] if wpe != NULL).
+ * cpu_gather_forward (backend.py:525-529), gather_forward_kernel
+ * (metal_ops.metal:390-404), add_pos_forward (metal_ops.metal:205-218). */
+int agrad_gather_forward(agrad_ctx* ctx, int dtype, const int32_t* ids,
+                         const void* W, const void* wpe, void* out,
+                         uint64_t N, uint32_t T, uint32_t C, uint32_t V);
+
+/* Embedding gradient dW[ids[n],:] += dY[n,:], deterministic: rows are sorted by
+ * token id (stable), then each token's run is summed in ascending row order
+ * (cpu_gather_backward = np.add.at, backend.py:531-538; replaces the float-atomic
+ * gather_backward_kernel, metal_ops.metal:406-427).
+ * Without AGRAD_ACC_PARAM_GRAD the touched rows of dW are overwritten (correct on
+ * a table that was just zero-filled); untouched rows are never written. */
+uint64_t agrad_embedding_backward_workspace_bytes(uint64_t N, uint32_t C, uint32_t V, int dtype);
+int agrad_embedding_backward(agrad_ctx* ctx, int dtype, const int32_t* ids, const void* dY, void* dW,
+                             void* workspace, uint64_t workspace_bytes,
+                             uint64_t N, uint32_t C, uint32_t V, uint32_t flags);
+/* dwpe[t,:] (+)= sum_b dY[b,t,:], b ascending (pos_emb_grad, metal_ops.metal:220-234;
+ * broadcast branch of cpu_add_backward, backend.py:78-105). */
+int agrad_pos_embedding_backward(agrad_ctx* ctx, int dtype, const void* dY, void* dwpe,
+                                 uint32_t B, uint32_t T, uint32_t C, uint32_t flags);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AUTOGRAD_HIP_H */

@@ -1,0 +1,355 @@
+"""CPU restatement of the reference's fused layer-op kernels (numpy, fp32).
+
+TEST INFRASTRUCTURE ONLY.  This module is the checker for the HIP kernels: it is
+imported by tests/, by __graft_entry__.smoke() and by the cpu_baseline leg of
+bench.py, and by nothing in the autograd_amd package.
+
+Each function performs the same sequence of whole-array fp32 numpy operations
+as the reference function it cites (every step rounds to fp32, no FMA), so its
+results are what the reference's "cpu" device produces with the same numpy.
+Citations are file:line in the reference repository.
+
+Pinning (what shows these functions are the right functions; tests/test_oracle.py):
+  * layernorm / gelu: the reference's own independent numpy oracles
+    (verify_model.py:127-135 restated in oracle/closed_form.py), float64 closed
+    forms, finite differences, row invariants.
+  * rmsnorm / swiglu / rope: the closed forms of debug/check_qwen_kernel.py:195-342,
+    577-645 (restated in float64), finite differences, rotation invariants.
+  * gather: numpy fancy indexing; backward: brute-force row loop.
+  * bf16: bit-exact against an exhaustive integer restatement of utils.py:20-27.
+Parity unpinned by the reference:
+  * relu2_* -- the reference has no ReLU^2; pinned by its closed form only.
+  * d(gamma), d(beta) at large row counts -- numpy sums rows sequentially in
+    fp32 (backend.py:461,466); the value is pinned, its rounding noise (~1e-4
+    absolute at N = 16384) is numpy behaviour that no GPU reduction order
+    reproduces bit for bit.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+F32 = np.float32
+
+# backend.py:18-20
+GELU_C = 0.7978845608028654
+GELU_A = 0.044715
+GELU_A3 = 0.134145
+
+
+# --------------------------------------------------------------------------
+# Add  (cpu_add_forward / cpu_add_backward, backend.py:74-105)
+# --------------------------------------------------------------------------
+def add_forward(x, y):
+    return np.add(x, y)
+
+
+def add_backward_into(g, grad):
+    """grad += g, summing g over the leading axes it was broadcast along."""
+    if g.shape == grad.shape:
+        np.add(grad, g, out=grad)
+        return
+    lead = g.ndim - grad.ndim
+    padded = (1,) * lead + grad.shape
+    axes = tuple(i for i, (gi, ti) in enumerate(zip(g.shape, padded)) if ti == 1 and gi != 1)
+    tmp = np.sum(g, axis=axes) if axes else g
+    np.add(grad, tmp.reshape(grad.shape), out=grad)
+
+
+# --------------------------------------------------------------------------
+# GELU-tanh  (cpu_gelu_forward / cpu_gelu_backward, backend.py:376-414)
+# --------------------------------------------------------------------------
+def _gelu_tanh(x):
+    b = np.multiply(x, x)
+    np.multiply(b, x, out=b)
+    np.multiply(b, GELU_A, out=b)
+    np.add(x, b, out=b)
+    np.multiply(b, GELU_C, out=b)
+    np.tanh(b, out=b)
+    return b
+
+
+def gelu_forward(x):
+    b = _gelu_tanh(x)
+    np.add(b, 1.0, out=b)
+    np.multiply(x, b, out=b)
+    return np.multiply(b, 0.5)
+
+
+def gelu_backward_into(x, dy, dx):
+    t = _gelu_tanh(x)
+    a = np.multiply(t, t)
+    np.subtract(1.0, a, out=a)
+    d_inner = GELU_C * (1.0 + GELU_A3 * x * x)
+    np.multiply(a, 0.5 * x * d_inner, out=a)
+    np.add(t, 1.0, out=t)
+    np.multiply(t, 0.5, out=t)
+    np.add(t, a, out=t)
+    np.multiply(dy, t, out=a)
+    np.add(dx, a, out=dx)
+
+
+# --------------------------------------------------------------------------
+# ReLU^2  (no reference counterpart: y = max(x,0)^2, dx += 2 max(x,0) dy)
+# --------------------------------------------------------------------------
+def relu2_forward(x):
+    r = np.maximum(x, F32(0))
+    return np.multiply(r, r)
+
+
+def relu2_backward_into(x, dy, dx):
+    r = np.maximum(x, F32(0))
+    np.multiply(r, F32(2), out=r)
+    np.multiply(r, dy, out=r)
+    np.add(dx, r, out=dx)
+
+
+# --------------------------------------------------------------------------
+# LayerNorm  (cpu_layernorm_forward / backward, backend.py:416-487)
+# --------------------------------------------------------------------------
+def _ln_stats(x, eps):
+    """returns (inv_std [.., 1], x_hat) computed as backend.py:420-430 does."""
+    r = np.mean(x, axis=-1, keepdims=True)
+    f = np.subtract(x, r)
+    np.multiply(f, f, out=f)
+    np.mean(f, axis=-1, keepdims=True, out=r)
+    np.add(r, eps, out=r)
+    np.sqrt(r, out=r)
+    np.reciprocal(r, out=r)
+    np.subtract(x, np.mean(x, axis=-1, keepdims=True), out=f)
+    np.multiply(f, r, out=f)
+    return r, f
+
+
+def layernorm_forward(x, gamma, beta, eps):
+    _, f = _ln_stats(x, eps)
+    y = np.multiply(f, gamma)
+    np.add(y, beta, out=y)
+    return y
+
+
+def layernorm_backward_into(x, gamma, dy, eps, dx=None, dgamma=None, dbeta=None):
+    inv_std, x_hat = _ln_stats(x, eps)
+    lead = tuple(range(x.ndim - 1))
+    if dgamma is not None:
+        f2 = np.multiply(dy, x_hat)
+        tmp = np.sum(f2, axis=lead)
+        np.add(dgamma, tmp.reshape(dgamma.shape), out=dgamma)
+    if dbeta is not None:
+        tmp = np.sum(dy, axis=lead)
+        np.add(dbeta, tmp.reshape(dbeta.shape), out=dbeta)
+    if dx is not None:
+        f2 = np.multiply(dy, gamma)
+        f3 = np.multiply(f2, inv_std)
+        np.add(dx, f3, out=dx)
+        r2 = np.mean(f2, axis=-1, keepdims=True)
+        np.multiply(r2, inv_std, out=r2)
+        np.subtract(dx, r2, out=dx)
+        np.multiply(f2, x_hat, out=f2)
+        np.mean(f2, axis=-1, keepdims=True, out=r2)
+        np.multiply(r2, inv_std, out=r2)
+        np.multiply(x_hat, r2, out=f3)
+        np.subtract(dx, f3, out=dx)
+
+
+# --------------------------------------------------------------------------
+# RMSNorm  (slices of the fused ops: forward backend.py:1097-1108, 1737-1745;
+#           backward backend.py:1228-1251, 1990-2011)
+# --------------------------------------------------------------------------
+def _rms_inv(x, eps):
+    t = np.multiply(x, x)
+    inv = np.mean(t, axis=-1, keepdims=True)
+    np.add(inv, F32(eps), out=inv)
+    np.sqrt(inv, out=inv)
+    np.reciprocal(inv, out=inv)
+    return inv
+
+
+def rmsnorm_forward(x, gamma, eps):
+    inv = _rms_inv(x, eps)
+    z = np.multiply(x, inv)
+    if gamma is not None:
+        np.multiply(z, gamma, out=z)
+    return z
+
+
+def rmsnorm_backward_into(x, gamma, dz, eps, dx=None, dgamma=None):
+    """backend.py:1990-2011 (weighted) / 1228-1251 (gamma optional)."""
+    inv = _rms_inv(x, eps)
+    x_hat = np.multiply(x, inv)
+    lead = tuple(range(x.ndim - 1))
+    if dgamma is not None:
+        t = np.multiply(dz, x_hat)
+        tmp = np.sum(t, axis=lead)
+        np.add(dgamma, tmp, out=dgamma)
+    if dx is not None:
+        d = np.multiply(dz, gamma) if gamma is not None else np.array(dz, copy=True)
+        t = np.multiply(d, x_hat)
+        m = np.mean(t, axis=-1, keepdims=True)
+        np.multiply(x_hat, m, out=t)
+        np.subtract(d, t, out=t)
+        np.multiply(t, inv, out=t)
+        np.add(dx, t, out=dx)
+
+
+# --------------------------------------------------------------------------
+# residual add fused with a norm: cpu_add_forward then the norm; backward is
+# the norm backward accumulated onto the gradient already sitting on h, then
+# cpu_add_backward hands that gradient to both operands (backend.py:74-105).
+# --------------------------------------------------------------------------
+def add_norm_forward(kind, x, res, gamma, beta, eps):
+    h = add_forward(x, res)
+    if kind == "layer":
+        return h, layernorm_forward(h, gamma, beta, eps)
+    return h, rmsnorm_forward(h, gamma, eps)
+
+
+# --------------------------------------------------------------------------
+# SwiGLU  (forward backend.py:1113-1126; backward backend.py:1180-1217)
+# --------------------------------------------------------------------------
+def _sigmoid_ref(g):
+    s = np.negative(g)
+    np.exp(s, out=s)
+    np.add(s, 1.0, out=s)
+    np.reciprocal(s, out=s)
+    return s
+
+
+def swiglu_forward(gu):
+    H = gu.shape[-1] // 2
+    g, u = gu[..., :H], gu[..., H:]
+    with np.errstate(over="ignore"):
+        h = _sigmoid_ref(g)
+    np.multiply(g, h, out=h)
+    np.multiply(h, u, out=h)
+    return h
+
+
+def swiglu_backward(gu, dh):
+    """returns dgu = [dg | du] (the reference overwrites gu with it)."""
+    H = gu.shape[-1] // 2
+    g, u = gu[..., :H], gu[..., H:]
+    with np.errstate(over="ignore"):
+        s = _sigmoid_ref(g)
+    dgu = np.empty_like(gu)
+    dg, du = dgu[..., :H], dgu[..., H:]
+    np.subtract(1.0, s, out=dg)
+    np.multiply(dg, g, out=dg)
+    np.add(dg, 1.0, out=dg)
+    np.multiply(dg, s, out=dg)
+    np.multiply(dg, u, out=dg)
+    np.multiply(dg, dh, out=dg)
+    np.multiply(g, s, out=du)
+    np.multiply(du, dh, out=du)
+    return dgu
+
+
+# --------------------------------------------------------------------------
+# RoPE
+# --------------------------------------------------------------------------
+def rope_tables(T, D, theta):
+    """module.py:247-255: fp32 tables cos/sin[T, D/2]."""
+    pos = np.arange(T, dtype=np.float32)[:, None]
+    ch = np.arange(0, D, 2, dtype=np.float32)[None, :]
+    inv = np.float32(theta) ** (-ch / np.float32(D))
+    f = pos * inv
+    return np.cos(f).astype(np.float32), np.sin(f).astype(np.float32)
+
+
+def rope_nanochat(q, k, cos, sin, backward=False):
+    """apply_rope_np / apply_rope_backward_np (backend.py:1382-1417); q, k are
+    [B, T, H, D] and are rotated in place."""
+    d2 = q.shape[-1] // 2
+    c = cos[None, :, None, :]
+    s = sin[None, :, None, :]
+    for a in (q, k):
+        if a is None:
+            continue
+        a1 = a[..., :d2].copy()
+        a2 = a[..., d2:].copy()
+        if not backward:
+            a[..., :d2] = a1 * c + a2 * s
+            a[..., d2:] = -a1 * s + a2 * c
+        else:
+            a[..., :d2] = a1 * c - a2 * s
+            a[..., d2:] = a1 * s + a2 * c
+
+
+def rope_signed(q, k, cos, sin, rope_sign, backward=False):
+    """The GQA loops (forward backend.py:1761-1782, backward 1938-1958): per
+    (batch, head) slice, in place, with the rope_sign convention (+1 = HF)."""
+    half = q.shape[-1] // 2
+    T = q.shape[1]
+    cos = cos[:T]
+    sin = sin[:T]
+    plus = (rope_sign == 1) != backward  # True: lo' = p - q, hi' = hi*c + lo*s
+    r0 = np.empty((T, half), dtype=np.float32)
+    r1 = np.empty((T, half), dtype=np.float32)
+    for data in (q, k):
+        if data is None:
+            continue
+        for b in range(data.shape[0]):
+            for h in range(data.shape[2]):
+                lo = data[b, :, h, :half]
+                hi = data[b, :, h, half:]
+                np.multiply(lo, cos, out=r0)
+                np.multiply(hi, sin, out=r1)
+                if plus:
+                    np.subtract(r0, r1, out=r0)
+                else:
+                    np.add(r0, r1, out=r0)
+                np.multiply(lo, sin, out=r1)
+                np.multiply(hi, cos, out=hi)
+                if plus:
+                    np.add(hi, r1, out=hi)
+                else:
+                    np.subtract(hi, r1, out=hi)
+                np.copyto(lo, r0)
+
+
+# --------------------------------------------------------------------------
+# Embedding  (cpu_gather_forward / backward, backend.py:525-538)
+# --------------------------------------------------------------------------
+def gather_forward(ids, W):
+    return W[ids.astype(np.int64)]
+
+
+def gather_backward_into(ids, dY, dW):
+    np.add.at(dW, ids.astype(np.int64).ravel(), dY.reshape(-1, dW.shape[-1]))
+
+
+def embedding_sum_forward(ids, wte, wpe):
+    """x0 = tok_emb(ids) + pos_emb(pos_ids), pos_ids = tile(arange(T))
+    (check_tiny_gpt2_kernel.py:282,301)."""
+    B, T = ids.shape
+    pos = np.tile(np.arange(T, dtype=np.int32), (B, 1))
+    return add_forward(gather_forward(ids, wte), gather_forward(pos, wpe))
+
+
+def embedding_sum_backward_into(ids, dY, dwte, dwpe):
+    B, T = ids.shape
+    pos = np.tile(np.arange(T, dtype=np.int32), (B, 1))
+    if dwte is not None:
+        gather_backward_into(ids, dY, dwte)
+    if dwpe is not None:
+        gather_backward_into(pos, dY, dwpe)
+
+
+# --------------------------------------------------------------------------
+# bf16 storage  (bf16_bits, utils.py:20-27; array form backend.py:5090-5113)
+# --------------------------------------------------------------------------
+def f32_to_bf16_bits(a):
+    bits = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+    rounded = (bits + np.uint32(0x7FFF) + ((bits >> np.uint32(16)) & np.uint32(1))) >> np.uint32(16)
+    special = (bits & np.uint32(0x7F800000)) == np.uint32(0x7F800000)
+    nan = special & ((bits & np.uint32(0x007FFFFF)) != np.uint32(0))
+    special_bits = (bits >> np.uint32(16)) | np.where(nan, np.uint32(0x0040), np.uint32(0))
+    return np.where(special, special_bits, rounded).astype(np.uint16)
+
+
+def bf16_bits_to_f32(b):
+    return (np.asarray(b, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def round_bf16(a):
+    """fp32 array rounded to the nearest bf16 value, returned as fp32."""
+    return bf16_bits_to_f32(f32_to_bf16_bits(a)).reshape(np.shape(a))

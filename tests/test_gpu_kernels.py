@@ -1,0 +1,539 @@
+"""Parity of every HIP kernel against the CPU restatement, through the C ABI.
+
+Tolerances: fp32 outputs rtol 1e-5 / atol 1e-6 (helpers.FP32_*); gather and
+fill / cast are bit-exact; bf16-I/O outputs 1e-2 relative to the fp32 path fed
+the same bf16-rounded inputs (helpers.BF16_REL).  Row-summed parameter
+gradients (dgamma, dbeta) are compared to the fp32 CPU result at probe sizes and
+to the float64 closed form at large row counts, where the CPU's own sequential
+fp32 row sum is the noisier of the two.
+
+Seeds follow the reference's probes (SEED = 1333, check_tiny_gpt2_kernel.py:47).
+"""
+import numpy as np
+import pytest
+
+from autograd_amd import capi
+from oracle import closed_form as cf
+from oracle import cpu_ops as ref
+from tests import gpu_ops as G
+from tests.helpers import (assert_bf16_close, assert_fp32_close, from_bf16_bits, to_bf16_bits)
+
+pytestmark = pytest.mark.gpu
+SEED = 1333
+KINDS = {"layer": capi.NORM_LAYER, "rms": capi.NORM_RMS}
+
+
+def _rng(k):
+    return np.random.default_rng(SEED + k)
+
+
+def _norm_ref_forward(kind, x, gamma, beta, eps):
+    if kind == "layer":
+        return ref.layernorm_forward(x, gamma, beta, eps)
+    return ref.rmsnorm_forward(x, gamma, eps)
+
+
+def _norm_ref_backward(kind, x, gamma, dy, eps, want_params=True):
+    dx = np.zeros_like(x)
+    dgamma = np.zeros_like(gamma) if want_params else None
+    if kind == "layer":
+        dbeta = np.zeros_like(gamma) if want_params else None
+        ref.layernorm_backward_into(x, gamma, dy, eps, dx, dgamma, dbeta)
+        return dx, dgamma, dbeta
+    ref.rmsnorm_backward_into(x, gamma, dy, eps, dx, dgamma)
+    return dx, dgamma, None
+
+
+# shapes cover every launch geometry: wave-per-row (C <= 1024) with 1..4 vectors
+# per lane, workgroup-per-row (256 and 1024 threads), and the scalar fallback
+NORM_SHAPES = [
+    ((2, 16, 64), 1e-5),     # the reference's probe_layernorm shape (check_tiny_gpt2_kernel.py:758-782)
+    ((512, 128), 1e-5),      # config 1
+    ((67, 384), 1e-5),       # config 2 width, ragged row count
+    ((45, 768), 1e-5),       # config 3 width
+    ((33, 1024), 1e-6),
+    ((21, 1536), 1e-6),      # config 4 width
+    ((9, 4096), 1e-5),       # config 5 width
+    ((5, 8192), 1e-5),       # 1024-thread rows
+    ((7, 50), 1e-5),         # C % 4 != 0 -> scalar kernel
+    ((3, 20000), 1e-5),      # wider than any register-resident geometry
+    ((1, 4), 1e-5),
+]
+
+
+@pytest.mark.parametrize("kind", ["layer", "rms"])
+@pytest.mark.parametrize("shape,eps", NORM_SHAPES)
+def test_norm_forward_fp32(ctx, kind, shape, eps):
+    rng = _rng(4)
+    C = shape[-1]
+    x = rng.standard_normal(shape, dtype=np.float32)
+    gamma = (1 + 0.02 * rng.standard_normal(C)).astype(np.float32)
+    beta = (0.02 * rng.standard_normal(C)).astype(np.float32) if kind == "layer" else None
+    got, _ = G.norm_forward(ctx, KINDS[kind], x, gamma, beta, eps)
+    assert_fp32_close(got, _norm_ref_forward(kind, x, gamma, beta, eps), f"{kind} forward {shape}")
+
+
+def test_norm_forward_probe_recipe(ctx):
+    """probe_layernorm: seed+4, (2,16,64), gamma/beta ~ N(0,1), eps 1e-5."""
+    rng = _rng(4)
+    x = rng.standard_normal((2, 16, 64), dtype=np.float32)
+    g = rng.standard_normal((64,), dtype=np.float32)
+    b = rng.standard_normal((64,), dtype=np.float32)
+    up = rng.standard_normal((2, 16, 64), dtype=np.float32)
+    got, _ = G.norm_forward(ctx, capi.NORM_LAYER, x, g, b, 1e-5)
+    assert_fp32_close(got, ref.layernorm_forward(x, g, b, 1e-5), "probe forward", rtol=1e-6, atol=1e-6)
+    out = G.norm_backward(ctx, capi.NORM_LAYER, x, g, up, 1e-5)
+    dx, dg, db = _norm_ref_backward("layer", x, g, up, 1e-5)
+    assert_fp32_close(out["dx"], dx, "probe x.grad")
+    assert_fp32_close(out["dgamma"], dg, "probe gamma.grad")
+    assert_fp32_close(out["dbeta"], db, "probe beta.grad")
+
+
+def test_rmsnorm_weightless_and_layernorm_without_affine(ctx):
+    rng = _rng(6)
+    x = rng.standard_normal((19, 384), dtype=np.float32)
+    got, _ = G.norm_forward(ctx, capi.NORM_RMS, x, None, None, 1e-6)
+    assert_fp32_close(got, ref.rmsnorm_forward(x, None, 1e-6), "weightless rms")
+    got, _ = G.norm_forward(ctx, capi.NORM_LAYER, x, None, None, 1e-5)
+    one, zero = np.ones(384, np.float32), np.zeros(384, np.float32)
+    assert_fp32_close(got, ref.layernorm_forward(x, one, zero, 1e-5), "plain layernorm")
+    # gamma = 1, beta = 0 (config 1): rows have mean 0 and variance 1
+    assert np.abs(got.mean(-1)).max() < 1e-6
+    assert np.abs(got.var(-1) - 1).max() < 1e-4
+    dy = rng.standard_normal(x.shape, dtype=np.float32)
+    out = G.norm_backward(ctx, capi.NORM_RMS, x, None, dy, 1e-6, want_dgamma=False, want_dbeta=False)
+    dx = np.zeros_like(x)
+    ref.rmsnorm_backward_into(x, None, dy, 1e-6, dx, None)
+    assert_fp32_close(out["dx"], dx, "weightless rms dx")
+
+
+@pytest.mark.parametrize("kind", ["layer", "rms"])
+@pytest.mark.parametrize("shape,eps", NORM_SHAPES)
+def test_norm_backward_fp32(ctx, kind, shape, eps):
+    rng = _rng(4)
+    C = shape[-1]
+    x = rng.standard_normal(shape, dtype=np.float32)
+    gamma = (1 + 0.02 * rng.standard_normal(C)).astype(np.float32)
+    dy = rng.standard_normal(shape, dtype=np.float32)
+    out = G.norm_backward(ctx, KINDS[kind], x, gamma, dy, eps, want_dbeta=(kind == "layer"))
+    dx, dgamma, dbeta = _norm_ref_backward(kind, x, gamma, dy, eps)
+    assert_fp32_close(out["dx"], dx, f"{kind} dx {shape}")
+    # few rows: the CPU's sequential row sum is still within the fp32 tolerance
+    assert_fp32_close(out["dgamma"], dgamma, f"{kind} dgamma {shape}", rtol=1e-5, atol=2e-6)
+    if kind == "layer":
+        assert_fp32_close(out["dbeta"], dbeta, f"{kind} dbeta {shape}", rtol=1e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("kind", ["layer", "rms"])
+def test_norm_backward_accumulate_and_residual_grad(ctx, kind):
+    """CPU semantics: grads accumulate (backend.py:477-487); the fused residual
+    gradient is added in the same pass (metal_ops.metal:8164); dx2 mirrors dx."""
+    rng = _rng(7)
+    shape = (37, 384)
+    x = rng.standard_normal(shape, dtype=np.float32)
+    gamma = (1 + 0.02 * rng.standard_normal(384)).astype(np.float32)
+    dy = rng.standard_normal(shape, dtype=np.float32)
+    dx0 = rng.standard_normal(shape, dtype=np.float32)
+    dres = rng.standard_normal(shape, dtype=np.float32)
+    dg0 = rng.standard_normal(384).astype(np.float32)
+    db0 = rng.standard_normal(384).astype(np.float32)
+    eps = 1e-5
+    flags = capi.ACC_INPUT_GRAD | capi.ACC_PARAM_GRAD
+    out = G.norm_backward(ctx, KINDS[kind], x, gamma, dy, eps, dres=dres, dx_init=dx0, want_dx2=True,
+                          dgamma_init=dg0, dbeta_init=db0, want_dbeta=(kind == "layer"), flags=flags)
+    dx, dgamma, dbeta = _norm_ref_backward(kind, x, gamma, dy, eps)
+    want = (dx0 + dres) + dx
+    assert_fp32_close(out["dx"], want, "accumulated dx", rtol=1e-5, atol=2e-6)
+    np.testing.assert_array_equal(out["dx"], out["dx2"])
+    assert_fp32_close(out["dgamma"], dg0 + dgamma, "accumulated dgamma", rtol=1e-5, atol=3e-6)
+    if kind == "layer":
+        assert_fp32_close(out["dbeta"], db0 + dbeta, "accumulated dbeta", rtol=1e-5, atol=3e-6)
+    # overwrite mode with a residual gradient and no accumulate
+    out = G.norm_backward(ctx, KINDS[kind], x, gamma, dy, eps, dres=dres, want_dgamma=False, want_dbeta=False)
+    assert_fp32_close(out["dx"], dres + dx, "dres + dx", rtol=1e-5, atol=2e-6)
+    # parameter grads only
+    out = G.norm_backward(ctx, KINDS[kind], x, gamma, dy, eps, want_dx=False, want_dbeta=(kind == "layer"))
+    assert out["dx"] is None
+    assert_fp32_close(out["dgamma"], dgamma, "dgamma only", rtol=1e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("kind,C,eps", [("layer", 384, 1e-5), ("layer", 768, 1e-5), ("rms", 1536, 1e-6)])
+def test_norm_backward_param_grads_many_rows(ctx, kind, C, eps):
+    """N = 16384 rows (configs 2-4).  The fp32 CPU result sums rows sequentially
+    and carries ~1e-4 of rounding noise, so the GPU is held to the float64 value
+    and must be at least as close to it as the CPU result is."""
+    rng = _rng(8)
+    N = 16384
+    x = rng.standard_normal((N, C), dtype=np.float32)
+    gamma = (1 + 0.02 * rng.standard_normal(C)).astype(np.float32)
+    dy = rng.standard_normal((N, C), dtype=np.float32)
+    out = G.norm_backward(ctx, KINDS[kind], x, gamma, dy, eps, want_dbeta=(kind == "layer"))
+    dx_cpu, dg_cpu, db_cpu = _norm_ref_backward(kind, x, gamma, dy, eps)
+    assert_fp32_close(out["dx"], dx_cpu, f"{kind} dx at N={N}")
+    if kind == "layer":
+        _, dg64, db64 = cf.layernorm_grads(x, gamma, dy, eps)
+    else:
+        _, dg64 = cf.rmsnorm_grads(x, gamma, dy, eps)
+        db64 = None
+    tol = 1e-6 * np.sqrt(N)
+    err_gpu = np.abs(out["dgamma"] - dg64).max()
+    err_cpu = np.abs(dg_cpu - dg64).max()
+    assert err_gpu <= tol, (err_gpu, tol)
+    assert err_gpu <= err_cpu + 1e-6, (err_gpu, err_cpu)
+    # and against the CPU restatement at the tolerance the reference's own
+    # checker uses for these sums (debug/check_qwen_kernel.py:128-130, atol 1e-4 scaled by sqrt(N/14))
+    assert_fp32_close(out["dgamma"], dg_cpu, "dgamma vs cpu", rtol=1e-5, atol=1e-4 * np.sqrt(N / 14))
+    if db64 is not None:
+        assert np.abs(out["dbeta"] - db64).max() <= tol
+        assert_fp32_close(out["dbeta"], db_cpu, "dbeta vs cpu", rtol=1e-5, atol=1e-4 * np.sqrt(N / 14))
+
+
+@pytest.mark.parametrize("kind", ["layer", "rms"])
+@pytest.mark.parametrize("C", [384, 1536, 4096, 50])
+def test_fused_residual_norm_forward(ctx, kind, C):
+    rng = _rng(9)
+    shape = (29, C)
+    x = rng.standard_normal(shape, dtype=np.float32)
+    r = rng.standard_normal(shape, dtype=np.float32)
+    gamma = (1 + 0.02 * rng.standard_normal(C)).astype(np.float32)
+    beta = (0.02 * rng.standard_normal(C)).astype(np.float32) if kind == "layer" else None
+    y, h = G.norm_forward(ctx, KINDS[kind], x, gamma, beta, 1e-5, residual=r, want_h=True)
+    h_ref, y_ref = ref.add_norm_forward(kind, x, r, gamma, beta, 1e-5)
+    np.testing.assert_array_equal(h, h_ref)   # a single fp32 add: bit-exact
+    assert_fp32_close(y, y_ref, f"add+{kind} forward")
+
+
+@pytest.mark.parametrize("kind", ["layer", "rms"])
+@pytest.mark.parametrize("C", [384, 1536, 4096, 8192, 72])
+def test_norm_bf16_io(ctx, kind, C):
+    rng = _rng(10)
+    shape = (23, C)
+    xb = to_bf16_bits(rng.standard_normal(shape, dtype=np.float32))
+    rb = to_bf16_bits(rng.standard_normal(shape, dtype=np.float32))
+    dyb = to_bf16_bits(rng.standard_normal(shape, dtype=np.float32))
+    gamma = (1 + 0.02 * rng.standard_normal(C)).astype(np.float32)
+    beta = (0.02 * rng.standard_normal(C)).astype(np.float32) if kind == "layer" else None
+    eps = 1e-5
+    x, r, dy = from_bf16_bits(xb), from_bf16_bits(rb), from_bf16_bits(dyb)
+    # forward, plain and with the residual fused
+    y, _ = G.norm_forward(ctx, KINDS[kind], xb, gamma, beta, eps)
+    assert_bf16_close(from_bf16_bits(y), _norm_ref_forward(kind, x, gamma, beta, eps), f"bf16 {kind} forward")
+    y, h = G.norm_forward(ctx, KINDS[kind], xb, gamma, beta, eps, residual=rb, want_h=True)
+    h_ref = ref.round_bf16(x + r)
+    np.testing.assert_array_equal(h, to_bf16_bits(x + r))
+    assert_bf16_close(from_bf16_bits(y), _norm_ref_forward(kind, h_ref, gamma, beta, eps), f"bf16 add+{kind}")
+    # backward
+    out = G.norm_backward(ctx, KINDS[kind], xb, gamma, dyb, eps, want_dbeta=(kind == "layer"))
+    dx, dgamma, dbeta = _norm_ref_backward(kind, x, gamma, dy, eps)
+    assert_bf16_close(from_bf16_bits(out["dx"]), dx, f"bf16 {kind} dx")
+    assert_fp32_close(out["dgamma"], dgamma, "bf16-io dgamma (fp32 accumulate)", rtol=1e-5, atol=2e-6)
+    if kind == "layer":
+        assert_fp32_close(out["dbeta"], dbeta, "bf16-io dbeta", rtol=1e-5, atol=2e-6)
+
+
+# ---------------------------------------------------------------------------
+# activations
+# ---------------------------------------------------------------------------
+ACT_SHAPES = [(2, 16, 64), (512, 512), (257, 1536), (3, 5, 7), (1,), (4099,)]
+
+
+@pytest.mark.parametrize("shape", ACT_SHAPES)
+def test_gelu_fp32(ctx, shape):
+    rng = _rng(5)
+    x = rng.standard_normal(shape, dtype=np.float32)
+    dy = rng.standard_normal(shape, dtype=np.float32)
+    assert_fp32_close(G.unary(ctx, "agrad_gelu_forward", x), ref.gelu_forward(x), f"gelu {shape}")
+    dx = np.zeros_like(x)
+    ref.gelu_backward_into(x, dy, dx)
+    assert_fp32_close(G.unary_backward(ctx, "agrad_gelu_backward", x, dy), dx, f"gelu bwd {shape}")
+    dx0 = rng.standard_normal(shape, dtype=np.float32)
+    acc = dx0.copy()
+    ref.gelu_backward_into(x, dy, acc)
+    got = G.unary_backward(ctx, "agrad_gelu_backward", x, dy, dx_init=dx0, flags=capi.ACC_INPUT_GRAD)
+    assert_fp32_close(got, acc, f"gelu bwd accumulate {shape}")
+
+
+def test_gelu_dense_sweep_and_special_values(ctx):
+    """tanhf on the device against np.tanh over [-10, 10], plus the limits."""
+    x = np.linspace(-10, 10, 2_000_001, dtype=np.float32)
+    got = G.unary(ctx, "agrad_gelu_forward", x)
+    assert_fp32_close(got, ref.gelu_forward(x), "gelu sweep")
+    assert np.abs(got - cf.gelu(x)).max() < 2e-6
+    one = np.ones_like(x)
+    dgot = G.unary_backward(ctx, "agrad_gelu_backward", x, one)
+    dref = np.zeros_like(x)
+    ref.gelu_backward_into(x, one, dref)
+    assert_fp32_close(dgot, dref, "gelu' sweep")
+    sp = np.array([0.0, -0.0, 30.0, -30.0, 1e-20, 80.0, -80.0], dtype=np.float32)
+    y = G.unary(ctx, "agrad_gelu_forward", sp)
+    assert y[0] == 0 and y[2] == 30.0 and y[3] == 0 and y[5] == 80.0 and y[6] == 0
+    d = G.unary_backward(ctx, "agrad_gelu_backward", sp, np.ones_like(sp))
+    assert d[0] == 0.5 and d[2] == 1.0 and d[3] == 0.0
+
+
+@pytest.mark.parametrize("shape", ACT_SHAPES)
+def test_relu2_fp32_bit_exact(ctx, shape):
+    rng = _rng(11)
+    x = rng.standard_normal(shape, dtype=np.float32)
+    dy = rng.standard_normal(shape, dtype=np.float32)
+    np.testing.assert_array_equal(G.unary(ctx, "agrad_relu2_forward", x), ref.relu2_forward(x))
+    dx = np.zeros_like(x)
+    ref.relu2_backward_into(x, dy, dx)
+    np.testing.assert_array_equal(G.unary_backward(ctx, "agrad_relu2_backward", x, dy) + 0.0, dx + 0.0)
+    # closed form: y = max(x,0)^2 and dx = 2 max(x,0) dy
+    assert np.abs(G.unary(ctx, "agrad_relu2_forward", x) - cf.relu2(x)).max() < 1e-6
+
+
+@pytest.mark.parametrize("rows,H", [(32, 64), (17, 8960), (5, 14336), (9, 50), (3, 1)])
+def test_swiglu_fp32(ctx, rows, H):
+    rng = _rng(12)
+    gu = rng.standard_normal((rows, 2 * H), dtype=np.float32) * 2
+    dh = rng.standard_normal((rows, H), dtype=np.float32)
+    assert_fp32_close(G.swiglu_forward(ctx, gu), ref.swiglu_forward(gu), f"swiglu {rows}x{H}")
+    want = ref.swiglu_backward(gu, dh)
+    assert_fp32_close(G.swiglu_backward(ctx, gu, dh, inplace=True), want, "swiglu bwd in place")
+    assert_fp32_close(G.swiglu_backward(ctx, gu, dh, inplace=False), want, "swiglu bwd out of place")
+    d0 = rng.standard_normal(gu.shape, dtype=np.float32)
+    got = G.swiglu_backward(ctx, gu, dh, inplace=False, dgu_init=d0, flags=capi.ACC_INPUT_GRAD)
+    assert_fp32_close(got, d0 + want, "swiglu bwd accumulate", rtol=1e-5, atol=2e-6)
+
+
+def test_swiglu_extremes(ctx):
+    g = np.array([[-100.0, -20.0, 0.0, 20.0, 100.0, -0.0]], dtype=np.float32)
+    u = np.full_like(g, 3.0)
+    gu = np.concatenate([g, u], axis=1)
+    got = G.swiglu_forward(ctx, gu)
+    assert_fp32_close(got, ref.swiglu_forward(gu), "swiglu extremes")
+    assert got[0, 2] == 0 and got[0, 4] == 300.0
+
+
+@pytest.mark.parametrize("name,fwd,bwd", [
+    ("gelu", ref.gelu_forward, ref.gelu_backward_into),
+    ("relu2", ref.relu2_forward, ref.relu2_backward_into)])
+def test_unary_bf16_io(ctx, name, fwd, bwd):
+    rng = _rng(13)
+    shape = (33, 1544)
+    xb = to_bf16_bits(rng.standard_normal(shape, dtype=np.float32))
+    dyb = to_bf16_bits(rng.standard_normal(shape, dtype=np.float32))
+    x, dy = from_bf16_bits(xb), from_bf16_bits(dyb)
+    y = G.unary(ctx, f"agrad_{name}_forward", xb)
+    if name == "relu2":   # exact fp32 arithmetic, one RNE on store
+        np.testing.assert_array_equal(y, to_bf16_bits(fwd(x)))
+    else:
+        assert_bf16_close(from_bf16_bits(y), fwd(x), f"bf16 {name}")
+    dx = np.zeros_like(x)
+    bwd(x, dy, dx)
+    got = G.unary_backward(ctx, f"agrad_{name}_backward", xb, dyb)
+    assert_bf16_close(from_bf16_bits(got), dx, f"bf16 {name} bwd")
+
+
+def test_swiglu_bf16_io(ctx):
+    rng = _rng(14)
+    rows, H = 19, 8960
+    gub = to_bf16_bits(rng.standard_normal((rows, 2 * H), dtype=np.float32))
+    dhb = to_bf16_bits(rng.standard_normal((rows, H), dtype=np.float32))
+    gu, dh = from_bf16_bits(gub), from_bf16_bits(dhb)
+    assert_bf16_close(from_bf16_bits(G.swiglu_forward(ctx, gub)), ref.swiglu_forward(gu), "bf16 swiglu")
+    assert_bf16_close(from_bf16_bits(G.swiglu_backward(ctx, gub, dhb)), ref.swiglu_backward(gu, dh), "bf16 swiglu bwd")
+
+
+# ---------------------------------------------------------------------------
+# RoPE
+# ---------------------------------------------------------------------------
+ROPE_CASES = [
+    # B, T, H, HKV, D, theta
+    (2, 16, 6, 6, 64, 1e4),      # config 2 heads
+    (2, 33, 12, 2, 128, 1e6),    # config 4 heads (GQA)
+    (1, 9, 32, 8, 128, 5e5),     # config 5 heads
+    (2, 5, 3, 1, 6, 1e4),        # D/2 = 3: scalar kernel
+]
+
+
+@pytest.mark.parametrize("B,T,H,HKV,D,theta", ROPE_CASES)
+@pytest.mark.parametrize("sign", [1, -1])
+@pytest.mark.parametrize("backward", [False, True])
+def test_rope_fp32_bit_exact(ctx, B, T, H, HKV, D, theta, sign, backward):
+    rng = _rng(15)
+    q = rng.standard_normal((B, T, H, D), dtype=np.float32)
+    k = rng.standard_normal((B, T, HKV, D), dtype=np.float32)
+    cos, sin = ref.rope_tables(T, D, theta)
+    gq, gk = G.rope(ctx, q, k, cos, sin, sign, backward)
+    rq, rk = q.copy(), k.copy()
+    ref.rope_signed(rq, rk, cos, sin, sign, backward)
+    # separate fp32 multiplies and adds in the reference's order: identical bits
+    np.testing.assert_array_equal(gq, rq)
+    np.testing.assert_array_equal(gk, rk)
+    if sign == -1:
+        nq, nk = q.copy(), k.copy()
+        ref.rope_nanochat(nq, nk, cos, sin, backward)
+        np.testing.assert_array_equal(gq, nq)
+        np.testing.assert_array_equal(gk, nk)
+
+
+def test_rope_invariants(ctx):
+    rng = _rng(16)
+    B, T, H, HKV, D = 2, 64, 12, 2, 128
+    q = rng.standard_normal((B, T, H, D), dtype=np.float32)
+    k = rng.standard_normal((B, T, HKV, D), dtype=np.float32)
+    cos, sin = ref.rope_tables(T, D, 1e6)
+    fq, fk = G.rope(ctx, q, k, cos, sin, 1, False)
+    # position 0 is the identity; the rotation preserves each (lo, hi) pair's norm
+    np.testing.assert_array_equal(fq[:, 0], q[:, 0])
+    half = D // 2
+    n0 = q[..., :half] ** 2 + q[..., half:] ** 2
+    n1 = fq[..., :half] ** 2 + fq[..., half:] ** 2
+    assert np.abs(n1 - n0).max() < 1e-5
+    # backward undoes forward; the two sign conventions are mutual inverses
+    bq, bk = G.rope(ctx, fq, fk, cos, sin, 1, True)
+    assert np.abs(bq - q).max() < 1e-6 and np.abs(bk - k).max() < 1e-6
+    iq, _ = G.rope(ctx, fq, fk, cos, sin, -1, False)
+    np.testing.assert_array_equal(iq, bq)
+    # q only
+    oq, ok = G.rope(ctx, q, None, cos, sin, 1, False)
+    np.testing.assert_array_equal(oq, fq)
+    assert ok is None
+    # float64 closed form
+    assert np.abs(fq - cf.rope(q, cos, sin, 1)).max() < 1e-6
+
+
+def test_rope_bf16_io(ctx):
+    rng = _rng(17)
+    B, T, H, HKV, D = 2, 31, 12, 2, 128
+    qb = to_bf16_bits(rng.standard_normal((B, T, H, D), dtype=np.float32))
+    kb = to_bf16_bits(rng.standard_normal((B, T, HKV, D), dtype=np.float32))
+    cos, sin = ref.rope_tables(T, D, 1e6)
+    gq, gk = G.rope(ctx, qb, kb, cos, sin, 1, False)
+    rq, rk = from_bf16_bits(qb), from_bf16_bits(kb)
+    ref.rope_signed(rq, rk, cos, sin, 1, False)
+    np.testing.assert_array_equal(gq, to_bf16_bits(rq))  # fp32 math is exact; one RNE on store
+    np.testing.assert_array_equal(gk, to_bf16_bits(rk))
+
+
+# ---------------------------------------------------------------------------
+# embedding
+# ---------------------------------------------------------------------------
+def test_gather_reference_case(ctx):
+    """verify_model.py:298-318: B,T,V,C = 2,3,11,4, seed 1234, w = 0.1 N(0,1)."""
+    rng = np.random.default_rng(1234)
+    B, T, V, C = 2, 3, 11, 4
+    idx = rng.integers(0, V, size=(B, T), dtype=np.int32)
+    w = (rng.standard_normal((V, C)) * 0.1).astype(np.float32)
+    got = G.gather_forward(ctx, idx, w)
+    np.testing.assert_array_equal(got.view(np.uint32), w[idx].view(np.uint32))
+    up = rng.standard_normal((B, T, C)).astype(np.float32)
+    dW = np.zeros_like(w)
+    ref.gather_backward_into(idx, up, dW)
+    np.testing.assert_array_equal(G.embedding_backward(ctx, idx, up, V), dW)
+
+
+@pytest.mark.parametrize("B,T,V,C", [(4, 128, 50257, 128), (3, 37, 1000, 384), (2, 50, 300, 768),
+                                     (2, 9, 97, 1536), (2, 7, 53, 50), (1, 1, 1, 4)])
+def test_gather_forward_bit_exact(ctx, B, T, V, C):
+    rng = _rng(18)
+    ids = rng.integers(0, V, size=(B, T), dtype=np.int32)
+    W = (0.02 * rng.standard_normal((V, C))).astype(np.float32)
+    W.reshape(-1)[:3] = [np.nan, -0.0, np.inf]          # payloads must survive the copy
+    ids.reshape(-1)[0] = 0
+    got = G.gather_forward(ctx, ids, W)
+    np.testing.assert_array_equal(got.view(np.uint32), ref.gather_forward(ids, W).view(np.uint32))
+    Wb = to_bf16_bits(W)
+    np.testing.assert_array_equal(G.gather_forward(ctx, ids, Wb), Wb[ids])
+
+
+@pytest.mark.parametrize("B,T,V,C", [(4, 128, 50257, 128), (3, 37, 1000, 768), (2, 7, 53, 50)])
+def test_embedding_sum_forward(ctx, B, T, V, C):
+    rng = _rng(19)
+    ids = rng.integers(0, V, size=(B, T), dtype=np.int32)
+    wte = (0.02 * rng.standard_normal((V, C))).astype(np.float32)
+    wpe = (0.02 * rng.standard_normal((T, C))).astype(np.float32)
+    got = G.gather_forward(ctx, ids, wte, wpe)
+    np.testing.assert_array_equal(got, ref.embedding_sum_forward(ids, wte, wpe))  # one fp32 add
+
+
+def test_gather_out_of_range_id_raises(ctx):
+    ids = np.array([[0, 5, 11]], dtype=np.int32)
+    W = np.ones((11, 8), np.float32)
+    with pytest.raises(IndexError):
+        G.gather_forward(ctx, ids, W)
+    with pytest.raises(IndexError):
+        G.embedding_backward(ctx, np.array([[0, -1]], np.int32), np.ones((1, 2, 8), np.float32), 11)
+    # the context stays usable
+    np.testing.assert_array_equal(G.gather_forward(ctx, np.array([[1, 2]], np.int32), W), W[[[1, 2]]])
+
+
+def _zipf_ids(rng, n, V, s=1.1):
+    p = np.arange(1, V + 1, dtype=np.float64) ** (-s)
+    p /= p.sum()
+    return rng.choice(V, size=n, p=p).astype(np.int32)
+
+
+@pytest.mark.parametrize("B,T,V,C,dist", [
+    (2, 16, 64, 64, "uniform"),
+    (4, 128, 50257, 128, "uniform"),      # config 1
+    (8, 512, 32768, 384, "uniform"),      # config 2 at a quarter of its rows
+    (3, 700, 97, 50, "uniform"),          # heavy duplication, scalar columns
+    (4, 1024, 1000, 768, "zipf"),         # long runs crossing chunk edges
+    (1, 3000, 1, 16, "uniform"),          # a single token: one run over every chunk
+])
+def test_embedding_backward_fp32(ctx, B, T, V, C, dist):
+    rng = _rng(20)
+    ids = (_zipf_ids(rng, B * T, V) if dist == "zipf" else rng.integers(0, V, size=B * T, dtype=np.int32)).reshape(B, T)
+    dY = rng.standard_normal((B, T, C), dtype=np.float32)
+    got = G.embedding_backward(ctx, ids, dY, V)
+    dW = np.zeros((V, C), np.float32)
+    ref.gather_backward_into(ids, dY, dW)
+    assert_fp32_close(got, dW, f"embedding backward {dist}", rtol=1e-5, atol=2e-6 if dist == "uniform" and V > 1 else 1e-4)
+    # rows of tokens that never occur stay exactly zero; column sums are preserved
+    unseen = np.setdiff1d(np.arange(V), ids.ravel())
+    assert not got[unseen].any()
+    assert np.abs(got.sum(0, dtype=np.float64) - dY.reshape(-1, C).sum(0, dtype=np.float64)).max() < 1e-3 * np.sqrt(B * T)
+    # against the float64 row loop, on the scale of the sum
+    d64 = cf.gather_backward(ids, dY, V)
+    assert np.abs(got - d64).max() <= 1e-6 * max(1.0, np.abs(d64).max()) * 8
+    # deterministic: a second run gives the same bits
+    np.testing.assert_array_equal(got, G.embedding_backward(ctx, ids, dY, V))
+    # accumulate onto an existing table
+    base = rng.standard_normal((V, C), dtype=np.float32)
+    acc = G.embedding_backward(ctx, ids, dY, V, dW_init=base, flags=capi.ACC_PARAM_GRAD)
+    assert_fp32_close(acc, base + dW, "embedding backward accumulate", rtol=1e-5, atol=1e-4)
+    np.testing.assert_array_equal(acc[unseen], base[unseen])
+
+
+def test_embedding_backward_short_runs_bit_exact(ctx):
+    """Runs that fit inside one chunk are summed in ascending row order: the
+    same sequence of fp32 adds as np.add.at."""
+    rng = _rng(21)
+    V, C, N = 4096, 128, 512
+    # every token occurs exactly four times, so sorted runs start at multiples of
+    # four and never straddle a chunk of eight positions
+    toks = rng.choice(V, size=N // 4, replace=False).astype(np.int32)
+    ids = rng.permutation(np.repeat(toks, 4)).reshape(1, N)
+    dY = rng.standard_normal((1, N, C), dtype=np.float32)
+    got = G.embedding_backward(ctx, ids, dY, V)
+    dW = np.zeros((V, C), np.float32)
+    ref.gather_backward_into(ids, dY, dW)
+    np.testing.assert_array_equal(got, dW)
+
+
+def test_embedding_backward_bf16_io(ctx):
+    rng = _rng(22)
+    B, T, V, C = 4, 256, 5000, 1536
+    ids = rng.integers(0, V, size=(B, T), dtype=np.int32)
+    dYb = to_bf16_bits(rng.standard_normal((B, T, C), dtype=np.float32))
+    got = G.embedding_backward(ctx, ids, dYb, V)
+    dW = np.zeros((V, C), np.float32)
+    ref.gather_backward_into(ids, from_bf16_bits(dYb), dW)
+    assert_bf16_close(from_bf16_bits(got), dW, "bf16 embedding backward")
+
+
+@pytest.mark.parametrize("B,T,C", [(4, 128, 128), (16, 64, 768), (3, 5, 7)])
+def test_pos_embedding_backward(ctx, B, T, C):
+    rng = _rng(23)
+    dY = rng.standard_normal((B, T, C), dtype=np.float32)
+    ids = rng.integers(0, 10, size=(B, T), dtype=np.int32)
+    dwpe = np.zeros((T, C), np.float32)
+    ref.embedding_sum_backward_into(ids, dY, None, dwpe)
+    np.testing.assert_array_equal(G.pos_embedding_backward(ctx, dY), dwpe)  # b ascending: same adds
+    base = rng.standard_normal((T, C), dtype=np.float32)
+    got = G.pos_embedding_backward(ctx, dY, dwpe_init=base, flags=capi.ACC_PARAM_GRAD)
+    assert_fp32_close(got, base + dwpe, "pos grad accumulate")
