@@ -1,0 +1,521 @@
+"""Backend of the "hip" device: binds each layer op to a gfx950 kernel.
+
+Counterpart of the reference's Backend / MetalBackend (backend.py:22-69,
+2611-2955, 4938-5113) for the fused layer-op path.  The contract is the
+reference's:
+
+  * a bound kernel is `fn(inputs, outputs, scratch=None)`, looked up by the
+    exact type of the op in `forward_kernels` / `backward_kernels`
+    (backend.py:4938-4950) and stored on `OpNode.forward / .backward`;
+  * op attributes are read through `out.op.op.<attr>` (backend.py:2916);
+  * backward kernels return early when `out.grad` is None, read `out.grad` and
+    write `x.grad.storage`;
+  * every launch is `ctx.dispatch_with_args_3d(name, buffer_ids, offsets,
+    uint32 args, gx, gy, gz, tg)` with floats passed as bit patterns
+    (backend.py:2911-2920).
+
+Differences, all on the CPU side of the reference's own CPU/Metal split:
+backward kernels accumulate into existing gradients like the CPU kernels do
+(backend.py:414, 477-487) unless the runtime marked this node as the first
+writer of a gradient in the pass, in which case they store; LayerNorm backward
+honours the op's eps; launch geometry is chosen by the native library, so the
+grid arguments are passed as zeros.
+
+There is no CPU fallback: every kernel here ends in a HIP launch.
+"""
+from __future__ import annotations
+
+from math import prod
+
+import numpy as np
+
+from .op import (AddLayerNormOp, AddOp, AddRMSNormOp, EmbeddingSumOp, GatherOp, GELUOp, LayerNormOp,
+                 ReLUSquaredOp, RMSNormOp, RopeOp, SwiGLUOp)
+from .scratch import single_slot
+from .utils import (bf16_bits, bf16_bits_to_f32_array, f32_array_to_bf16_bits, f32_bits, is_bf16,
+                    xavier_uniform)
+
+F32, BF16 = 0, 1
+ACC_INPUT_GRAD, ACC_PARAM_GRAD = 1, 2
+
+
+class Backend:
+    mixed_precision = False
+
+    def get_forward_kernel(self, op):
+        raise NotImplementedError()
+
+    def get_backward_kernel(self, op):
+        raise NotImplementedError()
+
+    def fill_storage(self, storage, value):
+        raise NotImplementedError()
+
+    def fill_storage2(self, storage, value):
+        raise NotImplementedError()
+
+    def fill_scalar(self, tensor, value):
+        self.fill_storage(tensor.storage, float(value))
+
+    def fill(self, tensor, value):
+        self.fill_scalar(tensor, float(value))
+
+    def init(self, tensor):
+        """materialise tensor.init_val: number, ndarray, "xavier" or "zeros" (backend.py:43-59)"""
+        v = tensor.init_val
+        if v is None:
+            return
+        try:
+            if isinstance(v, (int, float)):
+                self.fill_scalar(tensor, float(v))
+            elif isinstance(v, np.ndarray):
+                self.copy_from_host(tensor, v)
+            elif v == "xavier":
+                self.copy_from_host(tensor, xavier_uniform(tensor.shape, np.float32))
+            elif v == "zeros":
+                self.fill_scalar(tensor, 0.0)
+            else:
+                raise ValueError(f"unknown init_val: {v!r}")
+        finally:
+            tensor.init_val = None
+
+    def plan_scratch(self, node):
+        """(forward layout, backward layout) of scratch this backend's kernels need"""
+        return None, None
+
+    def begin_pass(self):
+        pass
+
+    def end_pass(self):
+        pass
+
+    def synchronize(self):
+        pass
+
+
+def _dt(t):
+    if is_bf16(t.dtype):
+        return BF16
+    if np.dtype(t.dtype) == np.dtype(np.float32):
+        return F32
+    raise RuntimeError(f"hip backend: unsupported dtype {t.dtype}")
+
+
+def _ids(*tensors_or_storages):
+    ids, offs = [], []
+    for s in tensors_or_storages:
+        if s is None:
+            ids.append(0)
+            offs.append(0)
+            continue
+        st = s.storage if hasattr(s, "storage") else s
+        ids.append(st.ptr.buffer_id)
+        offs.append(st.ptr.offset)
+    return ids, offs
+
+
+def _lo_hi(n):
+    return [n & 0xFFFFFFFF, (n >> 32) & 0xFFFFFFFF]
+
+
+def _mask(*present):
+    m = 0
+    for i, p in enumerate(present):
+        if p is not None:
+            m |= 1 << i
+    return m
+
+
+class HipBackend(Backend):
+    supports_grad_store = True   # kernels take a store / accumulate flag per gradient
+
+    def __init__(self, ctx=None):
+        if ctx is None:
+            from .device import hip_context
+            ctx = hip_context()
+        self.ctx = ctx
+        self.grad_scale = 1.0
+        self.accumulate_parameter_grads = False
+        self.use_fp16_gemm = False
+        self.forward_kernels = {
+            AddOp: self.hip_add_forward,
+            GatherOp: self.hip_gather_forward,
+            EmbeddingSumOp: self.hip_embedding_sum_forward,
+            GELUOp: self.hip_gelu_forward,
+            ReLUSquaredOp: self.hip_relu2_forward,
+            SwiGLUOp: self.hip_swiglu_forward,
+            LayerNormOp: self.hip_layernorm_forward,
+            RMSNormOp: self.hip_rmsnorm_forward,
+            AddLayerNormOp: self.hip_add_norm_forward,
+            AddRMSNormOp: self.hip_add_norm_forward,
+            RopeOp: self.hip_rope_forward,
+        }
+        self.backward_kernels = {
+            AddOp: self.hip_add_backward,
+            GatherOp: self.hip_gather_backward,
+            EmbeddingSumOp: self.hip_embedding_sum_backward,
+            GELUOp: self.hip_gelu_backward,
+            ReLUSquaredOp: self.hip_relu2_backward,
+            SwiGLUOp: self.hip_swiglu_backward,
+            LayerNormOp: self.hip_layernorm_backward,
+            RMSNormOp: self.hip_rmsnorm_backward,
+            AddLayerNormOp: self.hip_add_norm_backward,
+            AddRMSNormOp: self.hip_add_norm_backward,
+            RopeOp: self.hip_rope_backward,
+        }
+
+    # -- lookup (backend.py:4938-4950) -------------------------------------------
+    def get_forward_kernel(self, op):
+        return self.forward_kernels.get(type(op))
+
+    def get_backward_kernel(self, op):
+        return self.backward_kernels.get(type(op))
+
+    def bind_add_forward(self, node):
+        return self.hip_add_forward
+
+    def bind_add_backward(self, node):
+        return self.hip_add_backward
+
+    def _launch(self, name, tensors, args):
+        ids, offs = _ids(*tensors)
+        self.ctx.dispatch_with_args_3d(name, ids, offs, [int(a) & 0xFFFFFFFF for a in args], 0, 0, 0, 0)
+
+    # -- gradient write mode -------------------------------------------------------
+    def _input_flag(self, node, t):
+        return 0 if id(t.grad) in node.overwrite_grads else ACC_INPUT_GRAD
+
+    def _param_flag(self, node, *params):
+        if self.accumulate_parameter_grads:
+            return ACC_PARAM_GRAD
+        live = [p for p in params if p is not None and p.requires_grad and p.grad is not None]
+        if live and all(id(p.grad) in node.overwrite_grads for p in live):
+            return 0
+        return ACC_PARAM_GRAD
+
+    def _grad_flag(self, node, t):
+        """flag for a gradient that may belong to a parameter or an activation"""
+        if t.op is None:
+            return ACC_INPUT_GRAD if self._param_flag(node, t) else 0
+        return self._input_flag(node, t)
+
+    # -- scratch -----------------------------------------------------------------
+    def plan_scratch(self, node):
+        op = node.op
+        if isinstance(op, (LayerNormOp, RMSNormOp, AddLayerNormOp, AddRMSNormOp)):
+            first_param = 2 if isinstance(op, (AddLayerNormOp, AddRMSNormOp)) else 1
+            if any(p.requires_grad for p in node.inputs[first_param:]):
+                x = node.inputs[0]
+                rows, C = prod(x.shape[:-1]), x.shape[-1]
+                return None, single_slot("workspace", self.ctx.norm_backward_workspace_bytes(rows, C, _dt(x)))
+        if isinstance(op, (GatherOp, EmbeddingSumOp)):
+            ids, w = node.inputs[0], node.inputs[1]
+            if w.requires_grad:
+                nbytes = self.ctx.embedding_backward_workspace_bytes(prod(ids.shape), w.shape[1], w.shape[0], _dt(w))
+                return None, single_slot("workspace", nbytes)
+        return None, None
+
+    # -- Add (cpu_add_forward / cpu_add_backward, backend.py:74-105) ----------------
+    def hip_add_forward(self, inputs, outputs, scratch=None):
+        x, y, out = inputs[0], inputs[1], outputs[0]
+        if x.shape != y.shape:
+            raise RuntimeError(f"Unsupported Add shape: x.shape={x.shape}, y.shape={y.shape}")
+        self._launch("add_residual_forward", [x, y, out], [_dt(out)] + _lo_hi(out.numel))
+
+    def hip_add_backward(self, inputs, outputs, scratch=None):
+        out = outputs[0]
+        if out.grad is None:
+            return
+        node = out.op
+        for t in inputs[:2]:
+            if not t.requires_grad or t.grad is None:
+                continue
+            if t.shape == out.shape:
+                self._launch("add_residual_backward", [out.grad, t.grad],
+                             [_dt(out), self._grad_flag(node, t)] + _lo_hi(out.numel))
+            elif out.shape[len(out.shape) - t.ndim:] == t.shape:
+                lead = prod(out.shape[:len(out.shape) - t.ndim])
+                flag = ACC_PARAM_GRAD if self._grad_flag(node, t) else 0
+                self._launch("pos_emb_grad", [out.grad, t.grad], [_dt(out), lead, 1, t.numel, flag])
+            else:
+                raise RuntimeError(f"Unsupported Add backward shape: {t.shape} from {out.shape}")
+
+    # -- embedding (backend.py:525-538, 2777-2815) ----------------------------------
+    def hip_gather_forward(self, inputs, outputs, scratch=None):
+        indices, weight, out = inputs[0], inputs[1], outputs[0]
+        V, C = weight.shape
+        self._launch("gather_forward_kernel", [indices, weight, out], [_dt(weight), prod(indices.shape), C, V])
+
+    def _embedding_grad(self, node, indices, weight, out, scratch):
+        if scratch is None:
+            raise RuntimeError("embedding backward needs its arena workspace (plan_scratch)")
+        ws = scratch["workspace"]
+        V, C = weight.shape
+        self._launch("gather_backward_kernel", [indices, out.grad, weight.grad, ws],
+                     [_dt(weight), prod(indices.shape), C, V, self._param_flag(node, weight)] + _lo_hi(ws.nbytes))
+
+    def hip_gather_backward(self, inputs, outputs, scratch=None):
+        indices, weight, out = inputs[0], inputs[1], outputs[0]
+        if out.grad is None or not weight.requires_grad:
+            return
+        self._embedding_grad(out.op, indices, weight, out, scratch)
+
+    def hip_embedding_sum_forward(self, inputs, outputs, scratch=None):
+        indices, wte, wpe = inputs
+        out = outputs[0]
+        V, C = wte.shape
+        B, T = indices.shape
+        self._launch("embedding_sum_forward", [indices, wte, wpe, out], [_dt(wte), B * T, T, C, V])
+
+    def hip_embedding_sum_backward(self, inputs, outputs, scratch=None):
+        indices, wte, wpe = inputs
+        out = outputs[0]
+        if out.grad is None:
+            return
+        B, T = indices.shape
+        if wte.requires_grad:
+            self._embedding_grad(out.op, indices, wte, out, scratch)
+        if wpe.requires_grad:
+            # rows beyond T of a longer table get no gradient
+            self._launch("pos_emb_grad", [out.grad, wpe.grad],
+                         [_dt(out), B, T, wpe.shape[1], self._param_flag(out.op, wpe)])
+
+    # -- activations ------------------------------------------------------------------
+    def _unary_forward(self, kernel, inputs, outputs):
+        x, out = inputs[0], outputs[0]
+        self._launch(kernel, [x, out], [_dt(x)] + _lo_hi(x.numel))
+
+    def _unary_backward(self, kernel, inputs, outputs):
+        x, out = inputs[0], outputs[0]
+        if out.grad is None or not x.requires_grad:
+            return
+        self._launch(kernel, [out.grad, x, x.grad], [_dt(x), self._grad_flag(out.op, x)] + _lo_hi(x.numel))
+
+    def hip_gelu_forward(self, inputs, outputs, scratch=None):
+        self._unary_forward("gelu_forward_kernel", inputs, outputs)
+
+    def hip_gelu_backward(self, inputs, outputs, scratch=None):
+        self._unary_backward("gelu_backward_kernel", inputs, outputs)
+
+    def hip_relu2_forward(self, inputs, outputs, scratch=None):
+        self._unary_forward("relu2_forward_kernel", inputs, outputs)
+
+    def hip_relu2_backward(self, inputs, outputs, scratch=None):
+        self._unary_backward("relu2_backward_kernel", inputs, outputs)
+
+    def hip_swiglu_forward(self, inputs, outputs, scratch=None):
+        gu, out = inputs[0], outputs[0]
+        H = out.shape[-1]
+        self._launch("swiglu_forward_kernel", [gu, out], [_dt(gu), prod(out.shape[:-1]), H])
+
+    def hip_swiglu_backward(self, inputs, outputs, scratch=None):
+        gu, out = inputs[0], outputs[0]
+        if out.grad is None or not gu.requires_grad:
+            return
+        H = out.shape[-1]
+        self._launch("swiglu_backward_kernel", [gu, out.grad, gu.grad],
+                     [_dt(gu), prod(out.shape[:-1]), H, self._grad_flag(out.op, gu)])
+
+    # -- norms ----------------------------------------------------------------------
+    def _norm_forward(self, kernel, x, residual, gamma, beta, h, y, eps):
+        rows, C = prod(x.shape[:-1]), x.shape[-1]
+        self._launch(kernel, [x, residual, gamma, beta, h, y],
+                     [_dt(x), rows, C, f32_bits(eps), _mask(x, residual, gamma, beta, h, y)])
+
+    def _norm_backward(self, kernel, node, x_saved, dy, gamma, beta, dres, dx, dx2, eps, flags, scratch):
+        rows, C = prod(x_saved.shape[:-1]), x_saved.shape[-1]
+        dgamma = gamma.grad if gamma is not None and gamma.requires_grad else None
+        dbeta = beta.grad if beta is not None and beta.requires_grad else None
+        ws = None
+        if dgamma is not None or dbeta is not None:
+            if scratch is None:
+                raise RuntimeError("norm backward needs its arena workspace (plan_scratch)")
+            ws = scratch["workspace"]
+        if dx is None and dgamma is None and dbeta is None:
+            return
+        self._launch(kernel, [x_saved, dy, gamma, dres, dx, dx2, dgamma, dbeta, ws],
+                     [_dt(x_saved), rows, C, f32_bits(eps), flags,
+                      _mask(x_saved, dy, gamma, dres, dx, dx2, dgamma, dbeta, ws)]
+                     + _lo_hi(ws.nbytes if ws is not None else 0))
+
+    def hip_layernorm_forward(self, inputs, outputs, scratch=None):
+        x, gamma, beta = inputs
+        self._norm_forward("layernorm_forward", x, None, gamma, beta, None, outputs[0], outputs[0].op.op.eps)
+
+    def hip_layernorm_backward(self, inputs, outputs, scratch=None):
+        x, gamma, beta = inputs
+        out = outputs[0]
+        if out.grad is None:
+            return
+        node = out.op
+        dx = x.grad if x.requires_grad else None
+        flags = (self._grad_flag(node, x) if dx is not None else 0) | self._param_flag(node, gamma, beta)
+        self._norm_backward("layernorm_backward_kernel", node, x, out.grad, gamma, beta, None, dx, None,
+                            node.op.eps, flags, scratch)
+
+    def hip_rmsnorm_forward(self, inputs, outputs, scratch=None):
+        x = inputs[0]
+        gamma = inputs[1] if len(inputs) > 1 else None
+        self._norm_forward("rmsnorm_forward", x, None, gamma, None, None, outputs[0], outputs[0].op.op.eps)
+
+    def hip_rmsnorm_backward(self, inputs, outputs, scratch=None):
+        x = inputs[0]
+        gamma = inputs[1] if len(inputs) > 1 else None
+        out = outputs[0]
+        if out.grad is None:
+            return
+        node = out.op
+        dx = x.grad if x.requires_grad else None
+        flags = (self._grad_flag(node, x) if dx is not None else 0) | self._param_flag(node, gamma)
+        self._norm_backward("rmsnorm_backward", node, x, out.grad, gamma, None, None, dx, None,
+                            node.op.eps, flags, scratch)
+
+    def hip_add_norm_forward(self, inputs, outputs, scratch=None):
+        x, res = inputs[0], inputs[1]
+        h, y = outputs
+        op = h.op.op
+        if isinstance(op, AddLayerNormOp):
+            self._norm_forward("layernorm_forward", x, res, inputs[2], inputs[3], h, y, op.eps)
+        else:
+            gamma = inputs[2] if len(inputs) > 2 else None
+            self._norm_forward("rmsnorm_forward", x, res, gamma, None, h, y, op.eps)
+
+    def hip_add_norm_backward(self, inputs, outputs, scratch=None):
+        """dh_total = h.grad + norm_backward(y.grad); both operands of the add
+        receive dh_total (cpu_add_backward, backend.py:78-105)."""
+        x, res = inputs[0], inputs[1]
+        h, y = outputs
+        node = h.op
+        op = node.op
+        is_ln = isinstance(op, AddLayerNormOp)
+        gamma = inputs[2] if len(inputs) > 2 else None
+        beta = inputs[3] if is_ln else None
+        kernel = "layernorm_backward_kernel" if is_ln else "rmsnorm_backward"
+        if y.grad is None:
+            # only the residual stream carries gradient: plain add backward
+            if h.grad is not None:
+                for t in (x, res):
+                    if t.requires_grad and t.grad is not None:
+                        self._launch("add_residual_backward", [h.grad, t.grad],
+                                     [_dt(h), self._grad_flag(node, t)] + _lo_hi(h.numel))
+            return
+        targets = [t for t in (x, res) if t.requires_grad and t.grad is not None]
+        dres = h.grad                      # may be None when nothing else consumed h
+        pflags = self._param_flag(node, gamma, beta)
+        if not targets:
+            self._norm_backward(kernel, node, h, y.grad, gamma, beta, None, None, None, op.eps, pflags, scratch)
+            return
+        first, second = targets[0], (targets[1] if len(targets) > 1 else None)
+        f1 = self._grad_flag(node, first)
+        if second is not None and self._grad_flag(node, second) == 0 and f1 == 0:
+            # both operands take a plain store: one launch writes both
+            self._norm_backward(kernel, node, h, y.grad, gamma, beta, dres, first.grad, second.grad,
+                                op.eps, pflags, scratch)
+            return
+        if second is None:
+            self._norm_backward(kernel, node, h, y.grad, gamma, beta, dres, first.grad, None,
+                                op.eps, f1 | pflags, scratch)
+            return
+        # mixed write modes: form dh_total in h.grad's place, then hand it on
+        if dres is None:
+            raise RuntimeError("fused add+norm backward: residual gradient buffer missing")
+        self._norm_backward(kernel, node, h, y.grad, gamma, beta, dres, dres, None, op.eps, pflags, scratch)
+        for t in targets:
+            self._launch("add_residual_backward", [dres, t.grad],
+                         [_dt(h), self._grad_flag(node, t)] + _lo_hi(h.numel))
+
+    # -- rotary (backend.py:1382-1417, 1755-1782, 1937-1958) ----------------------------
+    def _rope(self, q, k, cos, sin, sign, backward):
+        B, T, H, D = q.shape
+        HKV = k.shape[2] if k is not None else 0
+        self._launch("rope_qk_inplace", [q, k, cos, sin],
+                     [_dt(q), B, T, H, HKV, D, 1 if sign == 1 else 0, 1 if backward else 0, _mask(q, k)])
+
+    @staticmethod
+    def _same_memory(a, b):
+        return (a.storage.ptr.buffer_id, a.storage.ptr.offset) == (b.storage.ptr.buffer_id, b.storage.ptr.offset)
+
+    def hip_rope_forward(self, inputs, outputs, scratch=None):
+        """The kernel rotates in place.  When the runtime could alias an output
+        with its input they are one buffer; otherwise (a leaf input, or one that
+        is read elsewhere) the input is copied first."""
+        q, k, cos, sin = inputs
+        q2, k2 = outputs
+        for a, b in ((q, q2), (k, k2)):
+            if not self._same_memory(a, b):
+                self._launch("copy_kernel", [a, b], _lo_hi(b.storage.nbytes))
+        self._rope(q2, k2, cos, sin, q2.op.op.rope_sign, False)
+
+    def hip_rope_backward(self, inputs, outputs, scratch=None):
+        q, k, cos, sin = inputs
+        q2, k2 = outputs
+        gq = q2.grad if q.requires_grad else None
+        gk = k2.grad if k.requires_grad else None
+        if gq is None and gk is None:
+            return
+        sign = q2.op.op.rope_sign
+        if gq is not None:
+            self._rope(gq, gk, cos, sin, sign, True)
+        else:
+            B, T, H, D = gk.shape
+            self._launch("rope_qk_inplace", [gk, None, cos, sin],
+                         [_dt(gk), B, T, H, 0, D, 1 if sign == 1 else 0, 1, _mask(gk, None)])
+        node = q2.op
+        for src, g in ((q, gq), (k, gk)):
+            if g is not None and src.grad is not None and not self._same_memory(src.grad, g):
+                self._launch("add_residual_backward", [g, src.grad],
+                             [_dt(src), self._grad_flag(node, src)] + _lo_hi(src.numel))
+
+    # -- fills and copies (backend.py:5069-5113) ---------------------------------------
+    def fill_storage(self, storage, value):
+        dt = np.dtype(storage.dtype)
+        n = prod(storage.shape)
+        if dt == np.dtype(np.float32):
+            self.ctx.fill_scalar("fill_scalar_kernel", [storage.ptr.buffer_id], [storage.ptr.offset], float(value), n)
+        else:
+            self.fill_storage2(storage, value)
+
+    def fill_storage2(self, storage, value):
+        dt = np.dtype(storage.dtype)
+        if dt == np.dtype(np.uint16):
+            bits = bf16_bits(value)
+        elif dt == np.dtype(np.float32):
+            bits = f32_bits(value)
+        elif dt.kind in "iu":
+            bits = int(value) & (0xFFFFFFFF >> (8 * (4 - dt.itemsize))) if dt.itemsize <= 4 else None
+        else:
+            bits = None
+        if bits is None or dt.itemsize not in (1, 2, 4):
+            raise RuntimeError(f"fill: unsupported dtype {dt}")
+        self.ctx.fill_scalar2("fill_scalar_kernel2", [storage.ptr.buffer_id], [storage.ptr.offset],
+                              bits, dt.itemsize, prod(storage.shape))
+
+    def copy_from_host(self, tensor, host_np):
+        st = tensor.storage
+        dt = np.dtype(st.dtype)
+        host = np.asarray(host_np)
+        if dt == np.dtype(np.uint16) and host.dtype != np.dtype(np.uint16):
+            host = f32_array_to_bf16_bits(np.asarray(host, dtype=np.float32))
+        else:
+            host = np.ascontiguousarray(host, dtype=dt)
+        if host.size != prod(tensor.shape):
+            raise ValueError(f"copy_from_host: {host.shape} does not fill {tensor.shape}")
+        self.ctx.copy_from_host(st.ptr.buffer_id, st.ptr.offset, host.reshape(-1))
+
+    def copy_to_host(self, tensor):
+        """fp32 array for fp32 and bf16 tensors (bf16 is widened), raw otherwise"""
+        st = tensor.storage
+        dt = np.dtype(st.dtype)
+        raw = self.ctx.copy_to_host(st.ptr.buffer_id, st.ptr.offset, list(tensor.shape), dt.name)
+        if dt == np.dtype(np.uint16):
+            return bf16_bits_to_f32_array(raw).reshape(tensor.shape)
+        return raw
+
+    def begin_pass(self):
+        self.ctx.begin_pass()
+
+    def end_pass(self):
+        self.ctx.end_pass()
+
+    def synchronize(self):
+        self.ctx.synchronize()

@@ -35,19 +35,27 @@ struct GeluFwd {
     }
 };
 
-// in[0] = x, in[1] = dy
+// in[0] = x, in[1] = dy.  d/dx = (1 + t)/2 + (1 - t^2) * (x/2) * C (1 + A3 x^2),
+// t = tanh(z).  The reference forms 1 - t*t and (t + 1) from the rounded t
+// (backend.py:398-411), which loses every significant bit once |t| is within a
+// few ulp of 1; here both factors come from w = exp(-2|z|) with no
+// cancellation, so the device value is the accurate one and differs from the
+// CPU value by the CPU's own rounding noise only.
 struct GeluBwd {
     static __device__ __forceinline__ float apply(const float (&in)[2]) {
         const float x = in[0];
-        float t = gelu_tanh_arg(x);
-        float a = t * t;
-        a = 1.0f - a;
+        float z = x * x;
+        z = z * x;
+        z = z * kGeluA;
+        z = x + z;
+        z = z * kGeluC;
+        const float w = expf(-2.0f * fabsf(z));
+        const float inv = 1.0f / (1.0f + w);
+        const float half_one_plus_t = z >= 0.0f ? inv : w * inv;   // (1 + tanh z) / 2
+        const float sech2 = (4.0f * w) * (inv * inv);              // 1 - tanh^2 z
         const float d_inner = kGeluC * (1.0f + (kGeluA3 * x) * x);
-        a = a * ((0.5f * x) * d_inner);
-        t = t + 1.0f;
-        t = t * 0.5f;
-        t = t + a;
-        return in[1] * t;
+        const float a = sech2 * ((0.5f * x) * d_inner);
+        return in[1] * (half_one_plus_t + a);
     }
 };
 

@@ -1,0 +1,308 @@
+"""Graph operators of the fused layer-op path.
+
+Same contract as the reference's op.py: an Op instance is called on input
+Tensors, infers the output shape, and records an OpNode on every output
+(`out.op`); the runtime later binds `node.forward` / `node.backward` to backend
+kernels looked up by the exact type of the op (op.py:13-50, runtime.py:241-243).
+
+AddOp, GatherOp, GELUOp and LayerNormOp keep the reference's names, arguments
+and shape checks (op.py:52-59, 219-267).  RMSNorm, SwiGLU, rotary and the
+residual-fused norms exist in the reference only inside fused GEMM ops
+(op.py:395-507); here they are ops of their own.  ReLU^2 and EmbeddingSum are
+new.
+"""
+from __future__ import annotations
+
+from abc import ABC, abstractmethod
+
+import numpy as np
+
+from .tensor import Tensor
+from .utils import broadcast_shape
+
+
+class OpNode:
+    __slots__ = ("op", "inputs", "outputs", "forward", "backward", "scratch_fwd_layout",
+                 "scratch_bwd_layout", "name", "overwrite_grads")
+
+    def __init__(self, op, inputs, outputs, name=""):
+        self.op = op
+        self.inputs = tuple(inputs)
+        self.outputs = tuple(outputs)
+        self.forward = None
+        self.backward = None
+        self.scratch_fwd_layout = None
+        self.scratch_bwd_layout = None
+        self.name = name
+        # ids of gradient tensors this node is the first to write in a backward
+        # pass: its kernel may store instead of accumulate (set by the runtime)
+        self.overwrite_grads = frozenset()
+
+
+class Op(ABC):
+    op_name = "Op"
+    recompute_output = False
+    # indices (output i aliases input j): the kernel works in place, the
+    # runtime gives output and input (and their grads) the same memory
+    inplace_aliases: dict = {}
+
+    def __call__(self, *inputs):
+        shape = self.infer_shape(*inputs)
+        out = Tensor(shape=shape, dtype=self.infer_dtype(*inputs), device=inputs[0].device,
+                     requires_grad=any(t.requires_grad for t in inputs))
+        out.op = OpNode(op=self, inputs=inputs, outputs=(out,))
+        return out
+
+    @abstractmethod
+    def infer_shape(self, *inputs):
+        ...
+
+    def infer_dtype(self, *inputs):
+        return inputs[0].dtype
+
+    def save_for_backward(self, inputs, outputs):
+        return list(inputs) + list(outputs)
+
+    def is_recompute_output(self):
+        return self.recompute_output
+
+    def fully_written_inputs(self, inputs, outputs):
+        """indices of inputs whose whole gradient tensor this op's backward writes
+        (so a first writer may store instead of accumulating onto zeros)"""
+        return []
+
+    def __repr__(self):
+        return self.op_name
+
+
+class AddOp(Op):
+    op_name = "Add"
+
+    def infer_shape(self, x, y):
+        return broadcast_shape(x.shape, y.shape)
+
+    def save_for_backward(self, inputs, outputs):
+        return []
+
+    def fully_written_inputs(self, inputs, outputs):
+        return [0, 1]
+
+
+class GatherOp(Op):
+    """out[b, t, :] = weight[indices[b, t], :]"""
+    op_name = "Gather"
+
+    def infer_shape(self, indices, weight):
+        if indices.ndim != 2:
+            raise ValueError("Gather indices must be 2D (B, T)")
+        if weight.ndim != 2:
+            raise ValueError("Gather weight must be 2D (V, C)")
+        return indices.shape + (weight.shape[1],)
+
+    def __call__(self, indices, weight):
+        out = Tensor(shape=self.infer_shape(indices, weight), dtype=weight.dtype,
+                     requires_grad=weight.requires_grad, device=weight.device)
+        out.op = OpNode(op=self, inputs=(indices, weight), outputs=(out,))
+        return out
+
+    def save_for_backward(self, inputs, outputs):
+        return list(inputs)
+
+
+class EmbeddingSumOp(Op):
+    """out[b, t, :] = wte[indices[b, t], :] + wpe[t, :] -- the GPT-2 input
+    embedding tok_emb(ids) + pos_emb(arange(T)) as one op
+    (check_tiny_gpt2_kernel.py:282,301)."""
+    op_name = "EmbeddingSum"
+
+    def infer_shape(self, indices, wte, wpe):
+        if indices.ndim != 2 or wte.ndim != 2 or wpe.ndim != 2:
+            raise ValueError("EmbeddingSum takes indices (B, T), wte (V, C), wpe (T_max, C)")
+        if wte.shape[1] != wpe.shape[1]:
+            raise ValueError("EmbeddingSum C mismatch")
+        if wpe.shape[0] < indices.shape[1]:
+            raise ValueError("EmbeddingSum: position table shorter than the sequence")
+        return indices.shape + (wte.shape[1],)
+
+    def __call__(self, indices, wte, wpe):
+        out = Tensor(shape=self.infer_shape(indices, wte, wpe), dtype=wte.dtype, device=wte.device,
+                     requires_grad=wte.requires_grad or wpe.requires_grad)
+        out.op = OpNode(op=self, inputs=(indices, wte, wpe), outputs=(out,))
+        return out
+
+    def save_for_backward(self, inputs, outputs):
+        return [inputs[0]]
+
+    def fully_written_inputs(self, inputs, outputs):
+        return [2] if inputs[2].shape[0] == inputs[0].shape[1] else []
+
+
+class GELUOp(Op):
+    op_name = "GELU"
+
+    def infer_shape(self, x):
+        return x.shape
+
+    def save_for_backward(self, inputs, outputs):
+        return list(inputs)
+
+    def fully_written_inputs(self, inputs, outputs):
+        return [0]
+
+
+class ReLUSquaredOp(Op):
+    op_name = "ReLUSquared"
+
+    def infer_shape(self, x):
+        return x.shape
+
+    def save_for_backward(self, inputs, outputs):
+        return list(inputs)
+
+    def fully_written_inputs(self, inputs, outputs):
+        return [0]
+
+
+class SwiGLUOp(Op):
+    """gu[..., 2H] -> silu(gu[..., :H]) * gu[..., H:]"""
+    op_name = "SwiGLU"
+
+    def infer_shape(self, gu):
+        if gu.shape[-1] % 2 != 0:
+            raise ValueError("SwiGLU last dimension must be even (gate | up)")
+        return gu.shape[:-1] + (gu.shape[-1] // 2,)
+
+    def save_for_backward(self, inputs, outputs):
+        return list(inputs)
+
+    def fully_written_inputs(self, inputs, outputs):
+        return [0]
+
+
+class LayerNormOp(Op):
+    op_name = "LayerNorm"
+
+    def __init__(self, normalized_dim=-1, eps=1e-6):
+        if normalized_dim != -1:
+            raise ValueError("LayerNorm normalises the last dimension")
+        self.normalized_dim = normalized_dim
+        self.eps = eps
+
+    def infer_shape(self, x, gamma, beta):
+        if gamma.shape != beta.shape:
+            raise ValueError("gamma/beta shape mismatch")
+        if x.shape[self.normalized_dim] != gamma.shape[0]:
+            raise ValueError("LayerNorm C mismatch")
+        return x.shape
+
+    def save_for_backward(self, inputs, outputs):
+        return list(inputs)
+
+    def fully_written_inputs(self, inputs, outputs):
+        return [0, 1, 2]
+
+
+class RMSNormOp(Op):
+    """z = x / sqrt(mean(x^2) + eps) [* gamma]; inputs (x,) or (x, gamma)."""
+    op_name = "RMSNorm"
+
+    def __init__(self, eps=1e-6):
+        self.eps = eps
+
+    def infer_shape(self, x, gamma=None):
+        if gamma is not None and gamma.shape != (x.shape[-1],):
+            raise ValueError(f"norm_weight shape must be ({x.shape[-1]},), got {gamma.shape}")
+        return x.shape
+
+    def save_for_backward(self, inputs, outputs):
+        return list(inputs)
+
+    def fully_written_inputs(self, inputs, outputs):
+        return list(range(len(inputs)))
+
+
+class _AddNormOp(Op):
+    """(h, y) = (x + residual, norm(x + residual)).  Two outputs: h continues
+    the residual stream, y feeds the next block."""
+    n_norm_params = 0
+
+    def __call__(self, *inputs):
+        x, res = inputs[0], inputs[1]
+        if x.shape != res.shape:
+            raise ValueError("fused residual add needs operands of one shape")
+        self.infer_shape(*inputs)
+        req = any(t.requires_grad for t in inputs)
+        h = Tensor(shape=x.shape, dtype=x.dtype, device=x.device, requires_grad=req)
+        y = Tensor(shape=x.shape, dtype=x.dtype, device=x.device, requires_grad=req)
+        node = OpNode(op=self, inputs=inputs, outputs=(h, y))
+        h.op = node
+        y.op = node
+        return h, y
+
+    def save_for_backward(self, inputs, outputs):
+        return [outputs[0]] + list(inputs[2:])
+
+    def fully_written_inputs(self, inputs, outputs):
+        return list(range(len(inputs)))
+
+
+class AddLayerNormOp(_AddNormOp):
+    op_name = "AddLayerNorm"
+
+    def __init__(self, eps=1e-5):
+        self.eps = eps
+        self.normalized_dim = -1
+
+    def infer_shape(self, x, res, gamma, beta):
+        if gamma.shape != beta.shape or gamma.shape != (x.shape[-1],):
+            raise ValueError("AddLayerNorm gamma/beta shape mismatch")
+        return x.shape
+
+
+class AddRMSNormOp(_AddNormOp):
+    op_name = "AddRMSNorm"
+
+    def __init__(self, eps=1e-6):
+        self.eps = eps
+
+    def infer_shape(self, x, res, gamma=None):
+        if gamma is not None and gamma.shape != (x.shape[-1],):
+            raise ValueError("AddRMSNorm gamma shape mismatch")
+        return x.shape
+
+
+class RopeOp(Op):
+    """Split-half rotary embedding of q [B,T,H,D] and k [B,T,HKV,D] with tables
+    cos/sin [T_max, D/2].  rope_sign=+1 is the HF convention, -1 the nanochat
+    one (FusedRMSNormGQAOp.rope_sign, op.py:486-491).  Works in place: the
+    outputs take over the inputs' memory."""
+    op_name = "Rope"
+    inplace_aliases = {0: 0, 1: 1}
+
+    def __init__(self, rope_sign=1):
+        if rope_sign not in (1, -1):
+            raise ValueError("rope_sign must be +1 or -1")
+        self.rope_sign = rope_sign
+
+    def infer_shape(self, q, k, cos, sin):
+        if q.ndim != 4 or k.ndim != 4 or q.shape[:2] != k.shape[:2] or q.shape[3] != k.shape[3]:
+            raise ValueError("Rope takes q (B,T,H,D) and k (B,T,HKV,D)")
+        D = q.shape[3]
+        if D % 2 or cos.shape != sin.shape or cos.ndim != 2 or cos.shape[1] != D // 2 or cos.shape[0] < q.shape[1]:
+            raise ValueError("Rope tables must be (T_max >= T, D/2)")
+        return q.shape, k.shape
+
+    def __call__(self, q, k, cos, sin):
+        qs, ks = self.infer_shape(q, k, cos, sin)
+        q2 = Tensor(shape=qs, dtype=q.dtype, device=q.device, requires_grad=q.requires_grad)
+        k2 = Tensor(shape=ks, dtype=k.dtype, device=k.device, requires_grad=k.requires_grad)
+        node = OpNode(op=self, inputs=(q, k, cos, sin), outputs=(q2, k2))
+        q2.op = node
+        k2.op = node
+        return q2, k2
+
+    def save_for_backward(self, inputs, outputs):
+        return [inputs[2], inputs[3]]
+
+
+INT_DTYPES = (np.dtype(np.int32),)

@@ -1,0 +1,425 @@
+"""Graph compiler and executor for the layer-op path.
+
+Counterpart of the reference's runtime.py for what this path needs:
+topological order and gradient tensors (runtime.py:123-152), parameter slabs
+(runtime.py:154-206), kernel binding (runtime.py:241-246), lifetime analysis and
+the first-fit training arena (runtime.py:20-59, 272-513), and the execute /
+zero_grad / forward / backward_graph loops (runtime.py:802-854).
+
+The arena is ONE device allocation; every activation, activation gradient and
+scratch block is a `(buffer_id, byte offset)` view into it, 256-byte aligned.
+
+Gradient zeroing.  The reference's CPU path zero-fills a gradient right before
+the first backward kernel that adds into it (runtime.py:844-854).  Here that
+first writer is told to store instead (OpNode.overwrite_grads) whenever its
+kernel writes the whole tensor, which removes one full write and one full read
+of every activation gradient; the numbers are the same as accumulating onto
+zeros.  `fuse_grad_zeroing=False` restores fill-then-accumulate.
+"""
+from __future__ import annotations
+
+import functools
+from math import prod
+
+import numpy as np
+
+from .device import Device
+from .scratch import ScratchViews
+from .tensor import Tensor
+from .utils import align_up, is_bf16, itemsize
+
+ARENA_ALIGN = 256
+
+
+class MemoryPlanner:
+    """First-fit placement of byte ranges with explicit alloc / free
+    (runtime.py:20-59): a block goes to the lowest offset where it fits between
+    the live blocks."""
+
+    def __init__(self, align=ARENA_ALIGN):
+        self.align = align
+        self.live = {}      # key -> (offset, size)
+        self.offsets = {}   # key -> offset, kept after free
+        self.peak = 0
+
+    def alloc(self, key, nbytes):
+        if key in self.offsets:
+            return self.offsets[key]
+        size = align_up(max(int(nbytes), 1), self.align)
+        cursor = 0
+        for off, sz in sorted(self.live.values()):
+            if cursor + size <= off:
+                break
+            cursor = max(cursor, off + sz)
+        self.live[key] = (cursor, size)
+        self.offsets[key] = cursor
+        self.peak = max(self.peak, cursor + size)
+        return cursor
+
+    def free(self, key):
+        self.live.pop(key, None)
+
+    def get_offset(self, key):
+        return self.offsets.get(key)
+
+
+class _Scratch:
+    """stand-in for a per-node scratch block in the lifetime table"""
+    __slots__ = ("nbytes", "node", "phase")
+
+    def __init__(self, nbytes, node, phase):
+        self.nbytes, self.node, self.phase = nbytes, node, phase
+
+
+class Runtime:
+    _default_runtime = None
+
+    @classmethod
+    def get_default(cls):
+        if cls._default_runtime is None:
+            cls._default_runtime = Runtime()
+        return cls._default_runtime
+
+    def __init__(self, device="hip", forward_only=False, owns_params=True, use_fp16_gemm=False,
+                 fuse_grad_zeroing=True):
+        self.loss = None
+        self.topo = []
+        self.forward_only = forward_only
+        self.owns_params = owns_params
+        self.is_compiled = False
+        self.unified_arena = None
+        self.allocator = Device.get_allocator(device)
+        self.backend = Device.get_backend(device)
+        self.node_to_clear_grads = {}
+        self.grad_scale = 1.0
+        self.accumulate_parameter_grads = False
+        self.use_fp16_gemm = use_fp16_gemm
+        self.backend.use_fp16_gemm = use_fp16_gemm
+        # only a backend whose kernels honour OpNode.overwrite_grads can skip the fills
+        self.fuse_grad_zeroing = bool(fuse_grad_zeroing and getattr(self.backend, "supports_grad_store", False))
+        self.arena_bytes = 0
+        self.leaves = []
+        self.consumers = {}
+        self._alias_of = {}            # output tensor -> input tensor it shares memory with
+        self._stored_leaf_grads = set()   # ids of leaf grads whose first writer stores the whole tensor
+        self._slabs = []
+
+    # -- entry points (runtime.py:89-121) ------------------------------------------
+    def backward(self, loss, grad_scale=1.0, accumulate_parameter_grads=False):
+        self.loss = loss
+        self.grad_scale = float(grad_scale)
+        self.accumulate_parameter_grads = bool(accumulate_parameter_grads)
+        self.backend.accumulate_parameter_grads = self.accumulate_parameter_grads
+        self.backend.grad_scale = self.grad_scale
+        if not self.is_compiled:
+            self.build_topo(loss)
+            self.bind_memory()
+            self.is_compiled = True
+        self.execute()
+
+    def run_forward(self, output, feeds=None, return_value=True):
+        if not self.is_compiled:
+            self.loss = output
+            self.build_topo(output)
+            self.bind_memory()
+            self.is_compiled = True
+        for tensor, host_value in (feeds or {}).items():
+            self.backend.copy_from_host(tensor, host_value)
+        self.forward()
+        if not return_value:
+            return None
+        self.backend.synchronize()
+        return self.backend.copy_to_host(output)
+
+    # -- graph -------------------------------------------------------------------
+    def build_topo(self, loss):
+        self.loss = loss
+        seen_nodes, seen_tensors = set(), set()
+        self.topo, self.leaves = [], []
+
+        def visit(tensor):
+            node = tensor.op
+            if node is None or id(node) in seen_nodes:
+                return
+            seen_nodes.add(id(node))
+            for src in node.inputs:
+                visit(src)
+            for t in node.inputs + node.outputs:
+                if id(t) in seen_tensors:
+                    continue
+                seen_tensors.add(id(t))
+                if t.op is None:
+                    self.leaves.append(t)
+                if not self.forward_only and t.requires_grad and t.grad is None:
+                    gdt = t.grad_dtype if t.op is None else t.dtype
+                    t.grad = Tensor(shape=t.shape, dtype=gdt, requires_grad=False, device=t.device)
+            self.topo.append(node)
+
+        visit(loss)
+
+        self.consumers = {}
+        for node in self.topo:
+            for t in node.inputs:
+                self.consumers.setdefault(id(t), []).append(node)
+        # an output nobody reads never receives a gradient
+        for node in self.topo:
+            for t in node.outputs:
+                if t is not loss and id(t) not in self.consumers:
+                    t.grad = None
+
+        self._place_leaves()
+
+        for node in self.topo:
+            node.forward = self.backend.get_forward_kernel(node.op)
+            node.backward = self.backend.get_backward_kernel(node.op)
+            if node.forward is None or (node.backward is None and not self.forward_only):
+                raise RuntimeError(f"device {self.allocator.device!r} has no kernel for {type(node.op).__name__}")
+            fwd, bwd = self.backend.plan_scratch(node)
+            node.scratch_fwd_layout, node.scratch_bwd_layout = fwd, (None if self.forward_only else bwd)
+
+        self._resolve_aliases()
+
+    def _place_leaves(self):
+        """Parameters that need gradients are packed into one slab, their
+        gradients into another (runtime.py:154-206); other leaves get their own
+        allocation."""
+        params = [t for t in self.leaves
+                  if self.owns_params and not self.forward_only and t.requires_grad and t.grad is not None
+                  and t.storage is None and hasattr(self.allocator, "ctx")]
+        if params:
+            order = [t for t in params if t.ndim > 1] + [t for t in params if t.ndim <= 1]
+            poff, goff, pcur, gcur = {}, {}, 0, 0
+            for t in order:
+                pcur = align_up(pcur, ARENA_ALIGN)
+                poff[id(t)] = pcur
+                pcur += prod(t.shape) * itemsize(t.dtype)
+                gcur = align_up(gcur, ARENA_ALIGN)
+                goff[id(t)] = gcur
+                gcur += prod(t.shape) * itemsize(t.grad.dtype)
+            pslab = self.allocator.empty((align_up(pcur, ARENA_ALIGN),), np.uint8)
+            gslab = self.allocator.empty((align_up(gcur, ARENA_ALIGN),), np.uint8)
+            self.backend.fill_storage2(pslab, 0)
+            self.backend.fill_storage2(gslab, 0)
+            self._slabs += [pslab, gslab]
+            for t in order:
+                t.storage = self.allocator.view(pslab, poff[id(t)], t.shape, t.dtype)
+                t.grad.storage = self.allocator.view(gslab, goff[id(t)], t.shape, t.grad.dtype)
+                self.backend.init(t)
+        for t in self.leaves:
+            if t.requires_grad and not self.owns_params:
+                if t.storage is None or (not self.forward_only and t.grad.storage is None):
+                    raise RuntimeError(f"shared parameter {t.name} has no storage")
+                continue
+            if t.storage is None:
+                t.storage = self.allocator.alloc(t.shape, t.dtype)
+                self.backend.init(t)
+            if not self.forward_only and t.grad is not None and t.grad.storage is None:
+                t.grad.storage = self.allocator.alloc(t.grad.shape, t.grad.dtype)
+                self.backend.fill_storage2(t.grad.storage, 0)
+
+    def _resolve_aliases(self):
+        """In-place ops: an output shares its input's memory when the input is
+        an activation nobody else reads; otherwise the backend copies first."""
+        self._alias_of = {}
+        for node in self.topo:
+            for out_i, in_i in node.op.inplace_aliases.items():
+                src, dst = node.inputs[in_i], node.outputs[out_i]
+                if src.op is not None and len(self.consumers.get(id(src), [])) == 1 and src is not self.loss:
+                    self._alias_of[id(dst)] = src
+
+    def _root(self, t):
+        while id(t) in self._alias_of:
+            t = self._alias_of[id(t)]
+        return t
+
+    # -- memory ------------------------------------------------------------------
+    def bind_memory(self):
+        n = len(self.topo)
+        steps = [(0, node) for node in self.topo]
+        if not self.forward_only:
+            steps += [(1, node) for node in reversed(self.topo)]
+
+        # who zero-fills / first-writes which gradient (runtime.py:272-284)
+        self.node_to_clear_grads = {id(node): [] for node in self.topo}
+        self._stored_leaf_grads = set()
+        if not self.forward_only:
+            touched = set()
+            for node in reversed(self.topo):
+                overwrite = set()
+                full = {node.inputs[i] for i in node.op.fully_written_inputs(node.inputs, node.outputs)}
+                aliased_inputs = {id(self._alias_of[id(o)]) for o in node.outputs
+                                  if id(o) in self._alias_of and o.grad is not None}
+                for x in node.inputs:
+                    if not x.requires_grad or x.grad is None or id(x) in touched:
+                        continue
+                    touched.add(id(x))
+                    if id(x) in aliased_inputs:
+                        continue          # its gradient is the output's gradient, rotated in place
+                    storable = (self.fuse_grad_zeroing and any(x is f for f in full)
+                                and sum(1 for t in node.inputs if t is x) == 1)
+                    if storable:
+                        overwrite.add(id(x.grad))
+                        if x.op is None:
+                            self._stored_leaf_grads.add(id(x.grad))
+                    elif x.op is not None:
+                        self.node_to_clear_grads[id(node)].append(x)
+                node.overwrite_grads = frozenset(overwrite)
+
+        life = {}       # key object -> [first step, last step]
+        keyobj = {}
+
+        def touch(obj, step):
+            k = id(obj)
+            keyobj[k] = obj
+            if k in life:
+                life[k][0] = min(life[k][0], step)
+                life[k][1] = max(life[k][1], step)
+            else:
+                life[k] = [step, step]
+
+        for step, (phase, node) in enumerate(steps):
+            if phase == 0:
+                for t in node.outputs:
+                    touch(self._root(t), step)
+                for t in node.inputs:
+                    if t.op is not None:
+                        touch(self._root(t), step)
+                if node.scratch_fwd_layout is not None:
+                    touch(_Scratch(node.scratch_fwd_layout.nbytes, node, 0), step)
+            else:
+                for t in node.op.save_for_backward(node.inputs, node.outputs):
+                    if t.op is not None:
+                        touch(self._root(t), step)
+                for t in node.inputs + node.outputs:
+                    if t.grad is not None and t.op is not None:
+                        touch(self._root(t).grad if self._root(t).grad is not None else t.grad, step)
+                if node.scratch_bwd_layout is not None:
+                    touch(_Scratch(node.scratch_bwd_layout.nbytes, node, 1), step)
+        if self.loss is not None and self.loss.op is not None:
+            touch(self._root(self.loss), len(steps))
+            if self.loss.grad is not None:
+                # written by fill() between the forward and the backward loops
+                touch(self._root(self.loss).grad or self.loss.grad, n - 1 if n else 0)
+
+        planner = MemoryPlanner()
+        order = sorted(life.items(), key=lambda kv: kv[1][0])
+        by_start, by_end = {}, {}
+        for k, (a, b) in order:
+            by_start.setdefault(a, []).append(k)
+            by_end.setdefault(b, []).append(k)
+        last = max((b for _, (_, b) in order), default=-1)
+        for step in range(last + 1):
+            for k in by_end.get(step - 1, []):
+                planner.free(k)
+            for k in by_start.get(step, []):
+                obj = keyobj[k]
+                nbytes = obj.nbytes if isinstance(obj, _Scratch) else prod(obj.shape) * itemsize(obj.dtype)
+                planner.alloc(k, nbytes)
+
+        self.arena_bytes = planner.peak
+        self.memory_plan = {k: planner.get_offset(k) for k in life}
+        if planner.peak == 0:
+            self.unified_arena = None
+            return
+        print(f"Training arena need {planner.peak}")
+        self.unified_arena = self.allocator.empty((planner.peak,), np.uint8)
+        print(f"[ARENA-TRAIN-ALLOC] bytes={planner.peak} "
+              f"buffer_id={getattr(self.unified_arena.ptr, 'buffer_id', None)}", flush=True)
+        self._bind_views(planner, keyobj)
+
+    def bind_memory_new(self, arena):
+        """re-point every planned view at another arena of at least the same size
+        (runtime.py:718-732)"""
+        if arena.nbytes < self.arena_bytes:
+            raise RuntimeError(f"arena of {arena.nbytes} bytes is smaller than the plan ({self.arena_bytes})")
+        self.unified_arena = arena
+        planner = MemoryPlanner()
+        planner.offsets = dict(self.memory_plan)
+        self._bind_views(planner, self._keyobj)
+
+    def _bind_views(self, planner, keyobj):
+        self._keyobj = keyobj
+        arena = self.unified_arena
+        for k, obj in keyobj.items():
+            off = planner.get_offset(k)
+            if isinstance(obj, _Scratch):
+                node = obj.node
+                layout = node.scratch_fwd_layout if obj.phase == 0 else node.scratch_bwd_layout
+                block = self.allocator.view(arena, off, (obj.nbytes,), np.uint8)
+                views = ScratchViews({name: self.allocator.view(block, o, shape, dt)
+                                      for name, (o, shape, dt) in layout.slots.items()})
+                if obj.phase == 0:
+                    base = getattr(node.forward, "func", node.forward)
+                    node.forward = functools.partial(base, scratch=views)
+                else:
+                    base = getattr(node.backward, "func", node.backward)
+                    node.backward = functools.partial(base, scratch=views)
+            else:
+                obj.storage = self.allocator.view(arena, off, obj.shape, obj.dtype)
+        # aliased outputs (and their gradients) share their root's views
+        for node in self.topo:
+            for t in node.outputs:
+                if id(t) in self._alias_of:
+                    root = self._root(t)
+                    t.storage = root.storage
+                    if t.grad is not None and root.grad is not None:
+                        t.grad.storage = root.grad.storage
+                    elif t.grad is not None and root.grad is None:
+                        raise RuntimeError("aliased output needs a gradient but its input has none")
+        for node in self.topo:
+            for t in node.outputs:
+                if t.init_val is not None:
+                    self.backend.init(t)
+
+    # -- execution (runtime.py:802-854) ---------------------------------------------
+    def execute(self):
+        if self.forward_only:
+            self.forward()
+            return
+        if not self.accumulate_parameter_grads:
+            self.zero_grad()
+        self.forward()
+        self.backend.fill(self.loss.grad, self.grad_scale)
+        self.backward_graph()
+
+    def zero_grad(self):
+        """zero the parameter gradients, except those whose first backward kernel
+        stores the whole tensor anyway"""
+        seen = set()
+        for node in self.topo:
+            for t in node.inputs + node.outputs:
+                if id(t) in seen:
+                    continue
+                seen.add(id(t))
+                if t.grad is not None and t.op is None:
+                    if id(t.grad) in self._stored_leaf_grads and not self.accumulate_parameter_grads:
+                        continue
+                    self.backend.fill(t.grad, 0)
+
+    def forward(self):
+        self.backend.begin_pass()
+        for node in self.topo:
+            node.forward(node.inputs, node.outputs)
+        self.backend.end_pass()
+
+    def backward_graph(self):
+        self.backend.begin_pass()
+        for node in reversed(self.topo):
+            for t in self.node_to_clear_grads.get(id(node), ()):
+                if t.grad is not None:
+                    self.backend.fill(t.grad, 0)
+            node.backward(node.inputs, node.outputs)
+        self.backend.end_pass()
+
+    def release(self):
+        """return the arena and the parameter slabs to the device"""
+        rel = getattr(self.allocator, "release", None)
+        if rel is None:
+            return
+        self.backend.synchronize()
+        if self.unified_arena is not None:
+            rel(self.unified_arena)
+            self.unified_arena = None
+        for slab in self._slabs:
+            rel(slab)
+        self._slabs = []

@@ -118,10 +118,18 @@ def test_norm_backward_fp32(ctx, kind, shape, eps):
     out = G.norm_backward(ctx, KINDS[kind], x, gamma, dy, eps, want_dbeta=(kind == "layer"))
     dx, dgamma, dbeta = _norm_ref_backward(kind, x, gamma, dy, eps)
     assert_fp32_close(out["dx"], dx, f"{kind} dx {shape}")
-    # few rows: the CPU's sequential row sum is still within the fp32 tolerance
-    assert_fp32_close(out["dgamma"], dgamma, f"{kind} dgamma {shape}", rtol=1e-5, atol=2e-6)
+    # row sums: both sides round differently (the CPU adds rows one by one), so
+    # the absolute budget grows with sqrt(rows); at probe sizes it is 2e-6
+    rows = int(np.prod(shape[:-1]))
+    atol = max(2e-6, 1e-6 * np.sqrt(rows))
+    assert_fp32_close(out["dgamma"], dgamma, f"{kind} dgamma {shape}", rtol=1e-5, atol=atol)
     if kind == "layer":
-        assert_fp32_close(out["dbeta"], dbeta, f"{kind} dbeta {shape}", rtol=1e-5, atol=2e-6)
+        assert_fp32_close(out["dbeta"], dbeta, f"{kind} dbeta {shape}", rtol=1e-5, atol=atol)
+        _, dg64, db64 = cf.layernorm_grads(x, gamma, dy, eps)
+        assert np.abs(out["dbeta"] - db64).max() <= atol
+    else:
+        _, dg64 = cf.rmsnorm_grads(x, gamma, dy, eps)
+    assert np.abs(out["dgamma"] - dg64).max() <= atol
 
 
 @pytest.mark.parametrize("kind", ["layer", "rms"])
@@ -175,16 +183,16 @@ def test_norm_backward_param_grads_many_rows(ctx, kind, C, eps):
     else:
         _, dg64 = cf.rmsnorm_grads(x, gamma, dy, eps)
         db64 = None
-    tol = 1e-6 * np.sqrt(N)
-    err_gpu = np.abs(out["dgamma"] - dg64).max()
+    tol = 1e-6 * np.sqrt(N) + 2e-6 * np.abs(dg64)
+    err_gpu = np.abs(out["dgamma"] - dg64)
     err_cpu = np.abs(dg_cpu - dg64).max()
-    assert err_gpu <= tol, (err_gpu, tol)
-    assert err_gpu <= err_cpu + 1e-6, (err_gpu, err_cpu)
+    assert (err_gpu <= tol).all(), (err_gpu.max(), tol.max())
+    assert err_gpu.max() <= err_cpu + 1e-6, (err_gpu.max(), err_cpu)
     # and against the CPU restatement at the tolerance the reference's own
     # checker uses for these sums (debug/check_qwen_kernel.py:128-130, atol 1e-4 scaled by sqrt(N/14))
     assert_fp32_close(out["dgamma"], dg_cpu, "dgamma vs cpu", rtol=1e-5, atol=1e-4 * np.sqrt(N / 14))
     if db64 is not None:
-        assert np.abs(out["dbeta"] - db64).max() <= tol
+        assert (np.abs(out["dbeta"] - db64) <= 1e-6 * np.sqrt(N) + 2e-6 * np.abs(db64)).all()
         assert_fp32_close(out["dbeta"], db_cpu, "dbeta vs cpu", rtol=1e-5, atol=1e-4 * np.sqrt(N / 14))
 
 
@@ -263,7 +271,16 @@ def test_gelu_dense_sweep_and_special_values(ctx):
     dgot = G.unary_backward(ctx, "agrad_gelu_backward", x, one)
     dref = np.zeros_like(x)
     ref.gelu_backward_into(x, one, dref)
-    assert_fp32_close(dgot, dref, "gelu' sweep")
+    # The CPU forms 1 - t*t from the rounded tanh; one ulp of t moves its result
+    # by 6e-8 * |x| C (1 + A3 x^2), which passes 1e-6 at |x| ~ 4.9.  Inside that
+    # range the stated tolerance holds; over the whole sweep the device value is
+    # the one nearer the float64 derivative.
+    core = np.abs(x) <= 4.5
+    assert_fp32_close(dgot[core], dref[core], "gelu' sweep, |x| <= 4.5")
+    assert_fp32_close(dgot, dref, "gelu' sweep", rtol=1e-5, atol=3e-6)
+    d64 = cf.gelu_grad(x)
+    assert np.abs(dgot - d64).max() <= 4e-7   # values reach 1.13: two ulp
+    assert np.abs(dgot - d64).max() <= np.abs(dref - d64).max()
     sp = np.array([0.0, -0.0, 30.0, -30.0, 1e-20, 80.0, -80.0], dtype=np.float32)
     y = G.unary(ctx, "agrad_gelu_forward", sp)
     assert y[0] == 0 and y[2] == 30.0 and y[3] == 0 and y[5] == 80.0 and y[6] == 0

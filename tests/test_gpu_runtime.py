@@ -1,0 +1,319 @@
+"""The same graph on the numpy oracle device ("cpu") and on "hip", compared.
+
+This is the reference's own method: run_single_op builds a graph, runs forward,
+zeroes grads, writes an upstream gradient into out.grad, runs backward_graph and
+reads outputs and gradients back (check_tiny_gpt2_kernel.py:473-490), once per
+device.  The hip side goes Tensor -> Op -> HipBackend -> hip_ext.HipContext ->
+agrad_dispatch (C ABI) -> kernel.
+"""
+import numpy as np
+import pytest
+
+from autograd_amd.device import Device
+from autograd_amd.op import (AddLayerNormOp, AddOp, AddRMSNormOp, EmbeddingSumOp, GatherOp, GELUOp,
+                             LayerNormOp, ReLUSquaredOp, RMSNormOp, RopeOp, SwiGLUOp)
+from autograd_amd.runtime import Runtime
+from autograd_amd.tensor import Tensor
+from autograd_amd.utils import BF16
+from oracle import cpu_device
+from oracle import cpu_ops as ref
+from tests.helpers import assert_bf16_close, assert_fp32_close
+
+pytestmark = pytest.mark.gpu
+SEED = 1333
+cpu_device.register()
+
+
+def make_tensor(shape, dtype, device, requires_grad, value, name=""):
+    return Tensor(shape=tuple(shape), dtype=dtype, device=device, requires_grad=requires_grad,
+                  init_val=np.asarray(value), name=name)
+
+
+def run_single_op(device, build_fn, upstream=None, fuse=True):
+    rt = Runtime(device=device, fuse_grad_zeroing=fuse)
+    out, tracked = build_fn(device)
+    outs = out if isinstance(out, (tuple, list)) else (out,)
+    rt.loss = outs[0]
+    rt.build_topo(outs[0])
+    rt.bind_memory()
+    rt.forward()
+    rt.backend.synchronize()
+    if upstream is not None:
+        rt.zero_grad()
+        rt.backend.copy_from_host(outs[0].grad, np.asarray(upstream, dtype=np.float32))
+        rt.backward_graph()
+        rt.backend.synchronize()
+    host = [rt.backend.copy_to_host(o) for o in outs]
+    grads = {k: (None if t.grad is None else rt.backend.copy_to_host(t.grad)) for k, t in tracked.items()}
+    rt.release()
+    return host, grads
+
+
+def both(build_fn, upstream, fuse=True):
+    cpu = run_single_op("cpu", build_fn, upstream)
+    hip = run_single_op("hip", build_fn, upstream, fuse=fuse)
+    return cpu, hip
+
+
+def test_probe_layernorm():
+    """probe_layernorm (check_tiny_gpt2_kernel.py:758-782)."""
+    rng = np.random.default_rng(SEED + 4)
+    B, T, C = 2, 16, 64
+    x_np = rng.standard_normal((B, T, C), dtype=np.float32)
+    g_np = rng.standard_normal((C,), dtype=np.float32)
+    b_np = rng.standard_normal((C,), dtype=np.float32)
+    upstream = rng.standard_normal((B, T, C), dtype=np.float32)
+
+    def build(device):
+        x = make_tensor(x_np.shape, np.float32, device, True, x_np)
+        g = make_tensor(g_np.shape, np.float32, device, True, g_np)
+        b = make_tensor(b_np.shape, np.float32, device, True, b_np)
+        return LayerNormOp(eps=1e-5)(x, g, b), {"x": x, "gamma": g, "beta": b}
+
+    for fuse in (True, False):
+        (c_out, c_g), (h_out, h_g) = both(build, upstream, fuse)
+        assert_fp32_close(h_out[0], c_out[0], "forward")
+        for name in ("x", "gamma", "beta"):
+            assert_fp32_close(h_g[name], c_g[name], f"{name}.grad fuse={fuse}")
+
+
+def test_probe_gelu():
+    """probe_gelu (check_tiny_gpt2_kernel.py:783-794)."""
+    rng = np.random.default_rng(SEED + 5)
+    x_np = rng.standard_normal((2, 16, 64), dtype=np.float32)
+    upstream = rng.standard_normal(x_np.shape, dtype=np.float32)
+
+    def build(device):
+        x = make_tensor(x_np.shape, np.float32, device, True, x_np)
+        return GELUOp()(x), {"x": x}
+
+    (c_out, c_g), (h_out, h_g) = both(build, upstream)
+    assert_fp32_close(h_out[0], c_out[0], "forward")
+    assert_fp32_close(h_g["x"], c_g["x"], "x.grad")
+
+
+def test_probe_gather_position_table():
+    """probe_gather: GatherOp on a position table with pos_ids = tile(arange(T))
+    (check_tiny_gpt2_kernel.py:282, 875-890)."""
+    rng = np.random.default_rng(SEED + 6)
+    B, T, C = 2, 32, 256
+    pos_ids = np.tile(np.arange(T, dtype=np.int32), (B, 1))
+    w_np = (0.02 * rng.standard_normal((T, C))).astype(np.float32)
+    upstream = rng.standard_normal((B, T, C), dtype=np.float32)
+
+    def build(device):
+        idx = make_tensor(pos_ids.shape, np.int32, device, False, pos_ids)
+        w = make_tensor(w_np.shape, np.float32, device, True, w_np)
+        return GatherOp()(idx, w), {"w": w}
+
+    (c_out, c_g), (h_out, h_g) = both(build, upstream)
+    np.testing.assert_array_equal(h_out[0].view(np.uint32), c_out[0].view(np.uint32))
+    assert_fp32_close(h_g["w"], c_g["w"], "w.grad")
+
+
+def test_probe_fill_and_copy():
+    """probe_fill (check_tiny_gpt2_kernel.py:795-810) plus copy round trips."""
+    rt = Runtime(device="hip")
+    t = Tensor(shape=(8,), dtype=np.float32, requires_grad=False, device="hip")
+    t.storage = rt.allocator.alloc(t.shape, t.dtype)
+    rt.backend.copy_from_host(t, np.full((8,), 9.0, dtype=np.float32))
+    for v in (0.0, 1.0, -2.5):
+        rt.backend.begin_pass()
+        rt.backend.fill(t, v)
+        rt.backend.end_pass()
+        np.testing.assert_array_equal(rt.backend.copy_to_host(t), np.full((8,), v, np.float32))
+    # odd sizes and offsets through the arena view path
+    big = rt.allocator.alloc((1000,), np.float32)
+    rt.backend.fill_storage(big, 3.0)
+    view = rt.allocator.view(big, 4 * 3, (77,), np.float32)
+    rt.backend.fill_storage(view, 5.0)
+    host = rt.backend.ctx.copy_to_host(big.ptr.buffer_id, 0, [1000], "float32")
+    want = np.full(1000, 3.0, np.float32)
+    want[3:80] = 5.0
+    np.testing.assert_array_equal(host, want)
+    with pytest.raises(RuntimeError):
+        rt.allocator.view(big, 4 * 990, (11,), np.float32)
+    # bf16 storage: copy_from_host rounds to nearest even, copy_to_host widens
+    tb = Tensor(shape=(5,), dtype=BF16, requires_grad=False, device="hip")
+    tb.storage = rt.allocator.alloc(tb.shape, tb.dtype)
+    vals = np.array([1.0, 1.00390625, 3.14159, -2.7e-3, 65504.0], np.float32)
+    rt.backend.copy_from_host(tb, vals)
+    np.testing.assert_array_equal(rt.backend.copy_to_host(tb), ref.round_bf16(vals))
+    rt.backend.fill(tb, 0.1)
+    np.testing.assert_array_equal(rt.backend.copy_to_host(tb), np.full(5, ref.round_bf16(np.float32(0.1))))
+
+
+def test_unknown_device_and_kernel():
+    with pytest.raises(ValueError):
+        Device.get_backend("mps")
+    ctx = Device.get_backend("hip").ctx
+    with pytest.raises(RuntimeError):
+        ctx.dispatch_with_args_3d("softmax_forward", [], [], [], 1, 1, 1, 1)
+    with pytest.raises(ValueError):      # wrong operand count
+        ctx.dispatch_with_args_3d("gelu_forward_kernel", [0], [0], [0, 1, 0], 1, 1, 1, 1)
+    buf = ctx.alloc(64)
+    with pytest.raises(ValueError):      # range outside the buffer
+        ctx.dispatch_with_args_3d("gelu_forward_kernel", [buf, buf], [0, 0], [0, 1000, 0], 1, 1, 1, 1)
+    ctx.free(buf)
+
+
+def test_config1_tiny_gpt2_chain():
+    """BASELINE config 1: ids -> wte + wpe gather-sum -> LayerNorm (gamma 1, beta 0)
+    -> GELU, B=4 T=128 C=128 V=50257, fp32, forward then backward."""
+    rng = np.random.default_rng(SEED + 0)
+    B, T, C, V = 4, 128, 128, 50257
+    ids_np = rng.integers(0, V, size=(B, T), dtype=np.int32)
+    wte_np = (0.02 * rng.standard_normal((V, C))).astype(np.float32)
+    wpe_np = (0.02 * rng.standard_normal((T, C))).astype(np.float32)
+    upstream = rng.standard_normal((B, T, C), dtype=np.float32)
+
+    def build(device):
+        ids = make_tensor((B, T), np.int32, device, False, ids_np)
+        wte = make_tensor((V, C), np.float32, device, True, wte_np, "wte")
+        wpe = make_tensor((T, C), np.float32, device, True, wpe_np, "wpe")
+        g = make_tensor((C,), np.float32, device, True, np.ones(C, np.float32))
+        b = make_tensor((C,), np.float32, device, True, np.zeros(C, np.float32))
+        x0 = EmbeddingSumOp()(ids, wte, wpe)
+        y = LayerNormOp(eps=1e-5)(x0, g, b)
+        return GELUOp()(y), {"wte": wte, "wpe": wpe, "gamma": g, "beta": b}
+
+    (c_out, c_g), (h_out, h_g) = both(build, upstream)
+    assert_fp32_close(h_out[0], c_out[0], "config 1 forward")
+    assert_fp32_close(h_g["wte"], c_g["wte"], "wte.grad", rtol=1e-5, atol=2e-6)
+    assert_fp32_close(h_g["wpe"], c_g["wpe"], "wpe.grad", rtol=1e-5, atol=2e-6)
+    atol = 1e-6 * np.sqrt(B * T)
+    assert_fp32_close(h_g["gamma"], c_g["gamma"], "gamma.grad", rtol=1e-5, atol=atol)
+    assert_fp32_close(h_g["beta"], c_g["beta"], "beta.grad", rtol=1e-5, atol=atol)
+
+    # the unfused reference composition gives the same numbers: Gather x2 + Add
+    def build_unfused(device):
+        ids = make_tensor((B, T), np.int32, device, False, ids_np)
+        pos = make_tensor((B, T), np.int32, device, False, np.tile(np.arange(T, dtype=np.int32), (B, 1)))
+        wte = make_tensor((V, C), np.float32, device, True, wte_np)
+        wpe = make_tensor((T, C), np.float32, device, True, wpe_np)
+        g = make_tensor((C,), np.float32, device, True, np.ones(C, np.float32))
+        b = make_tensor((C,), np.float32, device, True, np.zeros(C, np.float32))
+        x0 = AddOp()(GatherOp()(ids, wte), GatherOp()(pos, wpe))
+        return GELUOp()(LayerNormOp(eps=1e-5)(x0, g, b)), {"wte": wte, "wpe": wpe}
+
+    u_out, u_g = run_single_op("hip", build_unfused, upstream)
+    np.testing.assert_array_equal(u_out[0], h_out[0])
+    np.testing.assert_array_equal(u_g["wpe"], h_g["wpe"])
+    np.testing.assert_array_equal(u_g["wte"], h_g["wte"])
+
+
+@pytest.mark.parametrize("dtype", [np.float32, BF16])
+def test_transformer_block_slice(dtype):
+    """A chain that uses every op once: gather -> add+RMSNorm -> rope on q/k views
+    is not expressible without GEMMs, so the slices are chained directly:
+    gather -> AddRMSNorm(residual) -> SwiGLU -> ReLU^2 -> AddLayerNorm -> Add."""
+    rng = np.random.default_rng(SEED + 7)
+    B, T, C, V = 2, 24, 256, 97
+    ids_np = rng.integers(0, V, size=(B, T), dtype=np.int32)
+    w_np = rng.standard_normal((V, C)).astype(np.float32)
+    r_np = rng.standard_normal((B, T, C)).astype(np.float32)
+    g1 = (1 + 0.02 * rng.standard_normal(C)).astype(np.float32)
+    g2 = (1 + 0.02 * rng.standard_normal(C // 2)).astype(np.float32)
+    b2 = (0.02 * rng.standard_normal(C // 2)).astype(np.float32)
+    upstream = rng.standard_normal((B, T, C // 2)).astype(np.float32)
+
+    def build(device):
+        ids = make_tensor((B, T), np.int32, device, False, ids_np)
+        w = make_tensor((V, C), dtype, device, True, w_np)
+        r = make_tensor((B, T, C), dtype, device, True, r_np)
+        ga = make_tensor((C,), np.float32, device, True, g1)
+        gb = make_tensor((C // 2,), np.float32, device, True, g2)
+        bb = make_tensor((C // 2,), np.float32, device, True, b2)
+        x = GatherOp()(ids, w)
+        h, y = AddRMSNormOp(eps=1e-6)(x, r, ga)
+        s = SwiGLUOp()(y)                    # [B,T,C/2]
+        a = ReLUSquaredOp()(s)
+        h2, y2 = AddLayerNormOp(eps=1e-5)(a, s, gb, bb)
+        out = AddOp()(h2, y2)
+        return out, {"w": w, "r": r, "ga": ga, "gb": gb, "bb": bb}
+
+    (c_out, c_g), (h_out, h_g) = both(build, upstream)
+    if dtype is BF16:
+        assert_bf16_close(h_out[0], c_out[0], "block forward", rel=2e-2)
+        for k in ("r",):
+            assert_bf16_close(h_g[k], c_g[k], f"{k}.grad", rel=3e-2)
+    else:
+        assert_fp32_close(h_out[0], c_out[0], "block forward", rtol=2e-5, atol=2e-6)
+        for k in ("w", "r"):
+            assert_fp32_close(h_g[k], c_g[k], f"{k}.grad", rtol=5e-5, atol=1e-5)
+        for k in ("ga", "gb", "bb"):
+            assert_fp32_close(h_g[k], c_g[k], f"{k}.grad", rtol=5e-5, atol=1e-4)
+    # fused zeroing and fill-then-accumulate agree bit for bit
+    n_out, n_g = run_single_op("hip", build, upstream, fuse=False)
+    np.testing.assert_array_equal(n_out[0], h_out[0])
+    for k in h_g:
+        np.testing.assert_array_equal(n_g[k] + 0.0, h_g[k] + 0.0)
+
+
+@pytest.mark.parametrize("sign", [1, -1])
+def test_rope_op_in_graph(sign):
+    """RopeOp on leaves (copy, then rotate) and on activations (aliased, in place)."""
+    rng = np.random.default_rng(SEED + 8)
+    B, T, H, HKV, D = 2, 16, 4, 2, 64
+    q_np = rng.standard_normal((B, T, H, D)).astype(np.float32)
+    k_np = rng.standard_normal((B, T, HKV, D)).astype(np.float32)
+    cos_np, sin_np = ref.rope_tables(32, D, 1e4)
+    up = rng.standard_normal((B, T, H, D)).astype(np.float32)
+
+    def build_leaf(device):
+        q = make_tensor(q_np.shape, np.float32, device, True, q_np)
+        k = make_tensor(k_np.shape, np.float32, device, True, k_np)
+        c = make_tensor(cos_np.shape, np.float32, device, False, cos_np)
+        s = make_tensor(sin_np.shape, np.float32, device, False, sin_np)
+        q2, k2 = RopeOp(rope_sign=sign)(q, k, c, s)
+        return (q2, k2), {"q": q, "k": k}
+
+    def build_act(device):
+        q = make_tensor(q_np.shape, np.float32, device, True, q_np)
+        k = make_tensor(k_np.shape, np.float32, device, True, k_np)
+        c = make_tensor(cos_np.shape, np.float32, device, False, cos_np)
+        s = make_tensor(sin_np.shape, np.float32, device, False, sin_np)
+        qa, ka = ReLUSquaredOp()(q), ReLUSquaredOp()(k)
+        q2, k2 = RopeOp(rope_sign=sign)(qa, ka, c, s)
+        out = AddOp()(q2, q2)
+        return (out, k2), {"q": q, "k": k}
+
+    want_q, want_k = q_np.copy(), k_np.copy()
+    ref.rope_signed(want_q, want_k, cos_np, sin_np, sign, False)
+    (c_out, c_g), (h_out, h_g) = both(build_leaf, up)
+    np.testing.assert_array_equal(h_out[0], want_q)
+    np.testing.assert_array_equal(c_out[0], want_q)
+    assert_fp32_close(h_g["q"], c_g["q"], "q.grad (leaf)")
+    back = up.copy()
+    ref.rope_signed(back, np.zeros_like(k_np), cos_np, sin_np, sign, True)
+    np.testing.assert_array_equal(h_g["q"], back)
+
+    (c_out, c_g), (h_out, h_g) = both(build_act, up)
+    assert_fp32_close(h_out[0], c_out[0], "rope on activations")
+    assert_fp32_close(h_g["q"], c_g["q"], "q.grad (aliased)")
+
+
+def test_accumulate_parameter_grads_and_rerun():
+    """Two backward passes with accumulate_parameter_grads give twice the
+    parameter gradient; without it the second pass starts from zero."""
+    rng = np.random.default_rng(SEED + 9)
+    x_np = rng.standard_normal((32, 384)).astype(np.float32)
+    g_np = (1 + 0.02 * rng.standard_normal(384)).astype(np.float32)
+    rt = Runtime(device="hip")
+    x = make_tensor(x_np.shape, np.float32, "hip", True, x_np)
+    g = make_tensor(g_np.shape, np.float32, "hip", True, g_np)
+    out = RMSNormOp(eps=1e-6)(x, g)
+    rt.backward(out, grad_scale=0.5)
+    first = rt.backend.copy_to_host(g.grad)
+    dx_first = rt.backend.copy_to_host(x.grad)
+    rt.backward(out, grad_scale=0.5)
+    np.testing.assert_array_equal(rt.backend.copy_to_host(g.grad), first)
+    rt.backward(out, grad_scale=0.5, accumulate_parameter_grads=True)
+    assert_fp32_close(rt.backend.copy_to_host(g.grad), 2 * first, "accumulated gamma.grad", atol=2e-6)
+    assert_fp32_close(rt.backend.copy_to_host(x.grad), 2 * dx_first, "accumulated x.grad", atol=2e-6)
+    dx = np.zeros_like(x_np)
+    dg = np.zeros_like(g_np)
+    ref.rmsnorm_backward_into(x_np, g_np, np.full_like(x_np, 0.5), 1e-6, dx, dg)
+    assert_fp32_close(first, dg, "gamma.grad", atol=4e-6)
+    assert_fp32_close(dx_first, dx, "x.grad")
+    rt.release()

@@ -1,0 +1,216 @@
+"""Host-side logic and the native library's load / export surface, no GPU needed."""
+import ctypes
+import re
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+from autograd_amd import capi
+from autograd_amd.device import Device
+from autograd_amd.op import (AddLayerNormOp, AddOp, AddRMSNormOp, EmbeddingSumOp, GatherOp, GELUOp,
+                             LayerNormOp, RMSNormOp, RopeOp, SwiGLUOp)
+from autograd_amd.runtime import MemoryPlanner, Runtime
+from autograd_amd.tensor import Tensor
+from autograd_amd.utils import BF16, bf16_bits, broadcast_shape, contiguous_strides, f32_bits, itemsize
+from oracle import cpu_device
+
+ROOT = Path(__file__).resolve().parents[1]
+cpu_device.register()
+
+
+def T(shape, dtype=np.float32, requires_grad=True, val=None):
+    return Tensor(shape=shape, dtype=dtype, device="cpu", requires_grad=requires_grad, init_val=val)
+
+
+# ---- native library: loads without a GPU and exports what the header declares ----
+def test_library_exports_every_declared_symbol():
+    header = (ROOT / "include" / "autograd_hip.h").read_text()
+    declared = set(re.findall(r"\b(agrad_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 35
+    lib = ctypes.CDLL(str(capi.LIB_PATH))
+    missing = [name for name in sorted(declared) if not hasattr(lib, name)]
+    assert not missing, f"declared but not exported: {missing}"
+    assert declared == set(capi.SIGNATURES), declared ^ set(capi.SIGNATURES)
+
+
+def test_library_reports_errors_without_gpu_or_kernel():
+    lib = capi.load_library()
+    assert lib.agrad_kernel_count() == 22
+    names = [lib.agrad_kernel_name(i).decode() for i in range(lib.agrad_kernel_count())]
+    for n in ("layernorm_forward", "layernorm_backward_kernel", "rmsnorm_forward", "rmsnorm_backward",
+              "gelu_forward_kernel", "gelu_backward_kernel", "swiglu_forward_kernel", "rope_qk_inplace",
+              "gather_forward_kernel", "gather_backward_kernel", "pos_emb_grad", "fill_scalar_kernel",
+              "fp32_to_bf16", "add_residual_forward"):
+        assert n in names
+    assert lib.agrad_kernel_signature(b"nope") is None
+    assert b"eps_bits" in lib.agrad_kernel_signature(b"layernorm_forward")
+    assert lib.agrad_kernel_name(-1) is None and lib.agrad_kernel_name(999) is None
+    # null context is refused, not dereferenced
+    assert lib.agrad_synchronize(None) == capi.EINVAL
+    assert b"null context" in lib.agrad_last_error()
+    assert lib.agrad_dispatch(None, b"x", None, None, 0, None, 0, 0, 0, 0, 0) == capi.EINVAL
+
+
+def test_pybind_module_imports_and_hip_device_is_loud_without_gpu():
+    from autograd_amd import hip_ext
+    assert hip_ext.F32 == 0 and hip_ext.BF16 == 1
+    if hip_ext.device_count() == 0:
+        with pytest.raises(RuntimeError):
+            hip_ext.HipContext(0)
+        with pytest.raises(RuntimeError):
+            Device.get_backend("hip")       # no silent CPU path
+
+
+def test_device_registry():
+    with pytest.raises(ValueError):
+        Device.get_allocator("mps")
+    with pytest.raises(ValueError):
+        Device.get_backend("cuda")
+    assert Device.get_backend("cpu") is Device.get_backend("cpu")
+    assert Device.get_allocator("cpu").device == "cpu"
+
+
+# ---- utils ------------------------------------------------------------------------
+def test_utils():
+    assert contiguous_strides((2, 3, 4)) == (12, 4, 1)
+    assert broadcast_shape((4, 1, 3), (5, 3)) == (4, 5, 3)
+    with pytest.raises(RuntimeError):
+        broadcast_shape((2, 3), (4, 3))
+    assert f32_bits(1.0) == 0x3F800000 and f32_bits(1e-5) == 0x3727C5AC
+    assert bf16_bits(1.0) == 0x3F80 and bf16_bits(float("inf")) == 0x7F80 and bf16_bits(float("nan")) & 0x7FC0 == 0x7FC0
+    assert itemsize(BF16) == 2 and itemsize(np.float32) == 4 and itemsize(np.int32) == 4
+
+
+# ---- ops: shape inference and error behaviour (op.py:219-267) ------------------------
+def test_op_shapes_and_errors():
+    ids = T((2, 5), np.int32, False)
+    w = T((11, 8))
+    assert GatherOp()(ids, w).shape == (2, 5, 8)
+    with pytest.raises(ValueError):
+        GatherOp()(T((10,), np.int32, False), w)
+    with pytest.raises(ValueError):
+        GatherOp()(ids, T((11, 8, 2)))
+    x = T((2, 5, 8))
+    g, b = T((8,)), T((8,))
+    y = LayerNormOp(eps=1e-5)(x, g, b)
+    assert y.shape == x.shape and y.op.op.eps == 1e-5 and y.op.inputs == (x, g, b)
+    assert LayerNormOp().eps == 1e-6          # the op's default (op.py:249)
+    assert x.layer_norm(g, b).op.op.eps == 1e-5   # the Tensor sugar's default (tensor.py:97)
+    with pytest.raises(ValueError):
+        LayerNormOp()(x, T((7,)), T((7,)))
+    with pytest.raises(ValueError):
+        LayerNormOp()(x, g, T((7,)))
+    with pytest.raises(ValueError):
+        RMSNormOp()(x, T((7,)))
+    assert RMSNormOp()(x).shape == x.shape and len(RMSNormOp()(x).op.inputs) == 1
+    assert SwiGLUOp()(x).shape == (2, 5, 4)
+    with pytest.raises(ValueError):
+        SwiGLUOp()(T((2, 5, 7)))
+    h, yy = AddLayerNormOp()(x, T((2, 5, 8)), g, b)
+    assert h.op is yy.op and h.op.outputs == (h, yy)
+    with pytest.raises(ValueError):
+        AddRMSNormOp()(x, T((2, 5, 4)))
+    q, k = T((2, 5, 4, 8)), T((2, 5, 2, 8))
+    c, s = T((16, 4), requires_grad=False), T((16, 4), requires_grad=False)
+    q2, k2 = RopeOp(rope_sign=-1)(q, k, c, s)
+    assert q2.shape == q.shape and k2.shape == k.shape
+    with pytest.raises(ValueError):
+        RopeOp(rope_sign=0)
+    with pytest.raises(ValueError):
+        RopeOp()(q, k, T((3, 4)), T((3, 4)))     # table shorter than T
+    assert EmbeddingSumOp()(ids, w, T((5, 8))).shape == (2, 5, 8)
+    with pytest.raises(ValueError):
+        EmbeddingSumOp()(ids, w, T((4, 8)))
+    assert (x + x).op.op.op_name == "Add" and x.gelu().op.op.op_name == "GELU"
+    # requires_grad propagates; gather ignores the integer operand
+    assert not GatherOp()(ids, T((11, 8), requires_grad=False)).requires_grad
+
+
+# ---- planner ------------------------------------------------------------------------
+def test_memory_planner_first_fit():
+    p = MemoryPlanner()
+    assert p.alloc("a", 100) == 0 and p.alloc("b", 300) == 256 and p.alloc("c", 10) == 768
+    p.free("a")
+    assert p.alloc("d", 200) == 0           # reuses the lowest hole that fits
+    p.free("b")
+    assert p.alloc("e", 512) == 256         # hole of 512 between d and c
+    assert p.alloc("f", 1) == 1024
+    assert p.peak == 1280 and p.alloc("a", 5) == 0   # known keys keep their offset
+    for off in p.offsets.values():
+        assert off % 256 == 0
+
+
+def test_planner_property_no_live_overlap():
+    rng = np.random.default_rng(7)
+    for _ in range(20):
+        n = 40
+        start = rng.integers(0, 30, n)
+        length = rng.integers(1, 10, n)
+        size = rng.integers(1, 5000, n)
+        p = MemoryPlanner()
+        end = start + length
+        for step in range(int(end.max()) + 1):
+            for i in range(n):
+                if end[i] == step - 1:
+                    p.free(i)
+            for i in range(n):
+                if start[i] == step:
+                    p.alloc(i, int(size[i]))
+        for i in range(n):
+            for j in range(i + 1, n):
+                if start[i] <= end[j] and start[j] <= end[i]:       # lifetimes intersect
+                    a0, a1 = p.offsets[i], p.offsets[i] + size[i]
+                    b0, b1 = p.offsets[j], p.offsets[j] + size[j]
+                    assert a1 <= b0 or b1 <= a0
+        assert p.peak >= max(p.offsets[i] + size[i] for i in range(n))
+
+
+def test_runtime_arena_views_and_execution_on_oracle_device():
+    rng = np.random.default_rng(3)
+    B, Tn, C, V = 2, 6, 16, 23
+    ids_np = rng.integers(0, V, (B, Tn), dtype=np.int32)
+    w_np = rng.standard_normal((V, C)).astype(np.float32)
+    ids, w = T((B, Tn), np.int32, False, ids_np), T((V, C), val=w_np)
+    g, b = T((C,), val=np.ones(C, np.float32)), T((C,), val=np.zeros(C, np.float32))
+    x = ids.gather(w)
+    h, y = x.add_layer_norm(x.gelu(), g, b)
+    out = h + y
+    rt = Runtime(device="cpu")
+    rt.backward(out, grad_scale=1.0)
+    # every activation and activation gradient is a view of the one arena
+    arena = rt.unified_arena.data
+    lo, hi = arena.ctypes.data, arena.ctypes.data + arena.nbytes
+    seen = []
+    for node in rt.topo:
+        for t in node.outputs:
+            for u in (t, t.grad):
+                if u is None:
+                    continue
+                a = u.storage.data
+                assert lo <= a.ctypes.data and a.ctypes.data + a.nbytes <= hi
+                assert (a.ctypes.data - lo) % 256 == 0
+                seen.append(u)
+    assert rt.arena_bytes == arena.nbytes and rt.arena_bytes % 256 == 0
+    # gradients flow: d(out)/dw is non-zero exactly on the gathered rows
+    dw = rt.backend.copy_to_host(w.grad)
+    used = np.zeros(V, bool)
+    used[ids_np.ravel()] = True
+    assert np.abs(dw[used]).sum() > 0 and not dw[~used].any()
+    # a second execute gives the same numbers (grads are re-zeroed)
+    rt.backward(out, grad_scale=1.0)
+    np.testing.assert_array_equal(rt.backend.copy_to_host(w.grad), dw)
+    # an output nobody consumes gets no gradient tensor
+    h2, y2 = x.add_rms_norm(x.gelu())
+    rt2 = Runtime(device="cpu")
+    rt2.build_topo(y2)
+    assert h2.grad is None and y2.grad is not None
+
+
+def test_runtime_rejects_ops_without_kernels():
+    class Bare(GELUOp):
+        pass
+    x = T((2, 4), val=np.zeros((2, 4), np.float32))
+    y = Bare()(x)
+    with pytest.raises(RuntimeError):
+        Runtime(device="cpu").build_topo(y)      # lookup is by exact type (backend.py:4938-4950)

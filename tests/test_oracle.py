@@ -1,0 +1,338 @@
+"""Pins the CPU restatement (oracle/cpu_ops.py) without a GPU.
+
+Each check is chosen so that a plausible mistake -- a dropped term, a wrong
+sign, a transposed operand, population vs sample variance, eps inside vs outside
+the square root -- fails it: float64 closed forms written independently
+(oracle/closed_form.py, after verify_model.py:127-135 and
+debug/check_qwen_kernel.py:195-342, 577-645), central finite differences
+(verify_model.py:65-77), algebraic invariants, and brute force on small inputs.
+"""
+import numpy as np
+import pytest
+
+from oracle import closed_form as cf
+from oracle import cpu_ops as K
+
+SEED = 1333
+
+
+def rng(k):
+    return np.random.default_rng(SEED + k)
+
+
+def close(a, b, rtol=1e-5, atol=1e-6):
+    np.testing.assert_allclose(np.asarray(a, np.float64), np.asarray(b, np.float64), rtol=rtol, atol=atol)
+
+
+# ---- GELU ---------------------------------------------------------------------
+def test_gelu_matches_closed_form_and_special_values():
+    x = rng(5).standard_normal((2, 16, 64), dtype=np.float32)      # probe_gelu recipe
+    close(K.gelu_forward(x), cf.gelu(x))
+    sp = np.array([0.0, 30.0, -30.0], np.float32)
+    y = K.gelu_forward(sp)
+    assert y[0] == 0 and y[1] == 30 and y[2] == 0
+    dx = np.zeros(3, np.float32)
+    K.gelu_backward_into(sp, np.ones(3, np.float32), dx)
+    assert dx[0] == 0.5 and dx[1] == 1.0 and dx[2] == 0.0
+    # the constants are the reference's (backend.py:18-20)
+    assert K.GELU_C == 0.7978845608028654 and K.GELU_A == 0.044715 and K.GELU_A3 == 0.134145
+    assert abs(K.GELU_C - np.sqrt(2 / np.pi)) < 1e-15 and abs(K.GELU_A3 - 3 * K.GELU_A) < 1e-15
+
+
+def test_gelu_backward_finite_difference_and_accumulate():
+    r = rng(5)
+    x = r.standard_normal((7, 33), dtype=np.float32)
+    dy = r.standard_normal((7, 33), dtype=np.float32)
+    dx = np.zeros_like(x)
+    K.gelu_backward_into(x, dy, dx)
+    close(dx, dy * cf.gelu_grad(x), rtol=2e-5, atol=2e-6)
+    idx = r.choice(x.size, 25, replace=False)
+    fd = cf.finite_diff(lambda a: float((cf.gelu(a) * dy).sum()), x, idx, eps=1e-4)
+    close(dx.reshape(-1)[idx], fd, rtol=1e-4, atol=1e-5)
+    base = r.standard_normal(x.shape, dtype=np.float32)
+    acc = base.copy()
+    K.gelu_backward_into(x, dy, acc)            # "grad += ..." (backend.py:414)
+    close(acc, base + dx, atol=2e-6)
+
+
+# ---- ReLU^2 (closed form only: the reference has none) ---------------------------
+def test_relu2():
+    r = rng(11)
+    x = r.standard_normal((5, 40), dtype=np.float32)
+    dy = r.standard_normal((5, 40), dtype=np.float32)
+    close(K.relu2_forward(x), cf.relu2(x))
+    dx = np.zeros_like(x)
+    K.relu2_backward_into(x, dy, dx)
+    close(dx, dy * cf.relu2_grad(x))
+    assert (K.relu2_forward(np.array([-1.0, 0.0, -0.0, 2.0], np.float32)) == [0, 0, 0, 4]).all()
+
+
+# ---- LayerNorm ------------------------------------------------------------------
+def _ln_case(k=4, shape=(2, 16, 64)):
+    r = rng(k)
+    C = shape[-1]
+    return (r.standard_normal(shape, dtype=np.float32), r.standard_normal(C, dtype=np.float32),
+            r.standard_normal(C, dtype=np.float32), r.standard_normal(shape, dtype=np.float32))
+
+
+def test_layernorm_forward_closed_form_and_invariants():
+    x, g, b, _ = _ln_case()
+    y64, _, _ = cf.layernorm(x, g, b, 1e-5)
+    close(K.layernorm_forward(x, g, b, 1e-5), y64, rtol=2e-5, atol=2e-6)
+    plain = K.layernorm_forward(x, np.ones_like(g), np.zeros_like(b), 1e-5)
+    assert np.abs(plain.mean(-1)).max() < 1e-6          # mean 0
+    assert np.abs(plain.var(-1) - 1).max() < 1e-4       # population variance 1 (not the sample one: 64/63)
+    # eps sits inside the square root: a constant row maps to beta
+    const = np.full((3, 8), 2.5, np.float32)
+    close(K.layernorm_forward(const, np.ones(8, np.float32), np.full(8, 0.25, np.float32), 1e-5), 0.25)
+
+
+def test_layernorm_backward_closed_form_fd_and_invariants():
+    x, g, b, dy = _ln_case()
+    dx, dg, db = np.zeros_like(x), np.zeros_like(g), np.zeros_like(b)
+    K.layernorm_backward_into(x, g, dy, 1e-5, dx, dg, db)
+    dx64, dg64, db64 = cf.layernorm_grads(x, g, dy, 1e-5)
+    close(dx, dx64, rtol=2e-5, atol=2e-6)
+    close(dg, dg64, rtol=2e-5, atol=5e-6)
+    close(db, db64, rtol=2e-5, atol=5e-6)
+    r = rng(40)
+    idx = r.choice(x.size, 20, replace=False)
+    fd = cf.finite_diff(lambda a: float((cf.layernorm(a, g, b, 1e-5)[0] * dy).sum()), x, idx, eps=1e-4)
+    close(dx.reshape(-1)[idx], fd, rtol=2e-3, atol=2e-4)
+    # gamma = 1: each row of dx sums to zero and is orthogonal to x_hat
+    one = np.ones_like(g)
+    dx1 = np.zeros_like(x)
+    K.layernorm_backward_into(x, one, dy, 1e-5, dx1, None, None)
+    _, _, xh = cf.layernorm(x, one, np.zeros_like(b), 1e-5)
+    assert np.abs(dx1.sum(-1)).max() < 2e-5
+    assert np.abs((dx1 * xh).sum(-1)).max() < 1e-3      # exact up to eps / (var + eps)
+    # accumulation into existing grads
+    base = r.standard_normal(x.shape, dtype=np.float32)
+    acc = base.copy()
+    K.layernorm_backward_into(x, g, dy, 1e-5, acc, None, None)
+    close(acc, base + dx, atol=3e-6)
+
+
+# ---- RMSNorm ----------------------------------------------------------------------
+def test_rmsnorm_forward_backward():
+    r = rng(6)
+    x = (0.02 * r.standard_normal((2, 8, 96))).astype(np.float32)   # x ~ 0.02 N (check_qwen_kernel.py:1097-1139)
+    g = (1 + 0.02 * r.standard_normal(96)).astype(np.float32)
+    g[0] = 0.0
+    dz = r.standard_normal(x.shape, dtype=np.float32)
+    z64, _, _ = cf.rmsnorm(x, g, 1e-6)
+    close(K.rmsnorm_forward(x, g, 1e-6), z64, rtol=2e-5, atol=2e-6)
+    close(K.rmsnorm_forward(x, None, 1e-6), cf.rmsnorm(x, None, 1e-6)[0], rtol=2e-5, atol=2e-6)
+    dx, dg = np.zeros_like(x), np.zeros_like(g)
+    K.rmsnorm_backward_into(x, g, dz, 1e-6, dx, dg)
+    dx64, dg64 = cf.rmsnorm_grads(x, g, dz, 1e-6)
+    close(dx, dx64, rtol=5e-5, atol=1e-4 * np.abs(dx64).max())
+    close(dg, dg64, rtol=2e-5, atol=1e-5)
+    idx = r.choice(x.size, 20, replace=False)
+    fd = cf.finite_diff(lambda a: float((cf.rmsnorm(a, g, 1e-6)[0] * dz).sum()), x, idx, eps=1e-6)
+    close(dx.reshape(-1)[idx], fd, rtol=5e-3, atol=5e-3 * np.abs(fd).max())
+    # gamma = 1 and eps -> 0: dx is orthogonal to x row by row
+    xb = r.standard_normal((5, 64), dtype=np.float32)
+    d1 = np.zeros_like(xb)
+    K.rmsnorm_backward_into(xb, None, dz.reshape(-1, 96)[:5, :64].copy(), 0.0, d1, None)
+    assert np.abs((d1 * xb).sum(-1)).max() < 1e-4
+    # unit-RMS rows come back unchanged
+    u = np.ones((2, 16), np.float32)
+    close(K.rmsnorm_forward(u, None, 0.0), u)
+
+
+def test_add_norm_is_add_then_norm():
+    r = rng(9)
+    x, res = r.standard_normal((4, 32), dtype=np.float32), r.standard_normal((4, 32), dtype=np.float32)
+    g, b = r.standard_normal(32, dtype=np.float32), r.standard_normal(32, dtype=np.float32)
+    h, y = K.add_norm_forward("layer", x, res, g, b, 1e-5)
+    assert np.array_equal(h, x + res) and np.array_equal(y, K.layernorm_forward(x + res, g, b, 1e-5))
+    h, z = K.add_norm_forward("rms", x, res, g, None, 1e-6)
+    assert np.array_equal(z, K.rmsnorm_forward(x + res, g, 1e-6))
+
+
+# ---- SwiGLU -------------------------------------------------------------------------
+def test_swiglu():
+    r = rng(12)
+    gu = (2 * r.standard_normal((6, 2 * 40))).astype(np.float32)
+    dh = r.standard_normal((6, 40), dtype=np.float32)
+    close(K.swiglu_forward(gu), cf.swiglu(gu), rtol=2e-5, atol=2e-6)
+    dgu = K.swiglu_backward(gu, dh)
+    close(dgu, cf.swiglu_grads(gu, dh), rtol=2e-5, atol=2e-6)
+    idx = r.choice(gu.size, 30, replace=False)
+    fd = cf.finite_diff(lambda a: float((cf.swiglu(a) * dh).sum()), gu, idx, eps=1e-5)
+    close(dgu.reshape(-1)[idx], fd, rtol=1e-4, atol=1e-5)
+    # gate = first half, up = second half; silu(0) = 0; the up gradient of a zero gate is 0
+    z = np.zeros((1, 8), np.float32)
+    z[0, 4:] = 3.0
+    assert not K.swiglu_forward(z).any()
+    d = K.swiglu_backward(z, np.ones((1, 4), np.float32))
+    close(d[0, :4], 0.5 * 3.0)       # d/dg silu(g) u at g = 0 is u / 2
+    assert not d[0, 4:].any()
+
+
+# ---- RoPE -----------------------------------------------------------------------------
+def test_rope_tables():
+    cos, sin = K.rope_tables(16, 8, 1e4)
+    assert cos.shape == (16, 4) and cos.dtype == np.float32
+    assert (cos[0] == 1).all() and (sin[0] == 0).all()
+    inv = 1e4 ** (-np.arange(0, 8, 2) / 8)
+    close(cos, np.cos(np.arange(16)[:, None] * inv), atol=2e-6)
+    close(sin, np.sin(np.arange(16)[:, None] * inv), atol=2e-6)
+
+
+@pytest.mark.parametrize("sign", [1, -1])
+def test_rope_signed_closed_form_and_invariants(sign):
+    r = rng(15)
+    B, T, H, HKV, D = 2, 9, 3, 1, 16
+    q = r.standard_normal((B, T, H, D), dtype=np.float32)
+    k = r.standard_normal((B, T, HKV, D), dtype=np.float32)
+    cos, sin = K.rope_tables(T, D, 1e6)
+    fq, fk = q.copy(), k.copy()
+    K.rope_signed(fq, fk, cos, sin, sign, False)
+    close(fq, cf.rope(q, cos, sin, sign), atol=2e-6)
+    close(fk, cf.rope(k, cos, sin, sign), atol=2e-6)
+    assert np.array_equal(fq[:, 0], q[:, 0])                 # position 0 is the identity
+    h = D // 2
+    close(fq[..., :h] ** 2 + fq[..., h:] ** 2, q[..., :h] ** 2 + q[..., h:] ** 2, atol=1e-5)
+    bq, bk = fq.copy(), fk.copy()
+    K.rope_signed(bq, bk, cos, sin, sign, True)              # backward is the transpose = inverse
+    close(bq, q, atol=2e-6)
+    iq, ik = fq.copy(), fk.copy()
+    K.rope_signed(iq, ik, cos, sin, -sign, False)            # the two conventions are mutual inverses
+    close(iq, q, atol=2e-6)
+    # <R x, g> = <x, R^T g>
+    g = r.standard_normal(q.shape, dtype=np.float32)
+    tg, _ = g.copy(), None
+    K.rope_signed(tg, k.copy(), cos, sin, sign, True)
+    assert abs(float((fq.astype(np.float64) * g).sum() - (q.astype(np.float64) * tg).sum())) < 1e-3
+
+
+def test_rope_nanochat_is_sign_minus_one():
+    r = rng(16)
+    q = r.standard_normal((2, 7, 2, 8), dtype=np.float32)
+    k = r.standard_normal((2, 7, 1, 8), dtype=np.float32)
+    cos, sin = K.rope_tables(7, 8, 1e5)
+    for backward in (False, True):
+        a, b = q.copy(), k.copy()
+        K.rope_nanochat(a, b, cos, sin, backward)
+        c, d = q.copy(), k.copy()
+        K.rope_signed(c, d, cos, sin, -1, backward)
+        assert np.array_equal(a, c) and np.array_equal(b, d)
+    # the sign: with cos = 0, sin = 1 the nanochat forward maps (lo, hi) -> (hi, -lo)
+    one = np.ones((1, 1), np.float32)
+    x = np.array([[[[2.0, 5.0]]]], np.float32)
+    y = x.copy()
+    K.rope_nanochat(y, None, 0 * one, one, False)
+    assert (y.ravel() == [5.0, -2.0]).all()
+    y = x.copy()
+    K.rope_signed(y, None, 0 * one, one, 1, False)           # HF: (lo, hi) -> (-hi, lo)
+    assert (y.ravel() == [-5.0, 2.0]).all()
+
+
+# ---- embedding -----------------------------------------------------------------------
+def test_gather_reference_vectors():
+    """verify_model.py:298-318 (seed 1234, B,T,V,C = 2,3,11,4)."""
+    r = np.random.default_rng(1234)
+    B, T, V, C = 2, 3, 11, 4
+    idx = r.integers(0, V, size=(B, T), dtype=np.int32)
+    w = (r.standard_normal((V, C)) * 0.1).astype(np.float32)
+    out = K.gather_forward(idx, w)
+    for b in range(B):
+        for t in range(T):
+            assert np.array_equal(out[b, t], w[idx[b, t]])
+    # d/dw of sum(out) counts occurrences (the scalar loss of the reference's case)
+    dW = np.zeros_like(w)
+    K.gather_backward_into(idx, np.ones((B, T, C), np.float32), dW)
+    assert np.array_equal(dW[:, 0], np.bincount(idx.ravel(), minlength=V).astype(np.float32))
+
+
+def test_gather_backward_is_row_order_loop():
+    r = rng(20)
+    B, T, V, C = 3, 50, 7, 5
+    ids = r.integers(0, V, size=(B, T), dtype=np.int32)
+    dY = r.standard_normal((B, T, C), dtype=np.float32)
+    dW = np.zeros((V, C), np.float32)
+    K.gather_backward_into(ids, dY, dW)
+    brute = np.zeros((V, C), np.float32)
+    for n, t in enumerate(ids.ravel()):
+        brute[t] += dY.reshape(-1, C)[n]              # fp32, ascending row order
+    assert np.array_equal(dW, brute)
+    close(dW.sum(0), dY.reshape(-1, C).sum(0), atol=1e-4)
+    close(dW, cf.gather_backward(ids, dY, V), atol=1e-5)
+    with pytest.raises(IndexError):
+        K.gather_forward(np.array([[V]], np.int32), np.zeros((V, C), np.float32))
+
+
+def test_embedding_sum():
+    r = rng(19)
+    B, T, V, C = 2, 6, 13, 4
+    ids = r.integers(0, V, size=(B, T), dtype=np.int32)
+    wte = r.standard_normal((V, C), dtype=np.float32)
+    wpe = r.standard_normal((T, C), dtype=np.float32)
+    out = K.embedding_sum_forward(ids, wte, wpe)
+    assert np.array_equal(out, wte[ids] + wpe[None, :, :])
+    dY = r.standard_normal((B, T, C), dtype=np.float32)
+    dwte, dwpe = np.zeros_like(wte), np.zeros_like(wpe)
+    K.embedding_sum_backward_into(ids, dY, dwte, dwpe)
+    seq = np.zeros_like(wpe)
+    for b in range(B):
+        seq += dY[b]
+    assert np.array_equal(dwpe, seq)                 # sum over batch, b ascending
+    ref = np.zeros_like(wte)
+    K.gather_backward_into(ids, dY, ref)
+    assert np.array_equal(dwte, ref)
+
+
+def test_add_backward_broadcast():
+    r = rng(21)
+    g = r.standard_normal((3, 4, 5), dtype=np.float32)
+    same, bc = np.zeros((3, 4, 5), np.float32), np.zeros((4, 5), np.float32)
+    K.add_backward_into(g, same)
+    K.add_backward_into(g, bc)
+    assert np.array_equal(same, g)
+    close(bc, g.sum(0), atol=1e-6)
+
+
+# ---- bf16 ---------------------------------------------------------------------------
+def _bf16_scalar(bits):
+    """integer restatement of utils.py:20-27 on a uint32 bit pattern"""
+    if bits & 0x7F800000 == 0x7F800000:
+        return ((bits >> 16) | (0x0040 if bits & 0x007FFFFF else 0)) & 0xFFFF
+    return ((bits + 0x7FFF + ((bits >> 16) & 1)) >> 16) & 0xFFFF
+
+
+def test_bf16_rounding_rule():
+    cases = {
+        0x3F800000: 0x3F80,   # 1.0
+        0x3F808000: 0x3F80,   # tie, even mantissa -> down
+        0x3F818000: 0x3F82,   # tie, odd mantissa -> up
+        0x3F808001: 0x3F81,   # just above the tie
+        0x7F800000: 0x7F80,   # +inf kept
+        0xFF800000: 0xFF80,   # -inf kept
+        0x7F800001: 0x7FC0,   # signalling NaN -> quiet
+        0x7FC00000: 0x7FC0,
+        0x7F7FFFFF: 0x7F80,   # max finite rounds to inf
+        0x80000000: 0x8000,   # -0
+        0x00000001: 0x0000,
+    }
+    bits = np.array(list(cases), dtype=np.uint32)
+    got = K.f32_to_bf16_bits(bits.view(np.float32))
+    assert got.tolist() == list(cases.values())
+    # dense sample of all 2^32 patterns against the scalar rule, plus every exponent edge
+    r = rng(30)
+    sample = np.concatenate([r.integers(0, 2 ** 32, size=200_000, dtype=np.uint64).astype(np.uint32),
+                             (np.arange(512, dtype=np.uint32) << 23)[:, None].repeat(4, 1).ravel()
+                             + np.tile(np.array([0, 0x7FFF, 0x8000, 0x8001], np.uint32), 512)])
+    got = K.f32_to_bf16_bits(sample.view(np.float32))
+    want = np.array([_bf16_scalar(int(b)) for b in sample], dtype=np.uint16)
+    assert np.array_equal(got, want)
+    # widening is exact and rounding is idempotent
+    back = K.bf16_bits_to_f32(got)
+    finite = np.isfinite(back)
+    assert np.array_equal(K.f32_to_bf16_bits(back[finite]), got[finite])
+    # product-side helpers implement the same rule
+    from autograd_amd import utils
+    assert np.array_equal(utils.f32_array_to_bf16_bits(sample.view(np.float32)), want)
+    assert all(utils.bf16_bits(float(np.uint32(b).view(np.float32))) == w
+               for b, w in cases.items() if not np.isnan(np.uint32(b).view(np.float32)))
