@@ -36,7 +36,7 @@ from .utils import (bf16_bits, bf16_bits_to_f32_array, f32_array_to_bf16_bits, f
                     xavier_uniform)
 
 F32, BF16 = 0, 1
-ACC_INPUT_GRAD, ACC_PARAM_GRAD = 1, 2
+ACC_INPUT_GRAD, ACC_PARAM_GRAD, ACC_INPUT_GRAD2 = 1, 2, 4
 
 
 class Backend:
@@ -406,23 +406,11 @@ class HipBackend(Backend):
             self._norm_backward(kernel, node, h, y.grad, gamma, beta, None, None, None, op.eps, pflags, scratch)
             return
         first, second = targets[0], (targets[1] if len(targets) > 1 else None)
-        f1 = self._grad_flag(node, first)
-        if second is not None and self._grad_flag(node, second) == 0 and f1 == 0:
-            # both operands take a plain store: one launch writes both
-            self._norm_backward(kernel, node, h, y.grad, gamma, beta, dres, first.grad, second.grad,
-                                op.eps, pflags, scratch)
-            return
-        if second is None:
-            self._norm_backward(kernel, node, h, y.grad, gamma, beta, dres, first.grad, None,
-                                op.eps, f1 | pflags, scratch)
-            return
-        # mixed write modes: form dh_total in h.grad's place, then hand it on
-        if dres is None:
-            raise RuntimeError("fused add+norm backward: residual gradient buffer missing")
-        self._norm_backward(kernel, node, h, y.grad, gamma, beta, dres, dres, None, op.eps, pflags, scratch)
-        for t in targets:
-            self._launch("add_residual_backward", [dres, t.grad],
-                         [_dt(h), self._grad_flag(node, t)] + _lo_hi(h.numel))
+        flags = pflags | self._grad_flag(node, first)
+        if second is not None and self._grad_flag(node, second):
+            flags |= ACC_INPUT_GRAD2
+        self._norm_backward(kernel, node, h, y.grad, gamma, beta, dres, first.grad,
+                            second.grad if second is not None else None, op.eps, flags, scratch)
 
     # -- rotary (backend.py:1382-1417, 1755-1782, 1937-1958) ----------------------------
     def _rope(self, q, k, cos, sin, sign, backward):

@@ -17,7 +17,7 @@ LIB_PATH = Path(__file__).resolve().parent / "libautograd_hip.so"
 
 F32, BF16 = 0, 1
 NORM_LAYER, NORM_RMS = 0, 1
-ACC_INPUT_GRAD, ACC_PARAM_GRAD = 1, 2
+ACC_INPUT_GRAD, ACC_PARAM_GRAD, ACC_INPUT_GRAD2 = 1, 2, 4
 OK, EINVAL, EHIP, ENOKERNEL, EINDEX, EWORKSPACE = 0, -1, -2, -3, -4, -5
 
 _ctx = C.c_void_p

@@ -189,6 +189,7 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
     const bool want_pg = a.pgamma != nullptr;
     const bool want_pb = a.pbeta != nullptr;
     const bool acc = (a.flags & AGRAD_ACC_INPUT_GRAD) != 0;
+    const bool acc2 = (a.flags & AGRAD_ACC_INPUT_GRAD2) != 0;
 
     bool on[NV];
     float gam[NV][VEC], pg[NV][VEC], pb[NV][VEC];
@@ -293,25 +294,31 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
                         for (int k = 0; k < VEC; ++k)
                             t[k] = (g[i][k] - xv[i][k] * c2) * scale;
                     }
-                    if (acc) {
-                        float old[VEC];
-                        VecIO<T, VEC>::load(a.dx + base + col, old);
-                        if (a.dres != nullptr) {
-                            float r[VEC];
-                            VecIO<T, VEC>::load(a.dres + base + col, r);
-#pragma unroll
-                            for (int k = 0; k < VEC; ++k) old[k] = old[k] + r[k];
-                        }
-#pragma unroll
-                        for (int k = 0; k < VEC; ++k) t[k] = old[k] + t[k];
-                    } else if (a.dres != nullptr) {
+                    if (a.dres != nullptr) {
                         float r[VEC];
                         VecIO<T, VEC>::load(a.dres + base + col, r);
 #pragma unroll
                         for (int k = 0; k < VEC; ++k) t[k] = r[k] + t[k];
                     }
+                    if (a.dx2 != nullptr) {
+                        float t2[VEC];
+                        if (acc2) {
+                            VecIO<T, VEC>::load(a.dx2 + base + col, t2);
+#pragma unroll
+                            for (int k = 0; k < VEC; ++k) t2[k] = t2[k] + t[k];
+                        } else {
+#pragma unroll
+                            for (int k = 0; k < VEC; ++k) t2[k] = t[k];
+                        }
+                        VecIO<T, VEC>::store(a.dx2 + base + col, t2);
+                    }
+                    if (acc) {
+                        float old[VEC];
+                        VecIO<T, VEC>::load(a.dx + base + col, old);
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) t[k] = old[k] + t[k];
+                    }
                     VecIO<T, VEC>::store(a.dx + base + col, t);
-                    if (a.dx2 != nullptr) VecIO<T, VEC>::store(a.dx2 + base + col, t);
                 }
             }
         }
@@ -444,6 +451,7 @@ __global__ void __launch_bounds__(256) norm_bwd_generic_kernel(const NormBwdArgs
     const float fC = (float)C;
     const bool is_ln = a.kind == AGRAD_NORM_LAYER;
     const bool acc = (a.flags & AGRAD_ACC_INPUT_GRAD) != 0;
+    const bool acc2 = (a.flags & AGRAD_ACC_INPUT_GRAD2) != 0;
     bool first = true;
     SlotRing ring;
     for (uint64_t row = blockIdx.x; row < a.rows; row += gridDim.x) {
@@ -500,15 +508,9 @@ __global__ void __launch_bounds__(256) norm_bwd_generic_kernel(const NormBwdArgs
                 } else {
                     t = (dyg - xh * c2) * scale;
                 }
-                if (acc) {
-                    float old = ld1(a.dx + base + c);
-                    if (a.dres != nullptr) old = old + ld1(a.dres + base + c);
-                    t = old + t;
-                } else if (a.dres != nullptr) {
-                    t = ld1(a.dres + base + c) + t;
-                }
-                st1(a.dx + base + c, t);
-                if (a.dx2 != nullptr) st1(a.dx2 + base + c, t);
+                if (a.dres != nullptr) t = ld1(a.dres + base + c) + t;
+                if (a.dx2 != nullptr) st1(a.dx2 + base + c, acc2 ? (ld1(a.dx2 + base + c) + t) : t);
+                st1(a.dx + base + c, acc ? (ld1(a.dx + base + c) + t) : t);
             }
         }
     }

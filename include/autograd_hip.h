@@ -43,7 +43,8 @@ enum { AGRAD_NORM_LAYER = 0, AGRAD_NORM_RMS = 1 };
 /* Flag bits for backward entry points.                                       */
 enum {
     AGRAD_ACC_INPUT_GRAD = 1u, /* dx += ... (CPU semantics, backend.py:414,477-487); else dx = ... */
-    AGRAD_ACC_PARAM_GRAD = 2u  /* dgamma/dbeta/dW += ...; else =                                   */
+    AGRAD_ACC_PARAM_GRAD = 2u, /* dgamma/dbeta/dW += ...; else =                                   */
+    AGRAD_ACC_INPUT_GRAD2 = 4u /* norm backward: the same choice for the second output dx2         */
 };
 
 /* ---- context, memory, passes --------------------------------------------
@@ -126,8 +127,9 @@ int agrad_norm_forward(agrad_ctx* ctx, int kind, int dtype,
 /* Bytes of workspace agrad_norm_backward needs for the column reductions.    */
 uint64_t agrad_norm_backward_workspace_bytes(uint64_t rows, uint32_t C, int dtype);
 /* Norm backward.  x is the tensor that was normalised (h when a residual was
- * fused).  dx = [dx if ACC_INPUT_GRAD] + [dres_in] + dnorm; dx2 (optional)
- * receives the same values (the second operand of a fused residual add).
+ * fused).  dx = [dx if ACC_INPUT_GRAD] + ([dres_in] + dnorm); dx2 (optional, the
+ * second operand of a fused residual add) = [dx2 if ACC_INPUT_GRAD2] + the same.
+ * dres_in may be the same buffer as dx or dx2 only when that output is stored.
  * dgamma / dbeta (optional) are reduced over rows in two deterministic stages.
  * cpu_layernorm_backward (backend.py:435-487); RMSNorm slices backend.py:1228-1251,
  * 1990-2011; rmsnorm_backward's fused residual_grad (metal_ops.metal:8107-8257). */

@@ -150,9 +150,13 @@ def test_norm_backward_accumulate_and_residual_grad(ctx, kind):
     out = G.norm_backward(ctx, KINDS[kind], x, gamma, dy, eps, dres=dres, dx_init=dx0, want_dx2=True,
                           dgamma_init=dg0, dbeta_init=db0, want_dbeta=(kind == "layer"), flags=flags)
     dx, dgamma, dbeta = _norm_ref_backward(kind, x, gamma, dy, eps)
-    want = (dx0 + dres) + dx
+    want = dx0 + (dres + dx)
     assert_fp32_close(out["dx"], want, "accumulated dx", rtol=1e-5, atol=2e-6)
-    np.testing.assert_array_equal(out["dx"], out["dx2"])
+    assert_fp32_close(out["dx2"], dres + dx, "stored dx2", rtol=1e-5, atol=2e-6)   # dx2 has its own flag
+    out2 = G.norm_backward(ctx, KINDS[kind], x, gamma, dy, eps, dres=dres, want_dx2=True,
+                           want_dgamma=False, want_dbeta=False, flags=capi.ACC_INPUT_GRAD2)
+    assert_fp32_close(out2["dx"], dres + dx, "stored dx", rtol=1e-5, atol=2e-6)
+    assert_fp32_close(out2["dx2"], 9 + (dres + dx), "accumulated dx2", rtol=1e-5, atol=4e-6)
     assert_fp32_close(out["dgamma"], dg0 + dgamma, "accumulated dgamma", rtol=1e-5, atol=3e-6)
     if kind == "layer":
         assert_fp32_close(out["dbeta"], db0 + dbeta, "accumulated dbeta", rtol=1e-5, atol=3e-6)

@@ -179,8 +179,12 @@ def test_config1_tiny_gpt2_chain():
 
     (c_out, c_g), (h_out, h_g) = both(build, upstream)
     assert_fp32_close(h_out[0], c_out[0], "config 1 forward")
-    assert_fp32_close(h_g["wte"], c_g["wte"], "wte.grad", rtol=1e-5, atol=2e-6)
-    assert_fp32_close(h_g["wpe"], c_g["wpe"], "wpe.grad", rtol=1e-5, atol=2e-6)
+    # Three ops deep, and LayerNorm of rows with std 0.03 multiplies dy by ~35:
+    # an element where that cancels to O(1) carries the rounding of O(35) terms,
+    # so the absolute budget is set on the gradient's own scale.
+    scale = max(1.0, float(np.abs(c_g["wte"]).max()))
+    assert_fp32_close(h_g["wte"], c_g["wte"], "wte.grad", rtol=1e-5, atol=2e-6 * scale)
+    assert_fp32_close(h_g["wpe"], c_g["wpe"], "wpe.grad", rtol=1e-5, atol=2e-6 * scale)
     atol = 1e-6 * np.sqrt(B * T)
     assert_fp32_close(h_g["gamma"], c_g["gamma"], "gamma.grad", rtol=1e-5, atol=atol)
     assert_fp32_close(h_g["beta"], c_g["beta"], "beta.grad", rtol=1e-5, atol=atol)
