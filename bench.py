@@ -1,0 +1,449 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused layer-op path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config I]
+                    [--workload-only] [--no-cpu] [--iters N]
+
+A step is one forward + backward pass of every op of the workload configuration
+(default --config 1: the nanochat d6 shape, fp32) over one batch of synthetic
+data already resident in HBM.  Prints ONE JSON line:
+
+  value / unit     whole-step algorithmic GB/s (sum of the ops' algorithmic bytes
+                   / wall-clock step time, synchronised on both sides)
+  tokens_per_s     B*T / step time
+  per_op           every op and direction of the workload, timed on its own with
+                   HIP events on the library's stream over rotating buffer sets
+                   (so the working set exceeds the 256 MB Infinity Cache)
+  roofline         the dominant kernel of the step (largest share of time)
+  cpu_baseline     the numpy restatement of the reference's CPU kernels, timed
+                   on this host with the reference's protocol (2 warm-up + 5
+                   timed passes, timing_ops.py:76-100)
+  all_configs      the same per-op table for the other configurations
+
+All device calls go through the C ABI (autograd_amd/capi.py).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import platform
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+from autograd_amd import capi  # noqa: E402
+from autograd_amd.configs import CONFIGS, op_bytes  # noqa: E402
+from autograd_amd.utils import f32_array_to_bf16_bits  # noqa: E402
+
+METRIC = "HBM GB/s (% of 8 TB/s) + tokens/s for fused norm/act/RoPE/embed fwd+bwd"
+HBM_PEAK_GBS = 8000.0
+ROTATE_BYTES = 768 << 20      # cycle at least this much distinct memory per op
+MAX_SETS = 8
+
+
+def vp(d, off=0):
+    return None if d is None else C.c_void_p(d.ptr + off)
+
+
+class Pool:
+    """Device buffers; large ones are filled by tiling a 16 MiB chunk of N(0,1)
+    samples on the device, so multi-GB operands need no multi-GB host arrays."""
+
+    def __init__(self, ctx, seed):
+        self.ctx = ctx
+        rng = np.random.default_rng(seed)
+        chunk = rng.standard_normal(4 << 20, dtype=np.float32)
+        self.src = {"f32": ctx.upload(chunk), "bf16": ctx.upload(f32_array_to_bf16_bits(chunk))}
+        self.bufs = []
+
+    def _new(self, numel, np_dtype):
+        d = self.ctx.empty((int(numel),), np_dtype)
+        self.bufs.append(d)
+        return d
+
+    def normal(self, numel, dtype):
+        d = self._new(numel, np.uint16 if dtype == "bf16" else np.float32)
+        src = self.src[dtype]
+        off = 0
+        while off < d.nbytes:
+            n = min(src.nbytes, d.nbytes - off)
+            self.ctx.call("agrad_copy", vp(src), vp(d, off), n)
+            off += n
+        return d
+
+    def empty(self, numel, dtype):
+        return self._new(numel, np.uint16 if dtype == "bf16" else np.float32)
+
+    def raw(self, nbytes):
+        return self._new(nbytes, np.uint8)
+
+    def upload(self, arr):
+        d = self.ctx.upload(arr)
+        self.bufs.append(d)
+        return d
+
+    def release(self):
+        self.ctx.synchronize()
+        for d in self.bufs:
+            d.free()
+        for d in self.src.values():
+            d.free()
+        self.bufs = []
+
+
+class Case:
+    def __init__(self, op, direction, nbytes, nsets, launch, kernel):
+        self.op, self.direction, self.nbytes, self.nsets = op, direction, nbytes, nsets
+        self.launch, self.kernel = launch, kernel
+        self.us = None
+
+
+def n_sets(working_bytes):
+    return int(max(1, min(MAX_SETS, -(-ROTATE_BYTES // max(working_bytes, 1)))))
+
+
+def token_ids(cfg, rng, n):
+    if cfg.embed_dist.startswith("zipf"):
+        s = float(cfg.embed_dist[4:])
+        p = np.arange(1, cfg.V + 1, dtype=np.float64) ** (-s)
+        p /= p.sum()
+        return rng.choice(cfg.V, size=n, p=p).astype(np.int32)
+    return rng.integers(0, cfg.V, size=n, dtype=np.int32)
+
+
+def build_cases(ctx, cfg, pool):
+    """every op of the config, forward and backward, as launchable cases"""
+    rng = np.random.default_rng(cfg.seed)
+    dt = capi.BF16 if cfg.dtype == "bf16" else capi.F32
+    N, Cw, e = cfg.N, cfg.C, cfg.esize
+    cases = []
+    ids0 = token_ids(cfg, rng, N) if cfg.embed else None
+    distinct = int(np.unique(ids0).size) if ids0 is not None else None
+    nbytes = op_bytes(cfg, distinct)
+
+    if cfg.embed:
+        name = cfg.embed
+        k = n_sets(2 * N * Cw * e)
+        W = pool.normal(cfg.V * Cw, cfg.dtype)
+        wpe = pool.normal(cfg.T * Cw, cfg.dtype) if name == "gather_sum" else None
+        ids = [pool.upload(ids0 if i == 0 else token_ids(cfg, rng, N)) for i in range(k)]
+        out = [pool.empty(N * Cw, cfg.dtype) for _ in range(k)]
+        dY = [pool.normal(N * Cw, cfg.dtype) for _ in range(k)]
+        dW = pool.empty(cfg.V * Cw, cfg.dtype)
+        dwpe = pool.empty(cfg.T * Cw, cfg.dtype) if wpe is not None else None
+        ws_bytes = ctx.lib.agrad_embedding_backward_workspace_bytes(N, Cw, cfg.V, dt)
+        ws = pool.raw(ws_bytes)
+        ctx.call("agrad_fill", dW.ptr, 0, 0, 1, dW.nbytes)
+
+        def fwd(i, ids=ids, out=out):
+            ctx.call("agrad_gather_forward", dt, vp(ids[i]), vp(W), vp(wpe), vp(out[i]), N, cfg.T, Cw, cfg.V)
+
+        def bwd(i, ids=ids, dY=dY):
+            ctx.call("agrad_embedding_backward", dt, vp(ids[i]), vp(dY[i]), vp(dW), vp(ws), ws_bytes, N, Cw, cfg.V, 0)
+            if dwpe is not None:
+                ctx.call("agrad_pos_embedding_backward", dt, vp(dY[i]), vp(dwpe), cfg.B, cfg.T, Cw, 0)
+
+        def zero(i):
+            ctx.call("agrad_fill", dW.ptr, 0, 0, 1, dW.nbytes)
+
+        cases.append(Case(name, "fwd", nbytes[name][0], k, fwd, "gather"))
+        cases.append(Case(name, "bwd", nbytes[name][1], k, bwd, "emb_segment_sum_kernel"))
+        cases.append(Case(name + "_grad_zero_fill", "aux", cfg.V * Cw * e, 1, zero, "fill16_kernel"))
+
+    if cfg.norm:
+        name = ("add+" if cfg.norm_residual else "") + cfg.norm + "norm"
+        kind = capi.NORM_LAYER if cfg.norm == "layer" else capi.NORM_RMS
+        k = n_sets(4 * N * Cw * e)
+        gamma = pool.upload((1 + 0.02 * rng.standard_normal(Cw)).astype(np.float32)) if cfg.norm_affine \
+            else pool.upload(np.ones(Cw, np.float32))
+        beta = None
+        if cfg.norm == "layer":
+            beta = pool.upload((0.02 * rng.standard_normal(Cw)).astype(np.float32) if cfg.norm_affine
+                               else np.zeros(Cw, np.float32))
+        a = [pool.normal(N * Cw, cfg.dtype) for _ in range(k)]     # x   / saved h
+        b = [pool.normal(N * Cw, cfg.dtype) for _ in range(k)]     # r   / incoming residual grad
+        c = [pool.normal(N * Cw, cfg.dtype) for _ in range(k)]     # h   / dy
+        d = [pool.empty(N * Cw, cfg.dtype) for _ in range(k)]      # y   / dx
+        dgamma = pool.empty(Cw, "f32")
+        dbeta = pool.empty(Cw, "f32") if beta is not None else None
+        ws_bytes = ctx.lib.agrad_norm_backward_workspace_bytes(N, Cw, dt)
+        ws = pool.raw(ws_bytes)
+        res = cfg.norm_residual
+
+        def fwd(i):
+            ctx.call("agrad_norm_forward", kind, dt, vp(a[i]), vp(b[i]) if res else None, vp(gamma), vp(beta),
+                     vp(c[i]) if res else None, vp(d[i]), N, Cw, cfg.norm_eps)
+
+        def bwd(i):
+            ctx.call("agrad_norm_backward", kind, dt, vp(a[i]), vp(c[i]), vp(gamma), vp(b[i]) if res else None,
+                     vp(d[i]), None, vp(dgamma), vp(dbeta), vp(ws), ws_bytes, N, Cw, cfg.norm_eps, 0)
+
+        cases.append(Case(name, "fwd", nbytes[name][0], k, fwd, "norm_fwd_kernel"))
+        cases.append(Case(name, "bwd", nbytes[name][1], k, bwd, "norm_bwd_kernel"))
+
+    if cfg.act:
+        H = cfg.act_width
+        rows = N
+        if cfg.act == "swiglu":
+            k = n_sets(5 * rows * H * e)
+            gu = [pool.normal(rows * 2 * H, cfg.dtype) for _ in range(k)]
+            h = [pool.normal(rows * H, cfg.dtype) for _ in range(k)]
+            dgu = [pool.empty(rows * 2 * H, cfg.dtype) for _ in range(k)]
+
+            def fwd(i):
+                ctx.call("agrad_swiglu_forward", dt, vp(gu[i]), vp(h[i]), rows, H)
+
+            def bwd(i):
+                ctx.call("agrad_swiglu_backward", dt, vp(gu[i]), vp(h[i]), vp(dgu[i]), rows, H, 0)
+
+            cases.append(Case("swiglu", "fwd", nbytes["swiglu"][0], k, fwd, "swiglu_fwd_kernel"))
+            cases.append(Case("swiglu", "bwd", nbytes["swiglu"][1], k, bwd, "swiglu_bwd_kernel"))
+        else:
+            n = rows * H
+            k = n_sets(3 * n * e)
+            x = [pool.normal(n, cfg.dtype) for _ in range(k)]
+            y = [pool.normal(n, cfg.dtype) for _ in range(k)]
+            dx = [pool.empty(n, cfg.dtype) for _ in range(k)]
+            f_name, b_name = f"agrad_{cfg.act}_forward", f"agrad_{cfg.act}_backward"
+
+            def fwd(i):
+                ctx.call(f_name, dt, vp(x[i]), vp(dx[i]), n)
+
+            def bwd(i):
+                ctx.call(b_name, dt, vp(x[i]), vp(y[i]), vp(dx[i]), n, 0)
+
+            cases.append(Case(cfg.act, "fwd", nbytes[cfg.act][0], k, fwd, "ew_kernel"))
+            cases.append(Case(cfg.act, "bwd", nbytes[cfg.act][1], k, bwd, "ew_kernel"))
+
+    if cfg.rope:
+        Hq, Hkv, D, theta, sign = cfg.rope
+        k = n_sets(nbytes["rope"][0] // 2)
+        pos = np.arange(cfg.T, dtype=np.float32)[:, None]
+        inv = np.float32(theta) ** (-np.arange(0, D, 2, dtype=np.float32)[None, :] / np.float32(D))
+        cos = pool.upload(np.cos(pos * inv).astype(np.float32))
+        sin = pool.upload(np.sin(pos * inv).astype(np.float32))
+        q = [pool.normal(N * Hq * D, cfg.dtype) for _ in range(k)]
+        kk = [pool.normal(N * Hkv * D, cfg.dtype) for _ in range(k)]
+
+        def fwd(i):
+            ctx.call("agrad_rope_qk", dt, vp(q[i]), vp(kk[i]), vp(cos), vp(sin), cfg.B, cfg.T, Hq, Hkv, D, sign, 0)
+
+        def bwd(i):
+            ctx.call("agrad_rope_qk", dt, vp(q[i]), vp(kk[i]), vp(cos), vp(sin), cfg.B, cfg.T, Hq, Hkv, D, sign, 1)
+
+        cases.append(Case("rope", "fwd", nbytes["rope"][0], k, fwd, "rope_kernel"))
+        cases.append(Case("rope", "bwd", nbytes["rope"][1], k, bwd, "rope_kernel"))
+    return cases
+
+
+def time_case(ctx, case, iters):
+    for i in range(min(case.nsets, 3)):
+        case.launch(i)
+    ctx.synchronize()
+    ctx.timer_start()
+    for it in range(iters):
+        case.launch(it % case.nsets)
+    ms = ctx.timer_stop()
+    ctx.synchronize()
+    case.us = ms * 1e3 / iters
+    return case.us
+
+
+def case_row(case):
+    gbps = case.nbytes / (case.us * 1e-6) / 1e9
+    return {"op": case.op, "dir": case.direction, "MB": round(case.nbytes / 1e6, 2), "us": round(case.us, 2),
+            "GBps": round(gbps, 1), "frac_hbm": round(gbps / HBM_PEAK_GBS, 4), "sets": case.nsets,
+            "kernel": case.kernel}
+
+
+def run_config(ctx, cfg, iters):
+    pool = Pool(ctx, cfg.seed)
+    try:
+        cases = build_cases(ctx, cfg, pool)
+        for case in cases:
+            time_case(ctx, case, iters)
+        return [case_row(c) for c in cases]
+    finally:
+        pool.release()
+
+
+def run_workload(ctx, cfg, steps, warmup, iters):
+    pool = Pool(ctx, cfg.seed)
+    try:
+        cases = build_cases(ctx, cfg, pool)
+        step_cases = [c for c in cases if c.direction == "fwd"] + [c for c in reversed(cases) if c.direction == "bwd"]
+        step_bytes = sum(c.nbytes for c in step_cases)
+
+        def step(s):
+            for c in step_cases:
+                c.launch(s % c.nsets)
+
+        for s in range(warmup):
+            step(s)
+        ctx.synchronize()
+        t0 = time.perf_counter()
+        for s in range(steps):
+            step(warmup + s)
+        ctx.synchronize()
+        wall = time.perf_counter() - t0
+        for case in cases:
+            time_case(ctx, case, iters)
+        return cases, step_bytes, wall
+    finally:
+        pool.release()
+
+
+# ---------------------------------------------------------------------------------
+# CPU baseline: the numpy restatement of the reference's CPU kernels (oracle/),
+# imported here only, as the thing that is timed beside the GPU numbers.
+# ---------------------------------------------------------------------------------
+def cpu_baseline(cfg):
+    from oracle import cpu_ops as K
+
+    rng = np.random.default_rng(cfg.seed)
+    rows = cfg.N if cfg.index <= 1 else min(cfg.N, 2048)
+    B = max(1, rows // cfg.T)
+    T = min(cfg.T, rows)
+    rows = B * T
+    Cw = cfg.C
+    widen = (lambda a: K.round_bf16(a)) if cfg.dtype == "bf16" else (lambda a: a)
+    work = []
+
+    if cfg.embed:
+        ids = token_ids(cfg, rng, rows).reshape(B, T)
+        W = widen((0.02 * rng.standard_normal((cfg.V, Cw))).astype(np.float32))
+        wpe = widen((0.02 * rng.standard_normal((T, Cw))).astype(np.float32)) if cfg.embed == "gather_sum" else None
+        dY = rng.standard_normal((B, T, Cw), dtype=np.float32)
+        dW = np.zeros_like(W)
+        dwpe = np.zeros_like(wpe) if wpe is not None else None
+
+        def emb():
+            if wpe is None:
+                K.gather_forward(ids, W)
+                K.gather_backward_into(ids, dY, dW)
+            else:
+                K.embedding_sum_forward(ids, W, wpe)
+                K.embedding_sum_backward_into(ids, dY, dW, dwpe)
+        work.append(emb)
+    if cfg.norm:
+        x = rng.standard_normal((rows, Cw), dtype=np.float32)
+        r = rng.standard_normal((rows, Cw), dtype=np.float32)
+        dy = rng.standard_normal((rows, Cw), dtype=np.float32)
+        g = (1 + 0.02 * rng.standard_normal(Cw)).astype(np.float32)
+        bta = (0.02 * rng.standard_normal(Cw)).astype(np.float32)
+        dx, dg, db = np.zeros_like(x), np.zeros_like(g), np.zeros_like(g)
+
+        def norm():
+            h = K.add_forward(x, r) if cfg.norm_residual else x
+            if cfg.norm == "layer":
+                K.layernorm_forward(h, g, bta, cfg.norm_eps)
+                K.layernorm_backward_into(h, g, dy, cfg.norm_eps, dx, dg, db)
+            else:
+                K.rmsnorm_forward(h, g, cfg.norm_eps)
+                K.rmsnorm_backward_into(h, g, dy, cfg.norm_eps, dx, dg)
+        work.append(norm)
+    if cfg.act:
+        H = cfg.act_width
+        if cfg.act == "swiglu":
+            gu = rng.standard_normal((rows, 2 * H), dtype=np.float32)
+            dh = rng.standard_normal((rows, H), dtype=np.float32)
+            work.append(lambda: (K.swiglu_forward(gu), K.swiglu_backward(gu, dh)))
+        else:
+            xa = rng.standard_normal((rows, H), dtype=np.float32)
+            dya = rng.standard_normal((rows, H), dtype=np.float32)
+            dxa = np.zeros_like(xa)
+            f, bfn = (K.gelu_forward, K.gelu_backward_into) if cfg.act == "gelu" else (K.relu2_forward, K.relu2_backward_into)
+            work.append(lambda: (f(xa), bfn(xa, dya, dxa)))
+    if cfg.rope:
+        Hq, Hkv, D, theta, sign = cfg.rope
+        q = rng.standard_normal((B, T, Hq, D), dtype=np.float32)
+        kk = rng.standard_normal((B, T, Hkv, D), dtype=np.float32)
+        cos, sin = K.rope_tables(T, D, theta)
+        work.append(lambda: (K.rope_signed(q, kk, cos, sin, sign, False), K.rope_signed(q, kk, cos, sin, sign, True)))
+
+    def one_pass():
+        for fn in work:
+            fn()
+
+    for _ in range(2):
+        one_pass()
+    t0 = time.perf_counter()
+    for _ in range(5):
+        one_pass()
+    sec = (time.perf_counter() - t0) / 5
+    scaled = LayerLike(cfg, B, T)
+    distinct = int(np.unique(ids).size) if cfg.embed else None
+    total = sum(f + b for f, b in op_bytes(scaled, distinct).values())
+    return {"value": round(total / sec / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"numpy restatement, fwd+bwd of every op at B={B} T={T} (rows {rows} of {cfg.N}), "
+                      f"2 warm-up + 5 timed passes, {sec * 1e3:.1f} ms/pass; host {platform.processor() or platform.machine()}, "
+                      f"os.cpu_count()={os.cpu_count()}, numpy {np.__version__}",
+            "tokens_per_s": round(rows / sec, 1), "ms_per_pass": round(sec * 1e3, 2)}
+
+
+def LayerLike(cfg, B, T):
+    from dataclasses import replace
+    return replace(cfg, B=B, T=T)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", type=int, default=1, help="index into autograd_amd.configs.CONFIGS")
+    ap.add_argument("--iters", type=int, default=30, help="launches per op in the per-op timing")
+    ap.add_argument("--workload-only", action="store_true", help="skip the per-op tables of the other configs")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this build has no multi-GPU path (asked for --gpus {args.gpus}); "
+              "every op is row-independent and would shard over rows with one all-reduce of the parameter grads",
+              file=sys.stderr)
+        return 2
+    cfg = CONFIGS[args.config]
+    ctx = capi.Context(0)
+    cases, step_bytes, wall = run_workload(ctx, cfg, args.steps, args.warmup, args.iters)
+    ms_per_step = wall * 1e3 / args.steps
+    gbps = step_bytes * args.steps / wall / 1e9
+    timed = [c for c in cases if c.direction in ("fwd", "bwd")]
+    dom = max(timed, key=lambda c: c.us)
+    dom_gbps = dom.nbytes / (dom.us * 1e-6) / 1e9
+    result = {
+        "metric": METRIC, "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": cfg.dtype, "data": "synthetic",
+        "config": {"workload": f"configs[{cfg.index}] {cfg.name}: B={cfg.B} T={cfg.T} C={cfg.C} V={cfg.V}, "
+                               f"ops {'/'.join(dict.fromkeys(c.op for c in timed))} fwd+bwd",
+                   "step_MB": round(step_bytes / 1e6, 1)},
+        "tokens_per_s": round(cfg.N * args.steps / wall, 1),
+        "pct_of_hbm_peak": round(100 * gbps / HBM_PEAK_GBS, 2),
+        "roofline": {"bound": "hbm", "kernel": dom.kernel, "op": f"{dom.op} {dom.direction}",
+                     "achieved": round(dom_gbps, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(dom_gbps / HBM_PEAK_GBS, 4), "traffic": None,
+                     "launch_us": round(dom.us, 2), "algorithmic_MB": round(dom.nbytes / 1e6, 2)},
+        "per_op": [case_row(c) for c in cases],
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(cfg)
+    if not args.workload_only:
+        others = {}
+        for other in CONFIGS:
+            if other.index != cfg.index:
+                others[f"configs[{other.index}] {other.name} ({other.dtype})"] = run_config(ctx, other, args.iters)
+        result["all_configs"] = others
+    ctx.synchronize()
+    ctx.close()
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
