@@ -121,13 +121,20 @@ def token_ids(cfg, rng, n):
 def build_cases(ctx, cfg, pool):
     """every op of the config, forward and backward, as launchable cases"""
     rng = np.random.default_rng(cfg.seed)
+    ids0 = token_ids(cfg, rng, cfg.N) if cfg.embed else None
+    distinct = int(np.unique(ids0).size) if ids0 is not None else None
+    nbytes = op_bytes(cfg, distinct)
+    cases = []
+    # one builder per op family: each keeps its buffers in its own scope
+    for builder in (_embed_cases, _norm_cases, _act_cases, _rope_cases):
+        cases += builder(ctx, cfg, pool, rng, nbytes, ids0)
+    return cases
+
+
+def _embed_cases(ctx, cfg, pool, rng, nbytes, ids0):
     dt = capi.BF16 if cfg.dtype == "bf16" else capi.F32
     N, Cw, e = cfg.N, cfg.C, cfg.esize
     cases = []
-    ids0 = token_ids(cfg, rng, N) if cfg.embed else None
-    distinct = int(np.unique(ids0).size) if ids0 is not None else None
-    nbytes = op_bytes(cfg, distinct)
-
     if cfg.embed:
         name = cfg.embed
         k = n_sets(2 * N * Cw * e)
@@ -142,10 +149,10 @@ def build_cases(ctx, cfg, pool):
         ws = pool.raw(ws_bytes)
         ctx.call("agrad_fill", dW.ptr, 0, 0, 1, dW.nbytes)
 
-        def fwd(i, ids=ids, out=out):
+        def fwd(i):
             ctx.call("agrad_gather_forward", dt, vp(ids[i]), vp(W), vp(wpe), vp(out[i]), N, cfg.T, Cw, cfg.V)
 
-        def bwd(i, ids=ids, dY=dY):
+        def bwd(i):
             ctx.call("agrad_embedding_backward", dt, vp(ids[i]), vp(dY[i]), vp(dW), vp(ws), ws_bytes, N, Cw, cfg.V, 0)
             if dwpe is not None:
                 ctx.call("agrad_pos_embedding_backward", dt, vp(dY[i]), vp(dwpe), cfg.B, cfg.T, Cw, 0)
@@ -156,7 +163,13 @@ def build_cases(ctx, cfg, pool):
         cases.append(Case(name, "fwd", nbytes[name][0], k, fwd, "gather"))
         cases.append(Case(name, "bwd", nbytes[name][1], k, bwd, "emb_segment_sum_kernel"))
         cases.append(Case(name + "_grad_zero_fill", "aux", cfg.V * Cw * e, 1, zero, "fill16_kernel"))
+    return cases
 
+
+def _norm_cases(ctx, cfg, pool, rng, nbytes, ids0):
+    dt = capi.BF16 if cfg.dtype == "bf16" else capi.F32
+    N, Cw, e = cfg.N, cfg.C, cfg.esize
+    cases = []
     if cfg.norm:
         name = ("add+" if cfg.norm_residual else "") + cfg.norm + "norm"
         kind = capi.NORM_LAYER if cfg.norm == "layer" else capi.NORM_RMS
@@ -187,7 +200,13 @@ def build_cases(ctx, cfg, pool):
 
         cases.append(Case(name, "fwd", nbytes[name][0], k, fwd, "norm_fwd_kernel"))
         cases.append(Case(name, "bwd", nbytes[name][1], k, bwd, "norm_bwd_kernel"))
+    return cases
 
+
+def _act_cases(ctx, cfg, pool, rng, nbytes, ids0):
+    dt = capi.BF16 if cfg.dtype == "bf16" else capi.F32
+    N, e = cfg.N, cfg.esize
+    cases = []
     if cfg.act:
         H = cfg.act_width
         rows = N
@@ -221,7 +240,13 @@ def build_cases(ctx, cfg, pool):
 
             cases.append(Case(cfg.act, "fwd", nbytes[cfg.act][0], k, fwd, "ew_kernel"))
             cases.append(Case(cfg.act, "bwd", nbytes[cfg.act][1], k, bwd, "ew_kernel"))
+    return cases
 
+
+def _rope_cases(ctx, cfg, pool, rng, nbytes, ids0):
+    dt = capi.BF16 if cfg.dtype == "bf16" else capi.F32
+    N = cfg.N
+    cases = []
     if cfg.rope:
         Hq, Hkv, D, theta, sign = cfg.rope
         k = n_sets(nbytes["rope"][0] // 2)
