@@ -170,7 +170,7 @@ swiglu_bwd_kernel(const T* gu, const T* __restrict__ dh, T* dgu, uint32_t H, uin
 template <typename T, int VEC>
 int swiglu_typed(hipStream_t s, const T* gu, const T* dh, T* out, uint64_t rows, uint32_t H,
                  bool backward, int acc) {
-    constexpr int UNROLL = sizeof(T) == 4 ? 2 : 1;
+    constexpr int UNROLL = 1;
     const uint32_t HV = H / VEC;
     const uint64_t max_rows = 0xf0000000ull / HV;
     for (uint64_t r0 = 0; r0 < rows; r0 += max_rows) {

@@ -32,28 +32,35 @@ __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) {
 // Vector I/O.  VecIO<T, V> moves V consecutive elements between memory and an
 // fp32 register array.  (float,4) and (bf16,8) are one 128-bit access.
 // ---------------------------------------------------------------------------
+// Activations and gradients are touched once per kernel, so their accesses
+// carry the non-temporal hint (measured on MI355X: a plain copy goes from 5.6 to
+// 6.5 TB/s with it).  Small re-read operands (gamma, beta, rotary tables, token
+// ids, partial sums) use ordinary loads and stay cached.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
 template <typename T, int V> struct VecIO;
 
 template <> struct VecIO<float, 4> {
     static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
-        float4 t = *reinterpret_cast<const float4*>(p);
+        const f32x4 t = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p));
         v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
     }
     static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
-        float4 t; t.x = v[0]; t.y = v[1]; t.z = v[2]; t.w = v[3];
-        *reinterpret_cast<float4*>(p) = t;
+        f32x4 t; t.x = v[0]; t.y = v[1]; t.z = v[2]; t.w = v[3];
+        __builtin_nontemporal_store(t, reinterpret_cast<f32x4*>(p));
     }
 };
 
 template <> struct VecIO<float, 1> {
-    static __device__ __forceinline__ void load(const float* p, float (&v)[1]) { v[0] = *p; }
-    static __device__ __forceinline__ void store(float* p, const float (&v)[1]) { *p = v[0]; }
+    static __device__ __forceinline__ void load(const float* p, float (&v)[1]) { v[0] = __builtin_nontemporal_load(p); }
+    static __device__ __forceinline__ void store(float* p, const float (&v)[1]) { __builtin_nontemporal_store(v[0], p); }
 };
 
 template <> struct VecIO<bf16_t, 8> {
     static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
-        uint4 t = *reinterpret_cast<const uint4*>(p);
-        uint32_t w[4] = {t.x, t.y, t.z, t.w};
+        const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+        const uint32_t w[4] = {t.x, t.y, t.z, t.w};
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             v[2 * i]     = __uint_as_float(w[i] << 16);
@@ -65,17 +72,17 @@ template <> struct VecIO<bf16_t, 8> {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
             w[i] = f32_to_bf16_bits(v[2 * i]) | (f32_to_bf16_bits(v[2 * i + 1]) << 16);
-        uint4 t; t.x = w[0]; t.y = w[1]; t.z = w[2]; t.w = w[3];
-        *reinterpret_cast<uint4*>(p) = t;
+        u32x4 t; t.x = w[0]; t.y = w[1]; t.z = w[2]; t.w = w[3];
+        __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
     }
 };
 
 template <> struct VecIO<bf16_t, 1> {
     static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[1]) {
-        v[0] = bf16_bits_to_f32(*p);
+        v[0] = bf16_bits_to_f32(__builtin_nontemporal_load(p));
     }
     static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[1]) {
-        *p = (bf16_t)f32_to_bf16_bits(v[0]);
+        __builtin_nontemporal_store((bf16_t)f32_to_bf16_bits(v[0]), p);
     }
 };
 

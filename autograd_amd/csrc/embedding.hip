@@ -41,25 +41,31 @@ gather_fwd_kernel(const int32_t* __restrict__ ids, const T* __restrict__ W, cons
                   T* __restrict__ out, uint32_t total, uint32_t CV, uint32_t C, uint32_t T_len,
                   uint32_t V, int* err_flag) {
     const uint32_t first = blockIdx.x * (kGatherBlock * UNROLL) + threadIdx.x;
-    float v[UNROLL][VEC], p[UNROLL][VEC];
-    bool ok[UNROLL];
-    uint64_t dst[UNROLL];
+    int32_t tok[UNROLL];
+    uint32_t rows[UNROLL], col[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
         const uint32_t idx = first + u * kGatherBlock;
-        ok[u] = false;
+        tok[u] = -1;
+        rows[u] = 0;
+        col[u] = 1;
         if (idx < total) {
-            const uint32_t row = idx / CV;
-            const uint32_t col = (idx - row * CV) * VEC;
-            const int32_t tok = ids[row];
-            dst[u] = (uint64_t)row * C + col;
-            if (tok >= 0 && (uint32_t)tok < V) {
-                ok[u] = true;
-                VecIO<T, VEC>::load(W + (uint64_t)tok * C + col, v[u]);
-                if (wpe != nullptr) VecIO<T, VEC>::load(wpe + (uint64_t)(row % T_len) * C + col, p[u]);
-            } else if (col == 0) {
-                *err_flag = 1;
-            }
+            rows[u] = idx / CV;
+            col[u] = (idx - rows[u] * CV) * VEC;
+            tok[u] = ids[rows[u]];
+        }
+    }
+    float v[UNROLL][VEC], p[UNROLL][VEC];
+    bool ok[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        const uint32_t idx = first + u * kGatherBlock;
+        ok[u] = idx < total && tok[u] >= 0 && (uint32_t)tok[u] < V;
+        if (ok[u]) {
+            VecIO<T, VEC>::load(W + (uint64_t)tok[u] * C + col[u], v[u]);
+            if (wpe != nullptr) VecIO<T, VEC>::load(wpe + (uint64_t)(rows[u] % T_len) * C + col[u], p[u]);
+        } else if (idx < total && col[u] == 0) {
+            *err_flag = 1;
         }
     }
 #pragma unroll
@@ -69,7 +75,7 @@ gather_fwd_kernel(const int32_t* __restrict__ ids, const T* __restrict__ W, cons
 #pragma unroll
                 for (int k = 0; k < VEC; ++k) v[u][k] = v[u][k] + p[u][k];
             }
-            VecIO<T, VEC>::store(out + dst[u], v[u]);
+            VecIO<T, VEC>::store(out + (uint64_t)rows[u] * C + col[u], v[u]);
         }
     }
 }
@@ -78,31 +84,37 @@ gather_fwd_kernel(const int32_t* __restrict__ ids, const T* __restrict__ W, cons
 // words, so NaN payloads and -0.0 survive untouched.
 template <int UNROLL>
 __global__ void __launch_bounds__(kGatherBlock)
-gather_rows16_kernel(const int32_t* __restrict__ ids, const uint4* __restrict__ W,
-                     uint4* __restrict__ out, uint32_t total, uint32_t CV, uint32_t V, int* err_flag) {
+gather_rows16_kernel(const int32_t* __restrict__ ids, const u32x4* __restrict__ W,
+                     u32x4* __restrict__ out, uint32_t total, uint32_t CV, uint32_t V, int* err_flag) {
     const uint32_t first = blockIdx.x * (kGatherBlock * UNROLL) + threadIdx.x;
-    uint4 v[UNROLL];
+    // phase 1: every token id this thread needs (independent loads)
+    int32_t tok[UNROLL];
+    uint32_t cv[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+        const uint32_t idx = first + u * kGatherBlock;
+        tok[u] = -1;
+        cv[u] = 1;
+        if (idx < total) {
+            const uint32_t row = idx / CV;
+            cv[u] = idx - row * CV;
+            tok[u] = ids[row];
+        }
+    }
+    // phase 2: the table rows, all in flight together
+    u32x4 v[UNROLL];
     bool ok[UNROLL];
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
         const uint32_t idx = first + u * kGatherBlock;
-        ok[u] = false;
-        if (idx < total) {
-            const uint32_t row = idx / CV;
-            const uint32_t cv = idx - row * CV;
-            const int32_t tok = ids[row];
-            if (tok >= 0 && (uint32_t)tok < V) {
-                ok[u] = true;
-                v[u] = W[(uint64_t)tok * CV + cv];
-            } else if (cv == 0) {
-                *err_flag = 1;
-            }
-        }
+        ok[u] = idx < total && tok[u] >= 0 && (uint32_t)tok[u] < V;
+        if (ok[u]) v[u] = __builtin_nontemporal_load(W + (uint64_t)tok[u] * CV + cv[u]);
+        else if (idx < total && cv[u] == 0) *err_flag = 1;
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
         const uint32_t idx = first + u * kGatherBlock;
-        if (ok[u]) out[idx] = v[u];
+        if (ok[u]) __builtin_nontemporal_store(v[u], out + idx);
     }
 }
 
@@ -392,7 +404,7 @@ int launch_gather_fwd(hipStream_t s, int dtype, const int32_t* ids, const void* 
         const uint32_t grid = (total + kGatherBlock * UNROLL - 1) / (kGatherBlock * UNROLL);
         if (wpe == nullptr) {
             hipLaunchKernelGGL((gather_rows16_kernel<UNROLL>), dim3(grid), dim3(kGatherBlock), 0, s, ids,
-                               (const uint4*)W, (uint4*)out, total, CV, V, err_flag);
+                               (const u32x4*)W, (u32x4*)out, total, CV, V, err_flag);
         } else if (dtype == AGRAD_F32) {
             hipLaunchKernelGGL((gather_fwd_kernel<float, 4, UNROLL>), dim3(grid), dim3(kGatherBlock), 0, s, ids,
                                (const float*)W, (const float*)wpe, (float*)out, total, CV, C, T, V, err_flag);

@@ -10,12 +10,12 @@ namespace agrad {
 namespace {
 
 // 16-byte body: every uint4 carries the item pattern replicated.
-__global__ void __launch_bounds__(kEwBlock) fill16_kernel(uint4* dst, uint4 pattern, uint64_t nvec) {
+__global__ void __launch_bounds__(kEwBlock) fill16_kernel(u32x4* dst, u32x4 pattern, uint64_t nvec) {
     const uint64_t first = (uint64_t)blockIdx.x * (kEwBlock * 4) + threadIdx.x;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
         const uint64_t idx = first + (uint64_t)u * kEwBlock;
-        if (idx < nvec) dst[idx] = pattern;
+        if (idx < nvec) __builtin_nontemporal_store(pattern, dst + idx);
     }
 }
 
@@ -34,19 +34,9 @@ fill_items_kernel(uint8_t* dst, uint32_t bits, uint32_t itemsize, uint64_t n) {
 }
 
 __global__ void __launch_bounds__(kEwBlock)
-copy16_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst, uint64_t nvec) {
-    const uint64_t first = (uint64_t)blockIdx.x * (kEwBlock * 4) + threadIdx.x;
-    uint4 v[4];
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        const uint64_t idx = first + (uint64_t)u * kEwBlock;
-        if (idx < nvec) v[u] = src[idx];
-    }
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        const uint64_t idx = first + (uint64_t)u * kEwBlock;
-        if (idx < nvec) dst[idx] = v[u];
-    }
+copy16_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst, uint64_t nvec) {
+    const uint64_t idx = (uint64_t)blockIdx.x * kEwBlock + threadIdx.x;
+    if (idx < nvec) __builtin_nontemporal_store(__builtin_nontemporal_load(src + idx), dst + idx);
 }
 
 __global__ void __launch_bounds__(kEwBlock)
@@ -147,8 +137,8 @@ int launch_fill(hipStream_t s, void* dst, uint32_t bits, int itemsize, uint64_t 
     const uint64_t nvec = items * itemsize / 16;
     if (nvec > 0) {
         if (int rc = grid_for(nvec, kEwBlock * 4, &grid)) return rc;
-        uint4 pat; pat.x = pat.y = pat.z = pat.w = word;
-        hipLaunchKernelGGL(fill16_kernel, dim3(grid), dim3(kEwBlock), 0, s, reinterpret_cast<uint4*>(p), pat, nvec);
+        u32x4 pat; pat.x = pat.y = pat.z = pat.w = word;
+        hipLaunchKernelGGL(fill16_kernel, dim3(grid), dim3(kEwBlock), 0, s, reinterpret_cast<u32x4*>(p), pat, nvec);
         p += nvec * 16;
         items -= nvec * 16 / itemsize;
     }
@@ -166,9 +156,9 @@ int launch_copy(hipStream_t s, const void* src, void* dst, uint64_t nbytes) {
     if (aligned16(src) && aligned16(dst)) {
         const uint64_t nvec = nbytes / 16;
         if (nvec > 0) {
-            if (int rc = grid_for(nvec, kEwBlock * 4, &grid)) return rc;
+            if (int rc = grid_for(nvec, kEwBlock, &grid)) return rc;
             hipLaunchKernelGGL(copy16_kernel, dim3(grid), dim3(kEwBlock), 0, s,
-                               static_cast<const uint4*>(src), static_cast<uint4*>(dst), nvec);
+                               static_cast<const u32x4*>(src), static_cast<u32x4*>(dst), nvec);
         }
         const uint64_t done = nvec * 16;
         if (done < nbytes) {

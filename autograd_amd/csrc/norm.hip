@@ -40,9 +40,155 @@ struct NormFwdArgs {
 template <typename T>
 struct NormBwdArgs {
     const T* x; const T* dy; const float* gamma; const T* dres; T* dx; T* dx2;
-    float* pgamma; float* pbeta;
+    float* pgamma; float* pbeta;      // [blocks, C] partial rows, one per workgroup
+    float* ggamma; float* gbeta;      // rows of the upper tree levels, level after level
+    float* dgamma; float* dbeta;      // results
+    uint32_t* counters;               // arrival tickets of every tree group, zero between launches
     uint64_t rows; uint32_t C; float eps; int kind; uint32_t flags;
 };
+
+constexpr uint32_t kGroupSize = 16;   // partial rows folded together at each level
+
+// Column sums of the per-workgroup partial rows, without a second launch and
+// without atomics on the data.  The partial rows form a 16-ary tree.  A
+// workgroup publishes its row and draws a ticket from the counter of its group
+// of 16; whoever draws the group's last ticket adds the group's rows, in row
+// order, into one row of the next level and moves up with it; the workgroup
+// that completes the root writes dgamma / dbeta.  Which workgroup does an
+// addition depends on timing, what is added in which order does not, so the
+// result is the same on every run.  All counters are left at zero.
+//
+// The rows cross between workgroups (and between the XCDs' separate L2 caches)
+// through agent-scope relaxed atomic stores and loads, which go to the coherent
+// level of the memory system by themselves; a device-wide release fence would
+// instead write back the whole L2 every time a workgroup finishes.
+//
+// A fold loads its (up to) 16 rows with independent loads before adding them,
+// so it costs one memory latency, not sixteen.
+__device__ __forceinline__ void publish2(float* p, float a, float b) {
+    const unsigned long long bits =
+        (unsigned long long)__float_as_uint(a) | ((unsigned long long)__float_as_uint(b) << 32);
+    __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void publish1(float* p, float a) {
+    __hip_atomic_store(reinterpret_cast<unsigned int*>(p), __float_as_uint(a), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float2 observe2(const float* p) {
+    const unsigned long long bits = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p),
+                                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    float2 r;
+    r.x = __uint_as_float((unsigned int)bits);
+    r.y = __uint_as_float((unsigned int)(bits >> 32));
+    return r;
+}
+__device__ __forceinline__ float observe1(const float* p) {
+    return __uint_as_float(__hip_atomic_load(reinterpret_cast<const unsigned int*>(p), __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT));
+}
+
+// dst = [dst +] sum of nrows rows of src; `final` rows go out with ordinary stores
+template <int BLOCK>
+__device__ __forceinline__ void fold_rows(const float* src, uint32_t nrows, uint32_t C, float* dst,
+                                          bool accumulate, bool final) {
+    if ((C & 1u) == 0) {
+        for (uint32_t c = threadIdx.x * 2; c < C; c += BLOCK * 2) {
+            float2 v[kGroupSize];
+#pragma unroll
+            for (uint32_t r = 0; r < kGroupSize; ++r)
+                if (r < nrows) v[r] = observe2(src + (uint64_t)r * C + c);
+            float2 s = v[0];
+#pragma unroll
+            for (uint32_t r = 1; r < kGroupSize; ++r)
+                if (r < nrows) { s.x = s.x + v[r].x; s.y = s.y + v[r].y; }
+            if (final) {
+                if (accumulate) { s.x = dst[c] + s.x; s.y = dst[c + 1] + s.y; }
+                dst[c] = s.x;
+                dst[c + 1] = s.y;
+            } else {
+                publish2(dst + c, s.x, s.y);
+            }
+        }
+    } else {
+        for (uint32_t c = threadIdx.x; c < C; c += BLOCK) {
+            float v[kGroupSize];
+#pragma unroll
+            for (uint32_t r = 0; r < kGroupSize; ++r)
+                if (r < nrows) v[r] = observe1(src + (uint64_t)r * C + c);
+            float s = v[0];
+#pragma unroll
+            for (uint32_t r = 1; r < kGroupSize; ++r)
+                if (r < nrows) s = s + v[r];
+            if (final) dst[c] = accumulate ? (dst[c] + s) : s;
+            else publish1(dst + c, s);
+        }
+    }
+}
+
+// rows of all tree levels above the leaves, for `blocks` leaves
+__host__ __device__ inline uint32_t tree_inner_rows(uint32_t blocks) {
+    uint32_t total = 0;
+    while (blocks > 1) {
+        blocks = (blocks + kGroupSize - 1) / kGroupSize;
+        if (blocks > 1) total += blocks;
+    }
+    return total;
+}
+// counters of all tree levels
+__host__ __device__ inline uint32_t tree_counters(uint32_t blocks) {
+    uint32_t total = 0;
+    do {
+        blocks = (blocks + kGroupSize - 1) / kGroupSize;
+        total += blocks;
+    } while (blocks > 1);
+    return total;
+}
+
+// FENCED: the leaf rows were written with ordinary stores (scalar fallback
+// kernel), so they need the device-wide fence before the ticket.
+template <typename T, int BLOCK, bool FENCED>
+__device__ __forceinline__ void finish_param_grads(const NormBwdArgs<T>& a) {
+    __shared__ uint32_t ticket;
+    const uint32_t C = a.C;
+    const bool accp = (a.flags & AGRAD_ACC_PARAM_GRAD) != 0;
+    const float* src_g = a.pgamma;
+    const float* src_b = a.pbeta;
+    float* up_g = a.ggamma;
+    float* up_b = a.gbeta;
+    uint32_t* counters = a.counters;
+    uint32_t rows = gridDim.x, me = blockIdx.x;
+    if constexpr (FENCED) __threadfence();
+    for (;;) {
+        const uint32_t ngroups = (rows + kGroupSize - 1) / kGroupSize;
+        const uint32_t group = me / kGroupSize;
+        const uint32_t first = group * kGroupSize;
+        const uint32_t members = rows - first < kGroupSize ? rows - first : kGroupSize;
+        // every published store of this workgroup has completed before the ticket is drawn
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        if (threadIdx.x == 0)
+            ticket = __hip_atomic_fetch_add(&counters[group], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (ticket != members - 1) return;
+        const bool root = ngroups == 1;
+        if (src_g != nullptr)
+            fold_rows<BLOCK>(src_g + (uint64_t)first * C, members, C, root ? a.dgamma : up_g + (uint64_t)group * C,
+                             root && accp, root);
+        if (src_b != nullptr)
+            fold_rows<BLOCK>(src_b + (uint64_t)first * C, members, C, root ? a.dbeta : up_b + (uint64_t)group * C,
+                             root && accp, root);
+        if (threadIdx.x == 0)
+            __hip_atomic_store(&counters[group], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (root) return;
+        src_g = src_g != nullptr ? up_g : nullptr;
+        src_b = src_b != nullptr ? up_b : nullptr;
+        up_g += (uint64_t)ngroups * C;
+        up_b += (uint64_t)ngroups * C;
+        counters += ngroups;
+        rows = ngroups;
+        me = group;
+    }
+}
 
 // gamma / beta are fp32 whatever the activation type: VEC of them is one or two
 // 128-bit loads.
@@ -347,12 +493,15 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
                     for (int i = 0; i < NV; ++i)
                         if (on[i]) {
                             const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
+                            float t[VEC];
 #pragma unroll
                             for (int k = 0; k < VEC; ++k) {
-                                float t = pass == 0 ? pg[i][k] : pb[i][k];
-                                for (int w = 0; w < RPB - 1; ++w) t = t + comb[(uint32_t)w * C + col + k];
-                                out[(uint64_t)blockIdx.x * C + col + k] = t;
+                                t[k] = pass == 0 ? pg[i][k] : pb[i][k];
+                                for (int w = 0; w < RPB - 1; ++w) t[k] = t[k] + comb[(uint32_t)w * C + col + k];
                             }
+#pragma unroll
+                            for (int k = 0; k < VEC; k += 2)
+                                publish2(out + (uint64_t)blockIdx.x * C + col + k, t[k], t[k + 1]);
                         }
                 }
                 __syncthreads();
@@ -363,33 +512,13 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
                 if (on[i]) {
                     const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
 #pragma unroll
-                    for (int k = 0; k < VEC; ++k) {
-                        if (want_pg) a.pgamma[(uint64_t)blockIdx.x * C + col + k] = pg[i][k];
-                        if (want_pb) a.pbeta[(uint64_t)blockIdx.x * C + col + k] = pb[i][k];
+                    for (int k = 0; k < VEC; k += 2) {
+                        if (want_pg) publish2(a.pgamma + (uint64_t)blockIdx.x * C + col + k, pg[i][k], pg[i][k + 1]);
+                        if (want_pb) publish2(a.pbeta + (uint64_t)blockIdx.x * C + col + k, pb[i][k], pb[i][k + 1]);
                     }
                 }
         }
-    }
-}
-
-// out[c] (+)= sum_p partial[p, c], p ascending inside each of 8 interleaved
-// row groups, the 8 group sums added in group order.
-__global__ void __launch_bounds__(256)
-colsum_finalize_kernel(const float* __restrict__ partial, uint32_t P, uint32_t C,
-                       float* __restrict__ out, int accumulate) {
-    __shared__ float tile[8][33];
-    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
-    const uint32_t col = blockIdx.x * 32 + tx;
-    float s = 0.0f;
-    if (col < C)
-        for (uint32_t p = ty; p < P; p += 8) s = s + partial[(uint64_t)p * C + col];
-    tile[ty][tx] = s;
-    __syncthreads();
-    if (ty == 0 && col < C) {
-        float t = tile[0][tx];
-#pragma unroll
-        for (int j = 1; j < 8; ++j) t = t + tile[j][tx];
-        out[col] = accumulate ? (out[col] + t) : t;
+        finish_param_grads<T, BLOCK, false>(a);
     }
 }
 
@@ -514,6 +643,7 @@ __global__ void __launch_bounds__(256) norm_bwd_generic_kernel(const NormBwdArgs
             }
         }
     }
+    if (a.pgamma != nullptr || a.pbeta != nullptr) finish_param_grads<T, 256, true>(a);
 }
 
 // ----------------------------------------------------------------------------
@@ -619,7 +749,7 @@ uint32_t norm_bwd_max_blocks() {
     static const uint32_t value = [] {
         const char* e = std::getenv("AGRAD_NORM_BWD_BLOCKS");
         long v = e ? std::atol(e) : 0;
-        return (uint32_t)(v > 0 && v <= 65536 ? v : 1024);
+        return (uint32_t)(v > 0 && v <= 2048 ? v : 1024);
     }();
     return value;
 }
@@ -633,7 +763,7 @@ uint64_t norm_bwd_workspace_bytes(uint64_t rows, uint32_t C, int dtype) {
         const uint64_t b = bwd_blocks(vecp, rows);
         if (b > blocks) blocks = b;
     }
-    return 2ull * blocks * C * sizeof(float);
+    return 2ull * (blocks + tree_inner_rows((uint32_t)blocks)) * C * sizeof(float);
 }
 
 int launch_norm_fwd(hipStream_t s, int kind, int dtype, const void* x, const void* residual,
@@ -663,7 +793,7 @@ int launch_norm_fwd(hipStream_t s, int kind, int dtype, const void* x, const voi
 int launch_norm_bwd(hipStream_t s, int kind, int dtype, const void* x, const void* dy,
                     const float* gamma, const void* dres_in, void* dx, void* dx2,
                     float* dgamma, float* dbeta, void* workspace, uint64_t workspace_bytes,
-                    uint64_t rows, uint32_t C, float eps, uint32_t flags) {
+                    uint64_t rows, uint32_t C, float eps, uint32_t flags, uint32_t* counters) {
     if (kind != AGRAD_NORM_LAYER && kind != AGRAD_NORM_RMS)
         return set_error(AGRAD_EINVAL, "norm backward: unknown kind %d", kind);
     if (dtype != AGRAD_F32 && dtype != AGRAD_BF16)
@@ -679,38 +809,41 @@ int launch_norm_bwd(hipStream_t s, int kind, int dtype, const void* x, const voi
     const NormPlan p = plan_norm(C, dtype, aligned);
     const uint32_t grid = bwd_blocks(p, rows);
     const bool want_params = dgamma != nullptr || dbeta != nullptr;
-    float* pg = nullptr;
-    float* pb = nullptr;
+    if (rows == 0) {
+        // nothing to add: stored parameter grads become zero, accumulated ones stay
+        if (want_params && !(flags & AGRAD_ACC_PARAM_GRAD)) {
+            if (dgamma) if (int rc = launch_fill(s, dgamma, 0, 4, C)) return rc;
+            if (dbeta) if (int rc = launch_fill(s, dbeta, 0, 4, C)) return rc;
+        }
+        return AGRAD_OK;
+    }
+    const uint32_t inner = tree_inner_rows(grid);
+    float *pg = nullptr, *pb = nullptr, *gg = nullptr, *gb = nullptr;
     if (want_params) {
-        const uint64_t need = 2ull * grid * C * sizeof(float);
+        const uint64_t need = 2ull * ((uint64_t)grid + inner) * C * sizeof(float);
         if (workspace == nullptr || workspace_bytes < need)
             return set_error(AGRAD_EWORKSPACE, "norm backward: workspace %llu < %llu bytes",
                              (unsigned long long)workspace_bytes, (unsigned long long)need);
-        if (dgamma) pg = (float*)workspace;
-        if (dbeta) pb = (float*)workspace + (uint64_t)grid * C;
+        if (!aligned16(workspace)) return set_error(AGRAD_EINVAL, "norm backward: workspace must be 16-byte aligned");
+        if (counters == nullptr || tree_counters(grid) > kNormCounters)
+            return set_error(AGRAD_EINVAL, "norm backward: no ticket counters");
+        float* w = (float*)workspace;
+        if (dgamma) { pg = w; gg = w + 2ull * grid * C; }
+        if (dbeta) { pb = w + (uint64_t)grid * C; gb = w + 2ull * grid * C + (uint64_t)inner * C; }
     }
-    int rc = AGRAD_OK;
-    if (rows > 0) {
-        if (dtype == AGRAD_F32) {
-            NormBwdArgs<float> a{(const float*)x, (const float*)dy, gamma, (const float*)dres_in,
-                                 (float*)dx, (float*)dx2, pg, pb, rows, C, eps, kind, flags};
-            rc = norm_bwd_typed<float>(s, p, a, grid);
-        } else {
-            NormBwdArgs<bf16_t> a{(const bf16_t*)x, (const bf16_t*)dy, gamma, (const bf16_t*)dres_in,
-                                  (bf16_t*)dx, (bf16_t*)dx2, pg, pb, rows, C, eps, kind, flags};
-            rc = norm_bwd_typed<bf16_t>(s, p, a, grid);
-        }
-        if (rc != AGRAD_OK) return rc;
+    int rc;
+    if (dtype == AGRAD_F32) {
+        NormBwdArgs<float> a{(const float*)x, (const float*)dy, gamma, (const float*)dres_in,
+                             (float*)dx, (float*)dx2, pg, pb, gg, gb, dgamma, dbeta, counters,
+                             rows, C, eps, kind, flags};
+        rc = norm_bwd_typed<float>(s, p, a, grid);
+    } else {
+        NormBwdArgs<bf16_t> a{(const bf16_t*)x, (const bf16_t*)dy, gamma, (const bf16_t*)dres_in,
+                              (bf16_t*)dx, (bf16_t*)dx2, pg, pb, gg, gb, dgamma, dbeta, counters,
+                              rows, C, eps, kind, flags};
+        rc = norm_bwd_typed<bf16_t>(s, p, a, grid);
     }
-    if (want_params) {
-        const int accp = (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0;
-        const uint32_t P = rows > 0 ? grid : 0;
-        const uint32_t fgrid = (C + 31) / 32;
-        if (dgamma)
-            hipLaunchKernelGGL(colsum_finalize_kernel, dim3(fgrid), dim3(256), 0, s, pg, P, C, dgamma, accp);
-        if (dbeta)
-            hipLaunchKernelGGL(colsum_finalize_kernel, dim3(fgrid), dim3(256), 0, s, pb, P, C, dbeta, accp);
-    }
+    if (rc != AGRAD_OK) return rc;
     return check_hip(hipGetLastError(), "norm backward launch");
 }
 

@@ -92,7 +92,7 @@ __global__ void __launch_bounds__(kRopeBlock) rope_kernel(const RopeArgs<T> a) {
 
 template <typename T, int VEC>
 int rope_typed(hipStream_t s, RopeArgs<T> a, uint32_t B) {
-    constexpr int UNROLL = 2;
+    constexpr int UNROLL = 1;
     a.J = a.D / 2 / VEC;
     a.Iq = a.H * a.J;
     a.I = (a.H + (a.k ? a.HKV : 0)) * a.J;

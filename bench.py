@@ -268,10 +268,30 @@ def _rope_cases(ctx, cfg, pool, rng, nbytes, ids0):
     return cases
 
 
+def spin_up(ctx, seconds=0.25):
+    """keep the GPU busy for a moment so that clocks have left their idle state
+    before anything is timed"""
+    n = 64 << 20
+    a, b = ctx.empty((n,), np.uint8), ctx.empty((n,), np.uint8)
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(50):
+            ctx.call("agrad_copy", vp(a), vp(b), n)
+        ctx.synchronize()
+    a.free()
+    b.free()
+
+
 def time_case(ctx, case, iters):
+    # at least `iters` launches and at least ~2 ms of GPU time
     for i in range(min(case.nsets, 3)):
         case.launch(i)
     ctx.synchronize()
+    ctx.timer_start()
+    for it in range(8):
+        case.launch(it % case.nsets)
+    probe_us = ctx.timer_stop() * 1e3 / 8
+    iters = int(max(iters, min(2000, 2000.0 / max(probe_us, 0.5))))
     ctx.timer_start()
     for it in range(iters):
         case.launch(it % case.nsets)
@@ -435,6 +455,7 @@ def main():
         return 2
     cfg = CONFIGS[args.config]
     ctx = capi.Context(0)
+    spin_up(ctx)
     cases, step_bytes, wall = run_workload(ctx, cfg, args.steps, args.warmup, args.iters)
     ms_per_step = wall * 1e3 / args.steps
     gbps = step_bytes * args.steps / wall / 1e9
