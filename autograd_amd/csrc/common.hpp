@@ -28,6 +28,21 @@ __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) {
     return __uint_as_float(b << 16);
 }
 
+// Two fp32 -> one packed pair of bf16 (a in the low half).  gfx950 converts a
+// pair with round-to-nearest-even in one instruction (v_cvt_pk_bf16_f32); that
+// takes every finite value and the infinities exactly where the integer rule
+// above takes them.  NaNs are re-done with the integer rule so that the kept
+// payload bits are the reference's.
+typedef __bf16 bf16x2_hw __attribute__((ext_vector_type(2)));
+typedef float f32x2_hw __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+    const f32x2_hw v = {a, b};
+    uint32_t r = __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_hw));
+    if (__builtin_expect(a != a, 0)) r = (r & 0xffff0000u) | f32_to_bf16_bits(a);
+    if (__builtin_expect(b != b, 0)) r = (r & 0x0000ffffu) | (f32_to_bf16_bits(b) << 16);
+    return r;
+}
+
 // ---------------------------------------------------------------------------
 // Vector I/O.  VecIO<T, V> moves V consecutive elements between memory and an
 // fp32 register array.  (float,4) and (bf16,8) are one 128-bit access.
@@ -70,8 +85,7 @@ template <> struct VecIO<bf16_t, 8> {
     static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[8]) {
         uint32_t w[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            w[i] = f32_to_bf16_bits(v[2 * i]) | (f32_to_bf16_bits(v[2 * i + 1]) << 16);
+        for (int i = 0; i < 4; ++i) w[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
         u32x4 t; t.x = w[0]; t.y = w[1]; t.z = w[2]; t.w = w[3];
         __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
     }
@@ -95,7 +109,6 @@ template <> struct WideVec<bf16_t> { static constexpr int value = 8; };
 // Cross-lane sums.  A wave64 is four DPP rows of 16 lanes: quad_perm and the
 // row mirrors fold a row without touching LDS, ds_swizzle folds row pairs, and
 // two readlanes fold the two 32-lane halves into a wave-uniform value.
-// Every lane of the wave must be active when these are called.
 // ---------------------------------------------------------------------------
 template <int CTRL>
 __device__ __forceinline__ float dpp_move(float v) {
@@ -109,35 +122,52 @@ constexpr int kDppRowHalfMirror = 0x141;
 constexpr int kDppRowMirror     = 0x140;
 constexpr int kSwizzleXor16     = 0x401F; // bit mode: and 0x1f, or 0, xor 0x10
 
-__device__ __forceinline__ float wave_sum(float v) {
+// Sum over aligned groups of TPR lanes (TPR = 16, 32 or 64); every lane of a
+// group receives the group's total.  A group never reads lanes outside itself,
+// so neighbouring groups of one wave may be masked off independently.
+template <int TPR>
+__device__ __forceinline__ float lanes_sum(float v) {
+    static_assert(TPR == 16 || TPR == 32 || TPR == 64, "lane group must be 16, 32 or 64");
     v = v + dpp_move<kDppQuadXor1>(v);
     v = v + dpp_move<kDppQuadXor2>(v);
     v = v + dpp_move<kDppRowHalfMirror>(v);
     v = v + dpp_move<kDppRowMirror>(v);
-    v = v + __builtin_bit_cast(
-                float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), kSwizzleXor16));
-    float lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
-    float hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
-    return lo + hi;
+    if constexpr (TPR >= 32)
+        v = v + __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, v), kSwizzleXor16));
+    if constexpr (TPR == 64) {
+        const float lo = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+        const float hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+        v = lo + hi;
+    }
+    return v;
 }
 
 // Two independent sums folded together so their DPP chains interleave.
-__device__ __forceinline__ void wave_sum2(float& a, float& b) {
+template <int TPR>
+__device__ __forceinline__ void lanes_sum2(float& a, float& b) {
+    static_assert(TPR == 16 || TPR == 32 || TPR == 64, "lane group must be 16, 32 or 64");
     a = a + dpp_move<kDppQuadXor1>(a);       b = b + dpp_move<kDppQuadXor1>(b);
     a = a + dpp_move<kDppQuadXor2>(a);       b = b + dpp_move<kDppQuadXor2>(b);
     a = a + dpp_move<kDppRowHalfMirror>(a);  b = b + dpp_move<kDppRowHalfMirror>(b);
     a = a + dpp_move<kDppRowMirror>(a);      b = b + dpp_move<kDppRowMirror>(b);
-    a = a + __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, a), kSwizzleXor16));
-    b = b + __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, b), kSwizzleXor16));
-    float a0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, a), 0));
-    float a1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, a), 32));
-    float b0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, b), 0));
-    float b1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, b), 32));
-    a = a0 + a1;
-    b = b0 + b1;
+    if constexpr (TPR >= 32) {
+        a = a + __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, a), kSwizzleXor16));
+        b = b + __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, b), kSwizzleXor16));
+    }
+    if constexpr (TPR == 64) {
+        const float a0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, a), 0));
+        const float a1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, a), 32));
+        const float b0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, b), 0));
+        const float b1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, b), 32));
+        a = a0 + a1;
+        b = b0 + b1;
+    }
 }
 
-// Sum over the TPR threads that share one row.  TPR == 64: pure DPP.  TPR > 64:
+__device__ __forceinline__ float wave_sum(float v) { return lanes_sum<kWave>(v); }
+__device__ __forceinline__ void wave_sum2(float& a, float& b) { lanes_sum2<kWave>(a, b); }
+
+// Sum over the TPR threads that share one row.  TPR <= 64: pure DPP.  TPR > 64:
 // each wave's total is staged in LDS and every thread adds the staged totals in
 // wave order.  `slot` selects one of a few LDS lines so that consecutive
 // reductions need only one barrier each (a slot is 2*TPR/64 floats; rotate at
@@ -145,8 +175,10 @@ __device__ __forceinline__ void wave_sum2(float& a, float& b) {
 // the barrier is reached by the whole workgroup.
 template <int TPR>
 __device__ __forceinline__ float row_sum(float v, float* lds, int slot) {
-    v = wave_sum(v);
-    if constexpr (TPR > kWave) {
+    if constexpr (TPR <= kWave) {
+        return lanes_sum<TPR>(v);
+    } else {
+        v = wave_sum(v);
         constexpr int NW = TPR / kWave;
         float* line = lds + slot * 2 * NW;
         if ((threadIdx.x & (kWave - 1)) == 0) line[threadIdx.x / kWave] = v;
@@ -154,15 +186,16 @@ __device__ __forceinline__ float row_sum(float v, float* lds, int slot) {
         float t = line[0];
 #pragma unroll
         for (int w = 1; w < NW; ++w) t = t + line[w];
-        v = t;
+        return t;
     }
-    return v;
 }
 
 template <int TPR>
 __device__ __forceinline__ void row_sum2(float& a, float& b, float* lds, int slot) {
-    wave_sum2(a, b);
-    if constexpr (TPR > kWave) {
+    if constexpr (TPR <= kWave) {
+        lanes_sum2<TPR>(a, b);
+    } else {
+        wave_sum2(a, b);
         constexpr int NW = TPR / kWave;
         float* line = lds + slot * 2 * NW;
         if ((threadIdx.x & (kWave - 1)) == 0) {

@@ -18,7 +18,6 @@ struct agrad_ctx {
     hipStream_t stream = nullptr;
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
     int* err_flag = nullptr;               // device word set by kernels that see a bad token id
-    uint32_t* counters = nullptr;          // zeroed ticket words for the norm backward
     uint64_t total_mem = 0;
     std::mutex mu;
     std::map<uint64_t, uint64_t> allocs;   // base address -> bytes
@@ -189,8 +188,7 @@ int h_norm_bwd(const Call& c) {
     RESOLVE_IF(present & 128u, 7, par, dbeta)
     RESOLVE_IF(present & 256u, 8, ws_bytes, ws)
     return launch_norm_bwd(c.ctx->stream, KIND, c.a[0], x, dy, (const float*)gamma, dres, dx, dx2,
-                           (float*)dgamma, (float*)dbeta, ws, ws ? ws_bytes : 0, rows, C, f32(c.a[3]), flags,
-                           c.ctx->counters);
+                           (float*)dgamma, (float*)dbeta, ws, ws ? ws_bytes : 0, rows, C, f32(c.a[3]), flags);
 }
 
 // buffers x, y | args dtype, n lo, hi
@@ -343,10 +341,8 @@ int agrad_ctx_create(int device, agrad_ctx** out) {
     hipError_t e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipEventCreate(&c->ev_start);
     if (e == hipSuccess) e = hipEventCreate(&c->ev_stop);
-    const size_t state_bytes = 256 + kNormCounters * sizeof(uint32_t);
-    if (e == hipSuccess) e = hipMalloc((void**)&c->err_flag, state_bytes);
-    if (e == hipSuccess) e = hipMemset(c->err_flag, 0, state_bytes);
-    if (e == hipSuccess) c->counters = reinterpret_cast<uint32_t*>(c->err_flag) + 64;
+    if (e == hipSuccess) e = hipMalloc((void**)&c->err_flag, 256);
+    if (e == hipSuccess) e = hipMemset(c->err_flag, 0, 256);
     if (e != hipSuccess) {
         agrad_ctx_destroy(c);
         return check_hip(e, "context setup");
@@ -524,7 +520,7 @@ int agrad_norm_backward(agrad_ctx* ctx, int kind, int dtype, const void* x, cons
                         uint64_t rows, uint32_t C, float eps, uint32_t flags) {
     CTX_OR_FAIL(ctx)
     return launch_norm_bwd(ctx->stream, kind, dtype, x, dy, gamma, dres_in, dx, dx2, dgamma, dbeta,
-                           workspace, workspace_bytes, rows, C, eps, flags, ctx->counters);
+                           workspace, workspace_bytes, rows, C, eps, flags);
 }
 
 int agrad_gelu_forward(agrad_ctx* ctx, int dtype, const void* x, void* y, uint64_t n) {

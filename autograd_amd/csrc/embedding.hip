@@ -18,6 +18,7 @@
 #include "common.hpp"
 #include "launch.hpp"
 
+#include <cstdlib>
 #include <cstring>
 
 #include <rocprim/device/device_radix_sort.hpp>
@@ -159,6 +160,116 @@ emb_prepare_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ keys,
     if (bad) *err_flag = 1;
     keys[i] = bad ? V : (uint32_t)t;
     vals[i] = i;
+}
+
+// One-launch replacement for the radix sort when N <= kGroupSortMaxN.  What the
+// segmented sum needs is not a total order by token, only that each token's
+// rows sit next to each other in ascending row order.  Workgroup g owns the
+// tokens whose hash falls in group g.  It reads ALL ids (64 KiB at N = 16384,
+// served by L2), keeps the (token, row) pairs it owns in LDS, counts how many
+// rows belong to lower-numbered groups (that is where its slice of the output
+// starts), sorts its pairs by (token, row) with a bitonic network in LDS, and
+// writes them out.  No atomics on global memory, no scratch, and the output is
+// the same on every run.
+constexpr int kSortBlock = 1024;
+constexpr uint32_t kGroupSortMaxN = 16384;
+constexpr uint32_t kWaveSortMax = 1024;      // lists up to this size are sorted by a single wave
+
+__global__ void __launch_bounds__(kSortBlock)
+emb_group_sort_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ tok_s,
+                      uint32_t* __restrict__ row_s, uint32_t N, uint32_t V, uint32_t log2G,
+                      int* err_flag) {
+    extern __shared__ unsigned long long keys[];   // pow2ceil(N) entries
+    __shared__ uint32_t s_count, s_less;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t g = blockIdx.x;
+    if (tid == 0) { s_count = 0; s_less = 0; }
+    __syncthreads();
+
+    uint32_t less = 0;
+    constexpr int ROUND = 16;                       // id loads in flight per thread
+    for (uint32_t base = 0; base < N; base += kSortBlock * ROUND) {
+        int32_t t[ROUND];
+#pragma unroll
+        for (int r = 0; r < ROUND; ++r) {
+            const uint32_t i = base + r * kSortBlock + tid;
+            t[r] = i < N ? ids[i] : -1;
+        }
+#pragma unroll
+        for (int r = 0; r < ROUND; ++r) {
+            const uint32_t i = base + r * kSortBlock + tid;
+            if (i < N) {
+                const bool bad = t[r] < 0 || (uint32_t)t[r] >= V;
+                const uint32_t tok = bad ? V : (uint32_t)t[r];
+                if (bad && g == 0) *err_flag = 1;
+                const uint32_t owner = log2G ? (tok * 0x9E3779B1u) >> (32 - log2G) : 0u;
+                less += owner < g ? 1u : 0u;
+                if (owner == g) {
+                    const uint32_t slot = atomicAdd(&s_count, 1u);
+                    keys[slot] = ((unsigned long long)tok << 32) | i;
+                }
+            }
+        }
+    }
+    // rows owned by lower groups: wave totals (exact integers) added in LDS
+    {
+        float unused = 0.0f; (void)unused;
+        uint32_t v = less;
+        v += __builtin_amdgcn_update_dpp(0, v, kDppQuadXor1, 0xf, 0xf, true);
+        v += __builtin_amdgcn_update_dpp(0, v, kDppQuadXor2, 0xf, 0xf, true);
+        v += __builtin_amdgcn_update_dpp(0, v, kDppRowHalfMirror, 0xf, 0xf, true);
+        v += __builtin_amdgcn_update_dpp(0, v, kDppRowMirror, 0xf, 0xf, true);
+        v += __builtin_amdgcn_ds_swizzle(v, kSwizzleXor16);
+        const uint32_t total = __builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 32);
+        if ((tid & (kWave - 1)) == 0) atomicAdd(&s_less, total);
+    }
+    __syncthreads();
+    const uint32_t count = s_count;
+    const uint32_t offset = s_less;
+    uint32_t n2 = 2;
+    while (n2 < count) n2 <<= 1;
+    for (uint32_t i = count + tid; i < n2; i += kSortBlock) keys[i] = ~0ull;
+    __syncthreads();
+    if (n2 <= kWaveSortMax) {
+        // small list (the usual case): one wave sorts it with no workgroup
+        // barriers; a wave's LDS operations complete in program order
+        if (tid < kWave) {
+            for (uint32_t k = 2; k <= n2; k <<= 1) {
+                for (uint32_t j = k >> 1; j > 0; j >>= 1) {
+                    for (uint32_t i = tid; i < n2; i += kWave) {
+                        const uint32_t partner = i ^ j;
+                        if (partner > i) {
+                            const unsigned long long a = keys[i], b = keys[partner];
+                            const bool ascending = (i & k) == 0;
+                            if ((a > b) == ascending) { keys[i] = b; keys[partner] = a; }
+                        }
+                    }
+                    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                }
+            }
+        }
+        __syncthreads();
+    } else {
+        for (uint32_t k = 2; k <= n2; k <<= 1) {
+            for (uint32_t j = k >> 1; j > 0; j >>= 1) {
+                for (uint32_t i = tid; i < n2; i += kSortBlock) {
+                    const uint32_t partner = i ^ j;
+                    if (partner > i) {
+                        const unsigned long long a = keys[i], b = keys[partner];
+                        const bool ascending = (i & k) == 0;
+                        if ((a > b) == ascending) { keys[i] = b; keys[partner] = a; }
+                    }
+                }
+                __syncthreads();
+            }
+        }
+    }
+    for (uint32_t i = tid; i < count; i += kSortBlock) {
+        const unsigned long long key = keys[i];
+        tok_s[offset + i] = (uint32_t)(key >> 32);
+        row_s[offset + i] = (uint32_t)key;
+    }
 }
 
 struct ChunkEdges {
@@ -313,6 +424,15 @@ pos_grad_kernel(const T* __restrict__ dY, T* dwpe, uint32_t B, uint64_t TCV, uin
     store_grad_row<T, VEC>(dwpe, off, acc, accumulate != 0);
 }
 
+// AGRAD_EMB_GROUP_SORT=0 forces the radix-sort path (for comparison runs)
+bool group_sort_enabled() {
+    static const bool on = [] {
+        const char* e = std::getenv("AGRAD_EMB_GROUP_SORT");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
 struct EmbPlan {
     uint32_t L, chunks;
     uint64_t off_keys_in, off_keys_out, off_vals_in, off_vals_out, off_temp, temp_bytes, off_head,
@@ -354,13 +474,32 @@ int embedding_bwd_typed(hipStream_t s, const EmbPlan& p, const int32_t* ids, con
     float* head = (float*)(ws + p.off_head);
     float* tail = (float*)(ws + p.off_tail);
 
-    hipLaunchKernelGGL(emb_prepare_kernel, dim3((N + 255) / 256), dim3(256), 0, s, ids, keys_in, vals_in, N, V, err_flag);
-    int bits = 1;
-    while ((1ull << bits) <= V) ++bits;
-    size_t temp = p.temp_bytes;
-    hipError_t err = rocprim::radix_sort_pairs(ws + p.off_temp, temp, keys_in, keys_out, vals_in, vals_out,
-                                               (size_t)N, 0u, (unsigned)bits, s, false);
-    if (err != hipSuccess) return check_hip(err, "radix sort");
+    bool grouped = false;
+    if (N <= kGroupSortMaxN && group_sort_enabled()) {
+        uint32_t cap = 2;
+        while (cap < N) cap <<= 1;
+        const size_t lds = (size_t)cap * sizeof(unsigned long long);
+        static const bool big_lds_ok = [] {
+            return hipFuncSetAttribute(reinterpret_cast<const void*>(emb_group_sort_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)(kGroupSortMaxN * sizeof(unsigned long long))) == hipSuccess;
+        }();
+        if (lds <= 48 * 1024 || big_lds_ok) {
+            const uint32_t log2G = N > 1024 ? 8u : 4u;
+            hipLaunchKernelGGL(emb_group_sort_kernel, dim3(1u << log2G), dim3(kSortBlock), lds, s, ids, keys_out,
+                               vals_out, N, V, log2G, err_flag);
+            grouped = true;
+        }
+    }
+    if (!grouped) {
+        hipLaunchKernelGGL(emb_prepare_kernel, dim3((N + 255) / 256), dim3(256), 0, s, ids, keys_in, vals_in, N, V, err_flag);
+        int bits = 1;
+        while ((1ull << bits) <= V) ++bits;
+        size_t temp = p.temp_bytes;
+        hipError_t err = rocprim::radix_sort_pairs(ws + p.off_temp, temp, keys_in, keys_out, vals_in, vals_out,
+                                                   (size_t)N, 0u, (unsigned)bits, s, false);
+        if (err != hipSuccess) return check_hip(err, "radix sort");
+    }
 
     const int acc = (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0;
     constexpr int WIDE = WideVec<T>::value;

@@ -18,9 +18,6 @@ inline uint32_t dtype_size(int dtype) { return dtype == AGRAD_BF16 ? 2u : 4u; }
 
 // Upper bound on the number of row-partials the norm backward keeps per column.
 uint32_t norm_bwd_max_blocks();
-// Words of zero-initialised device memory the norm backward uses as arrival
-// tickets; the kernels leave them at zero.
-constexpr uint32_t kNormCounters = 192;
 
 // memops.hip
 int launch_fill(hipStream_t s, void* dst, uint32_t bits, int itemsize, uint64_t n);
@@ -38,7 +35,7 @@ int launch_norm_fwd(hipStream_t s, int kind, int dtype, const void* x, const voi
 int launch_norm_bwd(hipStream_t s, int kind, int dtype, const void* x, const void* dy,
                     const float* gamma, const void* dres_in, void* dx, void* dx2,
                     float* dgamma, float* dbeta, void* workspace, uint64_t workspace_bytes,
-                    uint64_t rows, uint32_t C, float eps, uint32_t flags, uint32_t* counters);
+                    uint64_t rows, uint32_t C, float eps, uint32_t flags);
 
 // activation.hip
 int launch_gelu_fwd(hipStream_t s, int dtype, const void* x, void* y, uint64_t n);

@@ -2,14 +2,17 @@
 // fused in (forward: h = x + r is normalised and optionally stored; backward:
 // the incoming residual gradient is added to dx in the same pass).
 //
-// Row mapping.  A row of C elements is owned by TPR threads:
-//   TPR = 64   one wavefront per row, four rows per 256-thread workgroup,
-//              cross-lane sums by DPP / ds_swizzle only            (C <= 1024)
-//   TPR = 256  one workgroup per row, wave totals staged through LDS (C <= 4096)
-//   TPR = 1024 same with 16 waves                                   (C <= 16384)
-// Each thread keeps its NV 128-bit vectors of the row in registers, so a row is
-// read from HBM exactly once per pass; the two-pass mean / variance of the
-// reference (backend.py:416-433) runs on registers.
+// Row mapping.  A row of C elements is owned by TPR threads, the smallest TPR
+// that lets a thread hold its share (NV 128-bit vectors) in registers:
+//   TPR = 16, 32  four / two rows per wavefront (C = 384 is 16 lanes x 6 vectors);
+//                 narrow rows would otherwise leave lanes idle and pay the
+//                 per-row reductions once per row instead of once per 2-4 rows
+//   TPR = 64      one wavefront per row
+//                 (all three: cross-lane sums by DPP / ds_swizzle only, sixteen
+//                 to four rows per 256-thread workgroup)
+//   TPR = 128, 256, 1024  one workgroup per row, wave totals staged through LDS
+// A row is read from HBM exactly once per pass; the two-pass mean / variance of
+// the reference (backend.py:416-433) runs on registers.
 //
 // Backward keeps per-column partial sums of dgamma / dbeta in registers while a
 // workgroup walks its rows (grid-stride), writes one partial row per workgroup
@@ -29,7 +32,7 @@ namespace agrad {
 
 namespace {
 
-constexpr int kMaxEPT = 16;  // elements of a row a thread may keep in registers
+constexpr int kMaxEPT = 24;  // most elements of a row a thread may keep in registers
 
 template <typename T>
 struct NormFwdArgs {
@@ -41,152 +44,68 @@ template <typename T>
 struct NormBwdArgs {
     const T* x; const T* dy; const float* gamma; const T* dres; T* dx; T* dx2;
     float* pgamma; float* pbeta;      // [blocks, C] partial rows, one per workgroup
-    float* ggamma; float* gbeta;      // rows of the upper tree levels, level after level
-    float* dgamma; float* dbeta;      // results
-    uint32_t* counters;               // arrival tickets of every tree group, zero between launches
     uint64_t rows; uint32_t C; float eps; int kind; uint32_t flags;
 };
 
-constexpr uint32_t kGroupSize = 16;   // partial rows folded together at each level
-
-// Column sums of the per-workgroup partial rows, without a second launch and
-// without atomics on the data.  The partial rows form a 16-ary tree.  A
-// workgroup publishes its row and draws a ticket from the counter of its group
-// of 16; whoever draws the group's last ticket adds the group's rows, in row
-// order, into one row of the next level and moves up with it; the workgroup
-// that completes the root writes dgamma / dbeta.  Which workgroup does an
-// addition depends on timing, what is added in which order does not, so the
-// result is the same on every run.  All counters are left at zero.
+// Second stage of the dgamma / dbeta column sums: out[c] (+)= sum over the P
+// partial rows the backward kernel left in the workspace.  One workgroup covers
+// 16 column vectors with 64 row lanes; a row lane loads its rows 16 at a time
+// (independent loads, one memory latency per 1024 rows) and adds them in row
+// order; the 64 lane sums are then added in lane order.  Fixed order, no
+// atomics: the result is the same on every run.
 //
-// The rows cross between workgroups (and between the XCDs' separate L2 caches)
-// through agent-scope relaxed atomic stores and loads, which go to the coherent
-// level of the memory system by themselves; a device-wide release fence would
-// instead write back the whole L2 every time a workgroup finishes.
-//
-// A fold loads its (up to) 16 rows with independent loads before adding them,
-// so it costs one memory latency, not sixteen.
-__device__ __forceinline__ void publish2(float* p, float a, float b) {
-    const unsigned long long bits =
-        (unsigned long long)__float_as_uint(a) | ((unsigned long long)__float_as_uint(b) << 32);
-    __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void publish1(float* p, float a) {
-    __hip_atomic_store(reinterpret_cast<unsigned int*>(p), __float_as_uint(a), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ float2 observe2(const float* p) {
-    const unsigned long long bits = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p),
-                                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    float2 r;
-    r.x = __uint_as_float((unsigned int)bits);
-    r.y = __uint_as_float((unsigned int)(bits >> 32));
-    return r;
-}
-__device__ __forceinline__ float observe1(const float* p) {
-    return __uint_as_float(__hip_atomic_load(reinterpret_cast<const unsigned int*>(p), __ATOMIC_RELAXED,
-                                             __HIP_MEMORY_SCOPE_AGENT));
-}
-
-// dst = [dst +] sum of nrows rows of src; `final` rows go out with ordinary stores
-template <int BLOCK>
-__device__ __forceinline__ void fold_rows(const float* src, uint32_t nrows, uint32_t C, float* dst,
-                                          bool accumulate, bool final) {
-    if ((C & 1u) == 0) {
-        for (uint32_t c = threadIdx.x * 2; c < C; c += BLOCK * 2) {
-            float2 v[kGroupSize];
+// An in-kernel alternative (ticket counters, partial rows exchanged through
+// agent-scope atomic stores, a 16-ary tree) was measured 3 to 11 us slower per
+// call on MI355X than this second launch, and device-wide fences slower still
+// (each one writes back a whole L2), so the second launch stayed.
+template <int W>   // W = 4: float4 columns, W = 1: scalar columns
+__global__ void __launch_bounds__(1024)
+colsum_finalize_kernel(const float* __restrict__ pg, const float* __restrict__ pb, uint32_t P, uint32_t C,
+                       float* __restrict__ dgamma, float* __restrict__ dbeta, int accumulate) {
+    __shared__ float tile[64][16 * W];
+    const float* src = blockIdx.y == 0 ? pg : pb;
+    float* dst = blockIdx.y == 0 ? dgamma : dbeta;
+    if (src == nullptr) return;                      // uniform over the workgroup
+    const uint32_t cl = threadIdx.x & 15, rl = threadIdx.x >> 4;
+    const uint32_t c = (blockIdx.x * 16 + cl) * W;
+    float s[W];
 #pragma unroll
-            for (uint32_t r = 0; r < kGroupSize; ++r)
-                if (r < nrows) v[r] = observe2(src + (uint64_t)r * C + c);
-            float2 s = v[0];
+    for (int k = 0; k < W; ++k) s[k] = 0.0f;
+    if (c < C) {
+        for (uint32_t r0 = rl; r0 < P; r0 += 64 * 16) {
+            float v[16][W];
 #pragma unroll
-            for (uint32_t r = 1; r < kGroupSize; ++r)
-                if (r < nrows) { s.x = s.x + v[r].x; s.y = s.y + v[r].y; }
-            if (final) {
-                if (accumulate) { s.x = dst[c] + s.x; s.y = dst[c + 1] + s.y; }
-                dst[c] = s.x;
-                dst[c + 1] = s.y;
-            } else {
-                publish2(dst + c, s.x, s.y);
+            for (uint32_t j = 0; j < 16; ++j) {
+                const uint32_t r = r0 + j * 64;
+                if (r < P) {
+                    if constexpr (W == 4) {
+                        const float4 t = *reinterpret_cast<const float4*>(src + (uint64_t)r * C + c);
+                        v[j][0] = t.x; v[j][1] = t.y; v[j][2] = t.z; v[j][3] = t.w;
+                    } else {
+                        v[j][0] = src[(uint64_t)r * C + c];
+                    }
+                }
+            }
+#pragma unroll
+            for (uint32_t j = 0; j < 16; ++j) {
+                const uint32_t r = r0 + j * 64;
+                if (r < P) {
+#pragma unroll
+                    for (int k = 0; k < W; ++k) s[k] = s[k] + v[j][k];
+                }
             }
         }
-    } else {
-        for (uint32_t c = threadIdx.x; c < C; c += BLOCK) {
-            float v[kGroupSize];
+    }
 #pragma unroll
-            for (uint32_t r = 0; r < kGroupSize; ++r)
-                if (r < nrows) v[r] = observe1(src + (uint64_t)r * C + c);
-            float s = v[0];
+    for (int k = 0; k < W; ++k) tile[rl][cl * W + k] = s[k];
+    __syncthreads();
+    if (rl == 0 && c < C) {
 #pragma unroll
-            for (uint32_t r = 1; r < kGroupSize; ++r)
-                if (r < nrows) s = s + v[r];
-            if (final) dst[c] = accumulate ? (dst[c] + s) : s;
-            else publish1(dst + c, s);
+        for (int k = 0; k < W; ++k) {
+            float t = tile[0][cl * W + k];
+            for (int j = 1; j < 64; ++j) t = t + tile[j][cl * W + k];
+            dst[c + k] = accumulate ? (dst[c + k] + t) : t;
         }
-    }
-}
-
-// rows of all tree levels above the leaves, for `blocks` leaves
-__host__ __device__ inline uint32_t tree_inner_rows(uint32_t blocks) {
-    uint32_t total = 0;
-    while (blocks > 1) {
-        blocks = (blocks + kGroupSize - 1) / kGroupSize;
-        if (blocks > 1) total += blocks;
-    }
-    return total;
-}
-// counters of all tree levels
-__host__ __device__ inline uint32_t tree_counters(uint32_t blocks) {
-    uint32_t total = 0;
-    do {
-        blocks = (blocks + kGroupSize - 1) / kGroupSize;
-        total += blocks;
-    } while (blocks > 1);
-    return total;
-}
-
-// FENCED: the leaf rows were written with ordinary stores (scalar fallback
-// kernel), so they need the device-wide fence before the ticket.
-template <typename T, int BLOCK, bool FENCED>
-__device__ __forceinline__ void finish_param_grads(const NormBwdArgs<T>& a) {
-    __shared__ uint32_t ticket;
-    const uint32_t C = a.C;
-    const bool accp = (a.flags & AGRAD_ACC_PARAM_GRAD) != 0;
-    const float* src_g = a.pgamma;
-    const float* src_b = a.pbeta;
-    float* up_g = a.ggamma;
-    float* up_b = a.gbeta;
-    uint32_t* counters = a.counters;
-    uint32_t rows = gridDim.x, me = blockIdx.x;
-    if constexpr (FENCED) __threadfence();
-    for (;;) {
-        const uint32_t ngroups = (rows + kGroupSize - 1) / kGroupSize;
-        const uint32_t group = me / kGroupSize;
-        const uint32_t first = group * kGroupSize;
-        const uint32_t members = rows - first < kGroupSize ? rows - first : kGroupSize;
-        // every published store of this workgroup has completed before the ticket is drawn
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
-        if (threadIdx.x == 0)
-            ticket = __hip_atomic_fetch_add(&counters[group], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();
-        if (ticket != members - 1) return;
-        const bool root = ngroups == 1;
-        if (src_g != nullptr)
-            fold_rows<BLOCK>(src_g + (uint64_t)first * C, members, C, root ? a.dgamma : up_g + (uint64_t)group * C,
-                             root && accp, root);
-        if (src_b != nullptr)
-            fold_rows<BLOCK>(src_b + (uint64_t)first * C, members, C, root ? a.dbeta : up_b + (uint64_t)group * C,
-                             root && accp, root);
-        if (threadIdx.x == 0)
-            __hip_atomic_store(&counters[group], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (root) return;
-        src_g = src_g != nullptr ? up_g : nullptr;
-        src_b = src_b != nullptr ? up_b : nullptr;
-        up_g += (uint64_t)ngroups * C;
-        up_b += (uint64_t)ngroups * C;
-        counters += ngroups;
-        rows = ngroups;
-        me = group;
     }
 }
 
@@ -222,16 +141,16 @@ template <> __device__ __forceinline__ float round_through<bf16_t>(float v) {
 // forward, register-resident row
 // ----------------------------------------------------------------------------
 template <typename T, int VEC, int NV, int TPR>
-__global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
+__global__ void __launch_bounds__(TPR >= 128 ? TPR : 256)
 norm_fwd_kernel(const NormFwdArgs<T> a) {
-    constexpr int BLOCK = TPR > 256 ? TPR : 256;
+    constexpr int BLOCK = TPR >= 128 ? TPR : 256;
     constexpr int RPB = BLOCK / TPR;
-    __shared__ float lds[3 * 2 * (TPR / kWave)];
+    __shared__ float lds[3 * 2 * (TPR > kWave ? TPR / kWave : 1)];
 
     const int sub = threadIdx.x / TPR;
     const int lane = threadIdx.x % TPR;
     const uint64_t row = (uint64_t)blockIdx.x * RPB + sub;
-    if (row >= a.rows) return;  // whole waves only (TPR is a multiple of 64); RPB == 1 never exits
+    if (row >= a.rows) return;  // a lane group leaves alone: its sums never read other groups; RPB == 1 never exits
     const uint32_t C = a.C;
     const uint64_t base = row * C;
 
@@ -320,12 +239,13 @@ norm_fwd_kernel(const NormFwdArgs<T> a) {
 // backward, register-resident row, dgamma / dbeta partials per workgroup
 // ----------------------------------------------------------------------------
 template <typename T, int VEC, int NV, int TPR>
-__global__ void __launch_bounds__(TPR > 256 ? TPR : 256)
+__global__ void __launch_bounds__(TPR >= 128 ? TPR : 256)
 norm_bwd_kernel(const NormBwdArgs<T> a) {
-    constexpr int BLOCK = TPR > 256 ? TPR : 256;
+    constexpr int BLOCK = TPR >= 128 ? TPR : 256;
     constexpr int RPB = BLOCK / TPR;
-    __shared__ float lds[3 * 2 * (TPR / kWave)];
-    extern __shared__ float comb[];  // (RPB - 1) * C floats when RPB > 1
+    constexpr int NWAVES = BLOCK / kWave;
+    __shared__ float lds[3 * 2 * (TPR > kWave ? TPR / kWave : 1)];
+    extern __shared__ float comb[];  // (NWAVES - 1) * C floats when RPB > 1
 
     const int sub = threadIdx.x / TPR;
     const int lane = threadIdx.x % TPR;
@@ -473,22 +393,38 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
     // one partial row per workgroup
     if (want_pg || want_pb) {
         if constexpr (RPB > 1) {
+            // lane groups of one wave first (fixed order), then the waves through LDS
+            if constexpr (TPR < kWave) {
+#pragma unroll
+                for (int i = 0; i < NV; ++i)
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) {
+                        if constexpr (TPR == 16) {
+                            pg[i][k] = pg[i][k] + __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, pg[i][k]), kSwizzleXor16));
+                            pb[i][k] = pb[i][k] + __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, pb[i][k]), kSwizzleXor16));
+                        }
+                        pg[i][k] = pg[i][k] + __shfl_xor(pg[i][k], 32);
+                        pb[i][k] = pb[i][k] + __shfl_xor(pb[i][k], 32);
+                    }
+            }
+            const int wave = threadIdx.x / kWave;
+            const bool owner = (threadIdx.x % kWave) < TPR;   // one lane group per wave speaks for it
 #pragma unroll 1
             for (int pass = 0; pass < 2; ++pass) {
                 float* out = pass == 0 ? a.pgamma : a.pbeta;
                 if (out == nullptr) continue;  // uniform over the workgroup
-                if (sub > 0) {
+                if (wave > 0 && owner) {
 #pragma unroll
                     for (int i = 0; i < NV; ++i)
                         if (on[i]) {
                             const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
 #pragma unroll
                             for (int k = 0; k < VEC; ++k)
-                                comb[(uint32_t)(sub - 1) * C + col + k] = pass == 0 ? pg[i][k] : pb[i][k];
+                                comb[(uint32_t)(wave - 1) * C + col + k] = pass == 0 ? pg[i][k] : pb[i][k];
                         }
                 }
                 __syncthreads();
-                if (sub == 0) {
+                if (wave == 0 && owner) {
 #pragma unroll
                     for (int i = 0; i < NV; ++i)
                         if (on[i]) {
@@ -497,11 +433,11 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
 #pragma unroll
                             for (int k = 0; k < VEC; ++k) {
                                 t[k] = pass == 0 ? pg[i][k] : pb[i][k];
-                                for (int w = 0; w < RPB - 1; ++w) t[k] = t[k] + comb[(uint32_t)w * C + col + k];
+                                for (int w = 0; w < NWAVES - 1; ++w) t[k] = t[k] + comb[(uint32_t)w * C + col + k];
                             }
 #pragma unroll
                             for (int k = 0; k < VEC; k += 2)
-                                publish2(out + (uint64_t)blockIdx.x * C + col + k, t[k], t[k + 1]);
+                                { out[(uint64_t)blockIdx.x * C + col + k] = t[k]; out[(uint64_t)blockIdx.x * C + col + k + 1] = t[k + 1]; }
                         }
                 }
                 __syncthreads();
@@ -513,12 +449,11 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
                     const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
 #pragma unroll
                     for (int k = 0; k < VEC; k += 2) {
-                        if (want_pg) publish2(a.pgamma + (uint64_t)blockIdx.x * C + col + k, pg[i][k], pg[i][k + 1]);
-                        if (want_pb) publish2(a.pbeta + (uint64_t)blockIdx.x * C + col + k, pb[i][k], pb[i][k + 1]);
+                        if (want_pg) { a.pgamma[(uint64_t)blockIdx.x * C + col + k] = pg[i][k]; a.pgamma[(uint64_t)blockIdx.x * C + col + k + 1] = pg[i][k + 1]; }
+                        if (want_pb) { a.pbeta[(uint64_t)blockIdx.x * C + col + k] = pb[i][k]; a.pbeta[(uint64_t)blockIdx.x * C + col + k + 1] = pb[i][k + 1]; }
                     }
                 }
         }
-        finish_param_grads<T, BLOCK, false>(a);
     }
 }
 
@@ -643,7 +578,6 @@ __global__ void __launch_bounds__(256) norm_bwd_generic_kernel(const NormBwdArgs
             }
         }
     }
-    if (a.pgamma != nullptr || a.pbeta != nullptr) finish_param_grads<T, 256, true>(a);
 }
 
 // ----------------------------------------------------------------------------
@@ -651,22 +585,33 @@ __global__ void __launch_bounds__(256) norm_bwd_generic_kernel(const NormBwdArgs
 // ----------------------------------------------------------------------------
 struct NormPlan {
     bool generic;
-    int tpr;  // 64, 256, 1024
+    int tpr;  // 16, 32, 64, 128, 256, 1024
     int nv;   // vectors per thread
     int rpb;  // rows per workgroup
 };
 
-NormPlan plan_norm(uint32_t C, int dtype, bool aligned) {
+// elements of a row a thread may hold: more in forward (one array) than in
+// backward (x, dy, gamma and the two column accumulators)
+int norm_max_ept(bool backward) {
+    static const int fwd = [] { const char* e = std::getenv("AGRAD_NORM_EPT_FWD"); int v = e ? std::atoi(e) : 0; return v >= 4 && v <= kMaxEPT ? v : 24; }();
+    static const int bwd = [] { const char* e = std::getenv("AGRAD_NORM_EPT_BWD"); int v = e ? std::atoi(e) : 0; return v >= 4 && v <= kMaxEPT ? v : 16; }();
+    return backward ? bwd : fwd;
+}
+
+NormPlan plan_norm(uint32_t C, int dtype, bool aligned, bool backward) {
     const int vec = dtype == AGRAD_BF16 ? 8 : 4;
     NormPlan p{true, 256, 0, 1};
     if (!aligned || C % vec != 0) return p;
-    const int tprs[3] = {64, 256, 1024};
+    const uint32_t cv = C / vec;
+    const uint32_t max_nv = (uint32_t)(norm_max_ept(backward) / vec);
+    const int tprs[6] = {16, 32, 64, 128, 256, 1024};
     for (int t : tprs) {
-        if (C <= (uint32_t)t * kMaxEPT) {
+        const uint32_t nv = (cv + t - 1) / t;
+        if (nv <= max_nv) {
             p.generic = false;
             p.tpr = t;
-            p.nv = (int)((C + (uint32_t)t * vec - 1) / ((uint32_t)t * vec));
-            p.rpb = t == 64 ? 4 : 1;
+            p.nv = (int)nv;
+            p.rpb = t >= 128 ? 1 : 256 / t;
             return p;
         }
     }
@@ -681,7 +626,7 @@ uint32_t bwd_blocks(const NormPlan& p, uint64_t rows) {
 
 template <typename T, int VEC, int TPR>
 int fwd_pick_nv(hipStream_t s, const NormPlan& p, const NormFwdArgs<T>& a) {
-    constexpr int BLOCK = TPR > 256 ? TPR : 256;
+    constexpr int BLOCK = TPR >= 128 ? TPR : 256;
     const uint32_t grid = (uint32_t)((a.rows + p.rpb - 1) / p.rpb);
     switch (p.nv) {
 #define AGRAD_CASE(N)                                                                  \
@@ -691,7 +636,7 @@ int fwd_pick_nv(hipStream_t s, const NormPlan& p, const NormFwdArgs<T>& a) {
             return AGRAD_OK;                                                           \
         }                                                                              \
         break;
-        AGRAD_CASE(1) AGRAD_CASE(2) AGRAD_CASE(3) AGRAD_CASE(4)
+        AGRAD_CASE(1) AGRAD_CASE(2) AGRAD_CASE(3) AGRAD_CASE(4) AGRAD_CASE(5) AGRAD_CASE(6)
 #undef AGRAD_CASE
     }
     return set_error(AGRAD_EINVAL, "norm forward: no kernel for nv=%d", p.nv);
@@ -699,8 +644,8 @@ int fwd_pick_nv(hipStream_t s, const NormPlan& p, const NormFwdArgs<T>& a) {
 
 template <typename T, int VEC, int TPR>
 int bwd_pick_nv(hipStream_t s, const NormPlan& p, const NormBwdArgs<T>& a, uint32_t grid) {
-    constexpr int BLOCK = TPR > 256 ? TPR : 256;
-    const size_t dyn = p.rpb > 1 ? (size_t)(p.rpb - 1) * a.C * sizeof(float) : 0;
+    constexpr int BLOCK = TPR >= 128 ? TPR : 256;
+    const size_t dyn = p.rpb > 1 ? (size_t)(BLOCK / kWave - 1) * a.C * sizeof(float) : 0;
     switch (p.nv) {
 #define AGRAD_CASE(N)                                                                  \
     case N:                                                                            \
@@ -709,7 +654,7 @@ int bwd_pick_nv(hipStream_t s, const NormPlan& p, const NormBwdArgs<T>& a, uint3
             return AGRAD_OK;                                                           \
         }                                                                              \
         break;
-        AGRAD_CASE(1) AGRAD_CASE(2) AGRAD_CASE(3) AGRAD_CASE(4)
+        AGRAD_CASE(1) AGRAD_CASE(2) AGRAD_CASE(3) AGRAD_CASE(4) AGRAD_CASE(5) AGRAD_CASE(6)
 #undef AGRAD_CASE
     }
     return set_error(AGRAD_EINVAL, "norm backward: no kernel for nv=%d", p.nv);
@@ -723,7 +668,10 @@ int norm_fwd_typed(hipStream_t s, const NormPlan& p, const NormFwdArgs<T>& a) {
         return AGRAD_OK;
     }
     switch (p.tpr) {
+        case 16: return fwd_pick_nv<T, VEC, 16>(s, p, a);
+        case 32: return fwd_pick_nv<T, VEC, 32>(s, p, a);
         case 64: return fwd_pick_nv<T, VEC, 64>(s, p, a);
+        case 128: return fwd_pick_nv<T, VEC, 128>(s, p, a);
         case 256: return fwd_pick_nv<T, VEC, 256>(s, p, a);
         default: return fwd_pick_nv<T, VEC, 1024>(s, p, a);
     }
@@ -737,7 +685,10 @@ int norm_bwd_typed(hipStream_t s, const NormPlan& p, const NormBwdArgs<T>& a, ui
         return AGRAD_OK;
     }
     switch (p.tpr) {
+        case 16: return bwd_pick_nv<T, VEC, 16>(s, p, a, grid);
+        case 32: return bwd_pick_nv<T, VEC, 32>(s, p, a, grid);
         case 64: return bwd_pick_nv<T, VEC, 64>(s, p, a, grid);
+        case 128: return bwd_pick_nv<T, VEC, 128>(s, p, a, grid);
         case 256: return bwd_pick_nv<T, VEC, 256>(s, p, a, grid);
         default: return bwd_pick_nv<T, VEC, 1024>(s, p, a, grid);
     }
@@ -756,14 +707,14 @@ uint32_t norm_bwd_max_blocks() {
 
 uint64_t norm_bwd_workspace_bytes(uint64_t rows, uint32_t C, int dtype) {
     // sized for the larger of the vector and the scalar geometry
-    NormPlan vecp = plan_norm(C, dtype, true);
+    NormPlan vecp = plan_norm(C, dtype, true, true);
     NormPlan genp{true, 256, 0, 1};
     uint64_t blocks = bwd_blocks(genp, rows);
     if (!vecp.generic) {
         const uint64_t b = bwd_blocks(vecp, rows);
         if (b > blocks) blocks = b;
     }
-    return 2ull * (blocks + tree_inner_rows((uint32_t)blocks)) * C * sizeof(float);
+    return 2ull * blocks * C * sizeof(float);
 }
 
 int launch_norm_fwd(hipStream_t s, int kind, int dtype, const void* x, const void* residual,
@@ -779,7 +730,7 @@ int launch_norm_fwd(hipStream_t s, int kind, int dtype, const void* x, const voi
     const bool aligned = aligned16(x) && aligned16(y) && (!residual || aligned16(residual)) &&
                          (!h_out || aligned16(h_out)) && (!gamma || aligned16(gamma)) &&
                          (!beta || aligned16(beta));
-    const NormPlan p = plan_norm(C, dtype, aligned);
+    const NormPlan p = plan_norm(C, dtype, aligned, false);
     if (dtype == AGRAD_F32) {
         NormFwdArgs<float> a{(const float*)x, (const float*)residual, gamma, beta, (float*)h_out,
                              (float*)y, rows, C, eps, kind};
@@ -793,7 +744,7 @@ int launch_norm_fwd(hipStream_t s, int kind, int dtype, const void* x, const voi
 int launch_norm_bwd(hipStream_t s, int kind, int dtype, const void* x, const void* dy,
                     const float* gamma, const void* dres_in, void* dx, void* dx2,
                     float* dgamma, float* dbeta, void* workspace, uint64_t workspace_bytes,
-                    uint64_t rows, uint32_t C, float eps, uint32_t flags, uint32_t* counters) {
+                    uint64_t rows, uint32_t C, float eps, uint32_t flags) {
     if (kind != AGRAD_NORM_LAYER && kind != AGRAD_NORM_RMS)
         return set_error(AGRAD_EINVAL, "norm backward: unknown kind %d", kind);
     if (dtype != AGRAD_F32 && dtype != AGRAD_BF16)
@@ -806,7 +757,7 @@ int launch_norm_bwd(hipStream_t s, int kind, int dtype, const void* x, const voi
     const bool aligned = aligned16(x) && aligned16(dy) && (!dres_in || aligned16(dres_in)) &&
                          (!dx || aligned16(dx)) && (!dx2 || aligned16(dx2)) &&
                          (!gamma || aligned16(gamma));
-    const NormPlan p = plan_norm(C, dtype, aligned);
+    const NormPlan p = plan_norm(C, dtype, aligned, true);
     const uint32_t grid = bwd_blocks(p, rows);
     const bool want_params = dgamma != nullptr || dbeta != nullptr;
     if (rows == 0) {
@@ -817,33 +768,38 @@ int launch_norm_bwd(hipStream_t s, int kind, int dtype, const void* x, const voi
         }
         return AGRAD_OK;
     }
-    const uint32_t inner = tree_inner_rows(grid);
-    float *pg = nullptr, *pb = nullptr, *gg = nullptr, *gb = nullptr;
+    float *pg = nullptr, *pb = nullptr;
     if (want_params) {
-        const uint64_t need = 2ull * ((uint64_t)grid + inner) * C * sizeof(float);
+        const uint64_t need = 2ull * grid * C * sizeof(float);
         if (workspace == nullptr || workspace_bytes < need)
             return set_error(AGRAD_EWORKSPACE, "norm backward: workspace %llu < %llu bytes",
                              (unsigned long long)workspace_bytes, (unsigned long long)need);
         if (!aligned16(workspace)) return set_error(AGRAD_EINVAL, "norm backward: workspace must be 16-byte aligned");
-        if (counters == nullptr || tree_counters(grid) > kNormCounters)
-            return set_error(AGRAD_EINVAL, "norm backward: no ticket counters");
         float* w = (float*)workspace;
-        if (dgamma) { pg = w; gg = w + 2ull * grid * C; }
-        if (dbeta) { pb = w + (uint64_t)grid * C; gb = w + 2ull * grid * C + (uint64_t)inner * C; }
+        if (dgamma) pg = w;
+        if (dbeta) pb = w + (uint64_t)grid * C;
     }
     int rc;
     if (dtype == AGRAD_F32) {
         NormBwdArgs<float> a{(const float*)x, (const float*)dy, gamma, (const float*)dres_in,
-                             (float*)dx, (float*)dx2, pg, pb, gg, gb, dgamma, dbeta, counters,
-                             rows, C, eps, kind, flags};
+                             (float*)dx, (float*)dx2, pg, pb, rows, C, eps, kind, flags};
         rc = norm_bwd_typed<float>(s, p, a, grid);
     } else {
         NormBwdArgs<bf16_t> a{(const bf16_t*)x, (const bf16_t*)dy, gamma, (const bf16_t*)dres_in,
-                              (bf16_t*)dx, (bf16_t*)dx2, pg, pb, gg, gb, dgamma, dbeta, counters,
-                              rows, C, eps, kind, flags};
+                              (bf16_t*)dx, (bf16_t*)dx2, pg, pb, rows, C, eps, kind, flags};
         rc = norm_bwd_typed<bf16_t>(s, p, a, grid);
     }
     if (rc != AGRAD_OK) return rc;
+    if (want_params) {
+        const int accp = (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0;
+        const bool vec4 = C % 4 == 0 && (!dgamma || aligned16(dgamma)) && (!dbeta || aligned16(dbeta));
+        if (vec4)
+            hipLaunchKernelGGL((colsum_finalize_kernel<4>), dim3((C / 4 + 15) / 16, 2), dim3(1024), 0, s, pg, pb, grid,
+                               C, dgamma, dbeta, accp);
+        else
+            hipLaunchKernelGGL((colsum_finalize_kernel<1>), dim3((C + 15) / 16, 2), dim3(1024), 0, s, pg, pb, grid,
+                               C, dgamma, dbeta, accp);
+    }
     return check_hip(hipGetLastError(), "norm backward launch");
 }
 

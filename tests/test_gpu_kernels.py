@@ -558,3 +558,74 @@ def test_pos_embedding_backward(ctx, B, T, C):
     base = rng.standard_normal((T, C), dtype=np.float32)
     got = G.pos_embedding_backward(ctx, dY, dwpe_init=base, flags=capi.ACC_PARAM_GRAD)
     assert_fp32_close(got, base + dwpe, "pos grad accumulate")
+
+
+# ---------------------------------------------------------------------------
+# fills and casts
+# ---------------------------------------------------------------------------
+def test_cast_f32_bf16_bit_exact(ctx):
+    """fp32 -> bf16 on the device equals the reference's integer rule (utils.py:20-27)
+    on random bit patterns, ties, infinities and NaN payloads; accumulate adds the
+    widened old value first (metal_ops.metal:12010-12041)."""
+    import ctypes as C
+    rng = _rng(30)
+    bits = rng.integers(0, 2 ** 32, size=1_000_003, dtype=np.uint64).astype(np.uint32)
+    special = np.array([0x3F808000, 0x3F818000, 0x3F808001, 0x7F800000, 0xFF800000, 0x7F800001, 0x7FC00000,
+                        0xFFFFFFFF, 0x7FA12345, 0x7F7FFFFF, 0x80000000, 0x00000001, 0x00008000, 0x00018000],
+                       dtype=np.uint32)
+    bits[:special.size] = special
+    src = bits.view(np.float32)
+    d_src = ctx.upload(src)
+    d_dst = ctx.upload(np.zeros(src.size, np.uint16))
+    ctx.call("agrad_cast_f32_to_bf16", C.c_void_p(d_src.ptr), C.c_void_p(d_dst.ptr), src.size, 0)
+    ctx.synchronize()
+    got = d_dst.download()
+    np.testing.assert_array_equal(got, ref.f32_to_bf16_bits(src))
+    # widen back: exact
+    d_up = ctx.empty((src.size,), np.float32)
+    ctx.call("agrad_cast_bf16_to_f32", C.c_void_p(d_dst.ptr), C.c_void_p(d_up.ptr), src.size)
+    ctx.synchronize()
+    np.testing.assert_array_equal(d_up.download().view(np.uint32), got.astype(np.uint32) << 16)
+    # accumulate: dst = rne(src + widen(dst)) on finite values
+    a = rng.standard_normal(4099).astype(np.float32)
+    b = to_bf16_bits(rng.standard_normal(4099).astype(np.float32))
+    d_a, d_b = ctx.upload(a), ctx.upload(b)
+    ctx.call("agrad_cast_f32_to_bf16", C.c_void_p(d_a.ptr), C.c_void_p(d_b.ptr), a.size, 1)
+    ctx.synchronize()
+    np.testing.assert_array_equal(d_b.download(), ref.f32_to_bf16_bits(a + from_bf16_bits(b)))
+    for d in (d_src, d_dst, d_up, d_a, d_b):
+        d.free()
+
+
+@pytest.mark.parametrize("itemsize,n,offset", [(4, 1000, 0), (4, 77, 12), (2, 1001, 2), (1, 4099, 3), (4, 1, 4), (2, 0, 0)])
+def test_fill_patterns(ctx, itemsize, n, offset):
+    dt = {1: np.uint8, 2: np.uint16, 4: np.uint32}[itemsize]
+    total = 8192
+    base = ctx.upload(np.full(total, 0xAB, np.uint8))
+    bits = 0x3DCCCCCD if itemsize == 4 else (0x3DCD if itemsize == 2 else 0x5A)
+    ctx.call("agrad_fill", base.buffer_id, offset, bits, itemsize, n)
+    ctx.synchronize()
+    want = np.full(total, 0xAB, np.uint8)
+    want[offset:offset + n * itemsize] = np.full(n, bits, dtype=dt).view(np.uint8)
+    np.testing.assert_array_equal(base.download(), want)
+    base.free()
+
+
+def test_add_and_accumulate(ctx):
+    import ctypes as C
+    rng = _rng(31)
+    for n in (1, 5, 4096, 100_003):
+        x = rng.standard_normal(n).astype(np.float32)
+        y = rng.standard_normal(n).astype(np.float32)
+        dx, dy_ = ctx.upload(x), ctx.upload(y)
+        out = ctx.empty((n,), np.float32)
+        ctx.call("agrad_add_forward", capi.F32, C.c_void_p(dx.ptr), C.c_void_p(dy_.ptr), C.c_void_p(out.ptr), n)
+        ctx.call("agrad_grad_accumulate", capi.F32, C.c_void_p(dx.ptr), C.c_void_p(dy_.ptr), n, capi.ACC_INPUT_GRAD)
+        ctx.synchronize()
+        np.testing.assert_array_equal(out.download(), x + y)
+        np.testing.assert_array_equal(dy_.download(), y + x)
+        ctx.call("agrad_grad_accumulate", capi.F32, C.c_void_p(dx.ptr), C.c_void_p(dy_.ptr), n, 0)
+        ctx.synchronize()
+        np.testing.assert_array_equal(dy_.download(), x)
+        for d in (dx, dy_, out):
+            d.free()
