@@ -168,23 +168,53 @@ emb_prepare_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ keys,
 // tokens whose hash falls in group g.  It reads ALL ids (64 KiB at N = 16384,
 // served by L2), keeps the (token, row) pairs it owns in LDS, counts how many
 // rows belong to lower-numbered groups (that is where its slice of the output
-// starts), sorts its pairs by (token, row) with a bitonic network in LDS, and
-// writes them out.  No atomics on global memory, no scratch, and the output is
-// the same on every run.
+// starts), sorts its pairs by (token, row) with a bitonic network, and writes
+// them out.  No atomics on global memory, and the output is the same on every
+// run.  A group too large for LDS (one token holding a large share of all rows)
+// is gathered into its output slice and sorted there instead.
 constexpr int kSortBlock = 1024;
 constexpr uint32_t kGroupSortMaxN = 16384;
+constexpr uint32_t kSortLdsEntries = 4096;   // (token, row) pairs a workgroup keeps in LDS
 constexpr uint32_t kWaveSortMax = 1024;      // lists up to this size are sorted by a single wave
+
+// Bitonic network in its "flip" form: every comparator puts the smaller key at
+// the lower index, so positions >= n behave as +infinity and need no padding.
+// THREADS threads cooperate; SYNC() separates the steps.
+template <int THREADS, typename SyncFn>
+__device__ __forceinline__ void bitonic_sort_u64(unsigned long long* keys, uint32_t n, uint32_t tid, SyncFn sync) {
+    uint32_t n2 = 1;
+    while (n2 < n) n2 <<= 1;
+    for (uint32_t k = 2; k <= n2; k <<= 1) {
+        for (uint32_t j = k >> 1; j > 0; j >>= 1) {
+            const uint32_t mask = (j == (k >> 1)) ? (k - 1) : j;
+            for (uint32_t i = tid; i < n; i += THREADS) {
+                const uint32_t partner = i ^ mask;
+                if (partner > i && partner < n) {
+                    const unsigned long long a = keys[i], b = keys[partner];
+                    if (a > b) { keys[i] = b; keys[partner] = a; }
+                }
+            }
+            sync();
+        }
+    }
+}
 
 __global__ void __launch_bounds__(kSortBlock)
 emb_group_sort_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ tok_s,
-                      uint32_t* __restrict__ row_s, uint32_t N, uint32_t V, uint32_t log2G,
-                      int* err_flag) {
-    extern __shared__ unsigned long long keys[];   // pow2ceil(N) entries
+                      uint32_t* __restrict__ row_s, unsigned long long* __restrict__ spill,
+                      uint32_t N, uint32_t V, uint32_t log2G, int* err_flag) {
+    __shared__ unsigned long long keys[kSortLdsEntries];
     __shared__ uint32_t s_count, s_less;
     const uint32_t tid = threadIdx.x;
     const uint32_t g = blockIdx.x;
     if (tid == 0) { s_count = 0; s_less = 0; }
     __syncthreads();
+
+    auto owner_of = [&](int32_t t, uint32_t& tok) {
+        const bool bad = t < 0 || (uint32_t)t >= V;
+        tok = bad ? V : (uint32_t)t;
+        return log2G ? (tok * 0x9E3779B1u) >> (32 - log2G) : 0u;
+    };
 
     uint32_t less = 0;
     constexpr int ROUND = 16;                       // id loads in flight per thread
@@ -199,21 +229,19 @@ emb_group_sort_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ to
         for (int r = 0; r < ROUND; ++r) {
             const uint32_t i = base + r * kSortBlock + tid;
             if (i < N) {
-                const bool bad = t[r] < 0 || (uint32_t)t[r] >= V;
-                const uint32_t tok = bad ? V : (uint32_t)t[r];
-                if (bad && g == 0) *err_flag = 1;
-                const uint32_t owner = log2G ? (tok * 0x9E3779B1u) >> (32 - log2G) : 0u;
+                uint32_t tok;
+                const uint32_t owner = owner_of(t[r], tok);
+                if (tok == V && g == 0) *err_flag = 1;
                 less += owner < g ? 1u : 0u;
                 if (owner == g) {
                     const uint32_t slot = atomicAdd(&s_count, 1u);
-                    keys[slot] = ((unsigned long long)tok << 32) | i;
+                    if (slot < kSortLdsEntries) keys[slot] = ((unsigned long long)tok << 32) | i;
                 }
             }
         }
     }
-    // rows owned by lower groups: wave totals (exact integers) added in LDS
+    // rows owned by lower groups: exact integer wave totals, added in LDS
     {
-        float unused = 0.0f; (void)unused;
         uint32_t v = less;
         v += __builtin_amdgcn_update_dpp(0, v, kDppQuadXor1, 0xf, 0xf, true);
         v += __builtin_amdgcn_update_dpp(0, v, kDppQuadXor2, 0xf, 0xf, true);
@@ -226,47 +254,43 @@ emb_group_sort_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ to
     __syncthreads();
     const uint32_t count = s_count;
     const uint32_t offset = s_less;
-    uint32_t n2 = 2;
-    while (n2 < count) n2 <<= 1;
-    for (uint32_t i = count + tid; i < n2; i += kSortBlock) keys[i] = ~0ull;
-    __syncthreads();
-    if (n2 <= kWaveSortMax) {
-        // small list (the usual case): one wave sorts it with no workgroup
-        // barriers; a wave's LDS operations complete in program order
-        if (tid < kWave) {
-            for (uint32_t k = 2; k <= n2; k <<= 1) {
-                for (uint32_t j = k >> 1; j > 0; j >>= 1) {
-                    for (uint32_t i = tid; i < n2; i += kWave) {
-                        const uint32_t partner = i ^ j;
-                        if (partner > i) {
-                            const unsigned long long a = keys[i], b = keys[partner];
-                            const bool ascending = (i & k) == 0;
-                            if ((a > b) == ascending) { keys[i] = b; keys[partner] = a; }
-                        }
-                    }
+
+    if (count <= kSortLdsEntries) {
+        if (count <= kWaveSortMax) {
+            // the usual case: one wave sorts the list with no workgroup barriers
+            // (a wave's LDS operations complete in program order)
+            if (tid < kWave)
+                bitonic_sort_u64<kWave>(keys, count, tid, [] {
                     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
                     __builtin_amdgcn_wave_barrier();
-                }
-            }
+                });
+            __syncthreads();
+        } else {
+            bitonic_sort_u64<kSortBlock>(keys, count, tid, [] { __syncthreads(); });
         }
-        __syncthreads();
-    } else {
-        for (uint32_t k = 2; k <= n2; k <<= 1) {
-            for (uint32_t j = k >> 1; j > 0; j >>= 1) {
-                for (uint32_t i = tid; i < n2; i += kSortBlock) {
-                    const uint32_t partner = i ^ j;
-                    if (partner > i) {
-                        const unsigned long long a = keys[i], b = keys[partner];
-                        const bool ascending = (i & k) == 0;
-                        if ((a > b) == ascending) { keys[i] = b; keys[partner] = a; }
-                    }
-                }
-                __syncthreads();
-            }
+        for (uint32_t i = tid; i < count; i += kSortBlock) {
+            const unsigned long long key = keys[i];
+            tok_s[offset + i] = (uint32_t)(key >> 32);
+            row_s[offset + i] = (uint32_t)key;
         }
+        return;
     }
+
+    // oversized group: gather its pairs into this group's slice of `spill`
+    // (slices are disjoint: [offset, offset + count)), sort there, then split
+    __syncthreads();
+    if (tid == 0) s_count = 0;
+    __syncthreads();
+    unsigned long long* mine = spill + offset;
+    for (uint32_t i = tid; i < N; i += kSortBlock) {
+        uint32_t tok;
+        if (owner_of(ids[i], tok) == g) mine[atomicAdd(&s_count, 1u)] = ((unsigned long long)tok << 32) | i;
+    }
+    __threadfence_block();
+    __syncthreads();
+    bitonic_sort_u64<kSortBlock>(mine, count, tid, [] { __threadfence_block(); __syncthreads(); });
     for (uint32_t i = tid; i < count; i += kSortBlock) {
-        const unsigned long long key = keys[i];
+        const unsigned long long key = mine[i];
         tok_s[offset + i] = (uint32_t)(key >> 32);
         row_s[offset + i] = (uint32_t)key;
     }
@@ -452,9 +476,10 @@ int plan_embedding(uint64_t N, uint32_t C, uint32_t V, EmbPlan* p) {
                                                (unsigned)bits, (hipStream_t)0, false);
     if (err != hipSuccess) return check_hip(err, "radix sort temp-size query");
     uint64_t o = 0;
+    // keys_in and vals_in are adjacent: the grouping sort uses the pair as N 64-bit spill slots
     p->off_keys_in = o;  o += align256(N * 4);
-    p->off_keys_out = o; o += align256(N * 4);
     p->off_vals_in = o;  o += align256(N * 4);
+    p->off_keys_out = o; o += align256(N * 4);
     p->off_vals_out = o; o += align256(N * 4);
     p->off_temp = o;     o += align256(temp);
     p->temp_bytes = temp;
@@ -476,20 +501,13 @@ int embedding_bwd_typed(hipStream_t s, const EmbPlan& p, const int32_t* ids, con
 
     bool grouped = false;
     if (N <= kGroupSortMaxN && group_sort_enabled()) {
-        uint32_t cap = 2;
-        while (cap < N) cap <<= 1;
-        const size_t lds = (size_t)cap * sizeof(unsigned long long);
-        static const bool big_lds_ok = [] {
-            return hipFuncSetAttribute(reinterpret_cast<const void*>(emb_group_sort_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)(kGroupSortMaxN * sizeof(unsigned long long))) == hipSuccess;
-        }();
-        if (lds <= 48 * 1024 || big_lds_ok) {
-            const uint32_t log2G = N > 1024 ? 8u : 4u;
-            hipLaunchKernelGGL(emb_group_sort_kernel, dim3(1u << log2G), dim3(kSortBlock), lds, s, ids, keys_out,
-                               vals_out, N, V, log2G, err_flag);
-            grouped = true;
-        }
+        // keys_in / vals_in are adjacent and unused on this path: together they hold N 64-bit spill slots
+        static_assert(sizeof(unsigned long long) == 2 * sizeof(uint32_t), "spill layout");
+        unsigned long long* spill = reinterpret_cast<unsigned long long*>(ws + p.off_keys_in);
+        const uint32_t log2G = N > 1024 ? 8u : 4u;
+        hipLaunchKernelGGL(emb_group_sort_kernel, dim3(1u << log2G), dim3(kSortBlock), 0, s, ids, keys_out, vals_out,
+                           spill, N, V, log2G, err_flag);
+        grouped = true;
     }
     if (!grouped) {
         hipLaunchKernelGGL(emb_prepare_kernel, dim3((N + 255) / 256), dim3(256), 0, s, ids, keys_in, vals_in, N, V, err_flag);

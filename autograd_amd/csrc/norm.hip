@@ -49,10 +49,10 @@ struct NormBwdArgs {
 
 // Second stage of the dgamma / dbeta column sums: out[c] (+)= sum over the P
 // partial rows the backward kernel left in the workspace.  One workgroup covers
-// 16 column vectors with 64 row lanes; a row lane loads its rows 16 at a time
+// 8 column vectors with 128 row lanes; a row lane loads its rows 8 at a time
 // (independent loads, one memory latency per 1024 rows) and adds them in row
-// order; the 64 lane sums are then added in lane order.  Fixed order, no
-// atomics: the result is the same on every run.
+// order; the 128 lane sums are then added in lane order in two steps.  Fixed
+// order, no atomics: the result is the same on every run.
 //
 // An in-kernel alternative (ticket counters, partial rows exchanged through
 // agent-scope atomic stores, a 16-ary tree) was measured 3 to 11 us slower per
@@ -62,21 +62,23 @@ template <int W>   // W = 4: float4 columns, W = 1: scalar columns
 __global__ void __launch_bounds__(1024)
 colsum_finalize_kernel(const float* __restrict__ pg, const float* __restrict__ pb, uint32_t P, uint32_t C,
                        float* __restrict__ dgamma, float* __restrict__ dbeta, int accumulate) {
-    __shared__ float tile[64][16 * W];
+    constexpr int COLS = 8, LANES = 128, BATCH = 8;
+    __shared__ float tile[LANES][COLS * W];
+    __shared__ float tile2[LANES / 16][COLS * W];
     const float* src = blockIdx.y == 0 ? pg : pb;
     float* dst = blockIdx.y == 0 ? dgamma : dbeta;
     if (src == nullptr) return;                      // uniform over the workgroup
-    const uint32_t cl = threadIdx.x & 15, rl = threadIdx.x >> 4;
-    const uint32_t c = (blockIdx.x * 16 + cl) * W;
+    const uint32_t cl = threadIdx.x % COLS, rl = threadIdx.x / COLS;
+    const uint32_t c = (blockIdx.x * COLS + cl) * W;
     float s[W];
 #pragma unroll
     for (int k = 0; k < W; ++k) s[k] = 0.0f;
     if (c < C) {
-        for (uint32_t r0 = rl; r0 < P; r0 += 64 * 16) {
-            float v[16][W];
+        for (uint32_t r0 = rl; r0 < P; r0 += LANES * BATCH) {
+            float v[BATCH][W];
 #pragma unroll
-            for (uint32_t j = 0; j < 16; ++j) {
-                const uint32_t r = r0 + j * 64;
+            for (uint32_t j = 0; j < BATCH; ++j) {
+                const uint32_t r = r0 + j * LANES;
                 if (r < P) {
                     if constexpr (W == 4) {
                         const float4 t = *reinterpret_cast<const float4*>(src + (uint64_t)r * C + c);
@@ -87,8 +89,8 @@ colsum_finalize_kernel(const float* __restrict__ pg, const float* __restrict__ p
                 }
             }
 #pragma unroll
-            for (uint32_t j = 0; j < 16; ++j) {
-                const uint32_t r = r0 + j * 64;
+            for (uint32_t j = 0; j < BATCH; ++j) {
+                const uint32_t r = r0 + j * LANES;
                 if (r < P) {
 #pragma unroll
                     for (int k = 0; k < W; ++k) s[k] = s[k] + v[j][k];
@@ -99,11 +101,23 @@ colsum_finalize_kernel(const float* __restrict__ pg, const float* __restrict__ p
 #pragma unroll
     for (int k = 0; k < W; ++k) tile[rl][cl * W + k] = s[k];
     __syncthreads();
+    // 128 lane sums -> 8 (each adds 16 in lane order) -> 1
+    if (rl < LANES / 16) {
+#pragma unroll
+        for (int k = 0; k < W; ++k) {
+            float t = tile[rl * 16][cl * W + k];
+#pragma unroll
+            for (int j = 1; j < 16; ++j) t = t + tile[rl * 16 + j][cl * W + k];
+            tile2[rl][cl * W + k] = t;
+        }
+    }
+    __syncthreads();
     if (rl == 0 && c < C) {
 #pragma unroll
         for (int k = 0; k < W; ++k) {
-            float t = tile[0][cl * W + k];
-            for (int j = 1; j < 64; ++j) t = t + tile[j][cl * W + k];
+            float t = tile2[0][cl * W + k];
+#pragma unroll
+            for (int j = 1; j < LANES / 16; ++j) t = t + tile2[j][cl * W + k];
             dst[c + k] = accumulate ? (dst[c + k] + t) : t;
         }
     }
@@ -794,10 +808,10 @@ int launch_norm_bwd(hipStream_t s, int kind, int dtype, const void* x, const voi
         const int accp = (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0;
         const bool vec4 = C % 4 == 0 && (!dgamma || aligned16(dgamma)) && (!dbeta || aligned16(dbeta));
         if (vec4)
-            hipLaunchKernelGGL((colsum_finalize_kernel<4>), dim3((C / 4 + 15) / 16, 2), dim3(1024), 0, s, pg, pb, grid,
+            hipLaunchKernelGGL((colsum_finalize_kernel<4>), dim3((C / 4 + 7) / 8, 2), dim3(1024), 0, s, pg, pb, grid,
                                C, dgamma, dbeta, accp);
         else
-            hipLaunchKernelGGL((colsum_finalize_kernel<1>), dim3((C + 15) / 16, 2), dim3(1024), 0, s, pg, pb, grid,
+            hipLaunchKernelGGL((colsum_finalize_kernel<1>), dim3((C + 7) / 8, 2), dim3(1024), 0, s, pg, pb, grid,
                                C, dgamma, dbeta, accp);
     }
     return check_hip(hipGetLastError(), "norm backward launch");

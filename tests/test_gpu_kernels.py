@@ -495,6 +495,9 @@ def _zipf_ids(rng, n, V, s=1.1):
     (3, 700, 97, 50, "uniform"),          # heavy duplication, scalar columns
     (4, 1024, 1000, 768, "zipf"),         # long runs crossing chunk edges
     (1, 3000, 1, 16, "uniform"),          # a single token: one run over every chunk
+    (1, 12000, 1, 8, "uniform"),          # one token group larger than the sort's LDS list
+    (2, 8000, 5, 24, "uniform"),          # several such groups
+    (4, 8192, 4000, 64, "zipf"),          # N = 32768: the radix-sort path
 ])
 def test_embedding_backward_fp32(ctx, B, T, V, C, dist):
     rng = _rng(20)
@@ -503,7 +506,12 @@ def test_embedding_backward_fp32(ctx, B, T, V, C, dist):
     got = G.embedding_backward(ctx, ids, dY, V)
     dW = np.zeros((V, C), np.float32)
     ref.gather_backward_into(ids, dY, dW)
-    assert_fp32_close(got, dW, f"embedding backward {dist}", rtol=1e-5, atol=2e-6 if dist == "uniform" and V > 1 else 1e-4)
+    # the CPU adds a token's rows one by one in fp32: its own rounding noise grows
+    # with the longest run (about 6e-8 * run length for N(0,1) rows), so the
+    # absolute budget follows it; for runs of a few rows it is 2e-6
+    longest = int(np.bincount(ids.ravel(), minlength=V).max())
+    atol = max(2e-6, 2.5e-7 * longest)
+    assert_fp32_close(got, dW, f"embedding backward {dist}", rtol=1e-5, atol=atol)
     # rows of tokens that never occur stay exactly zero; column sums are preserved
     unseen = np.setdiff1d(np.arange(V), ids.ravel())
     assert not got[unseen].any()
@@ -516,7 +524,7 @@ def test_embedding_backward_fp32(ctx, B, T, V, C, dist):
     # accumulate onto an existing table
     base = rng.standard_normal((V, C), dtype=np.float32)
     acc = G.embedding_backward(ctx, ids, dY, V, dW_init=base, flags=capi.ACC_PARAM_GRAD)
-    assert_fp32_close(acc, base + dW, "embedding backward accumulate", rtol=1e-5, atol=1e-4)
+    assert_fp32_close(acc, base + dW, "embedding backward accumulate", rtol=1e-5, atol=max(1e-4, atol))
     np.testing.assert_array_equal(acc[unseen], base[unseen])
 
 
