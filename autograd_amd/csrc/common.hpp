@@ -100,6 +100,30 @@ template <> struct VecIO<bf16_t, 1> {
     }
 };
 
+// Raw access: the bits of one vector as loaded, unpacked to fp32 later.  A
+// kernel that prefetches the next row keeps it in this form, so the wait for
+// the data sits where the values are first used, not where they were requested.
+template <typename T, int V> struct RawVec;
+template <> struct RawVec<float, 4> {
+    typedef f32x4 type;
+    static __device__ __forceinline__ type load(const float* p) { return __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p)); }
+    static __device__ __forceinline__ type zero() { return f32x4{0.0f, 0.0f, 0.0f, 0.0f}; }
+    static __device__ __forceinline__ void unpack(const type& r, float (&v)[4]) { v[0] = r.x; v[1] = r.y; v[2] = r.z; v[3] = r.w; }
+};
+template <> struct RawVec<bf16_t, 8> {
+    typedef u32x4 type;
+    static __device__ __forceinline__ type load(const bf16_t* p) { return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)); }
+    static __device__ __forceinline__ type zero() { return u32x4{0u, 0u, 0u, 0u}; }
+    static __device__ __forceinline__ void unpack(const type& r, float (&v)[8]) {
+        const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            v[2 * i]     = __uint_as_float(w[i] << 16);
+            v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+    }
+};
+
 // Widest vector a dtype supports (16 bytes).
 template <typename T> struct WideVec;
 template <> struct WideVec<float>  { static constexpr int value = 4; };

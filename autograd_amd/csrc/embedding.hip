@@ -168,14 +168,15 @@ emb_prepare_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ keys,
 // tokens whose hash falls in group g.  It reads ALL ids (64 KiB at N = 16384,
 // served by L2), keeps the (token, row) pairs it owns in LDS, counts how many
 // rows belong to lower-numbered groups (that is where its slice of the output
-// starts), sorts its pairs by (token, row) with a bitonic network, and writes
-// them out.  No atomics on global memory, and the output is the same on every
+// starts), orders its pairs by (token, row) -- by rank counting when there is at
+// most one pair per thread, with a bitonic network otherwise -- and writes them
+// out.  No atomics on global memory, and the output is the same on every
 // run.  A group too large for LDS (one token holding a large share of all rows)
 // is gathered into its output slice and sorted there instead.
 constexpr int kSortBlock = 1024;
 constexpr uint32_t kGroupSortMaxN = 16384;
 constexpr uint32_t kSortLdsEntries = 4096;   // (token, row) pairs a workgroup keeps in LDS
-constexpr uint32_t kWaveSortMax = 1024;      // lists up to this size are sorted by a single wave
+constexpr uint32_t kRankSortMax = kSortBlock;  // lists up to one key per thread are placed by rank
 
 // Bitonic network in its "flip" form: every comparator puts the smaller key at
 // the lower index, so positions >= n behave as +infinity and need no padding.
@@ -255,19 +256,22 @@ emb_group_sort_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ to
     const uint32_t count = s_count;
     const uint32_t offset = s_less;
 
-    if (count <= kSortLdsEntries) {
-        if (count <= kWaveSortMax) {
-            // the usual case: one wave sorts the list with no workgroup barriers
-            // (a wave's LDS operations complete in program order)
-            if (tid < kWave)
-                bitonic_sort_u64<kWave>(keys, count, tid, [] {
-                    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-                    __builtin_amdgcn_wave_barrier();
-                });
-            __syncthreads();
-        } else {
-            bitonic_sort_u64<kSortBlock>(keys, count, tid, [] { __syncthreads(); });
+    if (count <= kRankSortMax) {
+        // the usual case (a few dozen pairs): every key is unique, so its place
+        // in the order is the number of smaller keys.  Each thread counts that
+        // for its own key with broadcast LDS reads -- no barriers, no exchanges.
+        const unsigned long long mine = tid < count ? keys[tid] : ~0ull;
+        uint32_t rank = 0;
+#pragma unroll 8
+        for (uint32_t j = 0; j < count; ++j) rank += keys[j] < mine ? 1u : 0u;
+        if (tid < count) {
+            tok_s[offset + rank] = (uint32_t)(mine >> 32);
+            row_s[offset + rank] = (uint32_t)mine;
         }
+        return;
+    }
+    if (count <= kSortLdsEntries) {
+        bitonic_sort_u64<kSortBlock>(keys, count, tid, [] { __syncthreads(); });
         for (uint32_t i = tid; i < count; i += kSortBlock) {
             const unsigned long long key = keys[i];
             tok_s[offset + i] = (uint32_t)(key >> 32);

@@ -287,19 +287,38 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
     }
     SlotRing ring;
 
-    for (uint64_t row = (uint64_t)blockIdx.x * RPB + sub; row < a.rows;
-         row += (uint64_t)gridDim.x * RPB) {
+    // Rows are software-pipelined: the x and dy vectors of the NEXT row are
+    // requested (as raw bits) before the current row is worked on, so a wave
+    // always has a row of loads in flight while it computes.
+    typedef RawVec<T, VEC> Raw;
+    typename Raw::type nx[NV], ng[NV];
+    const uint64_t stride = (uint64_t)gridDim.x * RPB;
+    uint64_t row = (uint64_t)blockIdx.x * RPB + sub;
+    if (row < a.rows) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
+            nx[i] = on[i] ? Raw::load(a.x + row * C + col) : Raw::zero();
+            ng[i] = on[i] ? Raw::load(a.dy + row * C + col) : Raw::zero();
+        }
+    }
+    for (; row < a.rows; row += stride) {
         const uint64_t base = row * C;
         float xv[NV][VEC], g[NV][VEC];
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
-            if (on[i]) {
-                VecIO<T, VEC>::load(a.x + base + col, xv[i]);
-                VecIO<T, VEC>::load(a.dy + base + col, g[i]);
-            } else {
+            Raw::unpack(nx[i], xv[i]);
+            Raw::unpack(ng[i], g[i]);
+        }
+        if (row + stride < a.rows) {
+            const uint64_t nbase = (row + stride) * C;
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) { xv[i][k] = 0.0f; g[i][k] = 0.0f; }
+            for (int i = 0; i < NV; ++i) {
+                const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
+                if (on[i]) {
+                    nx[i] = Raw::load(a.x + nbase + col);
+                    ng[i] = Raw::load(a.dy + nbase + col);
+                }
             }
         }
 
@@ -604,12 +623,17 @@ struct NormPlan {
     int rpb;  // rows per workgroup
 };
 
-// elements of a row a thread may hold: more in forward (one array) than in
-// backward (x, dy, gamma and the two column accumulators)
-int norm_max_ept(bool backward) {
-    static const int fwd = [] { const char* e = std::getenv("AGRAD_NORM_EPT_FWD"); int v = e ? std::atoi(e) : 0; return v >= 4 && v <= kMaxEPT ? v : 24; }();
-    static const int bwd = [] { const char* e = std::getenv("AGRAD_NORM_EPT_BWD"); int v = e ? std::atoi(e) : 0; return v >= 4 && v <= kMaxEPT ? v : 16; }();
-    return backward ? bwd : fwd;
+// Elements of a row a thread may hold.  Forward keeps one array; backward keeps
+// x, dy, gamma, the two column accumulators and the prefetched next row, so it
+// gets fewer -- except bf16, whose prefetched rows stay packed (half the
+// registers).  Measured on MI355X over the benchmark shapes; the environment
+// variables override for sweeps.
+int norm_max_ept(bool backward, int dtype) {
+    static const int fwd = [] { const char* e = std::getenv("AGRAD_NORM_EPT_FWD"); int v = e ? std::atoi(e) : 0; return v >= 4 && v <= kMaxEPT ? v : 0; }();
+    static const int bwd = [] { const char* e = std::getenv("AGRAD_NORM_EPT_BWD"); int v = e ? std::atoi(e) : 0; return v >= 4 && v <= kMaxEPT ? v : 0; }();
+    if (!backward) return fwd ? fwd : 24;
+    if (bwd) return bwd;
+    return dtype == AGRAD_BF16 ? 24 : 16;
 }
 
 NormPlan plan_norm(uint32_t C, int dtype, bool aligned, bool backward) {
@@ -617,7 +641,7 @@ NormPlan plan_norm(uint32_t C, int dtype, bool aligned, bool backward) {
     NormPlan p{true, 256, 0, 1};
     if (!aligned || C % vec != 0) return p;
     const uint32_t cv = C / vec;
-    const uint32_t max_nv = (uint32_t)(norm_max_ept(backward) / vec);
+    const uint32_t max_nv = (uint32_t)(norm_max_ept(backward, dtype) / vec);
     const int tprs[6] = {16, 32, 64, 128, 256, 1024};
     for (int t : tprs) {
         const uint32_t nv = (cv + t - 1) / t;
@@ -634,7 +658,9 @@ NormPlan plan_norm(uint32_t C, int dtype, bool aligned, bool backward) {
 
 uint32_t bwd_blocks(const NormPlan& p, uint64_t rows) {
     const uint64_t want = (rows + p.rpb - 1) / p.rpb;
-    const uint64_t cap = norm_bwd_max_blocks();
+    // more partial rows buy more rows in flight; worth it once there are many rows
+    uint64_t cap = norm_bwd_max_blocks();
+    if (cap == 0) cap = rows >= 32768 ? 2048 : 1024;
     return (uint32_t)(want < cap ? (want ? want : 1) : cap);
 }
 
@@ -714,7 +740,7 @@ uint32_t norm_bwd_max_blocks() {
     static const uint32_t value = [] {
         const char* e = std::getenv("AGRAD_NORM_BWD_BLOCKS");
         long v = e ? std::atol(e) : 0;
-        return (uint32_t)(v > 0 && v <= 2048 ? v : 1024);
+        return (uint32_t)(v > 0 && v <= 4096 ? v : 0);   // 0: choose from the row count
     }();
     return value;
 }
