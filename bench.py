@@ -44,6 +44,13 @@ from autograd_amd.utils import f32_array_to_bf16_bits  # noqa: E402
 
 METRIC = "HBM GB/s (% of 8 TB/s) + tokens/s for fused norm/act/RoPE/embed fwd+bwd"
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of a workload's dominant kernel, from two `rocprofv3 --pmc`
+# runs of this file (FETCH_SIZE, then WRITE_SIZE), each scaled by what the counter
+# reads for the 64 MiB copy of spin_up(); the run and its numbers are recorded in
+# profiles/hbm_traffic_*.txt.  Keyed by config index, then "op direction".
+MEASURED_TRAFFIC_BYTES = {
+    1: {"relu2 bwd": 301.95e6},
+}
 ROTATE_BYTES = 768 << 20      # cycle at least this much distinct memory per op
 MAX_SETS = 8
 
@@ -282,8 +289,9 @@ def spin_up(ctx, seconds=0.25):
     b.free()
 
 
-def time_case(ctx, case, iters):
-    # at least `iters` launches and at least ~2 ms of GPU time
+def time_case(ctx, case, iters, exact=False):
+    # at least `iters` launches and at least ~2 ms of GPU time (exactly `iters`
+    # launches when exact: a counter-collection run pays per dispatch)
     for i in range(min(case.nsets, 3)):
         case.launch(i)
     ctx.synchronize()
@@ -291,7 +299,8 @@ def time_case(ctx, case, iters):
     for it in range(8):
         case.launch(it % case.nsets)
     probe_us = ctx.timer_stop() * 1e3 / 8
-    iters = int(max(iters, min(2000, 2000.0 / max(probe_us, 0.5))))
+    if not exact:
+        iters = int(max(iters, min(2000, 2000.0 / max(probe_us, 0.5))))
     ctx.timer_start()
     for it in range(iters):
         case.launch(it % case.nsets)
@@ -319,7 +328,7 @@ def run_config(ctx, cfg, iters):
         pool.release()
 
 
-def run_workload(ctx, cfg, steps, warmup, iters):
+def run_workload(ctx, cfg, steps, warmup, iters, exact=False):
     pool = Pool(ctx, cfg.seed)
     try:
         cases = build_cases(ctx, cfg, pool)
@@ -339,7 +348,7 @@ def run_workload(ctx, cfg, steps, warmup, iters):
         ctx.synchronize()
         wall = time.perf_counter() - t0
         for case in cases:
-            time_case(ctx, case, iters)
+            time_case(ctx, case, iters, exact)
         return cases, step_bytes, wall
     finally:
         pool.release()
@@ -447,6 +456,9 @@ def main():
     ap.add_argument("--iters", type=int, default=30, help="launches per op in the per-op timing")
     ap.add_argument("--workload-only", action="store_true", help="skip the per-op tables of the other configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--exact-iters", action="store_true",
+                    help="time each op over exactly --iters launches and shorten the clock spin-up "
+                         "(for rocprofv3 --pmc runs, which serialise every dispatch)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this build has no multi-GPU path (asked for --gpus {args.gpus}); "
@@ -455,8 +467,8 @@ def main():
         return 2
     cfg = CONFIGS[args.config]
     ctx = capi.Context(0)
-    spin_up(ctx)
-    cases, step_bytes, wall = run_workload(ctx, cfg, args.steps, args.warmup, args.iters)
+    spin_up(ctx, 0.02 if args.exact_iters else 0.25)
+    cases, step_bytes, wall = run_workload(ctx, cfg, args.steps, args.warmup, args.iters, args.exact_iters)
     ms_per_step = wall * 1e3 / args.steps
     gbps = step_bytes * args.steps / wall / 1e9
     timed = [c for c in cases if c.direction in ("fwd", "bwd")]
@@ -473,8 +485,9 @@ def main():
         "pct_of_hbm_peak": round(100 * gbps / HBM_PEAK_GBS, 2),
         "roofline": {"bound": "hbm", "kernel": dom.kernel, "op": f"{dom.op} {dom.direction}",
                      "achieved": round(dom_gbps, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(dom_gbps / HBM_PEAK_GBS, 4), "traffic": None,
-                     "launch_us": round(dom.us, 2), "algorithmic_MB": round(dom.nbytes / 1e6, 2)},
+                     "frac": round(dom_gbps / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.index, {}).get(f"{dom.op} {dom.direction}"),
+                     "launch_us": round(dom.us, 2), "algorithmic_bytes": dom.nbytes},
         "per_op": [case_row(c) for c in cases],
     }
     if not args.no_cpu:
