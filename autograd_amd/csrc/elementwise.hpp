@@ -11,7 +11,7 @@
 
 namespace agrad {
 
-constexpr int kEwBlock = 256;
+constexpr int kEwBlock = 64;
 
 template <typename T, int NIN>
 struct EwArgs {

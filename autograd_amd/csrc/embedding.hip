@@ -335,7 +335,7 @@ __device__ __forceinline__ void store_grad_row(T* dW, uint64_t off, const float 
 // j, j + blockDim, ...  Control flow depends only on the (uniform) token run
 // structure, so a workgroup never diverges except on the column mask.
 template <typename T, int VEC>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(512)
 emb_segment_sum_kernel(const uint32_t* __restrict__ tok_s, const uint32_t* __restrict__ row_s,
                        const T* __restrict__ dY, T* dW, float* __restrict__ carry_head,
                        float* __restrict__ carry_tail, uint32_t N, uint32_t C, uint32_t CV,
@@ -401,36 +401,149 @@ emb_segment_sum_kernel(const uint32_t* __restrict__ tok_s, const uint32_t* __res
 }
 
 // A run that crosses chunk edges starts as the tail partial of its first chunk
-// and continues as head partials of the following chunks.  The workgroup of the
-// first chunk adds them in chunk order and stores the token's row.
+// (its origin) and continues as head partials of the following chunks.  One
+// workgroup per chunk:
+//   * a run with at most kFixLanes head partials (every run of a spread-out
+//     token distribution) is finished by its origin, a thread per column;
+//   * a long run -- a hot token under a Zipf distribution spans hundreds of
+//     chunks -- is finished slab by slab (kFixCols column vectors each).  The
+//     chunks in the middle of the run have nothing else to do, so middle chunk
+//     i takes slab i and the origin takes the slabs left over.  Within a slab,
+//     kFixLanes lanes per column each add every kFixLanes-th partial in chunk
+//     order with kFixBatch loads in flight, and the lanes are then added in
+//     lane order: a fixed association, the same on every run.
+// Run ends come from binary searches on "equals this token" over the sorted
+// positions (equal tokens are contiguous whichever sorter ran).
+constexpr int kFixCols = 64;    // column vectors per slab
+constexpr int kFixLanes = 4;    // partial-sum lanes per column
+constexpr int kFixBatch = 8;    // partial rows a lane keeps in flight
+
 template <typename T, int VEC>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(kFixCols * kFixLanes)
 emb_carry_fix_kernel(const uint32_t* __restrict__ tok_s, T* dW, const float* __restrict__ carry_head,
                      const float* __restrict__ carry_tail, uint32_t N, uint32_t C, uint32_t CV,
-                     uint32_t V, uint32_t L, uint32_t chunks, int accumulate) {
-    const ChunkEdges e = chunk_edges(tok_s, blockIdx.x, L, N);
+                     uint32_t V, uint32_t L, int accumulate) {
+    __shared__ float part[kFixLanes][kFixCols * VEC];
+    const uint32_t chunk = blockIdx.x;
+    const ChunkEdges e = chunk_edges(tok_s, chunk, L, N);
     const bool origin = e.open_right && !(e.single && e.open_left);
-    if (!origin) return;
+    const bool middle = e.single && e.open_left && e.open_right;
+    if (!origin && !middle) return;
     const uint32_t tok = tok_s[e.end - 1];
     if (tok >= V) return;
-    // number of following chunks the run reaches into
-    uint32_t last = blockIdx.x + 1;
-    while (last < chunks) {
-        const ChunkEdges f = chunk_edges(tok_s, last, L, N);
-        if (!(f.single && f.open_right)) break;
-        ++last;
+    // Equal tokens are contiguous, but the order of distinct tokens is the
+    // sorter's business (the grouping sort orders by hash group first), so the
+    // searches below test "equals tok", galloping outwards from the chunk (most
+    // runs end in the next chunk) and then bisecting the bracket.
+    // First position after the run: smallest p > e.end with p == N or tok_s[p] != tok.
+    uint32_t lo = e.end + 1, hi = e.end + L < N ? e.end + L : N;
+    for (uint32_t span = L; hi < N && tok_s[hi] == tok;) {
+        lo = hi + 1;
+        span *= 2;
+        hi = span < N - hi ? hi + span : N;
     }
-    if (last >= chunks) last = chunks - 1;
-    for (uint32_t cv = threadIdx.x; cv < CV; cv += blockDim.x) {
+    while (lo < hi) {
+        const uint32_t mid = lo + (hi - lo) / 2;
+        if (tok_s[mid] == tok) lo = mid + 1; else hi = mid;
+    }
+    const uint32_t c1 = (lo - 1) / L;            // chunk holding the run's last position
+    uint32_t c0 = chunk;                         // chunk holding its first
+    if (middle) {
+        // first position of the run: smallest p < e.start with tok_s[p] == tok
+        hi = e.start - 1;                        // known to hold tok
+        lo = hi > L ? hi - L : 0;
+        for (uint32_t span = L; lo > 0 && tok_s[lo] == tok;) {
+            hi = lo;
+            span *= 2;
+            lo = lo > span ? lo - span : 0;
+        }
+        while (lo < hi) {
+            const uint32_t mid = lo + (hi - lo) / 2;
+            if (tok_s[mid] != tok) lo = mid + 1; else hi = mid;
+        }
+        c0 = lo / L;
+    }
+    const uint32_t count = c1 - c0;              // head partials live in chunks c0+1 .. c1
+    const float* tail = carry_tail + (uint64_t)c0 * C;
+    const float* heads = carry_head + (uint64_t)(c0 + 1) * C;
+
+    if (count <= (uint32_t)kFixLanes) {
+        if (!origin) return;
+        for (uint32_t cv = threadIdx.x; cv < CV; cv += blockDim.x) {
+            const uint32_t col = cv * VEC;
+            float sum[VEC], v[kFixLanes][VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) sum[k] = tail[col + k];
+#pragma unroll
+            for (int q = 0; q < kFixLanes; ++q)
+                if ((uint32_t)q < count) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) v[q][k] = heads[(uint64_t)q * C + col + k];
+                }
+#pragma unroll
+            for (int q = 0; q < kFixLanes; ++q)
+                if ((uint32_t)q < count) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) sum[k] = sum[k] + v[q][k];
+                }
+            store_grad_row<T, VEC>(dW, (uint64_t)tok * C + col, sum, accumulate != 0);
+        }
+        return;
+    }
+
+    const uint32_t slabs = (CV + kFixCols - 1) / kFixCols;
+    const uint32_t helpers = count - 1 < slabs ? count - 1 : slabs;   // middle chunks that take a slab
+    uint32_t slab_begin, slab_end;
+    if (origin) {
+        slab_begin = helpers; slab_end = slabs;
+    } else {
+        slab_begin = chunk - c0 - 1; slab_end = slab_begin + 1;
+        if (slab_begin >= helpers) return;
+    }
+    const uint32_t colv = threadIdx.x % kFixCols;
+    const uint32_t lane = threadIdx.x / kFixCols;
+    for (uint32_t slab = slab_begin; slab < slab_end; ++slab) {
+        const uint32_t cv = slab * kFixCols + colv;
+        const bool live = cv < CV;
         const uint32_t col = cv * VEC;
         float acc[VEC];
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) acc[k] = carry_tail[(uint64_t)blockIdx.x * C + col + k];
-        for (uint32_t c = blockIdx.x + 1; c <= last; ++c) {
+        for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
+        if (live) {
+            for (uint32_t q0 = lane; q0 < count; q0 += kFixLanes * kFixBatch) {
+                float v[kFixBatch][VEC];
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + carry_head[(uint64_t)c * C + col + k];
+                for (int b = 0; b < kFixBatch; ++b) {
+                    const uint32_t q = q0 + (uint32_t)b * kFixLanes;
+                    if (q < count) {
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) v[b][k] = heads[(uint64_t)q * C + col + k];
+                    }
+                }
+#pragma unroll
+                for (int b = 0; b < kFixBatch; ++b) {
+                    const uint32_t q = q0 + (uint32_t)b * kFixLanes;
+                    if (q < count) {
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + v[b][k];
+                    }
+                }
+            }
         }
-        store_grad_row<T, VEC>(dW, (uint64_t)tok * C + col, acc, accumulate != 0);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) part[lane][colv * VEC + k] = acc[k];
+        __syncthreads();
+        if (lane == 0 && live) {
+            float sum[VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) sum[k] = tail[col + k];
+#pragma unroll
+            for (int q = 0; q < kFixLanes; ++q)
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) sum[k] = sum[k] + part[q][colv * VEC + k];
+            store_grad_row<T, VEC>(dW, (uint64_t)tok * C + col, sum, accumulate != 0);
+        }
+        __syncthreads();
     }
 }
 
@@ -529,18 +642,18 @@ int embedding_bwd_typed(hipStream_t s, const EmbPlan& p, const int32_t* ids, con
     if (wide) {
         const uint32_t CV = C / WIDE;
         uint32_t block = ((CV + 63) / 64) * 64;
-        if (block > 256) block = 256;
+        if (block > 512) block = 512;
         hipLaunchKernelGGL((emb_segment_sum_kernel<T, WIDE>), dim3(p.chunks), dim3(block), 0, s, keys_out,
                            vals_out, dY, dW, head, tail, N, C, CV, V, p.L, acc);
-        hipLaunchKernelGGL((emb_carry_fix_kernel<T, WIDE>), dim3(p.chunks), dim3(block), 0, s, keys_out, dW,
-                           head, tail, N, C, CV, V, p.L, p.chunks, acc);
+        hipLaunchKernelGGL((emb_carry_fix_kernel<T, WIDE>), dim3(p.chunks), dim3(kFixCols * kFixLanes), 0, s,
+                           keys_out, dW, head, tail, N, C, CV, V, p.L, acc);
     } else {
         uint32_t block = ((C + 63) / 64) * 64;
         if (block > 256) block = 256;
         hipLaunchKernelGGL((emb_segment_sum_kernel<T, 1>), dim3(p.chunks), dim3(block), 0, s, keys_out,
                            vals_out, dY, dW, head, tail, N, C, C, V, p.L, acc);
-        hipLaunchKernelGGL((emb_carry_fix_kernel<T, 1>), dim3(p.chunks), dim3(block), 0, s, keys_out, dW,
-                           head, tail, N, C, C, V, p.L, p.chunks, acc);
+        hipLaunchKernelGGL((emb_carry_fix_kernel<T, 1>), dim3(p.chunks), dim3(kFixCols * kFixLanes), 0, s,
+                           keys_out, dW, head, tail, N, C, C, V, p.L, acc);
     }
     return check_hip(hipGetLastError(), "embedding backward launch");
 }

@@ -154,10 +154,15 @@ template <> __device__ __forceinline__ float round_through<bf16_t>(float v) {
 // ----------------------------------------------------------------------------
 // forward, register-resident row
 // ----------------------------------------------------------------------------
+// Workgroup size of the forward kernel when a row needs at most one wave: the
+// rows of a workgroup never talk to each other, so the smallest workgroup (one
+// wave) gives the dispatcher the most freedom.
+constexpr int kFwdGroupBlock = 64;
+
 template <typename T, int VEC, int NV, int TPR>
-__global__ void __launch_bounds__(TPR >= 128 ? TPR : 256)
+__global__ void __launch_bounds__(TPR >= 128 ? TPR : kFwdGroupBlock)
 norm_fwd_kernel(const NormFwdArgs<T> a) {
-    constexpr int BLOCK = TPR >= 128 ? TPR : 256;
+    constexpr int BLOCK = TPR >= 128 ? TPR : kFwdGroupBlock;
     constexpr int RPB = BLOCK / TPR;
     __shared__ float lds[3 * 2 * (TPR > kWave ? TPR / kWave : 1)];
 
@@ -649,7 +654,7 @@ NormPlan plan_norm(uint32_t C, int dtype, bool aligned, bool backward) {
             p.generic = false;
             p.tpr = t;
             p.nv = (int)nv;
-            p.rpb = t >= 128 ? 1 : 256 / t;
+            p.rpb = t >= 128 ? 1 : (backward ? 256 : kFwdGroupBlock) / t;
             return p;
         }
     }
@@ -666,7 +671,7 @@ uint32_t bwd_blocks(const NormPlan& p, uint64_t rows) {
 
 template <typename T, int VEC, int TPR>
 int fwd_pick_nv(hipStream_t s, const NormPlan& p, const NormFwdArgs<T>& a) {
-    constexpr int BLOCK = TPR >= 128 ? TPR : 256;
+    constexpr int BLOCK = TPR >= 128 ? TPR : kFwdGroupBlock;
     const uint32_t grid = (uint32_t)((a.rows + p.rpb - 1) / p.rpb);
     switch (p.nv) {
 #define AGRAD_CASE(N)                                                                  \
