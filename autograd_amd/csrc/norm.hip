@@ -661,12 +661,36 @@ NormPlan plan_norm(uint32_t C, int dtype, bool aligned, bool backward) {
     return p;
 }
 
-uint32_t bwd_blocks(const NormPlan& p, uint64_t rows) {
+// The backward kernel is a persistent grid: every workgroup walks rows with a
+// stride of the grid and leaves one partial dgamma/dbeta row.  Measured on
+// MI355X over the benchmark shapes: a grid larger than what the GPU holds at
+// once (`resident`, from the occupancy query -- register use differs a lot
+// between instantiations) loses to one round, because the stragglers of the
+// second round run on a mostly idle chip; and beyond 1024 workgroups more
+// waves only add loads in flight that the memory system does not need.
+constexpr uint32_t kMaxBwdBlocks = 1024;
+
+uint32_t bwd_blocks(const NormPlan& p, uint64_t rows, uint32_t resident) {
     const uint64_t want = (rows + p.rpb - 1) / p.rpb;
-    // more partial rows buy more rows in flight; worth it once there are many rows
     uint64_t cap = norm_bwd_max_blocks();
-    if (cap == 0) cap = rows >= 32768 ? 2048 : 1024;
+    if (cap == 0) cap = resident && resident < kMaxBwdBlocks ? resident : kMaxBwdBlocks;
     return (uint32_t)(want < cap ? (want ? want : 1) : cap);
+}
+
+uint32_t cu_count() {
+    static const uint32_t value = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess) return 0u;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0u;
+        return (uint32_t)(n > 0 ? n : 0);
+    }();
+    return value;
+}
+
+template <int TPR>
+inline size_t bwd_dyn_lds(const NormPlan& p, uint32_t C) {
+    constexpr int BLOCK = TPR >= 128 ? TPR : 256;
+    return p.rpb > 1 ? (size_t)(BLOCK / kWave - 1) * C * sizeof(float) : 0;
 }
 
 template <typename T, int VEC, int TPR>
@@ -690,7 +714,7 @@ int fwd_pick_nv(hipStream_t s, const NormPlan& p, const NormFwdArgs<T>& a) {
 template <typename T, int VEC, int TPR>
 int bwd_pick_nv(hipStream_t s, const NormPlan& p, const NormBwdArgs<T>& a, uint32_t grid) {
     constexpr int BLOCK = TPR >= 128 ? TPR : 256;
-    const size_t dyn = p.rpb > 1 ? (size_t)(BLOCK / kWave - 1) * a.C * sizeof(float) : 0;
+    const size_t dyn = bwd_dyn_lds<TPR>(p, a.C);
     switch (p.nv) {
 #define AGRAD_CASE(N)                                                                  \
     case N:                                                                            \
@@ -703,6 +727,45 @@ int bwd_pick_nv(hipStream_t s, const NormPlan& p, const NormBwdArgs<T>& a, uint3
 #undef AGRAD_CASE
     }
     return set_error(AGRAD_EINVAL, "norm backward: no kernel for nv=%d", p.nv);
+}
+
+// workgroups of the chosen backward instantiation the GPU holds at once (0: unknown)
+template <typename T, int VEC, int TPR>
+uint32_t bwd_resident_nv(const NormPlan& p, uint32_t C) {
+    constexpr int BLOCK = TPR >= 128 ? TPR : 256;
+    const size_t dyn = bwd_dyn_lds<TPR>(p, C);
+    int per_cu = 0;
+    switch (p.nv) {
+#define AGRAD_CASE(N)                                                                  \
+    case N:                                                                            \
+        if constexpr (N * VEC <= kMaxEPT) {                                            \
+            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, norm_bwd_kernel<T, VEC, N, TPR>, BLOCK, dyn) != hipSuccess) \
+                per_cu = 0;                                                            \
+        }                                                                              \
+        break;
+        AGRAD_CASE(1) AGRAD_CASE(2) AGRAD_CASE(3) AGRAD_CASE(4) AGRAD_CASE(5) AGRAD_CASE(6)
+#undef AGRAD_CASE
+    }
+    if (per_cu <= 0) { (void)hipGetLastError(); return 0; }
+    return (uint32_t)per_cu * cu_count();
+}
+
+template <typename T>
+uint32_t bwd_resident_typed(const NormPlan& p, uint32_t C) {
+    constexpr int VEC = WideVec<T>::value;
+    if (p.generic) return 0;
+    switch (p.tpr) {
+        case 16: return bwd_resident_nv<T, VEC, 16>(p, C);
+        case 32: return bwd_resident_nv<T, VEC, 32>(p, C);
+        case 64: return bwd_resident_nv<T, VEC, 64>(p, C);
+        case 128: return bwd_resident_nv<T, VEC, 128>(p, C);
+        case 256: return bwd_resident_nv<T, VEC, 256>(p, C);
+        default: return bwd_resident_nv<T, VEC, 1024>(p, C);
+    }
+}
+
+uint32_t bwd_resident(const NormPlan& p, uint32_t C, int dtype) {
+    return dtype == AGRAD_BF16 ? bwd_resident_typed<bf16_t>(p, C) : bwd_resident_typed<float>(p, C);
 }
 
 template <typename T>
@@ -754,9 +817,9 @@ uint64_t norm_bwd_workspace_bytes(uint64_t rows, uint32_t C, int dtype) {
     // sized for the larger of the vector and the scalar geometry
     NormPlan vecp = plan_norm(C, dtype, true, true);
     NormPlan genp{true, 256, 0, 1};
-    uint64_t blocks = bwd_blocks(genp, rows);
+    uint64_t blocks = bwd_blocks(genp, rows, 0);
     if (!vecp.generic) {
-        const uint64_t b = bwd_blocks(vecp, rows);
+        const uint64_t b = bwd_blocks(vecp, rows, bwd_resident(vecp, C, dtype));
         if (b > blocks) blocks = b;
     }
     return 2ull * blocks * C * sizeof(float);
@@ -803,7 +866,7 @@ int launch_norm_bwd(hipStream_t s, int kind, int dtype, const void* x, const voi
                          (!dx || aligned16(dx)) && (!dx2 || aligned16(dx2)) &&
                          (!gamma || aligned16(gamma));
     const NormPlan p = plan_norm(C, dtype, aligned, true);
-    const uint32_t grid = bwd_blocks(p, rows);
+    const uint32_t grid = bwd_blocks(p, rows, bwd_resident(p, C, dtype));
     const bool want_params = dgamma != nullptr || dbeta != nullptr;
     if (rows == 0) {
         // nothing to add: stored parameter grads become zero, accumulated ones stay
