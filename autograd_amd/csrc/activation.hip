@@ -80,6 +80,17 @@ __device__ __forceinline__ float sigmoid_ref(float g) {
     return 1.0f / h;
 }
 
+// The sigmoid by I/O type.  fp32 tensors get the reference's sequence (accurate
+// expf, IEEE division).  bf16 tensors round their result to 8 significant bits,
+// and at 2 bytes per element the accurate sequence (about 25 instructions) makes
+// the kernel instruction-bound rather than memory-bound; the hardware exp2 and
+// reciprocal (1 ulp each) are indistinguishable after the bf16 rounding.
+template <typename T> __device__ __forceinline__ float sigmoid_io(float g) { return sigmoid_ref(g); }
+template <> __device__ __forceinline__ float sigmoid_io<bf16_t>(float g) {
+    const float e = __builtin_amdgcn_exp2f(g * -1.44269504088896341f);   // exp(-g); overflows to +inf -> result 0
+    return __builtin_amdgcn_rcpf(1.0f + e);
+}
+
 // gu[rows, 2H] -> h[rows, H]; a "vector" is VEC consecutive columns of one row.
 template <typename T, int VEC, int UNROLL>
 __global__ void __launch_bounds__(kEwBlock)
@@ -106,7 +117,7 @@ swiglu_fwd_kernel(const T* __restrict__ gu, T* __restrict__ h, uint32_t H, uint3
             float o[VEC];
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
-                float t = sigmoid_ref(g[j][k]);
+                float t = sigmoid_io<T>(g[j][k]);
                 t = g[j][k] * t;
                 o[k] = t * u[j][k];
             }
@@ -143,7 +154,7 @@ swiglu_bwd_kernel(const T* gu, const T* __restrict__ dh, T* dgu, uint32_t H, uin
             float dg[VEC], du[VEC];
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
-                const float sg = sigmoid_ref(g[j][k]);
+                const float sg = sigmoid_io<T>(g[j][k]);
                 float t = 1.0f - sg;
                 t = t * g[j][k];
                 t = t + 1.0f;
