@@ -13,7 +13,9 @@ data already resident in HBM.  Prints ONE JSON line:
   tokens_per_s     B*T / step time
   per_op           every op and direction of the workload, timed on its own with
                    HIP events on the library's stream over rotating buffer sets
-                   (so the working set exceeds the 256 MB Infinity Cache)
+                   (so the working set exceeds the 256 MB Infinity Cache);
+                   copy_us / vs_copy compare with a plain copy kernel moving the
+                   same number of bytes the same way
   roofline         the dominant kernel of the step (largest share of time)
   cpu_baseline     the numpy restatement of the reference's CPU kernels, timed
                    on this host with the reference's protocol (2 warm-up + 5
@@ -310,11 +312,33 @@ def time_case(ctx, case, iters, exact=False):
     return case.us
 
 
+def time_copy_of(ctx, nbytes, iters, exact=False):
+    """What a plain 16-byte-per-lane copy kernel needs to move the same number of
+    bytes (half read, half written) over the same rotation of buffer sets: the
+    practical ceiling of this GPU for a stream of that size, launch ramp included."""
+    half = max(16, (nbytes // 2) // 16 * 16)
+    k = n_sets(nbytes)
+    bufs = [(ctx.empty((half,), np.uint8), ctx.empty((half,), np.uint8)) for _ in range(k)]
+    try:
+        case = Case("copy", "ref", 2 * half, k,
+                    lambda i: ctx.call("agrad_copy", vp(bufs[i][0]), vp(bufs[i][1]), half), "copy16_kernel")
+        return time_case(ctx, case, iters, exact)
+    finally:
+        ctx.synchronize()
+        for a, b in bufs:
+            a.free()
+            b.free()
+
+
 def case_row(case):
     gbps = case.nbytes / (case.us * 1e-6) / 1e9
-    return {"op": case.op, "dir": case.direction, "MB": round(case.nbytes / 1e6, 2), "us": round(case.us, 2),
-            "GBps": round(gbps, 1), "frac_hbm": round(gbps / HBM_PEAK_GBS, 4), "sets": case.nsets,
-            "kernel": case.kernel}
+    row = {"op": case.op, "dir": case.direction, "MB": round(case.nbytes / 1e6, 2), "us": round(case.us, 2),
+           "GBps": round(gbps, 1), "frac_hbm": round(gbps / HBM_PEAK_GBS, 4), "sets": case.nsets,
+           "kernel": case.kernel}
+    if getattr(case, "copy_us", None):
+        row["copy_us"] = round(case.copy_us, 2)          # same bytes through the plain copy kernel
+        row["vs_copy"] = round(case.copy_us / case.us, 3)
+    return row
 
 
 def run_config(ctx, cfg, iters):
@@ -323,9 +347,11 @@ def run_config(ctx, cfg, iters):
         cases = build_cases(ctx, cfg, pool)
         for case in cases:
             time_case(ctx, case, iters)
-        return [case_row(c) for c in cases]
     finally:
         pool.release()
+    for case in cases:
+        case.copy_us = time_copy_of(ctx, case.nbytes, iters)
+    return [case_row(c) for c in cases]
 
 
 def run_workload(ctx, cfg, steps, warmup, iters, exact=False):
@@ -349,9 +375,11 @@ def run_workload(ctx, cfg, steps, warmup, iters, exact=False):
         wall = time.perf_counter() - t0
         for case in cases:
             time_case(ctx, case, iters, exact)
-        return cases, step_bytes, wall
     finally:
         pool.release()
+    for case in cases:
+        case.copy_us = time_copy_of(ctx, case.nbytes, iters, exact)
+    return cases, step_bytes, wall
 
 
 # ---------------------------------------------------------------------------------
@@ -487,7 +515,8 @@ def main():
                      "achieved": round(dom_gbps, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(dom_gbps / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.index, {}).get(f"{dom.op} {dom.direction}"),
-                     "launch_us": round(dom.us, 2), "algorithmic_bytes": dom.nbytes},
+                     "launch_us": round(dom.us, 2), "algorithmic_bytes": dom.nbytes,
+                     "same_bytes_copy_us": round(dom.copy_us, 2) if getattr(dom, "copy_us", None) else None},
         "per_op": [case_row(c) for c in cases],
     }
     if not args.no_cpu:
