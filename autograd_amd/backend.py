@@ -499,6 +499,33 @@ class HipBackend(Backend):
             return bf16_bits_to_f32_array(raw).reshape(tensor.shape)
         return raw
 
+    def storage_to_host(self, storage):
+        """raw host copy of a storage (no dtype widening)"""
+        return self.ctx.copy_to_host(storage.ptr.buffer_id, storage.ptr.offset, list(storage.shape),
+                                     np.dtype(storage.dtype).name)
+
+    # -- optimizer (backend.py:5115-5140) ------------------------------------------------
+    def grad_norm_sq(self, g_storage, partial, numel):
+        """partial[i] = sum of squares of 256-element group i of the gradient"""
+        self._launch("grad_norm_sq", [g_storage, partial], _lo_hi(int(numel)) + [_dt(g_storage)])
+
+    def adamw_step(self, p_storage, g_storage, m_storage, v_storage, tmp_storage,
+                   lr, lr_t, b1, b2, eps, weight_decay, numel=None, decay_numel=None, grad_scale=1.0,
+                   lr_bc1=None, inv_sqrt_bc2=1.0):
+        """One AdamW step on a flat slab.  Scalars are rounded to fp32 the way
+        numpy rounds the Python floats of cpu_adamw_step (backend.py:2013-2038):
+        lr*weight_decay, 1.0-b1 and 1.0-b2 are formed in double first."""
+        if numel is None:
+            numel = prod(p_storage.shape)
+        if decay_numel is None:
+            decay_numel = numel if weight_decay != 0.0 else 0
+        lr_wd = float(lr) * float(weight_decay) if weight_decay > 0.0 else 0.0
+        step_lr = lr_t if lr_bc1 is None else lr_bc1
+        floats = [lr_wd, b1, 1.0 - b1, b2, 1.0 - b2, eps, step_lr, inv_sqrt_bc2, grad_scale]
+        self._launch("adamw_step", [p_storage, g_storage, m_storage, v_storage],
+                     [f32_bits(x) for x in floats] + _lo_hi(int(numel)) + _lo_hi(int(decay_numel))
+                     + [_dt(g_storage)])
+
     def begin_pass(self):
         self.ctx.begin_pass()
 

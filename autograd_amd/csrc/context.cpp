@@ -269,6 +269,24 @@ int h_pos_grad(const Call& c) {
     return launch_pos_embedding_bwd(c.ctx->stream, c.a[0], dY, dwpe, c.a[1], c.a[2], c.a[3], c.a[4]);
 }
 
+// buffers p, g, m, v | args (float bits) lr_wd, b1, 1-b1, b2, 1-b2, eps, step_lr, inv_sqrt_bc2, grad_scale,
+//                       then numel lo, hi, decay_numel lo, hi, grad dtype
+int h_adamw(const Call& c) {
+    NEED_DTYPE(c.a[13])
+    const uint64_t n = u64(c.a, 9), dn = u64(c.a, 11);
+    RESOLVE(0, n * 4, p) RESOLVE(1, n * dtype_size(c.a[13]), g) RESOLVE(2, n * 4, m) RESOLVE(3, n * 4, v)
+    return launch_adamw(c.ctx->stream, (int)c.a[13], (float*)p, g, (float*)m, (float*)v, n, dn, f32(c.a[0]),
+                        f32(c.a[1]), f32(c.a[2]), f32(c.a[3]), f32(c.a[4]), f32(c.a[5]), f32(c.a[6]),
+                        f32(c.a[7]), f32(c.a[8]));
+}
+// buffers g, partial | args numel lo, hi, dtype
+int h_grad_norm(const Call& c) {
+    NEED_DTYPE(c.a[2])
+    const uint64_t n = u64(c.a, 0);
+    RESOLVE(0, n * dtype_size(c.a[2]), g) RESOLVE(1, grad_norm_groups(n) * 4, partial)
+    return launch_grad_norm_sq(c.ctx->stream, (int)c.a[2], g, (float*)partial, n);
+}
+
 const Entry kTable[] = {
     {"fill_scalar_kernel", 1, 3, "out | bits, n_lo, n_hi", h_fill},
     {"fill_scalar_kernel2", 1, 4, "out | bits, itemsize, n_lo, n_hi", h_fill2},
@@ -292,6 +310,8 @@ const Entry kTable[] = {
     {"embedding_sum_forward", 4, 5, "ids, W, wpe, out | dtype, N, T, C, V", h_embed_sum_fwd},
     {"gather_backward_kernel", 4, 7, "ids, dY, dW, workspace | dtype, N, C, V, flags, ws_lo, ws_hi", h_gather_bwd},
     {"pos_emb_grad", 2, 5, "dY, dwpe | dtype, B, T, C, flags", h_pos_grad},
+    {"adamw_step", 4, 14, "p, g, m, v | lr_wd, b1, one_minus_b1, b2, one_minus_b2, eps, step_lr, inv_sqrt_bc2, grad_scale (float bits), n_lo, n_hi, decay_lo, decay_hi, grad_dtype", h_adamw},
+    {"grad_norm_sq", 2, 3, "g, partial | n_lo, n_hi, dtype", h_grad_norm},
 };
 constexpr int kTableSize = (int)(sizeof(kTable) / sizeof(kTable[0]));
 
@@ -574,6 +594,20 @@ int agrad_pos_embedding_backward(agrad_ctx* ctx, int dtype, const void* dY, void
                                  uint32_t T, uint32_t C, uint32_t flags) {
     CTX_OR_FAIL(ctx)
     return launch_pos_embedding_bwd(ctx->stream, dtype, dY, dwpe, B, T, C, flags);
+}
+
+int agrad_adamw_step(agrad_ctx* ctx, int grad_dtype, float* p, const void* g, float* m, float* v,
+                     uint64_t numel, uint64_t decay_numel, float lr_wd, float b1, float one_minus_b1,
+                     float b2, float one_minus_b2, float eps, float step_lr, float inv_sqrt_bc2,
+                     float grad_scale) {
+    CTX_OR_FAIL(ctx)
+    return launch_adamw(ctx->stream, grad_dtype, p, g, m, v, numel, decay_numel, lr_wd, b1, one_minus_b1, b2,
+                        one_minus_b2, eps, step_lr, inv_sqrt_bc2, grad_scale);
+}
+uint64_t agrad_grad_norm_groups(uint64_t numel) { return grad_norm_groups(numel); }
+int agrad_grad_norm_sq(agrad_ctx* ctx, int dtype, const void* g, float* partial, uint64_t numel) {
+    CTX_OR_FAIL(ctx)
+    return launch_grad_norm_sq(ctx->stream, dtype, g, partial, numel);
 }
 
 }  // extern "C"

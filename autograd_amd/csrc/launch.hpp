@@ -60,4 +60,11 @@ int launch_embedding_bwd(hipStream_t s, int dtype, const int32_t* ids, const voi
 int launch_pos_embedding_bwd(hipStream_t s, int dtype, const void* dY, void* dwpe, uint32_t B,
                              uint32_t T, uint32_t C, uint32_t flags);
 
+// optimizer.hip
+int launch_adamw(hipStream_t s, int grad_dtype, float* p, const void* g, float* m, float* v,
+                 uint64_t numel, uint64_t decay_numel, float lr_wd, float b1, float one_minus_b1,
+                 float b2, float one_minus_b2, float eps, float step_lr, float inv_sqrt_bc2, float grad_scale);
+uint64_t grad_norm_groups(uint64_t numel);
+int launch_grad_norm_sq(hipStream_t s, int dtype, const void* g, float* partial, uint64_t numel);
+
 }  // namespace agrad

@@ -135,7 +135,7 @@ def build_cases(ctx, cfg, pool):
     nbytes = op_bytes(cfg, distinct)
     cases = []
     # one builder per op family: each keeps its buffers in its own scope
-    for builder in (_embed_cases, _norm_cases, _act_cases, _rope_cases):
+    for builder in (_embed_cases, _norm_cases, _act_cases, _rope_cases, _opt_cases):
         cases += builder(ctx, cfg, pool, rng, nbytes, ids0)
     return cases
 
@@ -275,6 +275,37 @@ def _rope_cases(ctx, cfg, pool, rng, nbytes, ids0):
         cases.append(Case("rope", "fwd", nbytes["rope"][0], k, fwd, "rope_kernel"))
         cases.append(Case("rope", "bwd", nbytes["rope"][1], k, bwd, "rope_kernel"))
     return cases
+
+
+def _opt_cases(ctx, cfg, pool, rng, nbytes, ids0):
+    """AdamW over the embedding table's slab (the consumer of the gradients above)
+    and the gradient-norm partial sums; fp32 parameters and moments, gradients in
+    the configuration's I/O type.  Reported beside the step, not part of it."""
+    if not cfg.embed:
+        return []
+    n = cfg.V * cfg.C
+    gdt = capi.BF16 if cfg.dtype == "bf16" else capi.F32
+    per_elem = 24 + 2 * cfg.esize            # read p, m, v, g; write p, m, v
+    k = n_sets(per_elem * n)
+    sets = []
+    for _ in range(k):
+        sets.append((pool.normal(n, "f32"), pool.normal(n, cfg.dtype), pool.empty(n, "f32"), pool.empty(n, "f32")))
+        ctx.call("agrad_fill", sets[-1][2].ptr, 0, 0, 4, n)
+        ctx.call("agrad_fill", sets[-1][3].ptr, 0, 0, 4, n)
+    groups = ctx.lib.agrad_grad_norm_groups(n)
+    partial = pool.empty(groups, "f32")
+    lr, b1, b2 = 1e-3, 0.9, 0.999
+
+    def step(i):
+        p, g, m, v = sets[i]
+        ctx.call("agrad_adamw_step", gdt, vp(p), vp(g), vp(m), vp(v), n, n, lr * 0.01, b1, 1.0 - b1, b2, 1.0 - b2,
+                 1e-8, lr, 1.0, 1.0)
+
+    def norm(i):
+        ctx.call("agrad_grad_norm_sq", gdt, vp(sets[i][1]), vp(partial), n)
+
+    return [Case("adamw", "opt", per_elem * n, k, step, "adamw_vec_kernel"),
+            Case("grad_norm_sq", "opt", cfg.esize * n + 4 * groups, k, norm, "grad_norm_sq_kernel")]
 
 
 def spin_up(ctx, seconds=0.25):

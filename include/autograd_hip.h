@@ -188,6 +188,36 @@ int agrad_embedding_backward(agrad_ctx* ctx, int dtype, const int32_t* ids, cons
 int agrad_pos_embedding_backward(agrad_ctx* ctx, int dtype, const void* dY, void* dwpe,
                                  uint32_t B, uint32_t T, uint32_t C, uint32_t flags);
 
+/* ---- optimizer step over the parameter slab (the consumer of the gradients above) ---- */
+
+/* One AdamW step on numel fp32 parameters with fp32 moments, in place; the
+ * gradient is fp32 or bf16 (grad_dtype).  Per element, each operation rounded
+ * once, in the order of cpu_adamw_step (backend.py:2013-2038):
+ *     g *= grad_scale                               (skipped when grad_scale == 1)
+ *     p -= p * lr_wd                                (elements [0, decay_numel) only, and only if lr_wd != 0)
+ *     m  = m*b1 + g*one_minus_b1
+ *     v  = v*b2 + (g*g)*one_minus_b2
+ *     p -= (m / (sqrt(v)*inv_sqrt_bc2 + eps)) * step_lr      (the multiply is skipped when inv_sqrt_bc2 == 1)
+ * The reference's CPU path calls this with lr_wd = lr*weight_decay, step_lr =
+ * lr*sqrt(1-b2^t)/(1-b1^t), inv_sqrt_bc2 = grad_scale = 1 (optimizer.py:443-446,
+ * 488-498); its Metal path (Backend.adamw_step, backend.py:5122-5140; adamw_step,
+ * metal_ops.metal:10139-10228) with step_lr = lr/(1-b1^t), inv_sqrt_bc2 =
+ * 1/sqrt(1-b2^t), grad_scale = the clip coefficient and decay_numel = the
+ * matrix-shaped prefix of a merged slab (optimizer.py:97-140).
+ * one_minus_b1 / one_minus_b2 are separate arguments because the reference
+ * forms 1.0 - b in double precision before rounding to fp32. */
+int agrad_adamw_step(agrad_ctx* ctx, int grad_dtype, float* p, const void* g, float* m, float* v,
+                     uint64_t numel, uint64_t decay_numel, float lr_wd, float b1, float one_minus_b1,
+                     float b2, float one_minus_b2, float eps, float step_lr, float inv_sqrt_bc2,
+                     float grad_scale);
+
+/* partial[i] = sum of squares of g[256 i .. 256 i + 255] for i < agrad_grad_norm_groups(numel);
+ * the caller adds the partials in double precision and takes the square root
+ * (grad_norm_sq, metal_ops.metal:10103-10137; Backend.grad_norm_sq,
+ * backend.py:5115-5120; the host side of optimizer.py:579-600). */
+uint64_t agrad_grad_norm_groups(uint64_t numel);
+int agrad_grad_norm_sq(agrad_ctx* ctx, int dtype, const void* g, float* partial, uint64_t numel);
+
 #ifdef __cplusplus
 }
 #endif

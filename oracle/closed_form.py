@@ -130,3 +130,20 @@ def finite_diff(fn, x, idxs, eps=1e-3):
         flat[i] = orig
         out[j] = (plus - minus) / (2.0 * eps)
     return out
+
+
+def adamw_reference(p0, grads, lr, b1, b2, eps, weight_decay):
+    """Textbook AdamW in float64 (Loshchilov & Hutter, with the bias correction
+    folded into the step size the way the reference folds it, optimizer.py:445):
+    returns the parameters after len(grads) steps and the final moments."""
+    p = f64(p0).copy()
+    m = np.zeros_like(p)
+    v = np.zeros_like(p)
+    for t, g in enumerate(grads, start=1):
+        g = f64(g)
+        p = p * (1.0 - lr * weight_decay)
+        m = b1 * m + (1.0 - b1) * g
+        v = b2 * v + (1.0 - b2) * g * g
+        lr_t = lr * np.sqrt(1.0 - b2 ** t) / (1.0 - b1 ** t)
+        p = p - lr_t * m / (np.sqrt(v) + eps)
+    return p, m, v

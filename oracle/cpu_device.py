@@ -320,6 +320,32 @@ class CPUBackend(Backend):
             return K.bf16_bits_to_f32(d).reshape(tensor.shape).copy()
         return np.array(d, copy=True)
 
+    def storage_to_host(self, storage):
+        return np.array(storage.data, copy=True)
+
+    # CPUBackend.adamw_step (backend.py:2602-2605) with the keyword arguments of
+    # the Metal backend's (backend.py:5122-5124) so one optimizer drives both
+    def adamw_step(self, p_storage, g_storage, m_storage, v_storage, tmp_storage,
+                   lr, lr_t, b1, b2, eps, weight_decay, numel=None, decay_numel=None, grad_scale=1.0,
+                   lr_bc1=None, inv_sqrt_bc2=1.0):
+        g = g_storage.data
+        if g.dtype == np.uint16:
+            g = K.bf16_bits_to_f32(g).reshape(g.shape)
+        p, m, v = p_storage.data, m_storage.data, v_storage.data
+        n = p.size if numel is None else int(numel)
+        dn = (n if weight_decay != 0.0 else 0) if decay_numel is None else int(decay_numel)
+        if lr_bc1 is None and inv_sqrt_bc2 == 1.0 and grad_scale == 1.0 and dn in (0, n):
+            K.adamw_step(p, g, m, v, lr, lr_t, b1, b2, eps, weight_decay if dn else 0.0)
+        else:
+            K.adamw_step_split(p, g, m, v, lr * weight_decay if weight_decay > 0.0 else 0.0, b1, b2, eps,
+                               lr_t if lr_bc1 is None else lr_bc1, inv_sqrt_bc2, grad_scale, dn)
+
+    def grad_norm_sq(self, g_storage, partial, numel):
+        g = g_storage.data
+        if g.dtype == np.uint16:
+            g = K.bf16_bits_to_f32(g)
+        partial.data.reshape(-1)[:] = K.grad_norm_partials(g.reshape(-1)[:int(numel)]).astype(np.float32)
+
 
 def register():
     """make "cpu" available to Runtime(device="cpu")"""

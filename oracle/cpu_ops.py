@@ -17,6 +17,8 @@ Pinning (what shows these functions are the right functions; tests/test_oracle.p
     577-645 (restated in float64), finite differences, rotation invariants.
   * gather: numpy fancy indexing; backward: brute-force row loop.
   * bf16: bit-exact against an exhaustive integer restatement of utils.py:20-27.
+  * adamw: the textbook bias-corrected recurrence in float64 over several steps;
+    the first step from zero moments moves every weight by lr * sign(g).
 Parity unpinned by the reference:
   * relu2_* -- the reference has no ReLU^2; pinned by its closed form only.
   * d(gamma), d(beta) at large row counts -- numpy sums rows sequentially in
@@ -304,6 +306,69 @@ def rope_signed(q, k, cos, sin, rope_sign, backward=False):
                 else:
                     np.subtract(hi, r1, out=hi)
                 np.copyto(lo, r0)
+
+
+# --------------------------------------------------------------------------
+# AdamW  (cpu_adamw_step, backend.py:2013-2038; the step size lr_t comes from
+# optimizer.py:445)
+# --------------------------------------------------------------------------
+def adamw_step(p, g, m, v, lr, lr_t, b1, b2, eps, weight_decay):
+    """In place on p, m, v (fp32 arrays); g is read.  Python-float scalars meet
+    fp32 arrays, so each scalar is rounded to fp32 once and every numpy call
+    rounds its result once."""
+    tmp = np.empty_like(p)
+    if weight_decay > 0.0:
+        np.multiply(p, lr * weight_decay, out=tmp)
+        np.subtract(p, tmp, out=p)
+    np.multiply(m, b1, out=m)
+    np.multiply(g, 1.0 - b1, out=tmp)
+    np.add(m, tmp, out=m)
+    np.multiply(v, b2, out=v)
+    np.multiply(g, g, out=tmp)
+    np.multiply(tmp, 1.0 - b2, out=tmp)
+    np.add(v, tmp, out=v)
+    np.sqrt(v, out=tmp)
+    np.add(tmp, eps, out=tmp)
+    np.divide(m, tmp, out=tmp)
+    np.multiply(tmp, lr_t, out=tmp)
+    np.subtract(p, tmp, out=p)
+
+
+def adamw_step_split(p, g, m, v, lr_wd, b1, b2, eps, step_lr, inv_sqrt_bc2, grad_scale, decay_numel=None):
+    """The same sequence with the Metal kernel's extra factors (adamw_step,
+    metal_ops.metal:10139-10228): the gradient times grad_scale, sqrt(v) times
+    inv_sqrt_bc2 before eps, weight decay on the first decay_numel elements."""
+    g = np.multiply(g, F32(grad_scale)) if grad_scale != 1.0 else g
+    tmp = np.empty_like(p)
+    if lr_wd != 0.0:
+        n = p.size if decay_numel is None else decay_numel
+        flat = p.reshape(-1)
+        np.multiply(flat[:n], lr_wd, out=tmp.reshape(-1)[:n])
+        np.subtract(flat[:n], tmp.reshape(-1)[:n], out=flat[:n])
+    np.multiply(m, b1, out=m)
+    np.multiply(g, 1.0 - b1, out=tmp)
+    np.add(m, tmp, out=m)
+    np.multiply(v, b2, out=v)
+    np.multiply(g, g, out=tmp)
+    np.multiply(tmp, 1.0 - b2, out=tmp)
+    np.add(v, tmp, out=v)
+    np.sqrt(v, out=tmp)
+    if inv_sqrt_bc2 != 1.0:
+        np.multiply(tmp, inv_sqrt_bc2, out=tmp)
+    np.add(tmp, eps, out=tmp)
+    np.divide(m, tmp, out=tmp)
+    np.multiply(tmp, step_lr, out=tmp)
+    np.subtract(p, tmp, out=p)
+
+
+def grad_norm_partials(g):
+    """sum of squares of every 256-element group of g (grad_norm_sq,
+    metal_ops.metal:10103-10137), in float64 so that it checks any fp32 order"""
+    flat = np.asarray(g, dtype=np.float64).reshape(-1)
+    pad = (-flat.size) % 256
+    if pad:
+        flat = np.concatenate([flat, np.zeros(pad)])
+    return (flat * flat).reshape(-1, 256).sum(1)
 
 
 # --------------------------------------------------------------------------

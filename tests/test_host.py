@@ -36,7 +36,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_library_reports_errors_without_gpu_or_kernel():
     lib = capi.load_library()
-    assert lib.agrad_kernel_count() == 22
+    assert lib.agrad_kernel_count() == 24
     names = [lib.agrad_kernel_name(i).decode() for i in range(lib.agrad_kernel_count())]
     for n in ("layernorm_forward", "layernorm_backward_kernel", "rmsnorm_forward", "rmsnorm_backward",
               "gelu_forward_kernel", "gelu_backward_kernel", "swiglu_forward_kernel", "rope_qk_inplace",
@@ -214,3 +214,45 @@ def test_runtime_rejects_ops_without_kernels():
     y = Bare()(x)
     with pytest.raises(RuntimeError):
         Runtime(device="cpu").build_topo(y)      # lookup is by exact type (backend.py:4938-4950)
+
+
+def test_adamw_host_logic_on_oracle_device():
+    """AdamW over a runtime on the oracle device: per-parameter dispatches, decay on
+    matrices only, step-size bookkeeping, clip coefficient (optimizer.py:443-500)."""
+    import math
+    from autograd_amd.optimizer import AdamW
+    from oracle import cpu_ops as K
+    rng = np.random.default_rng(5)
+    B, Tn, C, V = 2, 6, 16, 23
+    ids = T((B, Tn), np.int32, False, rng.integers(0, V, (B, Tn), dtype=np.int32))
+    w = T((V, C), val=rng.standard_normal((V, C)).astype(np.float32))
+    g = T((C,), val=np.ones(C, np.float32))
+    b = T((C,), val=np.zeros(C, np.float32))
+    out = ids.gather(w).layer_norm(g, b).gelu()
+    rt = Runtime(device="cpu")
+    rt.backward(out, grad_scale=1.0)
+    with pytest.raises(ValueError):
+        AdamW([w], state_mode="4bit", runtime=rt)
+    with pytest.raises(NotImplementedError):
+        AdamW([w], state_mode="8bit", runtime=rt)
+    lr, betas, eps, wd = 1e-2, (0.9, 0.95), 1e-8, 0.1
+    opt = AdamW([w, g, b, ids], lr=lr, betas=betas, eps=eps, weight_decay=wd, runtime=rt)
+    assert len(opt.params) == 3                       # ids needs no gradient
+    assert [d[5] for d in opt.dispatches] == [V * C, 0, 0]
+    clip = opt.build_grad_clip()
+    want = {k: rt.backend.copy_to_host(t) for k, t in (("w", w), ("g", g), ("b", b))}
+    mom = {k: (np.zeros_like(a), np.zeros_like(a)) for k, a in want.items()}
+    for t in range(1, 3):
+        rt.backward(out, grad_scale=1.0)
+        grads = {k: rt.backend.copy_to_host(p.grad) for k, p in (("w", w), ("g", g), ("b", b))}
+        norm, coef = clip(0.5)
+        total = math.sqrt(sum(float((a.astype(np.float64) ** 2).sum()) for a in grads.values()))
+        assert norm == pytest.approx(total, rel=1e-6) and coef == pytest.approx(min(1.0, 0.5 / (total + 1e-6)))
+        opt.step()
+        lr_t = lr * math.sqrt(1 - betas[1] ** t) / (1 - betas[0] ** t)
+        for k, p in (("w", w), ("g", g), ("b", b)):
+            K.adamw_step(want[k], grads[k], *mom[k], lr, lr_t, betas[0], betas[1], eps, wd if p.ndim > 1 else 0.0)
+            np.testing.assert_array_equal(rt.backend.copy_to_host(p), want[k])
+    assert opt.t == 2
+    opt.zero_grad()
+    assert not rt.backend.copy_to_host(w.grad).any()

@@ -336,3 +336,80 @@ def test_bf16_rounding_rule():
     assert np.array_equal(utils.f32_array_to_bf16_bits(sample.view(np.float32)), want)
     assert all(utils.bf16_bits(float(np.uint32(b).view(np.float32))) == w
                for b, w in cases.items() if not np.isnan(np.uint32(b).view(np.float32)))
+
+
+# ---------------------------------------------------------------------------
+# AdamW (cpu_adamw_step, backend.py:2013-2038)
+# ---------------------------------------------------------------------------
+def _adam_case(k, n=513):
+    r = rng(k)
+    p = r.standard_normal(n).astype(np.float32)
+    grads = [r.standard_normal(n).astype(np.float32) for _ in range(5)]
+    return p, grads
+
+
+def test_adamw_first_step_is_lr_times_sign_and_matches_textbook():
+    import math
+    lr, b1, b2, eps, wd = 1e-3, 0.9, 0.999, 1e-8, 0.0
+    p0, grads = _adam_case(40)
+    p, m, v = p0.copy(), np.zeros_like(p0), np.zeros_like(p0)
+    lr_t = lr * math.sqrt(1.0 - b2) / (1.0 - b1)
+    K.adamw_step(p, grads[0], m, v, lr, lr_t, b1, b2, eps, wd)
+    # from zero moments the first Adam step is lr * sign(g) (eps only matters for |g| ~ 1e-8)
+    big = np.abs(grads[0]) > 1e-3
+    assert np.abs((p0 - p)[big] - lr * np.sign(grads[0])[big]).max() < 2e-7
+    # several steps, with weight decay, against the float64 recurrence
+    wd = 0.1
+    p, m, v = p0.copy(), np.zeros_like(p0), np.zeros_like(p0)
+    for t, g in enumerate(grads, start=1):
+        lr_t = lr * math.sqrt(1.0 - b2 ** t) / (1.0 - b1 ** t)
+        K.adamw_step(p, g, m, v, lr, lr_t, b1, b2, eps, wd)
+    p64, m64, v64 = cf.adamw_reference(p0, grads, lr, b1, b2, eps, wd)
+    close(p, p64)
+    close(m, m64, 1e-5, 1e-7)
+    close(v, v64, 1e-5, 1e-7)
+    # decoupled decay: with zero gradients only the (1 - lr*wd)^t shrink remains
+    p, m, v = p0.copy(), np.zeros_like(p0), np.zeros_like(p0)
+    zero = np.zeros_like(p0)
+    for t in range(1, 4):
+        K.adamw_step(p, zero, m, v, lr, lr, b1, b2, eps, wd)
+    close(p, p0.astype(np.float64) * (1 - lr * wd) ** 3)
+    assert not m.any() and not v.any()
+
+
+def test_adamw_split_form_is_the_same_update():
+    import math
+    lr, b1, b2, eps, wd = 3e-4, 0.9, 0.95, 1e-8, 0.05
+    p0, grads = _adam_case(41)
+    a = [p0.copy(), np.zeros_like(p0), np.zeros_like(p0)]
+    b = [p0.copy(), np.zeros_like(p0), np.zeros_like(p0)]
+    c = [p0.copy(), np.zeros_like(p0), np.zeros_like(p0)]
+    for t, g in enumerate(grads, start=1):
+        lr_t = lr * math.sqrt(1.0 - b2 ** t) / (1.0 - b1 ** t)
+        K.adamw_step(a[0], g, a[1], a[2], lr, lr_t, b1, b2, eps, wd)
+        # neutral extra factors: the very same bits
+        K.adamw_step_split(b[0], g, b[1], b[2], lr * wd, b1, b2, eps, lr_t, 1.0, 1.0)
+        # the Metal path's split of the bias correction differs only in where eps sits
+        K.adamw_step_split(c[0], g, c[1], c[2], lr * wd, b1, b2, eps, lr / (1.0 - b1 ** t),
+                             1.0 / math.sqrt(1.0 - b2 ** t), 1.0)
+    for x, y in zip(a, b):
+        np.testing.assert_array_equal(x, y)
+    close(c[0], a[0], 1e-5, 1e-6)
+    # clipping by grad_scale is scaling the gradient; decay_numel limits the decay to a prefix
+    g = grads[0]
+    d = [p0.copy(), np.zeros_like(p0), np.zeros_like(p0)]
+    e = [p0.copy(), np.zeros_like(p0), np.zeros_like(p0)]
+    K.adamw_step_split(d[0], g, d[1], d[2], lr * wd, b1, b2, eps, lr, 1.0, 0.25, decay_numel=100)
+    K.adamw_step_split(e[0][:100], g[:100] * np.float32(0.25), e[1][:100], e[2][:100], lr * wd, b1, b2, eps, lr, 1.0, 1.0)
+    K.adamw_step_split(e[0][100:], g[100:] * np.float32(0.25), e[1][100:], e[2][100:], 0.0, b1, b2, eps, lr, 1.0, 1.0)
+    for x, y in zip(d, e):
+        np.testing.assert_array_equal(x, y)
+
+
+def test_grad_norm_partials():
+    r = rng(42)
+    g = r.standard_normal(1000).astype(np.float32)
+    part = K.grad_norm_partials(g)
+    assert part.shape == (4,)
+    assert abs(part.sum() - float(np.dot(g.astype(np.float64), g.astype(np.float64)))) < 1e-9
+    assert abs(part[3] - float((g[768:].astype(np.float64) ** 2).sum())) < 1e-12
