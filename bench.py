@@ -51,7 +51,7 @@ HBM_PEAK_GBS = 8000.0
 # reads for the 64 MiB copy of spin_up(); the run and its numbers are recorded in
 # profiles/hbm_traffic_*.txt.  Keyed by config index, then "op direction".
 MEASURED_TRAFFIC_BYTES = {
-    1: {"relu2 bwd": 301.95e6},
+    1: {"relu2 bwd": 301.97e6},
 }
 ROTATE_BYTES = 768 << 20      # cycle at least this much distinct memory per op
 MAX_SETS = 8
@@ -285,7 +285,7 @@ def _opt_cases(ctx, cfg, pool, rng, nbytes, ids0):
         return []
     n = cfg.V * cfg.C
     gdt = capi.BF16 if cfg.dtype == "bf16" else capi.F32
-    per_elem = 24 + 2 * cfg.esize            # read p, m, v, g; write p, m, v
+    per_elem = 24 + cfg.esize                # read p, m, v (12) and g; write p, m, v (12)
     k = n_sets(per_elem * n)
     sets = []
     for _ in range(k):
