@@ -29,8 +29,8 @@ from math import prod
 
 import numpy as np
 
-from .op import (AddLayerNormOp, AddOp, AddRMSNormOp, EmbeddingSumOp, GatherOp, GELUOp, LayerNormOp,
-                 ReLUSquaredOp, RMSNormOp, RopeOp, SwiGLUOp)
+from .op import (AddLayerNormOp, AddOp, AddRMSNormOp, CrossEntropyLossOp, EmbeddingSumOp, GatherOp, GELUOp,
+                 LayerNormOp, ReLUSquaredOp, RMSNormOp, RopeOp, SwiGLUOp)
 from .scratch import single_slot
 from .utils import (bf16_bits, bf16_bits_to_f32_array, f32_array_to_bf16_bits, f32_bits, is_bf16,
                     xavier_uniform)
@@ -149,6 +149,7 @@ class HipBackend(Backend):
             AddLayerNormOp: self.hip_add_norm_forward,
             AddRMSNormOp: self.hip_add_norm_forward,
             RopeOp: self.hip_rope_forward,
+            CrossEntropyLossOp: self.hip_cross_entropy_forward,
         }
         self.backward_kernels = {
             AddOp: self.hip_add_backward,
@@ -162,6 +163,7 @@ class HipBackend(Backend):
             AddLayerNormOp: self.hip_add_norm_backward,
             AddRMSNormOp: self.hip_add_norm_backward,
             RopeOp: self.hip_rope_backward,
+            CrossEntropyLossOp: self.hip_cross_entropy_backward,
         }
 
     # -- lookup (backend.py:4938-4950) -------------------------------------------
@@ -453,6 +455,24 @@ class HipBackend(Backend):
             if g is not None and src.grad is not None and not self._same_memory(src.grad, g):
                 self._launch("add_residual_backward", [g, src.grad],
                              [_dt(src), self._grad_flag(node, src)] + _lo_hi(src.numel))
+
+    # -- cross-entropy (backend.py:489-524) -----------------------------------------------
+    def hip_cross_entropy_forward(self, inputs, outputs, scratch=None):
+        logits, labels = inputs
+        loss, lse = outputs
+        rows, V = prod(logits.shape[:-1]), logits.shape[-1]
+        self._launch("cross_entropy_forward", [logits, labels, loss, lse],
+                     [_dt(logits)] + _lo_hi(rows) + [V, _mask(logits, labels, loss, lse)])
+
+    def hip_cross_entropy_backward(self, inputs, outputs, scratch=None):
+        logits, labels = inputs
+        loss, lse = outputs
+        if loss.grad is None or not logits.requires_grad or logits.grad is None:
+            return
+        rows, V = prod(logits.shape[:-1]), logits.shape[-1]
+        self._launch("cross_entropy_backward", [logits, labels, loss.grad, lse, logits.grad],
+                     [_dt(logits)] + _lo_hi(rows) + [V, self._grad_flag(loss.op, logits),
+                                                    _mask(logits, labels, loss.grad, lse, logits.grad)])
 
     # -- fills and copies (backend.py:5069-5113) ---------------------------------------
     def fill_storage(self, storage, value):

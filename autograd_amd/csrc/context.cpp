@@ -269,6 +269,28 @@ int h_pos_grad(const Call& c) {
     return launch_pos_embedding_bwd(c.ctx->stream, c.a[0], dY, dwpe, c.a[1], c.a[2], c.a[3], c.a[4]);
 }
 
+// buffers logits, labels, loss, lse | args dtype, rows lo, hi, V, present_mask
+int h_ce_fwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t rows = u64(c.a, 1);
+    const uint32_t V = c.a[3], mask = c.a[4];
+    RESOLVE(0, rows * V * dtype_size(c.a[0]), logits) RESOLVE(1, rows * 4, labels) RESOLVE(2, rows * 4, loss)
+    RESOLVE_IF(mask & 8u, 3, rows * 4, lse)
+    return launch_ce_fwd(c.ctx->stream, (int)c.a[0], logits, (const int32_t*)labels, (float*)loss, (float*)lse,
+                         rows, V, c.ctx->err_flag);
+}
+// buffers logits, labels, dloss, lse, dlogits | args dtype, rows lo, hi, V, flags, present_mask
+int h_ce_bwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t rows = u64(c.a, 1);
+    const uint32_t V = c.a[3], mask = c.a[5];
+    const uint64_t bytes = rows * V * dtype_size(c.a[0]);
+    RESOLVE(0, bytes, logits) RESOLVE(1, rows * 4, labels) RESOLVE(2, rows * 4, dloss)
+    RESOLVE_IF(mask & 8u, 3, rows * 4, lse)
+    RESOLVE(4, bytes, dlogits)
+    return launch_ce_bwd(c.ctx->stream, (int)c.a[0], logits, (const int32_t*)labels, (const float*)dloss,
+                         (const float*)lse, dlogits, rows, V, c.a[4], c.ctx->err_flag);
+}
 // buffers p, g, m, v | args (float bits) lr_wd, b1, 1-b1, b2, 1-b2, eps, step_lr, inv_sqrt_bc2, grad_scale,
 //                       then numel lo, hi, decay_numel lo, hi, grad dtype
 int h_adamw(const Call& c) {
@@ -310,6 +332,8 @@ const Entry kTable[] = {
     {"embedding_sum_forward", 4, 5, "ids, W, wpe, out | dtype, N, T, C, V", h_embed_sum_fwd},
     {"gather_backward_kernel", 4, 7, "ids, dY, dW, workspace | dtype, N, C, V, flags, ws_lo, ws_hi", h_gather_bwd},
     {"pos_emb_grad", 2, 5, "dY, dwpe | dtype, B, T, C, flags", h_pos_grad},
+    {"cross_entropy_forward", 4, 5, "logits, labels, loss, lse | dtype, rows_lo, rows_hi, V, present_mask", h_ce_fwd},
+    {"cross_entropy_backward", 5, 6, "logits, labels, dloss, lse, dlogits | dtype, rows_lo, rows_hi, V, flags, present_mask", h_ce_bwd},
     {"adamw_step", 4, 14, "p, g, m, v | lr_wd, b1, one_minus_b1, b2, one_minus_b2, eps, step_lr, inv_sqrt_bc2, grad_scale (float bits), n_lo, n_hi, decay_lo, decay_hi, grad_dtype", h_adamw},
     {"grad_norm_sq", 2, 3, "g, partial | n_lo, n_hi, dtype", h_grad_norm},
 };
@@ -594,6 +618,18 @@ int agrad_pos_embedding_backward(agrad_ctx* ctx, int dtype, const void* dY, void
                                  uint32_t T, uint32_t C, uint32_t flags) {
     CTX_OR_FAIL(ctx)
     return launch_pos_embedding_bwd(ctx->stream, dtype, dY, dwpe, B, T, C, flags);
+}
+
+int agrad_cross_entropy_forward(agrad_ctx* ctx, int dtype, const void* logits, const int32_t* labels,
+                                float* loss, float* lse_out, uint64_t rows, uint32_t V) {
+    CTX_OR_FAIL(ctx)
+    return launch_ce_fwd(ctx->stream, dtype, logits, labels, loss, lse_out, rows, V, ctx->err_flag);
+}
+int agrad_cross_entropy_backward(agrad_ctx* ctx, int dtype, const void* logits, const int32_t* labels,
+                                 const float* dloss, const float* lse, void* dlogits,
+                                 uint64_t rows, uint32_t V, uint32_t flags) {
+    CTX_OR_FAIL(ctx)
+    return launch_ce_bwd(ctx->stream, dtype, logits, labels, dloss, lse, dlogits, rows, V, flags, ctx->err_flag);
 }
 
 int agrad_adamw_step(agrad_ctx* ctx, int grad_dtype, float* p, const void* g, float* m, float* v,

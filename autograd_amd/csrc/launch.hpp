@@ -67,4 +67,10 @@ int launch_adamw(hipStream_t s, int grad_dtype, float* p, const void* g, float* 
 uint64_t grad_norm_groups(uint64_t numel);
 int launch_grad_norm_sq(hipStream_t s, int dtype, const void* g, float* partial, uint64_t numel);
 
+// loss.hip
+int launch_ce_fwd(hipStream_t s, int dtype, const void* logits, const int32_t* labels, float* loss,
+                  float* lse_out, uint64_t rows, uint32_t V, int* err_flag);
+int launch_ce_bwd(hipStream_t s, int dtype, const void* logits, const int32_t* labels, const float* dloss,
+                  const float* lse, void* dlogits, uint64_t rows, uint32_t V, uint32_t flags, int* err_flag);
+
 }  // namespace agrad

@@ -1,0 +1,373 @@
+// Cross-entropy over the last axis of logits[rows, V] with integer labels.
+//
+//   forward   loss[r] = -((x[r, label] - max_r) - log(sum_v exp(x[r, v] - max_r)))
+//             (cpu_crossentropy_forward, backend.py:489-503) and, optionally,
+//             lse[r] = max_r + log(sum) for the backward pass;
+//   backward  dlogits[r, v] (+)= (softmax(x[r, :])[v] - [v == label]) * dloss[r]
+//             (cpu_crossentropy_backward, backend.py:505-524).
+//
+// Both are streams over [rows, V]: forward reads the logits once (running
+// maximum and rescaled sum, so no second pass), backward reads them once and
+// writes the gradient once when the forward pass left lse (otherwise it first
+// recomputes it with a second read of the row, which the caches serve).
+// One workgroup per row; a lane keeps kCeUnroll 16-byte vectors in flight.
+// Rows of odd length (V = 50257) start at any element alignment, so each row is
+// split into an element-wise head up to the next 16-byte boundary, a vector
+// body and an element-wise tail.
+//
+// exp: fp32 logits use expf; bf16 logits use the hardware exp2 (the result is
+// rounded to 8 bits anyway and the accurate sequence would make the bf16
+// kernels instruction-bound).  loss, lse and dloss are fp32 for both.
+#include "common.hpp"
+#include "launch.hpp"
+
+#include <cmath>
+
+namespace agrad {
+
+namespace {
+
+constexpr int kCeBlock = 256;
+constexpr int kCeUnroll = 4;      // forward (read-only): vectors a lane keeps in flight
+#ifndef AGRAD_CE_BWD_UNROLL
+#define AGRAD_CE_BWD_UNROLL 2
+#endif
+constexpr int kCeBwdUnroll = AGRAD_CE_BWD_UNROLL;   // backward (read + write)
+constexpr float kLog2e = 1.44269504088896341f;
+
+template <typename T> __device__ __forceinline__ float exp_io(float x) { return expf(x); }
+template <> __device__ __forceinline__ float exp_io<bf16_t>(float x) { return __builtin_amdgcn_exp2f(x * kLog2e); }
+
+// running (maximum, sum of exp(x - maximum))
+struct MaxSum {
+    float m, s;
+};
+
+template <typename T>
+__device__ __forceinline__ void absorb(MaxSum& a, float x) {
+    if (x > a.m) {
+        a.s = a.s * exp_io<T>(a.m - x) + 1.0f;   // exp(-inf) = 0 on the first element
+        a.m = x;
+    } else if (a.m > -INFINITY) {                // (-inf) - (-inf) would poison the sum
+        a.s = a.s + exp_io<T>(x - a.m);
+    }
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void absorb_vec(MaxSum& a, const float (&v)[VEC]) {
+    float vm = v[0];
+#pragma unroll
+    for (int k = 1; k < VEC; ++k) vm = fmaxf(vm, v[k]);
+    if (vm > a.m) {
+        a.s = a.s * exp_io<T>(a.m - vm);
+        a.m = vm;
+    }
+    if (a.m > -INFINITY) {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) a.s = a.s + exp_io<T>(v[k] - a.m);
+    }
+}
+
+template <typename T>
+__device__ __forceinline__ MaxSum merge(const MaxSum& a, const MaxSum& b) {
+    MaxSum r;
+    r.m = fmaxf(a.m, b.m);
+    if (r.m == -INFINITY) { r.s = 0.0f; return r; }
+    r.s = a.s * exp_io<T>(a.m - r.m) + b.s * exp_io<T>(b.m - r.m);
+    return r;
+}
+
+// how a row of V elements starting at `base` splits into head / vectors / tail
+template <typename T, int VEC>
+struct RowSplit {
+    uint32_t head, nvec, tail_start;
+    __device__ __forceinline__ RowSplit(const T* base, uint32_t V) {
+        if constexpr (VEC == 1) {
+            head = 0; nvec = V; tail_start = V;
+        } else {
+            const uint32_t mis = (uint32_t)(reinterpret_cast<uintptr_t>(base) & 15u) / (uint32_t)sizeof(T);
+            head = mis ? (uint32_t)(16 / sizeof(T)) - mis : 0;
+            if (head > V) head = V;
+            nvec = (V - head) / VEC;
+            tail_start = head + nvec * VEC;
+        }
+    }
+};
+
+// (max, sum) of one row, identical in every thread of the workgroup on return
+template <typename T, int VEC>
+__device__ __forceinline__ MaxSum row_max_sum(const T* base, uint32_t V, MaxSum* lds) {
+    const RowSplit<T, VEC> sp(base, V);
+    MaxSum acc{-INFINITY, 0.0f};
+    if constexpr (VEC > 1) {
+        // head and tail elements, one per thread (fewer than 2 * VEC of them)
+        const uint32_t extra = sp.head + (V - sp.tail_start);
+        if (threadIdx.x < extra) {
+            const uint32_t e = threadIdx.x < sp.head ? threadIdx.x : sp.tail_start + (threadIdx.x - sp.head);
+            float x[1];
+            VecIO<T, 1>::load(base + e, x);
+            absorb<T>(acc, x[0]);
+        }
+    }
+    const T* body = base + sp.head;
+    for (uint32_t i0 = threadIdx.x; i0 < sp.nvec; i0 += kCeBlock * kCeUnroll) {
+        float v[kCeUnroll][VEC];
+#pragma unroll
+        for (int u = 0; u < kCeUnroll; ++u) {
+            const uint32_t i = i0 + u * kCeBlock;
+            if (i < sp.nvec) VecIO<T, VEC>::load(body + (uint64_t)i * VEC, v[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < kCeUnroll; ++u) {
+            const uint32_t i = i0 + u * kCeBlock;
+            if (i < sp.nvec) absorb_vec<T, VEC>(acc, v[u]);
+        }
+    }
+    // lanes of a wave, then the waves through LDS; the order is fixed
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        MaxSum o{__shfl_xor(acc.m, off), __shfl_xor(acc.s, off)};
+        acc = merge<T>(acc, o);
+    }
+    const int wave = threadIdx.x / kWave;
+    if (threadIdx.x % kWave == 0) lds[wave] = acc;
+    __syncthreads();
+    MaxSum total = lds[0];
+#pragma unroll
+    for (int w = 1; w < kCeBlock / kWave; ++w) total = merge<T>(total, lds[w]);
+    __syncthreads();
+    return total;
+}
+
+template <typename T, int VEC>
+__global__ void __launch_bounds__(kCeBlock)
+ce_fwd_kernel(const T* __restrict__ x, const int32_t* __restrict__ labels, float* __restrict__ loss,
+              float* __restrict__ lse_out, uint32_t V, int* err_flag) {
+    __shared__ MaxSum lds[kCeBlock / kWave];
+    const uint64_t row = blockIdx.x;
+    const T* base = x + row * V;
+    const MaxSum t = row_max_sum<T, VEC>(base, V, lds);
+    if (threadIdx.x == 0) {
+        const float lg = logf(t.s);
+        if (lse_out != nullptr) lse_out[row] = t.m + lg;
+        const int32_t label = labels[row];
+        if (label < 0 || (uint32_t)label >= V) {
+            *err_flag = 1;
+            loss[row] = 0.0f;
+        } else {
+            float xl[1];
+            VecIO<T, 1>::load(base + label, xl);
+            float f = xl[0] - t.m;
+            f = f - lg;
+            loss[row] = -f;
+        }
+    }
+}
+
+template <typename T, int VEC>
+__device__ __forceinline__ void ce_grad_elems(const float (&xv)[VEC], float (&d)[VEC], float lse, float gl,
+                                              uint32_t first_elem, uint32_t label) {
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+        float p = exp_io<T>(xv[k] - lse);
+        if (first_elem + k == label) p = p - 1.0f;
+        d[k] = p * gl;
+    }
+}
+
+template <typename T, int VEC>
+__global__ void __launch_bounds__(kCeBlock)
+ce_bwd_kernel(const T* __restrict__ x, const int32_t* __restrict__ labels, const float* __restrict__ dloss,
+              const float* __restrict__ lse_in, T* dx, uint32_t V, int accumulate, int* err_flag) {
+    __shared__ MaxSum lds[kCeBlock / kWave];
+    const uint64_t row = blockIdx.x;
+    const T* base = x + row * V;
+    T* out = dx + row * V;
+    float lse;
+    if (lse_in != nullptr) {
+        lse = lse_in[row];
+    } else {
+        const MaxSum t = row_max_sum<T, VEC>(base, V, lds);
+        lse = t.m + logf(t.s);
+    }
+    const float gl = dloss[row];
+    const int32_t lab = labels[row];
+    uint32_t label = 0xffffffffu;          // matches no element: the row gets softmax * dloss
+    if (lab < 0 || (uint32_t)lab >= V) {
+        if (threadIdx.x == 0) *err_flag = 1;
+    } else {
+        label = (uint32_t)lab;
+    }
+    const RowSplit<T, VEC> sp(base, V);
+    if constexpr (VEC > 1) {
+        const uint32_t extra = sp.head + (V - sp.tail_start);
+        if (threadIdx.x < extra) {
+            const uint32_t e = threadIdx.x < sp.head ? threadIdx.x : sp.tail_start + (threadIdx.x - sp.head);
+            float xv[1], d[1];
+            VecIO<T, 1>::load(base + e, xv);
+            ce_grad_elems<T, 1>(xv, d, lse, gl, e, label);
+            if (accumulate) {
+                float old[1];
+                VecIO<T, 1>::load(out + e, old);
+                d[0] = old[0] + d[0];
+            }
+            VecIO<T, 1>::store(out + e, d);
+        }
+    }
+    const T* body = base + sp.head;
+    T* obody = out + sp.head;
+    for (uint32_t i0 = threadIdx.x; i0 < sp.nvec; i0 += kCeBlock * kCeBwdUnroll) {
+        float v[kCeBwdUnroll][VEC], old[kCeBwdUnroll][VEC];
+#pragma unroll
+        for (int u = 0; u < kCeBwdUnroll; ++u) {
+            const uint32_t i = i0 + u * kCeBlock;
+            if (i < sp.nvec) {
+                VecIO<T, VEC>::load(body + (uint64_t)i * VEC, v[u]);
+                if (accumulate) VecIO<T, VEC>::load(obody + (uint64_t)i * VEC, old[u]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kCeBwdUnroll; ++u) {
+            const uint32_t i = i0 + u * kCeBlock;
+            if (i < sp.nvec) {
+                float d[VEC];
+                ce_grad_elems<T, VEC>(v[u], d, lse, gl, sp.head + i * VEC, label);
+                if (accumulate) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) d[k] = old[u][k] + d[k];
+                }
+                VecIO<T, VEC>::store(obody + (uint64_t)i * VEC, d);
+            }
+        }
+    }
+}
+
+// The same gradient with the row's log-sum-exp given, as a one-shot grid: a
+// workgroup is one wave and takes 64 vectors of one row (chunk blockIdx.y of row
+// blockIdx.x), one vector per lane, and chunk 0 also takes the row's head and
+// tail elements.  Measured on MI355X, many small one-shot workgroups stream
+// about 20% faster than a workgroup looping along its row.
+constexpr int kCeFlatBlock = 64;
+
+template <typename T, int VEC>
+__global__ void __launch_bounds__(kCeFlatBlock)
+ce_bwd_flat_kernel(const T* __restrict__ x, const int32_t* __restrict__ labels, const float* __restrict__ dloss,
+                   const float* __restrict__ lse_in, T* dx, uint32_t V, uint32_t chunks, int accumulate,
+                   int* err_flag) {
+    // consecutive workgroups take consecutive chunks of one row, so that the
+    // workgroups in flight together touch neighbouring memory
+    const uint32_t row32 = blockIdx.x / chunks;
+    const uint32_t chunk = blockIdx.x - row32 * chunks;
+    const uint64_t row = row32;
+    const T* base = x + row * V;
+    T* out = dx + row * V;
+    const RowSplit<T, VEC> sp(base, V);
+    const uint32_t i = chunk * kCeFlatBlock + threadIdx.x;
+    const bool extras = VEC > 1 && chunk == 0;
+    if (i >= sp.nvec && !extras) return;
+    const float lse = lse_in[row];
+    const float gl = dloss[row];
+    const int32_t lab = labels[row];
+    uint32_t label = 0xffffffffu;
+    if (lab < 0 || (uint32_t)lab >= V) {
+        if (chunk == 0 && threadIdx.x == 0) *err_flag = 1;
+    } else {
+        label = (uint32_t)lab;
+    }
+    float v[VEC], old[VEC];
+    const bool live = i < sp.nvec;
+    if (live) {
+        VecIO<T, VEC>::load(base + sp.head + (uint64_t)i * VEC, v);
+        if (accumulate) VecIO<T, VEC>::load(out + sp.head + (uint64_t)i * VEC, old);
+    }
+    if constexpr (VEC > 1) {
+        const uint32_t extra = sp.head + (V - sp.tail_start);
+        if (extras && threadIdx.x < extra) {
+            const uint32_t e = threadIdx.x < sp.head ? threadIdx.x : sp.tail_start + (threadIdx.x - sp.head);
+            float xv[1], d[1];
+            VecIO<T, 1>::load(base + e, xv);
+            ce_grad_elems<T, 1>(xv, d, lse, gl, e, label);
+            if (accumulate) {
+                float o1[1];
+                VecIO<T, 1>::load(out + e, o1);
+                d[0] = o1[0] + d[0];
+            }
+            VecIO<T, 1>::store(out + e, d);
+        }
+    }
+    if (live) {
+        float d[VEC];
+        ce_grad_elems<T, VEC>(v, d, lse, gl, sp.head + i * VEC, label);
+        if (accumulate) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) d[k] = old[k] + d[k];
+        }
+        VecIO<T, VEC>::store(out + sp.head + (uint64_t)i * VEC, d);
+    }
+}
+
+template <typename T>
+int ce_typed(hipStream_t s, bool backward, const T* x, const int32_t* labels, float* loss, float* lse_out,
+             const float* dloss, const float* lse_in, T* dx, uint64_t rows, uint32_t V, int acc, int* err_flag) {
+    constexpr int WIDE = WideVec<T>::value;
+    // the element-wise head realigns every row, which needs the two tensors to
+    // share their alignment and the element size to divide 16
+    const bool wide = V >= 4 * WIDE && aligned16(x) && (!backward || aligned16(dx));
+    const dim3 grid((uint32_t)rows), block(kCeBlock);
+    if (!backward) {
+        if (wide) hipLaunchKernelGGL((ce_fwd_kernel<T, WIDE>), grid, block, 0, s, x, labels, loss, lse_out, V, err_flag);
+        else hipLaunchKernelGGL((ce_fwd_kernel<T, 1>), grid, block, 0, s, x, labels, loss, lse_out, V, err_flag);
+    } else if (lse_in != nullptr) {
+        const uint32_t vecs = wide ? V / WIDE : V;             // an upper bound on a row's vectors
+        const uint32_t chunks = (vecs + kCeFlatBlock - 1) / kCeFlatBlock;
+        // rows are launched in slabs that keep the flat workgroup index within 31 bits
+        const uint64_t max_rows = 0x7fffffffull / chunks;
+        for (uint64_t r0 = 0; r0 < rows; r0 += max_rows) {
+            const uint64_t nr = rows - r0 < max_rows ? rows - r0 : max_rows;
+            const dim3 fgrid((uint32_t)(nr * chunks)), fblock(kCeFlatBlock);
+            const T* xs = x + r0 * V;
+            T* ds = dx + r0 * V;
+            if (wide) hipLaunchKernelGGL((ce_bwd_flat_kernel<T, WIDE>), fgrid, fblock, 0, s, xs, labels + r0, dloss + r0, lse_in + r0, ds, V, chunks, acc, err_flag);
+            else hipLaunchKernelGGL((ce_bwd_flat_kernel<T, 1>), fgrid, fblock, 0, s, xs, labels + r0, dloss + r0, lse_in + r0, ds, V, chunks, acc, err_flag);
+        }
+    } else {
+        if (wide) hipLaunchKernelGGL((ce_bwd_kernel<T, WIDE>), grid, block, 0, s, x, labels, dloss, lse_in, dx, V, acc, err_flag);
+        else hipLaunchKernelGGL((ce_bwd_kernel<T, 1>), grid, block, 0, s, x, labels, dloss, lse_in, dx, V, acc, err_flag);
+    }
+    return check_hip(hipGetLastError(), "cross-entropy launch");
+}
+
+int ce_check(const char* what, int dtype, uint64_t rows, uint32_t V) {
+    if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "%s: unknown dtype %d", what, dtype);
+    if (rows > 0x7fffffffull) return set_error(AGRAD_EINVAL, "%s: too many rows", what);
+    if (V >= 0x7fffffffu) return set_error(AGRAD_EINVAL, "%s: vocabulary too large", what);
+    return AGRAD_OK;
+}
+
+}  // namespace
+
+int launch_ce_fwd(hipStream_t s, int dtype, const void* logits, const int32_t* labels, float* loss,
+                  float* lse_out, uint64_t rows, uint32_t V, int* err_flag) {
+    if (int rc = ce_check("cross-entropy forward", dtype, rows, V)) return rc;
+    if (rows == 0) return AGRAD_OK;
+    if (V == 0) return set_error(AGRAD_EINVAL, "cross-entropy forward: empty class axis");
+    if (logits == nullptr || labels == nullptr || loss == nullptr)
+        return set_error(AGRAD_EINVAL, "cross-entropy forward: null operand");
+    if (dtype == AGRAD_F32)
+        return ce_typed<float>(s, false, (const float*)logits, labels, loss, lse_out, nullptr, nullptr, nullptr, rows, V, 0, err_flag);
+    return ce_typed<bf16_t>(s, false, (const bf16_t*)logits, labels, loss, lse_out, nullptr, nullptr, nullptr, rows, V, 0, err_flag);
+}
+
+int launch_ce_bwd(hipStream_t s, int dtype, const void* logits, const int32_t* labels, const float* dloss,
+                  const float* lse, void* dlogits, uint64_t rows, uint32_t V, uint32_t flags, int* err_flag) {
+    if (int rc = ce_check("cross-entropy backward", dtype, rows, V)) return rc;
+    if (rows == 0 || V == 0) return AGRAD_OK;
+    if (logits == nullptr || labels == nullptr || dloss == nullptr || dlogits == nullptr)
+        return set_error(AGRAD_EINVAL, "cross-entropy backward: null operand");
+    const int acc = (flags & AGRAD_ACC_INPUT_GRAD) ? 1 : 0;
+    if (dtype == AGRAD_F32)
+        return ce_typed<float>(s, true, (const float*)logits, labels, nullptr, nullptr, dloss, lse, (float*)dlogits, rows, V, acc, err_flag);
+    return ce_typed<bf16_t>(s, true, (const bf16_t*)logits, labels, nullptr, nullptr, dloss, lse, (bf16_t*)dlogits, rows, V, acc, err_flag);
+}
+
+}  // namespace agrad

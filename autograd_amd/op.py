@@ -221,6 +221,41 @@ class RMSNormOp(Op):
         return list(range(len(inputs)))
 
 
+class CrossEntropyLossOp(Op):
+    """loss[b, t] = -log softmax(logits[b, t, :])[labels[b, t]]  (op.py:269-284).
+
+    The node has a second, gradient-free output: the row's log-sum-exp, which
+    the backward kernel uses instead of reducing the row again.  `__call__`
+    returns the loss only, like the reference's op.  loss is fp32 whatever the
+    logits' type."""
+    op_name = "CrossEntropyLoss"
+
+    def __init__(self, dim=-1):
+        if dim != -1:
+            raise ValueError("CrossEntropyLoss reduces the last axis")
+        self.dim = dim
+
+    def infer_shape(self, logits, labels):
+        if logits.shape[:-1] != labels.shape:
+            raise ValueError("CE shape mismatch")
+        return labels.shape
+
+    def __call__(self, logits, labels):
+        shape = self.infer_shape(logits, labels)
+        loss = Tensor(shape=shape, dtype=np.float32, requires_grad=logits.requires_grad, device=logits.device)
+        lse = Tensor(shape=shape, dtype=np.float32, requires_grad=False, device=logits.device)
+        node = OpNode(op=self, inputs=(logits, labels), outputs=(loss, lse))
+        loss.op = node
+        lse.op = node
+        return loss
+
+    def save_for_backward(self, inputs, outputs):
+        return list(inputs) + [outputs[1]]
+
+    def fully_written_inputs(self, inputs, outputs):
+        return [0]
+
+
 class _AddNormOp(Op):
     """(h, y) = (x + residual, norm(x + residual)).  Two outputs: h continues
     the residual stream, y feeds the next block."""

@@ -135,7 +135,7 @@ def build_cases(ctx, cfg, pool):
     nbytes = op_bytes(cfg, distinct)
     cases = []
     # one builder per op family: each keeps its buffers in its own scope
-    for builder in (_embed_cases, _norm_cases, _act_cases, _rope_cases, _opt_cases):
+    for builder in (_embed_cases, _norm_cases, _act_cases, _rope_cases, _loss_cases, _opt_cases):
         cases += builder(ctx, cfg, pool, rng, nbytes, ids0)
     return cases
 
@@ -275,6 +275,31 @@ def _rope_cases(ctx, cfg, pool, rng, nbytes, ids0):
         cases.append(Case("rope", "fwd", nbytes["rope"][0], k, fwd, "rope_kernel"))
         cases.append(Case("rope", "bwd", nbytes["rope"][1], k, bwd, "rope_kernel"))
     return cases
+
+
+def _loss_cases(ctx, cfg, pool, rng, nbytes, ids0):
+    """cross-entropy over logits [N, V]: forward reads the logits once, backward
+    reads them and writes the gradient (the forward pass leaves the row
+    log-sum-exp).  Reported beside the step, not part of it."""
+    if not cfg.embed:
+        return []
+    dt = capi.BF16 if cfg.dtype == "bf16" else capi.F32
+    N, V, e = cfg.N, cfg.V, cfg.esize
+    k = n_sets(2 * N * V * e)
+    logits = [pool.normal(N * V, cfg.dtype) for _ in range(k)]
+    dlogits = [pool.empty(N * V, cfg.dtype) for _ in range(k)]
+    labels = pool.upload(rng.integers(0, V, N, dtype=np.int32))
+    loss, lse, dloss = pool.empty(N, "f32"), pool.empty(N, "f32"), pool.normal(N, "f32")
+
+    def fwd(i):
+        ctx.call("agrad_cross_entropy_forward", dt, vp(logits[i]), vp(labels), vp(loss), vp(lse), N, V)
+
+    def bwd(i):
+        ctx.call("agrad_cross_entropy_backward", dt, vp(logits[i]), vp(labels), vp(dloss), vp(lse), vp(dlogits[i]), N, V, 0)
+
+    fwd(0)   # lse for the backward timing
+    return [Case("cross_entropy", "loss-fwd", N * V * e + 12 * N, k, fwd, "ce_fwd_kernel"),
+            Case("cross_entropy", "loss-bwd", 2 * N * V * e + 12 * N, k, bwd, "ce_bwd_kernel")]
 
 
 def _opt_cases(ctx, cfg, pool, rng, nbytes, ids0):

@@ -188,6 +188,24 @@ int agrad_embedding_backward(agrad_ctx* ctx, int dtype, const int32_t* ids, cons
 int agrad_pos_embedding_backward(agrad_ctx* ctx, int dtype, const void* dY, void* dwpe,
                                  uint32_t B, uint32_t T, uint32_t C, uint32_t flags);
 
+/* ---- cross-entropy over the last axis (the loss that produces the upstream gradient) ---- */
+
+/* loss[r] = -((x[r, labels[r]] - max_r) - log(sum_v exp(x[r, v] - max_r))) for logits
+ * x[rows, V] (fp32 or bf16) and int32 labels (cpu_crossentropy_forward,
+ * backend.py:489-503; CrossEntropyLossOp, op.py:269-284).  loss is fp32.  If
+ * lse_out is not NULL it receives max_r + log(sum) per row (fp32) for the
+ * backward pass.  A label outside [0, V) sets the deferred index error
+ * (reported by agrad_end_pass / agrad_synchronize) and that row's loss is 0. */
+int agrad_cross_entropy_forward(agrad_ctx* ctx, int dtype, const void* logits, const int32_t* labels,
+                                float* loss, float* lse_out, uint64_t rows, uint32_t V);
+/* dlogits[r, v] (+)= (exp(x[r, v] - lse[r]) - [v == labels[r]]) * dloss[r]
+ * (cpu_crossentropy_backward, backend.py:505-524).  lse may be NULL: the row's
+ * log-sum-exp is then recomputed first (one more read of the logits).
+ * AGRAD_ACC_INPUT_GRAD accumulates into dlogits, otherwise it is overwritten. */
+int agrad_cross_entropy_backward(agrad_ctx* ctx, int dtype, const void* logits, const int32_t* labels,
+                                 const float* dloss, const float* lse, void* dlogits,
+                                 uint64_t rows, uint32_t V, uint32_t flags);
+
 /* ---- optimizer step over the parameter slab (the consumer of the gradients above) ---- */
 
 /* One AdamW step on numel fp32 parameters with fp32 moments, in place; the

@@ -147,3 +147,19 @@ def adamw_reference(p0, grads, lr, b1, b2, eps, weight_decay):
         lr_t = lr * np.sqrt(1.0 - b2 ** t) / (1.0 - b1 ** t)
         p = p - lr_t * m / (np.sqrt(v) + eps)
     return p, m, v
+
+
+def cross_entropy(x, labels):
+    """-log softmax(x)[label] in float64 through scipy's logsumexp"""
+    from scipy.special import logsumexp
+    x = f64(x)
+    picked = np.take_along_axis(x, np.asarray(labels, np.int64)[..., None], axis=-1)[..., 0]
+    return logsumexp(x, axis=-1) - picked
+
+
+def cross_entropy_grad(x, labels, dloss):
+    from scipy.special import softmax
+    p = softmax(f64(x), axis=-1)
+    onehot = np.zeros_like(p)
+    np.put_along_axis(onehot, np.asarray(labels, np.int64)[..., None], 1.0, axis=-1)
+    return (p - onehot) * f64(dloss)[..., None]

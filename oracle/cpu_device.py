@@ -17,8 +17,8 @@ import numpy as np
 
 from autograd_amd.backend import Backend
 from autograd_amd.device import Device
-from autograd_amd.op import (AddLayerNormOp, AddOp, AddRMSNormOp, EmbeddingSumOp, GatherOp, GELUOp,
-                             LayerNormOp, ReLUSquaredOp, RMSNormOp, RopeOp, SwiGLUOp)
+from autograd_amd.op import (AddLayerNormOp, AddOp, AddRMSNormOp, CrossEntropyLossOp, EmbeddingSumOp, GatherOp,
+                             GELUOp, LayerNormOp, ReLUSquaredOp, RMSNormOp, RopeOp, SwiGLUOp)
 from autograd_amd.storage import Allocator, Storage
 from autograd_amd.utils import is_bf16, storage_dtype
 
@@ -249,6 +249,24 @@ def cpu_add_norm_backward(inputs, outputs, scratch=None):
                 np.add(acc, total, out=acc)
 
 
+def cpu_cross_entropy_forward(inputs, outputs, scratch=None):
+    logits, labels = inputs
+    x = _val(logits)
+    _put(outputs[0], K.cross_entropy_forward(x, labels.storage.data))
+    # the second output (row log-sum-exp) is an aid for the device kernels only
+    m = x.max(-1, keepdims=True)
+    _put(outputs[1], (m + np.log(np.exp(x - m).sum(-1, keepdims=True)))[..., 0])
+
+
+def cpu_cross_entropy_backward(inputs, outputs, scratch=None):
+    logits, labels = inputs
+    loss = outputs[0]
+    if loss.grad is None or not logits.requires_grad:
+        return
+    with _Acc(logits.grad) as acc:
+        K.cross_entropy_backward_into(_val(logits), labels.storage.data, _val(loss.grad), acc)
+
+
 def cpu_rope_forward(inputs, outputs, scratch=None):
     q, k, cos, sin = inputs
     q2, k2 = outputs
@@ -284,12 +302,14 @@ class CPUBackend(Backend):
             GELUOp: cpu_gelu_forward, ReLUSquaredOp: cpu_relu2_forward, SwiGLUOp: cpu_swiglu_forward,
             LayerNormOp: cpu_layernorm_forward, RMSNormOp: cpu_rmsnorm_forward,
             AddLayerNormOp: cpu_add_norm_forward, AddRMSNormOp: cpu_add_norm_forward, RopeOp: cpu_rope_forward,
+            CrossEntropyLossOp: cpu_cross_entropy_forward,
         }
         self.backward_kernels = {
             AddOp: cpu_add_backward, GatherOp: cpu_gather_backward, EmbeddingSumOp: cpu_embedding_sum_backward,
             GELUOp: cpu_gelu_backward, ReLUSquaredOp: cpu_relu2_backward, SwiGLUOp: cpu_swiglu_backward,
             LayerNormOp: cpu_layernorm_backward, RMSNormOp: cpu_rmsnorm_backward,
             AddLayerNormOp: cpu_add_norm_backward, AddRMSNormOp: cpu_add_norm_backward, RopeOp: cpu_rope_backward,
+            CrossEntropyLossOp: cpu_cross_entropy_backward,
         }
 
     def get_forward_kernel(self, op):

@@ -17,6 +17,8 @@ Pinning (what shows these functions are the right functions; tests/test_oracle.p
     577-645 (restated in float64), finite differences, rotation invariants.
   * gather: numpy fancy indexing; backward: brute-force row loop.
   * bf16: bit-exact against an exhaustive integer restatement of utils.py:20-27.
+  * cross-entropy: scipy.special.logsumexp / softmax in float64, finite
+    differences, rows of the gradient sum to zero, uniform logits give log V.
   * adamw: the textbook bias-corrected recurrence in float64 over several steps;
     the first step from zero moments moves every weight by lr * sign(g).
 Parity unpinned by the reference:
@@ -306,6 +308,37 @@ def rope_signed(q, k, cos, sin, rope_sign, backward=False):
                 else:
                     np.subtract(hi, r1, out=hi)
                 np.copyto(lo, r0)
+
+
+# --------------------------------------------------------------------------
+# Cross-entropy over the last axis  (cpu_crossentropy_forward / backward,
+# backend.py:489-524)
+# --------------------------------------------------------------------------
+def cross_entropy_forward(x, labels):
+    """x [..., V] fp32, labels [...] int -> loss [...]"""
+    r = np.max(x, axis=-1, keepdims=True)
+    f = np.subtract(x, r)
+    e = np.exp(f)
+    np.sum(e, axis=-1, keepdims=True, out=r)
+    np.log(r, out=r)
+    np.subtract(f, r, out=f)
+    idx = labels.astype(np.int64)
+    gathered = np.take_along_axis(f, idx[..., None], axis=-1)[..., 0]
+    return np.negative(gathered)
+
+
+def cross_entropy_backward_into(x, labels, dloss, dx):
+    """dx += (softmax(x) - onehot(labels)) * dloss[..., None]"""
+    r = np.max(x, axis=-1, keepdims=True)
+    f = np.subtract(x, r)
+    np.exp(f, out=f)
+    np.sum(f, axis=-1, keepdims=True, out=r)
+    np.divide(f, r, out=f)
+    V = x.shape[-1]
+    flat = f.reshape(-1, V)
+    flat[np.arange(flat.shape[0]), labels.astype(np.int64).ravel()] -= 1.0
+    np.multiply(f, dloss[..., None], out=f)
+    np.add(dx, f, out=dx)
 
 
 # --------------------------------------------------------------------------

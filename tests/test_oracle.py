@@ -413,3 +413,36 @@ def test_grad_norm_partials():
     assert part.shape == (4,)
     assert abs(part.sum() - float(np.dot(g.astype(np.float64), g.astype(np.float64)))) < 1e-9
     assert abs(part[3] - float((g[768:].astype(np.float64) ** 2).sum())) < 1e-12
+
+
+# ---------------------------------------------------------------------------
+# cross-entropy (cpu_crossentropy_forward / backward, backend.py:489-524)
+# ---------------------------------------------------------------------------
+def test_cross_entropy_closed_form_fd_and_invariants():
+    r = rng(50)
+    B, Tn, V = 2, 5, 37
+    x = (3.0 * r.standard_normal((B, Tn, V))).astype(np.float32)
+    labels = r.integers(0, V, (B, Tn), dtype=np.int32)
+    loss = K.cross_entropy_forward(x, labels)
+    close(loss, cf.cross_entropy(x, labels))
+    # uniform logits: every class has probability 1/V
+    close(K.cross_entropy_forward(np.full((1, 1, V), 0.7, np.float32), np.array([[3]], np.int32)), np.log(V))
+    # a dominant correct class costs nothing, a dominant wrong class costs the margin
+    big = np.zeros((1, 2, V), np.float32)
+    big[0, 0, 4] = 50.0
+    big[0, 1, 9] = 50.0
+    close(K.cross_entropy_forward(big, np.array([[4, 4]], np.int32)), [[0.0, 50.0]], atol=1e-5)
+    # shifting a row changes nothing
+    close(K.cross_entropy_forward(x + np.float32(5.0), labels), loss, atol=5e-6)
+    dloss = r.standard_normal((B, Tn)).astype(np.float32)
+    dx = np.zeros_like(x)
+    K.cross_entropy_backward_into(x, labels, dloss, dx)
+    close(dx, cf.cross_entropy_grad(x, labels, dloss))
+    assert np.abs(dx.sum(-1, dtype=np.float64)).max() < 1e-6        # softmax sums to one
+    base = np.ones_like(x)
+    K.cross_entropy_backward_into(x, labels, dloss, base)            # accumulates
+    close(base - 1.0, dx, atol=2e-6)
+    where = [0, (1 * Tn + 3) * V + 7, (1 * Tn + 4) * V + int(labels[1, 4])]
+    fd = cf.finite_diff(lambda a: float((cf.cross_entropy(a, labels) * dloss).sum()), x, where)
+    for i, val in zip(where, fd):
+        assert abs(val - dx.reshape(-1)[i]) < 2e-3 * max(1.0, abs(val))
