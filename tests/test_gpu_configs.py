@@ -379,3 +379,43 @@ def test_embedding_full_shape(ctx, cfg):
             assert np.abs(gp - ref).max() <= (1e-2 if d.bf16 else 1e-5) * max(1.0, np.abs(ref).max())
     finally:
         d.release()
+
+
+# ---------------------------------------------------------------------------------
+@pytest.mark.parametrize("cfg", FULL, ids=IDS)
+def test_cross_entropy_full_shape(ctx, cfg):
+    """logits [N, V] at the configuration's N and vocabulary: a block of R distinct
+    rows repeated, labels drawn for all N rows.  The loss of every row follows from
+    the block's log-sum-exp; the gradient is compared on sampled rows, including the
+    first and last rows of the tensor (the backward kernel cuts very large tensors
+    into slabs of rows)."""
+    from scipy.special import logsumexp
+    rng = np.random.default_rng(cfg.seed + 400)
+    N, V = cfg.N, cfg.V
+    R = 16
+    d = Dev(ctx, cfg)
+    try:
+        xs, xv = d.host(3.0 * rng.standard_normal((R, V)))
+        labels = rng.integers(0, V, N, dtype=np.int32)
+        dloss = rng.standard_normal(N).astype(np.float32)
+        x = d.tiled(xs, N // R)
+        dl, dg = d.upload(labels), d.upload(dloss)
+        loss, lse = d.empty(N, np.float32), d.empty(N, np.float32)
+        dx = d.empty(N * V)
+        ctx.call("agrad_cross_entropy_forward", d.dt, vp(x), vp(dl), vp(loss), vp(lse), N, V)
+        ctx.call("agrad_cross_entropy_backward", d.dt, vp(x), vp(dl), vp(dg), vp(lse), vp(dx), N, V, 0)
+        ctx.synchronize()
+        lse64 = logsumexp(xv.astype(np.float64), axis=-1)
+        blk = np.arange(N) % R
+        want_loss = lse64[blk] - xv[blk, labels].astype(np.float64)
+        tol = 1e-4 if d.bf16 else 1e-5            # bf16 logits go through the hardware exp2
+        got_loss = loss.download()
+        assert np.abs(got_loss - want_loss).max() <= tol * max(1.0, np.abs(want_loss).max())
+        assert np.abs(lse.download() - lse64[blk]).max() <= tol * max(1.0, np.abs(lse64).max())
+        for n in sorted({0, 1, R - 1, N // 2 + 3, N - R, N - 1} | set(rng.integers(0, N, 6).tolist())):
+            got = d.rows(dx, n, 1, V)[0]
+            ref = np.zeros((1, V), np.float32)
+            K.cross_entropy_backward_into(xv[n % R][None], labels[n:n + 1], dloss[n:n + 1], ref)
+            d.close_enough(got[None], ref, f"{cfg.name} dlogits row {n}")
+    finally:
+        d.release()
