@@ -5,14 +5,19 @@
 //
 // Backward dW[ids[n],:] += dY[n,:] (np.add.at, backend.py:531-538) is done
 // without float atomics:
-//   1. keys = ids, values = row numbers; stable LSD radix sort by key, so each
-//      token's rows form one run of the sorted order, in ascending row order;
+//   1. (token, row) pairs are ordered so that each token's rows form one run,
+//      in ascending row order.  Up to 16384 rows this is ONE launch: every
+//      workgroup owns a hash group of tokens, scans all ids for its own, and
+//      orders its pairs in LDS (runs of distinct tokens then follow hash-group
+//      order, which is all the later steps need).  Larger inputs take a stable
+//      LSD radix sort by token (rocPRIM);
 //   2. the sorted order is cut into chunks of L positions, one workgroup each;
 //      a workgroup sums every run inside its chunk in order (fp32) and stores
 //      it straight to dW when the run lies wholly inside the chunk;
 //   3. a run that crosses a chunk edge leaves fp32 partial rows in a carry
-//      buffer; a second kernel adds the partial rows of such a run in chunk
-//      order and stores the total.
+//      buffer; a second kernel adds the partial rows of such a run in a fixed
+//      order and stores the total (a hot token's many partial rows are shared
+//      out over the run's own middle chunks).
 // Every sum has a fixed order, so the result is run-to-run identical, and runs
 // inside one chunk are bit-identical to the sequential CPU sum.
 #include "common.hpp"
