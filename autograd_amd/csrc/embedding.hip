@@ -679,7 +679,7 @@ int launch_gather_fwd(hipStream_t s, int dtype, const int32_t* ids, const void* 
     if (wide && total_vec < 0xffff0000ull) {
         const uint32_t CV = C / per16;
         const uint32_t total = (uint32_t)total_vec;
-        constexpr int UNROLL = 4;
+        constexpr int UNROLL = 1;
         const uint32_t grid = (total + kGatherBlock * UNROLL - 1) / (kGatherBlock * UNROLL);
         if (wpe == nullptr) {
             hipLaunchKernelGGL((gather_rows16_kernel<UNROLL>), dim3(grid), dim3(kGatherBlock), 0, s, ids,
@@ -688,9 +688,8 @@ int launch_gather_fwd(hipStream_t s, int dtype, const int32_t* ids, const void* 
             hipLaunchKernelGGL((gather_fwd_kernel<float, 4, UNROLL>), dim3(grid), dim3(kGatherBlock), 0, s, ids,
                                (const float*)W, (const float*)wpe, (float*)out, total, CV, C, T, V, err_flag);
         } else {
-            hipLaunchKernelGGL((gather_fwd_kernel<bf16_t, 8, 2>), dim3((total + kGatherBlock * 2 - 1) / (kGatherBlock * 2)),
-                               dim3(kGatherBlock), 0, s, ids, (const bf16_t*)W, (const bf16_t*)wpe,
-                               (bf16_t*)out, total, CV, C, T, V, err_flag);
+            hipLaunchKernelGGL((gather_fwd_kernel<bf16_t, 8, UNROLL>), dim3(grid), dim3(kGatherBlock), 0, s, ids,
+                               (const bf16_t*)W, (const bf16_t*)wpe, (bf16_t*)out, total, CV, C, T, V, err_flag);
         }
     } else {
         const uint64_t total = N * C;
