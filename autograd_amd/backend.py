@@ -210,6 +210,14 @@ class HipBackend(Backend):
                 x = node.inputs[0]
                 rows, C = prod(x.shape[:-1]), x.shape[-1]
                 return None, single_slot("workspace", self.ctx.norm_backward_workspace_bytes(rows, C, _dt(x)))
+        if isinstance(op, AddOp):
+            out = node.outputs[0]
+            need = 0
+            for t in node.inputs[:2]:
+                if t.requires_grad and t.shape != out.shape and t.numel:
+                    need = max(need, self.ctx.broadcast_grad_workspace_bytes(out.numel // t.numel, t.numel))
+            if need:
+                return None, single_slot("workspace", need)
         if isinstance(op, (GatherOp, EmbeddingSumOp)):
             ids, w = node.inputs[0], node.inputs[1]
             if w.requires_grad:
@@ -218,11 +226,27 @@ class HipBackend(Backend):
         return None, None
 
     # -- Add (cpu_add_forward / cpu_add_backward, backend.py:74-105) ----------------
+    @staticmethod
+    def _trailing(small, big):
+        """True if `small` (after dropping leading 1s) is the trailing shape of `big`"""
+        sh = tuple(small)
+        while sh and sh[0] == 1:
+            sh = sh[1:]
+        return len(sh) <= len(big) and tuple(big[len(big) - len(sh):]) == sh
+
     def hip_add_forward(self, inputs, outputs, scratch=None):
         x, y, out = inputs[0], inputs[1], outputs[0]
-        if x.shape != y.shape:
+        if x.shape == y.shape:
+            self._launch("add_residual_forward", [x, y, out], [_dt(out)] + _lo_hi(out.numel))
+            return
+        # one operand has the output's shape, the other its trailing shape (a bias,
+        # a position table): add_pos_forward / bias add of the reference's Metal backend
+        big, small = (x, y) if x.shape == out.shape else (y, x)
+        if big.shape != out.shape or not self._trailing(small.shape, out.shape) or _dt(big) != _dt(small):
             raise RuntimeError(f"Unsupported Add shape: x.shape={x.shape}, y.shape={y.shape}")
-        self._launch("add_residual_forward", [x, y, out], [_dt(out)] + _lo_hi(out.numel))
+        inner = small.numel
+        self._launch("add_broadcast_forward", [big, small, out],
+                     [_dt(out)] + _lo_hi(out.numel // max(inner, 1)) + _lo_hi(inner))
 
     def hip_add_backward(self, inputs, outputs, scratch=None):
         out = outputs[0]
@@ -235,10 +259,14 @@ class HipBackend(Backend):
             if t.shape == out.shape:
                 self._launch("add_residual_backward", [out.grad, t.grad],
                              [_dt(out), self._grad_flag(node, t)] + _lo_hi(out.numel))
-            elif out.shape[len(out.shape) - t.ndim:] == t.shape:
-                lead = prod(out.shape[:len(out.shape) - t.ndim])
+            elif self._trailing(t.shape, out.shape) and _dt(t.grad) == _dt(out.grad):
+                inner = t.numel
+                lead = out.numel // max(inner, 1)
                 flag = ACC_PARAM_GRAD if self._grad_flag(node, t) else 0
-                self._launch("pos_emb_grad", [out.grad, t.grad], [_dt(out), lead, 1, t.numel, flag])
+                ws = scratch["workspace"] if scratch and "workspace" in scratch else None
+                self._launch("add_broadcast_backward", [out.grad, t.grad, ws],
+                             [_dt(out)] + _lo_hi(lead) + _lo_hi(inner) + [flag]
+                             + _lo_hi(ws.nbytes if ws is not None else 0) + [_mask(out.grad, t.grad, ws)])
             else:
                 raise RuntimeError(f"Unsupported Add backward shape: {t.shape} from {out.shape}")
 

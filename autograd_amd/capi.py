@@ -70,6 +70,9 @@ SIGNATURES = {
     "agrad_embedding_backward_workspace_bytes": (_u64, [_u64, _u32, _u32, _int]),
     "agrad_embedding_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u64, _u32, _u32, _u32]),
     "agrad_pos_embedding_backward": (_int, [_ctx, _int, _ptr, _ptr, _u32, _u32, _u32, _u32]),
+    "agrad_broadcast_add_forward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _u64, _u64]),
+    "agrad_broadcast_grad_workspace_bytes": (_u64, [_u64, _u64]),
+    "agrad_broadcast_add_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _u64, _u64, _u64, _u32]),
     "agrad_cross_entropy_forward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u32]),
     "agrad_cross_entropy_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _u64, _u32, _u32]),
     "agrad_adamw_step": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u64] + [_f32] * 9),

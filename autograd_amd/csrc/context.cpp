@@ -142,6 +142,21 @@ int h_add_bwd(const Call& c) {
     RESOLVE(0, bytes, src) RESOLVE(1, bytes, dst)
     return launch_accumulate(c.ctx->stream, c.a[0], src, dst, n, c.a[1]);
 }
+// buffers x, y, out | args dtype, lead lo, hi, inner lo, hi
+int h_bcast_add(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t lead = u64(c.a, 1), inner = u64(c.a, 3), es = dtype_size(c.a[0]);
+    RESOLVE(0, lead * inner * es, x) RESOLVE(1, inner * es, y) RESOLVE(2, lead * inner * es, out)
+    return launch_broadcast_add(c.ctx->stream, (int)c.a[0], x, y, out, lead, inner);
+}
+// buffers g, dy, workspace | args dtype, lead lo, hi, inner lo, hi, flags, ws lo, hi, present_mask
+int h_bcast_grad(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t lead = u64(c.a, 1), inner = u64(c.a, 3), es = dtype_size(c.a[0]), wsb = u64(c.a, 6);
+    RESOLVE(0, lead * inner * es, g) RESOLVE(1, inner * es, dy)
+    RESOLVE_IF(c.a[8] & 4u, 2, wsb, ws)
+    return launch_broadcast_grad(c.ctx->stream, (int)c.a[0], g, dy, ws, ws ? wsb : 0, lead, inner, c.a[5]);
+}
 int h_cast_down(const Call& c) {
     const uint64_t n = u64(c.a, 1);
     RESOLVE(0, n * 4, src) RESOLVE(1, n * 2, dst)
@@ -315,6 +330,8 @@ const Entry kTable[] = {
     {"copy_kernel", 2, 2, "src, dst | nbytes_lo, nbytes_hi", h_copy},
     {"add_residual_forward", 3, 3, "x, y, out | dtype, n_lo, n_hi", h_add_fwd},
     {"add_residual_backward", 2, 4, "g, dst | dtype, flags, n_lo, n_hi", h_add_bwd},
+    {"add_broadcast_forward", 3, 5, "x, y, out | dtype, lead_lo, lead_hi, inner_lo, inner_hi", h_bcast_add},
+    {"add_broadcast_backward", 3, 9, "g, dy, workspace | dtype, lead_lo, lead_hi, inner_lo, inner_hi, flags, ws_lo, ws_hi, present_mask", h_bcast_grad},
     {"fp32_to_bf16", 2, 3, "src, dst | accumulate, n_lo, n_hi", h_cast_down},
     {"bf16_to_fp32", 2, 2, "src, dst | n_lo, n_hi", h_cast_up},
     {"layernorm_forward", 6, 5, "x, residual, gamma, beta, h, y | dtype, rows, C, eps_bits, present_mask", h_norm_fwd<AGRAD_NORM_LAYER>},
@@ -618,6 +635,20 @@ int agrad_pos_embedding_backward(agrad_ctx* ctx, int dtype, const void* dY, void
                                  uint32_t T, uint32_t C, uint32_t flags) {
     CTX_OR_FAIL(ctx)
     return launch_pos_embedding_bwd(ctx->stream, dtype, dY, dwpe, B, T, C, flags);
+}
+
+int agrad_broadcast_add_forward(agrad_ctx* ctx, int dtype, const void* x, const void* y, void* out,
+                                uint64_t lead, uint64_t inner) {
+    CTX_OR_FAIL(ctx)
+    return launch_broadcast_add(ctx->stream, dtype, x, y, out, lead, inner);
+}
+uint64_t agrad_broadcast_grad_workspace_bytes(uint64_t lead, uint64_t inner) {
+    return broadcast_grad_workspace_bytes(lead, inner);
+}
+int agrad_broadcast_add_backward(agrad_ctx* ctx, int dtype, const void* g, void* dy, void* workspace,
+                                 uint64_t workspace_bytes, uint64_t lead, uint64_t inner, uint32_t flags) {
+    CTX_OR_FAIL(ctx)
+    return launch_broadcast_grad(ctx->stream, dtype, g, dy, workspace, workspace_bytes, lead, inner, flags);
 }
 
 int agrad_cross_entropy_forward(agrad_ctx* ctx, int dtype, const void* logits, const int32_t* labels,

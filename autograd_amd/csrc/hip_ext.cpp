@@ -114,6 +114,9 @@ public:
     uint64_t norm_backward_workspace_bytes(uint64_t rows, uint32_t C, int dtype) {
         return agrad_norm_backward_workspace_bytes(rows, C, dtype);
     }
+    uint64_t broadcast_grad_workspace_bytes(uint64_t lead, uint64_t inner) {
+        return agrad_broadcast_grad_workspace_bytes(lead, inner);
+    }
     uint64_t embedding_backward_workspace_bytes(uint64_t N, uint32_t C, uint32_t V, int dtype) {
         return agrad_embedding_backward_workspace_bytes(N, C, V, dtype);
     }
@@ -164,6 +167,7 @@ PYBIND11_MODULE(hip_ext, m) {
              py::arg("shape"), py::arg("dtype") = "float32")
         .def("norm_backward_workspace_bytes", &HipContext::norm_backward_workspace_bytes)
         .def("embedding_backward_workspace_bytes", &HipContext::embedding_backward_workspace_bytes)
+        .def("broadcast_grad_workspace_bytes", &HipContext::broadcast_grad_workspace_bytes)
         .def("kernel_names", &HipContext::kernel_names)
         .def("kernel_signature", &HipContext::kernel_signature)
         .def("handle", &HipContext::handle)

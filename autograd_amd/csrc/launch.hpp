@@ -37,6 +37,16 @@ int launch_norm_bwd(hipStream_t s, int kind, int dtype, const void* x, const voi
                     float* dgamma, float* dbeta, void* workspace, uint64_t workspace_bytes,
                     uint64_t rows, uint32_t C, float eps, uint32_t flags);
 
+// out_a[c] (+)= sum over the P rows of pa[P, C] (same for pb -> out_b; either pair may be null)
+int launch_colsum_finalize(hipStream_t s, const float* pa, const float* pb, uint32_t P, uint32_t C,
+                           float* out_a, float* out_b, int accumulate);
+
+// reduce.hip
+int launch_broadcast_add(hipStream_t s, int dtype, const void* x, const void* y, void* out, uint64_t lead, uint64_t inner);
+uint64_t broadcast_grad_workspace_bytes(uint64_t lead, uint64_t inner);
+int launch_broadcast_grad(hipStream_t s, int dtype, const void* g, void* dy, void* workspace, uint64_t workspace_bytes,
+                          uint64_t lead, uint64_t inner, uint32_t flags);
+
 // activation.hip
 int launch_gelu_fwd(hipStream_t s, int dtype, const void* x, void* y, uint64_t n);
 int launch_gelu_bwd(hipStream_t s, int dtype, const void* x, const void* dy, void* dx, uint64_t n, uint32_t flags);

@@ -804,6 +804,19 @@ int norm_bwd_typed(hipStream_t s, const NormPlan& p, const NormBwdArgs<T>& a, ui
 
 }  // namespace
 
+int launch_colsum_finalize(hipStream_t s, const float* pa, const float* pb, uint32_t P, uint32_t C,
+                           float* out_a, float* out_b, int accumulate) {
+    const bool vec4 = C % 4 == 0 && (!out_a || aligned16(out_a)) && (!out_b || aligned16(out_b)) &&
+                      (!pa || aligned16(pa)) && (!pb || aligned16(pb));
+    if (vec4)
+        hipLaunchKernelGGL((colsum_finalize_kernel<4>), dim3((C / 4 + 7) / 8, 2), dim3(1024), 0, s, pa, pb, P, C,
+                           out_a, out_b, accumulate);
+    else
+        hipLaunchKernelGGL((colsum_finalize_kernel<1>), dim3((C + 7) / 8, 2), dim3(1024), 0, s, pa, pb, P, C,
+                           out_a, out_b, accumulate);
+    return check_hip(hipGetLastError(), "column-sum finalize launch");
+}
+
 uint32_t norm_bwd_max_blocks() {
     static const uint32_t value = [] {
         const char* e = std::getenv("AGRAD_NORM_BWD_BLOCKS");
@@ -898,16 +911,8 @@ int launch_norm_bwd(hipStream_t s, int kind, int dtype, const void* x, const voi
         rc = norm_bwd_typed<bf16_t>(s, p, a, grid);
     }
     if (rc != AGRAD_OK) return rc;
-    if (want_params) {
-        const int accp = (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0;
-        const bool vec4 = C % 4 == 0 && (!dgamma || aligned16(dgamma)) && (!dbeta || aligned16(dbeta));
-        if (vec4)
-            hipLaunchKernelGGL((colsum_finalize_kernel<4>), dim3((C / 4 + 7) / 8, 2), dim3(1024), 0, s, pg, pb, grid,
-                               C, dgamma, dbeta, accp);
-        else
-            hipLaunchKernelGGL((colsum_finalize_kernel<1>), dim3((C + 7) / 8, 2), dim3(1024), 0, s, pg, pb, grid,
-                               C, dgamma, dbeta, accp);
-    }
+    if (want_params)
+        return launch_colsum_finalize(s, pg, pb, grid, C, dgamma, dbeta, (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0);
     return check_hip(hipGetLastError(), "norm backward launch");
 }
 

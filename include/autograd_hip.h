@@ -104,6 +104,21 @@ const char* agrad_kernel_signature(const char* name);
 /* out[i] = x[i] + y[i]  (cpu_add_forward, backend.py:74-76; add_residual_forward,
  * metal_ops.metal:161-181). */
 int agrad_add_forward(agrad_ctx* ctx, int dtype, const void* x, const void* y, void* out, uint64_t n);
+/* out[l, j] = x[l, j] + y[j] for x [lead, inner] and y of the trailing shape [inner]
+ * (a bias, or a position table added to every batch entry: the broadcasting branch
+ * of cpu_add_forward, backend.py:74-76; add_pos_forward, metal_ops.metal:205-218). */
+int agrad_broadcast_add_forward(agrad_ctx* ctx, int dtype, const void* x, const void* y, void* out,
+                                uint64_t lead, uint64_t inner);
+/* dy[j] (+)= sum_l g[l, j], l ascending within a fixed two-level order (the
+ * broadcasting branch of cpu_add_backward, backend.py:78-105; pos_emb_grad and
+ * the bias-gradient column reductions, metal_ops.metal:220-234, 1002-1193).
+ * AGRAD_ACC_PARAM_GRAD accumulates into dy.  fp32 tensors with more than 64
+ * leading rows need a workspace of agrad_broadcast_grad_workspace_bytes(lead, inner)
+ * bytes (16-byte aligned); otherwise workspace may be NULL. */
+uint64_t agrad_broadcast_grad_workspace_bytes(uint64_t lead, uint64_t inner);
+int agrad_broadcast_add_backward(agrad_ctx* ctx, int dtype, const void* g, void* dy,
+                                 void* workspace, uint64_t workspace_bytes,
+                                 uint64_t lead, uint64_t inner, uint32_t flags);
 /* dst[i] (+)= src[i]  (same-shape branch of cpu_add_backward, backend.py:78-105). */
 int agrad_grad_accumulate(agrad_ctx* ctx, int dtype, const void* src, void* dst, uint64_t n, uint32_t flags);
 /* dst_bf16[i] = rne(src_f32[i]) (+ dst if accumulate) (fp32_to_bf16, metal_ops.metal:12010-12041). */

@@ -321,3 +321,27 @@ def test_accumulate_parameter_grads_and_rerun():
     assert_fp32_close(first, dg, "gamma.grad", atol=4e-6)
     assert_fp32_close(dx_first, dx, "x.grad")
     rt.release()
+
+
+def test_add_with_a_broadcast_operand():
+    """x[B, T, C] + bias[C] and + table[T, C]: forward and both gradients through the
+    runtime on both devices (the broadcasting branch of cpu_add_backward,
+    backend.py:78-105; lead = 144 rows takes the two-stage column sum)."""
+    rng = np.random.default_rng(SEED + 30)
+    B, T, C = 9, 16, 48
+    x_np = rng.standard_normal((B, T, C), dtype=np.float32)
+    bias_np = rng.standard_normal((C,), dtype=np.float32)
+    tab_np = rng.standard_normal((T, C), dtype=np.float32)
+    upstream = rng.standard_normal((B, T, C), dtype=np.float32)
+
+    def build(device):
+        x = make_tensor(x_np.shape, np.float32, device, True, x_np)
+        bias = make_tensor(bias_np.shape, np.float32, device, True, bias_np)
+        tab = make_tensor(tab_np.shape, np.float32, device, True, tab_np)
+        return ReLUSquaredOp()((x + bias) + tab), {"x": x, "bias": bias, "tab": tab}
+
+    (c_out, c_g), (h_out, h_g) = both(build, upstream)
+    assert_fp32_close(h_out[0], c_out[0], "forward")
+    assert_fp32_close(h_g["x"], c_g["x"], "x.grad")
+    assert_fp32_close(h_g["tab"], c_g["tab"], "tab.grad", atol=4e-6)
+    assert_fp32_close(h_g["bias"], c_g["bias"], "bias.grad", atol=2e-5)
