@@ -137,6 +137,7 @@ class HipBackend(Backend):
         self.grad_scale = 1.0
         self.accumulate_parameter_grads = False
         self.use_fp16_gemm = False
+        self._capturing = False
         self.forward_kernels = {
             AddOp: self.hip_add_forward,
             GatherOp: self.hip_gather_forward,
@@ -575,10 +576,29 @@ class HipBackend(Backend):
                      + [_dt(g_storage)])
 
     def begin_pass(self):
-        self.ctx.begin_pass()
+        if not self._capturing:
+            self.ctx.begin_pass()
 
     def end_pass(self):
-        self.ctx.end_pass()
+        # a pass boundary waits for the GPU, which a recording cannot contain
+        if not self._capturing:
+            self.ctx.end_pass()
+
+    # -- graphs -----------------------------------------------------------------------
+    def capture_begin(self):
+        """record every launch until capture_end instead of running it"""
+        self.ctx.graph_begin()
+        self._capturing = True
+
+    def capture_end(self):
+        self._capturing = False
+        return self.ctx.graph_end()
+
+    def graph_launch(self, graph_id):
+        self.ctx.graph_launch(graph_id)
+
+    def graph_destroy(self, graph_id):
+        self.ctx.graph_destroy(graph_id)
 
     def synchronize(self):
         self.ctx.synchronize()

@@ -21,6 +21,9 @@ struct agrad_ctx {
     uint64_t total_mem = 0;
     std::mutex mu;
     std::map<uint64_t, uint64_t> allocs;   // base address -> bytes
+    bool capturing = false;                // between agrad_graph_begin and agrad_graph_end
+    std::map<uint64_t, hipGraphExec_t> graphs;
+    uint64_t next_graph = 1;
 };
 
 namespace agrad {
@@ -36,6 +39,10 @@ int set_error(int code, const char* fmt, ...) {
     g_last_error = buf;
     return code;
 }
+
+static thread_local bool g_capturing = false;
+void set_capturing(bool on) { g_capturing = on; }
+bool is_capturing() { return g_capturing; }
 
 int check_hip(hipError_t e, const char* what) {
     if (e == hipSuccess) return AGRAD_OK;
@@ -70,13 +77,19 @@ int resolve(agrad_ctx* ctx, uint64_t id, uint64_t off, uint64_t need, const char
     return AGRAD_OK;
 }
 
+int no_capture(agrad_ctx* ctx, const char* what) {
+    if (ctx->capturing) return set_error(AGRAD_EINVAL, "%s cannot be recorded into a graph (it waits for the GPU)", what);
+    return AGRAD_OK;
+}
+
 int finish_stream(agrad_ctx* ctx) {
+    if (int rc = no_capture(ctx, "synchronize / end_pass")) return rc;
     if (int rc = check_hip(hipStreamSynchronize(ctx->stream), "stream synchronize")) return rc;
     int flag = 0;
     if (int rc = check_hip(hipMemcpy(&flag, ctx->err_flag, sizeof(int), hipMemcpyDeviceToHost), "error flag read")) return rc;
     if (flag != 0) {
         (void)hipMemset(ctx->err_flag, 0, sizeof(int));
-        return set_error(AGRAD_EINDEX, "token id out of range in an embedding kernel");
+        return set_error(AGRAD_EINDEX, "index out of range on the device (a token id or a class label)");
     }
     return AGRAD_OK;
 }
@@ -416,6 +429,7 @@ int agrad_ctx_destroy(agrad_ctx* ctx) {
     if (ctx == nullptr) return AGRAD_OK;
     (void)hipSetDevice(ctx->device);
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
+    for (auto& kv : ctx->graphs) (void)hipGraphExecDestroy(kv.second);
     for (auto& kv : ctx->allocs) (void)hipFree(reinterpret_cast<void*>(kv.first));
     if (ctx->err_flag) (void)hipFree(ctx->err_flag);
     if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
@@ -447,6 +461,7 @@ int agrad_alloc(agrad_ctx* ctx, uint64_t bytes, uint64_t* buffer_id) {
 
 int agrad_free(agrad_ctx* ctx, uint64_t buffer_id) {
     CTX_OR_FAIL(ctx)
+    if (int rc = no_capture(ctx, "free")) return rc;
     {
         std::lock_guard<std::mutex> lock(ctx->mu);
         auto it = ctx->allocs.find(buffer_id);
@@ -476,6 +491,7 @@ int agrad_copy_from_host(agrad_ctx* ctx, uint64_t buffer_id, uint64_t offset, co
     CTX_OR_FAIL(ctx)
     if (nbytes == 0) return AGRAD_OK;
     if (src == nullptr) return set_error(AGRAD_EINVAL, "copy_from_host: null source");
+    if (int rc = no_capture(ctx, "copy_from_host")) return rc;
     void* dst = nullptr;
     if (int rc = resolve(ctx, buffer_id, offset, nbytes, "copy_from_host", &dst)) return rc;
     if (int rc = check_hip(hipMemcpyAsync(dst, src, nbytes, hipMemcpyHostToDevice, ctx->stream), "hipMemcpyAsync H2D")) return rc;
@@ -486,6 +502,7 @@ int agrad_copy_to_host(agrad_ctx* ctx, uint64_t buffer_id, uint64_t offset, void
     CTX_OR_FAIL(ctx)
     if (nbytes == 0) return AGRAD_OK;
     if (dst == nullptr) return set_error(AGRAD_EINVAL, "copy_to_host: null destination");
+    if (int rc = no_capture(ctx, "copy_to_host")) return rc;
     void* src = nullptr;
     if (int rc = resolve(ctx, buffer_id, offset, nbytes, "copy_to_host", &src)) return rc;
     if (int rc = check_hip(hipMemcpyAsync(dst, src, nbytes, hipMemcpyDeviceToHost, ctx->stream), "hipMemcpyAsync D2H")) return rc;
@@ -509,15 +526,77 @@ int agrad_stream(agrad_ctx* ctx, void** stream) {
 
 int agrad_timer_start(agrad_ctx* ctx) {
     CTX_OR_FAIL(ctx)
+    if (int rc = no_capture(ctx, "timer")) return rc;
     return check_hip(hipEventRecord(ctx->ev_start, ctx->stream), "hipEventRecord");
 }
 
 int agrad_timer_stop(agrad_ctx* ctx, float* elapsed_ms) {
     CTX_OR_FAIL(ctx)
     if (elapsed_ms == nullptr) return set_error(AGRAD_EINVAL, "null out pointer");
+    if (int rc = no_capture(ctx, "timer")) return rc;
     if (int rc = check_hip(hipEventRecord(ctx->ev_stop, ctx->stream), "hipEventRecord")) return rc;
     if (int rc = check_hip(hipEventSynchronize(ctx->ev_stop), "hipEventSynchronize")) return rc;
     return check_hip(hipEventElapsedTime(elapsed_ms, ctx->ev_start, ctx->ev_stop), "hipEventElapsedTime");
+}
+
+// ---- graphs: record the launches between begin and end once, replay them as one submission ----
+int agrad_graph_begin(agrad_ctx* ctx) {
+    CTX_OR_FAIL(ctx)
+    if (ctx->capturing) return set_error(AGRAD_EINVAL, "graph capture is already open");
+    // relaxed mode: allocations and queries made by other code meanwhile stay legal
+    if (int rc = check_hip(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed), "hipStreamBeginCapture")) return rc;
+    ctx->capturing = true;
+    set_capturing(true);
+    return AGRAD_OK;
+}
+
+int agrad_graph_end(agrad_ctx* ctx, uint64_t* graph_id) {
+    CTX_OR_FAIL(ctx)
+    if (graph_id == nullptr) return set_error(AGRAD_EINVAL, "null out pointer");
+    *graph_id = 0;
+    if (!ctx->capturing) return set_error(AGRAD_EINVAL, "no graph capture is open");
+    ctx->capturing = false;
+    set_capturing(false);
+    hipGraph_t graph = nullptr;
+    if (int rc = check_hip(hipStreamEndCapture(ctx->stream, &graph), "hipStreamEndCapture")) return rc;
+    if (graph == nullptr) return set_error(AGRAD_EHIP, "graph capture was invalidated");
+    hipGraphExec_t exec = nullptr;
+    const hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (int rc = check_hip(e, "hipGraphInstantiate")) return rc;
+    std::lock_guard<std::mutex> lock(ctx->mu);
+    const uint64_t id = ctx->next_graph++;
+    ctx->graphs[id] = exec;
+    *graph_id = id;
+    return AGRAD_OK;
+}
+
+int agrad_graph_launch(agrad_ctx* ctx, uint64_t graph_id) {
+    CTX_OR_FAIL(ctx)
+    if (int rc = no_capture(ctx, "graph launch")) return rc;
+    hipGraphExec_t exec = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(ctx->mu);
+        auto it = ctx->graphs.find(graph_id);
+        if (it == ctx->graphs.end()) return set_error(AGRAD_EINVAL, "graph %llu does not exist", (unsigned long long)graph_id);
+        exec = it->second;
+    }
+    return check_hip(hipGraphLaunch(exec, ctx->stream), "hipGraphLaunch");
+}
+
+int agrad_graph_destroy(agrad_ctx* ctx, uint64_t graph_id) {
+    CTX_OR_FAIL(ctx)
+    if (int rc = no_capture(ctx, "graph destroy")) return rc;
+    hipGraphExec_t exec = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(ctx->mu);
+        auto it = ctx->graphs.find(graph_id);
+        if (it == ctx->graphs.end()) return set_error(AGRAD_EINVAL, "graph %llu does not exist", (unsigned long long)graph_id);
+        exec = it->second;
+        ctx->graphs.erase(it);
+    }
+    if (int rc = check_hip(hipStreamSynchronize(ctx->stream), "stream synchronize")) return rc;
+    return check_hip(hipGraphExecDestroy(exec), "hipGraphExecDestroy");
 }
 
 int agrad_dispatch(agrad_ctx* ctx, const char* name, const uint64_t* buffer_ids, const uint64_t* offsets,

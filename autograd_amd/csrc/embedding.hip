@@ -632,6 +632,9 @@ int embedding_bwd_typed(hipStream_t s, const EmbPlan& p, const int32_t* ids, con
         grouped = true;
     }
     if (!grouped) {
+        if (is_capturing())
+            return set_error(AGRAD_EINVAL, "embedding backward over %u rows uses the library radix sort, which is not "
+                             "recorded into graphs (up to %u rows are)", N, kGroupSortMaxN);
         hipLaunchKernelGGL(emb_prepare_kernel, dim3((N + 255) / 256), dim3(256), 0, s, ids, keys_in, vals_in, N, V, err_flag);
         int bits = 1;
         while ((1ull << bits) <= V) ++bits;

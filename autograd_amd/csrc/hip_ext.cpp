@@ -59,6 +59,15 @@ public:
         py::gil_scoped_acquire gil;
         raise_for(rc);
     }
+    // record the launches between graph_begin and graph_end, replay them with graph_launch
+    void graph_begin() { raise_for(agrad_graph_begin(ctx_)); }
+    uint64_t graph_end() {
+        uint64_t id = 0;
+        raise_for(agrad_graph_end(ctx_, &id));
+        return id;
+    }
+    void graph_launch(uint64_t id) { raise_for(agrad_graph_launch(ctx_, id)); }
+    void graph_destroy(uint64_t id) { raise_for(agrad_graph_destroy(ctx_, id)); }
     void synchronize() {
         py::gil_scoped_release nogil;
         int rc = agrad_synchronize(ctx_);
@@ -171,5 +180,9 @@ PYBIND11_MODULE(hip_ext, m) {
         .def("kernel_names", &HipContext::kernel_names)
         .def("kernel_signature", &HipContext::kernel_signature)
         .def("handle", &HipContext::handle)
+        .def("graph_begin", &HipContext::graph_begin)
+        .def("graph_end", &HipContext::graph_end)
+        .def("graph_launch", &HipContext::graph_launch)
+        .def("graph_destroy", &HipContext::graph_destroy)
         .def("synchronize", &HipContext::synchronize);
 }

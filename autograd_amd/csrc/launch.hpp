@@ -12,6 +12,10 @@ namespace agrad {
 
 int set_error(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 int check_hip(hipError_t e, const char* what);
+// true while the calling thread records launches into a graph: launchers whose
+// work is not a plain sequence of kernels on the stream refuse
+void set_capturing(bool on);
+bool is_capturing();
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline uint32_t dtype_size(int dtype) { return dtype == AGRAD_BF16 ? 2u : 4u; }

@@ -71,6 +71,23 @@ class _Scratch:
         self.nbytes, self.node, self.phase = nbytes, node, phase
 
 
+class CapturedGraph:
+    """a recorded sequence of launches; see Runtime.capture"""
+
+    def __init__(self, backend, graph_id):
+        self.backend, self.graph_id = backend, graph_id
+
+    def launch(self):
+        if self.graph_id is None:
+            raise RuntimeError("graph was destroyed")
+        self.backend.graph_launch(self.graph_id)
+
+    def destroy(self):
+        if self.graph_id is not None:
+            self.backend.graph_destroy(self.graph_id)
+            self.graph_id = None
+
+
 class Runtime:
     _default_runtime = None
 
@@ -410,6 +427,26 @@ class Runtime:
                     self.backend.fill(t.grad, 0)
             node.backward(node.inputs, node.outputs)
         self.backend.end_pass()
+
+    def capture(self, fn):
+        """Record everything `fn()` launches (for example `rt.execute`) into a device
+        graph and return a CapturedGraph; `graph.launch()` replays it as one
+        submission, which removes the per-launch cost that dominates chains of small
+        ops.  `fn` must already have run once eagerly (kernels load on first use), may
+        not read results back, and the replay uses the tensors as they are bound now.
+        Requires a backend with capture_begin / capture_end (the "hip" device)."""
+        if not hasattr(self.backend, "capture_begin"):
+            raise RuntimeError(f"device {self.allocator.device!r} cannot record graphs")
+        self.backend.capture_begin()
+        try:
+            fn()
+        except BaseException:
+            try:
+                self.backend.capture_end()
+            except Exception:
+                pass
+            raise
+        return CapturedGraph(self.backend, self.backend.capture_end())
 
     def release(self):
         """return the arena and the parameter slabs to the device"""

@@ -20,6 +20,8 @@ data already resident in HBM.  Prints ONE JSON line:
   cpu_baseline     the numpy restatement of the reference's CPU kernels, timed
                    on this host with the reference's protocol (2 warm-up + 5
                    timed passes, timing_ops.py:76-100)
+  graph_replay     the launch-bound chain of config 0 launched op by op and
+                   replayed from a recorded device graph
   all_configs      the same per-op table for the other configurations
 
 All device calls go through the C ABI (autograd_amd/capi.py).
@@ -438,6 +440,43 @@ def run_workload(ctx, cfg, steps, warmup, iters, exact=False):
     return cases, step_bytes, wall
 
 
+def graph_replay(ctx, cfg, iters=200):
+    """The launch-bound chain (a few MB per op): every op of `cfg` forward then
+    backward, launched one by one and replayed from a recorded graph."""
+    pool = Pool(ctx, cfg.seed)
+    try:
+        cases = [c for c in build_cases(ctx, cfg, pool) if c.direction in ("fwd", "bwd")]
+        chain = [c for c in cases if c.direction == "fwd"] + [c for c in reversed(cases) if c.direction == "bwd"]
+
+        def step():
+            for c in chain:
+                c.launch(0)
+
+        for _ in range(3):
+            step()
+        ctx.synchronize()
+        ctx.call("agrad_graph_begin")
+        step()
+        gid = C.c_uint64(0)
+        ctx.call("agrad_graph_end", C.byref(gid))
+        out = {}
+        for name, fn in (("eager_us", step), ("graph_us", lambda: ctx.call("agrad_graph_launch", gid.value))):
+            for _ in range(5):
+                fn()
+            ctx.synchronize()
+            ctx.timer_start()
+            for _ in range(iters):
+                fn()
+            out[name] = round(ctx.timer_stop() * 1e3 / iters, 2)
+        ctx.synchronize()
+        ctx.call("agrad_graph_destroy", gid.value)
+        out["workload"] = f"configs[{cfg.index}] {cfg.name}: {len(chain)} ops forward then backward, one set of buffers"
+        out["speedup"] = round(out["eager_us"] / out["graph_us"], 2)
+        return out
+    finally:
+        pool.release()
+
+
 # ---------------------------------------------------------------------------------
 # CPU baseline: the numpy restatement of the reference's CPU kernels (oracle/),
 # imported here only, as the thing that is timed beside the GPU numbers.
@@ -582,6 +621,7 @@ def main():
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(cfg)
     if not args.workload_only:
+        result["graph_replay"] = graph_replay(ctx, CONFIGS[0])
         others = {}
         for other in CONFIGS:
             if other.index != cfg.index:

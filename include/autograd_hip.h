@@ -97,6 +97,21 @@ const char* agrad_kernel_name(int index);
 /* Human-readable "buffers | args" description of a kernel, or NULL.          */
 const char* agrad_kernel_signature(const char* name);
 
+/* ---- graphs -----------------------------------------------------------------
+ * Launch-bound chains (ops of a few MB, where the ~4 us per launch dominates) can
+ * be recorded once and replayed as one submission.  Between agrad_graph_begin
+ * and agrad_graph_end every launch on the context's stream is recorded instead
+ * of run; calls that wait for the GPU (synchronize, end_pass, host copies,
+ * timers, free) fail with AGRAD_EINVAL, as does an embedding backward too large
+ * for the one-launch sort.  Run the chain once eagerly first (kernels are loaded
+ * on first use).  The recorded launches keep their addresses and sizes: replay
+ * with the same buffers.  No counterpart in the reference (Metal command buffers
+ * are re-encoded every pass, metal_ext.mm:202-213). */
+int agrad_graph_begin(agrad_ctx* ctx);
+int agrad_graph_end(agrad_ctx* ctx, uint64_t* graph_id);
+int agrad_graph_launch(agrad_ctx* ctx, uint64_t graph_id);
+int agrad_graph_destroy(agrad_ctx* ctx, uint64_t graph_id);
+
 /* ---- typed entry points (device addresses, already offset) ----------------
  * `dtype` is the storage type of activations / gradients / embedding tables;
  * gamma, beta, dgamma, dbeta, cos, sin are always fp32; ids are int32.       */

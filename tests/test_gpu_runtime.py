@@ -345,3 +345,63 @@ def test_add_with_a_broadcast_operand():
     assert_fp32_close(h_g["x"], c_g["x"], "x.grad")
     assert_fp32_close(h_g["tab"], c_g["tab"], "tab.grad", atol=4e-6)
     assert_fp32_close(h_g["bias"], c_g["bias"], "bias.grad", atol=2e-5)
+
+
+def test_captured_graph_replays_match_eager():
+    """Record forward + zero_grad + upstream copy + backward of the tiny GPT-2 chain
+    once, replay it several times with eager work and synchronisations in between,
+    and compare every replay with the eager result bit for bit."""
+    rng = np.random.default_rng(SEED + 40)
+    B, T, C, V = 4, 32, 64, 500
+    ids_np = rng.integers(0, V, (B, T), dtype=np.int32)
+    dev = "hip"
+    rt = Runtime(device=dev)
+    ids = make_tensor(ids_np.shape, np.int32, dev, False, ids_np)
+    wte = make_tensor((V, C), np.float32, dev, True, (0.5 * rng.standard_normal((V, C))).astype(np.float32))
+    wpe = make_tensor((T, C), np.float32, dev, True, (0.5 * rng.standard_normal((T, C))).astype(np.float32))
+    g = make_tensor((C,), np.float32, dev, True, (1 + 0.1 * rng.standard_normal(C)).astype(np.float32))
+    b = make_tensor((C,), np.float32, dev, True, (0.1 * rng.standard_normal(C)).astype(np.float32))
+    up = make_tensor((B, T, C), np.float32, dev, False, rng.standard_normal((B, T, C)).astype(np.float32))
+    out = GELUOp()(LayerNormOp(eps=1e-5)(EmbeddingSumOp()(ids, wte, wpe), g, b))
+    rt.loss = out
+    rt.build_topo(out)
+    rt.bind_memory()
+    up.storage = rt.allocator.alloc(up.shape, up.dtype)
+    rt.backend.init(up)
+
+    def step():
+        rt.forward()
+        rt.zero_grad()
+        rt.backend._launch("copy_kernel", [up, out.grad], [up.numel * 4, 0])   # device-side upstream gradient
+        rt.backward_graph()
+
+    def read():
+        rt.backend.synchronize()
+        return [rt.backend.copy_to_host(t).copy() for t in (out, wte.grad, wpe.grad, g.grad, b.grad)]
+
+    step()
+    eager = read()
+    graph = rt.capture(step)
+    for replay in range(3):
+        # eager work between replays: scribble over the outputs and the gradients
+        for t in (out, wte.grad, g.grad):
+            rt.backend.fill(t, float(replay + 1))
+        rt.backend.synchronize()
+        graph.launch()
+        got = read()
+        for a, e in zip(got, eager):
+            np.testing.assert_array_equal(a, e, err_msg=f"replay {replay}")
+    # calls that wait for the GPU are refused while recording, and the recording survives that
+    rt.backend.capture_begin()
+    with pytest.raises((RuntimeError, ValueError)):
+        rt.backend.ctx.synchronize()
+    rt.forward()
+    g2 = rt.backend.capture_end()
+    rt.backend.graph_launch(g2)
+    rt.backend.synchronize()
+    np.testing.assert_array_equal(rt.backend.copy_to_host(out), eager[0])
+    rt.backend.graph_destroy(g2)
+    graph.destroy()
+    with pytest.raises(RuntimeError):
+        graph.launch()
+    rt.release()
