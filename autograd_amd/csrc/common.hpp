@@ -194,9 +194,11 @@ __device__ __forceinline__ void wave_sum2(float& a, float& b) { lanes_sum2<kWave
 // Sum over the TPR threads that share one row.  TPR <= 64: pure DPP.  TPR > 64:
 // each wave's total is staged in LDS and every thread adds the staged totals in
 // wave order.  `slot` selects one of a few LDS lines so that consecutive
-// reductions need only one barrier each (a slot is 2*TPR/64 floats; rotate at
-// least two slots).  Callers with TPR > 64 run exactly one row per workgroup, so
+// reductions need only one barrier each (a slot is kRowSumSlot*TPR/64 floats;
+// rotate at least two slots).  Callers with TPR > 64 run exactly one row per workgroup, so
 // the barrier is reached by the whole workgroup.
+constexpr int kRowSumSlot = 3;   // values one reduction may stage per wave
+
 template <int TPR>
 __device__ __forceinline__ float row_sum(float v, float* lds, int slot) {
     if constexpr (TPR <= kWave) {
@@ -204,7 +206,7 @@ __device__ __forceinline__ float row_sum(float v, float* lds, int slot) {
     } else {
         v = wave_sum(v);
         constexpr int NW = TPR / kWave;
-        float* line = lds + slot * 2 * NW;
+        float* line = lds + slot * kRowSumSlot * NW;
         if ((threadIdx.x & (kWave - 1)) == 0) line[threadIdx.x / kWave] = v;
         __syncthreads();
         float t = line[0];
@@ -221,7 +223,7 @@ __device__ __forceinline__ void row_sum2(float& a, float& b, float* lds, int slo
     } else {
         wave_sum2(a, b);
         constexpr int NW = TPR / kWave;
-        float* line = lds + slot * 2 * NW;
+        float* line = lds + slot * kRowSumSlot * NW;
         if ((threadIdx.x & (kWave - 1)) == 0) {
             line[threadIdx.x / kWave] = a;
             line[NW + threadIdx.x / kWave] = b;
@@ -231,6 +233,30 @@ __device__ __forceinline__ void row_sum2(float& a, float& b, float* lds, int slo
 #pragma unroll
         for (int w = 1; w < NW; ++w) { ta = ta + line[w]; tb = tb + line[NW + w]; }
         a = ta; b = tb;
+    }
+}
+
+// three sums in one phase (one barrier when TPR > 64)
+template <int TPR>
+__device__ __forceinline__ void row_sum3(float& a, float& b, float& c, float* lds, int slot) {
+    if constexpr (TPR <= kWave) {
+        lanes_sum2<TPR>(a, b);
+        c = lanes_sum<TPR>(c);
+    } else {
+        wave_sum2(a, b);
+        c = wave_sum(c);
+        constexpr int NW = TPR / kWave;
+        float* line = lds + slot * kRowSumSlot * NW;
+        if ((threadIdx.x & (kWave - 1)) == 0) {
+            line[threadIdx.x / kWave] = a;
+            line[NW + threadIdx.x / kWave] = b;
+            line[2 * NW + threadIdx.x / kWave] = c;
+        }
+        __syncthreads();
+        float ta = line[0], tb = line[NW], tc = line[2 * NW];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) { ta = ta + line[w]; tb = tb + line[NW + w]; tc = tc + line[2 * NW + w]; }
+        a = ta; b = tb; c = tc;
     }
 }
 

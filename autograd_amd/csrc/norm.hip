@@ -164,7 +164,7 @@ __global__ void __launch_bounds__(TPR >= 128 ? TPR : kFwdGroupBlock)
 norm_fwd_kernel(const NormFwdArgs<T> a) {
     constexpr int BLOCK = TPR >= 128 ? TPR : kFwdGroupBlock;
     constexpr int RPB = BLOCK / TPR;
-    __shared__ float lds[3 * 2 * (TPR > kWave ? TPR / kWave : 1)];
+    __shared__ float lds[3 * kRowSumSlot * (TPR > kWave ? TPR / kWave : 1)];
 
     const int sub = threadIdx.x / TPR;
     const int lane = threadIdx.x % TPR;
@@ -263,7 +263,7 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
     constexpr int BLOCK = TPR >= 128 ? TPR : 256;
     constexpr int RPB = BLOCK / TPR;
     constexpr int NWAVES = BLOCK / kWave;
-    __shared__ float lds[3 * 2 * (TPR > kWave ? TPR / kWave : 1)];
+    __shared__ float lds[3 * kRowSumSlot * (TPR > kWave ? TPR / kWave : 1)];
     extern __shared__ float comb[];  // (NWAVES - 1) * C floats when RPB > 1
 
     const int sub = threadIdx.x / TPR;
@@ -327,8 +327,10 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
             }
         }
 
-        // recompute the row statistics; xv becomes x_hat
-        float scale;
+        // Row statistics and the two row sums of the dx formula in ONE reduction
+        // phase (after the mean, for LayerNorm).  With d = x - mean (or x):
+        //   q = sum d^2,   s1 = sum dy*gamma,   s2r = sum dy*gamma*d,
+        // and sum dy*gamma*x_hat = s2r * scale.  xv becomes d, then x_hat.
         if (is_ln) {
             float s = 0.0f;
 #pragma unroll
@@ -336,28 +338,27 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
 #pragma unroll
                 for (int k = 0; k < VEC; ++k) s = s + xv[i][k];
             const float mean = row_sum<TPR>(s, lds, ring.next()) / fC;
-            float q = 0.0f;
 #pragma unroll
             for (int i = 0; i < NV; ++i)
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) {
-                    const float d = on[i] ? (xv[i][k] - mean) : 0.0f;
-                    xv[i][k] = d;
-                    q = q + d * d;
-                }
-            const float var = row_sum<TPR>(q, lds, ring.next()) / fC;
-            scale = 1.0f / sqrtf(var + a.eps);
-        } else {
-            float q = 0.0f;
-#pragma unroll
-            for (int i = 0; i < NV; ++i)
-#pragma unroll
-                for (int k = 0; k < VEC; ++k) q = q + xv[i][k] * xv[i][k];
-            const float ms = row_sum<TPR>(q, lds, ring.next()) / fC;
-            scale = 1.0f / sqrtf(ms + a.eps);
+                for (int k = 0; k < VEC; ++k) xv[i][k] = on[i] ? (xv[i][k] - mean) : 0.0f;
         }
+        float q = 0.0f, s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                const float d = xv[i][k];
+                q = q + d * d;
+                const float dyg = g[i][k] * gam[i][k];
+                s1 = s1 + dyg;
+                s2 = s2 + dyg * d;
+            }
+        if (a.dx != nullptr) row_sum3<TPR>(q, s1, s2, lds, ring.next());
+        else q = row_sum<TPR>(q, lds, ring.next());
+        const float scale = 1.0f / sqrtf(q / fC + a.eps);
+        s2 = s2 * scale;
 
-        float s1 = 0.0f, s2 = 0.0f;
 #pragma unroll
         for (int i = 0; i < NV; ++i)
 #pragma unroll
@@ -366,20 +367,16 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
                 xv[i][k] = xh;
                 if (want_pg) pg[i][k] = pg[i][k] + g[i][k] * xh;
                 if (want_pb) pb[i][k] = pb[i][k] + g[i][k];
-                const float dyg = g[i][k] * gam[i][k];
-                g[i][k] = dyg;
-                s1 = s1 + dyg;
-                s2 = s2 + dyg * xh;
+                g[i][k] = g[i][k] * gam[i][k];
             }
 
         if (a.dx != nullptr) {
             float c1 = 0.0f, c2;
             if (is_ln) {
-                row_sum2<TPR>(s1, s2, lds, ring.next());
                 c1 = (s1 / fC) * scale;
                 c2 = (s2 / fC) * scale;
             } else {
-                c2 = row_sum<TPR>(s2, lds, ring.next()) / fC;
+                c2 = s2 / fC;
             }
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
@@ -513,7 +510,7 @@ __device__ __forceinline__ float generic_row_value(const NormFwdArgs<T>& a, uint
 
 template <typename T>
 __global__ void __launch_bounds__(256) norm_fwd_generic_kernel(const NormFwdArgs<T> a) {
-    __shared__ float lds[3 * 2 * 4];
+    __shared__ float lds[3 * kRowSumSlot * 4];
     const uint32_t C = a.C;
     const float fC = (float)C;
     const uint64_t base = (uint64_t)blockIdx.x * C;
@@ -548,7 +545,7 @@ __global__ void __launch_bounds__(256) norm_fwd_generic_kernel(const NormFwdArgs
 
 template <typename T>
 __global__ void __launch_bounds__(256) norm_bwd_generic_kernel(const NormBwdArgs<T> a) {
-    __shared__ float lds[3 * 2 * 4];
+    __shared__ float lds[3 * kRowSumSlot * 4];
     const uint32_t C = a.C;
     const float fC = (float)C;
     const bool is_ln = a.kind == AGRAD_NORM_LAYER;

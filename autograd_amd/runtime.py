@@ -399,9 +399,17 @@ class Runtime:
         self.backend.fill(self.loss.grad, self.grad_scale)
         self.backward_graph()
 
+    def _sync_backend(self):
+        """the backend is one object per device, shared by every Runtime: before this
+        runtime launches anything it puts its own settings there"""
+        self.backend.accumulate_parameter_grads = self.accumulate_parameter_grads
+        self.backend.grad_scale = self.grad_scale
+        self.backend.use_fp16_gemm = self.use_fp16_gemm
+
     def zero_grad(self):
         """zero the parameter gradients, except those whose first backward kernel
         stores the whole tensor anyway"""
+        self._sync_backend()
         seen = set()
         for node in self.topo:
             for t in node.inputs + node.outputs:
@@ -414,12 +422,14 @@ class Runtime:
                     self.backend.fill(t.grad, 0)
 
     def forward(self):
+        self._sync_backend()
         self.backend.begin_pass()
         for node in self.topo:
             node.forward(node.inputs, node.outputs)
         self.backend.end_pass()
 
     def backward_graph(self):
+        self._sync_backend()
         self.backend.begin_pass()
         for node in reversed(self.topo):
             for t in self.node_to_clear_grads.get(id(node), ()):
