@@ -579,17 +579,13 @@ bool group_sort_enabled() {
     return on;
 }
 
-struct EmbPlan {
-    uint32_t L, chunks;
-    uint64_t off_keys_in, off_keys_out, off_vals_in, off_vals_out, off_temp, temp_bytes, off_head,
-        off_tail, total;
+// Scratch of the ordering step: input key / value arrays of the radix path (the
+// grouping sort uses the same bytes as N 64-bit spill slots) and rocPRIM's temp.
+struct SortPlan {
+    uint64_t off_keys_in, off_vals_in, off_temp, temp_bytes, total;
 };
 
-int plan_embedding(uint64_t N, uint32_t C, uint32_t V, EmbPlan* p) {
-    uint32_t per = (uint32_t)((N + (uint64_t)kBatch * kMaxChunks - 1) / ((uint64_t)kBatch * kMaxChunks));
-    if (per == 0) per = 1;
-    p->L = kBatch * per;
-    p->chunks = (uint32_t)((N + p->L - 1) / p->L);
+int plan_sort(uint64_t N, uint32_t V, SortPlan* p) {
     size_t temp = 0;
     uint32_t* nil = nullptr;
     int bits = 1;
@@ -601,49 +597,36 @@ int plan_embedding(uint64_t N, uint32_t C, uint32_t V, EmbPlan* p) {
     // keys_in and vals_in are adjacent: the grouping sort uses the pair as N 64-bit spill slots
     p->off_keys_in = o;  o += align256(N * 4);
     p->off_vals_in = o;  o += align256(N * 4);
-    p->off_keys_out = o; o += align256(N * 4);
-    p->off_vals_out = o; o += align256(N * 4);
     p->off_temp = o;     o += align256(temp);
     p->temp_bytes = temp;
-    p->off_head = o;     o += align256((uint64_t)p->chunks * C * 4);
-    p->off_tail = o;     o += align256((uint64_t)p->chunks * C * 4);
     p->total = o;
     return AGRAD_OK;
 }
 
+// Scratch of the summing step: one head and one tail carry row per chunk.
+struct SumPlan {
+    uint32_t L, chunks;
+    uint64_t off_head, off_tail, total;
+};
+
+void plan_sum(uint64_t N, uint32_t C, SumPlan* p) {
+    uint32_t per = (uint32_t)((N + (uint64_t)kBatch * kMaxChunks - 1) / ((uint64_t)kBatch * kMaxChunks));
+    if (per == 0) per = 1;
+    p->L = kBatch * per;
+    p->chunks = (uint32_t)((N + p->L - 1) / p->L);
+    uint64_t o = 0;
+    p->off_head = o;     o += align256((uint64_t)p->chunks * C * 4);
+    p->off_tail = o;     o += align256((uint64_t)p->chunks * C * 4);
+    p->total = o;
+}
+
+inline uint64_t order_bytes(uint64_t N) { return align256(N * 8); }   // tok_s[N] then row_s[N]
+
 template <typename T>
-int embedding_bwd_typed(hipStream_t s, const EmbPlan& p, const int32_t* ids, const T* dY, T* dW,
-                        uint8_t* ws, uint32_t N, uint32_t C, uint32_t V, uint32_t flags, int* err_flag) {
-    uint32_t* keys_in = (uint32_t*)(ws + p.off_keys_in);
-    uint32_t* keys_out = (uint32_t*)(ws + p.off_keys_out);
-    uint32_t* vals_in = (uint32_t*)(ws + p.off_vals_in);
-    uint32_t* vals_out = (uint32_t*)(ws + p.off_vals_out);
+int embedding_sum_typed(hipStream_t s, const SumPlan& p, const uint32_t* tok_s, const uint32_t* row_s, const T* dY,
+                        T* dW, uint8_t* ws, uint32_t N, uint32_t C, uint32_t V, uint32_t flags) {
     float* head = (float*)(ws + p.off_head);
     float* tail = (float*)(ws + p.off_tail);
-
-    bool grouped = false;
-    if (N <= kGroupSortMaxN && group_sort_enabled()) {
-        // keys_in / vals_in are adjacent and unused on this path: together they hold N 64-bit spill slots
-        static_assert(sizeof(unsigned long long) == 2 * sizeof(uint32_t), "spill layout");
-        unsigned long long* spill = reinterpret_cast<unsigned long long*>(ws + p.off_keys_in);
-        const uint32_t log2G = N > 1024 ? 8u : 4u;
-        hipLaunchKernelGGL(emb_group_sort_kernel, dim3(1u << log2G), dim3(kSortBlock), 0, s, ids, keys_out, vals_out,
-                           spill, N, V, log2G, err_flag);
-        grouped = true;
-    }
-    if (!grouped) {
-        if (is_capturing())
-            return set_error(AGRAD_EINVAL, "embedding backward over %u rows uses the library radix sort, which is not "
-                             "recorded into graphs (up to %u rows are)", N, kGroupSortMaxN);
-        hipLaunchKernelGGL(emb_prepare_kernel, dim3((N + 255) / 256), dim3(256), 0, s, ids, keys_in, vals_in, N, V, err_flag);
-        int bits = 1;
-        while ((1ull << bits) <= V) ++bits;
-        size_t temp = p.temp_bytes;
-        hipError_t err = rocprim::radix_sort_pairs(ws + p.off_temp, temp, keys_in, keys_out, vals_in, vals_out,
-                                                   (size_t)N, 0u, (unsigned)bits, s, false);
-        if (err != hipSuccess) return check_hip(err, "radix sort");
-    }
-
     const int acc = (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0;
     constexpr int WIDE = WideVec<T>::value;
     const bool wide = C % WIDE == 0 && aligned16(dY) && aligned16(dW);
@@ -651,22 +634,104 @@ int embedding_bwd_typed(hipStream_t s, const EmbPlan& p, const int32_t* ids, con
         const uint32_t CV = C / WIDE;
         uint32_t block = ((CV + 63) / 64) * 64;
         if (block > 512) block = 512;
-        hipLaunchKernelGGL((emb_segment_sum_kernel<T, WIDE>), dim3(p.chunks), dim3(block), 0, s, keys_out,
-                           vals_out, dY, dW, head, tail, N, C, CV, V, p.L, acc);
+        hipLaunchKernelGGL((emb_segment_sum_kernel<T, WIDE>), dim3(p.chunks), dim3(block), 0, s, tok_s,
+                           row_s, dY, dW, head, tail, N, C, CV, V, p.L, acc);
         hipLaunchKernelGGL((emb_carry_fix_kernel<T, WIDE>), dim3(p.chunks), dim3(kFixCols * kFixLanes), 0, s,
-                           keys_out, dW, head, tail, N, C, CV, V, p.L, acc);
+                           tok_s, dW, head, tail, N, C, CV, V, p.L, acc);
     } else {
         uint32_t block = ((C + 63) / 64) * 64;
-        if (block > 256) block = 256;
-        hipLaunchKernelGGL((emb_segment_sum_kernel<T, 1>), dim3(p.chunks), dim3(block), 0, s, keys_out,
-                           vals_out, dY, dW, head, tail, N, C, C, V, p.L, acc);
+        if (block > 512) block = 512;
+        hipLaunchKernelGGL((emb_segment_sum_kernel<T, 1>), dim3(p.chunks), dim3(block), 0, s, tok_s,
+                           row_s, dY, dW, head, tail, N, C, C, V, p.L, acc);
         hipLaunchKernelGGL((emb_carry_fix_kernel<T, 1>), dim3(p.chunks), dim3(kFixCols * kFixLanes), 0, s,
-                           keys_out, dW, head, tail, N, C, C, V, p.L, acc);
+                           tok_s, dW, head, tail, N, C, C, V, p.L, acc);
     }
     return check_hip(hipGetLastError(), "embedding backward launch");
 }
 
+int check_embedding_sizes(const char* what, uint64_t N, uint32_t V) {
+    if (N >= 0x7fffffffull) return set_error(AGRAD_EINVAL, "%s: too many rows", what);
+    if (V == 0 || V >= 0x7fffffffu) return set_error(AGRAD_EINVAL, "%s: bad vocabulary size %u", what, V);
+    return AGRAD_OK;
+}
+
 }  // namespace
+
+uint64_t embedding_order_bytes(uint64_t N) { return N ? order_bytes(N) : 0; }
+
+uint64_t embedding_sort_workspace_bytes(uint64_t N, uint32_t V) {
+    if (N == 0) return 0;
+    SortPlan p;
+    if (plan_sort(N, V, &p) != AGRAD_OK) return 0;
+    return p.total;
+}
+
+// order[0 .. N) = tokens, order[N .. 2N) = rows: each token's rows adjacent, ascending
+int launch_embedding_sort(hipStream_t s, const int32_t* ids, uint32_t* order, void* workspace,
+                          uint64_t workspace_bytes, uint64_t N, uint32_t V, int* err_flag) {
+    if (N == 0) return AGRAD_OK;
+    if (int rc = check_embedding_sizes("embedding sort", N, V)) return rc;
+    if (ids == nullptr || order == nullptr) return set_error(AGRAD_EINVAL, "embedding sort: null operand");
+    SortPlan p;
+    if (int rc = plan_sort(N, V, &p)) return rc;
+    if (workspace == nullptr || workspace_bytes < p.total)
+        return set_error(AGRAD_EWORKSPACE, "embedding sort: workspace %llu < %llu bytes",
+                         (unsigned long long)workspace_bytes, (unsigned long long)p.total);
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
+        return set_error(AGRAD_EINVAL, "embedding sort: workspace must be 256-byte aligned");
+    uint8_t* ws = (uint8_t*)workspace;
+    uint32_t* tok_s = order;
+    uint32_t* row_s = order + N;
+    const uint32_t n = (uint32_t)N;
+    if (n <= kGroupSortMaxN && group_sort_enabled()) {
+        static_assert(sizeof(unsigned long long) == 2 * sizeof(uint32_t), "spill layout");
+        unsigned long long* spill = reinterpret_cast<unsigned long long*>(ws + p.off_keys_in);
+        const uint32_t log2G = n > 1024 ? 8u : 4u;
+        hipLaunchKernelGGL(emb_group_sort_kernel, dim3(1u << log2G), dim3(kSortBlock), 0, s, ids, tok_s, row_s,
+                           spill, n, V, log2G, err_flag);
+        return check_hip(hipGetLastError(), "embedding sort launch");
+    }
+    if (is_capturing())
+        return set_error(AGRAD_EINVAL, "an embedding gradient over %u rows uses the library radix sort, which is not "
+                         "recorded into graphs (up to %u rows are)", n, kGroupSortMaxN);
+    uint32_t* keys_in = (uint32_t*)(ws + p.off_keys_in);
+    uint32_t* vals_in = (uint32_t*)(ws + p.off_vals_in);
+    hipLaunchKernelGGL(emb_prepare_kernel, dim3((n + 255) / 256), dim3(256), 0, s, ids, keys_in, vals_in, n, V, err_flag);
+    int bits = 1;
+    while ((1ull << bits) <= V) ++bits;
+    size_t temp = p.temp_bytes;
+    hipError_t err = rocprim::radix_sort_pairs(ws + p.off_temp, temp, keys_in, tok_s, vals_in, row_s,
+                                               (size_t)N, 0u, (unsigned)bits, s, false);
+    return check_hip(err, "radix sort");
+}
+
+uint64_t embedding_bwd_sorted_workspace_bytes(uint64_t N, uint32_t C) {
+    if (N == 0 || C == 0) return 0;
+    SumPlan p;
+    plan_sum(N, C, &p);
+    return p.total;
+}
+
+int launch_embedding_bwd_sorted(hipStream_t s, int dtype, const uint32_t* order, const void* dY, void* dW,
+                                void* workspace, uint64_t workspace_bytes, uint64_t N, uint32_t C,
+                                uint32_t V, uint32_t flags) {
+    if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "embedding backward: unknown dtype %d", dtype);
+    if (N == 0 || C == 0) return AGRAD_OK;
+    if (int rc = check_embedding_sizes("embedding backward", N, V)) return rc;
+    if (order == nullptr || dY == nullptr || dW == nullptr) return set_error(AGRAD_EINVAL, "embedding backward: null operand");
+    SumPlan p;
+    plan_sum(N, C, &p);
+    if (workspace == nullptr || workspace_bytes < p.total)
+        return set_error(AGRAD_EWORKSPACE, "embedding backward: workspace %llu < %llu bytes",
+                         (unsigned long long)workspace_bytes, (unsigned long long)p.total);
+    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
+        return set_error(AGRAD_EINVAL, "embedding backward: workspace must be 256-byte aligned");
+    if (dtype == AGRAD_F32)
+        return embedding_sum_typed<float>(s, p, order, order + N, (const float*)dY, (float*)dW, (uint8_t*)workspace,
+                                          (uint32_t)N, C, V, flags);
+    return embedding_sum_typed<bf16_t>(s, p, order, order + N, (const bf16_t*)dY, (bf16_t*)dW, (uint8_t*)workspace,
+                                       (uint32_t)N, C, V, flags);
+}
 
 int launch_gather_fwd(hipStream_t s, int dtype, const int32_t* ids, const void* W, const void* wpe,
                       void* out, uint64_t N, uint32_t T, uint32_t C, uint32_t V, int* err_flag) {
@@ -708,12 +773,11 @@ int launch_gather_fwd(hipStream_t s, int dtype, const int32_t* ids, const void* 
     return check_hip(hipGetLastError(), "gather launch");
 }
 
+// one workspace for the unsorted entry point: [order | sort scratch | carry rows]
 uint64_t embedding_bwd_workspace_bytes(uint64_t N, uint32_t C, uint32_t V, int dtype) {
     (void)dtype;
     if (N == 0 || C == 0) return 0;
-    EmbPlan p;
-    if (plan_embedding(N, C, V, &p) != AGRAD_OK) return 0;
-    return p.total;
+    return order_bytes(N) + embedding_sort_workspace_bytes(N, V) + embedding_bwd_sorted_workspace_bytes(N, C);
 }
 
 int launch_embedding_bwd(hipStream_t s, int dtype, const int32_t* ids, const void* dY, void* dW,
@@ -722,20 +786,19 @@ int launch_embedding_bwd(hipStream_t s, int dtype, const int32_t* ids, const voi
     if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "embedding backward: unknown dtype %d", dtype);
     if (N == 0 || C == 0) return AGRAD_OK;
     if (ids == nullptr || dY == nullptr || dW == nullptr) return set_error(AGRAD_EINVAL, "embedding backward: null operand");
-    if (N >= 0x7fffffffull) return set_error(AGRAD_EINVAL, "embedding backward: too many rows");
-    if (V == 0 || V >= 0x7fffffffu) return set_error(AGRAD_EINVAL, "embedding backward: bad vocabulary size %u", V);
-    EmbPlan p;
-    if (int rc = plan_embedding(N, C, V, &p)) return rc;
-    if (workspace == nullptr || workspace_bytes < p.total)
+    if (int rc = check_embedding_sizes("embedding backward", N, V)) return rc;
+    const uint64_t sort_bytes = embedding_sort_workspace_bytes(N, V);
+    const uint64_t sum_bytes = embedding_bwd_sorted_workspace_bytes(N, C);
+    const uint64_t need = order_bytes(N) + sort_bytes + sum_bytes;
+    if (workspace == nullptr || workspace_bytes < need)
         return set_error(AGRAD_EWORKSPACE, "embedding backward: workspace %llu < %llu bytes",
-                         (unsigned long long)workspace_bytes, (unsigned long long)p.total);
+                         (unsigned long long)workspace_bytes, (unsigned long long)need);
     if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
         return set_error(AGRAD_EINVAL, "embedding backward: workspace must be 256-byte aligned");
-    if (dtype == AGRAD_F32)
-        return embedding_bwd_typed<float>(s, p, ids, (const float*)dY, (float*)dW, (uint8_t*)workspace,
-                                          (uint32_t)N, C, V, flags, err_flag);
-    return embedding_bwd_typed<bf16_t>(s, p, ids, (const bf16_t*)dY, (bf16_t*)dW, (uint8_t*)workspace,
-                                       (uint32_t)N, C, V, flags, err_flag);
+    uint8_t* ws = (uint8_t*)workspace;
+    uint32_t* order = (uint32_t*)ws;
+    if (int rc = launch_embedding_sort(s, ids, order, ws + order_bytes(N), sort_bytes, N, V, err_flag)) return rc;
+    return launch_embedding_bwd_sorted(s, dtype, order, dY, dW, ws + order_bytes(N) + sort_bytes, sum_bytes, N, C, V, flags);
 }
 
 int launch_pos_embedding_bwd(hipStream_t s, int dtype, const void* dY, void* dwpe, uint32_t B,
