@@ -222,7 +222,11 @@ class HipBackend(Backend):
         if isinstance(op, (GatherOp, EmbeddingSumOp)):
             ids, w = node.inputs[0], node.inputs[1]
             if w.requires_grad:
-                nbytes = self.ctx.embedding_backward_workspace_bytes(prod(ids.shape), w.shape[1], w.shape[0], _dt(w))
+                n = prod(ids.shape)
+                if len(node.outputs) > 1:
+                    return (single_slot("sort_workspace", self.ctx.embedding_sort_workspace_bytes(n, w.shape[0])),
+                            single_slot("workspace", self.ctx.embedding_backward_sorted_workspace_bytes(n, w.shape[1])))
+                nbytes = self.ctx.embedding_backward_workspace_bytes(n, w.shape[1], w.shape[0], _dt(w))
                 return None, single_slot("workspace", nbytes)
         return None, None
 
@@ -272,31 +276,49 @@ class HipBackend(Backend):
                 raise RuntimeError(f"Unsupported Add backward shape: {t.shape} from {out.shape}")
 
     # -- embedding (backend.py:525-538, 2777-2815) ----------------------------------
-    def hip_gather_forward(self, inputs, outputs, scratch=None):
-        indices, weight, out = inputs[0], inputs[1], outputs[0]
-        V, C = weight.shape
-        self._launch("gather_forward_kernel", [indices, weight, out], [_dt(weight), prod(indices.shape), C, V])
+    # When the table needs a gradient the op carries an `order` output: the forward
+    # kernel then also orders the ids (one launch, beside the gather) and the
+    # backward kernel starts at the segmented sum.
+    def _embedding_forward(self, indices, table, wpe, outputs, scratch):
+        out = outputs[0]
+        V, C = table.shape
+        B, T = indices.shape
+        if len(outputs) > 1:
+            if scratch is None:
+                raise RuntimeError("embedding forward needs its arena workspace (plan_scratch)")
+            ws = scratch["sort_workspace"]
+            self._launch("gather_forward_sorted", [indices, table, wpe, out, outputs[1], ws],
+                         [_dt(table), B * T, T, C, V] + _lo_hi(ws.nbytes) + [_mask(indices, table, wpe, out, outputs[1], ws)])
+        elif wpe is None:
+            self._launch("gather_forward_kernel", [indices, table, out], [_dt(table), B * T, C, V])
+        else:
+            self._launch("embedding_sum_forward", [indices, table, wpe, out], [_dt(table), B * T, T, C, V])
 
-    def _embedding_grad(self, node, indices, weight, out, scratch):
+    def _embedding_grad(self, node, indices, weight, outputs, scratch):
         if scratch is None:
             raise RuntimeError("embedding backward needs its arena workspace (plan_scratch)")
+        out = outputs[0]
         ws = scratch["workspace"]
         V, C = weight.shape
-        self._launch("gather_backward_kernel", [indices, out.grad, weight.grad, ws],
-                     [_dt(weight), prod(indices.shape), C, V, self._param_flag(node, weight)] + _lo_hi(ws.nbytes))
+        flag = self._param_flag(node, weight)
+        if len(outputs) > 1:
+            self._launch("gather_backward_sorted", [outputs[1], out.grad, weight.grad, ws],
+                         [_dt(weight), prod(indices.shape), C, V, flag] + _lo_hi(ws.nbytes))
+        else:
+            self._launch("gather_backward_kernel", [indices, out.grad, weight.grad, ws],
+                         [_dt(weight), prod(indices.shape), C, V, flag] + _lo_hi(ws.nbytes))
+
+    def hip_gather_forward(self, inputs, outputs, scratch=None):
+        self._embedding_forward(inputs[0], inputs[1], None, outputs, scratch)
 
     def hip_gather_backward(self, inputs, outputs, scratch=None):
         indices, weight, out = inputs[0], inputs[1], outputs[0]
         if out.grad is None or not weight.requires_grad:
             return
-        self._embedding_grad(out.op, indices, weight, out, scratch)
+        self._embedding_grad(out.op, indices, weight, outputs, scratch)
 
     def hip_embedding_sum_forward(self, inputs, outputs, scratch=None):
-        indices, wte, wpe = inputs
-        out = outputs[0]
-        V, C = wte.shape
-        B, T = indices.shape
-        self._launch("embedding_sum_forward", [indices, wte, wpe, out], [_dt(wte), B * T, T, C, V])
+        self._embedding_forward(inputs[0], inputs[1], inputs[2], outputs, scratch)
 
     def hip_embedding_sum_backward(self, inputs, outputs, scratch=None):
         indices, wte, wpe = inputs
@@ -305,7 +327,7 @@ class HipBackend(Backend):
             return
         B, T = indices.shape
         if wte.requires_grad:
-            self._embedding_grad(out.op, indices, wte, out, scratch)
+            self._embedding_grad(out.op, indices, wte, outputs, scratch)
         if wpe.requires_grad:
             # rows beyond T of a longer table get no gradient
             self._launch("pos_emb_grad", [out.grad, wpe.grad],

@@ -69,6 +69,10 @@ SIGNATURES = {
     "agrad_gather_forward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u32, _u32, _u32]),
     "agrad_embedding_backward_workspace_bytes": (_u64, [_u64, _u32, _u32, _int]),
     "agrad_embedding_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u64, _u32, _u32, _u32]),
+    "agrad_embedding_sort_workspace_bytes": (_u64, [_u64, _u32]),
+    "agrad_gather_forward_sorted": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u32, _u32, _u32, _ptr, _ptr, _u64]),
+    "agrad_embedding_backward_sorted_workspace_bytes": (_u64, [_u64, _u32]),
+    "agrad_embedding_backward_sorted": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u64, _u32, _u32, _u32]),
     "agrad_pos_embedding_backward": (_int, [_ctx, _int, _ptr, _ptr, _u32, _u32, _u32, _u32]),
     "agrad_graph_begin": (_int, [_ctx]),
     "agrad_graph_end": (_int, [_ctx, C.POINTER(_u64)]),

@@ -289,6 +289,25 @@ int h_gather_bwd(const Call& c) {
     return launch_embedding_bwd(c.ctx->stream, c.a[0], (const int32_t*)ids, dY, dW, ws, ws_bytes, N, C, V,
                                 c.a[4], c.ctx->err_flag);
 }
+// buffers ids, W, wpe, out, order, sort_ws | args dtype, N, T, C, V, ws lo, hi, present_mask
+int h_gather_fwd_sorted(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t N = c.a[1], es = dtype_size(c.a[0]), wsb = u64(c.a, 5);
+    const uint32_t T = c.a[2], C = c.a[3], V = c.a[4], mask = c.a[7];
+    RESOLVE(0, N * 4, ids) RESOLVE(1, (uint64_t)V * C * es, W)
+    RESOLVE_IF(mask & 4u, 2, (uint64_t)T * C * es, wpe)
+    RESOLVE(3, N * C * es, out) RESOLVE(4, N * 8, order) RESOLVE(5, wsb, ws)
+    return launch_gather_fwd_sorted(c.ctx->stream, (int)c.a[0], (const int32_t*)ids, W, wpe, out, N, T, C, V,
+                                    (uint32_t*)order, ws, wsb, c.ctx->err_flag);
+}
+// buffers order, dY, dW, workspace | args dtype, N, C, V, flags, ws lo, hi
+int h_gather_bwd_sorted(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t N = c.a[1], es = dtype_size(c.a[0]), wsb = u64(c.a, 5);
+    const uint32_t C = c.a[2], V = c.a[3];
+    RESOLVE(0, N * 8, order) RESOLVE(1, N * C * es, dY) RESOLVE(2, (uint64_t)V * C * es, dW) RESOLVE(3, wsb, ws)
+    return launch_embedding_bwd_sorted(c.ctx->stream, (int)c.a[0], (const uint32_t*)order, dY, dW, ws, wsb, N, C, V, c.a[4]);
+}
 // buffers dY, dwpe | args dtype, B, T, C, flags
 int h_pos_grad(const Call& c) {
     NEED_DTYPE(c.a[0])
@@ -361,6 +380,8 @@ const Entry kTable[] = {
     {"gather_forward_kernel", 3, 4, "ids, W, out | dtype, N, C, V", h_gather_fwd},
     {"embedding_sum_forward", 4, 5, "ids, W, wpe, out | dtype, N, T, C, V", h_embed_sum_fwd},
     {"gather_backward_kernel", 4, 7, "ids, dY, dW, workspace | dtype, N, C, V, flags, ws_lo, ws_hi", h_gather_bwd},
+    {"gather_forward_sorted", 6, 8, "ids, W, wpe, out, order, sort_workspace | dtype, N, T, C, V, ws_lo, ws_hi, present_mask", h_gather_fwd_sorted},
+    {"gather_backward_sorted", 4, 7, "order, dY, dW, workspace | dtype, N, C, V, flags, ws_lo, ws_hi", h_gather_bwd_sorted},
     {"pos_emb_grad", 2, 5, "dY, dwpe | dtype, B, T, C, flags", h_pos_grad},
     {"cross_entropy_forward", 4, 5, "logits, labels, loss, lse | dtype, rows_lo, rows_hi, V, present_mask", h_ce_fwd},
     {"cross_entropy_backward", 5, 6, "logits, labels, dloss, lse, dlogits | dtype, rows_lo, rows_hi, V, flags, present_mask", h_ce_bwd},
@@ -709,6 +730,23 @@ int agrad_embedding_backward(agrad_ctx* ctx, int dtype, const int32_t* ids, cons
     CTX_OR_FAIL(ctx)
     return launch_embedding_bwd(ctx->stream, dtype, ids, dY, dW, workspace, workspace_bytes, N, C, V,
                                 flags, ctx->err_flag);
+}
+uint64_t agrad_embedding_sort_workspace_bytes(uint64_t N, uint32_t V) { return embedding_sort_workspace_bytes(N, V); }
+int agrad_gather_forward_sorted(agrad_ctx* ctx, int dtype, const int32_t* ids, const void* W, const void* wpe,
+                                void* out, uint64_t N, uint32_t T, uint32_t C, uint32_t V,
+                                uint32_t* order, void* sort_workspace, uint64_t sort_workspace_bytes) {
+    CTX_OR_FAIL(ctx)
+    return launch_gather_fwd_sorted(ctx->stream, dtype, ids, W, wpe, out, N, T, C, V, order, sort_workspace,
+                                    sort_workspace_bytes, ctx->err_flag);
+}
+uint64_t agrad_embedding_backward_sorted_workspace_bytes(uint64_t N, uint32_t C) {
+    return embedding_bwd_sorted_workspace_bytes(N, C);
+}
+int agrad_embedding_backward_sorted(agrad_ctx* ctx, int dtype, const uint32_t* order, const void* dY, void* dW,
+                                    void* workspace, uint64_t workspace_bytes, uint64_t N, uint32_t C,
+                                    uint32_t V, uint32_t flags) {
+    CTX_OR_FAIL(ctx)
+    return launch_embedding_bwd_sorted(ctx->stream, dtype, order, dY, dW, workspace, workspace_bytes, N, C, V, flags);
 }
 int agrad_pos_embedding_backward(agrad_ctx* ctx, int dtype, const void* dY, void* dwpe, uint32_t B,
                                  uint32_t T, uint32_t C, uint32_t flags) {

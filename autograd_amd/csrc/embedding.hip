@@ -205,14 +205,14 @@ __device__ __forceinline__ void bitonic_sort_u64(unsigned long long* keys, uint3
     }
 }
 
-__global__ void __launch_bounds__(kSortBlock)
-emb_group_sort_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ tok_s,
-                      uint32_t* __restrict__ row_s, unsigned long long* __restrict__ spill,
-                      uint32_t N, uint32_t V, uint32_t log2G, int* err_flag) {
+// the work of workgroup `g` of the grouping sort (kSortBlock threads)
+__device__ __forceinline__ void
+emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __restrict__ tok_s,
+                    uint32_t* __restrict__ row_s, unsigned long long* __restrict__ spill,
+                    uint32_t N, uint32_t V, uint32_t log2G, int* err_flag) {
     __shared__ unsigned long long keys[kSortLdsEntries];
     __shared__ uint32_t s_count, s_less;
     const uint32_t tid = threadIdx.x;
-    const uint32_t g = blockIdx.x;
     if (tid == 0) { s_count = 0; s_less = 0; }
     __syncthreads();
 
@@ -302,6 +302,52 @@ emb_group_sort_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ to
         const unsigned long long key = mine[i];
         tok_s[offset + i] = (uint32_t)(key >> 32);
         row_s[offset + i] = (uint32_t)key;
+    }
+}
+
+__global__ void __launch_bounds__(kSortBlock)
+emb_group_sort_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ tok_s,
+                      uint32_t* __restrict__ row_s, unsigned long long* __restrict__ spill,
+                      uint32_t N, uint32_t V, uint32_t log2G, int* err_flag) {
+    emb_group_sort_body(blockIdx.x, ids, tok_s, row_s, spill, N, V, log2G, err_flag);
+}
+
+// Forward gather and the ordering of the ids for the later gradient in ONE
+// launch.  The two only share their input, the gather is bound by memory
+// bandwidth and the ordering by latency, so the first `groups` workgroups do the
+// ordering (they are dispatched first and are done within a few microseconds)
+// while all the others stream table rows: the ordering then costs the backward
+// pass nothing and the forward pass next to nothing.  (Doing the same with a
+// second stream and events was measured three times more expensive than the
+// ordering itself.)  One 16-byte vector per thread; with a position table the
+// rows are added in fp32.
+template <typename T, int VEC, bool RAW>
+__global__ void __launch_bounds__(kSortBlock)
+gather_sort_kernel(const int32_t* __restrict__ ids, const T* __restrict__ W, const T* __restrict__ wpe,
+                   T* __restrict__ out, uint32_t total, uint32_t CV, uint32_t C, uint32_t T_len, uint32_t V,
+                   uint32_t* __restrict__ tok_s, uint32_t* __restrict__ row_s, unsigned long long* __restrict__ spill,
+                   uint32_t N, uint32_t log2G, int* err_flag) {
+    const uint32_t groups = 1u << log2G;
+    if (blockIdx.x < groups) {
+        emb_group_sort_body(blockIdx.x, ids, tok_s, row_s, spill, N, V, log2G, err_flag);
+        return;
+    }
+    const uint32_t idx = (blockIdx.x - groups) * kSortBlock + threadIdx.x;
+    if (idx >= total) return;
+    const uint32_t row = idx / CV;
+    const uint32_t cv = idx - row * CV;
+    const int32_t tok = ids[row];
+    if (tok < 0 || (uint32_t)tok >= V) return;      // the ordering workgroups report bad ids
+    if constexpr (RAW) {
+        const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(W) + (uint64_t)tok * CV + cv);
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(out) + idx);
+    } else {
+        float v[VEC], p[VEC];
+        VecIO<T, VEC>::load(W + (uint64_t)tok * C + cv * VEC, v);
+        VecIO<T, VEC>::load(wpe + (uint64_t)(row % T_len) * C + cv * VEC, p);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) v[k] = v[k] + p[k];
+        VecIO<T, VEC>::store(out + (uint64_t)row * C + cv * VEC, v);
     }
 }
 
@@ -703,6 +749,52 @@ int launch_embedding_sort(hipStream_t s, const int32_t* ids, uint32_t* order, vo
     hipError_t err = rocprim::radix_sort_pairs(ws + p.off_temp, temp, keys_in, tok_s, vals_in, row_s,
                                                (size_t)N, 0u, (unsigned)bits, s, false);
     return check_hip(err, "radix sort");
+}
+
+// out = W[ids] (+ wpe) and order = the ids' ordering for the later gradient
+int launch_gather_fwd_sorted(hipStream_t s, int dtype, const int32_t* ids, const void* W, const void* wpe,
+                             void* out, uint64_t N, uint32_t T, uint32_t C, uint32_t V, uint32_t* order,
+                             void* sort_workspace, uint64_t sort_workspace_bytes, int* err_flag) {
+    if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "gather: unknown dtype %d", dtype);
+    if (N == 0) return AGRAD_OK;
+    if (order == nullptr) return set_error(AGRAD_EINVAL, "gather: null order buffer");
+    const uint32_t esz = dtype_size(dtype);
+    const uint32_t per16 = 16 / esz;
+    const bool wide = C > 0 && C % per16 == 0 && W != nullptr && out != nullptr && aligned16(W) && aligned16(out) &&
+                      (!wpe || aligned16(wpe));
+    const uint64_t total_vec = wide ? N * (C / per16) : 0;
+    const bool fused = wide && N <= kGroupSortMaxN && group_sort_enabled() && total_vec < 0xff000000ull &&
+                       ids != nullptr && (wpe == nullptr || T > 0);
+    if (!fused) {
+        if (int rc = launch_embedding_sort(s, ids, order, sort_workspace, sort_workspace_bytes, N, V, err_flag)) return rc;
+        if (C == 0) return AGRAD_OK;
+        return launch_gather_fwd(s, dtype, ids, W, wpe, out, N, T, C, V, err_flag);
+    }
+    if (int rc = check_embedding_sizes("gather", N, V)) return rc;
+    SortPlan p;
+    if (int rc = plan_sort(N, V, &p)) return rc;
+    if (sort_workspace == nullptr || sort_workspace_bytes < p.total)
+        return set_error(AGRAD_EWORKSPACE, "gather: sort workspace %llu < %llu bytes",
+                         (unsigned long long)sort_workspace_bytes, (unsigned long long)p.total);
+    if ((reinterpret_cast<uintptr_t>(sort_workspace) & 255u) != 0)
+        return set_error(AGRAD_EINVAL, "gather: sort workspace must be 256-byte aligned");
+    unsigned long long* spill = reinterpret_cast<unsigned long long*>((uint8_t*)sort_workspace + p.off_keys_in);
+    const uint32_t n = (uint32_t)N, CV = C / per16, total = (uint32_t)total_vec;
+    const uint32_t log2G = n > 1024 ? 8u : 4u;
+    const uint32_t grid = (1u << log2G) + (total + kSortBlock - 1) / kSortBlock;
+    uint32_t* tok_s = order;
+    uint32_t* row_s = order + N;
+    if (wpe == nullptr) {
+        hipLaunchKernelGGL((gather_sort_kernel<float, 4, true>), dim3(grid), dim3(kSortBlock), 0, s, ids, (const float*)W,
+                           (const float*)nullptr, (float*)out, total, CV, C, T ? T : 1u, V, tok_s, row_s, spill, n, log2G, err_flag);
+    } else if (dtype == AGRAD_F32) {
+        hipLaunchKernelGGL((gather_sort_kernel<float, 4, false>), dim3(grid), dim3(kSortBlock), 0, s, ids, (const float*)W,
+                           (const float*)wpe, (float*)out, total, CV, C, T, V, tok_s, row_s, spill, n, log2G, err_flag);
+    } else {
+        hipLaunchKernelGGL((gather_sort_kernel<bf16_t, 8, false>), dim3(grid), dim3(kSortBlock), 0, s, ids, (const bf16_t*)W,
+                           (const bf16_t*)wpe, (bf16_t*)out, total, CV, C, T, V, tok_s, row_s, spill, n, log2G, err_flag);
+    }
+    return check_hip(hipGetLastError(), "gather launch");
 }
 
 uint64_t embedding_bwd_sorted_workspace_bytes(uint64_t N, uint32_t C) {

@@ -123,6 +123,12 @@ public:
     uint64_t norm_backward_workspace_bytes(uint64_t rows, uint32_t C, int dtype) {
         return agrad_norm_backward_workspace_bytes(rows, C, dtype);
     }
+    uint64_t embedding_sort_workspace_bytes(uint64_t N, uint32_t V) {
+        return agrad_embedding_sort_workspace_bytes(N, V);
+    }
+    uint64_t embedding_backward_sorted_workspace_bytes(uint64_t N, uint32_t C) {
+        return agrad_embedding_backward_sorted_workspace_bytes(N, C);
+    }
     uint64_t broadcast_grad_workspace_bytes(uint64_t lead, uint64_t inner) {
         return agrad_broadcast_grad_workspace_bytes(lead, inner);
     }
@@ -177,6 +183,8 @@ PYBIND11_MODULE(hip_ext, m) {
         .def("norm_backward_workspace_bytes", &HipContext::norm_backward_workspace_bytes)
         .def("embedding_backward_workspace_bytes", &HipContext::embedding_backward_workspace_bytes)
         .def("broadcast_grad_workspace_bytes", &HipContext::broadcast_grad_workspace_bytes)
+        .def("embedding_sort_workspace_bytes", &HipContext::embedding_sort_workspace_bytes)
+        .def("embedding_backward_sorted_workspace_bytes", &HipContext::embedding_backward_sorted_workspace_bytes)
         .def("kernel_names", &HipContext::kernel_names)
         .def("kernel_signature", &HipContext::kernel_signature)
         .def("handle", &HipContext::handle)

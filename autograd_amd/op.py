@@ -88,6 +88,20 @@ class AddOp(Op):
         return [0, 1]
 
 
+def _order_output(indices, table):
+    """When the table needs a gradient, the embedding ops carry a second,
+    gradient-free output: the (token, row) order of the indices, 2N uint32.  A
+    device may fill it in its forward kernel (where ordering the ids is free) and
+    start its backward kernel from it; a device that has no use for it leaves it
+    alone.  `__call__` still returns the embedding only."""
+    if not table.requires_grad:
+        return ()
+    n = 1
+    for d in indices.shape:
+        n *= d
+    return (Tensor(shape=(2 * n,), dtype=np.uint32, requires_grad=False, device=table.device),)
+
+
 class GatherOp(Op):
     """out[b, t, :] = weight[indices[b, t], :]"""
     op_name = "Gather"
@@ -102,11 +116,14 @@ class GatherOp(Op):
     def __call__(self, indices, weight):
         out = Tensor(shape=self.infer_shape(indices, weight), dtype=weight.dtype,
                      requires_grad=weight.requires_grad, device=weight.device)
-        out.op = OpNode(op=self, inputs=(indices, weight), outputs=(out,))
+        outputs = (out,) + _order_output(indices, weight)
+        node = OpNode(op=self, inputs=(indices, weight), outputs=outputs)
+        for t in outputs:
+            t.op = node
         return out
 
     def save_for_backward(self, inputs, outputs):
-        return list(inputs)
+        return list(inputs) + list(outputs[1:])
 
 
 class EmbeddingSumOp(Op):
@@ -127,11 +144,14 @@ class EmbeddingSumOp(Op):
     def __call__(self, indices, wte, wpe):
         out = Tensor(shape=self.infer_shape(indices, wte, wpe), dtype=wte.dtype, device=wte.device,
                      requires_grad=wte.requires_grad or wpe.requires_grad)
-        out.op = OpNode(op=self, inputs=(indices, wte, wpe), outputs=(out,))
+        outputs = (out,) + _order_output(indices, wte)
+        node = OpNode(op=self, inputs=(indices, wte, wpe), outputs=outputs)
+        for t in outputs:
+            t.op = node
         return out
 
     def save_for_backward(self, inputs, outputs):
-        return [inputs[0]]
+        return [inputs[0]] + list(outputs[1:])
 
     def fully_written_inputs(self, inputs, outputs):
         return [2] if inputs[2].shape[0] == inputs[0].shape[1] else []

@@ -156,17 +156,28 @@ def _embed_cases(ctx, cfg, pool, rng, nbytes, ids0):
         dY = [pool.normal(N * Cw, cfg.dtype) for _ in range(k)]
         dW = pool.empty(cfg.V * Cw, cfg.dtype)
         dwpe = pool.empty(cfg.T * Cw, cfg.dtype) if wpe is not None else None
-        ws_bytes = ctx.lib.agrad_embedding_backward_workspace_bytes(N, Cw, cfg.V, dt)
+        # the forward call also orders the ids (one launch: the ordering runs beside the
+        # bandwidth-bound gather); the backward call consumes that order.  Same results
+        # as agrad_gather_forward + agrad_embedding_backward.
+        order = [pool.raw(8 * N) for _ in range(k)]
+        sort_ws_bytes = ctx.lib.agrad_embedding_sort_workspace_bytes(N, cfg.V)
+        sort_ws = pool.raw(sort_ws_bytes)
+        ws_bytes = ctx.lib.agrad_embedding_backward_sorted_workspace_bytes(N, Cw)
         ws = pool.raw(ws_bytes)
         ctx.call("agrad_fill", dW.ptr, 0, 0, 1, dW.nbytes)
 
         def fwd(i):
-            ctx.call("agrad_gather_forward", dt, vp(ids[i]), vp(W), vp(wpe), vp(out[i]), N, cfg.T, Cw, cfg.V)
+            ctx.call("agrad_gather_forward_sorted", dt, vp(ids[i]), vp(W), vp(wpe), vp(out[i]), N, cfg.T, Cw, cfg.V,
+                     vp(order[i]), vp(sort_ws), sort_ws_bytes)
 
         def bwd(i):
-            ctx.call("agrad_embedding_backward", dt, vp(ids[i]), vp(dY[i]), vp(dW), vp(ws), ws_bytes, N, Cw, cfg.V, 0)
+            ctx.call("agrad_embedding_backward_sorted", dt, vp(order[i]), vp(dY[i]), vp(dW), vp(ws), ws_bytes, N, Cw,
+                     cfg.V, 0)
             if dwpe is not None:
                 ctx.call("agrad_pos_embedding_backward", dt, vp(dY[i]), vp(dwpe), cfg.B, cfg.T, Cw, 0)
+
+        for i in range(k):
+            fwd(i)          # every set's order exists before backward is timed on its own
 
         def zero(i):
             ctx.call("agrad_fill", dW.ptr, 0, 0, 1, dW.nbytes)

@@ -213,6 +213,25 @@ uint64_t agrad_embedding_backward_workspace_bytes(uint64_t N, uint32_t C, uint32
 int agrad_embedding_backward(agrad_ctx* ctx, int dtype, const int32_t* ids, const void* dY, void* dW,
                              void* workspace, uint64_t workspace_bytes,
                              uint64_t N, uint32_t C, uint32_t V, uint32_t flags);
+/* The same pair with the ordering of the ids done in the forward call, where it
+ * is free: up to 16384 rows the gather and the ordering are ONE launch (the
+ * ordering workgroups run beside the bandwidth-bound gather), and the backward
+ * call starts at the segmented sum.  The forward call also writes order[0..N) =
+ * tokens and order[N..2N) = rows (each token's rows adjacent, ascending; 2N
+ * uint32).  sort_workspace (256-byte aligned, agrad_embedding_sort_workspace_bytes(N, V)
+ * bytes) is free again when the call's work has run; the backward call's
+ * workspace holds agrad_embedding_backward_sorted_workspace_bytes(N, C) bytes.
+ * Same results, bit for bit, as agrad_gather_forward + agrad_embedding_backward.
+ * (The reference orders nothing: np.add.at, backend.py:531-538, and float
+ * atomics, metal_ops.metal:406-427.) */
+uint64_t agrad_embedding_sort_workspace_bytes(uint64_t N, uint32_t V);
+int agrad_gather_forward_sorted(agrad_ctx* ctx, int dtype, const int32_t* ids, const void* W, const void* wpe,
+                                void* out, uint64_t N, uint32_t T, uint32_t C, uint32_t V,
+                                uint32_t* order, void* sort_workspace, uint64_t sort_workspace_bytes);
+uint64_t agrad_embedding_backward_sorted_workspace_bytes(uint64_t N, uint32_t C);
+int agrad_embedding_backward_sorted(agrad_ctx* ctx, int dtype, const uint32_t* order, const void* dY, void* dW,
+                                    void* workspace, uint64_t workspace_bytes,
+                                    uint64_t N, uint32_t C, uint32_t V, uint32_t flags);
 /* dwpe[t,:] (+)= sum_b dY[b,t,:], b ascending (pos_emb_grad, metal_ops.metal:220-234;
  * broadcast branch of cpu_add_backward, backend.py:78-105). */
 int agrad_pos_embedding_backward(agrad_ctx* ctx, int dtype, const void* dY, void* dwpe,

@@ -691,3 +691,67 @@ def test_broadcast_add_and_gradient(ctx, lead, inner, dtype):
         assert_fp32_close(results[0], cpu, "column sum vs cpu", rtol=1e-5, atol=max(2e-6, 1e-4 * np.sqrt(lead / 14)))
     for d in (dxs, dys, dgs, out, ws):
         d.free()
+
+
+@pytest.mark.parametrize("B,T,V,C,dist", [(4, 128, 50257, 128, "uniform"), (2, 700, 300, 48, "zipf"),
+                                          (32, 512, 32768, 384, "uniform"), (5, 4000, 1000, 64, "zipf"),
+                                          (3, 50, 77, 10, "uniform")])
+@pytest.mark.parametrize("with_wpe", [False, True])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_presorted_embedding_pair_matches_the_plain_pair(ctx, B, T, V, C, dist, with_wpe, dtype):
+    """agrad_gather_forward_sorted (gather and id ordering in one launch) +
+    agrad_embedding_backward_sorted give the very bits of agrad_gather_forward +
+    agrad_embedding_backward, call after call; (5, 4000) takes the radix path and
+    C = 10 the element-wise one."""
+    import ctypes as Ct
+    rng = _rng(60 + C)
+    N = B * T
+    if dist == "zipf":
+        p = np.arange(1, V + 1, dtype=np.float64) ** -1.1
+        ids = rng.choice(V, size=(B, T), p=p / p.sum()).astype(np.int32)
+    else:
+        ids = rng.integers(0, V, (B, T), dtype=np.int32)
+    W = (0.02 * rng.standard_normal((V, C))).astype(np.float32)
+    wpe = (0.02 * rng.standard_normal((T, C))).astype(np.float32) if with_wpe else None
+    dY = rng.standard_normal((B, T, C)).astype(np.float32)
+    if dtype == "bf16":
+        W, dY = to_bf16_bits(W), to_bf16_bits(dY)
+        wpe = to_bf16_bits(wpe) if wpe is not None else None
+        dt = capi.BF16
+    else:
+        dt = capi.F32
+    want_out = G.gather_forward(ctx, ids, W, wpe)
+    want_dW = G.embedding_backward(ctx, ids, dY, V)
+
+    def vp(d):
+        return Ct.c_void_p(d.ptr) if d is not None else None
+    d_ids, d_W, d_dY = ctx.upload(ids), ctx.upload(W), ctx.upload(dY)
+    d_wpe = ctx.upload(wpe) if wpe is not None else None
+    out = ctx.empty((N, C), W.dtype)
+    order = ctx.empty((2 * N,), np.uint32)
+    sws_b = ctx.lib.agrad_embedding_sort_workspace_bytes(N, V)
+    bws_b = ctx.lib.agrad_embedding_backward_sorted_workspace_bytes(N, C)
+    sws, bws = ctx.empty((sws_b,), np.uint8), ctx.empty((bws_b,), np.uint8)
+    for rep in range(3):
+        dW = ctx.zeros((V, C), W.dtype)
+        ctx.call("agrad_gather_forward_sorted", dt, vp(d_ids), vp(d_W), vp(d_wpe), vp(out), N, T, C, V,
+                 vp(order), vp(sws), sws_b)
+        # the sort scratch is free once the forward call's work is queued: scribble over it
+        ctx.call("agrad_fill", sws.ptr, 0, 0xFFFFFFFF, 4, sws_b // 4)
+        ctx.call("agrad_embedding_backward_sorted", dt, vp(order), vp(d_dY), vp(dW), vp(bws), bws_b, N, C, V,
+                 capi.ACC_PARAM_GRAD)
+        ctx.synchronize()
+        np.testing.assert_array_equal(out.download().reshape(B, T, C), want_out)
+        np.testing.assert_array_equal(dW.download(), want_dW)
+        got = order.download()
+        toks, rows = got[:N], got[N:]
+        np.testing.assert_array_equal(np.sort(rows), np.arange(N))
+        np.testing.assert_array_equal(toks, ids.reshape(-1)[rows])
+        # each token's rows are adjacent and ascending
+        d_tok = np.diff(toks.astype(np.int64))
+        assert len(np.unique(toks)) == int((d_tok != 0).sum()) + 1
+        assert (np.diff(rows.astype(np.int64))[d_tok == 0] > 0).all()
+        dW.free()
+    for d in (d_ids, d_W, d_dY, d_wpe, out, order, sws, bws):
+        if d is not None:
+            d.free()
