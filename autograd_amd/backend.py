@@ -36,7 +36,7 @@ from .utils import (bf16_bits, bf16_bits_to_f32_array, f32_array_to_bf16_bits, f
                     xavier_uniform)
 
 F32, BF16 = 0, 1
-ACC_INPUT_GRAD, ACC_PARAM_GRAD, ACC_INPUT_GRAD2 = 1, 2, 4
+ACC_INPUT_GRAD, ACC_PARAM_GRAD, ACC_INPUT_GRAD2, ACC_PARAM_GRAD2 = 1, 2, 4, 8
 
 
 class Backend:
@@ -294,7 +294,9 @@ class HipBackend(Backend):
         else:
             self._launch("embedding_sum_forward", [indices, table, wpe, out], [_dt(table), B * T, T, C, V])
 
-    def _embedding_grad(self, node, indices, weight, outputs, scratch):
+    def _embedding_grad(self, node, indices, weight, outputs, scratch, wpe=None):
+        """Token-table gradient; returns True when the position table's gradient (wpe
+        given) went into the same launch."""
         if scratch is None:
             raise RuntimeError("embedding backward needs its arena workspace (plan_scratch)")
         out = outputs[0]
@@ -302,8 +304,16 @@ class HipBackend(Backend):
         V, C = weight.shape
         flag = self._param_flag(node, weight)
         if len(outputs) > 1:
-            self._launch("gather_backward_sorted", [outputs[1], out.grad, weight.grad, ws],
-                         [_dt(weight), prod(indices.shape), C, V, flag] + _lo_hi(ws.nbytes))
+            T = 0
+            if wpe is not None:
+                T = indices.shape[1]
+                if self._param_flag(node, wpe):
+                    flag |= ACC_PARAM_GRAD2
+            dwpe = wpe.grad if wpe is not None else None
+            self._launch("gather_backward_sorted", [outputs[1], out.grad, weight.grad, ws, dwpe],
+                         [_dt(weight), prod(indices.shape), C, V, flag] + _lo_hi(ws.nbytes)
+                         + [T, _mask(outputs[1], out.grad, weight.grad, ws, dwpe)])
+            return wpe is not None
         else:
             self._launch("gather_backward_kernel", [indices, out.grad, weight.grad, ws],
                          [_dt(weight), prod(indices.shape), C, V, flag] + _lo_hi(ws.nbytes))
@@ -326,9 +336,11 @@ class HipBackend(Backend):
         if out.grad is None:
             return
         B, T = indices.shape
+        fused = False
         if wte.requires_grad:
-            self._embedding_grad(out.op, indices, wte, outputs, scratch)
-        if wpe.requires_grad:
+            fused = self._embedding_grad(out.op, indices, wte, outputs, scratch,
+                                         wpe if wpe.requires_grad and wpe.grad is not None else None)
+        if wpe.requires_grad and not fused:
             # rows beyond T of a longer table get no gradient
             self._launch("pos_emb_grad", [out.grad, wpe.grad],
                          [_dt(out), B, T, wpe.shape[1], self._param_flag(out.op, wpe)])

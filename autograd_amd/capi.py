@@ -17,7 +17,7 @@ LIB_PATH = Path(__file__).resolve().parent / "libautograd_hip.so"
 
 F32, BF16 = 0, 1
 NORM_LAYER, NORM_RMS = 0, 1
-ACC_INPUT_GRAD, ACC_PARAM_GRAD, ACC_INPUT_GRAD2 = 1, 2, 4
+ACC_INPUT_GRAD, ACC_PARAM_GRAD, ACC_INPUT_GRAD2, ACC_PARAM_GRAD2 = 1, 2, 4, 8
 OK, EINVAL, EHIP, ENOKERNEL, EINDEX, EWORKSPACE = 0, -1, -2, -3, -4, -5
 
 _ctx = C.c_void_p
@@ -72,7 +72,7 @@ SIGNATURES = {
     "agrad_embedding_sort_workspace_bytes": (_u64, [_u64, _u32]),
     "agrad_gather_forward_sorted": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u32, _u32, _u32, _ptr, _ptr, _u64]),
     "agrad_embedding_backward_sorted_workspace_bytes": (_u64, [_u64, _u32]),
-    "agrad_embedding_backward_sorted": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u64, _u32, _u32, _u32]),
+    "agrad_embedding_backward_sorted": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _u64, _u64, _u32, _u32, _u32, _u32]),
     "agrad_pos_embedding_backward": (_int, [_ctx, _int, _ptr, _ptr, _u32, _u32, _u32, _u32]),
     "agrad_graph_begin": (_int, [_ctx]),
     "agrad_graph_end": (_int, [_ctx, C.POINTER(_u64)]),

@@ -300,13 +300,15 @@ int h_gather_fwd_sorted(const Call& c) {
     return launch_gather_fwd_sorted(c.ctx->stream, (int)c.a[0], (const int32_t*)ids, W, wpe, out, N, T, C, V,
                                     (uint32_t*)order, ws, wsb, c.ctx->err_flag);
 }
-// buffers order, dY, dW, workspace | args dtype, N, C, V, flags, ws lo, hi
+// buffers order, dY, dW, workspace, dwpe | args dtype, N, C, V, flags, ws lo, hi, T, present mask
 int h_gather_bwd_sorted(const Call& c) {
     NEED_DTYPE(c.a[0])
     const uint64_t N = c.a[1], es = dtype_size(c.a[0]), wsb = u64(c.a, 5);
-    const uint32_t C = c.a[2], V = c.a[3];
+    const uint32_t C = c.a[2], V = c.a[3], T = c.a[7], mask = c.a[8];
     RESOLVE(0, N * 8, order) RESOLVE(1, N * C * es, dY) RESOLVE(2, (uint64_t)V * C * es, dW) RESOLVE(3, wsb, ws)
-    return launch_embedding_bwd_sorted(c.ctx->stream, (int)c.a[0], (const uint32_t*)order, dY, dW, ws, wsb, N, C, V, c.a[4]);
+    RESOLVE_IF(mask & 16u, 4, (uint64_t)T * C * es, dwpe)
+    return launch_embedding_bwd_sorted(c.ctx->stream, (int)c.a[0], (const uint32_t*)order, dY, dW, dwpe, ws, wsb, N, T,
+                                       C, V, c.a[4]);
 }
 // buffers dY, dwpe | args dtype, B, T, C, flags
 int h_pos_grad(const Call& c) {
@@ -381,7 +383,7 @@ const Entry kTable[] = {
     {"embedding_sum_forward", 4, 5, "ids, W, wpe, out | dtype, N, T, C, V", h_embed_sum_fwd},
     {"gather_backward_kernel", 4, 7, "ids, dY, dW, workspace | dtype, N, C, V, flags, ws_lo, ws_hi", h_gather_bwd},
     {"gather_forward_sorted", 6, 8, "ids, W, wpe, out, order, sort_workspace | dtype, N, T, C, V, ws_lo, ws_hi, present_mask", h_gather_fwd_sorted},
-    {"gather_backward_sorted", 4, 7, "order, dY, dW, workspace | dtype, N, C, V, flags, ws_lo, ws_hi", h_gather_bwd_sorted},
+    {"gather_backward_sorted", 5, 9, "order, dY, dW, workspace, dwpe | dtype, N, C, V, flags, ws_lo, ws_hi, T, present_mask", h_gather_bwd_sorted},
     {"pos_emb_grad", 2, 5, "dY, dwpe | dtype, B, T, C, flags", h_pos_grad},
     {"cross_entropy_forward", 4, 5, "logits, labels, loss, lse | dtype, rows_lo, rows_hi, V, present_mask", h_ce_fwd},
     {"cross_entropy_backward", 5, 6, "logits, labels, dloss, lse, dlogits | dtype, rows_lo, rows_hi, V, flags, present_mask", h_ce_bwd},
@@ -743,10 +745,11 @@ uint64_t agrad_embedding_backward_sorted_workspace_bytes(uint64_t N, uint32_t C)
     return embedding_bwd_sorted_workspace_bytes(N, C);
 }
 int agrad_embedding_backward_sorted(agrad_ctx* ctx, int dtype, const uint32_t* order, const void* dY, void* dW,
-                                    void* workspace, uint64_t workspace_bytes, uint64_t N, uint32_t C,
-                                    uint32_t V, uint32_t flags) {
+                                    void* dwpe, void* workspace, uint64_t workspace_bytes, uint64_t N, uint32_t T,
+                                    uint32_t C, uint32_t V, uint32_t flags) {
     CTX_OR_FAIL(ctx)
-    return launch_embedding_bwd_sorted(ctx->stream, dtype, order, dY, dW, workspace, workspace_bytes, N, C, V, flags);
+    return launch_embedding_bwd_sorted(ctx->stream, dtype, order, dY, dW, dwpe, workspace, workspace_bytes, N, T, C, V,
+                                       flags);
 }
 int agrad_pos_embedding_backward(agrad_ctx* ctx, int dtype, const void* dY, void* dwpe, uint32_t B,
                                  uint32_t T, uint32_t C, uint32_t flags) {

@@ -390,7 +390,27 @@ __global__ void __launch_bounds__(512)
 emb_segment_sum_kernel(const uint32_t* __restrict__ tok_s, const uint32_t* __restrict__ row_s,
                        const T* __restrict__ dY, T* dW, float* __restrict__ carry_head,
                        float* __restrict__ carry_tail, uint32_t N, uint32_t C, uint32_t CV,
-                       uint32_t V, uint32_t L, int accumulate) {
+                       uint32_t V, uint32_t L, int accumulate, uint32_t chunks, T* dwpe, uint32_t B,
+                       uint32_t T_len, int accumulate_pos) {
+    if (blockIdx.x >= chunks) {
+        // Workgroups past the chunks (present only when a position table wants its
+        // gradient) add dY over the batch, b ascending: dwpe[t, :] (+)= sum_b dY[b, t, :].
+        // Independent of the token sums, so it rides in the same launch.
+        const uint64_t TC = (uint64_t)T_len * C;
+        const uint64_t idx = (uint64_t)(blockIdx.x - chunks) * blockDim.x + threadIdx.x;
+        if (idx * VEC >= TC) return;
+        const uint64_t off = idx * VEC;
+        float acc[VEC];
+        VecIO<T, VEC>::load(dY + off, acc);
+        for (uint32_t b = 1; b < B; ++b) {
+            float v[VEC];
+            VecIO<T, VEC>::load(dY + (uint64_t)b * TC + off, v);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + v[k];
+        }
+        store_grad_row<T, VEC>(dwpe, off, acc, accumulate_pos != 0);
+        return;
+    }
     const ChunkEdges e = chunk_edges(tok_s, blockIdx.x, L, N);
     for (uint32_t cv = threadIdx.x; cv < CV; cv += blockDim.x) {
         const uint32_t col = cv * VEC;
@@ -670,25 +690,32 @@ inline uint64_t order_bytes(uint64_t N) { return align256(N * 8); }   // tok_s[N
 
 template <typename T>
 int embedding_sum_typed(hipStream_t s, const SumPlan& p, const uint32_t* tok_s, const uint32_t* row_s, const T* dY,
-                        T* dW, uint8_t* ws, uint32_t N, uint32_t C, uint32_t V, uint32_t flags) {
+                        T* dW, uint8_t* ws, uint32_t N, uint32_t C, uint32_t V, uint32_t flags, T* dwpe,
+                        uint32_t B, uint32_t T_len) {
     float* head = (float*)(ws + p.off_head);
     float* tail = (float*)(ws + p.off_tail);
     const int acc = (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0;
+    const int acc_pos = (flags & AGRAD_ACC_PARAM_GRAD2) ? 1 : 0;
     constexpr int WIDE = WideVec<T>::value;
-    const bool wide = C % WIDE == 0 && aligned16(dY) && aligned16(dW);
+    const bool wide = C % WIDE == 0 && aligned16(dY) && aligned16(dW) && (!dwpe || aligned16(dwpe));
+    const uint64_t TC = dwpe ? (uint64_t)T_len * C : 0;
     if (wide) {
         const uint32_t CV = C / WIDE;
         uint32_t block = ((CV + 63) / 64) * 64;
         if (block > 512) block = 512;
-        hipLaunchKernelGGL((emb_segment_sum_kernel<T, WIDE>), dim3(p.chunks), dim3(block), 0, s, tok_s,
-                           row_s, dY, dW, head, tail, N, C, CV, V, p.L, acc);
+        const uint64_t extra = (TC / WIDE + block - 1) / block;
+        if (p.chunks + extra > 0x7fffffffull) return set_error(AGRAD_EINVAL, "embedding backward: position table too large");
+        hipLaunchKernelGGL((emb_segment_sum_kernel<T, WIDE>), dim3(p.chunks + (uint32_t)extra), dim3(block), 0, s, tok_s,
+                           row_s, dY, dW, head, tail, N, C, CV, V, p.L, acc, p.chunks, dwpe, B, T_len, acc_pos);
         hipLaunchKernelGGL((emb_carry_fix_kernel<T, WIDE>), dim3(p.chunks), dim3(kFixCols * kFixLanes), 0, s,
                            tok_s, dW, head, tail, N, C, CV, V, p.L, acc);
     } else {
         uint32_t block = ((C + 63) / 64) * 64;
         if (block > 512) block = 512;
-        hipLaunchKernelGGL((emb_segment_sum_kernel<T, 1>), dim3(p.chunks), dim3(block), 0, s, tok_s,
-                           row_s, dY, dW, head, tail, N, C, C, V, p.L, acc);
+        const uint64_t extra = (TC + block - 1) / block;
+        if (p.chunks + extra > 0x7fffffffull) return set_error(AGRAD_EINVAL, "embedding backward: position table too large");
+        hipLaunchKernelGGL((emb_segment_sum_kernel<T, 1>), dim3(p.chunks + (uint32_t)extra), dim3(block), 0, s, tok_s,
+                           row_s, dY, dW, head, tail, N, C, C, V, p.L, acc, p.chunks, dwpe, B, T_len, acc_pos);
         hipLaunchKernelGGL((emb_carry_fix_kernel<T, 1>), dim3(p.chunks), dim3(kFixCols * kFixLanes), 0, s,
                            tok_s, dW, head, tail, N, C, C, V, p.L, acc);
     }
@@ -805,12 +832,17 @@ uint64_t embedding_bwd_sorted_workspace_bytes(uint64_t N, uint32_t C) {
 }
 
 int launch_embedding_bwd_sorted(hipStream_t s, int dtype, const uint32_t* order, const void* dY, void* dW,
-                                void* workspace, uint64_t workspace_bytes, uint64_t N, uint32_t C,
-                                uint32_t V, uint32_t flags) {
+                                void* dwpe, void* workspace, uint64_t workspace_bytes, uint64_t N, uint32_t T,
+                                uint32_t C, uint32_t V, uint32_t flags) {
     if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "embedding backward: unknown dtype %d", dtype);
     if (N == 0 || C == 0) return AGRAD_OK;
     if (int rc = check_embedding_sizes("embedding backward", N, V)) return rc;
     if (order == nullptr || dY == nullptr || dW == nullptr) return set_error(AGRAD_EINVAL, "embedding backward: null operand");
+    uint32_t B = 0;
+    if (dwpe != nullptr) {
+        if (T == 0 || N % T != 0) return set_error(AGRAD_EINVAL, "embedding backward: %llu rows are not a whole number of sequences of %u", (unsigned long long)N, T);
+        B = (uint32_t)(N / T);
+    }
     SumPlan p;
     plan_sum(N, C, &p);
     if (workspace == nullptr || workspace_bytes < p.total)
@@ -820,9 +852,9 @@ int launch_embedding_bwd_sorted(hipStream_t s, int dtype, const uint32_t* order,
         return set_error(AGRAD_EINVAL, "embedding backward: workspace must be 256-byte aligned");
     if (dtype == AGRAD_F32)
         return embedding_sum_typed<float>(s, p, order, order + N, (const float*)dY, (float*)dW, (uint8_t*)workspace,
-                                          (uint32_t)N, C, V, flags);
+                                          (uint32_t)N, C, V, flags, (float*)dwpe, B, T);
     return embedding_sum_typed<bf16_t>(s, p, order, order + N, (const bf16_t*)dY, (bf16_t*)dW, (uint8_t*)workspace,
-                                       (uint32_t)N, C, V, flags);
+                                       (uint32_t)N, C, V, flags, (bf16_t*)dwpe, B, T);
 }
 
 int launch_gather_fwd(hipStream_t s, int dtype, const int32_t* ids, const void* W, const void* wpe,
@@ -890,7 +922,7 @@ int launch_embedding_bwd(hipStream_t s, int dtype, const int32_t* ids, const voi
     uint8_t* ws = (uint8_t*)workspace;
     uint32_t* order = (uint32_t*)ws;
     if (int rc = launch_embedding_sort(s, ids, order, ws + order_bytes(N), sort_bytes, N, V, err_flag)) return rc;
-    return launch_embedding_bwd_sorted(s, dtype, order, dY, dW, ws + order_bytes(N) + sort_bytes, sum_bytes, N, C, V, flags);
+    return launch_embedding_bwd_sorted(s, dtype, order, dY, dW, nullptr, ws + order_bytes(N) + sort_bytes, sum_bytes, N, 0, C, V, flags);
 }
 
 int launch_pos_embedding_bwd(hipStream_t s, int dtype, const void* dY, void* dwpe, uint32_t B,

@@ -160,6 +160,7 @@ PYBIND11_MODULE(hip_ext, m) {
     m.attr("BF16") = (int)AGRAD_BF16;
     m.attr("ACC_INPUT_GRAD") = (unsigned)AGRAD_ACC_INPUT_GRAD;
     m.attr("ACC_PARAM_GRAD") = (unsigned)AGRAD_ACC_PARAM_GRAD;
+    m.attr("ACC_PARAM_GRAD2") = (unsigned)AGRAD_ACC_PARAM_GRAD2;
     m.def("device_count", [] {
         int n = 0;
         agrad_device_count(&n);

@@ -77,9 +77,10 @@ int launch_gather_fwd_sorted(hipStream_t s, int dtype, const int32_t* ids, const
                              void* out, uint64_t N, uint32_t T, uint32_t C, uint32_t V, uint32_t* order,
                              void* sort_workspace, uint64_t sort_workspace_bytes, int* err_flag);
 uint64_t embedding_bwd_sorted_workspace_bytes(uint64_t N, uint32_t C);
+// dwpe (optional, [T, C]): the position table's gradient sum_b dY[b, t, :] rides in the same launch
 int launch_embedding_bwd_sorted(hipStream_t s, int dtype, const uint32_t* order, const void* dY, void* dW,
-                                void* workspace, uint64_t workspace_bytes, uint64_t N, uint32_t C,
-                                uint32_t V, uint32_t flags);
+                                void* dwpe, void* workspace, uint64_t workspace_bytes, uint64_t N, uint32_t T,
+                                uint32_t C, uint32_t V, uint32_t flags);
 int launch_embedding_bwd(hipStream_t s, int dtype, const int32_t* ids, const void* dY, void* dW,
                          void* workspace, uint64_t workspace_bytes, uint64_t N, uint32_t C,
                          uint32_t V, uint32_t flags, int* err_flag);

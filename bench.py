@@ -171,10 +171,9 @@ def _embed_cases(ctx, cfg, pool, rng, nbytes, ids0):
                      vp(order[i]), vp(sort_ws), sort_ws_bytes)
 
         def bwd(i):
-            ctx.call("agrad_embedding_backward_sorted", dt, vp(order[i]), vp(dY[i]), vp(dW), vp(ws), ws_bytes, N, Cw,
-                     cfg.V, 0)
-            if dwpe is not None:
-                ctx.call("agrad_pos_embedding_backward", dt, vp(dY[i]), vp(dwpe), cfg.B, cfg.T, Cw, 0)
+            # the position table's gradient, when there is one, rides in the same launch
+            ctx.call("agrad_embedding_backward_sorted", dt, vp(order[i]), vp(dY[i]), vp(dW), vp(dwpe), vp(ws), ws_bytes,
+                     N, cfg.T, Cw, cfg.V, 0)
 
         for i in range(k):
             fwd(i)          # every set's order exists before backward is timed on its own

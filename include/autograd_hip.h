@@ -44,7 +44,8 @@ enum { AGRAD_NORM_LAYER = 0, AGRAD_NORM_RMS = 1 };
 enum {
     AGRAD_ACC_INPUT_GRAD = 1u, /* dx += ... (CPU semantics, backend.py:414,477-487); else dx = ... */
     AGRAD_ACC_PARAM_GRAD = 2u, /* dgamma/dbeta/dW += ...; else =                                   */
-    AGRAD_ACC_INPUT_GRAD2 = 4u /* norm backward: the same choice for the second output dx2         */
+    AGRAD_ACC_INPUT_GRAD2 = 4u, /* norm backward: the same choice for the second output dx2        */
+    AGRAD_ACC_PARAM_GRAD2 = 8u  /* sorted embedding backward: the same choice for dwpe             */
 };
 
 /* ---- context, memory, passes --------------------------------------------
@@ -229,9 +230,12 @@ int agrad_gather_forward_sorted(agrad_ctx* ctx, int dtype, const int32_t* ids, c
                                 void* out, uint64_t N, uint32_t T, uint32_t C, uint32_t V,
                                 uint32_t* order, void* sort_workspace, uint64_t sort_workspace_bytes);
 uint64_t agrad_embedding_backward_sorted_workspace_bytes(uint64_t N, uint32_t C);
+/* dwpe may be NULL; otherwise it is the [T, C] position table's gradient
+ * dwpe[t,:] (+)= sum_b dY[b,t,:] (N = B*T rows), computed by extra workgroups of
+ * the same launch; AGRAD_ACC_PARAM_GRAD2 accumulates into it. */
 int agrad_embedding_backward_sorted(agrad_ctx* ctx, int dtype, const uint32_t* order, const void* dY, void* dW,
-                                    void* workspace, uint64_t workspace_bytes,
-                                    uint64_t N, uint32_t C, uint32_t V, uint32_t flags);
+                                    void* dwpe, void* workspace, uint64_t workspace_bytes,
+                                    uint64_t N, uint32_t T, uint32_t C, uint32_t V, uint32_t flags);
 /* dwpe[t,:] (+)= sum_b dY[b,t,:], b ascending (pos_emb_grad, metal_ops.metal:220-234;
  * broadcast branch of cpu_add_backward, backend.py:78-105). */
 int agrad_pos_embedding_backward(agrad_ctx* ctx, int dtype, const void* dY, void* dwpe,

@@ -701,8 +701,10 @@ def test_broadcast_add_and_gradient(ctx, lead, inner, dtype):
 def test_presorted_embedding_pair_matches_the_plain_pair(ctx, B, T, V, C, dist, with_wpe, dtype):
     """agrad_gather_forward_sorted (gather and id ordering in one launch) +
     agrad_embedding_backward_sorted give the very bits of agrad_gather_forward +
-    agrad_embedding_backward, call after call; (5, 4000) takes the radix path and
-    C = 10 the element-wise one."""
+    agrad_embedding_backward (+ agrad_pos_embedding_backward for the position
+    table, whose sum rides in the sorted call's launch), call after call, both
+    overwriting and accumulating; (5, 4000) takes the radix path and C = 10 the
+    element-wise one."""
     import ctypes as Ct
     rng = _rng(60 + C)
     N = B * T
@@ -722,6 +724,19 @@ def test_presorted_embedding_pair_matches_the_plain_pair(ctx, B, T, V, C, dist, 
         dt = capi.F32
     want_out = G.gather_forward(ctx, ids, W, wpe)
     want_dW = G.embedding_backward(ctx, ids, dY, V)
+    d_dwpe = want_dwpe = None
+    if with_wpe:
+        d_dwpe = ctx.zeros((T, C), W.dtype)
+        plain = ctx.zeros((T, C), W.dtype)
+        d_plain_dY = ctx.upload(dY)
+        # expected: one overwriting call, then two accumulating ones, as below
+        for flag in (0, capi.ACC_PARAM_GRAD, capi.ACC_PARAM_GRAD):
+            ctx.call("agrad_pos_embedding_backward", dt, Ct.c_void_p(d_plain_dY.ptr), Ct.c_void_p(plain.ptr), B, T, C,
+                     flag)
+        ctx.synchronize()
+        want_dwpe = plain.download()
+        plain.free()
+        d_plain_dY.free()
 
     def vp(d):
         return Ct.c_void_p(d.ptr) if d is not None else None
@@ -738,8 +753,8 @@ def test_presorted_embedding_pair_matches_the_plain_pair(ctx, B, T, V, C, dist, 
                  vp(order), vp(sws), sws_b)
         # the sort scratch is free once the forward call's work is queued: scribble over it
         ctx.call("agrad_fill", sws.ptr, 0, 0xFFFFFFFF, 4, sws_b // 4)
-        ctx.call("agrad_embedding_backward_sorted", dt, vp(order), vp(d_dY), vp(dW), vp(bws), bws_b, N, C, V,
-                 capi.ACC_PARAM_GRAD)
+        ctx.call("agrad_embedding_backward_sorted", dt, vp(order), vp(d_dY), vp(dW), vp(d_dwpe), vp(bws), bws_b, N, T,
+                 C, V, capi.ACC_PARAM_GRAD | (capi.ACC_PARAM_GRAD2 if rep else 0))
         ctx.synchronize()
         np.testing.assert_array_equal(out.download().reshape(B, T, C), want_out)
         np.testing.assert_array_equal(dW.download(), want_dW)
@@ -752,6 +767,8 @@ def test_presorted_embedding_pair_matches_the_plain_pair(ctx, B, T, V, C, dist, 
         assert len(np.unique(toks)) == int((d_tok != 0).sum()) + 1
         assert (np.diff(rows.astype(np.int64))[d_tok == 0] > 0).all()
         dW.free()
-    for d in (d_ids, d_W, d_dY, d_wpe, out, order, sws, bws):
+    if with_wpe:
+        np.testing.assert_array_equal(d_dwpe.download(), want_dwpe)
+    for d in (d_ids, d_W, d_dY, d_wpe, d_dwpe, out, order, sws, bws):
         if d is not None:
             d.free()
