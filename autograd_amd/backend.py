@@ -29,11 +29,12 @@ from math import prod
 
 import numpy as np
 
-from .op import (AddLayerNormOp, AddOp, AddRMSNormOp, CrossEntropyLossOp, EmbeddingSumOp, GatherOp, GELUOp,
-                 LayerNormOp, ReLUSquaredOp, RMSNormOp, RopeOp, SwiGLUOp)
+from .op import (AddLayerNormOp, AddOp, AddRMSNormOp, ContiguousOp, CrossEntropyLossOp, EmbeddingSumOp, GatherOp,
+                 GELUOp, LayerNormOp, PermuteOp, ReLUSquaredOp, ReshapeOp, RMSNormOp, RopeOp, SwiGLUOp,
+                 TransposeOp, ViewOp)
 from .scratch import single_slot
-from .utils import (bf16_bits, bf16_bits_to_f32_array, f32_array_to_bf16_bits, f32_bits, is_bf16,
-                    xavier_uniform)
+from .utils import (bf16_bits, bf16_bits_to_f32_array, contiguous_strides, f32_array_to_bf16_bits, f32_bits,
+                    is_bf16, xavier_uniform)
 
 F32, BF16 = 0, 1
 ACC_INPUT_GRAD, ACC_PARAM_GRAD, ACC_INPUT_GRAD2, ACC_PARAM_GRAD2 = 1, 2, 4, 8
@@ -151,6 +152,11 @@ class HipBackend(Backend):
             AddRMSNormOp: self.hip_add_norm_forward,
             RopeOp: self.hip_rope_forward,
             CrossEntropyLossOp: self.hip_cross_entropy_forward,
+            ViewOp: self.hip_view_forward,
+            ReshapeOp: self.hip_view_forward,
+            PermuteOp: self.hip_view_forward,
+            TransposeOp: self.hip_view_forward,
+            ContiguousOp: self.hip_contiguous_forward,
         }
         self.backward_kernels = {
             AddOp: self.hip_add_backward,
@@ -165,6 +171,11 @@ class HipBackend(Backend):
             AddRMSNormOp: self.hip_add_norm_backward,
             RopeOp: self.hip_rope_backward,
             CrossEntropyLossOp: self.hip_cross_entropy_backward,
+            ViewOp: self.hip_dense_grad_backward,
+            ReshapeOp: self.hip_dense_grad_backward,
+            PermuteOp: self.hip_permute_backward,
+            TransposeOp: self.hip_permute_backward,
+            ContiguousOp: self.hip_dense_grad_backward,
         }
 
     # -- lookup (backend.py:4938-4950) -------------------------------------------
@@ -274,6 +285,54 @@ class HipBackend(Backend):
                              + _lo_hi(ws.nbytes if ws is not None else 0) + [_mask(out.grad, t.grad, ws)])
             else:
                 raise RuntimeError(f"Unsupported Add backward shape: {t.shape} from {out.shape}")
+
+    # -- views and layout changes (backend.py:263-318, 2754-2866) --------------------
+    # View / Reshape / Permute / Transpose outputs share their input's memory, so
+    # their forward launches nothing; the gradients are dense tensors of their own.
+    def hip_view_forward(self, inputs, outputs, scratch=None):
+        pass
+
+    def hip_dense_grad_backward(self, inputs, outputs, scratch=None):
+        """x.grad (+)= out.grad, element for element (View, Reshape, Contiguous)"""
+        x, out = inputs[0], outputs[0]
+        if out.grad is None or not x.requires_grad or x.grad is None:
+            return
+        self._launch("add_residual_backward", [out.grad, x.grad],
+                     [_dt(out), self._grad_flag(out.op, x)] + _lo_hi(out.numel))
+
+    def _gather_strided(self, name, src, src_offset_elems, dst, shape, strides, flags):
+        st = src.storage if hasattr(src, "storage") else src
+        dstst = dst.storage if hasattr(dst, "storage") else dst
+        es = np.dtype(st.dtype).itemsize
+        if es not in (2, 4) or np.dtype(dstst.dtype).itemsize != es:
+            raise RuntimeError(f"strided copy: unsupported element types {st.dtype} -> {dstst.dtype}")
+        if any(s < 0 for s in strides):
+            raise RuntimeError("strided copy: negative strides")
+        self.ctx.dispatch_contiguous(name, st.ptr.buffer_id, st.ptr.offset + int(src_offset_elems) * es,
+                                     dstst.ptr.buffer_id, dstst.ptr.offset, [int(d) for d in shape],
+                                     [int(s) for s in strides], prod(shape), 1 if es == 2 else 0, flags)
+
+    def hip_permute_backward(self, inputs, outputs, scratch=None):
+        """x.grad[c] (+)= out.grad[c permuted]: a strided read of the dense out.grad"""
+        x, out = inputs[0], outputs[0]
+        if out.grad is None or not x.requires_grad or x.grad is None:
+            return
+        op = out.op.op
+        n = x.ndim
+        dims = tuple(d % n for d in op.dims) if isinstance(op, PermuteOp) else None
+        if dims is None:
+            dims = list(range(n))
+            dims[op.dim0 % n], dims[op.dim1 % n] = dims[op.dim1 % n], dims[op.dim0 % n]
+        dense = contiguous_strides(out.shape)
+        strides = [0] * n
+        for i, d in enumerate(dims):
+            strides[d] = dense[i]         # x's dimension d is out's dimension i
+        self._gather_strided("strided_add_backward_kernel", out.grad, 0, x.grad, x.shape, strides,
+                             self._grad_flag(out.op, x))
+
+    def hip_contiguous_forward(self, inputs, outputs, scratch=None):
+        x, out = inputs[0], outputs[0]
+        self._gather_strided("contiguous_forward_kernel", x, x.offset, out, x.shape, x.strides, 0)
 
     # -- embedding (backend.py:525-538, 2777-2815) ----------------------------------
     # When the table needs a gradient the op carries an `order` output: the forward
@@ -575,6 +634,8 @@ class HipBackend(Backend):
 
     def copy_to_host(self, tensor):
         """fp32 array for fp32 and bf16 tensors (bf16 is widened), raw otherwise"""
+        if not tensor.is_contiguous:
+            raise RuntimeError("copy_to_host of a permuted view: call contiguous() in the graph first")
         st = tensor.storage
         dt = np.dtype(st.dtype)
         raw = self.ctx.copy_to_host(st.ptr.buffer_id, st.ptr.offset, list(tensor.shape), dt.name)

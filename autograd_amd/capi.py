@@ -71,6 +71,7 @@ SIGNATURES = {
     "agrad_embedding_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u64, _u32, _u32, _u32]),
     "agrad_embedding_sort_workspace_bytes": (_u64, [_u64, _u32]),
     "agrad_gather_forward_sorted": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u32, _u32, _u32, _ptr, _ptr, _u64]),
+    "agrad_strided_copy": (_int, [_ctx, _int, _ptr, _ptr, _int, _ptr, _ptr, _u32]),
     "agrad_embedding_backward_sorted_workspace_bytes": (_u64, [_u64, _u32]),
     "agrad_embedding_backward_sorted": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _u64, _u64, _u32, _u32, _u32, _u32]),
     "agrad_pos_embedding_backward": (_int, [_ctx, _int, _ptr, _ptr, _u32, _u32, _u32, _u32]),

@@ -175,6 +175,26 @@ int h_cast_down(const Call& c) {
     RESOLVE(0, n * 4, src) RESOLVE(1, n * 2, dst)
     return launch_cast_f32_bf16(c.ctx->stream, src, dst, n, c.a[0] != 0);
 }
+// buffers src, dst | args dtype, flags, ndim, shape[8], (stride lo, hi)[8]; slots past ndim are ignored
+int h_strided_copy(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint32_t ndim = c.a[2];
+    if (ndim > AGRAD_MAX_DIMS) return set_error(AGRAD_EINVAL, "strided copy: %u dimensions (at most %d)", ndim, AGRAD_MAX_DIMS);
+    uint32_t shape[AGRAD_MAX_DIMS];
+    uint64_t strides[AGRAD_MAX_DIMS];
+    uint64_t numel = 1;
+    for (uint32_t i = 0; i < ndim; ++i) {
+        shape[i] = c.a[3 + i];
+        strides[i] = u64(c.a, 3 + AGRAD_MAX_DIMS + 2 * (int)i);
+        if (shape[i] != 0 && numel > 0xffffffffffffull / shape[i]) return set_error(AGRAD_EINVAL, "strided copy: shape too large");
+        numel *= shape[i];
+        if (shape[i] > 1 && strides[i] > 0xffffffffffffull / shape[i]) return set_error(AGRAD_EINVAL, "strided copy: stride too large");
+    }
+    if (numel == 0) return AGRAD_OK;
+    const uint64_t es = dtype_size(c.a[0]);
+    RESOLVE(0, strided_extent((int)ndim, shape, strides) * es, src) RESOLVE(1, numel * es, dst)
+    return launch_strided_copy(c.ctx->stream, (int)c.a[0], src, dst, (int)ndim, shape, strides, c.a[1]);
+}
 int h_cast_up(const Call& c) {
     const uint64_t n = u64(c.a, 0);
     RESOLVE(0, n * 2, src) RESOLVE(1, n * 4, dst)
@@ -368,6 +388,8 @@ const Entry kTable[] = {
     {"add_broadcast_backward", 3, 9, "g, dy, workspace | dtype, lead_lo, lead_hi, inner_lo, inner_hi, flags, ws_lo, ws_hi, present_mask", h_bcast_grad},
     {"fp32_to_bf16", 2, 3, "src, dst | accumulate, n_lo, n_hi", h_cast_down},
     {"bf16_to_fp32", 2, 2, "src, dst | n_lo, n_hi", h_cast_up},
+    {"contiguous_forward_kernel", 2, 27, "src, dst | dtype, flags, ndim, shape[8], stride_lo_hi[8]", h_strided_copy},
+    {"strided_add_backward_kernel", 2, 27, "src, dst | dtype, flags, ndim, shape[8], stride_lo_hi[8]", h_strided_copy},
     {"layernorm_forward", 6, 5, "x, residual, gamma, beta, h, y | dtype, rows, C, eps_bits, present_mask", h_norm_fwd<AGRAD_NORM_LAYER>},
     {"rmsnorm_forward", 6, 5, "x, residual, gamma, beta, h, y | dtype, rows, C, eps_bits, present_mask", h_norm_fwd<AGRAD_NORM_RMS>},
     {"layernorm_backward_kernel", 9, 8, "x, dy, gamma, dres, dx, dx2, dgamma, dbeta, workspace | dtype, rows, C, eps_bits, flags, present_mask, ws_lo, ws_hi", h_norm_bwd<AGRAD_NORM_LAYER>},
@@ -658,6 +680,12 @@ int agrad_grad_accumulate(agrad_ctx* ctx, int dtype, const void* src, void* dst,
 int agrad_cast_f32_to_bf16(agrad_ctx* ctx, const void* src, void* dst, uint64_t n, int accumulate) {
     CTX_OR_FAIL(ctx)
     return launch_cast_f32_bf16(ctx->stream, src, dst, n, accumulate);
+}
+int agrad_strided_copy(agrad_ctx* ctx, int dtype, const void* src, void* dst, int ndim, const uint32_t* shape,
+                       const uint64_t* strides, uint32_t flags) {
+    CTX_OR_FAIL(ctx)
+    if (!dtype_ok((uint32_t)dtype)) return set_error(AGRAD_EINVAL, "unknown dtype %d", dtype);
+    return launch_strided_copy(ctx->stream, dtype, src, dst, ndim, shape, strides, flags);
 }
 int agrad_cast_bf16_to_f32(agrad_ctx* ctx, const void* src, void* dst, uint64_t n) {
     CTX_OR_FAIL(ctx)

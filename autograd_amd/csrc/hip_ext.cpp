@@ -94,6 +94,29 @@ public:
                                  (int)args.size(), gx, gy, gz, tg));
     }
 
+    // dst[dense index] (+)= src[strided index]: the reference's dispatch_contiguous and
+    // dispatch_strided (metal_ext.mm:512-557) with the element type and the write mode
+    // as optional trailing arguments; grid_size is implied by the shape
+    void dispatch_gather_strided(const std::string& name, uint64_t src_id, uint64_t src_off, uint64_t dst_id,
+                                 uint64_t dst_off, const std::vector<uint32_t>& shape,
+                                 const std::vector<uint64_t>& strides, uint64_t grid_size, int dtype,
+                                 uint32_t flags) {
+        (void)grid_size;
+        if (shape.size() != strides.size()) throw py::value_error("shape and strides differ in length");
+        if (shape.size() > AGRAD_MAX_DIMS) throw py::value_error("too many dimensions");
+        std::vector<uint32_t> args(3 + 3 * AGRAD_MAX_DIMS, 0u);
+        args[0] = (uint32_t)dtype;
+        args[1] = flags;
+        args[2] = (uint32_t)shape.size();
+        for (size_t i = 0; i < shape.size(); ++i) {
+            args[3 + i] = shape[i];
+            args[3 + AGRAD_MAX_DIMS + 2 * i] = (uint32_t)(strides[i] & 0xffffffffull);
+            args[3 + AGRAD_MAX_DIMS + 2 * i + 1] = (uint32_t)(strides[i] >> 32);
+        }
+        const uint64_t ids[2] = {src_id, dst_id}, offs[2] = {src_off, dst_off};
+        raise_for(agrad_dispatch(ctx_, name.c_str(), ids, offs, 2, args.data(), (int)args.size(), 0, 0, 0, 0));
+    }
+
     void fill_scalar(const std::string& name, const std::vector<uint64_t>& ids,
                      const std::vector<uint64_t>& offs, float value, uint64_t n) {
         (void)name;
@@ -176,6 +199,13 @@ PYBIND11_MODULE(hip_ext, m) {
         .def("begin_pass_profiled", &HipContext::begin_pass_profiled)
         .def("end_pass_profiled", &HipContext::end_pass_profiled)
         .def("dispatch_with_args_3d", &HipContext::dispatch_with_args_3d)
+        .def("dispatch_contiguous", &HipContext::dispatch_gather_strided, py::arg("kernel_name"),
+             py::arg("x_id"), py::arg("x_offset"), py::arg("out_id"), py::arg("out_offset"), py::arg("shape"),
+             py::arg("strides"), py::arg("grid_size") = 0, py::arg("dtype") = (int)AGRAD_F32, py::arg("flags") = 0u)
+        .def("dispatch_strided", &HipContext::dispatch_gather_strided, py::arg("kernel_name"),
+             py::arg("grad_out_id"), py::arg("grad_out_offset"), py::arg("grad_x_id"), py::arg("grad_x_offset"),
+             py::arg("shape"), py::arg("strides"), py::arg("grid_size") = 0, py::arg("dtype") = (int)AGRAD_F32,
+             py::arg("flags") = 0u)
         .def("fill_scalar", &HipContext::fill_scalar)
         .def("fill_scalar2", &HipContext::fill_scalar2)
         .def("copy_from_host", &HipContext::copy_from_host)

@@ -51,6 +51,12 @@ uint64_t broadcast_grad_workspace_bytes(uint64_t lead, uint64_t inner);
 int launch_broadcast_grad(hipStream_t s, int dtype, const void* g, void* dy, void* workspace, uint64_t workspace_bytes,
                           uint64_t lead, uint64_t inner, uint32_t flags);
 
+// strided.hip
+// elements spanned by the view: 1 + sum (shape[i] - 1) * strides[i]; 0 for an empty shape
+uint64_t strided_extent(int ndim, const uint32_t* shape, const uint64_t* strides);
+int launch_strided_copy(hipStream_t s, int dtype, const void* src, void* dst, int ndim, const uint32_t* shape,
+                        const uint64_t* strides, uint32_t flags);
+
 // activation.hip
 int launch_gelu_fwd(hipStream_t s, int dtype, const void* x, void* y, uint64_t n);
 int launch_gelu_bwd(hipStream_t s, int dtype, const void* x, const void* dy, void* dx, uint64_t n, uint32_t flags);

@@ -45,8 +45,22 @@ class Op(ABC):
     # indices (output i aliases input j): the kernel works in place, the
     # runtime gives output and input (and their grads) the same memory
     inplace_aliases: dict = {}
+    # index of the input that output 0 is a view of (same memory, other shape or
+    # strides); such an output gets no memory of its own
+    view_of_input = None
+    # only ops that read through strides take a permuted / transposed view
+    accepts_strided = False
+
+    def require_contiguous(self, inputs):
+        if self.accepts_strided:
+            return
+        for t in inputs:
+            if not t.is_contiguous:
+                raise RuntimeError(f"{self.op_name} requires contiguous inputs (got strides {t.strides} for shape "
+                                   f"{t.shape}); call contiguous() first")
 
     def __call__(self, *inputs):
+        self.require_contiguous(inputs)
         shape = self.infer_shape(*inputs)
         out = Tensor(shape=shape, dtype=self.infer_dtype(*inputs), device=inputs[0].device,
                      requires_grad=any(t.requires_grad for t in inputs))
@@ -88,6 +102,127 @@ class AddOp(Op):
         return [0, 1]
 
 
+# -- views and layout changes (op.py:89-185) --------------------------------------
+def resolve_reshape_shape(numel, target_shape):
+    """target shape with its single -1 filled in (utils.py:85-100)"""
+    shape = list(target_shape)
+    holes = [i for i, d in enumerate(shape) if d == -1]
+    if len(holes) > 1:
+        raise ValueError(f"reshape: at most one -1, got {tuple(target_shape)}")
+    known = 1
+    for d in shape:
+        if d != -1:
+            known *= d
+    if known == 0:
+        raise ValueError(f"reshape: invalid target_shape {tuple(target_shape)}")
+    if holes:
+        if numel % known != 0:
+            raise ValueError(f"reshape: numel {numel} not divisible by {known},target={tuple(target_shape)}")
+        shape[holes[0]] = numel // known
+    elif known != numel:
+        raise ValueError(f"reshape: numel mismatch: {numel} -> {tuple(shape)}")
+    return tuple(shape)
+
+
+class _LayoutOp(Op):
+    """output 0 shares input 0's memory; forward launches nothing"""
+    view_of_input = 0
+    accepts_strided = True
+
+    def _make(self, x, shape, strides, is_contiguous):
+        out = Tensor(shape=shape, dtype=x.dtype, strides=strides, offset=x.offset, is_contiguous=is_contiguous,
+                     requires_grad=x.requires_grad, device=x.device)
+        out.op = OpNode(op=self, inputs=(x,), outputs=(out,))
+        return out
+
+    def save_for_backward(self, inputs, outputs):
+        return []       # the gradient kernels read gradients only
+
+    def fully_written_inputs(self, inputs, outputs):
+        return [0]
+
+
+class ReshapeOp(_LayoutOp):
+    """same elements under another shape; the input must be contiguous (utils.py:102-109)"""
+    op_name = "Reshape"
+
+    def __init__(self, shape):
+        if len(shape) == 1 and isinstance(shape[0], (tuple, list)):
+            shape = shape[0]
+        self.shape = tuple(shape)
+
+    def infer_shape(self, x):
+        return resolve_reshape_shape(x.numel, self.shape)
+
+    def __call__(self, x):
+        shape = self.infer_shape(x)
+        if not x.is_contiguous:
+            raise RuntimeError("reshape view requires contiguous input")
+        return self._make(x, shape, None, True)
+
+
+class ViewOp(ReshapeOp):
+    op_name = "View"
+
+    def __call__(self, x):
+        if not x.is_contiguous:
+            raise RuntimeError("view requires contiguous")
+        return super().__call__(x)
+
+
+class PermuteOp(_LayoutOp):
+    """out.shape[i] = x.shape[dims[i]]; a view with permuted strides"""
+    op_name = "Permute"
+
+    def __init__(self, dims):
+        if len(dims) == 1 and isinstance(dims[0], (tuple, list)):
+            dims = dims[0]
+        self.dims = tuple(int(d) for d in dims)
+
+    def infer_shape(self, x):
+        if sorted(d % x.ndim for d in self.dims) != list(range(x.ndim)):
+            raise ValueError(f"permute: {self.dims} is not a permutation of {x.ndim} dimensions")
+        return tuple(x.shape[d] for d in self.dims)
+
+    def __call__(self, x):
+        shape = self.infer_shape(x)
+        return self._make(x, shape, tuple(x.strides[d] for d in self.dims), False)
+
+
+class TransposeOp(_LayoutOp):
+    op_name = "Transpose"
+
+    def __init__(self, dim0, dim1):
+        self.dim0 = dim0
+        self.dim1 = dim1
+
+    def infer_shape(self, x):
+        shape = list(x.shape)
+        shape[self.dim0], shape[self.dim1] = shape[self.dim1], shape[self.dim0]
+        return tuple(shape)
+
+    def __call__(self, x):
+        shape = self.infer_shape(x)
+        strides = list(x.strides)
+        strides[self.dim0], strides[self.dim1] = strides[self.dim1], strides[self.dim0]
+        return self._make(x, shape, tuple(strides), False)
+
+
+class ContiguousOp(Op):
+    """a dense copy of a (possibly permuted) view"""
+    op_name = "Contiguous"
+    accepts_strided = True
+
+    def infer_shape(self, x):
+        return x.shape
+
+    def save_for_backward(self, inputs, outputs):
+        return []
+
+    def fully_written_inputs(self, inputs, outputs):
+        return [0]
+
+
 def _order_output(indices, table):
     """When the table needs a gradient, the embedding ops carry a second,
     gradient-free output: the (token, row) order of the indices, 2N uint32.  A
@@ -114,6 +249,7 @@ class GatherOp(Op):
         return indices.shape + (weight.shape[1],)
 
     def __call__(self, indices, weight):
+        self.require_contiguous((indices, weight))
         out = Tensor(shape=self.infer_shape(indices, weight), dtype=weight.dtype,
                      requires_grad=weight.requires_grad, device=weight.device)
         outputs = (out,) + _order_output(indices, weight)
@@ -142,6 +278,7 @@ class EmbeddingSumOp(Op):
         return indices.shape + (wte.shape[1],)
 
     def __call__(self, indices, wte, wpe):
+        self.require_contiguous((indices, wte, wpe))
         out = Tensor(shape=self.infer_shape(indices, wte, wpe), dtype=wte.dtype, device=wte.device,
                      requires_grad=wte.requires_grad or wpe.requires_grad)
         outputs = (out,) + _order_output(indices, wte)
@@ -261,6 +398,7 @@ class CrossEntropyLossOp(Op):
         return labels.shape
 
     def __call__(self, logits, labels):
+        self.require_contiguous((logits, labels))
         shape = self.infer_shape(logits, labels)
         loss = Tensor(shape=shape, dtype=np.float32, requires_grad=logits.requires_grad, device=logits.device)
         lse = Tensor(shape=shape, dtype=np.float32, requires_grad=False, device=logits.device)
@@ -282,6 +420,7 @@ class _AddNormOp(Op):
     n_norm_params = 0
 
     def __call__(self, *inputs):
+        self.require_contiguous(inputs)
         x, res = inputs[0], inputs[1]
         if x.shape != res.shape:
             raise ValueError("fused residual add needs operands of one shape")
@@ -348,6 +487,7 @@ class RopeOp(Op):
         return q.shape, k.shape
 
     def __call__(self, q, k, cos, sin):
+        self.require_contiguous((q, k, cos, sin))
         qs, ks = self.infer_shape(q, k, cos, sin)
         q2 = Tensor(shape=qs, dtype=q.dtype, device=q.device, requires_grad=q.requires_grad)
         k2 = Tensor(shape=ks, dtype=k.dtype, device=k.device, requires_grad=k.requires_grad)

@@ -117,7 +117,8 @@ class Runtime:
         self.arena_bytes = 0
         self.leaves = []
         self.consumers = {}
-        self._alias_of = {}            # output tensor -> input tensor it shares memory with
+        self._alias_of = {}            # output tensor -> input tensor it shares memory and gradient with
+        self._view_of = {}             # output tensor -> input tensor whose memory it re-reads (layout ops)
         self._stored_leaf_grads = set()   # ids of leaf grads whose first writer stores the whole tensor
         self._slabs = []
 
@@ -238,13 +239,30 @@ class Runtime:
         """In-place ops: an output shares its input's memory when the input is
         an activation nobody else reads; otherwise the backend copies first."""
         self._alias_of = {}
+        self._view_of = {}
+        for node in self.topo:
+            if node.op.view_of_input is not None:
+                self._view_of[id(node.outputs[0])] = node.inputs[node.op.view_of_input]
         for node in self.topo:
             for out_i, in_i in node.op.inplace_aliases.items():
                 src, dst = node.inputs[in_i], node.outputs[out_i]
-                if src.op is not None and len(self.consumers.get(id(src), [])) == 1 and src is not self.loss:
+                # a view's memory belongs to its base, which others may still read
+                if src.op is not None and len(self.consumers.get(id(src), [])) == 1 and src is not self.loss \
+                        and id(src) not in self._view_of:
                     self._alias_of[id(dst)] = src
 
     def _root(self, t):
+        """the tensor whose memory `t` lives in (views: same memory, own gradient)"""
+        while True:
+            if id(t) in self._alias_of:
+                t = self._alias_of[id(t)]
+            elif id(t) in self._view_of:
+                t = self._view_of[id(t)]
+            else:
+                return t
+
+    def _grad_root(self, t):
+        """the tensor whose gradient memory `t`'s gradient lives in"""
         while id(t) in self._alias_of:
             t = self._alias_of[id(t)]
         return t
@@ -296,27 +314,26 @@ class Runtime:
 
         for step, (phase, node) in enumerate(steps):
             if phase == 0:
-                for t in node.outputs:
-                    touch(self._root(t), step)
-                for t in node.inputs:
-                    if t.op is not None:
+                for t in node.inputs + node.outputs:
+                    if self._root(t).op is not None:     # leaves (and views of leaves) live outside the arena
                         touch(self._root(t), step)
                 if node.scratch_fwd_layout is not None:
                     touch(_Scratch(node.scratch_fwd_layout.nbytes, node, 0), step)
             else:
                 for t in node.op.save_for_backward(node.inputs, node.outputs):
-                    if t.op is not None:
+                    if self._root(t).op is not None:
                         touch(self._root(t), step)
                 for t in node.inputs + node.outputs:
                     if t.grad is not None and t.op is not None:
-                        touch(self._root(t).grad if self._root(t).grad is not None else t.grad, step)
+                        g = self._grad_root(t).grad
+                        touch(g if g is not None else t.grad, step)
                 if node.scratch_bwd_layout is not None:
                     touch(_Scratch(node.scratch_bwd_layout.nbytes, node, 1), step)
         if self.loss is not None and self.loss.op is not None:
             touch(self._root(self.loss), len(steps))
             if self.loss.grad is not None:
                 # written by fill() between the forward and the backward loops
-                touch(self._root(self.loss).grad or self.loss.grad, n - 1 if n else 0)
+                touch(self._grad_root(self.loss).grad or self.loss.grad, n - 1 if n else 0)
 
         planner = MemoryPlanner()
         order = sorted(life.items(), key=lambda kv: kv[1][0])
@@ -373,16 +390,20 @@ class Runtime:
                     node.backward = functools.partial(base, scratch=views)
             else:
                 obj.storage = self.allocator.view(arena, off, obj.shape, obj.dtype)
-        # aliased outputs (and their gradients) share their root's views
+        # in topological order, so that chains resolve: in-place outputs (and their
+        # gradients) share their input's views; layout ops re-view their input's memory
         for node in self.topo:
             for t in node.outputs:
                 if id(t) in self._alias_of:
-                    root = self._root(t)
-                    t.storage = root.storage
-                    if t.grad is not None and root.grad is not None:
-                        t.grad.storage = root.grad.storage
-                    elif t.grad is not None and root.grad is None:
+                    src = self._alias_of[id(t)]
+                    t.storage = src.storage
+                    if t.grad is not None and src.grad is not None:
+                        t.grad.storage = src.grad.storage
+                    elif t.grad is not None and src.grad is None:
                         raise RuntimeError("aliased output needs a gradient but its input has none")
+                elif id(t) in self._view_of:
+                    base = self._view_of[id(t)]
+                    t.storage = self.allocator.view(base.storage, 0, t.shape, t.dtype)
         for node in self.topo:
             for t in node.outputs:
                 if t.init_val is not None:

@@ -137,7 +137,7 @@ def build_cases(ctx, cfg, pool):
     nbytes = op_bytes(cfg, distinct)
     cases = []
     # one builder per op family: each keeps its buffers in its own scope
-    for builder in (_embed_cases, _norm_cases, _act_cases, _rope_cases, _loss_cases, _opt_cases):
+    for builder in (_embed_cases, _norm_cases, _act_cases, _rope_cases, _layout_cases, _loss_cases, _opt_cases):
         cases += builder(ctx, cfg, pool, rng, nbytes, ids0)
     return cases
 
@@ -261,6 +261,36 @@ def _act_cases(ctx, cfg, pool, rng, nbytes, ids0):
 
             cases.append(Case(cfg.act, "fwd", nbytes[cfg.act][0], k, fwd, "ew_kernel"))
             cases.append(Case(cfg.act, "bwd", nbytes[cfg.act][1], k, bwd, "ew_kernel"))
+    return cases
+
+
+def _layout_cases(ctx, cfg, pool, rng, nbytes, ids0):
+    """layout changes beside the hot path: q from [B,T,H,D] to [B,H,T,D] (rows kernel)
+    and the [N, C] activation transposed to [C, N] (tile kernel); 2 * numel * e bytes"""
+    import ctypes as C
+    dt = capi.BF16 if cfg.dtype == "bf16" else capi.F32
+    e = cfg.esize
+    cases = []
+
+    def add(name, dense_shape, dims):
+        numel = int(np.prod(dense_shape))
+        k = n_sets(numel * e)
+        src = [pool.normal(numel, cfg.dtype) for _ in range(k)]
+        dst = [pool.empty(numel, cfg.dtype) for _ in range(k)]
+        base = np.cumprod((1,) + tuple(dense_shape[::-1]))[:-1][::-1]
+        shape = (C.c_uint32 * len(dims))(*[dense_shape[d] for d in dims])
+        strides = (C.c_uint64 * len(dims))(*[int(base[d]) for d in dims])
+
+        def run(i):
+            ctx.call("agrad_strided_copy", dt, vp(src[i]), vp(dst[i]), len(dims), shape, strides, 0)
+
+        cases.append(Case(name, "layout", 2 * numel * e, k, run, "strided_"))
+
+    if cfg.rope:
+        Hq, _, D, _, _ = cfg.rope
+        add("permute_bthd_bhtd", (cfg.B, cfg.T, Hq, D), (0, 2, 1, 3))
+    if cfg.norm:
+        add("transpose_nc_cn", (cfg.N, cfg.C), (1, 0))
     return cases
 
 

@@ -140,6 +140,19 @@ int agrad_grad_accumulate(agrad_ctx* ctx, int dtype, const void* src, void* dst,
 /* dst_bf16[i] = rne(src_f32[i]) (+ dst if accumulate) (fp32_to_bf16, metal_ops.metal:12010-12041). */
 int agrad_cast_f32_to_bf16(agrad_ctx* ctx, const void* src, void* dst, uint64_t n, int accumulate);
 int agrad_cast_bf16_to_f32(agrad_ctx* ctx, const void* src, void* dst, uint64_t n);
+/* Strided gather into a dense tensor: dst[dense index over shape] (+)=
+ * src[sum_i coord_i * strides[i]], strides in elements (0 broadcasts), ndim <=
+ * AGRAD_MAX_DIMS.  Contiguous forward of a permuted / transposed view and the
+ * Permute / Transpose gradients (contiguous_forward_kernel and
+ * strided_add_backward_kernel, metal_ops.metal:429-449, 1002-1023, bound through
+ * dispatch_contiguous / dispatch_strided, metal_ext.mm:512-557; CPU:
+ * cpu_permute_backward, cpu_transpose_backward, cpu_contiguous_forward,
+ * backend.py:286-313).  Overwriting moves raw bits of any 2-byte (AGRAD_BF16) or
+ * 4-byte (AGRAD_F32) element; AGRAD_ACC_INPUT_GRAD adds onto dst, as the CPU
+ * backward kernels do.  src and dst may not overlap. */
+#define AGRAD_MAX_DIMS 8
+int agrad_strided_copy(agrad_ctx* ctx, int dtype, const void* src, void* dst, int ndim,
+                       const uint32_t* shape, const uint64_t* strides, uint32_t flags);
 /* plain device copy kernel; the calibration kernel for bandwidth and counters. */
 int agrad_copy(agrad_ctx* ctx, const void* src, void* dst, uint64_t nbytes);
 

@@ -17,8 +17,9 @@ import numpy as np
 
 from autograd_amd.backend import Backend
 from autograd_amd.device import Device
-from autograd_amd.op import (AddLayerNormOp, AddOp, AddRMSNormOp, CrossEntropyLossOp, EmbeddingSumOp, GatherOp,
-                             GELUOp, LayerNormOp, ReLUSquaredOp, RMSNormOp, RopeOp, SwiGLUOp)
+from autograd_amd.op import (AddLayerNormOp, AddOp, AddRMSNormOp, ContiguousOp, CrossEntropyLossOp, EmbeddingSumOp,
+                             GatherOp, GELUOp, LayerNormOp, PermuteOp, ReLUSquaredOp, ReshapeOp, RMSNormOp, RopeOp,
+                             SwiGLUOp, TransposeOp, ViewOp)
 from autograd_amd.storage import Allocator, Storage
 from autograd_amd.utils import is_bf16, storage_dtype
 
@@ -86,6 +87,40 @@ def cpu_add_backward(inputs, outputs, scratch=None):
         if t.requires_grad and t.grad is not None:
             with _Acc(t.grad) as acc:
                 K.add_backward_into(g, acc)
+
+
+# views share their input's memory: nothing to do going forward (backend.py:263-313)
+def cpu_view_forward(inputs, outputs, scratch=None):
+    pass
+
+
+def cpu_dense_grad_backward(inputs, outputs, scratch=None):
+    x, out = inputs[0], outputs[0]
+    if out.grad is None or not x.requires_grad or x.grad is None:
+        return
+    with _Acc(x.grad) as acc:
+        K.add_backward_into(_val(out.grad).reshape(x.shape), acc)
+
+
+def cpu_permute_backward(inputs, outputs, scratch=None):
+    x, out = inputs[0], outputs[0]
+    if out.grad is None or not x.requires_grad or x.grad is None:
+        return
+    with _Acc(x.grad) as acc:
+        K.permute_backward_into(_val(out.grad), [d % x.ndim for d in out.op.op.dims], acc)
+
+
+def cpu_transpose_backward(inputs, outputs, scratch=None):
+    x, out = inputs[0], outputs[0]
+    if out.grad is None or not x.requires_grad or x.grad is None:
+        return
+    with _Acc(x.grad) as acc:
+        K.transpose_backward_into(_val(out.grad), out.op.op.dim0, out.op.op.dim1, acc)
+
+
+def cpu_contiguous_forward(inputs, outputs, scratch=None):
+    x, out = inputs[0], outputs[0]
+    out.storage.data[...] = K.contiguous_forward(x.storage.data, x.shape, x.strides, x.offset)
 
 
 def cpu_gather_forward(inputs, outputs, scratch=None):
@@ -303,6 +338,8 @@ class CPUBackend(Backend):
             LayerNormOp: cpu_layernorm_forward, RMSNormOp: cpu_rmsnorm_forward,
             AddLayerNormOp: cpu_add_norm_forward, AddRMSNormOp: cpu_add_norm_forward, RopeOp: cpu_rope_forward,
             CrossEntropyLossOp: cpu_cross_entropy_forward,
+            ViewOp: cpu_view_forward, ReshapeOp: cpu_view_forward, PermuteOp: cpu_view_forward,
+            TransposeOp: cpu_view_forward, ContiguousOp: cpu_contiguous_forward,
         }
         self.backward_kernels = {
             AddOp: cpu_add_backward, GatherOp: cpu_gather_backward, EmbeddingSumOp: cpu_embedding_sum_backward,
@@ -310,6 +347,8 @@ class CPUBackend(Backend):
             LayerNormOp: cpu_layernorm_backward, RMSNormOp: cpu_rmsnorm_backward,
             AddLayerNormOp: cpu_add_norm_backward, AddRMSNormOp: cpu_add_norm_backward, RopeOp: cpu_rope_backward,
             CrossEntropyLossOp: cpu_cross_entropy_backward,
+            ViewOp: cpu_dense_grad_backward, ReshapeOp: cpu_dense_grad_backward, PermuteOp: cpu_permute_backward,
+            TransposeOp: cpu_transpose_backward, ContiguousOp: cpu_dense_grad_backward,
         }
 
     def get_forward_kernel(self, op):

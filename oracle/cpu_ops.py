@@ -19,6 +19,8 @@ Pinning (what shows these functions are the right functions; tests/test_oracle.p
   * bf16: bit-exact against an exhaustive integer restatement of utils.py:20-27.
   * cross-entropy: scipy.special.logsumexp / softmax in float64, finite
     differences, rows of the gradient sum to zero, uniform logits give log V.
+  * strided views / permute gradients: an explicit loop over every dense index
+    with the index arithmetic written out, on small shapes.
   * adamw: the textbook bias-corrected recurrence in float64 over several steps;
     the first step from zero moments moves every weight by lr * sign(g).
 Parity unpinned by the reference:
@@ -57,6 +59,35 @@ def add_backward_into(g, grad):
     axes = tuple(i for i, (gi, ti) in enumerate(zip(g.shape, padded)) if ti == 1 and gi != 1)
     tmp = np.sum(g, axis=axes) if axes else g
     np.add(grad, tmp.reshape(grad.shape), out=grad)
+
+
+# --------------------------------------------------------------------------
+# Views and layout changes  (tensor_to_numpy, utils.py:111-125;
+# cpu_permute_backward / cpu_transpose_backward / cpu_contiguous_forward,
+# backend.py:286-313)
+# --------------------------------------------------------------------------
+def strided_view(flat, shape, strides, offset=0):
+    """the [shape] view of the flat buffer that starts `offset` elements in and
+    steps `strides` elements per dimension"""
+    flat = flat.reshape(-1)[offset:]
+    byte_strides = tuple(int(s) * flat.itemsize for s in strides)
+    return np.lib.stride_tricks.as_strided(flat, shape=tuple(shape), strides=byte_strides, writeable=False)
+
+
+def contiguous_forward(flat, shape, strides, offset=0):
+    return np.ascontiguousarray(strided_view(flat, shape, strides, offset))
+
+
+def permute_backward_into(g_out, dims, grad):
+    """grad += g_out with the permutation undone (out.shape[i] = x.shape[dims[i]])"""
+    inv = [0] * len(dims)
+    for i, d in enumerate(dims):
+        inv[d] = i
+    np.add(grad, np.ascontiguousarray(np.transpose(g_out, inv)), out=grad)
+
+
+def transpose_backward_into(g_out, dim0, dim1, grad):
+    np.add(grad, np.ascontiguousarray(np.swapaxes(g_out, dim0, dim1)), out=grad)
 
 
 # --------------------------------------------------------------------------

@@ -347,6 +347,41 @@ def test_add_with_a_broadcast_operand():
     assert_fp32_close(h_g["bias"], c_g["bias"], "bias.grad", atol=2e-5)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, BF16])
+def test_layout_ops_in_a_graph(dtype):
+    """reshape -> permute -> contiguous around compute ops, a transposed parameter and
+    a transposed activation gradient, on both devices: forward and every gradient.
+    Layout changes move bits, so the two devices differ only where GELU does."""
+    rng = np.random.default_rng(SEED + 31)
+    B, T, H, D = 3, 40, 6, 32
+    x_np = rng.standard_normal((B, T, H * D), dtype=np.float32)
+    w_np = rng.standard_normal((D, T), dtype=np.float32)
+    upstream = rng.standard_normal((B, H, D, T), dtype=np.float32)
+
+    def build(device):
+        x = make_tensor(x_np.shape, dtype, device, True, x_np)
+        w = make_tensor(w_np.shape, dtype, device, True, w_np)
+        a = ReLUSquaredOp()(x)
+        heads = a.reshape(B, T, H, D).permute(0, 2, 1, 3).contiguous()       # [B, H, T, D]: rows kernel
+        y = heads + w.transpose(0, 1).contiguous()                             # [T, D] under [B, H]: tile kernel
+        out = ReLUSquaredOp()(y).transpose(2, 3).contiguous()                  # [B, H, D, T]
+        return out.view(B, H, D * T).reshape(B, H, D, T), {"x": x, "w": w}
+
+    (c_out, c_g), (h_out, h_g) = both(build, upstream)
+    if dtype is BF16:
+        assert_bf16_close(h_out[0], c_out[0], "forward")
+        assert_bf16_close(h_g["x"], c_g["x"], "x.grad")
+        assert_bf16_close(h_g["w"], c_g["w"], "w.grad")
+    else:
+        np.testing.assert_array_equal(h_out[0], c_out[0])
+        np.testing.assert_array_equal(h_g["x"], c_g["x"])
+        assert_fp32_close(h_g["w"], c_g["w"], "w.grad", atol=2e-5)
+    if dtype is not BF16:
+        a_np = ref.relu2_forward(x_np)
+        y_np = np.transpose(a_np.reshape(B, T, H, D), (0, 2, 1, 3)) + w_np.T
+        np.testing.assert_array_equal(c_out[0], np.swapaxes(ref.relu2_forward(y_np), 2, 3))
+
+
 def test_captured_graph_replays_match_eager():
     """Record forward + zero_grad + upstream copy + backward of the tiny GPT-2 chain
     once, replay it several times with eager work and synchronisations in between,

@@ -36,7 +36,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_library_reports_errors_without_gpu_or_kernel():
     lib = capi.load_library()
-    assert lib.agrad_kernel_count() == 30
+    assert lib.agrad_kernel_count() == 32
     names = [lib.agrad_kernel_name(i).decode() for i in range(lib.agrad_kernel_count())]
     for n in ("layernorm_forward", "layernorm_backward_kernel", "rmsnorm_forward", "rmsnorm_backward",
               "gelu_forward_kernel", "gelu_backward_kernel", "swiglu_forward_kernel", "rope_qk_inplace",
@@ -125,6 +125,80 @@ def test_op_shapes_and_errors():
     assert (x + x).op.op.op_name == "Add" and x.gelu().op.op.op_name == "GELU"
     # requires_grad propagates; gather ignores the integer operand
     assert not GatherOp()(ids, T((11, 8), requires_grad=False)).requires_grad
+
+
+def test_layout_ops_shapes_strides_and_errors():
+    """View / Reshape / Permute / Transpose are views with the reference's shape and
+    stride rules (op.py:89-171, utils.py:85-109); only Contiguous reads through strides"""
+    x = T((2, 3, 4, 5))
+    assert x.strides == (60, 20, 5, 1) and x.is_contiguous
+    p = x.permute(0, 2, 1, 3)
+    assert p.shape == (2, 4, 3, 5) and p.strides == (60, 5, 20, 1) and not p.is_contiguous
+    t = x.transpose(1, 3)
+    assert t.shape == (2, 5, 4, 3) and t.strides == (60, 1, 5, 20) and not t.is_contiguous
+    assert p.transpose(-1, -2).strides == (60, 5, 1, 20)          # views compose
+    r = x.reshape(6, -1)
+    assert r.shape == (6, 20) and r.strides == (20, 1) and r.is_contiguous
+    assert x.view(-1).shape == (120,) and x.view(2, 60).op.op.op_name == "View"
+    c = p.contiguous()
+    assert c.shape == p.shape and c.is_contiguous and c.strides == contiguous_strides(p.shape)
+    for bad in (lambda: x.reshape(7, -1), lambda: x.reshape(-1, -1), lambda: x.reshape(3, 5), lambda: x.reshape(0, -1)):
+        with pytest.raises(ValueError):
+            bad()
+    with pytest.raises(ValueError):
+        x.permute(0, 1, 1, 3)
+    with pytest.raises(RuntimeError):
+        p.reshape(2, 60)            # reshape view requires contiguous input (utils.py:106-107)
+    with pytest.raises(RuntimeError):
+        p.view(2, 60)
+    with pytest.raises(RuntimeError):
+        p.gelu()                    # compute kernels read dense tensors
+    with pytest.raises(RuntimeError):
+        AddOp()(p, p)
+    assert p.contiguous().gelu().shape == p.shape
+    assert not T((2, 3), requires_grad=False).permute(1, 0).requires_grad
+
+
+def test_layout_ops_in_a_graph_on_the_oracle_device():
+    """x -> reshape -> permute -> contiguous -> gelu and a transpose branch of a
+    parameter: forward values and gradients against numpy written out directly;
+    views own no arena memory and an in-place consumer never writes through one"""
+    rng = np.random.default_rng(5)
+    B, Tn, H, D = 2, 6, 3, 4
+    x_np = rng.standard_normal((B, Tn, H * D)).astype(np.float32)
+    w_np = rng.standard_normal((D, Tn)).astype(np.float32)
+    up = rng.standard_normal((B, H, Tn, D)).astype(np.float32)
+    x, w = T((B, Tn, H * D), val=x_np), T((D, Tn), val=w_np)
+    a = x.gelu()                                     # an activation, so that its views live in the arena
+    heads = a.reshape(B, Tn, H, D).permute(0, 2, 1, 3)
+    dense = heads.contiguous()
+    out = dense + w.transpose(0, 1).contiguous()     # [Tn, D] broadcast over [B, H]
+    rt = Runtime(device="cpu")
+    rt.loss = out
+    rt.build_topo(out)
+    rt.bind_memory()
+    rt.forward()
+    from oracle import cpu_ops as K
+    a_np = K.gelu_forward(x_np)
+    want = np.transpose(a_np.reshape(B, Tn, H, D), (0, 2, 1, 3)) + w_np.T
+    np.testing.assert_array_equal(rt.backend.copy_to_host(out), want)
+    # the reshape and permute outputs are the gelu output's bytes
+    assert np.shares_memory(heads.storage.data, a.storage.data)
+    assert heads.grad.storage.data.shape == heads.shape       # a dense gradient of its own
+    rt.zero_grad()
+    rt.backend.copy_from_host(out.grad, up)
+    rt.backward_graph()
+    da = np.transpose(up, (0, 2, 1, 3)).reshape(B, Tn, H * D)
+    dx = np.zeros_like(x_np)
+    K.gelu_backward_into(x_np, np.ascontiguousarray(da), dx)
+    np.testing.assert_array_equal(rt.backend.copy_to_host(x.grad), dx)
+    np.testing.assert_allclose(rt.backend.copy_to_host(w.grad), up.sum((0, 1)).T, rtol=1e-5, atol=1e-6)
+    # second run: same numbers
+    rt.zero_grad()
+    rt.forward()
+    rt.backend.copy_from_host(out.grad, up)
+    rt.backward_graph()
+    np.testing.assert_array_equal(rt.backend.copy_to_host(x.grad), dx)
 
 
 # ---- planner ------------------------------------------------------------------------

@@ -446,3 +446,47 @@ def test_cross_entropy_closed_form_fd_and_invariants():
     fd = cf.finite_diff(lambda a: float((cf.cross_entropy(a, labels) * dloss).sum()), x, where)
     for i, val in zip(where, fd):
         assert abs(val - dx.reshape(-1)[i]) < 2e-3 * max(1.0, abs(val))
+
+
+# ---------------------------------------------------------------------------
+# strided views and the permute / transpose gradients: an explicit loop over every
+# dense index with the index arithmetic written out
+# ---------------------------------------------------------------------------
+def _loop_gather(flat, shape, strides, offset):
+    out = np.empty(shape, flat.dtype)
+    for idx in np.ndindex(*shape):
+        out[idx] = flat[offset + sum(c * s for c, s in zip(idx, strides))]
+    return out
+
+
+def test_strided_view_matches_the_index_loop():
+    rng = np.random.default_rng(SEED + 70)
+    flat = rng.standard_normal(600).astype(np.float32)
+    for shape, strides, offset in [((3, 4, 5), (20, 5, 1), 0), ((5, 4, 3), (1, 5, 20), 0), ((4, 6), (0, 2), 3),
+                                   ((2, 3, 4), (100, 1, 7), 11), ((7,), (3,), 2)]:
+        got = K.contiguous_forward(flat, shape, strides, offset)
+        assert got.flags["C_CONTIGUOUS"]
+        np.testing.assert_array_equal(got, _loop_gather(flat, shape, strides, offset))
+
+
+def test_permute_and_transpose_gradients_match_the_index_loop():
+    rng = np.random.default_rng(SEED + 71)
+    xshape = (2, 3, 4, 5)
+    for dims in [(0, 2, 1, 3), (3, 2, 1, 0), (1, 3, 0, 2)]:
+        oshape = tuple(xshape[d] for d in dims)
+        g = rng.standard_normal(oshape).astype(np.float32)
+        base = rng.standard_normal(xshape).astype(np.float32)
+        want = base.copy()
+        for idx in np.ndindex(*xshape):       # out[j] = x[idx] where j[i] = idx[dims[i]]
+            want[idx] = base[idx] + g[tuple(idx[d] for d in dims)]
+        got = base.copy()
+        K.permute_backward_into(g, list(dims), got)
+        np.testing.assert_array_equal(got, want)
+    g = rng.standard_normal((2, 5, 4, 3)).astype(np.float32)
+    base = rng.standard_normal(xshape).astype(np.float32)
+    want = base.copy()
+    for idx in np.ndindex(*xshape):
+        want[idx] = base[idx] + g[idx[0], idx[3], idx[2], idx[1]]
+    got = base.copy()
+    K.transpose_backward_into(g, 1, 3, got)
+    np.testing.assert_array_equal(got, want)
