@@ -115,6 +115,9 @@ class Runtime:
         # only a backend whose kernels honour OpNode.overwrite_grads can skip the fills
         self.fuse_grad_zeroing = bool(fuse_grad_zeroing and getattr(self.backend, "supports_grad_store", False))
         self.arena_bytes = 0
+        self._owns_arena = False       # release() frees only an arena this runtime allocated
+        self.memory_plan = None        # key -> arena offset, set by plan_memory()
+        self._keyobj = {}
         self.leaves = []
         self.consumers = {}
         self._alias_of = {}            # output tensor -> input tensor it shares memory and gradient with
@@ -269,6 +272,23 @@ class Runtime:
 
     # -- memory ------------------------------------------------------------------
     def bind_memory(self):
+        """plan the arena, allocate it and bind every view (runtime.py:272-513)"""
+        self.plan_memory(force=True)
+        if self.arena_bytes == 0:
+            self.unified_arena = None
+            return
+        print(f"Training arena need {self.arena_bytes}")
+        self.unified_arena = self.allocator.empty((self.arena_bytes,), np.uint8)
+        self._owns_arena = True
+        print(f"[ARENA-TRAIN-ALLOC] bytes={self.arena_bytes} "
+              f"buffer_id={getattr(self.unified_arena.ptr, 'buffer_id', None)}", flush=True)
+        self._bind_views()
+
+    def plan_memory(self, force=False):
+        """lifetimes -> first-fit offsets in one arena; allocates nothing
+        (runtime.py:515-716).  Sets arena_bytes and returns {key: offset}."""
+        if self.memory_plan is not None and not force:
+            return self.memory_plan
         n = len(self.topo)
         steps = [(0, node) for node in self.topo]
         if not self.forward_only:
@@ -352,30 +372,28 @@ class Runtime:
 
         self.arena_bytes = planner.peak
         self.memory_plan = {k: planner.get_offset(k) for k in life}
-        if planner.peak == 0:
-            self.unified_arena = None
-            return
-        print(f"Training arena need {planner.peak}")
-        self.unified_arena = self.allocator.empty((planner.peak,), np.uint8)
-        print(f"[ARENA-TRAIN-ALLOC] bytes={planner.peak} "
-              f"buffer_id={getattr(self.unified_arena.ptr, 'buffer_id', None)}", flush=True)
-        self._bind_views(planner, keyobj)
-
-    def bind_memory_new(self, arena):
-        """re-point every planned view at another arena of at least the same size
-        (runtime.py:718-732)"""
-        if arena.nbytes < self.arena_bytes:
-            raise RuntimeError(f"arena of {arena.nbytes} bytes is smaller than the plan ({self.arena_bytes})")
-        self.unified_arena = arena
-        planner = MemoryPlanner()
-        planner.offsets = dict(self.memory_plan)
-        self._bind_views(planner, self._keyobj)
-
-    def _bind_views(self, planner, keyobj):
         self._keyobj = keyobj
+        return self.memory_plan
+
+    def bind_memory_new(self, arena=None):
+        """bind every planned view into `arena` (allocated here when None): several
+        runtimes -- a training plan and an inference plan over the same parameters --
+        can live in one arena sized for the largest (runtime.py:718-732)"""
+        self.plan_memory()
+        self._owns_arena = False
+        if arena is None and self.arena_bytes:
+            arena = self.allocator.empty((self.arena_bytes,), np.uint8)
+            self._owns_arena = True
+            print(f"[ARENA-ALLOC] bytes={arena.nbytes} buffer_id={getattr(arena.ptr, 'buffer_id', None)}", flush=True)
+        if self.arena_bytes and arena.nbytes < self.arena_bytes:
+            raise RuntimeError(f"arena too small: need={self.arena_bytes}, have={arena.nbytes}")
+        self.unified_arena = arena
+        self._bind_views()
+
+    def _bind_views(self):
         arena = self.unified_arena
-        for k, obj in keyobj.items():
-            off = planner.get_offset(k)
+        for k, obj in self._keyobj.items():
+            off = self.memory_plan[k]
             if isinstance(obj, _Scratch):
                 node = obj.node
                 layout = node.scratch_fwd_layout if obj.phase == 0 else node.scratch_bwd_layout
@@ -442,7 +460,12 @@ class Runtime:
                         continue
                     self.backend.fill(t.grad, 0)
 
+    def _require_bound(self):
+        if self.memory_plan is not None and self.arena_bytes and self.unified_arena is None:
+            raise RuntimeError("this runtime's memory is planned but not bound: call bind_memory_new / bind_to first")
+
     def forward(self):
+        self._require_bound()
         self._sync_backend()
         self.backend.begin_pass()
         for node in self.topo:
@@ -450,6 +473,7 @@ class Runtime:
         self.backend.end_pass()
 
     def backward_graph(self):
+        self._require_bound()
         self._sync_backend()
         self.backend.begin_pass()
         for node in reversed(self.topo):
@@ -485,9 +509,77 @@ class Runtime:
         if rel is None:
             return
         self.backend.synchronize()
-        if self.unified_arena is not None:
+        if self.unified_arena is not None and self._owns_arena:
             rel(self.unified_arena)
-            self.unified_arena = None
+        self.unified_arena = None
+        self._owns_arena = False
         for slab in self._slabs:
             rel(slab)
         self._slabs = []
+
+
+# -- execution plans (runtime.py:857-947) -------------------------------------------
+class ExecutionPlan:
+    """A compiled graph with named feed tensors.  Several plans -- a training step
+    and forward-only plans at other sequence lengths -- are prepared separately,
+    then bound into ONE arena sized for the largest (`bind_plans`), the way the
+    reference's engine shares its training arena with the decode plans
+    (engine.py:133-170).  Method names are the reference's."""
+
+    def __init__(self, runtime, input_ids, output, target_ids=None, row_scale=None, seq_len=0, mode="train"):
+        self.runtime = runtime
+        self.input_ids = input_ids
+        self.target_ids = target_ids
+        self.row_scale = row_scale
+        self.output = output
+        self.seq_len = seq_len
+        self.mode = mode
+
+    def prepare(self):
+        rt = self.runtime
+        rt.loss = self.output
+        rt.build_topo(self.output)
+        rt.plan_memory(force=True)
+        rt.is_compiled = True
+        return self
+
+    def bind_to(self, arena):
+        self.runtime.bind_memory_new(arena)
+
+    def _feed(self, tensor, values, what):
+        if tensor is None:
+            raise ValueError(f"this plan has no {what}")
+        self.runtime.backend.copy_from_host(tensor, values)
+
+    def set_inputs(self, values):
+        self._feed(self.input_ids, values, "input tensor")
+
+    def set_targets(self, values):
+        self._feed(self.target_ids, values, "target tensor")
+
+    def set_row_scale(self, values):
+        self._feed(self.row_scale, values, "row scale tensor")
+
+    def forward(self, feeds=None, return_value=True):
+        return self.runtime.run_forward(self.output, feeds=feeds, return_value=return_value)
+
+    def backward(self, grad_scale=1.0, accumulate_parameter_grads=False):
+        if self.runtime.forward_only:
+            raise ValueError("inference plan cannot use backward()")
+        self.runtime.backward(self.output, grad_scale=grad_scale,
+                              accumulate_parameter_grads=accumulate_parameter_grads)
+
+
+def bind_plans(plans, arena=None):
+    """bind prepared plans into one arena (allocated with the first plan's allocator
+    when None) big enough for the largest; returns the arena.  The plans then
+    overwrite each other's activations: run one at a time."""
+    plans = list(plans)
+    need = max((p.runtime.arena_bytes for p in plans), default=0)
+    if arena is None and need:
+        arena = plans[0].runtime.allocator.empty((need,), np.uint8)
+    if need and arena.nbytes < need:
+        raise RuntimeError(f"arena too small: need={need}, have={arena.nbytes}")
+    for p in plans:
+        p.bind_to(arena)
+    return arena

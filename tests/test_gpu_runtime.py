@@ -12,7 +12,7 @@ import pytest
 from autograd_amd.device import Device
 from autograd_amd.op import (AddLayerNormOp, AddOp, AddRMSNormOp, EmbeddingSumOp, GatherOp, GELUOp,
                              LayerNormOp, ReLUSquaredOp, RMSNormOp, RopeOp, SwiGLUOp)
-from autograd_amd.runtime import Runtime
+from autograd_amd.runtime import ExecutionPlan, Runtime, bind_plans
 from autograd_amd.tensor import Tensor
 from autograd_amd.utils import BF16
 from oracle import cpu_device
@@ -380,6 +380,58 @@ def test_layout_ops_in_a_graph(dtype):
         a_np = ref.relu2_forward(x_np)
         y_np = np.transpose(a_np.reshape(B, T, H, D), (0, 2, 1, 3)) + w_np.T
         np.testing.assert_array_equal(c_out[0], np.swapaxes(ref.relu2_forward(y_np), 2, 3))
+
+
+def test_execution_plans_share_one_arena():
+    """training plan + forward-only plan at another length over the same parameters,
+    bound into one device arena (ExecutionPlan, runtime.py:857-892): alternating runs
+    reproduce the oracle device's results for each plan"""
+    rng = np.random.default_rng(SEED + 32)
+    V, C = 301, 96
+    w_np = (0.5 * rng.standard_normal((V, C))).astype(np.float32)
+    g_np = (1 + 0.1 * rng.standard_normal(C)).astype(np.float32)
+    feeds = {"train": rng.integers(0, V, (4, 48), dtype=np.int32), "eval": rng.integers(0, V, (1, 20), dtype=np.int32)}
+
+    def plans(device):
+        w = make_tensor((V, C), np.float32, device, True, w_np, "w")
+        g = make_tensor((C,), np.float32, device, True, g_np, "g")
+        out = {}
+        for mode, ids_np in feeds.items():
+            fwd_only = mode == "eval"
+            ids = Tensor(shape=ids_np.shape, dtype=np.int32, device=device, requires_grad=False, name=mode)
+            x = ids.gather(w)
+            h, y = AddRMSNormOp(eps=1e-6)(x, ReLUSquaredOp()(x), g)
+            o = (h + y).reshape(ids_np.size, C)
+            rt = Runtime(device=device, forward_only=fwd_only, owns_params=not fwd_only)
+            out[mode] = ExecutionPlan(runtime=rt, input_ids=ids, output=o, seq_len=ids_np.shape[1], mode=mode).prepare()
+        arena = bind_plans(out.values())
+        assert arena.nbytes == max(p.runtime.arena_bytes for p in out.values())
+        return out, w, g, arena
+
+    results = {}
+    for device in ("cpu", "hip"):
+        ps, w, g, arena = plans(device)
+        runs = []
+        for _ in range(2):
+            ps["train"].set_inputs(feeds["train"])
+            ps["train"].backward()
+            be = ps["train"].runtime.backend
+            be.synchronize()
+            runs.append((be.copy_to_host(ps["train"].output), be.copy_to_host(w.grad), be.copy_to_host(g.grad)))
+            ps["eval"].set_inputs(feeds["eval"])
+            runs.append((ps["eval"].forward(),))
+        results[device] = runs
+        ps["train"].runtime.release()
+        ps["eval"].runtime.release()
+        if hasattr(ps["train"].runtime.allocator, "release"):
+            ps["train"].runtime.allocator.release(arena)     # bind_plans' arena belongs to the caller
+    for c_run, h_run in zip(results["cpu"], results["hip"]):
+        for c_arr, h_arr in zip(c_run, h_run):
+            assert_fp32_close(h_arr, c_arr, "plan result", atol=5e-6)
+    # the second round equals the first on the device, bit for bit
+    for a, b in zip(results["hip"][:2], results["hip"][2:]):
+        for x0, x1 in zip(a, b):
+            np.testing.assert_array_equal(x0, x1)
 
 
 def test_captured_graph_replays_match_eager():

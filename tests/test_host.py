@@ -10,7 +10,7 @@ from autograd_amd import capi
 from autograd_amd.device import Device
 from autograd_amd.op import (AddLayerNormOp, AddOp, AddRMSNormOp, EmbeddingSumOp, GatherOp, GELUOp,
                              LayerNormOp, RMSNormOp, RopeOp, SwiGLUOp)
-from autograd_amd.runtime import MemoryPlanner, Runtime
+from autograd_amd.runtime import ExecutionPlan, MemoryPlanner, Runtime, bind_plans
 from autograd_amd.tensor import Tensor
 from autograd_amd.utils import BF16, bf16_bits, broadcast_shape, contiguous_strides, f32_bits, itemsize
 from oracle import cpu_device
@@ -199,6 +199,70 @@ def test_layout_ops_in_a_graph_on_the_oracle_device():
     rt.backend.copy_from_host(out.grad, up)
     rt.backward_graph()
     np.testing.assert_array_equal(rt.backend.copy_to_host(x.grad), dx)
+
+
+def _plan_graph(device, w, g, B, Tn, forward_only, owns_params=None):
+    ids = Tensor(shape=(B, Tn), dtype=np.int32, device=device, requires_grad=False, name=f"ids_{Tn}")
+    x = ids.gather(w)
+    h, y = x.add_rms_norm(x.gelu(), g)
+    out = (h + y).reshape(B * Tn, -1)
+    rt = Runtime(device=device, forward_only=forward_only,
+                 owns_params=(not forward_only) if owns_params is None else owns_params)
+    return ExecutionPlan(runtime=rt, input_ids=ids, output=out, seq_len=Tn, mode="eval" if forward_only else "train")
+
+
+def test_execution_plans_share_one_arena_on_the_oracle_device():
+    """a training plan and a forward-only plan at another length over the same
+    parameters, prepared separately and bound into one arena sized for the larger
+    (ExecutionPlan.prepare / bind_to, runtime.py:857-892; engine.py:133-170): each
+    gives what a runtime of its own gives"""
+    rng = np.random.default_rng(11)
+    V, C = 29, 16
+    w_np = rng.standard_normal((V, C)).astype(np.float32)
+    g_np = (1 + 0.1 * rng.standard_normal(C)).astype(np.float32)
+    ids_train = rng.integers(0, V, (2, 8), dtype=np.int32)
+    ids_eval = rng.integers(0, V, (1, 5), dtype=np.int32)
+
+    def solo(ids_np, forward_only):
+        w, g = T((V, C), val=w_np), T((C,), val=g_np)
+        plan = _plan_graph("cpu", w, g, *ids_np.shape, forward_only, owns_params=True)
+        rt = plan.runtime
+        rt.loss = plan.output
+        rt.build_topo(plan.output)
+        rt.bind_memory()
+        rt.is_compiled = True
+        rt.backend.copy_from_host(plan.input_ids, ids_np)
+        if forward_only:
+            return plan.forward(), None
+        plan.backward()
+        return rt.backend.copy_to_host(plan.output), rt.backend.copy_to_host(w.grad)
+
+    want_train, want_dw = solo(ids_train, False)
+    want_eval, _ = solo(ids_eval, True)
+
+    w, g = T((V, C), val=w_np), T((C,), val=g_np)
+    train = _plan_graph("cpu", w, g, 2, 8, False).prepare()       # owns the parameters
+    evalp = _plan_graph("cpu", w, g, 1, 5, True).prepare()        # borrows them
+    assert train.runtime.arena_bytes > evalp.runtime.arena_bytes > 0
+    with pytest.raises(RuntimeError):
+        train.forward()                                           # planned, not bound
+    arena = bind_plans([train, evalp])
+    assert arena.nbytes == train.runtime.arena_bytes
+    assert train.runtime.unified_arena is arena and evalp.runtime.unified_arena is arena
+    for _ in range(2):                                            # alternate: each plan re-runs cleanly
+        train.set_inputs(ids_train)
+        train.backward()
+        np.testing.assert_array_equal(train.runtime.backend.copy_to_host(train.output), want_train)
+        np.testing.assert_array_equal(train.runtime.backend.copy_to_host(w.grad), want_dw)
+        evalp.set_inputs(ids_eval)
+        np.testing.assert_array_equal(evalp.forward(), want_eval)
+    with pytest.raises(ValueError):
+        evalp.backward()
+    with pytest.raises(ValueError):
+        evalp.set_targets(ids_eval)
+    small = train.runtime.allocator.empty((evalp.runtime.arena_bytes,), np.uint8)
+    with pytest.raises(RuntimeError):
+        train.bind_to(small)
 
 
 # ---- planner ------------------------------------------------------------------------
