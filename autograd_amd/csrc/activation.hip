@@ -81,7 +81,7 @@ __device__ __forceinline__ float sigmoid_ref(float g) {
 }
 
 // The sigmoid by I/O type.  fp32 tensors get the reference's sequence (accurate
-// expf, IEEE division).  bf16 tensors round their result to 8 significant bits,
+// expf, IEEE division: the fp32 kernels are memory-bound with it).  bf16 tensors round their result to 8 significant bits,
 // and at 2 bytes per element the accurate sequence (about 25 instructions) makes
 // the kernel instruction-bound rather than memory-bound; the hardware exp2 and
 // reciprocal (1 ulp each) are indistinguishable after the bf16 rounding.
