@@ -34,6 +34,16 @@ namespace {
 
 constexpr int kMaxEPT = 24;  // most elements of a row a thread may keep in registers
 
+// a * b + c.  fp32 tensors: two roundings, like the CPU kernels (bit-level
+// closeness to numpy).  bf16 tensors: one fused instruction -- their results are
+// rounded to 8 bits anyway, and at 2 bytes per element the instruction count, not
+// HBM, is what the norm kernels run into first.
+template <typename T>
+__device__ __forceinline__ float mad(float a, float b, float c) {
+    if constexpr (sizeof(T) == 2) return __builtin_fmaf(a, b, c);
+    else return a * b + c;
+}
+
 template <typename T>
 struct NormFwdArgs {
     const T* x; const T* res; const float* gamma; const float* beta; T* h; T* y;
@@ -216,7 +226,7 @@ norm_fwd_kernel(const NormFwdArgs<T> a) {
             for (int k = 0; k < VEC; ++k) {
                 const float d = on[i] ? (v[i][k] - mean) : 0.0f;
                 v[i][k] = d;
-                q = q + d * d;
+                q = mad<T>(d, d, q);
             }
         const float var = row_sum<TPR>(q, lds, 1) / fC;
         scale = 1.0f / sqrtf(var + a.eps);
@@ -225,7 +235,7 @@ norm_fwd_kernel(const NormFwdArgs<T> a) {
 #pragma unroll
         for (int i = 0; i < NV; ++i)
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) q = q + v[i][k] * v[i][k];
+            for (int k = 0; k < VEC; ++k) q = mad<T>(v[i][k], v[i][k], q);
         const float ms = row_sum<TPR>(q, lds, 0) / fC;
         scale = 1.0f / sqrtf(ms + a.eps);
     }
@@ -349,10 +359,10 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
 #pragma unroll
             for (int k = 0; k < VEC; ++k) {
                 const float d = xv[i][k];
-                q = q + d * d;
+                q = mad<T>(d, d, q);
                 const float dyg = g[i][k] * gam[i][k];
                 s1 = s1 + dyg;
-                s2 = s2 + dyg * d;
+                s2 = mad<T>(dyg, d, s2);
             }
         if (a.dx != nullptr) row_sum3<TPR>(q, s1, s2, lds, ring.next());
         else q = row_sum<TPR>(q, lds, ring.next());
@@ -365,7 +375,7 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
             for (int k = 0; k < VEC; ++k) {
                 const float xh = xv[i][k] * scale;
                 xv[i][k] = xh;
-                if (want_pg) pg[i][k] = pg[i][k] + g[i][k] * xh;
+                if (want_pg) pg[i][k] = mad<T>(g[i][k], xh, pg[i][k]);
                 if (want_pb) pb[i][k] = pb[i][k] + g[i][k];
                 g[i][k] = g[i][k] * gam[i][k];
             }
@@ -386,14 +396,13 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
                     if (is_ln) {
 #pragma unroll
                         for (int k = 0; k < VEC; ++k) {
-                            float u = g[i][k] * scale;
-                            u = u - c1;
-                            t[k] = u - xv[i][k] * c2;
+                            const float u = mad<T>(g[i][k], scale, -c1);
+                            t[k] = mad<T>(-xv[i][k], c2, u);
                         }
                     } else {
 #pragma unroll
                         for (int k = 0; k < VEC; ++k)
-                            t[k] = (g[i][k] - xv[i][k] * c2) * scale;
+                            t[k] = mad<T>(-xv[i][k], c2, g[i][k]) * scale;
                     }
                     if (a.dres != nullptr) {
                         float r[VEC];
