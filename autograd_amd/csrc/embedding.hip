@@ -368,6 +368,33 @@ __device__ __forceinline__ ChunkEdges chunk_edges(const uint32_t* tok_s, uint32_
     return e;
 }
 
+// VEC consecutive floats of a carry row (fp32 partial sums in the workspace): as
+// 16-byte accesses when VEC is a multiple of 4 (the rows are 16-byte aligned and
+// col is a multiple of VEC then), cached -- the fix-up kernel re-reads them at once
+template <int VEC>
+__device__ __forceinline__ void load_carry(const float* __restrict__ p, float (&v)[VEC]) {
+    if constexpr (VEC % 4 == 0) {
+#pragma unroll
+        for (int k = 0; k < VEC; k += 4) {
+            const float4 t = *reinterpret_cast<const float4*>(p + k);
+            v[k] = t.x; v[k + 1] = t.y; v[k + 2] = t.z; v[k + 3] = t.w;
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) v[k] = p[k];
+    }
+}
+template <int VEC>
+__device__ __forceinline__ void store_carry(float* __restrict__ p, const float (&v)[VEC]) {
+    if constexpr (VEC % 4 == 0) {
+#pragma unroll
+        for (int k = 0; k < VEC; k += 4) *reinterpret_cast<float4*>(p + k) = make_float4(v[k], v[k + 1], v[k + 2], v[k + 3]);
+    } else {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) p[k] = v[k];
+    }
+}
+
 template <typename T, int VEC>
 __device__ __forceinline__ void store_grad_row(T* dW, uint64_t off, const float (&acc)[VEC], bool accumulate) {
     float o[VEC];
@@ -440,9 +467,7 @@ emb_segment_sum_kernel(const uint32_t* __restrict__ tok_s, const uint32_t* __res
                         if (have && cur < V) {
                             // the finished run cannot touch the chunk's right edge
                             if (run_is_first && e.open_left) {
-#pragma unroll
-                                for (int k = 0; k < VEC; ++k)
-                                    carry_head[(uint64_t)blockIdx.x * C + col + k] = acc[k];
+                                store_carry<VEC>(carry_head + (uint64_t)blockIdx.x * C + col, acc);
                             } else {
                                 store_grad_row<T, VEC>(dW, (uint64_t)cur * C + col, acc, accumulate != 0);
                             }
@@ -459,11 +484,9 @@ emb_segment_sum_kernel(const uint32_t* __restrict__ tok_s, const uint32_t* __res
         // the last run ends at the chunk's right edge
         if (have && cur < V) {
             if (run_is_first && e.open_left) {
-#pragma unroll
-                for (int k = 0; k < VEC; ++k) carry_head[(uint64_t)blockIdx.x * C + col + k] = acc[k];
+                store_carry<VEC>(carry_head + (uint64_t)blockIdx.x * C + col, acc);
             } else if (e.open_right) {
-#pragma unroll
-                for (int k = 0; k < VEC; ++k) carry_tail[(uint64_t)blockIdx.x * C + col + k] = acc[k];
+                store_carry<VEC>(carry_tail + (uint64_t)blockIdx.x * C + col, acc);
             } else {
                 store_grad_row<T, VEC>(dW, (uint64_t)cur * C + col, acc, accumulate != 0);
             }
@@ -485,6 +508,45 @@ emb_segment_sum_kernel(const uint32_t* __restrict__ tok_s, const uint32_t* __res
 //     lane order: a fixed association, the same on every run.
 // Run ends come from binary searches on "equals this token" over the sorted
 // positions (equal tokens are contiguous whichever sorter ran).
+// One end of the run of `tok` that position `at` touches, found by the whole
+// workgroup (every thread must call it, with the same arguments).
+//   FORWARD:  tok_s[at - 1] == tok; returns the smallest p >= at with p == N or tok_s[p] != tok.
+//   backward: tok_s[at] == tok;     returns the smallest p <= at with tok_s[p..at] all == tok.
+// Each step probes blockDim.x evenly spaced positions of the bracket (the first
+// step takes the positions next to `at`, where most runs end) and counts the
+// probes that still see the token: equal tokens are contiguous, so those are the
+// probes nearest to `at`.
+template <bool FORWARD>
+__device__ __forceinline__ uint32_t run_edge(const uint32_t* __restrict__ tok_s, uint32_t tok, uint32_t at, uint32_t N) {
+    const uint32_t nt = blockDim.x;
+    // distance from `at` (0, 1, 2, ... outwards) of the first position that is not `tok`, in [lo, hi]
+    uint32_t lo = FORWARD ? 0u : 1u;
+    uint32_t hi = FORWARD ? N - at : at + 1;     // at distance hi the array ends
+    uint32_t step = 1;
+    while (lo < hi) {
+        const uint64_t d = (uint64_t)lo + (uint64_t)threadIdx.x * step;   // probes lo, lo + step, ...
+        int same = 0;
+        if (d < hi) same = tok_s[FORWARD ? at + (uint32_t)d : at - (uint32_t)d] == tok;
+        const uint32_t cnt = (uint32_t)__syncthreads_count(same);
+        // probes 0 .. cnt-1 see the token, probe cnt (if any) does not
+        const uint32_t new_lo = cnt ? lo + (cnt - 1) * step + 1 : lo;
+        const uint64_t cap = (uint64_t)lo + (uint64_t)cnt * step;
+        const uint32_t new_hi = cap < hi ? (uint32_t)cap : hi;
+        if (cnt == nt && new_lo < hi) {
+            // every probe matched: widen the stride so that the next step spans the rest
+            lo = new_lo;
+            const uint32_t span = hi - lo;
+            step = (span + nt - 1) / nt;
+        } else {
+            lo = new_lo;
+            hi = new_hi;
+            const uint32_t span = hi > lo ? hi - lo : 0;
+            step = span ? (span + nt - 1) / nt : 1;
+        }
+    }
+    return FORWARD ? at + lo : at + 1 - lo;
+}
+
 constexpr int kFixCols = 64;    // column vectors per slab
 constexpr int kFixLanes = 4;    // partial-sum lanes per column
 constexpr int kFixBatch = 8;    // partial rows a lane keeps in flight
@@ -504,36 +566,20 @@ emb_carry_fix_kernel(const uint32_t* __restrict__ tok_s, T* dW, const float* __r
     if (tok >= V) return;
     // Equal tokens are contiguous, but the order of distinct tokens is the
     // sorter's business (the grouping sort orders by hash group first), so the
-    // searches below test "equals tok", galloping outwards from the chunk (most
-    // runs end in the next chunk) and then bisecting the bracket.
-    // First position after the run: smallest p > e.end with p == N or tok_s[p] != tok.
-    uint32_t lo = e.end + 1, hi = e.end + L < N ? e.end + L : N;
-    for (uint32_t span = L; hi < N && tok_s[hi] == tok;) {
-        lo = hi + 1;
-        span *= 2;
-        hi = span < N - hi ? hi + span : N;
-    }
-    while (lo < hi) {
-        const uint32_t mid = lo + (hi - lo) / 2;
-        if (tok_s[mid] == tok) lo = mid + 1; else hi = mid;
-    }
-    const uint32_t c1 = (lo - 1) / L;            // chunk holding the run's last position
-    uint32_t c0 = chunk;                         // chunk holding its first
+    // searches test "equals tok".  The whole workgroup searches: one probe per
+    // thread and a barrier count per step, so a run of any length is bracketed in
+    // two or three memory round trips (a hot token's run spans thousands of
+    // positions; bisecting it with dependent loads took longer than the sums).
+    const uint32_t slabs = (CV + kFixCols - 1) / kFixCols;
     if (middle) {
-        // first position of the run: smallest p < e.start with tok_s[p] == tok
-        hi = e.start - 1;                        // known to hold tok
-        lo = hi > L ? hi - L : 0;
-        for (uint32_t span = L; lo > 0 && tok_s[lo] == tok;) {
-            hi = lo;
-            span *= 2;
-            lo = lo > span ? lo - span : 0;
-        }
-        while (lo < hi) {
-            const uint32_t mid = lo + (hi - lo) / 2;
-            if (tok_s[mid] != tok) lo = mid + 1; else hi = mid;
-        }
-        c0 = lo / L;
+        // only the first `slabs` middle chunks of a run help; one probe tells the rest
+        const uint64_t far = (uint64_t)(slabs + 1) * L;
+        if (e.start >= far && tok_s[e.start - far] == tok) return;
     }
+    const uint32_t run_end = run_edge<true>(tok_s, tok, e.end, N);        // first position after the run
+    const uint32_t c1 = (run_end - 1) / L;       // chunk holding the run's last position
+    uint32_t c0 = chunk;                         // chunk holding its first
+    if (middle) c0 = run_edge<false>(tok_s, tok, e.start, N) / L;
     const uint32_t count = c1 - c0;              // head partials live in chunks c0+1 .. c1
     const float* tail = carry_tail + (uint64_t)c0 * C;
     const float* heads = carry_head + (uint64_t)(c0 + 1) * C;
@@ -543,13 +589,11 @@ emb_carry_fix_kernel(const uint32_t* __restrict__ tok_s, T* dW, const float* __r
         for (uint32_t cv = threadIdx.x; cv < CV; cv += blockDim.x) {
             const uint32_t col = cv * VEC;
             float sum[VEC], v[kFixLanes][VEC];
-#pragma unroll
-            for (int k = 0; k < VEC; ++k) sum[k] = tail[col + k];
+            load_carry<VEC>(tail + col, sum);
 #pragma unroll
             for (int q = 0; q < kFixLanes; ++q)
                 if ((uint32_t)q < count) {
-#pragma unroll
-                    for (int k = 0; k < VEC; ++k) v[q][k] = heads[(uint64_t)q * C + col + k];
+                    load_carry<VEC>(heads + (uint64_t)q * C + col, v[q]);
                 }
 #pragma unroll
             for (int q = 0; q < kFixLanes; ++q)
@@ -562,7 +606,6 @@ emb_carry_fix_kernel(const uint32_t* __restrict__ tok_s, T* dW, const float* __r
         return;
     }
 
-    const uint32_t slabs = (CV + kFixCols - 1) / kFixCols;
     const uint32_t helpers = count - 1 < slabs ? count - 1 : slabs;   // middle chunks that take a slab
     uint32_t slab_begin, slab_end;
     if (origin) {
@@ -587,8 +630,7 @@ emb_carry_fix_kernel(const uint32_t* __restrict__ tok_s, T* dW, const float* __r
                 for (int b = 0; b < kFixBatch; ++b) {
                     const uint32_t q = q0 + (uint32_t)b * kFixLanes;
                     if (q < count) {
-#pragma unroll
-                        for (int k = 0; k < VEC; ++k) v[b][k] = heads[(uint64_t)q * C + col + k];
+                        load_carry<VEC>(heads + (uint64_t)q * C + col, v[b]);
                     }
                 }
 #pragma unroll
@@ -606,8 +648,7 @@ emb_carry_fix_kernel(const uint32_t* __restrict__ tok_s, T* dW, const float* __r
         __syncthreads();
         if (lane == 0 && live) {
             float sum[VEC];
-#pragma unroll
-            for (int k = 0; k < VEC; ++k) sum[k] = tail[col + k];
+            load_carry<VEC>(tail + col, sum);
 #pragma unroll
             for (int q = 0; q < kFixLanes; ++q)
 #pragma unroll
