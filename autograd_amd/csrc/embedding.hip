@@ -34,7 +34,9 @@ namespace {
 
 constexpr int kGatherBlock = 256;
 constexpr int kBatch = 8;          // rows a thread keeps in flight in the segmented sum
-constexpr uint32_t kMaxChunks = 2048;
+constexpr uint32_t kMaxChunks = 2048;        // chunks of the segmented sum ...
+constexpr uint32_t kMaxChunksLarge = 1024;   // ... and from kLargeRows rows on: longer chunks, fewer carry rows to fix up
+constexpr uint64_t kLargeRows = 65536;
 
 inline uint64_t align256(uint64_t v) { return (v + 255) & ~255ull; }
 
@@ -717,7 +719,8 @@ struct SumPlan {
 };
 
 void plan_sum(uint64_t N, uint32_t C, SumPlan* p) {
-    uint32_t per = (uint32_t)((N + (uint64_t)kBatch * kMaxChunks - 1) / ((uint64_t)kBatch * kMaxChunks));
+    const uint64_t max_chunks = N >= kLargeRows ? kMaxChunksLarge : kMaxChunks;
+    uint32_t per = (uint32_t)((N + (uint64_t)kBatch * max_chunks - 1) / ((uint64_t)kBatch * max_chunks));
     if (per == 0) per = 1;
     p->L = kBatch * per;
     p->chunks = (uint32_t)((N + p->L - 1) / p->L);
