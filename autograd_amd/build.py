@@ -6,6 +6,8 @@
 Produces, next to this file:
     libautograd_hip.so   the C-ABI library (include/autograd_hip.h)
     hip_ext*.so          the pybind11 module `autograd_amd.hip_ext` (HipContext)
+and tests/c_abi/layer_check, a plain-C program (gcc, C99) that calls the library
+without Python; the GPU tests run it.
 
 The reference builds its Metal extension with setuptools (setup.py:13-31); here
 the device code must be cross-compiled by hipcc for one architecture, so the
@@ -91,9 +93,23 @@ def build_extension() -> Path:
     return out
 
 
+C_CHECK_SRC = PKG.parent / "tests" / "c_abi" / "layer_check.c"
+C_CHECK_BIN = C_CHECK_SRC.with_suffix("")
+
+
+def build_c_check() -> Path:
+    """the header and the library from plain C: gcc -std=c99 -pedantic, no hipcc"""
+    _run(["gcc", "-std=c99", "-O1", "-Wall", "-Wextra", "-pedantic", "-Werror", f"-I{PKG.parent / 'include'}",
+          str(C_CHECK_SRC), f"-L{PKG}", "-lautograd_hip", "-Wl,-rpath,$ORIGIN/../../autograd_amd", "-lm",
+          "-o", str(C_CHECK_BIN)])
+    return C_CHECK_BIN
+
+
 def build_all(jobs: int = 6) -> None:
     build_library(jobs)
     build_extension()
+    if C_CHECK_SRC.exists():
+        build_c_check()
 
 
 def is_built() -> bool:

@@ -164,3 +164,15 @@ def test_single_row_single_column(ctx):
     np.testing.assert_array_equal(d_dW.download().ravel(), np.array([0, 0, 0.75, 0], np.float32))
     for d in (d_ids, d_dY, d_dW, ws):
         d.free()
+
+
+def test_plain_c_program_drives_the_library():
+    """tests/c_abi/layer_check (gcc, C99, no Python in the process) runs LayerNorm
+    forward / backward and GELU through the C ABI and checks them against the
+    textbook formulas in double precision"""
+    import subprocess
+    from pathlib import Path
+    exe = Path(__file__).parent / "c_abi" / "layer_check"
+    assert exe.exists(), f"{exe} is missing: build it with `python -m autograd_amd.build`"
+    proc = subprocess.run([str(exe)], capture_output=True, text=True, timeout=100)
+    assert proc.returncode == 0 and proc.stdout.strip() == "ok", proc.stdout + proc.stderr

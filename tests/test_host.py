@@ -34,6 +34,21 @@ def test_library_exports_every_declared_symbol():
     assert declared == set(capi.SIGNATURES), declared ^ set(capi.SIGNATURES)
 
 
+def test_header_compiles_as_plain_c(tmp_path):
+    """include/autograd_hip.h is a C header: gcc -std=c99 -pedantic accepts a
+    translation unit that includes it and takes the address of every declared function"""
+    import subprocess
+    header = (ROOT / "include" / "autograd_hip.h").read_text()
+    names = sorted(set(re.findall(r"\b(agrad_[a-z0-9_]+)\s*\(", header)) - {"agrad_ctx"})
+    src = tmp_path / "use_header.c"
+    src.write_text('#include "autograd_hip.h"\n' + "void* table[] = {\n"
+                   + "".join(f"    (void*)(unsigned long){n},\n" for n in names) + "};\n")
+    proc = subprocess.run(["gcc", "-std=c99", "-Wall", "-pedantic", "-fsyntax-only", f"-I{ROOT / 'include'}", str(src)],
+                          capture_output=True, text=True)
+    assert proc.returncode == 0, proc.stderr
+    assert len(names) >= len(capi.SIGNATURES)
+
+
 def test_library_reports_errors_without_gpu_or_kernel():
     lib = capi.load_library()
     assert lib.agrad_kernel_count() == 32
