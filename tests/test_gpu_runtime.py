@@ -158,8 +158,8 @@ def test_unknown_device_and_kernel():
 
 
 def test_config1_tiny_gpt2_chain():
-    """BASELINE config 1: ids -> wte + wpe gather-sum -> LayerNorm (gamma 1, beta 0)
-    -> GELU, B=4 T=128 C=128 V=50257, fp32, forward then backward."""
+    """The tiny-gpt2 chain (benchmark configuration 0): ids -> wte + wpe gather-sum ->
+    LayerNorm (gamma 1, beta 0) -> GELU, B=4 T=128 C=128 V=50257, fp32, forward then backward."""
     rng = np.random.default_rng(SEED + 0)
     B, T, C, V = 4, 128, 128, 50257
     ids_np = rng.integers(0, V, size=(B, T), dtype=np.int32)
