@@ -307,6 +307,14 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
     }
 }
 
+// log2 of the number of hash groups (= ordering workgroups).  128 for all but tiny
+// inputs: beside the forward gather they take a quarter of the GPU's thread slots
+// for a few microseconds (256 took half: forward 13.2 -> 11.8 us at 16384 x 384
+// fp32, 38 -> 36.5 us at 16384 x 1536), and 64 make each group's ranking too long.
+// The stand-alone sort uses the same number, so that both ways to the order give
+// the same order and the gradient sums associate identically.
+inline uint32_t group_sort_log2g(uint32_t n) { return n > 1024 ? 7u : 4u; }
+
 __global__ void __launch_bounds__(kSortBlock)
 emb_group_sort_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ tok_s,
                       uint32_t* __restrict__ row_s, unsigned long long* __restrict__ spill,
@@ -803,7 +811,7 @@ int launch_embedding_sort(hipStream_t s, const int32_t* ids, uint32_t* order, vo
     if (n <= kGroupSortMaxN && group_sort_enabled()) {
         static_assert(sizeof(unsigned long long) == 2 * sizeof(uint32_t), "spill layout");
         unsigned long long* spill = reinterpret_cast<unsigned long long*>(ws + p.off_keys_in);
-        const uint32_t log2G = n > 1024 ? 8u : 4u;
+        const uint32_t log2G = group_sort_log2g(n);
         hipLaunchKernelGGL(emb_group_sort_kernel, dim3(1u << log2G), dim3(kSortBlock), 0, s, ids, tok_s, row_s,
                            spill, n, V, log2G, err_flag);
         return check_hip(hipGetLastError(), "embedding sort launch");
@@ -851,7 +859,7 @@ int launch_gather_fwd_sorted(hipStream_t s, int dtype, const int32_t* ids, const
         return set_error(AGRAD_EINVAL, "gather: sort workspace must be 256-byte aligned");
     unsigned long long* spill = reinterpret_cast<unsigned long long*>((uint8_t*)sort_workspace + p.off_keys_in);
     const uint32_t n = (uint32_t)N, CV = C / per16, total = (uint32_t)total_vec;
-    const uint32_t log2G = n > 1024 ? 8u : 4u;
+    const uint32_t log2G = group_sort_log2g(n);
     const uint32_t grid = (1u << log2G) + (total + kSortBlock - 1) / kSortBlock;
     uint32_t* tok_s = order;
     uint32_t* row_s = order + N;
