@@ -180,7 +180,7 @@ emb_prepare_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ keys,
 // out.  No atomics on global memory, and the output is the same on every
 // run.  A group too large for LDS (one token holding a large share of all rows)
 // is gathered into its output slice and sorted there instead.
-constexpr int kSortBlock = 1024;
+constexpr int kSortBlock = 512;
 constexpr uint32_t kGroupSortMaxN = 16384;
 constexpr uint32_t kSortLdsEntries = 4096;   // (token, row) pairs a workgroup keeps in LDS
 constexpr uint32_t kRankSortMax = kSortBlock;  // lists up to one key per thread are placed by rank
