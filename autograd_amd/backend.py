@@ -29,15 +29,17 @@ from math import prod
 
 import numpy as np
 
-from .op import (AddLayerNormOp, AddOp, AddRMSNormOp, ContiguousOp, CrossEntropyLossOp, EmbeddingSumOp, GatherOp,
-                 GELUOp, LayerNormOp, PermuteOp, ReLUSquaredOp, ReshapeOp, RMSNormOp, RopeOp, SwiGLUOp,
-                 TransposeOp, ViewOp)
+from .op import (AddLayerNormOp, AddOp, AddRMSNormOp, ContiguousOp, CrossEntropyLossOp, EmbeddingSumOp, ExpOp,
+                 GatherOp, GELUOp, LayerNormOp, LogOp, MulOp, PermuteOp, ReLUSquaredOp, ReshapeOp, RMSNormOp, RopeOp,
+                 RsqrtOp, SoftmaxOp, SwiGLUOp, TransposeOp, ViewOp)
 from .scratch import single_slot
 from .utils import (bf16_bits, bf16_bits_to_f32_array, contiguous_strides, f32_array_to_bf16_bits, f32_bits,
-                    is_bf16, xavier_uniform)
+                    is_bf16, mul_bcast_kind, xavier_uniform)
 
 F32, BF16 = 0, 1
 ACC_INPUT_GRAD, ACC_PARAM_GRAD, ACC_INPUT_GRAD2, ACC_PARAM_GRAD2 = 1, 2, 4, 8
+UNARY_OPS = {ExpOp: 0, LogOp: 1, RsqrtOp: 2}
+MUL_KINDS = {"same": 0, "row": 1, "col": 2, "scalar": 3}
 
 
 class Backend:
@@ -152,6 +154,11 @@ class HipBackend(Backend):
             AddRMSNormOp: self.hip_add_norm_forward,
             RopeOp: self.hip_rope_forward,
             CrossEntropyLossOp: self.hip_cross_entropy_forward,
+            MulOp: self.hip_mul_forward,
+            ExpOp: self.hip_unary_forward,
+            LogOp: self.hip_unary_forward,
+            RsqrtOp: self.hip_unary_forward,
+            SoftmaxOp: self.hip_softmax_forward,
             ViewOp: self.hip_view_forward,
             ReshapeOp: self.hip_view_forward,
             PermuteOp: self.hip_view_forward,
@@ -171,6 +178,11 @@ class HipBackend(Backend):
             AddRMSNormOp: self.hip_add_norm_backward,
             RopeOp: self.hip_rope_backward,
             CrossEntropyLossOp: self.hip_cross_entropy_backward,
+            MulOp: self.hip_mul_backward,
+            ExpOp: self.hip_unary_backward,
+            LogOp: self.hip_unary_backward,
+            RsqrtOp: self.hip_unary_backward,
+            SoftmaxOp: self.hip_softmax_backward,
             ViewOp: self.hip_dense_grad_backward,
             ReshapeOp: self.hip_dense_grad_backward,
             PermuteOp: self.hip_permute_backward,
@@ -230,6 +242,13 @@ class HipBackend(Backend):
                     need = max(need, self.ctx.broadcast_grad_workspace_bytes(out.numel // t.numel, t.numel))
             if need:
                 return None, single_slot("workspace", need)
+        if isinstance(op, MulOp):
+            x, y = node.inputs
+            if y.requires_grad:
+                kind, lead, inner = self._mul_geometry(x, y)
+                need = self.ctx.mul_backward_workspace_bytes(kind, lead, inner)
+                if need:
+                    return None, single_slot("workspace", need)
         if isinstance(op, (GatherOp, EmbeddingSumOp)):
             ids, w = node.inputs[0], node.inputs[1]
             if w.requires_grad:
@@ -285,6 +304,77 @@ class HipBackend(Backend):
                              + _lo_hi(ws.nbytes if ws is not None else 0) + [_mask(out.grad, t.grad, ws)])
             else:
                 raise RuntimeError(f"Unsupported Add backward shape: {t.shape} from {out.shape}")
+
+    # -- Mul, Exp, Log, Rsqrt, Softmax (backend.py:107-146, 320-374) ------------------
+    @staticmethod
+    def _mul_geometry(x, y):
+        """(native kind, lead, inner) of x * y: x is seen as [lead, inner]"""
+        kind = mul_bcast_kind(x.shape, y.shape)
+        if kind in ("row", "col"):
+            inner = x.shape[-1]
+        elif kind == "scalar":
+            inner = x.shape[-1] if x.ndim else 1      # rows of the full sum's first stage
+        else:
+            inner = x.numel
+        inner = max(inner, 1)
+        return MUL_KINDS[kind], x.numel // inner, inner
+
+    def hip_mul_forward(self, inputs, outputs, scratch=None):
+        x, y, out = inputs[0], inputs[1], outputs[0]
+        kind, lead, inner = self._mul_geometry(x, y)
+        self._launch("mul_forward_kernel", [x, y, out], [_dt(out), kind] + _lo_hi(lead) + _lo_hi(inner))
+
+    def hip_mul_backward(self, inputs, outputs, scratch=None):
+        x, y, out = inputs[0], inputs[1], outputs[0]
+        if out.grad is None:
+            return
+        node = out.op
+        kind, lead, inner = self._mul_geometry(x, y)
+        dx = x.grad if x.requires_grad and x.grad is not None else None
+        dy = y.grad if y.requires_grad and y.grad is not None else None
+        if dx is None and dy is None:
+            return
+        if x is y:
+            # x * x: both products land in the one gradient, the second call adds
+            self._launch("mul_backward_kernel", [out.grad, x, y, dx, None, None],
+                         [_dt(out), kind] + _lo_hi(lead) + _lo_hi(inner) + [self._grad_flag(node, x)] + _lo_hi(0)
+                         + [_mask(out.grad, x, y, dx, None, None)])
+            self._launch("mul_backward_kernel", [out.grad, x, y, None, dx, None],
+                         [_dt(out), kind] + _lo_hi(lead) + _lo_hi(inner) + [ACC_INPUT_GRAD2] + _lo_hi(0)
+                         + [_mask(out.grad, x, y, None, dx, None)])
+            return
+        flags = (ACC_INPUT_GRAD if dx is not None and self._grad_flag(node, x) else 0) \
+            | (ACC_INPUT_GRAD2 if dy is not None and self._grad_flag(node, y) else 0)
+        ws = scratch["workspace"] if scratch and "workspace" in scratch else None
+        self._launch("mul_backward_kernel", [out.grad, x, y, dx, dy, ws],
+                     [_dt(out), kind] + _lo_hi(lead) + _lo_hi(inner) + [flags]
+                     + _lo_hi(ws.nbytes if ws is not None else 0) + [_mask(out.grad, x, y, dx, dy, ws)])
+
+    def hip_unary_forward(self, inputs, outputs, scratch=None):
+        x, out = inputs[0], outputs[0]
+        self._launch("unary_forward", [x, out], [_dt(x), UNARY_OPS[type(out.op.op)]] + _lo_hi(x.numel))
+
+    def hip_unary_backward(self, inputs, outputs, scratch=None):
+        x, out = inputs[0], outputs[0]
+        if out.grad is None or not x.requires_grad:
+            return
+        op = out.op.op
+        saved = out if op.saves_output else x
+        self._launch("unary_backward", [out.grad, saved, x.grad],
+                     [_dt(x), UNARY_OPS[type(op)], self._grad_flag(out.op, x)] + _lo_hi(x.numel))
+
+    def hip_softmax_forward(self, inputs, outputs, scratch=None):
+        x, out = inputs[0], outputs[0]
+        V = x.shape[-1]
+        self._launch("softmax_forward", [x, out], [_dt(x)] + _lo_hi(x.numel // max(V, 1)) + [V])
+
+    def hip_softmax_backward(self, inputs, outputs, scratch=None):
+        x, out = inputs[0], outputs[0]
+        if out.grad is None or not x.requires_grad:
+            return
+        V = x.shape[-1]
+        self._launch("softmax_backward", [out, out.grad, x.grad],
+                     [_dt(x)] + _lo_hi(x.numel // max(V, 1)) + [V, self._grad_flag(out.op, x)])
 
     # -- views and layout changes (backend.py:263-318, 2754-2866) --------------------
     # View / Reshape / Permute / Transpose outputs share their input's memory, so

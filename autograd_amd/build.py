@@ -29,7 +29,7 @@ OBJ = PKG / "csrc" / "build"
 LIB = PKG / "libautograd_hip.so"
 ARCH = "gfx950"
 
-DEVICE_SOURCES = ["memops.hip", "norm.hip", "activation.hip", "rope.hip", "embedding.hip", "optimizer.hip", "loss.hip", "reduce.hip", "strided.hip"]
+DEVICE_SOURCES = ["memops.hip", "norm.hip", "activation.hip", "rope.hip", "embedding.hip", "optimizer.hip", "loss.hip", "reduce.hip", "strided.hip", "pointwise.hip"]
 HOST_SOURCES = ["context.cpp"]
 
 COMMON_FLAGS = [

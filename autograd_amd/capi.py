@@ -18,6 +18,8 @@ LIB_PATH = Path(__file__).resolve().parent / "libautograd_hip.so"
 F32, BF16 = 0, 1
 NORM_LAYER, NORM_RMS = 0, 1
 ACC_INPUT_GRAD, ACC_PARAM_GRAD, ACC_INPUT_GRAD2, ACC_PARAM_GRAD2 = 1, 2, 4, 8
+UNARY_EXP, UNARY_LOG, UNARY_RSQRT = 0, 1, 2
+MUL_SAME, MUL_ROW, MUL_COL, MUL_SCALAR = 0, 1, 2, 3
 OK, EINVAL, EHIP, ENOKERNEL, EINDEX, EWORKSPACE = 0, -1, -2, -3, -4, -5
 
 _ctx = C.c_void_p
@@ -71,6 +73,13 @@ SIGNATURES = {
     "agrad_embedding_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u64, _u32, _u32, _u32]),
     "agrad_embedding_sort_workspace_bytes": (_u64, [_u64, _u32]),
     "agrad_gather_forward_sorted": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u32, _u32, _u32, _ptr, _ptr, _u64]),
+    "agrad_unary_forward": (_int, [_ctx, _int, _int, _ptr, _ptr, _u64]),
+    "agrad_unary_backward": (_int, [_ctx, _int, _int, _ptr, _ptr, _ptr, _u64, _u32]),
+    "agrad_mul_forward": (_int, [_ctx, _int, _int, _ptr, _ptr, _ptr, _u64, _u64]),
+    "agrad_mul_backward_workspace_bytes": (_u64, [_int, _u64, _u64]),
+    "agrad_mul_backward": (_int, [_ctx, _int, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _u64, _u64, _u64, _u32]),
+    "agrad_softmax_forward": (_int, [_ctx, _int, _ptr, _ptr, _u64, _u32]),
+    "agrad_softmax_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _u64, _u32, _u32]),
     "agrad_strided_copy": (_int, [_ctx, _int, _ptr, _ptr, _int, _ptr, _ptr, _u32]),
     "agrad_embedding_backward_sorted_workspace_bytes": (_u64, [_u64, _u32]),
     "agrad_embedding_backward_sorted": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _u64, _u64, _u32, _u32, _u32, _u32]),

@@ -170,6 +170,58 @@ int h_bcast_grad(const Call& c) {
     RESOLVE_IF(c.a[8] & 4u, 2, wsb, ws)
     return launch_broadcast_grad(c.ctx->stream, (int)c.a[0], g, dy, ws, ws ? wsb : 0, lead, inner, c.a[5]);
 }
+// buffers x, y | args dtype, op, n lo, hi
+int h_unary_fwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t n = u64(c.a, 2), bytes = n * dtype_size(c.a[0]);
+    RESOLVE(0, bytes, x) RESOLVE(1, bytes, y)
+    return launch_unary_fwd(c.ctx->stream, (int)c.a[1], (int)c.a[0], x, y, n);
+}
+// buffers dy, saved, dx | args dtype, op, flags, n lo, hi
+int h_unary_bwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t n = u64(c.a, 3), bytes = n * dtype_size(c.a[0]);
+    RESOLVE(0, bytes, dy) RESOLVE(1, bytes, saved) RESOLVE(2, bytes, dx)
+    return launch_unary_bwd(c.ctx->stream, (int)c.a[1], (int)c.a[0], dy, saved, dx, n, c.a[2]);
+}
+inline uint64_t mul_small_elems(uint32_t kind, uint64_t lead, uint64_t inner) {
+    return kind == AGRAD_MUL_SAME ? lead * inner : kind == AGRAD_MUL_ROW ? inner : kind == AGRAD_MUL_COL ? lead : 1;
+}
+// buffers x, y, out | args dtype, kind, lead lo, hi, inner lo, hi
+int h_mul_fwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    if (c.a[1] > AGRAD_MUL_SCALAR) return set_error(AGRAD_EINVAL, "mul: unknown broadcast kind %u", c.a[1]);
+    const uint64_t lead = u64(c.a, 2), inner = u64(c.a, 4), es = dtype_size(c.a[0]);
+    RESOLVE(0, lead * inner * es, x) RESOLVE(1, mul_small_elems(c.a[1], lead, inner) * es, y) RESOLVE(2, lead * inner * es, out)
+    return launch_mul_fwd(c.ctx->stream, (int)c.a[0], (int)c.a[1], x, y, out, lead, inner);
+}
+// buffers g, x, y, dx, dy, workspace | args dtype, kind, lead lo, hi, inner lo, hi, flags, ws lo, hi, present_mask
+int h_mul_bwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    if (c.a[1] > AGRAD_MUL_SCALAR) return set_error(AGRAD_EINVAL, "mul backward: unknown broadcast kind %u", c.a[1]);
+    const uint64_t lead = u64(c.a, 2), inner = u64(c.a, 4), es = dtype_size(c.a[0]), wsb = u64(c.a, 7);
+    const uint64_t big = lead * inner * es, small = mul_small_elems(c.a[1], lead, inner) * es;
+    const uint32_t mask = c.a[9];
+    RESOLVE(0, big, g)
+    RESOLVE_IF(mask & 2u, 1, big, x) RESOLVE_IF(mask & 4u, 2, small, y)
+    RESOLVE_IF(mask & 8u, 3, big, dx) RESOLVE_IF(mask & 16u, 4, small, dy)
+    RESOLVE_IF(mask & 32u, 5, wsb, ws)
+    return launch_mul_bwd(c.ctx->stream, (int)c.a[0], (int)c.a[1], g, x, y, dx, dy, ws, ws ? wsb : 0, lead, inner, c.a[6]);
+}
+// buffers x, y | args dtype, rows lo, hi, V
+int h_softmax_fwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t rows = u64(c.a, 1), bytes = rows * c.a[3] * dtype_size(c.a[0]);
+    RESOLVE(0, bytes, x) RESOLVE(1, bytes, y)
+    return launch_softmax_fwd(c.ctx->stream, (int)c.a[0], x, y, rows, c.a[3]);
+}
+// buffers y, dy, dx | args dtype, rows lo, hi, V, flags
+int h_softmax_bwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t rows = u64(c.a, 1), bytes = rows * c.a[3] * dtype_size(c.a[0]);
+    RESOLVE(0, bytes, y) RESOLVE(1, bytes, dy) RESOLVE(2, bytes, dx)
+    return launch_softmax_bwd(c.ctx->stream, (int)c.a[0], y, dy, dx, rows, c.a[3], c.a[4]);
+}
 int h_cast_down(const Call& c) {
     const uint64_t n = u64(c.a, 1);
     RESOLVE(0, n * 4, src) RESOLVE(1, n * 2, dst)
@@ -388,6 +440,12 @@ const Entry kTable[] = {
     {"add_broadcast_backward", 3, 9, "g, dy, workspace | dtype, lead_lo, lead_hi, inner_lo, inner_hi, flags, ws_lo, ws_hi, present_mask", h_bcast_grad},
     {"fp32_to_bf16", 2, 3, "src, dst | accumulate, n_lo, n_hi", h_cast_down},
     {"bf16_to_fp32", 2, 2, "src, dst | n_lo, n_hi", h_cast_up},
+    {"unary_forward", 2, 4, "x, y | dtype, op, n_lo, n_hi", h_unary_fwd},
+    {"unary_backward", 3, 5, "dy, saved, dx | dtype, op, flags, n_lo, n_hi", h_unary_bwd},
+    {"mul_forward_kernel", 3, 6, "x, y, out | dtype, kind, lead_lo, lead_hi, inner_lo, inner_hi", h_mul_fwd},
+    {"mul_backward_kernel", 6, 10, "g, x, y, dx, dy, workspace | dtype, kind, lead_lo, lead_hi, inner_lo, inner_hi, flags, ws_lo, ws_hi, present_mask", h_mul_bwd},
+    {"softmax_forward", 2, 4, "x, y | dtype, rows_lo, rows_hi, V", h_softmax_fwd},
+    {"softmax_backward", 3, 5, "y, dy, dx | dtype, rows_lo, rows_hi, V, flags", h_softmax_bwd},
     {"contiguous_forward_kernel", 2, 27, "src, dst | dtype, flags, ndim, shape[8], stride_lo_hi[8]", h_strided_copy},
     {"strided_add_backward_kernel", 2, 27, "src, dst | dtype, flags, ndim, shape[8], stride_lo_hi[8]", h_strided_copy},
     {"layernorm_forward", 6, 5, "x, residual, gamma, beta, h, y | dtype, rows, C, eps_bits, present_mask", h_norm_fwd<AGRAD_NORM_LAYER>},
@@ -680,6 +738,38 @@ int agrad_grad_accumulate(agrad_ctx* ctx, int dtype, const void* src, void* dst,
 int agrad_cast_f32_to_bf16(agrad_ctx* ctx, const void* src, void* dst, uint64_t n, int accumulate) {
     CTX_OR_FAIL(ctx)
     return launch_cast_f32_bf16(ctx->stream, src, dst, n, accumulate);
+}
+int agrad_unary_forward(agrad_ctx* ctx, int op, int dtype, const void* x, void* y, uint64_t n) {
+    CTX_OR_FAIL(ctx)
+    return launch_unary_fwd(ctx->stream, op, dtype, x, y, n);
+}
+int agrad_unary_backward(agrad_ctx* ctx, int op, int dtype, const void* dy, const void* saved, void* dx, uint64_t n,
+                         uint32_t flags) {
+    CTX_OR_FAIL(ctx)
+    return launch_unary_bwd(ctx->stream, op, dtype, dy, saved, dx, n, flags);
+}
+int agrad_mul_forward(agrad_ctx* ctx, int dtype, int kind, const void* x, const void* y, void* out, uint64_t lead,
+                      uint64_t inner) {
+    CTX_OR_FAIL(ctx)
+    return launch_mul_fwd(ctx->stream, dtype, kind, x, y, out, lead, inner);
+}
+uint64_t agrad_mul_backward_workspace_bytes(int kind, uint64_t lead, uint64_t inner) {
+    return mul_bwd_workspace_bytes(kind, lead, inner);
+}
+int agrad_mul_backward(agrad_ctx* ctx, int dtype, int kind, const void* g, const void* x, const void* y, void* dx,
+                       void* dy, void* workspace, uint64_t workspace_bytes, uint64_t lead, uint64_t inner,
+                       uint32_t flags) {
+    CTX_OR_FAIL(ctx)
+    return launch_mul_bwd(ctx->stream, dtype, kind, g, x, y, dx, dy, workspace, workspace_bytes, lead, inner, flags);
+}
+int agrad_softmax_forward(agrad_ctx* ctx, int dtype, const void* x, void* y, uint64_t rows, uint32_t V) {
+    CTX_OR_FAIL(ctx)
+    return launch_softmax_fwd(ctx->stream, dtype, x, y, rows, V);
+}
+int agrad_softmax_backward(agrad_ctx* ctx, int dtype, const void* y, const void* dy, void* dx, uint64_t rows,
+                           uint32_t V, uint32_t flags) {
+    CTX_OR_FAIL(ctx)
+    return launch_softmax_bwd(ctx->stream, dtype, y, dy, dx, rows, V, flags);
 }
 int agrad_strided_copy(agrad_ctx* ctx, int dtype, const void* src, void* dst, int ndim, const uint32_t* shape,
                        const uint64_t* strides, uint32_t flags) {

@@ -51,6 +51,21 @@ uint64_t broadcast_grad_workspace_bytes(uint64_t lead, uint64_t inner);
 int launch_broadcast_grad(hipStream_t s, int dtype, const void* g, void* dy, void* workspace, uint64_t workspace_bytes,
                           uint64_t lead, uint64_t inner, uint32_t flags);
 
+// pointwise.hip
+int launch_unary_fwd(hipStream_t s, int op, int dtype, const void* x, void* y, uint64_t n);
+int launch_unary_bwd(hipStream_t s, int op, int dtype, const void* dy, const void* saved, void* dx, uint64_t n,
+                     uint32_t flags);
+int launch_mul_same(hipStream_t s, int dtype, const void* a, const void* b, void* out, uint64_t n, int accumulate);
+// reduce.hip: Mul with a broadcast operand and its gradients
+int launch_mul_fwd(hipStream_t s, int dtype, int kind, const void* x, const void* y, void* out, uint64_t lead, uint64_t inner);
+uint64_t mul_bwd_workspace_bytes(int kind, uint64_t lead, uint64_t inner);
+int launch_mul_bwd(hipStream_t s, int dtype, int kind, const void* g, const void* x, const void* y, void* dx, void* dy,
+                   void* workspace, uint64_t workspace_bytes, uint64_t lead, uint64_t inner, uint32_t flags);
+// loss.hip: softmax over the last axis
+int launch_softmax_fwd(hipStream_t s, int dtype, const void* x, void* y, uint64_t rows, uint32_t V);
+int launch_softmax_bwd(hipStream_t s, int dtype, const void* y, const void* dy, void* dx, uint64_t rows, uint32_t V,
+                       uint32_t flags);
+
 // strided.hip
 // elements spanned by the view: 1 + sum (shape[i] - 1) * strides[i]; 0 for an empty shape
 uint64_t strided_extent(int ndim, const uint32_t* shape, const uint64_t* strides);

@@ -94,8 +94,8 @@ struct RowSplit {
     }
 };
 
-// (max, sum) of one row, identical in every thread of the workgroup on return
-template <typename T, int VEC>
+// (max, sum) of one row, identical in every thread of the workgroup (BLOCK threads) on return
+template <typename T, int VEC, int BLOCK = kCeBlock>
 __device__ __forceinline__ MaxSum row_max_sum(const T* base, uint32_t V, MaxSum* lds) {
     const RowSplit<T, VEC> sp(base, V);
     MaxSum acc{-INFINITY, 0.0f};
@@ -110,16 +110,16 @@ __device__ __forceinline__ MaxSum row_max_sum(const T* base, uint32_t V, MaxSum*
         }
     }
     const T* body = base + sp.head;
-    for (uint32_t i0 = threadIdx.x; i0 < sp.nvec; i0 += kCeBlock * kCeUnroll) {
+    for (uint32_t i0 = threadIdx.x; i0 < sp.nvec; i0 += BLOCK * kCeUnroll) {
         float v[kCeUnroll][VEC];
 #pragma unroll
         for (int u = 0; u < kCeUnroll; ++u) {
-            const uint32_t i = i0 + u * kCeBlock;
+            const uint32_t i = i0 + u * BLOCK;
             if (i < sp.nvec) VecIO<T, VEC>::load(body + (uint64_t)i * VEC, v[u]);
         }
 #pragma unroll
         for (int u = 0; u < kCeUnroll; ++u) {
-            const uint32_t i = i0 + u * kCeBlock;
+            const uint32_t i = i0 + u * BLOCK;
             if (i < sp.nvec) absorb_vec<T, VEC>(acc, v[u]);
         }
     }
@@ -134,7 +134,7 @@ __device__ __forceinline__ MaxSum row_max_sum(const T* base, uint32_t V, MaxSum*
     __syncthreads();
     MaxSum total = lds[0];
 #pragma unroll
-    for (int w = 1; w < kCeBlock / kWave; ++w) total = merge<T>(total, lds[w]);
+    for (int w = 1; w < BLOCK / kWave; ++w) total = merge<T>(total, lds[w]);
     __syncthreads();
     return total;
 }
@@ -342,6 +342,281 @@ int ce_typed(hipStream_t s, bool backward, const T* x, const int32_t* labels, fl
     return check_hip(hipGetLastError(), "cross-entropy launch");
 }
 
+// ---------------------------------------------------------------------------
+// Softmax over the last axis (cpu_softmax_forward / backward, backend.py:354-374):
+//   forward   y = exp(x - max) / sum(exp(x - max))          (a division, as on the CPU)
+//   backward  dx (+)= y * (dy - sum(dy * y))
+// One workgroup per row, two passes over the row (the second one is served by the
+// caches): statistics first, then the element-wise pass.  Rows of up to 4 KB take
+// one-wave workgroups, longer rows 256 threads.
+// ---------------------------------------------------------------------------
+template <typename T, int VEC, int BLOCK>
+__global__ void __launch_bounds__(BLOCK)
+softmax_fwd_kernel(const T* __restrict__ x, T* __restrict__ y, uint32_t V) {
+    __shared__ MaxSum lds[BLOCK / kWave];
+    const uint64_t row = blockIdx.x;
+    const T* base = x + row * V;
+    T* out = y + row * V;
+    const MaxSum t = row_max_sum<T, VEC, BLOCK>(base, V, lds);
+    const RowSplit<T, VEC> sp(base, V);
+    if constexpr (VEC > 1) {
+        const uint32_t extra = sp.head + (V - sp.tail_start);
+        if (threadIdx.x < extra) {
+            const uint32_t e = threadIdx.x < sp.head ? threadIdx.x : sp.tail_start + (threadIdx.x - sp.head);
+            float v[1];
+            VecIO<T, 1>::load(base + e, v);
+            v[0] = exp_io<T>(v[0] - t.m) / t.s;
+            VecIO<T, 1>::store(out + e, v);
+        }
+    }
+    const T* body = base + sp.head;
+    T* obody = out + sp.head;
+    for (uint32_t i0 = threadIdx.x; i0 < sp.nvec; i0 += BLOCK * kCeBwdUnroll) {
+        float v[kCeBwdUnroll][VEC];
+#pragma unroll
+        for (int u = 0; u < kCeBwdUnroll; ++u) {
+            const uint32_t i = i0 + u * BLOCK;
+            if (i < sp.nvec) VecIO<T, VEC>::load(body + (uint64_t)i * VEC, v[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < kCeBwdUnroll; ++u) {
+            const uint32_t i = i0 + u * BLOCK;
+            if (i < sp.nvec) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) v[u][k] = exp_io<T>(v[u][k] - t.m) / t.s;
+                VecIO<T, VEC>::store(obody + (uint64_t)i * VEC, v[u]);
+            }
+        }
+    }
+}
+
+// sum over the workgroup, fixed order: lanes by xor butterflies, waves in index order
+template <int BLOCK>
+__device__ __forceinline__ float block_sum(float v, float* lds) {
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) v = v + __shfl_xor(v, off);
+    if constexpr (BLOCK > kWave) {
+        if (threadIdx.x % kWave == 0) lds[threadIdx.x / kWave] = v;
+        __syncthreads();
+        v = lds[0];
+#pragma unroll
+        for (int w = 1; w < BLOCK / kWave; ++w) v = v + lds[w];
+        __syncthreads();
+    }
+    return v;
+}
+
+template <typename T, int VEC, int BLOCK>
+__global__ void __launch_bounds__(BLOCK)
+softmax_bwd_kernel(const T* __restrict__ y, const T* __restrict__ dy, T* dx, uint32_t V, int accumulate) {
+    __shared__ float lds[BLOCK / kWave];
+    const uint64_t row = blockIdx.x;
+    const T* yb = y + row * V;
+    const T* gb = dy + row * V;
+    T* out = dx + row * V;
+    const RowSplit<T, VEC> sp(yb, V);      // the launcher checked that the three tensors share their alignment
+    const uint32_t extra = VEC > 1 ? sp.head + (V - sp.tail_start) : 0;
+    const uint32_t e = threadIdx.x < sp.head ? threadIdx.x : sp.tail_start + (threadIdx.x - sp.head);
+    float dot = 0.0f;
+    if (threadIdx.x < extra) {
+        float a[1], b[1];
+        VecIO<T, 1>::load(yb + e, a);
+        VecIO<T, 1>::load(gb + e, b);
+        dot = b[0] * a[0];
+    }
+    for (uint32_t i0 = threadIdx.x; i0 < sp.nvec; i0 += BLOCK * kCeBwdUnroll) {
+        float a[kCeBwdUnroll][VEC], b[kCeBwdUnroll][VEC];
+#pragma unroll
+        for (int u = 0; u < kCeBwdUnroll; ++u) {
+            const uint32_t i = i0 + u * BLOCK;
+            if (i < sp.nvec) {
+                VecIO<T, VEC>::load(yb + sp.head + (uint64_t)i * VEC, a[u]);
+                VecIO<T, VEC>::load(gb + sp.head + (uint64_t)i * VEC, b[u]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kCeBwdUnroll; ++u) {
+            const uint32_t i = i0 + u * BLOCK;
+            if (i < sp.nvec) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) dot = dot + b[u][k] * a[u][k];
+            }
+        }
+    }
+    dot = block_sum<BLOCK>(dot, lds);
+    if (threadIdx.x < extra) {
+        float a[1], b[1];
+        VecIO<T, 1>::load(yb + e, a);
+        VecIO<T, 1>::load(gb + e, b);
+        b[0] = a[0] * (b[0] - dot);
+        if (accumulate) {
+            float o[1];
+            VecIO<T, 1>::load(out + e, o);
+            b[0] = o[0] + b[0];
+        }
+        VecIO<T, 1>::store(out + e, b);
+    }
+    for (uint32_t i0 = threadIdx.x; i0 < sp.nvec; i0 += BLOCK * kCeBwdUnroll) {
+        float a[kCeBwdUnroll][VEC], b[kCeBwdUnroll][VEC], o[kCeBwdUnroll][VEC];
+#pragma unroll
+        for (int u = 0; u < kCeBwdUnroll; ++u) {
+            const uint32_t i = i0 + u * BLOCK;
+            if (i < sp.nvec) {
+                VecIO<T, VEC>::load(yb + sp.head + (uint64_t)i * VEC, a[u]);
+                VecIO<T, VEC>::load(gb + sp.head + (uint64_t)i * VEC, b[u]);
+                if (accumulate) VecIO<T, VEC>::load(out + sp.head + (uint64_t)i * VEC, o[u]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kCeBwdUnroll; ++u) {
+            const uint32_t i = i0 + u * BLOCK;
+            if (i < sp.nvec) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) {
+                    float t = a[u][k] * (b[u][k] - dot);
+                    if (accumulate) t = o[u][k] + t;
+                    b[u][k] = t;
+                }
+                VecIO<T, VEC>::store(out + sp.head + (uint64_t)i * VEC, b[u]);
+            }
+        }
+    }
+}
+
+// Rows of up to 64 * NV vectors whose length is a whole number of vectors: one wave
+// holds the row in registers, so it is read once (forward: 2 passes of traffic in
+// all, backward 3) and there is no barrier.  Same arithmetic as the two-pass kernels.
+template <typename T, int VEC, int NV>
+__global__ void __launch_bounds__(kWave)
+softmax_fwd_reg_kernel(const T* __restrict__ x, T* __restrict__ y, uint32_t V, uint32_t VV) {
+    const uint64_t row = blockIdx.x;
+    const T* base = x + row * V;
+    T* out = y + row * V;
+    float v[NV][VEC];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint32_t c = i * kWave + threadIdx.x;
+        if (c < VV) VecIO<T, VEC>::load(base + (uint64_t)c * VEC, v[i]);
+    }
+    // the CPU's order: row maximum, exp(x - max) once per element, their sum, a division
+    float m = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint32_t c = i * kWave + threadIdx.x;
+        if (c < VV) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) m = fmaxf(m, v[i][k]);
+        }
+    }
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) m = fmaxf(m, __shfl_xor(m, off));
+    float sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint32_t c = i * kWave + threadIdx.x;
+        if (c < VV) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                v[i][k] = exp_io<T>(v[i][k] - m);      // a row of -inf only: exp(nan) -> nan, as on the CPU
+                sum = sum + v[i][k];
+            }
+        }
+    }
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) sum = sum + __shfl_xor(sum, off);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint32_t c = i * kWave + threadIdx.x;
+        if (c < VV) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) v[i][k] = v[i][k] / sum;
+            VecIO<T, VEC>::store(out + (uint64_t)c * VEC, v[i]);
+        }
+    }
+}
+
+template <typename T, int VEC, int NV>
+__global__ void __launch_bounds__(kWave)
+softmax_bwd_reg_kernel(const T* __restrict__ y, const T* __restrict__ dy, T* dx, uint32_t V, uint32_t VV, int accumulate) {
+    const uint64_t row = blockIdx.x;
+    const T* yb = y + row * V;
+    const T* gb = dy + row * V;
+    T* out = dx + row * V;
+    float a[NV][VEC], b[NV][VEC];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint32_t c = i * kWave + threadIdx.x;
+        if (c < VV) {
+            VecIO<T, VEC>::load(yb + (uint64_t)c * VEC, a[i]);
+            VecIO<T, VEC>::load(gb + (uint64_t)c * VEC, b[i]);
+        }
+    }
+    float dot = 0.0f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint32_t c = i * kWave + threadIdx.x;
+        if (c < VV) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) dot = dot + b[i][k] * a[i][k];
+        }
+    }
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) dot = dot + __shfl_xor(dot, off);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint32_t c = i * kWave + threadIdx.x;
+        if (c < VV) {
+            float o[VEC];
+            if (accumulate) VecIO<T, VEC>::load(out + (uint64_t)c * VEC, o);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                const float t = a[i][k] * (b[i][k] - dot);
+                o[k] = accumulate ? (o[k] + t) : t;
+            }
+            VecIO<T, VEC>::store(out + (uint64_t)c * VEC, o);
+        }
+    }
+}
+
+template <typename T, int VEC, int NV>
+void softmax_reg_launch(hipStream_t s, bool backward, const T* a, const T* b, T* out, uint64_t rows, uint32_t V, int acc) {
+    const dim3 grid((uint32_t)rows);
+    if (!backward) hipLaunchKernelGGL((softmax_fwd_reg_kernel<T, VEC, NV>), grid, dim3(kWave), 0, s, a, out, V, V / VEC);
+    else hipLaunchKernelGGL((softmax_bwd_reg_kernel<T, VEC, NV>), grid, dim3(kWave), 0, s, a, b, out, V, V / VEC, acc);
+}
+
+template <typename T>
+int softmax_typed(hipStream_t s, bool backward, const T* a, const T* b, T* out, uint64_t rows, uint32_t V, int acc) {
+    constexpr int WIDE = WideVec<T>::value;
+    // rows of any length keep 16-byte accesses through the head / tail split, which
+    // needs every tensor to sit at the same offset within 16 bytes
+    const uintptr_t mis = reinterpret_cast<uintptr_t>(a) & 15u;
+    const bool same = (reinterpret_cast<uintptr_t>(out) & 15u) == mis && (!b || (reinterpret_cast<uintptr_t>(b) & 15u) == mis);
+    const bool wide = V >= 4 * WIDE && same && mis % sizeof(T) == 0;
+    const bool small = (uint64_t)V * sizeof(T) <= 4096;
+    const dim3 grid((uint32_t)rows);
+    if (mis == 0 && same && V % WIDE == 0 && V / WIDE <= 8 * kWave) {
+        // every row starts 16-byte aligned and fits a wave's registers
+        const uint32_t nv = (V / WIDE + kWave - 1) / kWave;
+        if (nv <= 1) softmax_reg_launch<T, WIDE, 1>(s, backward, a, b, out, rows, V, acc);
+        else if (nv <= 2) softmax_reg_launch<T, WIDE, 2>(s, backward, a, b, out, rows, V, acc);
+        else if (nv <= 4) softmax_reg_launch<T, WIDE, 4>(s, backward, a, b, out, rows, V, acc);
+        else softmax_reg_launch<T, WIDE, 8>(s, backward, a, b, out, rows, V, acc);
+        return check_hip(hipGetLastError(), "softmax launch");
+    }
+#define AGRAD_SM(VEC, BLOCK)                                                                                     \
+    do {                                                                                                         \
+        if (!backward) hipLaunchKernelGGL((softmax_fwd_kernel<T, VEC, BLOCK>), grid, dim3(BLOCK), 0, s, a, out, V); \
+        else hipLaunchKernelGGL((softmax_bwd_kernel<T, VEC, BLOCK>), grid, dim3(BLOCK), 0, s, a, b, out, V, acc);   \
+    } while (0)
+    if (wide && small) AGRAD_SM(WIDE, 64);
+    else if (wide) AGRAD_SM(WIDE, 256);
+    else if (small) AGRAD_SM(1, 64);
+    else AGRAD_SM(1, 256);
+#undef AGRAD_SM
+    return check_hip(hipGetLastError(), "softmax launch");
+}
+
 int ce_check(const char* what, int dtype, uint64_t rows, uint32_t V) {
     if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "%s: unknown dtype %d", what, dtype);
     if (rows > 0x7fffffffull) return set_error(AGRAD_EINVAL, "%s: too many rows", what);
@@ -373,6 +648,24 @@ int launch_ce_bwd(hipStream_t s, int dtype, const void* logits, const int32_t* l
     if (dtype == AGRAD_F32)
         return ce_typed<float>(s, true, (const float*)logits, labels, nullptr, nullptr, dloss, lse, (float*)dlogits, rows, V, acc, err_flag);
     return ce_typed<bf16_t>(s, true, (const bf16_t*)logits, labels, nullptr, nullptr, dloss, lse, (bf16_t*)dlogits, rows, V, acc, err_flag);
+}
+
+int launch_softmax_fwd(hipStream_t s, int dtype, const void* x, void* y, uint64_t rows, uint32_t V) {
+    if (int rc = ce_check("softmax forward", dtype, rows, V)) return rc;
+    if (rows == 0 || V == 0) return AGRAD_OK;
+    if (x == nullptr || y == nullptr) return set_error(AGRAD_EINVAL, "softmax forward: null operand");
+    if (dtype == AGRAD_F32) return softmax_typed<float>(s, false, (const float*)x, nullptr, (float*)y, rows, V, 0);
+    return softmax_typed<bf16_t>(s, false, (const bf16_t*)x, nullptr, (bf16_t*)y, rows, V, 0);
+}
+
+int launch_softmax_bwd(hipStream_t s, int dtype, const void* y, const void* dy, void* dx, uint64_t rows, uint32_t V,
+                       uint32_t flags) {
+    if (int rc = ce_check("softmax backward", dtype, rows, V)) return rc;
+    if (rows == 0 || V == 0) return AGRAD_OK;
+    if (y == nullptr || dy == nullptr || dx == nullptr) return set_error(AGRAD_EINVAL, "softmax backward: null operand");
+    const int acc = (flags & AGRAD_ACC_INPUT_GRAD) ? 1 : 0;
+    if (dtype == AGRAD_F32) return softmax_typed<float>(s, true, (const float*)y, (const float*)dy, (float*)dx, rows, V, acc);
+    return softmax_typed<bf16_t>(s, true, (const bf16_t*)y, (const bf16_t*)dy, (bf16_t*)dx, rows, V, acc);
 }
 
 }  // namespace agrad

@@ -13,6 +13,12 @@
 // partial row (read-only stream, several rows in flight per lane), and the
 // column-sum finalize kernel of the norm backward folds the partial rows.
 // Every sum has a fixed order.
+//
+// Broadcast Mul (cpu_mul_forward / cpu_mul_backward, backend.py:107-146) has the
+// same shapes plus two more: out[l, j] = x[l, j] * y[..] with y[j] ("row"), y[l]
+// ("col": one factor per row) or y[0] ("scalar").  dx (+)= g * y[..] is the forward
+// kernel again; dy is a column sum, a row sum or a full sum of the product g * x,
+// each in a fixed order.
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -57,31 +63,186 @@ bcast_add_kernel(const T* __restrict__ x, const T* __restrict__ y, T* __restrict
 // partial[blockIdx.x, :] = sum over rows blockIdx.x, blockIdx.x + gridDim.x, ... of g[row, :]
 template <typename T, int VEC>
 __global__ void __launch_bounds__(kColBlock)
-colsum_partial_kernel(const T* __restrict__ g, float* __restrict__ partial, uint64_t lead, uint32_t inner,
-                      uint32_t inner_vec) {
+colsum_partial_kernel(const T* __restrict__ g, const T* __restrict__ x2, float* __restrict__ partial, uint64_t lead,
+                      uint32_t inner, uint32_t inner_vec) {
     for (uint32_t cv = threadIdx.x; cv < inner_vec; cv += kColBlock) {
         const uint32_t col = cv * VEC;
         float acc[VEC];
 #pragma unroll
         for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
         for (uint64_t r0 = blockIdx.x; r0 < lead; r0 += (uint64_t)gridDim.x * kColRows) {
-            float v[kColRows][VEC];
+            float v[kColRows][VEC], w[kColRows][VEC];
 #pragma unroll
             for (int u = 0; u < kColRows; ++u) {
                 const uint64_t r = r0 + (uint64_t)u * gridDim.x;
-                if (r < lead) VecIO<T, VEC>::load(g + r * inner + col, v[u]);
+                if (r < lead) {
+                    VecIO<T, VEC>::load(g + r * inner + col, v[u]);
+                    if (x2 != nullptr) VecIO<T, VEC>::load(x2 + r * inner + col, w[u]);   // uniform branch
+                }
             }
 #pragma unroll
             for (int u = 0; u < kColRows; ++u) {
                 const uint64_t r = r0 + (uint64_t)u * gridDim.x;
                 if (r < lead) {
 #pragma unroll
-                    for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + v[u][k];
+                    for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + (x2 != nullptr ? v[u][k] * w[u][k] : v[u][k]);
                 }
             }
         }
 #pragma unroll
         for (int k = 0; k < VEC; ++k) partial[(uint64_t)blockIdx.x * inner + col + k] = acc[k];
+    }
+}
+
+// ---- broadcast Mul --------------------------------------------------------------
+// out (+)= a[l, j] * y[..]: KIND AGRAD_MUL_ROW y[j], AGRAD_MUL_COL y[l], AGRAD_MUL_SCALAR y[0]
+template <typename T> __device__ __forceinline__ float small_elem(const T* y, uint64_t i) {
+    if constexpr (sizeof(T) == 2) return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(y)[i]);
+    else return reinterpret_cast<const float*>(y)[i];
+}
+
+template <typename T, int VEC, int KIND>
+__global__ void __launch_bounds__(kBcastBlock)
+bcast_mul_kernel(const T* __restrict__ a, const T* __restrict__ y, T* out, uint64_t nvec, uint32_t inner_vec, int accumulate) {
+    const uint64_t idx = (uint64_t)blockIdx.x * kBcastBlock + threadIdx.x;
+    if (idx >= nvec) return;
+    float v[VEC], b[VEC];
+    VecIO<T, VEC>::load(a + idx * VEC, v);
+    if constexpr (KIND == AGRAD_MUL_ROW) {
+        // the small operand is re-read by every leading row: ordinary (cached) loads
+        const uint64_t j = (idx % inner_vec) * VEC;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) b[k] = small_elem<T>(y, j + k);
+    } else {
+        const float f = small_elem<T>(y, KIND == AGRAD_MUL_COL ? idx / inner_vec : 0);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) b[k] = f;
+    }
+    float o[VEC];
+    if (accumulate) VecIO<T, VEC>::load(out + idx * VEC, o);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+        const float t = v[k] * b[k];
+        o[k] = accumulate ? (o[k] + t) : t;
+    }
+    VecIO<T, VEC>::store(out + idx * VEC, o);
+}
+
+// dy[j] (+)= sum_l g[l, j] * x[l, j], l ascending: a thread owns a column vector (few
+// leading rows, or bf16 storage, where the result is rounded once at the end)
+template <typename T, int VEC>
+__global__ void __launch_bounds__(256)
+colprod_direct_kernel(const T* __restrict__ g, const T* __restrict__ x, T* dy, uint64_t lead, uint32_t inner,
+                      uint32_t inner_vec, int accumulate) {
+    const uint32_t cv = blockIdx.x * 256 + threadIdx.x;
+    if (cv >= inner_vec) return;
+    const uint32_t col = cv * VEC;
+    float acc[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
+    for (uint64_t l0 = 0; l0 < lead; l0 += kColRows) {
+        float v[kColRows][VEC], w[kColRows][VEC];
+#pragma unroll
+        for (int u = 0; u < kColRows; ++u)
+            if (l0 + u < lead) {
+                VecIO<T, VEC>::load(g + (l0 + u) * inner + col, v[u]);
+                VecIO<T, VEC>::load(x + (l0 + u) * inner + col, w[u]);
+            }
+#pragma unroll
+        for (int u = 0; u < kColRows; ++u)
+            if (l0 + u < lead) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + v[u][k] * w[u][k];
+            }
+    }
+    if (accumulate) {
+        float o[VEC];
+        VecIO<T, VEC>::load(dy + col, o);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc[k] = o[k] + acc[k];
+    }
+    VecIO<T, VEC>::store(dy + col, acc);
+}
+
+// One workgroup per row: dot[l] = sum_j g[l, j] * x[l, j].  Lanes add their strided
+// share in order, the wave folds by xor butterflies, waves are added in index order.
+// TO_F32: the dots go to an fp32 array (first stage of the full sum); otherwise they
+// are the gradient of the per-row factor, dy[l] (+)= dot[l].
+template <typename T, int VEC, int BLOCK, bool TO_F32>
+__global__ void __launch_bounds__(BLOCK)
+rowdot_kernel(const T* __restrict__ g, const T* __restrict__ x, void* dst, uint32_t inner, uint32_t inner_vec,
+              int accumulate) {
+    __shared__ float lds[BLOCK / kWave];
+    const uint64_t row = blockIdx.x;
+    const T* gr = g + row * inner;
+    const T* xr = x + row * inner;
+    float dot = 0.0f;
+    for (uint32_t i0 = threadIdx.x; i0 < inner_vec; i0 += BLOCK * kColRows) {
+        float v[kColRows][VEC], w[kColRows][VEC];
+#pragma unroll
+        for (int u = 0; u < kColRows; ++u) {
+            const uint32_t i = i0 + u * BLOCK;
+            if (i < inner_vec) {
+                VecIO<T, VEC>::load(gr + (uint64_t)i * VEC, v[u]);
+                VecIO<T, VEC>::load(xr + (uint64_t)i * VEC, w[u]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kColRows; ++u) {
+            const uint32_t i = i0 + u * BLOCK;
+            if (i < inner_vec) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) dot = dot + v[u][k] * w[u][k];
+            }
+        }
+    }
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) dot = dot + __shfl_xor(dot, off);
+    if constexpr (BLOCK > kWave) {
+        if (threadIdx.x % kWave == 0) lds[threadIdx.x / kWave] = dot;
+        __syncthreads();
+        dot = lds[0];
+#pragma unroll
+        for (int w = 1; w < BLOCK / kWave; ++w) dot = dot + lds[w];
+    }
+    if (threadIdx.x == 0) {
+        if constexpr (TO_F32) {
+            static_cast<float*>(dst)[row] = dot;
+        } else {
+            T* dy = static_cast<T*>(dst);
+            float o[1] = {dot};
+            if (accumulate) {
+                float old[1];
+                VecIO<T, 1>::load(dy + row, old);
+                o[0] = old[0] + dot;
+            }
+            VecIO<T, 1>::store(dy + row, o);
+        }
+    }
+}
+
+// dy[0] (+)= sum of n fp32 values: one workgroup, thread t adds t, t + 1024, ... in
+// order, then the 1024 sums fold as in rowdot_kernel
+template <typename T>
+__global__ void __launch_bounds__(1024)
+sum_finalize_kernel(const float* __restrict__ part, T* dy, uint64_t n, int accumulate) {
+    __shared__ float lds[1024 / kWave];
+    float acc = 0.0f;
+    for (uint64_t i = threadIdx.x; i < n; i += 1024) acc = acc + part[i];
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) acc = acc + __shfl_xor(acc, off);
+    if (threadIdx.x % kWave == 0) lds[threadIdx.x / kWave] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float t = lds[0];
+        for (int w = 1; w < 1024 / kWave; ++w) t = t + lds[w];
+        float o[1] = {t};
+        if (accumulate) {
+            float old[1];
+            VecIO<T, 1>::load(dy, old);
+            o[0] = old[0] + t;
+        }
+        VecIO<T, 1>::store(dy, o);
     }
 }
 
@@ -110,10 +271,36 @@ int launch_broadcast_add(hipStream_t s, int dtype, const void* x, const void* y,
     return bcast_add_typed<bf16_t>(s, (const bf16_t*)x, (const bf16_t*)y, (bf16_t*)out, lead, inner);
 }
 
+// partial rows, plus one fp32 row in which a bf16 destination's sum is finished before it is rounded
 uint64_t broadcast_grad_workspace_bytes(uint64_t lead, uint64_t inner) {
     if (lead <= kColDirectLead || inner == 0) return 0;
-    return (uint64_t)colsum_blocks(lead) * inner * sizeof(float);
+    return ((uint64_t)colsum_blocks(lead) + 1) * inner * sizeof(float);
 }
+
+namespace {
+
+// dy[j] (+)= sum_l g[l, j] (* x2[l, j]) in two stages through `workspace`; bf16 sums are
+// finished in fp32 and rounded once
+template <typename T>
+int colsum_two_stage(hipStream_t s, const T* g, const T* x2, T* dy, void* workspace, uint64_t lead, uint64_t inner,
+                     int accumulate) {
+    constexpr int WIDE = WideVec<T>::value;
+    const uint32_t blocks = colsum_blocks(lead);
+    float* partial = (float*)workspace;
+    const bool wide = inner % WIDE == 0 && aligned16(g) && (!x2 || aligned16(x2));
+    if (wide) hipLaunchKernelGGL((colsum_partial_kernel<T, WIDE>), dim3(blocks), dim3(kColBlock), 0, s, g, x2, partial, lead, (uint32_t)inner, (uint32_t)(inner / WIDE));
+    else hipLaunchKernelGGL((colsum_partial_kernel<T, 1>), dim3(blocks), dim3(kColBlock), 0, s, g, x2, partial, lead, (uint32_t)inner, (uint32_t)inner);
+    if (int rc = check_hip(hipGetLastError(), "column sum launch")) return rc;
+    if constexpr (sizeof(T) == 4) {
+        return launch_colsum_finalize(s, partial, nullptr, blocks, (uint32_t)inner, (float*)dy, nullptr, accumulate);
+    } else {
+        float* row = partial + (uint64_t)blocks * inner;
+        if (int rc = launch_colsum_finalize(s, partial, nullptr, blocks, (uint32_t)inner, row, nullptr, 0)) return rc;
+        return launch_cast_f32_bf16(s, row, dy, inner, accumulate);
+    }
+}
+
+}  // namespace
 
 int launch_broadcast_grad(hipStream_t s, int dtype, const void* g, void* dy, void* workspace, uint64_t workspace_bytes,
                           uint64_t lead, uint64_t inner, uint32_t flags) {
@@ -128,21 +315,149 @@ int launch_broadcast_grad(hipStream_t s, int dtype, const void* g, void* dy, voi
     }
     if (g == nullptr) return set_error(AGRAD_EINVAL, "broadcast gradient: null operand");
     const uint64_t need = broadcast_grad_workspace_bytes(lead, inner);
-    // the two-stage path produces fp32; a bf16 destination keeps the direct path
-    if (need == 0 || dtype == AGRAD_BF16)
+    // few rows: a thread per column adds them itself.  (A bf16 caller without a workspace
+    // gets the same kernel whatever the row count: correct, but one thread walks the column.)
+    if (need == 0 || (dtype == AGRAD_BF16 && workspace == nullptr))
         return launch_pos_embedding_bwd(s, dtype, g, dy, (uint32_t)lead, 1, (uint32_t)inner, flags);
     if (workspace == nullptr || workspace_bytes < need)
         return set_error(AGRAD_EWORKSPACE, "broadcast gradient: workspace %llu < %llu bytes",
                          (unsigned long long)workspace_bytes, (unsigned long long)need);
     if (!aligned16(workspace)) return set_error(AGRAD_EINVAL, "broadcast gradient: workspace must be 16-byte aligned");
-    const uint32_t blocks = colsum_blocks(lead);
-    float* partial = (float*)workspace;
-    const bool wide = inner % 4 == 0 && aligned16(g);
-    if (wide) hipLaunchKernelGGL((colsum_partial_kernel<float, 4>), dim3(blocks), dim3(kColBlock), 0, s, (const float*)g, partial, lead, (uint32_t)inner, (uint32_t)(inner / 4));
-    else hipLaunchKernelGGL((colsum_partial_kernel<float, 1>), dim3(blocks), dim3(kColBlock), 0, s, (const float*)g, partial, lead, (uint32_t)inner, (uint32_t)inner);
-    if (int rc = check_hip(hipGetLastError(), "broadcast gradient launch")) return rc;
-    return launch_colsum_finalize(s, partial, nullptr, blocks, (uint32_t)inner, (float*)dy, nullptr,
-                                  (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0);
+    const int acc = (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0;
+    if (dtype == AGRAD_F32) return colsum_two_stage<float>(s, (const float*)g, nullptr, (float*)dy, workspace, lead, inner, acc);
+    return colsum_two_stage<bf16_t>(s, (const bf16_t*)g, nullptr, (bf16_t*)dy, workspace, lead, inner, acc);
+}
+
+namespace {
+
+template <typename T, int KIND>
+int bcast_mul_typed(hipStream_t s, const T* a, const T* y, T* out, uint64_t lead, uint64_t inner, int acc) {
+    constexpr int WIDE = WideVec<T>::value;
+    const uint64_t n = lead * inner;
+    // a vector never straddles two rows, and the row operand is read at vector offsets
+    const bool wide = inner % WIDE == 0 && aligned16(a) && aligned16(out);
+    const uint64_t nvec = wide ? n / WIDE : n;
+    const uint64_t inner_vec = wide ? inner / WIDE : inner;
+    const uint64_t grid = (nvec + kBcastBlock - 1) / kBcastBlock;
+    if (grid > 0x7fffffffull || inner_vec >= 0xffffffffull) return set_error(AGRAD_EINVAL, "broadcast mul: tensor too large");
+    if (wide) hipLaunchKernelGGL((bcast_mul_kernel<T, WIDE, KIND>), dim3((uint32_t)grid), dim3(kBcastBlock), 0, s, a, y, out, nvec, (uint32_t)inner_vec, acc);
+    else hipLaunchKernelGGL((bcast_mul_kernel<T, 1, KIND>), dim3((uint32_t)grid), dim3(kBcastBlock), 0, s, a, y, out, nvec, (uint32_t)inner_vec, acc);
+    return check_hip(hipGetLastError(), "broadcast mul launch");
+}
+
+template <typename T>
+int bcast_mul_kind(hipStream_t s, int kind, const void* a, const void* y, void* out, uint64_t lead, uint64_t inner, int acc) {
+    switch (kind) {
+        case AGRAD_MUL_ROW: return bcast_mul_typed<T, AGRAD_MUL_ROW>(s, (const T*)a, (const T*)y, (T*)out, lead, inner, acc);
+        case AGRAD_MUL_COL: return bcast_mul_typed<T, AGRAD_MUL_COL>(s, (const T*)a, (const T*)y, (T*)out, lead, inner, acc);
+        default: return bcast_mul_typed<T, AGRAD_MUL_SCALAR>(s, (const T*)a, (const T*)y, (T*)out, lead, inner, acc);
+    }
+}
+
+template <typename T, bool TO_F32>
+int rowdot_typed(hipStream_t s, const T* g, const T* x, void* dst, uint64_t lead, uint64_t inner, int acc) {
+    constexpr int WIDE = WideVec<T>::value;
+    if (lead > 0x7fffffffull || inner >= 0xffffffffull) return set_error(AGRAD_EINVAL, "mul backward: tensor too large");
+    const bool wide = inner % WIDE == 0 && aligned16(g) && aligned16(x);
+    const uint32_t iv = (uint32_t)(wide ? inner / WIDE : inner);
+    const bool small = inner * sizeof(T) <= 4096;
+    const dim3 grid((uint32_t)lead);
+#define AGRAD_RD(VEC, BLOCK) hipLaunchKernelGGL((rowdot_kernel<T, VEC, BLOCK, TO_F32>), grid, dim3(BLOCK), 0, s, g, x, dst, (uint32_t)inner, iv, acc)
+    if (wide && small) AGRAD_RD(WIDE, 64);
+    else if (wide) AGRAD_RD(WIDE, 256);
+    else if (small) AGRAD_RD(1, 64);
+    else AGRAD_RD(1, 256);
+#undef AGRAD_RD
+    return check_hip(hipGetLastError(), "mul backward launch");
+}
+
+bool mul_kind_ok(int kind) { return kind >= AGRAD_MUL_SAME && kind <= AGRAD_MUL_SCALAR; }
+
+}  // namespace
+
+int launch_mul_fwd(hipStream_t s, int dtype, int kind, const void* x, const void* y, void* out, uint64_t lead, uint64_t inner) {
+    if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "mul: unknown dtype %d", dtype);
+    if (!mul_kind_ok(kind)) return set_error(AGRAD_EINVAL, "mul: unknown broadcast kind %d", kind);
+    if (lead == 0 || inner == 0) return AGRAD_OK;
+    if (x == nullptr || y == nullptr || out == nullptr) return set_error(AGRAD_EINVAL, "mul: null operand");
+    if (kind == AGRAD_MUL_SAME) return launch_mul_same(s, dtype, x, y, out, lead * inner, 0);
+    if (dtype == AGRAD_F32) return bcast_mul_kind<float>(s, kind, x, y, out, lead, inner, 0);
+    return bcast_mul_kind<bf16_t>(s, kind, x, y, out, lead, inner, 0);
+}
+
+uint64_t mul_bwd_workspace_bytes(int kind, uint64_t lead, uint64_t inner) {
+    if (kind == AGRAD_MUL_ROW) return broadcast_grad_workspace_bytes(lead, inner);
+    if (kind == AGRAD_MUL_SCALAR) return (lead * sizeof(float) + 255) & ~255ull;
+    return 0;
+}
+
+int launch_mul_bwd(hipStream_t s, int dtype, int kind, const void* g, const void* x, const void* y, void* dx, void* dy,
+                   void* workspace, uint64_t workspace_bytes, uint64_t lead, uint64_t inner, uint32_t flags) {
+    if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "mul backward: unknown dtype %d", dtype);
+    if (!mul_kind_ok(kind)) return set_error(AGRAD_EINVAL, "mul backward: unknown broadcast kind %d", kind);
+    const int acc_x = (flags & AGRAD_ACC_INPUT_GRAD) ? 1 : 0;
+    const int acc_y = (flags & AGRAD_ACC_INPUT_GRAD2) ? 1 : 0;
+    const uint32_t es = dtype_size(dtype);
+    if (lead == 0 || inner == 0) {
+        // an empty product: stored gradients of the small operand become zero
+        if (dy != nullptr && !acc_y && kind != AGRAD_MUL_SAME) {
+            const uint64_t ny = kind == AGRAD_MUL_ROW ? inner : (kind == AGRAD_MUL_COL ? lead : 1);
+            if (ny) return launch_fill(s, dy, 0, (int)es, ny);
+        }
+        return AGRAD_OK;
+    }
+    if (g == nullptr) return set_error(AGRAD_EINVAL, "mul backward: null upstream gradient");
+    if (dx != nullptr) {
+        if (y == nullptr) return set_error(AGRAD_EINVAL, "mul backward: dx needs y");
+        int rc;
+        if (kind == AGRAD_MUL_SAME) rc = launch_mul_same(s, dtype, g, y, dx, lead * inner, acc_x);
+        else if (dtype == AGRAD_F32) rc = bcast_mul_kind<float>(s, kind, g, y, dx, lead, inner, acc_x);
+        else rc = bcast_mul_kind<bf16_t>(s, kind, g, y, dx, lead, inner, acc_x);
+        if (rc) return rc;
+    }
+    if (dy == nullptr) return AGRAD_OK;
+    if (x == nullptr) return set_error(AGRAD_EINVAL, "mul backward: dy needs x");
+    if (kind == AGRAD_MUL_SAME) return launch_mul_same(s, dtype, g, x, dy, lead * inner, acc_y);
+    if (kind == AGRAD_MUL_COL) {
+        if (dtype == AGRAD_F32) return rowdot_typed<float, false>(s, (const float*)g, (const float*)x, dy, lead, inner, acc_y);
+        return rowdot_typed<bf16_t, false>(s, (const bf16_t*)g, (const bf16_t*)x, dy, lead, inner, acc_y);
+    }
+    const uint64_t need = mul_bwd_workspace_bytes(kind, lead, inner);
+    if (kind == AGRAD_MUL_SCALAR) {
+        if (workspace == nullptr || workspace_bytes < need)
+            return set_error(AGRAD_EWORKSPACE, "mul backward: workspace %llu < %llu bytes",
+                             (unsigned long long)workspace_bytes, (unsigned long long)need);
+        if (!aligned16(workspace)) return set_error(AGRAD_EINVAL, "mul backward: workspace must be 16-byte aligned");
+        int rc = dtype == AGRAD_F32
+                     ? rowdot_typed<float, true>(s, (const float*)g, (const float*)x, workspace, lead, inner, 0)
+                     : rowdot_typed<bf16_t, true>(s, (const bf16_t*)g, (const bf16_t*)x, workspace, lead, inner, 0);
+        if (rc) return rc;
+        if (dtype == AGRAD_F32) hipLaunchKernelGGL((sum_finalize_kernel<float>), dim3(1), dim3(1024), 0, s, (const float*)workspace, (float*)dy, lead, acc_y);
+        else hipLaunchKernelGGL((sum_finalize_kernel<bf16_t>), dim3(1), dim3(1024), 0, s, (const float*)workspace, (bf16_t*)dy, lead, acc_y);
+        return check_hip(hipGetLastError(), "mul backward launch");
+    }
+    // AGRAD_MUL_ROW: a column sum of the product
+    if (inner >= 0x7fffffffull || lead >= 0x7fffffffull) return set_error(AGRAD_EINVAL, "mul backward: tensor too large");
+    if (need == 0) {
+        if (dtype == AGRAD_F32) {
+            const bool wide = inner % 4 == 0 && aligned16(g) && aligned16(x) && aligned16(dy);
+            const uint32_t iv = (uint32_t)(wide ? inner / 4 : inner);
+            if (wide) hipLaunchKernelGGL((colprod_direct_kernel<float, 4>), dim3((iv + 255) / 256), dim3(256), 0, s, (const float*)g, (const float*)x, (float*)dy, lead, (uint32_t)inner, iv, acc_y);
+            else hipLaunchKernelGGL((colprod_direct_kernel<float, 1>), dim3((iv + 255) / 256), dim3(256), 0, s, (const float*)g, (const float*)x, (float*)dy, lead, (uint32_t)inner, iv, acc_y);
+        } else {
+            const bool wide = inner % 8 == 0 && aligned16(g) && aligned16(x) && aligned16(dy);
+            const uint32_t iv = (uint32_t)(wide ? inner / 8 : inner);
+            if (wide) hipLaunchKernelGGL((colprod_direct_kernel<bf16_t, 8>), dim3((iv + 255) / 256), dim3(256), 0, s, (const bf16_t*)g, (const bf16_t*)x, (bf16_t*)dy, lead, (uint32_t)inner, iv, acc_y);
+            else hipLaunchKernelGGL((colprod_direct_kernel<bf16_t, 1>), dim3((iv + 255) / 256), dim3(256), 0, s, (const bf16_t*)g, (const bf16_t*)x, (bf16_t*)dy, lead, (uint32_t)inner, iv, acc_y);
+        }
+        return check_hip(hipGetLastError(), "mul backward launch");
+    }
+    if (workspace == nullptr || workspace_bytes < need)
+        return set_error(AGRAD_EWORKSPACE, "mul backward: workspace %llu < %llu bytes",
+                         (unsigned long long)workspace_bytes, (unsigned long long)need);
+    if (!aligned16(workspace)) return set_error(AGRAD_EINVAL, "mul backward: workspace must be 16-byte aligned");
+    if (dtype == AGRAD_F32) return colsum_two_stage<float>(s, (const float*)g, (const float*)x, (float*)dy, workspace, lead, inner, acc_y);
+    return colsum_two_stage<bf16_t>(s, (const bf16_t*)g, (const bf16_t*)x, (bf16_t*)dy, workspace, lead, inner, acc_y);
 }
 
 }  // namespace agrad

@@ -18,7 +18,7 @@ from abc import ABC, abstractmethod
 import numpy as np
 
 from .tensor import Tensor
-from .utils import broadcast_shape
+from .utils import broadcast_shape, mul_bcast_kind
 
 
 class OpNode:
@@ -100,6 +100,64 @@ class AddOp(Op):
 
     def fully_written_inputs(self, inputs, outputs):
         return [0, 1]
+
+
+class MulOp(Op):
+    """out = x * y; y has x's shape, its trailing [C], one factor per row ([..., 1]) or
+    one element (op.py:61-69; the broadcast kinds of utils.py:134-143)"""
+    op_name = "Mul"
+
+    def infer_shape(self, x, y):
+        shape = broadcast_shape(x.shape, y.shape)
+        if tuple(shape) != tuple(x.shape):
+            raise RuntimeError(f"Mul: the second operand is the broadcast one, got x={x.shape} y={y.shape}")
+        mul_bcast_kind(x.shape, y.shape)      # raises on a kind the kernels do not have
+        return shape
+
+    def save_for_backward(self, inputs, outputs):
+        return list(inputs)
+
+    def fully_written_inputs(self, inputs, outputs):
+        return [0, 1]
+
+
+class _UnaryOp(Op):
+    saves_output = True      # backward reads y (exp, rsqrt) rather than x (log)
+
+    def infer_shape(self, x):
+        return x.shape
+
+    def save_for_backward(self, inputs, outputs):
+        return list(outputs) if self.saves_output else list(inputs)
+
+    def fully_written_inputs(self, inputs, outputs):
+        return [0]
+
+
+class ExpOp(_UnaryOp):
+    op_name = "Exp"
+
+
+class LogOp(_UnaryOp):
+    op_name = "Log"
+    saves_output = False
+
+
+class RsqrtOp(_UnaryOp):
+    op_name = "Rsqrt"
+
+
+class SoftmaxOp(_UnaryOp):
+    """softmax over `dim`; the kernels take the last axis (op.py:205-218)"""
+    op_name = "Softmax"
+
+    def __init__(self, dim=-1):
+        self.dim = dim
+
+    def infer_shape(self, x):
+        if self.dim % max(x.ndim, 1) != x.ndim - 1:
+            raise ValueError(f"Softmax: only the last axis is supported, got dim={self.dim} for {x.ndim} axes")
+        return x.shape
 
 
 # -- views and layout changes (op.py:89-185) --------------------------------------

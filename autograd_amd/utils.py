@@ -50,6 +50,21 @@ def broadcast_shape(a, b):
     return tuple(reversed(out))
 
 
+def mul_bcast_kind(x_shape, y_shape) -> str:
+    """how y is broadcast against x in x * y: 'scalar', 'row' ([C] against [..., C]),
+    'col' ([..., 1] against [..., C]) or 'same' (utils.py:134-143)"""
+    x_shape, y_shape = tuple(x_shape), tuple(y_shape)
+    if len(y_shape) == 0 or prod(y_shape) == 1:
+        return "scalar"
+    if len(y_shape) == 1 and x_shape[-1] == y_shape[0]:
+        return "row"
+    if len(y_shape) == len(x_shape) and y_shape[:-1] == x_shape[:-1] and y_shape[-1] == 1:
+        return "col"
+    if y_shape == x_shape:
+        return "same"
+    raise RuntimeError(f"Mul backward: unsupported broadcast x={x_shape} y={y_shape}")
+
+
 def f32_bits(x) -> int:
     return struct.unpack("<I", struct.pack("<f", float(x)))[0]
 

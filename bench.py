@@ -137,7 +137,8 @@ def build_cases(ctx, cfg, pool):
     nbytes = op_bytes(cfg, distinct)
     cases = []
     # one builder per op family: each keeps its buffers in its own scope
-    for builder in (_embed_cases, _norm_cases, _act_cases, _rope_cases, _layout_cases, _loss_cases, _opt_cases):
+    for builder in (_embed_cases, _norm_cases, _act_cases, _rope_cases, _layout_cases, _primitive_cases, _loss_cases,
+                    _opt_cases):
         cases += builder(ctx, cfg, pool, rng, nbytes, ids0)
     return cases
 
@@ -291,6 +292,61 @@ def _layout_cases(ctx, cfg, pool, rng, nbytes, ids0):
         add("permute_bthd_bhtd", (cfg.B, cfg.T, Hq, D), (0, 2, 1, 3))
     if cfg.norm:
         add("transpose_nc_cn", (cfg.N, cfg.C), (1, 0))
+    return cases
+
+
+def _primitive_cases(ctx, cfg, pool, rng, nbytes, ids0):
+    """the primitive ops beside the hot path: softmax over attention-shaped rows
+    [B*H*T, T] (2 / 3 passes of n*e bytes) and x[N, C] * gamma[C] with both gradients
+    (2*n*e forward; backward reads g and x and writes dx: 3*n*e)"""
+    dt = capi.BF16 if cfg.dtype == "bf16" else capi.F32
+    e = cfg.esize
+    cases = []
+    if cfg.rope:
+        Hq = cfg.rope[0]
+        rows = cfg.B * Hq * cfg.T
+        V = cfg.T
+        while rows * V * e > (1 << 30):       # keep the score matrix at a size one layer of one micro-batch has
+            rows //= 2
+        n = rows * V
+        k = n_sets(2 * n * e)
+        x = [pool.normal(n, cfg.dtype) for _ in range(k)]
+        y = [pool.empty(n, cfg.dtype) for _ in range(k)]
+        g = [pool.normal(n, cfg.dtype) for _ in range(k)]
+        dx = [pool.empty(n, cfg.dtype) for _ in range(k)]
+
+        def sm_fwd(i):
+            ctx.call("agrad_softmax_forward", dt, vp(x[i]), vp(y[i]), rows, V)
+
+        def sm_bwd(i):
+            ctx.call("agrad_softmax_backward", dt, vp(y[i]), vp(g[i]), vp(dx[i]), rows, V, 0)
+
+        for i in range(k):
+            sm_fwd(i)
+        cases.append(Case(f"softmax[{rows}x{V}]", "prim-fwd", 2 * n * e, k, sm_fwd, "softmax_fwd_kernel"))
+        cases.append(Case(f"softmax[{rows}x{V}]", "prim-bwd", 3 * n * e, k, sm_bwd, "softmax_bwd_kernel"))
+    if cfg.norm:
+        # (own names throughout: the softmax closures above still read theirs)
+        N, Cw = cfg.N, cfg.C
+        m_n = N * Cw
+        m_k = n_sets(2 * m_n * e)
+        m_x = [pool.normal(m_n, cfg.dtype) for _ in range(m_k)]
+        m_out = [pool.empty(m_n, cfg.dtype) for _ in range(m_k)]
+        gam = pool.normal(Cw, cfg.dtype)
+        dgam = pool.empty(Cw, cfg.dtype)
+        ws_bytes = ctx.lib.agrad_mul_backward_workspace_bytes(capi.MUL_ROW, N, Cw)
+        ws = pool.raw(max(ws_bytes, 256))
+
+        def mul_fwd(i):
+            ctx.call("agrad_mul_forward", dt, capi.MUL_ROW, vp(m_x[i]), vp(gam), vp(m_out[i]), N, Cw)
+
+        def mul_bwd(i):        # m_out[i] plays the upstream gradient, the next set's m_out receives dx
+            ctx.call("agrad_mul_backward", dt, capi.MUL_ROW, vp(m_out[i]), vp(m_x[i]), vp(gam), vp(m_out[(i + 1) % m_k]),
+                     vp(dgam), vp(ws), ws_bytes, N, Cw, 0)
+
+        cases.append(Case("mul_row", "prim-fwd", 2 * m_n * e, m_k, mul_fwd, "bcast_mul_kernel"))
+        if m_k > 1:
+            cases.append(Case("mul_row", "prim-bwd", 3 * m_n * e, m_k, mul_bwd, "bcast_mul_kernel"))
     return cases
 
 

@@ -128,9 +128,10 @@ int agrad_broadcast_add_forward(agrad_ctx* ctx, int dtype, const void* x, const 
 /* dy[j] (+)= sum_l g[l, j], l ascending within a fixed two-level order (the
  * broadcasting branch of cpu_add_backward, backend.py:78-105; pos_emb_grad and
  * the bias-gradient column reductions, metal_ops.metal:220-234, 1002-1193).
- * AGRAD_ACC_PARAM_GRAD accumulates into dy.  fp32 tensors with more than 64
- * leading rows need a workspace of agrad_broadcast_grad_workspace_bytes(lead, inner)
- * bytes (16-byte aligned); otherwise workspace may be NULL. */
+ * AGRAD_ACC_PARAM_GRAD accumulates into dy.  With more than 64 leading rows the sum
+ * runs in two stages through a workspace of agrad_broadcast_grad_workspace_bytes(lead,
+ * inner) bytes (16-byte aligned; bf16 sums are finished in fp32 and rounded once).
+ * fp32 needs it then; a bf16 call may pass NULL and gets a one-thread-per-column sum. */
 uint64_t agrad_broadcast_grad_workspace_bytes(uint64_t lead, uint64_t inner);
 int agrad_broadcast_add_backward(agrad_ctx* ctx, int dtype, const void* g, void* dy,
                                  void* workspace, uint64_t workspace_bytes,
@@ -140,6 +141,41 @@ int agrad_grad_accumulate(agrad_ctx* ctx, int dtype, const void* src, void* dst,
 /* dst_bf16[i] = rne(src_f32[i]) (+ dst if accumulate) (fp32_to_bf16, metal_ops.metal:12010-12041). */
 int agrad_cast_f32_to_bf16(agrad_ctx* ctx, const void* src, void* dst, uint64_t n, int accumulate);
 int agrad_cast_bf16_to_f32(agrad_ctx* ctx, const void* src, void* dst, uint64_t n);
+/* The element-wise primitives Exp, Log and Rsqrt (op.py:187-204).
+ *   forward   y = exp(x) | log(x) | 1 / sqrt(x)                  (cpu_exp_forward, cpu_log_forward,
+ *                                                                  cpu_rsqrt_forward, backend.py:320-345)
+ *   backward  dx (+)= dy * y | dy / x | (((dy * -0.5) * y) * y) * y;  `saved` is y for exp
+ *             and rsqrt and x for log (cpu_*_backward, backend.py:324-352).
+ * AGRAD_ACC_INPUT_GRAD accumulates into dx. */
+enum { AGRAD_UNARY_EXP = 0, AGRAD_UNARY_LOG = 1, AGRAD_UNARY_RSQRT = 2 };
+int agrad_unary_forward(agrad_ctx* ctx, int op, int dtype, const void* x, void* y, uint64_t n);
+int agrad_unary_backward(agrad_ctx* ctx, int op, int dtype, const void* dy, const void* saved, void* dx,
+                         uint64_t n, uint32_t flags);
+
+/* Mul with the reference's broadcast kinds (mul_bcast_kind, utils.py:134-143): x is
+ * [lead, inner]; y is the same shape (SAME), [inner] (ROW), [lead] -- one factor per
+ * row (COL) -- or one element (SCALAR).  out = x * y (cpu_mul_forward, backend.py:107-111).
+ * Backward (cpu_mul_backward, backend.py:113-146): dx (+)= g * y and dy (+)= the
+ * product g * x summed over what y was broadcast along, in a fixed order; either may
+ * be NULL.  AGRAD_ACC_INPUT_GRAD accumulates into dx, AGRAD_ACC_INPUT_GRAD2 into dy.
+ * ROW (fp32, more than 64 rows) and SCALAR need agrad_mul_backward_workspace_bytes
+ * bytes of 16-byte aligned workspace. */
+enum { AGRAD_MUL_SAME = 0, AGRAD_MUL_ROW = 1, AGRAD_MUL_COL = 2, AGRAD_MUL_SCALAR = 3 };
+int agrad_mul_forward(agrad_ctx* ctx, int dtype, int kind, const void* x, const void* y, void* out,
+                      uint64_t lead, uint64_t inner);
+uint64_t agrad_mul_backward_workspace_bytes(int kind, uint64_t lead, uint64_t inner);
+int agrad_mul_backward(agrad_ctx* ctx, int dtype, int kind, const void* g, const void* x, const void* y,
+                       void* dx, void* dy, void* workspace, uint64_t workspace_bytes,
+                       uint64_t lead, uint64_t inner, uint32_t flags);
+
+/* Softmax over the last axis of x[rows, V] (SoftmaxOp(dim=-1), op.py:205-218):
+ *   forward   y = exp(x - max) / sum exp(x - max)    (cpu_softmax_forward, backend.py:354-362)
+ *   backward  dx (+)= y * (dy - sum(dy * y))          (cpu_softmax_backward, backend.py:364-374)
+ * y may be x (in place).  AGRAD_ACC_INPUT_GRAD accumulates into dx. */
+int agrad_softmax_forward(agrad_ctx* ctx, int dtype, const void* x, void* y, uint64_t rows, uint32_t V);
+int agrad_softmax_backward(agrad_ctx* ctx, int dtype, const void* y, const void* dy, void* dx,
+                           uint64_t rows, uint32_t V, uint32_t flags);
+
 /* Strided gather into a dense tensor: dst[dense index over shape] (+)=
  * src[sum_i coord_i * strides[i]], strides in elements (0 broadcasts), ndim <=
  * AGRAD_MAX_DIMS.  Contiguous forward of a permuted / transposed view and the

@@ -18,8 +18,8 @@ import numpy as np
 from autograd_amd.backend import Backend
 from autograd_amd.device import Device
 from autograd_amd.op import (AddLayerNormOp, AddOp, AddRMSNormOp, ContiguousOp, CrossEntropyLossOp, EmbeddingSumOp,
-                             GatherOp, GELUOp, LayerNormOp, PermuteOp, ReLUSquaredOp, ReshapeOp, RMSNormOp, RopeOp,
-                             SwiGLUOp, TransposeOp, ViewOp)
+                             ExpOp, GatherOp, GELUOp, LayerNormOp, LogOp, MulOp, PermuteOp, ReLUSquaredOp, ReshapeOp,
+                             RMSNormOp, RopeOp, RsqrtOp, SoftmaxOp, SwiGLUOp, TransposeOp, ViewOp)
 from autograd_amd.storage import Allocator, Storage
 from autograd_amd.utils import is_bf16, storage_dtype
 
@@ -87,6 +87,43 @@ def cpu_add_backward(inputs, outputs, scratch=None):
         if t.requires_grad and t.grad is not None:
             with _Acc(t.grad) as acc:
                 K.add_backward_into(g, acc)
+
+
+def cpu_mul_forward(inputs, outputs, scratch=None):
+    _put(outputs[0], K.mul_forward(_val(inputs[0]), _val(inputs[1])))
+
+
+def cpu_mul_backward(inputs, outputs, scratch=None):
+    x, y, out = inputs[0], inputs[1], outputs[0]
+    if out.grad is None:
+        return
+    g, xv, yv = _val(out.grad), _val(x), _val(y)
+    if x.requires_grad and x.grad is not None:
+        with _Acc(x.grad) as acc:
+            K.mul_backward_into(g, xv, yv, dx=acc)
+    if y.requires_grad and y.grad is not None:
+        with _Acc(y.grad) as acc:
+            K.mul_backward_into(g, xv, yv, dy=acc)
+
+
+def _cpu_unary(fwd, bwd, saves_output):
+    def forward(inputs, outputs, scratch=None):
+        _put(outputs[0], fwd(_val(inputs[0])))
+
+    def backward(inputs, outputs, scratch=None):
+        x, out = inputs[0], outputs[0]
+        if out.grad is None or not x.requires_grad:
+            return
+        with _Acc(x.grad) as acc:
+            bwd(_val(out.grad), _val(out if saves_output else x), acc)
+    return forward, backward
+
+
+cpu_exp_forward, cpu_exp_backward = _cpu_unary(K.exp_forward, K.exp_backward_into, True)
+cpu_log_forward, cpu_log_backward = _cpu_unary(K.log_forward, K.log_backward_into, False)
+cpu_rsqrt_forward, cpu_rsqrt_backward = _cpu_unary(K.rsqrt_forward, K.rsqrt_backward_into, True)
+cpu_softmax_forward, cpu_softmax_backward = _cpu_unary(
+    K.softmax_forward, lambda g, y, acc: K.softmax_backward_into(y, g, acc), True)
 
 
 # views share their input's memory: nothing to do going forward (backend.py:263-313)
@@ -338,6 +375,8 @@ class CPUBackend(Backend):
             LayerNormOp: cpu_layernorm_forward, RMSNormOp: cpu_rmsnorm_forward,
             AddLayerNormOp: cpu_add_norm_forward, AddRMSNormOp: cpu_add_norm_forward, RopeOp: cpu_rope_forward,
             CrossEntropyLossOp: cpu_cross_entropy_forward,
+            MulOp: cpu_mul_forward, ExpOp: cpu_exp_forward, LogOp: cpu_log_forward, RsqrtOp: cpu_rsqrt_forward,
+            SoftmaxOp: cpu_softmax_forward,
             ViewOp: cpu_view_forward, ReshapeOp: cpu_view_forward, PermuteOp: cpu_view_forward,
             TransposeOp: cpu_view_forward, ContiguousOp: cpu_contiguous_forward,
         }
@@ -347,6 +386,8 @@ class CPUBackend(Backend):
             LayerNormOp: cpu_layernorm_backward, RMSNormOp: cpu_rmsnorm_backward,
             AddLayerNormOp: cpu_add_norm_backward, AddRMSNormOp: cpu_add_norm_backward, RopeOp: cpu_rope_backward,
             CrossEntropyLossOp: cpu_cross_entropy_backward,
+            MulOp: cpu_mul_backward, ExpOp: cpu_exp_backward, LogOp: cpu_log_backward, RsqrtOp: cpu_rsqrt_backward,
+            SoftmaxOp: cpu_softmax_backward,
             ViewOp: cpu_dense_grad_backward, ReshapeOp: cpu_dense_grad_backward, PermuteOp: cpu_permute_backward,
             TransposeOp: cpu_transpose_backward, ContiguousOp: cpu_dense_grad_backward,
         }

@@ -21,6 +21,9 @@ Pinning (what shows these functions are the right functions; tests/test_oracle.p
     differences, rows of the gradient sum to zero, uniform logits give log V.
   * strided views / permute gradients: an explicit loop over every dense index
     with the index arithmetic written out, on small shapes.
+  * mul / exp / log / rsqrt / softmax: float64 closed forms (scipy.special.softmax,
+    the softmax Jacobian written out), explicit index loops for the broadcast sums
+    of the mul gradient, finite differences, rows of a softmax sum to one.
   * adamw: the textbook bias-corrected recurrence in float64 over several steps;
     the first step from zero moments moves every weight by lr * sign(g).
 Parity unpinned by the reference:
@@ -59,6 +62,95 @@ def add_backward_into(g, grad):
     axes = tuple(i for i, (gi, ti) in enumerate(zip(g.shape, padded)) if ti == 1 and gi != 1)
     tmp = np.sum(g, axis=axes) if axes else g
     np.add(grad, tmp.reshape(grad.shape), out=grad)
+
+
+# --------------------------------------------------------------------------
+# Mul  (cpu_mul_forward / cpu_mul_backward, backend.py:107-146; mul_bcast_kind,
+# utils.py:134-143)
+# --------------------------------------------------------------------------
+def mul_kind(x_shape, y_shape):
+    x_shape, y_shape = tuple(x_shape), tuple(y_shape)
+    if len(y_shape) == 0 or int(np.prod(y_shape)) == 1:
+        return "scalar"
+    if len(y_shape) == 1 and x_shape[-1] == y_shape[0]:
+        return "row"
+    if len(y_shape) == len(x_shape) and y_shape[:-1] == x_shape[:-1] and y_shape[-1] == 1:
+        return "col"
+    if y_shape == x_shape:
+        return "same"
+    raise RuntimeError(f"Mul backward: unsupported broadcast x={x_shape} y={y_shape}")
+
+
+def mul_forward(x, y):
+    return np.multiply(x, y)
+
+
+def mul_backward_into(g, x, y, dx=None, dy=None):
+    kind = mul_kind(g.shape, y.shape)
+    if dx is not None:
+        if kind == "scalar":
+            s = y.reshape(())
+            np.add(dx, g if s == 1 else np.multiply(g, s, dtype=g.dtype), out=dx)
+        else:
+            np.add(dx, np.multiply(g, y, dtype=g.dtype), out=dx)
+    if dy is None:
+        return
+    full = np.multiply(g, x, dtype=dy.dtype)
+    if kind == "scalar":
+        red = np.empty(dy.shape, dy.dtype)
+        red[...] = np.sum(full, dtype=dy.dtype)
+    elif kind == "row":
+        red = np.sum(full, axis=tuple(range(g.ndim - 1)))
+    elif kind == "col":
+        red = np.sum(full, axis=-1, keepdims=True)
+    else:
+        red = full
+    np.add(dy, red.reshape(dy.shape), out=dy)
+
+
+# --------------------------------------------------------------------------
+# Exp, Log, Rsqrt, Softmax  (backend.py:320-374)
+# --------------------------------------------------------------------------
+def exp_forward(x):
+    return np.exp(x)
+
+
+def exp_backward_into(dy, y, dx):
+    np.add(dx, dy * y, out=dx)
+
+
+def log_forward(x):
+    return np.log(x)
+
+
+def log_backward_into(dy, x, dx):
+    np.add(dx, dy / x, out=dx)
+
+
+def rsqrt_forward(x):
+    t = np.sqrt(x)
+    return np.reciprocal(t)
+
+
+def rsqrt_backward_into(dy, y, dx):
+    np.add(dx, dy * (-0.5) * y * y * y, out=dx)
+
+
+def softmax_forward(x):
+    m = np.max(x, axis=-1, keepdims=True)
+    e = np.subtract(x, m)
+    np.exp(e, out=e)
+    s = np.sum(e, axis=-1, keepdims=True)
+    np.divide(e, s, out=e)
+    return e
+
+
+def softmax_backward_into(y, g, dx):
+    t = np.multiply(g, y)
+    dot = np.sum(t, axis=-1, keepdims=True)
+    np.subtract(g, dot, out=t)
+    np.multiply(y, t, out=t)
+    np.add(dx, t, out=dx)
 
 
 # --------------------------------------------------------------------------

@@ -148,7 +148,7 @@ def test_unknown_device_and_kernel():
         Device.get_backend("mps")
     ctx = Device.get_backend("hip").ctx
     with pytest.raises(RuntimeError):
-        ctx.dispatch_with_args_3d("softmax_forward", [], [], [], 1, 1, 1, 1)
+        ctx.dispatch_with_args_3d("sdpa_forward", [], [], [], 1, 1, 1, 1)     # attention is not part of this library
     with pytest.raises(ValueError):      # wrong operand count
         ctx.dispatch_with_args_3d("gelu_forward_kernel", [0], [0], [0, 1, 0], 1, 1, 1, 1)
     buf = ctx.alloc(64)
@@ -432,6 +432,47 @@ def test_execution_plans_share_one_arena():
     for a, b in zip(results["hip"][:2], results["hip"][2:]):
         for x0, x1 in zip(a, b):
             np.testing.assert_array_equal(x0, x1)
+
+
+def test_primitive_ops_in_a_graph():
+    """Mul in all four broadcast kinds (one of them x * x), Softmax, Exp, Log and Rsqrt
+    chained in one graph on both devices (the reference probes them one at a time:
+    check_tiny_gpt2_kernel.py:699-724, verify_ops.py:47-91)"""
+    rng = np.random.default_rng(SEED + 33)
+    B, T, C = 3, 70, 96
+    x_np = rng.standard_normal((B, T, C), dtype=np.float32)
+    w_np = (1 + 0.2 * rng.standard_normal(C)).astype(np.float32)
+    s_np = np.array([0.37], np.float32)
+    c_np = rng.uniform(0.5, 1.5, (B, T, 1)).astype(np.float32)
+    upstream = rng.standard_normal((B, T, C), dtype=np.float32)
+
+    def build(device):
+        x = make_tensor(x_np.shape, np.float32, device, True, x_np, "x")
+        w = make_tensor(w_np.shape, np.float32, device, True, w_np, "w")
+        sc = make_tensor(s_np.shape, np.float32, device, True, s_np, "s")
+        cv = make_tensor(c_np.shape, np.float32, device, True, c_np, "c")
+        p = (x * w).softmax(-1)            # row kind, softmax
+        r = (p * sc).exp()                 # scalar kind, exp: a little above 1
+        u = (x * x) + r                    # same kind with both operands one tensor; >= 1
+        out = ((u.log() + r) * cv).rsqrt()   # log, col kind, rsqrt (every step well-conditioned)
+        return out, {"x": x, "w": w, "s": sc, "c": cv}
+
+    (c_out, c_g), (h_out, h_g) = both(build, upstream)
+    assert_fp32_close(h_out[0], c_out[0], "forward", rtol=2e-5, atol=2e-6)
+    scale = float(np.abs(c_g["x"]).max())
+    assert_fp32_close(h_g["x"], c_g["x"], "x.grad", rtol=1e-4, atol=1e-5 * scale)
+    for name, terms in (("w", B * T), ("s", B * T * C), ("c", C)):
+        ref_g = c_g[name]
+        bound = 1e-5 * np.sqrt(terms) * (np.abs(ref_g).max() + 1.0)
+        assert np.abs(h_g[name] - ref_g).max() <= bound, (name, np.abs(h_g[name] - ref_g).max(), bound)
+    # float64 check of the forward value, so that both devices agreeing is not the only evidence
+    x64, w64 = x_np.astype(np.float64), w_np.astype(np.float64)
+    a = x64 * w64
+    p64 = np.exp(a - a.max(-1, keepdims=True))
+    p64 /= p64.sum(-1, keepdims=True)
+    r64 = np.exp(p64 * float(s_np[0]))
+    want = ((np.log(x64 * x64 + r64) + r64) * c_np.astype(np.float64)) ** -0.5
+    np.testing.assert_allclose(h_out[0], want, rtol=2e-5, atol=1e-6)
 
 
 def test_captured_graph_replays_match_eager():

@@ -51,7 +51,7 @@ def test_header_compiles_as_plain_c(tmp_path):
 
 def test_library_reports_errors_without_gpu_or_kernel():
     lib = capi.load_library()
-    assert lib.agrad_kernel_count() == 32
+    assert lib.agrad_kernel_count() == 38
     names = [lib.agrad_kernel_name(i).decode() for i in range(lib.agrad_kernel_count())]
     for n in ("layernorm_forward", "layernorm_backward_kernel", "rmsnorm_forward", "rmsnorm_backward",
               "gelu_forward_kernel", "gelu_backward_kernel", "swiglu_forward_kernel", "rope_qk_inplace",
@@ -140,6 +140,26 @@ def test_op_shapes_and_errors():
     assert (x + x).op.op.op_name == "Add" and x.gelu().op.op.op_name == "GELU"
     # requires_grad propagates; gather ignores the integer operand
     assert not GatherOp()(ids, T((11, 8), requires_grad=False)).requires_grad
+
+
+def test_primitive_op_shapes_and_errors():
+    """Mul's broadcast kinds are the reference's (utils.py:134-143); Softmax takes the last axis"""
+    from autograd_amd.utils import mul_bcast_kind
+    x = T((2, 3, 8))
+    assert (x * T((2, 3, 8))).shape == (2, 3, 8) and (x * T((8,))).shape == (2, 3, 8)
+    assert (x * T((2, 3, 1))).shape == (2, 3, 8) and (x * T((1,))).op.op.op_name == "Mul"
+    assert [mul_bcast_kind((2, 3, 8), s) for s in ((2, 3, 8), (8,), (2, 3, 1), (1,), ())] == \
+        ["same", "row", "col", "scalar", "scalar"]
+    with pytest.raises(RuntimeError):
+        x * T((3, 8))                  # no kernel for a middle-axes broadcast
+    with pytest.raises(RuntimeError):
+        T((8,)) * x                    # the broadcast operand goes second
+    assert x.exp().shape == x.log().shape == x.rsqrt().shape == x.shape
+    assert x.softmax(-1).op.op.dim == -1 and x.softmax(2).shape == x.shape
+    with pytest.raises(ValueError):
+        x.softmax(1)
+    assert x.exp().op.op.save_for_backward((x,), ("y",)) == ["y"]
+    assert x.log().op.op.save_for_backward((x,), ("y",)) == [x]
 
 
 def test_layout_ops_shapes_strides_and_errors():

@@ -490,3 +490,88 @@ def test_permute_and_transpose_gradients_match_the_index_loop():
     got = base.copy()
     K.transpose_backward_into(g, 1, 3, got)
     np.testing.assert_array_equal(got, want)
+
+
+# ---------------------------------------------------------------------------
+# Mul / Exp / Log / Rsqrt / Softmax: float64 closed forms, explicit loops,
+# finite differences
+# ---------------------------------------------------------------------------
+def test_mul_gradients_match_the_index_loops():
+    rng = np.random.default_rng(SEED + 80)
+    x = rng.standard_normal((3, 4, 5)).astype(np.float32)
+    g = rng.standard_normal((3, 4, 5)).astype(np.float32)
+    for yshape in [(3, 4, 5), (5,), (3, 4, 1), (1,)]:
+        y = rng.standard_normal(yshape).astype(np.float32)
+        np.testing.assert_array_equal(K.mul_forward(x, y), x * y)
+        dx0 = rng.standard_normal(x.shape).astype(np.float32)
+        dy0 = rng.standard_normal(yshape).astype(np.float32)
+        dx, dy = dx0.copy(), dy0.copy()
+        K.mul_backward_into(g, x, y, dx=dx, dy=dy)
+        yb = np.broadcast_to(y, x.shape)
+        want_dx = dx0.astype(np.float64)
+        want_dy = dy0.astype(np.float64).copy()
+        for idx in np.ndindex(*x.shape):
+            want_dx[idx] += float(g[idx]) * float(yb[idx])
+            if yshape == x.shape:
+                want_dy[idx] += float(g[idx]) * float(x[idx])
+            elif yshape == (5,):
+                want_dy[idx[2]] += float(g[idx]) * float(x[idx])
+            elif yshape == (3, 4, 1):
+                want_dy[idx[0], idx[1], 0] += float(g[idx]) * float(x[idx])
+            else:
+                want_dy[0] += float(g[idx]) * float(x[idx])
+        np.testing.assert_allclose(dx, want_dx, rtol=1e-6, atol=1e-6)
+        np.testing.assert_allclose(dy, want_dy, rtol=1e-5, atol=1e-5)
+    with pytest.raises(RuntimeError):
+        K.mul_kind((3, 4, 5), (4, 5))
+
+
+def test_unary_primitives_against_float64_and_finite_differences():
+    rng = np.random.default_rng(SEED + 81)
+    x = rng.uniform(0.1, 3.0, (7, 9)).astype(np.float32)
+    dy = rng.standard_normal((7, 9)).astype(np.float32)
+    x64 = x.astype(np.float64)
+    cases = [
+        (K.exp_forward, K.exp_backward_into, True, np.exp, np.exp),
+        (K.log_forward, K.log_backward_into, False, np.log, lambda v: 1.0 / v),
+        (K.rsqrt_forward, K.rsqrt_backward_into, True, lambda v: v ** -0.5, lambda v: -0.5 * v ** -1.5),
+    ]
+    for fwd, bwd, saves_y, f64, d64 in cases:
+        y = fwd(x)
+        assert y.dtype == np.float32
+        np.testing.assert_allclose(y, f64(x64), rtol=2e-7, atol=0)
+        dx = np.zeros_like(x)
+        bwd(dy, y if saves_y else x, dx)
+        np.testing.assert_allclose(dx, dy * d64(x64), rtol=1e-6, atol=1e-7)
+        h = 1e-4                                   # central difference of the float64 function
+        fd = (f64(x64 + h) - f64(x64 - h)) / (2 * h)
+        np.testing.assert_allclose(d64(x64), fd, rtol=1e-6, atol=1e-7)
+    # rsqrt is sqrt then reciprocal, each correctly rounded (backend.py:342-345)
+    np.testing.assert_array_equal(K.rsqrt_forward(x), np.float32(1.0) / np.sqrt(x))
+
+
+def test_softmax_against_scipy_and_its_jacobian():
+    from scipy.special import softmax as sp_softmax
+    rng = np.random.default_rng(SEED + 82)
+    x = (4.0 * rng.standard_normal((5, 6, 33))).astype(np.float32)
+    g = rng.standard_normal(x.shape).astype(np.float32)
+    y = K.softmax_forward(x)
+    want = sp_softmax(x.astype(np.float64), axis=-1)
+    np.testing.assert_allclose(y, want, rtol=2e-6, atol=1e-8)
+    np.testing.assert_allclose(y.sum(-1), 1.0, rtol=0, atol=2e-6)
+    # invariance to a per-row shift, and a row of equal logits gives 1/V
+    np.testing.assert_allclose(K.softmax_forward(x + np.float32(3.0)), y, rtol=3e-6, atol=1e-8)
+    np.testing.assert_allclose(K.softmax_forward(np.full((2, 8), 1.5, np.float32)), 0.125, rtol=1e-7)
+    dx = np.zeros_like(x)
+    K.softmax_backward_into(y, g, dx)
+    # J = diag(y) - y y^T, dx = J g, written out per row in float64
+    for r in np.ndindex(*x.shape[:-1]):
+        yr, gr = want[r], g[r].astype(np.float64)
+        J = np.diag(yr) - np.outer(yr, yr)
+        np.testing.assert_allclose(dx[r], J @ gr, rtol=2e-5, atol=2e-7)
+    np.testing.assert_allclose(dx.sum(-1), 0.0, atol=2e-6)      # rows of J sum to zero
+    # masked logits: exp(-inf) = 0 and no NaN
+    xm = x.copy()
+    xm[..., 5:9] = -np.inf
+    ym = K.softmax_forward(xm)
+    assert np.isfinite(ym).all() and not ym[..., 5:9].any()
