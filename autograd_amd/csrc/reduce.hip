@@ -60,46 +60,70 @@ bcast_add_kernel(const T* __restrict__ x, const T* __restrict__ y, T* __restrict
     VecIO<T, VEC>::store(out + idx * VEC, a);
 }
 
-// partial[blockIdx.x, :] = sum over rows blockIdx.x, blockIdx.x + gridDim.x, ... of g[row, :]
+// element i of a small operand that many rows re-read: an ordinary (cached) load
+template <typename T> __device__ __forceinline__ float small_elem(const T* y, uint64_t i) {
+    if constexpr (sizeof(T) == 2) return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(y)[i]);
+    else return reinterpret_cast<const float*>(y)[i];
+}
+
+// partial[p, :] = sum over rows p, p + P, p + 2P, ... of g[row, :] (* x2[row, :]), for P partial
+// rows.  `lanes` threads share a row (a multiple of 64 that covers the row's vectors, at most
+// the workgroup), so a workgroup of 256 takes 256 / lanes partial rows: narrow tensors
+// (C = 384: 96 vectors) keep three quarters of their lanes busy instead of three eighths.
+// With dx given the kernel also writes dx[row, :] (+)= g[row, :] * y[:] -- the other gradient
+// of x * y[:], from the g it has in registers anyway.
 template <typename T, int VEC>
 __global__ void __launch_bounds__(kColBlock)
-colsum_partial_kernel(const T* __restrict__ g, const T* __restrict__ x2, float* __restrict__ partial, uint64_t lead,
-                      uint32_t inner, uint32_t inner_vec) {
-    for (uint32_t cv = threadIdx.x; cv < inner_vec; cv += kColBlock) {
+colsum_partial_kernel(const T* __restrict__ g, const T* __restrict__ x2, const T* __restrict__ ysmall, T* dx,
+                      float* __restrict__ partial, uint64_t lead, uint32_t inner, uint32_t inner_vec, uint32_t lanes,
+                      uint32_t P, int acc_dx) {
+    const uint32_t sub = threadIdx.x / lanes, lane = threadIdx.x - sub * lanes;
+    const uint32_t p = blockIdx.x * (blockDim.x / lanes) + sub;
+    if (p >= P) return;
+    for (uint32_t cv = lane; cv < inner_vec; cv += lanes) {
         const uint32_t col = cv * VEC;
-        float acc[VEC];
+        float acc[VEC], yv[VEC];
 #pragma unroll
         for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
-        for (uint64_t r0 = blockIdx.x; r0 < lead; r0 += (uint64_t)gridDim.x * kColRows) {
-            float v[kColRows][VEC], w[kColRows][VEC];
+        if (dx != nullptr) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) yv[k] = small_elem<T>(ysmall, col + k);
+        }
+        for (uint64_t r0 = p; r0 < lead; r0 += (uint64_t)P * kColRows) {
+            float v[kColRows][VEC], w[kColRows][VEC], o[kColRows][VEC];
 #pragma unroll
             for (int u = 0; u < kColRows; ++u) {
-                const uint64_t r = r0 + (uint64_t)u * gridDim.x;
+                const uint64_t r = r0 + (uint64_t)u * P;
                 if (r < lead) {
                     VecIO<T, VEC>::load(g + r * inner + col, v[u]);
-                    if (x2 != nullptr) VecIO<T, VEC>::load(x2 + r * inner + col, w[u]);   // uniform branch
+                    if (x2 != nullptr) VecIO<T, VEC>::load(x2 + r * inner + col, w[u]);   // uniform branches
+                    if (dx != nullptr && acc_dx) VecIO<T, VEC>::load(dx + r * inner + col, o[u]);
                 }
             }
 #pragma unroll
             for (int u = 0; u < kColRows; ++u) {
-                const uint64_t r = r0 + (uint64_t)u * gridDim.x;
+                const uint64_t r = r0 + (uint64_t)u * P;
                 if (r < lead) {
 #pragma unroll
                     for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + (x2 != nullptr ? v[u][k] * w[u][k] : v[u][k]);
+                    if (dx != nullptr) {
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) {
+                            const float t = v[u][k] * yv[k];
+                            o[u][k] = acc_dx ? (o[u][k] + t) : t;
+                        }
+                        VecIO<T, VEC>::store(dx + r * inner + col, o[u]);
+                    }
                 }
             }
         }
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) partial[(uint64_t)blockIdx.x * inner + col + k] = acc[k];
+        for (int k = 0; k < VEC; ++k) partial[(uint64_t)p * inner + col + k] = acc[k];
     }
 }
 
 // ---- broadcast Mul --------------------------------------------------------------
 // out (+)= a[l, j] * y[..]: KIND AGRAD_MUL_ROW y[j], AGRAD_MUL_COL y[l], AGRAD_MUL_SCALAR y[0]
-template <typename T> __device__ __forceinline__ float small_elem(const T* y, uint64_t i) {
-    if constexpr (sizeof(T) == 2) return bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(y)[i]);
-    else return reinterpret_cast<const float*>(y)[i];
-}
 
 template <typename T, int VEC, int KIND>
 __global__ void __launch_bounds__(kBcastBlock)
@@ -283,13 +307,18 @@ namespace {
 // finished in fp32 and rounded once
 template <typename T>
 int colsum_two_stage(hipStream_t s, const T* g, const T* x2, T* dy, void* workspace, uint64_t lead, uint64_t inner,
-                     int accumulate) {
+                     int accumulate, const T* ysmall = nullptr, T* dx = nullptr, int acc_dx = 0) {
     constexpr int WIDE = WideVec<T>::value;
-    const uint32_t blocks = colsum_blocks(lead);
+    const uint32_t blocks = colsum_blocks(lead);     // partial rows
     float* partial = (float*)workspace;
-    const bool wide = inner % WIDE == 0 && aligned16(g) && (!x2 || aligned16(x2));
-    if (wide) hipLaunchKernelGGL((colsum_partial_kernel<T, WIDE>), dim3(blocks), dim3(kColBlock), 0, s, g, x2, partial, lead, (uint32_t)inner, (uint32_t)(inner / WIDE));
-    else hipLaunchKernelGGL((colsum_partial_kernel<T, 1>), dim3(blocks), dim3(kColBlock), 0, s, g, x2, partial, lead, (uint32_t)inner, (uint32_t)inner);
+    const bool wide = inner % WIDE == 0 && aligned16(g) && (!x2 || aligned16(x2)) && (!dx || aligned16(dx));
+    const uint32_t iv = (uint32_t)(wide ? inner / WIDE : inner);
+    uint32_t lanes = (iv + kWave - 1) / kWave * kWave;
+    if (lanes > (uint32_t)kColBlock) lanes = kColBlock;
+    const uint32_t per_wg = kColBlock / lanes;       // partial rows per workgroup
+    const dim3 grid((blocks + per_wg - 1) / per_wg), block(lanes * per_wg);
+    if (wide) hipLaunchKernelGGL((colsum_partial_kernel<T, WIDE>), grid, block, 0, s, g, x2, ysmall, dx, partial, lead, (uint32_t)inner, iv, lanes, blocks, acc_dx);
+    else hipLaunchKernelGGL((colsum_partial_kernel<T, 1>), grid, block, 0, s, g, x2, ysmall, dx, partial, lead, (uint32_t)inner, iv, lanes, blocks, acc_dx);
     if (int rc = check_hip(hipGetLastError(), "column sum launch")) return rc;
     if constexpr (sizeof(T) == 4) {
         return launch_colsum_finalize(s, partial, nullptr, blocks, (uint32_t)inner, (float*)dy, nullptr, accumulate);
@@ -407,6 +436,19 @@ int launch_mul_bwd(hipStream_t s, int dtype, int kind, const void* g, const void
         return AGRAD_OK;
     }
     if (g == nullptr) return set_error(AGRAD_EINVAL, "mul backward: null upstream gradient");
+    // x * y[:] with many rows and both gradients wanted: the column-sum kernel writes dx as
+    // well, from the g it has loaded anyway (g is then read once, not twice)
+    const bool fused = kind == AGRAD_MUL_ROW && dx != nullptr && dy != nullptr && x != nullptr && y != nullptr &&
+                       mul_bwd_workspace_bytes(kind, lead, inner) > 0 && workspace != nullptr &&
+                       workspace_bytes >= mul_bwd_workspace_bytes(kind, lead, inner) && aligned16(workspace) &&
+                       inner < 0x7fffffffull && lead < 0x7fffffffull;
+    if (fused) {
+        if (dtype == AGRAD_F32)
+            return colsum_two_stage<float>(s, (const float*)g, (const float*)x, (float*)dy, workspace, lead, inner, acc_y,
+                                           (const float*)y, (float*)dx, acc_x);
+        return colsum_two_stage<bf16_t>(s, (const bf16_t*)g, (const bf16_t*)x, (bf16_t*)dy, workspace, lead, inner, acc_y,
+                                        (const bf16_t*)y, (bf16_t*)dx, acc_x);
+    }
     if (dx != nullptr) {
         if (y == nullptr) return set_error(AGRAD_EINVAL, "mul backward: dx needs y");
         int rc;
