@@ -175,15 +175,28 @@ emb_prepare_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ keys,
 // tokens whose hash falls in group g.  It reads ALL ids (64 KiB at N = 16384,
 // served by L2), keeps the (token, row) pairs it owns in LDS, counts how many
 // rows belong to lower-numbered groups (that is where its slice of the output
-// starts), orders its pairs by (token, row) -- by rank counting when there is at
-// most one pair per thread, with a bitonic network otherwise -- and writes them
-// out.  No atomics on global memory, and the output is the same on every
-// run.  A group too large for LDS (one token holding a large share of all rows)
-// is gathered into its output slice and sorted there instead.
+// starts), orders its pairs by (token, row) and writes them out.  No atomics on
+// global memory, and the output is the same on every run.
+//
+// How a group orders its pairs depends on how many it has:
+//  * up to one per thread (the usual case: a few dozen): by rank counting;
+//  * more: some token is frequent (padding, a newline, "the").  The rows of ONE
+//    token need no sorting network: they are distinct integers below N, so the
+//    group marks them in an N-bit map and a row's place is the number of set
+//    bits below it.  The group picks its most frequent token from a sample,
+//    moves that token's rows into the bit map and orders only what is left --
+//    by rank when that fits one pair per thread, with a bitonic network in LDS
+//    otherwise.  (All rows one token: 640 us with the network over the whole
+//    list, against 40 us this way, at N = 16384.)
+//  * what is left after taking the frequent token out still exceeds LDS (two
+//    tokens of one group holding most rows): gathered into the group's slice of
+//    `spill` and sorted there -- slow, correct, and rare.
 constexpr int kSortBlock = 512;
 constexpr uint32_t kGroupSortMaxN = 16384;
 constexpr uint32_t kSortLdsEntries = 4096;   // (token, row) pairs a workgroup keeps in LDS
 constexpr uint32_t kRankSortMax = kSortBlock;  // lists up to one key per thread are placed by rank
+constexpr uint32_t kRowMapWords = kGroupSortMaxN / 32;
+static_assert(kRowMapWords == (uint32_t)kSortBlock, "one word of the row map per thread");
 
 // Bitonic network in its "flip" form: every comparator puts the smaller key at
 // the lower index, so positions >= n behave as +infinity and need no padding.
@@ -213,9 +226,16 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
                     uint32_t* __restrict__ row_s, unsigned long long* __restrict__ spill,
                     uint32_t N, uint32_t V, uint32_t log2G, int* err_flag) {
     __shared__ unsigned long long keys[kSortLdsEntries];
-    __shared__ uint32_t s_count, s_less;
+    __shared__ unsigned long long few[kRankSortMax];
+    __shared__ uint32_t row_map[kRowMapWords];
+    __shared__ uint32_t s_count, s_less, s_rest, s_below, s_wave_rows[kSortBlock / kWave];
     const uint32_t tid = threadIdx.x;
-    if (tid == 0) { s_count = 0; s_less = 0; }
+    const uint32_t lane = tid & (kWave - 1);
+    auto lanes_below = [&](unsigned long long mask) {     // set bits of `mask` below this lane
+        return (uint32_t)__builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+    };
+    if (tid == 0) { s_count = 0; s_less = 0; s_rest = 0; s_below = 0; }
+    row_map[tid] = 0;
     __syncthreads();
 
     auto owner_of = [&](int32_t t, uint32_t& tok) {
@@ -233,17 +253,40 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
             const uint32_t i = base + r * kSortBlock + tid;
             t[r] = i < N ? ids[i] : -1;
         }
+        // The pairs this group owns go into the list.  One LDS atomic per wave and
+        // eight loads, not one per pair: a frequent token would otherwise queue
+        // thousands of them on one address, and waiting for each one's return
+        // value in turn costs the usual case a microsecond.
+        constexpr int AGG = 8;
 #pragma unroll
-        for (int r = 0; r < ROUND; ++r) {
-            const uint32_t i = base + r * kSortBlock + tid;
-            if (i < N) {
+        for (int r0 = 0; r0 < ROUND; r0 += AGG) {
+            unsigned long long owners[AGG];
+            uint32_t wave_total = 0;
+#pragma unroll
+            for (int a = 0; a < AGG; ++a) {
+                const uint32_t i = base + (r0 + a) * kSortBlock + tid;
+                const bool live = i < N;
                 uint32_t tok;
-                const uint32_t owner = owner_of(t[r], tok);
-                if (tok == V && g == 0) *err_flag = 1;
-                less += owner < g ? 1u : 0u;
-                if (owner == g) {
-                    const uint32_t slot = atomicAdd(&s_count, 1u);
-                    if (slot < kSortLdsEntries) keys[slot] = ((unsigned long long)tok << 32) | i;
+                const uint32_t owner = owner_of(t[r0 + a], tok);
+                if (live && tok == V && g == 0) *err_flag = 1;
+                less += live && owner < g ? 1u : 0u;
+                owners[a] = __ballot(live && owner == g);
+                wave_total += (uint32_t)__popcll(owners[a]);
+            }
+            if (wave_total) {
+                uint32_t first = 0;
+                if (lane == 0) first = atomicAdd(&s_count, wave_total);
+                first = (uint32_t)__builtin_amdgcn_readfirstlane((int)first);
+#pragma unroll
+                for (int a = 0; a < AGG; ++a) {
+                    const uint32_t i = base + (r0 + a) * kSortBlock + tid;
+                    const uint32_t slot = first + lanes_below(owners[a]);
+                    if (((owners[a] >> lane) & 1ull) && slot < kSortLdsEntries) {
+                        const int32_t id = t[r0 + a];
+                        const uint32_t tok = id < 0 || (uint32_t)id >= V ? V : (uint32_t)id;
+                        keys[slot] = ((unsigned long long)tok << 32) | i;
+                    }
+                    first += (uint32_t)__popcll(owners[a]);
                 }
             }
         }
@@ -257,16 +300,16 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
         v += __builtin_amdgcn_update_dpp(0, v, kDppRowMirror, 0xf, 0xf, true);
         v += __builtin_amdgcn_ds_swizzle(v, kSwizzleXor16);
         const uint32_t total = __builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 32);
-        if ((tid & (kWave - 1)) == 0) atomicAdd(&s_less, total);
+        if (lane == 0) atomicAdd(&s_less, total);
     }
     __syncthreads();
     const uint32_t count = s_count;
     const uint32_t offset = s_less;
 
     if (count <= kRankSortMax) {
-        // the usual case (a few dozen pairs): every key is unique, so its place
-        // in the order is the number of smaller keys.  Each thread counts that
-        // for its own key with broadcast LDS reads -- no barriers, no exchanges.
+        // every key is unique, so its place in the order is the number of
+        // smaller keys.  Each thread counts that for its own key with broadcast
+        // LDS reads -- no barriers, no exchanges.
         const unsigned long long mine = tid < count ? keys[tid] : ~0ull;
         uint32_t rank = 0;
 #pragma unroll 8
@@ -277,33 +320,168 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
         }
         return;
     }
-    if (count <= kSortLdsEntries) {
-        bitonic_sort_u64<kSortBlock>(keys, count, tid, [] { __syncthreads(); });
+
+    // -- a frequent token: of 64 evenly spaced pairs of the list, the token seen
+    // most often among 16 candidates.  Every wave works it out for itself from
+    // the same samples.  (Which pairs the list holds, and in what order, varies
+    // from run to run; a different choice changes the time taken, never the output.)
+    const uint32_t listed = count < kSortLdsEntries ? count : kSortLdsEntries;
+    const bool reread = count > kSortLdsEntries;
+    uint32_t hot = 0;
+    {
+        const uint32_t sample = (uint32_t)(keys[(lane * listed) / kWave] >> 32);
+        uint32_t best_votes = 0;
+#pragma nounroll
+        for (int k = 0; k < kWave; k += 4) {
+            const uint32_t candidate = (uint32_t)__builtin_amdgcn_readlane((int)sample, k);
+            const uint32_t votes = (uint32_t)__popcll(__ballot(sample == candidate));
+            if (votes > best_votes) { best_votes = votes; hot = candidate; }
+        }
+    }
+    if (reread) __syncthreads();         // `keys` is about to be overwritten
+
+    // its rows go into the row map, every other pair into `rest`.  A list that
+    // fits LDS is split from LDS and stays intact; a longer one is read again
+    // from the ids, and `keys` becomes the rest.
+    unsigned long long* rest = reread ? keys : few;
+    const uint32_t rest_cap = reread ? kSortLdsEntries : kRankSortMax;
+    auto split = [&](uint32_t tok, uint32_t row) {
+        if (tok == hot) {
+            atomicOr(&row_map[row >> 5], 1u << (row & 31));
+        } else {
+            const uint32_t slot = atomicAdd(&s_rest, 1u);
+            if (slot < rest_cap) rest[slot] = ((unsigned long long)tok << 32) | row;
+        }
+    };
+    if (!reread) {
         for (uint32_t i = tid; i < count; i += kSortBlock) {
             const unsigned long long key = keys[i];
+            split((uint32_t)(key >> 32), (uint32_t)key);
+        }
+    } else {
+        // a wave looks at 64 consecutive rows: two whole words of the map, stored
+        // once each, no atomics
+        constexpr int AGAIN = 8;
+        for (uint32_t base = 0; base < N; base += kSortBlock * AGAIN) {
+            int32_t t[AGAIN];
+#pragma unroll
+            for (int r = 0; r < AGAIN; ++r) {
+                const uint32_t i = base + r * kSortBlock + tid;
+                t[r] = i < N ? ids[i] : -1;
+            }
+#pragma unroll
+            for (int r = 0; r < AGAIN; ++r) {
+                const uint32_t i = base + r * kSortBlock + tid;      // below kGroupSortMaxN, also when >= N
+                uint32_t tok;
+                const bool own = owner_of(t[r], tok) == g && i < N;
+                const bool is_hot = own && tok == hot;
+                const unsigned long long marks = __ballot(is_hot);
+                if (i < kGroupSortMaxN) {
+                    if (lane == 0) row_map[i >> 5] = (uint32_t)marks;
+                    if (lane == 32) row_map[i >> 5] = (uint32_t)(marks >> 32);
+                }
+                if (own && !is_hot) split(tok, i);
+            }
+        }
+    }
+    __syncthreads();
+    const uint32_t rest_n = s_rest;
+
+    if (rest_n > rest_cap) {
+        if (!reread) {
+            // no single frequent token: the network over the whole list
+            bitonic_sort_u64<kSortBlock>(keys, count, tid, [] { __syncthreads(); });
+            for (uint32_t i = tid; i < count; i += kSortBlock) {
+                const unsigned long long key = keys[i];
+                tok_s[offset + i] = (uint32_t)(key >> 32);
+                row_s[offset + i] = (uint32_t)key;
+            }
+            return;
+        }
+        // gather the group's pairs into its slice of `spill` (slices are
+        // disjoint: [offset, offset + count)), sort there, then split
+        __syncthreads();
+        if (tid == 0) s_count = 0;
+        __syncthreads();
+        unsigned long long* mine = spill + offset;
+        for (uint32_t i = tid; i < N; i += kSortBlock) {
+            uint32_t tok;
+            if (owner_of(ids[i], tok) == g) mine[atomicAdd(&s_count, 1u)] = ((unsigned long long)tok << 32) | i;
+        }
+        __threadfence_block();
+        __syncthreads();
+        bitonic_sort_u64<kSortBlock>(mine, count, tid, [] { __threadfence_block(); __syncthreads(); });
+        for (uint32_t i = tid; i < count; i += kSortBlock) {
+            const unsigned long long key = mine[i];
             tok_s[offset + i] = (uint32_t)(key >> 32);
             row_s[offset + i] = (uint32_t)key;
         }
         return;
     }
 
-    // oversized group: gather its pairs into this group's slice of `spill`
-    // (slices are disjoint: [offset, offset + count)), sort there, then split
-    __syncthreads();
-    if (tid == 0) s_count = 0;
-    __syncthreads();
-    unsigned long long* mine = spill + offset;
-    for (uint32_t i = tid; i < N; i += kSortBlock) {
-        uint32_t tok;
-        if (owner_of(ids[i], tok) == g) mine[atomicAdd(&s_count, 1u)] = ((unsigned long long)tok << 32) | i;
+    // -- the rest, in order; pairs above the frequent token leave room for its rows
+    const uint32_t hot_rows = count - rest_n;
+    uint32_t below;                                // pairs of the rest that sort before the frequent token
+    if (rest_n <= kRankSortMax) {
+        const unsigned long long mine = tid < rest_n ? rest[tid] : ~0ull;
+        const uint32_t tok = (uint32_t)(mine >> 32);
+        uint32_t rank = 0;
+#pragma unroll 8
+        for (uint32_t j = 0; j < rest_n; ++j) rank += rest[j] < mine ? 1u : 0u;
+        if (tid < rest_n) {
+            const uint32_t at = offset + rank + (tok > hot ? hot_rows : 0u);
+            tok_s[at] = tok;
+            row_s[at] = (uint32_t)mine;
+        }
+        below = (uint32_t)__syncthreads_count(tid < rest_n && tok < hot);
+    } else {
+        bitonic_sort_u64<kSortBlock>(rest, rest_n, tid, [] { __syncthreads(); });
+        uint32_t n_below = 0;
+        for (uint32_t i = tid; i < rest_n; i += kSortBlock) {
+            const unsigned long long key = rest[i];
+            const uint32_t tok = (uint32_t)(key >> 32);
+            n_below += tok < hot ? 1u : 0u;
+            const uint32_t at = offset + i + (tok > hot ? hot_rows : 0u);
+            tok_s[at] = tok;
+            row_s[at] = (uint32_t)key;
+        }
+        if (n_below) atomicAdd(&s_below, n_below);
+        __syncthreads();
+        below = s_below;
     }
-    __threadfence_block();
+
+    // -- the frequent token's rows.  Word w of the map holds rows 32 w ... 32 w + 31;
+    // a wave takes 64 words, two at a time: each half-wave gives one word's 32
+    // rows a lane each, and a marked row's place is the count of marks before it,
+    // so a store instruction writes up to 64 neighbouring entries.
+    {
+        uint32_t v = (uint32_t)__popc(row_map[tid]);
+        v += __builtin_amdgcn_update_dpp(0, v, kDppQuadXor1, 0xf, 0xf, true);
+        v += __builtin_amdgcn_update_dpp(0, v, kDppQuadXor2, 0xf, 0xf, true);
+        v += __builtin_amdgcn_update_dpp(0, v, kDppRowHalfMirror, 0xf, 0xf, true);
+        v += __builtin_amdgcn_update_dpp(0, v, kDppRowMirror, 0xf, 0xf, true);
+        v += __builtin_amdgcn_ds_swizzle(v, kSwizzleXor16);
+        const uint32_t wave_rows = __builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 32);   // read with every lane active
+        if (lane == 0) s_wave_rows[tid / kWave] = wave_rows;
+    }
     __syncthreads();
-    bitonic_sort_u64<kSortBlock>(mine, count, tid, [] { __threadfence_block(); __syncthreads(); });
-    for (uint32_t i = tid; i < count; i += kSortBlock) {
-        const unsigned long long key = mine[i];
-        tok_s[offset + i] = (uint32_t)(key >> 32);
-        row_s[offset + i] = (uint32_t)key;
+    const uint32_t wave = tid / kWave;
+    uint32_t at = offset + below;
+    for (uint32_t w = 0; w < wave; ++w) at += s_wave_rows[w];
+    if (s_wave_rows[wave] == 0) return;
+    const uint32_t upper = lane >> 5, bit = lane & 31u;
+#pragma nounroll
+    for (uint32_t pair = 0; pair < kWave / 2; ++pair) {
+        const uint32_t w0 = wave * kWave + 2 * pair;
+        const uint32_t word0 = row_map[w0], word1 = row_map[w0 + 1];
+        const uint32_t n0 = (uint32_t)__popc(word0);
+        const uint32_t word = upper ? word1 : word0;
+        if ((word >> bit) & 1u) {
+            const uint32_t to = at + (upper ? n0 : 0u) + (uint32_t)__popc(word & ((1u << bit) - 1u));
+            tok_s[to] = hot;
+            row_s[to] = (w0 + upper) * 32u + bit;
+        }
+        at += n0 + (uint32_t)__popc(word1);
     }
 }
 
@@ -330,9 +508,11 @@ emb_group_sort_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ to
 // pass nothing and the forward pass next to nothing.  (Doing the same with a
 // second stream and events was measured three times more expensive than the
 // ordering itself.)  One 16-byte vector per thread; with a position table the
-// rows are added in fp32.
+// rows are added in fp32.  Held to 80 scalar registers: compiled to 86 or more
+// (the ordering code's appetite, the gather needs a dozen) the gather ran 5 %
+// slower -- 38.2 against 36.2 us at 16384 x 1536 fp32.
 template <typename T, int VEC, bool RAW>
-__global__ void __launch_bounds__(kSortBlock)
+__global__ void __launch_bounds__(kSortBlock) __attribute__((amdgpu_num_sgpr(80)))
 gather_sort_kernel(const int32_t* __restrict__ ids, const T* __restrict__ W, const T* __restrict__ wpe,
                    T* __restrict__ out, uint32_t total, uint32_t CV, uint32_t C, uint32_t T_len, uint32_t V,
                    uint32_t* __restrict__ tok_s, uint32_t* __restrict__ row_s, unsigned long long* __restrict__ spill,

@@ -772,3 +772,91 @@ def test_presorted_embedding_pair_matches_the_plain_pair(ctx, B, T, V, C, dist, 
     for d in (d_ids, d_W, d_dY, d_wpe, d_dwpe, out, order, sws, bws):
         if d is not None:
             d.free()
+
+
+def _same_group_tokens(V, how_many, log2g=7):
+    """tokens below V that the grouping sort hands to one workgroup (its hash:
+    the top log2g bits of token * 0x9E3779B1 mod 2^32)"""
+    toks = np.arange(V, dtype=np.uint64)
+    group = ((toks * np.uint64(0x9E3779B1)) & np.uint64(0xFFFFFFFF)) >> np.uint64(32 - log2g)
+    best = np.bincount(group.astype(np.int64)).argmax()
+    found = toks[group == best][:how_many].astype(np.int32)
+    assert len(found) == how_many
+    return found
+
+
+_SKEWED = {
+    # name: (N, [(rows of a token, how many such tokens)...] all within one hash group, rest of N uniform)
+    "all_rows_one_token": (16384, [(16384, 1)]),
+    "padding_third": (16384, [(5500, 1)]),
+    "two_tokens_split": (16384, [(8192, 2)]),                 # what is left after the frequent one exceeds LDS
+    "frequent_plus_few": (16384, [(5000, 1), (3, 100)]),      # ids read again, the rest placed by rank
+    "frequent_plus_many": (16384, [(5000, 1), (20, 100)]),    # ids read again, the rest through the network
+    "listed_frequent_plus_few": (8192, [(1500, 1), (2, 100)]),   # list fits LDS, the rest placed by rank
+    "listed_no_frequent": (8192, [(400, 3)]),                 # list fits LDS, no single frequent token
+    "short_input": (1500, [(1400, 1)]),                       # fewer rows than the row map has bits
+    "bad_ids_frequent": (4096, [(0, 1)]),                     # out-of-range ids (one sentinel token) dominate
+}
+
+
+@pytest.mark.parametrize("case", sorted(_SKEWED))
+def test_id_ordering_with_frequent_tokens(ctx, case):
+    """The one-launch ordering on skewed ids: one token holding most rows (its rows
+    go through a bit map instead of the sorting network), several such tokens in
+    one hash group, and the fall-backs behind them.  Checked on the order itself
+    (each token's rows adjacent and ascending, every row once) and on the
+    gradient built from it, bit for bit against the atomic-free plain call."""
+    import ctypes as Ct
+    N, spec = _SKEWED[case]
+    V, C = 30000, 64
+    rng = _rng(abs(hash(case)) % 1000)
+    ids = rng.integers(0, V, N, dtype=np.int32)
+    if case == "bad_ids_frequent":
+        ids[rng.permutation(N)[:3000]] = -5
+    else:
+        same = _same_group_tokens(V, sum(k for _, k in spec))
+        slots = rng.permutation(N)
+        at = t = 0
+        for rows, k in spec:
+            for _ in range(k):
+                ids[slots[at:at + rows]] = same[t]
+                at += rows
+                t += 1
+    dY = rng.standard_normal((N, C)).astype(np.float32)
+    W = np.zeros((V, C), np.float32)
+
+    def vp(d):
+        return Ct.c_void_p(d.ptr)
+    d_ids, d_W, d_dY = ctx.upload(ids), ctx.upload(W), ctx.upload(dY)
+    out = ctx.empty((N, C), np.float32)
+    order = ctx.empty((2 * N,), np.uint32)
+    sws_b = ctx.lib.agrad_embedding_sort_workspace_bytes(N, V)
+    bws_b = ctx.lib.agrad_embedding_backward_sorted_workspace_bytes(N, C)
+    sws, bws = ctx.empty((sws_b,), np.uint8), ctx.empty((bws_b,), np.uint8)
+    valid = (ids >= 0) & (ids < V)
+    want_dW = np.zeros((V, C), np.float32)
+    if case != "bad_ids_frequent":
+        want_dW = G.embedding_backward(ctx, ids.reshape(1, N), dY.reshape(1, N, C), V)
+    for rep in range(2):
+        dW = ctx.zeros((V, C), np.float32)
+        ctx.call("agrad_gather_forward_sorted", capi.F32, vp(d_ids), vp(d_W), None, vp(out), N, 1, C, V,
+                 vp(order), vp(sws), sws_b)
+        if case == "bad_ids_frequent":
+            with pytest.raises(IndexError):
+                ctx.synchronize()
+        ctx.synchronize()
+        got = order.download()
+        toks, rows = got[:N], got[N:]
+        np.testing.assert_array_equal(np.sort(rows), np.arange(N))
+        np.testing.assert_array_equal(toks, np.where(valid, ids, V)[rows])
+        d_tok = np.diff(toks.astype(np.int64))
+        assert len(np.unique(toks)) == int((d_tok != 0).sum()) + 1
+        assert (np.diff(rows.astype(np.int64))[d_tok == 0] > 0).all()
+        if case != "bad_ids_frequent":
+            ctx.call("agrad_embedding_backward_sorted", capi.F32, vp(order), vp(d_dY), vp(dW), None, vp(bws), bws_b,
+                     N, 1, C, V, 0)
+            ctx.synchronize()
+            np.testing.assert_array_equal(dW.download(), want_dW)
+        dW.free()
+    for d in (d_ids, d_W, d_dY, out, order, sws, bws):
+        d.free()
