@@ -737,16 +737,27 @@ __device__ __forceinline__ uint32_t run_edge(const uint32_t* __restrict__ tok_s,
     return FORWARD ? at + lo : at + 1 - lo;
 }
 
-constexpr int kFixCols = 64;    // column vectors per slab
-constexpr int kFixLanes = 4;    // partial-sum lanes per column
-constexpr int kFixBatch = 8;    // partial rows a lane keeps in flight
+// A workgroup of the carry fix-up is kFixThreads threads laid out as columns x
+// lanes over one slab of the row: 64 column vectors x 4 partial-sum lanes for the
+// usual run of a few chunks, 16 x 16 for a run of more than kFixLongRun chunks (a
+// frequent token: four times the slabs, so four times the workgroups, and a
+// quarter of the partial rows per lane -- all rows one token, 16384 x 384 fp32:
+// backward 53 -> 25 us).
+constexpr int kFixThreads = 256;
+constexpr int kFixCols = 64;        // column vectors per slab ...
+constexpr int kFixLanes = 4;        // ... and partial-sum lanes per column
+constexpr int kFixColsLong = 16;    // the same for a long run
+constexpr int kFixLanesLong = 16;
+constexpr uint32_t kFixLongRun = 64;
+constexpr int kFixBatch = 8;        // partial rows a lane keeps in flight
+static_assert(kFixCols * kFixLanes == kFixThreads && kFixColsLong * kFixLanesLong == kFixThreads, "carry fix layout");
 
 template <typename T, int VEC>
-__global__ void __launch_bounds__(kFixCols * kFixLanes)
+__global__ void __launch_bounds__(kFixThreads)
 emb_carry_fix_kernel(const uint32_t* __restrict__ tok_s, T* dW, const float* __restrict__ carry_head,
                      const float* __restrict__ carry_tail, uint32_t N, uint32_t C, uint32_t CV,
                      uint32_t V, uint32_t L, int accumulate) {
-    __shared__ float part[kFixLanes][kFixCols * VEC];
+    __shared__ float part[kFixThreads * VEC];
     const uint32_t chunk = blockIdx.x;
     const ChunkEdges e = chunk_edges(tok_s, chunk, L, N);
     const bool origin = e.open_right && !(e.single && e.open_left);
@@ -760,10 +771,10 @@ emb_carry_fix_kernel(const uint32_t* __restrict__ tok_s, T* dW, const float* __r
     // thread and a barrier count per step, so a run of any length is bracketed in
     // two or three memory round trips (a hot token's run spans thousands of
     // positions; bisecting it with dependent loads took longer than the sums).
-    const uint32_t slabs = (CV + kFixCols - 1) / kFixCols;
     if (middle) {
-        // only the first `slabs` middle chunks of a run help; one probe tells the rest
-        const uint64_t far = (uint64_t)(slabs + 1) * L;
+        // only the first `slabs` middle chunks of a run help (slabs of the long-run
+        // layout at most); one probe tells the rest
+        const uint64_t far = (uint64_t)((CV + kFixColsLong - 1) / kFixColsLong + 1) * L;
         if (e.start >= far && tok_s[e.start - far] == tok) return;
     }
     const uint32_t run_end = run_edge<true>(tok_s, tok, e.end, N);        // first position after the run
@@ -796,6 +807,10 @@ emb_carry_fix_kernel(const uint32_t* __restrict__ tok_s, T* dW, const float* __r
         return;
     }
 
+    const bool long_run = count > kFixLongRun;
+    const uint32_t cols = long_run ? kFixColsLong : kFixCols;
+    const uint32_t lanes = long_run ? kFixLanesLong : kFixLanes;
+    const uint32_t slabs = (CV + cols - 1) / cols;
     const uint32_t helpers = count - 1 < slabs ? count - 1 : slabs;   // middle chunks that take a slab
     uint32_t slab_begin, slab_end;
     if (origin) {
@@ -804,28 +819,28 @@ emb_carry_fix_kernel(const uint32_t* __restrict__ tok_s, T* dW, const float* __r
         slab_begin = chunk - c0 - 1; slab_end = slab_begin + 1;
         if (slab_begin >= helpers) return;
     }
-    const uint32_t colv = threadIdx.x % kFixCols;
-    const uint32_t lane = threadIdx.x / kFixCols;
+    const uint32_t colv = threadIdx.x % cols;
+    const uint32_t lane = threadIdx.x / cols;
     for (uint32_t slab = slab_begin; slab < slab_end; ++slab) {
-        const uint32_t cv = slab * kFixCols + colv;
+        const uint32_t cv = slab * cols + colv;
         const bool live = cv < CV;
         const uint32_t col = cv * VEC;
         float acc[VEC];
 #pragma unroll
         for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
         if (live) {
-            for (uint32_t q0 = lane; q0 < count; q0 += kFixLanes * kFixBatch) {
+            for (uint32_t q0 = lane; q0 < count; q0 += lanes * kFixBatch) {
                 float v[kFixBatch][VEC];
 #pragma unroll
                 for (int b = 0; b < kFixBatch; ++b) {
-                    const uint32_t q = q0 + (uint32_t)b * kFixLanes;
+                    const uint32_t q = q0 + (uint32_t)b * lanes;
                     if (q < count) {
                         load_carry<VEC>(heads + (uint64_t)q * C + col, v[b]);
                     }
                 }
 #pragma unroll
                 for (int b = 0; b < kFixBatch; ++b) {
-                    const uint32_t q = q0 + (uint32_t)b * kFixLanes;
+                    const uint32_t q = q0 + (uint32_t)b * lanes;
                     if (q < count) {
 #pragma unroll
                         for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + v[b][k];
@@ -834,15 +849,14 @@ emb_carry_fix_kernel(const uint32_t* __restrict__ tok_s, T* dW, const float* __r
             }
         }
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) part[lane][colv * VEC + k] = acc[k];
+        for (int k = 0; k < VEC; ++k) part[(lane * cols + colv) * VEC + k] = acc[k];
         __syncthreads();
         if (lane == 0 && live) {
             float sum[VEC];
             load_carry<VEC>(tail + col, sum);
+            for (uint32_t q = 0; q < lanes; ++q)
 #pragma unroll
-            for (int q = 0; q < kFixLanes; ++q)
-#pragma unroll
-                for (int k = 0; k < VEC; ++k) sum[k] = sum[k] + part[q][colv * VEC + k];
+                for (int k = 0; k < VEC; ++k) sum[k] = sum[k] + part[(q * cols + colv) * VEC + k];
             store_grad_row<T, VEC>(dW, (uint64_t)tok * C + col, sum, accumulate != 0);
         }
         __syncthreads();
@@ -939,7 +953,7 @@ int embedding_sum_typed(hipStream_t s, const SumPlan& p, const uint32_t* tok_s, 
         if (p.chunks + extra > 0x7fffffffull) return set_error(AGRAD_EINVAL, "embedding backward: position table too large");
         hipLaunchKernelGGL((emb_segment_sum_kernel<T, WIDE>), dim3(p.chunks + (uint32_t)extra), dim3(block), 0, s, tok_s,
                            row_s, dY, dW, head, tail, N, C, CV, V, p.L, acc, p.chunks, dwpe, B, T_len, acc_pos);
-        hipLaunchKernelGGL((emb_carry_fix_kernel<T, WIDE>), dim3(p.chunks), dim3(kFixCols * kFixLanes), 0, s,
+        hipLaunchKernelGGL((emb_carry_fix_kernel<T, WIDE>), dim3(p.chunks), dim3(kFixThreads), 0, s,
                            tok_s, dW, head, tail, N, C, CV, V, p.L, acc);
     } else {
         uint32_t block = ((C + 63) / 64) * 64;
@@ -948,7 +962,7 @@ int embedding_sum_typed(hipStream_t s, const SumPlan& p, const uint32_t* tok_s, 
         if (p.chunks + extra > 0x7fffffffull) return set_error(AGRAD_EINVAL, "embedding backward: position table too large");
         hipLaunchKernelGGL((emb_segment_sum_kernel<T, 1>), dim3(p.chunks + (uint32_t)extra), dim3(block), 0, s, tok_s,
                            row_s, dY, dW, head, tail, N, C, C, V, p.L, acc, p.chunks, dwpe, B, T_len, acc_pos);
-        hipLaunchKernelGGL((emb_carry_fix_kernel<T, 1>), dim3(p.chunks), dim3(kFixCols * kFixLanes), 0, s,
+        hipLaunchKernelGGL((emb_carry_fix_kernel<T, 1>), dim3(p.chunks), dim3(kFixThreads), 0, s,
                            tok_s, dW, head, tail, N, C, C, V, p.L, acc);
     }
     return check_hip(hipGetLastError(), "embedding backward launch");
