@@ -6,7 +6,7 @@
 // Backward dW[ids[n],:] += dY[n,:] (np.add.at, backend.py:531-538) is done
 // without float atomics:
 //   1. (token, row) pairs are ordered so that each token's rows form one run,
-//      in ascending row order.  Up to 16384 rows this is ONE launch: every
+//      in ascending row order.  Up to 65536 rows this is ONE launch: every
 //      workgroup owns a hash group of tokens, scans all ids for its own, and
 //      orders its pairs in LDS (runs of distinct tokens then follow hash-group
 //      order, which is all the later steps need).  Larger inputs take a stable
@@ -192,11 +192,12 @@ emb_prepare_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ keys,
 //    tokens of one group holding most rows): gathered into the group's slice of
 //    `spill` and sorted there -- slow, correct, and rare.
 constexpr int kSortBlock = 512;
-constexpr uint32_t kGroupSortMaxN = 16384;
-constexpr uint32_t kSortLdsEntries = 4096;   // (token, row) pairs a workgroup keeps in LDS
+constexpr uint32_t kGroupSortMaxN = 65536;
+constexpr uint32_t kSortLdsEntries = 3072;   // (token, row) pairs a workgroup keeps in LDS
 constexpr uint32_t kRankSortMax = kSortBlock;  // lists up to one key per thread are placed by rank
 constexpr uint32_t kRowMapWords = kGroupSortMaxN / 32;
-static_assert(kRowMapWords == (uint32_t)kSortBlock, "one word of the row map per thread");
+constexpr uint32_t kSortWaves = kSortBlock / kWave;
+static_assert(kRowMapWords % (2 * kSortWaves) == 0, "the waves share the row map in whole pairs of words");
 
 // Bitonic network in its "flip" form: every comparator puts the smaller key at
 // the lower index, so positions >= n behave as +infinity and need no padding.
@@ -228,14 +229,14 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
     __shared__ unsigned long long keys[kSortLdsEntries];
     __shared__ unsigned long long few[kRankSortMax];
     __shared__ uint32_t row_map[kRowMapWords];
-    __shared__ uint32_t s_count, s_less, s_rest, s_below, s_wave_rows[kSortBlock / kWave];
+    __shared__ uint32_t s_count, s_less, s_rest, s_below, s_wave_rows[kSortWaves];
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & (kWave - 1);
     auto lanes_below = [&](unsigned long long mask) {     // set bits of `mask` below this lane
         return (uint32_t)__builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
     };
     if (tid == 0) { s_count = 0; s_less = 0; s_rest = 0; s_below = 0; }
-    row_map[tid] = 0;
+    for (uint32_t w = tid; w < kRowMapWords; w += kSortBlock) row_map[w] = 0;
     __syncthreads();
 
     auto owner_of = [&](int32_t t, uint32_t& tok) {
@@ -450,29 +451,33 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
         below = s_below;
     }
 
-    // -- the frequent token's rows.  Word w of the map holds rows 32 w ... 32 w + 31;
-    // a wave takes 64 words, two at a time: each half-wave gives one word's 32
+    // -- the frequent token's rows.  Word w of the map holds rows 32 w ... 32 w + 31.
+    // The waves share the words that rows below N can mark, an even number each;
+    // a wave takes its words two at a time: each half-wave gives one word's 32
     // rows a lane each, and a marked row's place is the count of marks before it,
     // so a store instruction writes up to 64 neighbouring entries.
+    const uint32_t wave = tid / kWave;
+    const uint32_t words = (N + 31) / 32;
+    const uint32_t per_wave = ((words + kSortWaves - 1) / kSortWaves + 1) & ~1u;     // at most kRowMapWords / kSortWaves
+    const uint32_t w_begin = wave * per_wave;
     {
-        uint32_t v = (uint32_t)__popc(row_map[tid]);
+        uint32_t v = 0;
+        for (uint32_t j = lane; j < per_wave; j += kWave) v += (uint32_t)__popc(row_map[w_begin + j]);
         v += __builtin_amdgcn_update_dpp(0, v, kDppQuadXor1, 0xf, 0xf, true);
         v += __builtin_amdgcn_update_dpp(0, v, kDppQuadXor2, 0xf, 0xf, true);
         v += __builtin_amdgcn_update_dpp(0, v, kDppRowHalfMirror, 0xf, 0xf, true);
         v += __builtin_amdgcn_update_dpp(0, v, kDppRowMirror, 0xf, 0xf, true);
         v += __builtin_amdgcn_ds_swizzle(v, kSwizzleXor16);
         const uint32_t wave_rows = __builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 32);   // read with every lane active
-        if (lane == 0) s_wave_rows[tid / kWave] = wave_rows;
+        if (lane == 0) s_wave_rows[wave] = wave_rows;
     }
     __syncthreads();
-    const uint32_t wave = tid / kWave;
     uint32_t at = offset + below;
     for (uint32_t w = 0; w < wave; ++w) at += s_wave_rows[w];
     if (s_wave_rows[wave] == 0) return;
     const uint32_t upper = lane >> 5, bit = lane & 31u;
 #pragma nounroll
-    for (uint32_t pair = 0; pair < kWave / 2; ++pair) {
-        const uint32_t w0 = wave * kWave + 2 * pair;
+    for (uint32_t w0 = w_begin; w0 < w_begin + per_wave; w0 += 2) {
         const uint32_t word0 = row_map[w0], word1 = row_map[w0 + 1];
         const uint32_t n0 = (uint32_t)__popc(word0);
         const uint32_t word = upper ? word1 : word0;
@@ -485,13 +490,17 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
     }
 }
 
-// log2 of the number of hash groups (= ordering workgroups).  128 for all but tiny
-// inputs: beside the forward gather they take a quarter of the GPU's thread slots
+// log2 of the number of hash groups (= ordering workgroups).  128 up to 16384
+// rows: beside the forward gather they take a quarter of the GPU's thread slots
 // for a few microseconds (256 took half: forward 13.2 -> 11.8 us at 16384 x 384
 // fp32, 38 -> 36.5 us at 16384 x 1536), and 64 make each group's ranking too long.
+// Above that the groups double with the rows, which keeps a group at a hundred or
+// so pairs; every group still reads all ids (256 KiB at 65536 rows, from L2),
+// about 10 us beside a gather of 100 us or more, where the radix sort's launches
+// took 37 us before the gather could start (65536 x 1024 fp32: 127 -> 106 us).
 // The stand-alone sort uses the same number, so that both ways to the order give
 // the same order and the gradient sums associate identically.
-inline uint32_t group_sort_log2g(uint32_t n) { return n > 1024 ? 7u : 4u; }
+inline uint32_t group_sort_log2g(uint32_t n) { return n > 32768 ? 9u : n > 16384 ? 8u : n > 1024 ? 7u : 4u; }
 
 __global__ void __launch_bounds__(kSortBlock)
 emb_group_sort_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ tok_s,

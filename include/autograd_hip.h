@@ -264,7 +264,7 @@ int agrad_embedding_backward(agrad_ctx* ctx, int dtype, const int32_t* ids, cons
                              void* workspace, uint64_t workspace_bytes,
                              uint64_t N, uint32_t C, uint32_t V, uint32_t flags);
 /* The same pair with the ordering of the ids done in the forward call, where it
- * is free: up to 16384 rows the gather and the ordering are ONE launch (the
+ * is free: up to 65536 rows the gather and the ordering are ONE launch (the
  * ordering workgroups run beside the bandwidth-bound gather), and the backward
  * call starts at the segmented sum.  The forward call also writes order[0..N) =
  * tokens and order[N..2N) = rows (each token's rows adjacent, ascending; 2N

@@ -497,7 +497,9 @@ def _zipf_ids(rng, n, V, s=1.1):
     (1, 3000, 1, 16, "uniform"),          # a single token: one run over every chunk
     (1, 12000, 1, 8, "uniform"),          # one token group larger than the sort's LDS list
     (2, 8000, 5, 24, "uniform"),          # several such groups
-    (4, 8192, 4000, 64, "zipf"),          # N = 32768: the radix-sort path
+    (4, 8192, 4000, 64, "zipf"),          # N = 32768: 256 hash groups
+    (2, 24000, 4000, 64, "zipf"),         # N = 48000: 512 hash groups
+    (3, 23000, 4000, 32, "zipf"),         # N = 69000: the radix-sort path
 ])
 def test_embedding_backward_fp32(ctx, B, T, V, C, dist):
     rng = _rng(20)
@@ -695,7 +697,7 @@ def test_broadcast_add_and_gradient(ctx, lead, inner, dtype):
 
 @pytest.mark.parametrize("B,T,V,C,dist", [(4, 128, 50257, 128, "uniform"), (2, 700, 300, 48, "zipf"),
                                           (32, 512, 32768, 384, "uniform"), (5, 4000, 1000, 64, "zipf"),
-                                          (3, 50, 77, 10, "uniform")])
+                                          (5, 14000, 3000, 32, "zipf"), (3, 50, 77, 10, "uniform")])
 @pytest.mark.parametrize("with_wpe", [False, True])
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_presorted_embedding_pair_matches_the_plain_pair(ctx, B, T, V, C, dist, with_wpe, dtype):
@@ -703,7 +705,7 @@ def test_presorted_embedding_pair_matches_the_plain_pair(ctx, B, T, V, C, dist, 
     agrad_embedding_backward_sorted give the very bits of agrad_gather_forward +
     agrad_embedding_backward (+ agrad_pos_embedding_backward for the position
     table, whose sum rides in the sorted call's launch), call after call, both
-    overwriting and accumulating; (5, 4000) takes the radix path and C = 10 the
+    overwriting and accumulating; (5, 14000) takes the radix path and C = 10 the
     element-wise one."""
     import ctypes as Ct
     rng = _rng(60 + C)
@@ -774,9 +776,11 @@ def test_presorted_embedding_pair_matches_the_plain_pair(ctx, B, T, V, C, dist, 
             d.free()
 
 
-def _same_group_tokens(V, how_many, log2g=7):
+def _same_group_tokens(V, how_many, N):
     """tokens below V that the grouping sort hands to one workgroup (its hash:
-    the top log2g bits of token * 0x9E3779B1 mod 2^32)"""
+    the top log2g bits of token * 0x9E3779B1 mod 2^32; 128, 256 or 512 groups
+    by the number of rows)"""
+    log2g = 9 if N > 32768 else 8 if N > 16384 else 7
     toks = np.arange(V, dtype=np.uint64)
     group = ((toks * np.uint64(0x9E3779B1)) & np.uint64(0xFFFFFFFF)) >> np.uint64(32 - log2g)
     best = np.bincount(group.astype(np.int64)).argmax()
@@ -795,6 +799,10 @@ _SKEWED = {
     "listed_frequent_plus_few": (8192, [(1500, 1), (2, 100)]),   # list fits LDS, the rest placed by rank
     "listed_no_frequent": (8192, [(400, 3)]),                 # list fits LDS, no single frequent token
     "short_input": (1500, [(1400, 1)]),                       # fewer rows than the row map has bits
+    "most_rows_one_token_64k": (65536, [(60000, 1)]),         # 512 groups, every word of the row map
+    "padding_40k": (40001, [(15000, 1), (3, 40)]),            # 512 groups, a ragged last word
+    "padding_20k": (20001, [(7000, 1), (3, 80)]),             # 256 groups
+    "two_frequent_one_group_64k": (65536, [(9000, 1), (1500, 1), (2, 50)]),
     "bad_ids_frequent": (4096, [(0, 1)]),                     # out-of-range ids (one sentinel token) dominate
 }
 
@@ -814,7 +822,7 @@ def test_id_ordering_with_frequent_tokens(ctx, case):
     if case == "bad_ids_frequent":
         ids[rng.permutation(N)[:3000]] = -5
     else:
-        same = _same_group_tokens(V, sum(k for _, k in spec))
+        same = _same_group_tokens(V, sum(k for _, k in spec), N)
         slots = rng.permutation(N)
         at = t = 0
         for rows, k in spec:
