@@ -29,7 +29,7 @@ from math import prod
 
 import numpy as np
 
-from .op import (AddLayerNormOp, AddOp, AddRMSNormOp, ContiguousOp, CrossEntropyLossOp, EmbeddingSumOp, ExpOp,
+from .op import (AddLayerNormOp, AddOp, AddRMSNormOp, BiasGELUOp, ContiguousOp, CrossEntropyLossOp, EmbeddingSumOp, ExpOp,
                  GatherOp, GELUOp, LayerNormOp, LogOp, MulOp, PermuteOp, ReLUSquaredOp, ReshapeOp, RMSNormOp, RopeOp,
                  RsqrtOp, SoftmaxOp, SwiGLUOp, TransposeOp, ViewOp)
 from .scratch import single_slot
@@ -146,6 +146,7 @@ class HipBackend(Backend):
             GatherOp: self.hip_gather_forward,
             EmbeddingSumOp: self.hip_embedding_sum_forward,
             GELUOp: self.hip_gelu_forward,
+            BiasGELUOp: self.hip_bias_gelu_forward,
             ReLUSquaredOp: self.hip_relu2_forward,
             SwiGLUOp: self.hip_swiglu_forward,
             LayerNormOp: self.hip_layernorm_forward,
@@ -170,6 +171,7 @@ class HipBackend(Backend):
             GatherOp: self.hip_gather_backward,
             EmbeddingSumOp: self.hip_embedding_sum_backward,
             GELUOp: self.hip_gelu_backward,
+            BiasGELUOp: self.hip_bias_gelu_backward,
             ReLUSquaredOp: self.hip_relu2_backward,
             SwiGLUOp: self.hip_swiglu_backward,
             LayerNormOp: self.hip_layernorm_backward,
@@ -242,6 +244,12 @@ class HipBackend(Backend):
                     need = max(need, self.ctx.broadcast_grad_workspace_bytes(out.numel // t.numel, t.numel))
             if need:
                 return None, single_slot("workspace", need)
+        if isinstance(op, BiasGELUOp):
+            h, b = node.inputs
+            if b.requires_grad:
+                need = self.ctx.gelu_bias_backward_workspace_bytes(prod(h.shape[:-1]), h.shape[-1])
+                if need:
+                    return None, single_slot("workspace", need)
         if isinstance(op, MulOp):
             x, y = node.inputs
             if y.requires_grad:
@@ -510,6 +518,34 @@ class HipBackend(Backend):
 
     def hip_gelu_backward(self, inputs, outputs, scratch=None):
         self._unary_backward("gelu_backward_kernel", inputs, outputs)
+
+    # -- GELU(h + b) (gelu_add_bias_kernel / gelu_backward_bias_kernel, metal_ops.metal:3737-3773)
+    def hip_bias_gelu_forward(self, inputs, outputs, scratch=None):
+        h, b, out = inputs[0], inputs[1], outputs[0]
+        self._launch("gelu_add_bias_kernel", [h, b, out], [_dt(h)] + _lo_hi(prod(h.shape[:-1])) + [h.shape[-1]])
+
+    def hip_bias_gelu_backward(self, inputs, outputs, scratch=None):
+        h, b, out = inputs[0], inputs[1], outputs[0]
+        if out.grad is None:
+            return
+        node = out.op
+        dh = h.grad if h.requires_grad else None
+        db = b.grad if b.requires_grad else None
+        if dh is None and db is None:
+            return
+        flags, ws, ws_bytes = 0, None, 0
+        if dh is not None:
+            flags |= self._grad_flag(node, h)
+        if db is not None:
+            if scratch is None:
+                raise RuntimeError("BiasGELU backward needs its arena workspace (plan_scratch)")
+            ws = scratch["workspace"]
+            ws_bytes = ws.nbytes
+            if self._grad_flag(node, b):
+                flags |= ACC_PARAM_GRAD
+        self._launch("gelu_backward_bias_kernel", [out.grad, h, b, dh, db, ws],
+                     [_dt(h)] + _lo_hi(prod(h.shape[:-1])) + [h.shape[-1], flags] + _lo_hi(ws_bytes)
+                     + [_mask(out.grad, h, b, dh, db, ws)])
 
     def hip_relu2_forward(self, inputs, outputs, scratch=None):
         self._unary_forward("relu2_forward_kernel", inputs, outputs)

@@ -63,6 +63,9 @@ SIGNATURES = {
                                    _ptr, _u64, _u64, _u32, _f32, _u32]),
     "agrad_gelu_forward": (_int, [_ctx, _int, _ptr, _ptr, _u64]),
     "agrad_gelu_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _u64, _u32]),
+    "agrad_gelu_bias_forward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _u64, _u32]),
+    "agrad_gelu_bias_backward_workspace_bytes": (_u64, [_u64, _u32]),
+    "agrad_gelu_bias_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _u64, _u64, _u32, _u32]),
     "agrad_relu2_forward": (_int, [_ctx, _int, _ptr, _ptr, _u64]),
     "agrad_relu2_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _u64, _u32]),
     "agrad_swiglu_forward": (_int, [_ctx, _int, _ptr, _ptr, _u64, _u32]),

@@ -7,56 +7,19 @@
 // SwiGLU backend.py:1113-1126 and 1206-1217.  ReLU^2 has no counterpart in the
 // reference: y = max(x, 0)^2, dx = (2 max(x, 0)) dy.
 #include "elementwise.hpp"
+#include "gelu_math.hpp"
 
 namespace agrad {
 
 namespace {
 
-constexpr float kGeluC = 0.7978845608028654f;
-constexpr float kGeluA = 0.044715f;
-constexpr float kGeluA3 = 0.134145f;
-
-__device__ __forceinline__ float gelu_tanh_arg(float x) {
-    float b = x * x;
-    b = b * x;
-    b = b * kGeluA;
-    b = x + b;
-    b = b * kGeluC;
-    return tanhf(b);
-}
-
 struct GeluFwd {
-    static __device__ __forceinline__ float apply(const float (&in)[1]) {
-        const float x = in[0];
-        float b = gelu_tanh_arg(x);
-        b = b + 1.0f;
-        b = x * b;
-        return b * 0.5f;
-    }
+    static __device__ __forceinline__ float apply(const float (&in)[1]) { return gelu_value(in[0]); }
 };
 
-// in[0] = x, in[1] = dy.  d/dx = (1 + t)/2 + (1 - t^2) * (x/2) * C (1 + A3 x^2),
-// t = tanh(z).  The reference forms 1 - t*t and (t + 1) from the rounded t
-// (backend.py:398-411), which loses every significant bit once |t| is within a
-// few ulp of 1; here both factors come from w = exp(-2|z|) with no
-// cancellation, so the device value is the accurate one and differs from the
-// CPU value by the CPU's own rounding noise only.
+// in[0] = x, in[1] = dy
 struct GeluBwd {
-    static __device__ __forceinline__ float apply(const float (&in)[2]) {
-        const float x = in[0];
-        float z = x * x;
-        z = z * x;
-        z = z * kGeluA;
-        z = x + z;
-        z = z * kGeluC;
-        const float w = expf(-2.0f * fabsf(z));
-        const float inv = 1.0f / (1.0f + w);
-        const float half_one_plus_t = z >= 0.0f ? inv : w * inv;   // (1 + tanh z) / 2
-        const float sech2 = (4.0f * w) * (inv * inv);              // 1 - tanh^2 z
-        const float d_inner = kGeluC * (1.0f + (kGeluA3 * x) * x);
-        const float a = sech2 * ((0.5f * x) * d_inner);
-        return in[1] * (half_one_plus_t + a);
-    }
+    static __device__ __forceinline__ float apply(const float (&in)[2]) { return in[1] * gelu_slope(in[0]); }
 };
 
 struct Relu2Fwd {

@@ -276,4 +276,25 @@ __device__ __forceinline__ void row_sum3(float& a, float& b, float& c, float* ld
     }
 }
 
+// Division of a 32-bit index by a divisor fixed at launch: one multiply-high and
+// two shifts on the device (Granlund & Montgomery's round-up form) in place of
+// the twenty-odd instructions of a hardware-less integer divide.  Exact for
+// every n < 2^32 and 1 <= d < 2^32.
+struct FastDiv32 {
+    uint32_t d, mul, shift1, shift2;
+    FastDiv32() : d(1), mul(1), shift1(0), shift2(0) {}
+    explicit FastDiv32(uint32_t divisor) : d(divisor) {
+        uint32_t l = 0;
+        while (l < 32 && (1ull << l) < (uint64_t)divisor) ++l;          // ceil(log2 d)
+        mul = (uint32_t)((((1ull << l) - divisor) << 32) / divisor + 1);
+        shift1 = l < 1 ? l : 1;
+        shift2 = l > 1 ? l - 1 : 0;
+    }
+    __device__ __forceinline__ uint32_t div(uint32_t n) const {
+        const uint32_t t = __umulhi(mul, n);
+        return (t + ((n - t) >> shift1)) >> shift2;
+    }
+    __device__ __forceinline__ uint32_t mod(uint32_t n) const { return n - div(n) * d; }
+};
+
 }  // namespace agrad

@@ -309,6 +309,23 @@ int h_act_bwd(const Call& c) {
     return WHICH == 0 ? launch_gelu_bwd(c.ctx->stream, c.a[0], x, dy, dx, n, c.a[1])
                       : launch_relu2_bwd(c.ctx->stream, c.a[0], x, dy, dx, n, c.a[1]);
 }
+// buffers h, b, out (the reference's order, metal_ops.metal:3737-3744) | args dtype, rows lo, hi, C
+int h_gelu_bias_fwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t rows = u64(c.a, 1), es = dtype_size(c.a[0]);
+    RESOLVE(0, rows * c.a[3] * es, h) RESOLVE(1, (uint64_t)c.a[3] * es, b) RESOLVE(2, rows * c.a[3] * es, out)
+    return launch_gelu_bias_fwd(c.ctx->stream, (int)c.a[0], h, b, out, rows, c.a[3]);
+}
+// buffers dy, h, b, dh (the reference's order, metal_ops.metal:3753-3760), db, workspace
+// args dtype, rows lo, hi, C, flags, ws lo, hi, present_mask
+int h_gelu_bias_bwd(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t rows = u64(c.a, 1), es = dtype_size(c.a[0]), wsb = u64(c.a, 5);
+    const uint64_t big = rows * c.a[3] * es, small = (uint64_t)c.a[3] * es;
+    RESOLVE(0, big, dy) RESOLVE(1, big, h) RESOLVE(2, small, b) RESOLVE_IF(c.a[7] & 8u, 3, big, dh)
+    RESOLVE_IF(c.a[7] & 16u, 4, small, db) RESOLVE_IF(c.a[7] & 32u, 5, wsb, ws)
+    return launch_gelu_bias_bwd(c.ctx->stream, (int)c.a[0], dy, h, b, dh, db, ws, ws ? wsb : 0, rows, c.a[3], c.a[4]);
+}
 // buffers gu, h | args dtype, rows, H
 int h_swiglu_fwd(const Call& c) {
     NEED_DTYPE(c.a[0])
@@ -454,6 +471,8 @@ const Entry kTable[] = {
     {"rmsnorm_backward", 9, 8, "x, dy, gamma, dres, dx, dx2, dgamma, dbeta, workspace | dtype, rows, C, eps_bits, flags, present_mask, ws_lo, ws_hi", h_norm_bwd<AGRAD_NORM_RMS>},
     {"gelu_forward_kernel", 2, 3, "x, y | dtype, n_lo, n_hi", h_act_fwd<0>},
     {"gelu_backward_kernel", 3, 4, "dy, x, dx | dtype, flags, n_lo, n_hi", h_act_bwd<0>},
+    {"gelu_add_bias_kernel", 3, 4, "h, b, out | dtype, rows_lo, rows_hi, C", h_gelu_bias_fwd},
+    {"gelu_backward_bias_kernel", 6, 8, "dy, h, b, dh, db, workspace | dtype, rows_lo, rows_hi, C, flags, ws_lo, ws_hi, present_mask", h_gelu_bias_bwd},
     {"relu2_forward_kernel", 2, 3, "x, y | dtype, n_lo, n_hi", h_act_fwd<1>},
     {"relu2_backward_kernel", 3, 4, "dy, x, dx | dtype, flags, n_lo, n_hi", h_act_bwd<1>},
     {"swiglu_forward_kernel", 2, 3, "gu, h | dtype, rows, H", h_swiglu_fwd},
@@ -807,6 +826,18 @@ int agrad_norm_backward(agrad_ctx* ctx, int kind, int dtype, const void* x, cons
 int agrad_gelu_forward(agrad_ctx* ctx, int dtype, const void* x, void* y, uint64_t n) {
     CTX_OR_FAIL(ctx)
     return launch_gelu_fwd(ctx->stream, dtype, x, y, n);
+}
+int agrad_gelu_bias_forward(agrad_ctx* ctx, int dtype, const void* h, const void* b, void* y, uint64_t rows, uint32_t C) {
+    CTX_OR_FAIL(ctx)
+    return launch_gelu_bias_fwd(ctx->stream, dtype, h, b, y, rows, C);
+}
+uint64_t agrad_gelu_bias_backward_workspace_bytes(uint64_t rows, uint32_t C) {
+    return gelu_bias_backward_workspace_bytes(rows, C);
+}
+int agrad_gelu_bias_backward(agrad_ctx* ctx, int dtype, const void* dy, const void* h, const void* b, void* dh, void* db,
+                             void* workspace, uint64_t workspace_bytes, uint64_t rows, uint32_t C, uint32_t flags) {
+    CTX_OR_FAIL(ctx)
+    return launch_gelu_bias_bwd(ctx->stream, dtype, dy, h, b, dh, db, workspace, workspace_bytes, rows, C, flags);
 }
 int agrad_gelu_backward(agrad_ctx* ctx, int dtype, const void* x, const void* dy, void* dx, uint64_t n, uint32_t flags) {
     CTX_OR_FAIL(ctx)

@@ -155,6 +155,9 @@ public:
     uint64_t broadcast_grad_workspace_bytes(uint64_t lead, uint64_t inner) {
         return agrad_broadcast_grad_workspace_bytes(lead, inner);
     }
+    uint64_t gelu_bias_backward_workspace_bytes(uint64_t rows, uint32_t C) {
+        return agrad_gelu_bias_backward_workspace_bytes(rows, C);
+    }
     uint64_t mul_backward_workspace_bytes(int kind, uint64_t lead, uint64_t inner) {
         return agrad_mul_backward_workspace_bytes(kind, lead, inner);
     }
@@ -218,6 +221,7 @@ PYBIND11_MODULE(hip_ext, m) {
         .def("embedding_backward_workspace_bytes", &HipContext::embedding_backward_workspace_bytes)
         .def("broadcast_grad_workspace_bytes", &HipContext::broadcast_grad_workspace_bytes)
         .def("mul_backward_workspace_bytes", &HipContext::mul_backward_workspace_bytes)
+        .def("gelu_bias_backward_workspace_bytes", &HipContext::gelu_bias_backward_workspace_bytes)
         .def("embedding_sort_workspace_bytes", &HipContext::embedding_sort_workspace_bytes)
         .def("embedding_backward_sorted_workspace_bytes", &HipContext::embedding_backward_sorted_workspace_bytes)
         .def("kernel_names", &HipContext::kernel_names)

@@ -42,11 +42,16 @@ int launch_norm_bwd(hipStream_t s, int kind, int dtype, const void* x, const voi
                     uint64_t rows, uint32_t C, float eps, uint32_t flags);
 
 // out_a[c] (+)= sum over the P rows of pa[P, C] (same for pb -> out_b; either pair may be null)
+// out_bf16: out_a / out_b point at bf16 elements (the sum is rounded once, after the optional accumulate)
 int launch_colsum_finalize(hipStream_t s, const float* pa, const float* pb, uint32_t P, uint32_t C,
-                           float* out_a, float* out_b, int accumulate);
+                           float* out_a, float* out_b, int accumulate, bool out_bf16 = false);
 
 // reduce.hip
 int launch_broadcast_add(hipStream_t s, int dtype, const void* x, const void* y, void* out, uint64_t lead, uint64_t inner);
+int launch_gelu_bias_fwd(hipStream_t s, int dtype, const void* h, const void* b, void* y, uint64_t rows, uint32_t C);
+uint64_t gelu_bias_backward_workspace_bytes(uint64_t rows, uint32_t C);
+int launch_gelu_bias_bwd(hipStream_t s, int dtype, const void* dy, const void* h, const void* b, void* dh, void* db,
+                         void* workspace, uint64_t workspace_bytes, uint64_t rows, uint32_t C, uint32_t flags);
 uint64_t broadcast_grad_workspace_bytes(uint64_t lead, uint64_t inner);
 int launch_broadcast_grad(hipStream_t s, int dtype, const void* g, void* dy, void* workspace, uint64_t workspace_bytes,
                           uint64_t lead, uint64_t inner, uint32_t flags);

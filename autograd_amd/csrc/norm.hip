@@ -71,7 +71,7 @@ struct NormBwdArgs {
 template <int W>   // W = 4: float4 columns, W = 1: scalar columns
 __global__ void __launch_bounds__(1024)
 colsum_finalize_kernel(const float* __restrict__ pg, const float* __restrict__ pb, uint32_t P, uint32_t C,
-                       float* __restrict__ dgamma, float* __restrict__ dbeta, int accumulate) {
+                       float* __restrict__ dgamma, float* __restrict__ dbeta, int accumulate, int out_bf16) {
     constexpr int COLS = 8, LANES = 128, BATCH = 8;
     __shared__ float tile[LANES][COLS * W];
     __shared__ float tile2[LANES / 16][COLS * W];
@@ -128,7 +128,14 @@ colsum_finalize_kernel(const float* __restrict__ pg, const float* __restrict__ p
             float t = tile2[0][cl * W + k];
 #pragma unroll
             for (int j = 1; j < LANES / 16; ++j) t = t + tile2[j][cl * W + k];
-            dst[c + k] = accumulate ? (dst[c + k] + t) : t;
+            if (out_bf16) {
+                // a bf16 destination: the sum is finished in fp32 and rounded once
+                bf16_t* d16 = reinterpret_cast<bf16_t*>(dst);
+                if (accumulate) t = bf16_bits_to_f32(d16[c + k]) + t;
+                d16[c + k] = (bf16_t)f32_to_bf16_bits(t);
+            } else {
+                dst[c + k] = accumulate ? (dst[c + k] + t) : t;
+            }
         }
     }
 }
@@ -859,15 +866,15 @@ int norm_bwd_typed(hipStream_t s, const NormPlan& p, const NormBwdArgs<T>& a, ui
 }  // namespace
 
 int launch_colsum_finalize(hipStream_t s, const float* pa, const float* pb, uint32_t P, uint32_t C,
-                           float* out_a, float* out_b, int accumulate) {
+                           float* out_a, float* out_b, int accumulate, bool out_bf16) {
     const bool vec4 = C % 4 == 0 && (!out_a || aligned16(out_a)) && (!out_b || aligned16(out_b)) &&
                       (!pa || aligned16(pa)) && (!pb || aligned16(pb));
     if (vec4)
         hipLaunchKernelGGL((colsum_finalize_kernel<4>), dim3((C / 4 + 7) / 8, 2), dim3(1024), 0, s, pa, pb, P, C,
-                           out_a, out_b, accumulate);
+                           out_a, out_b, accumulate, out_bf16 ? 1 : 0);
     else
         hipLaunchKernelGGL((colsum_finalize_kernel<1>), dim3((C + 7) / 8, 2), dim3(1024), 0, s, pa, pb, P, C,
-                           out_a, out_b, accumulate);
+                           out_a, out_b, accumulate, out_bf16 ? 1 : 0);
     return check_hip(hipGetLastError(), "column-sum finalize launch");
 }
 

@@ -9,9 +9,9 @@
 // The gradient is a column sum.  With few leading rows (a [T, C] table under a
 // batch of 16) a thread owns a column vector and adds the rows in order.  With
 // many (a [C] bias under 16384 rows) that would be C/4 threads walking the whole
-// tensor, so persistent workgroups each add a strided share of the rows into one
-// partial row (read-only stream, several rows in flight per lane), and the
-// column-sum finalize kernel of the norm backward folds the partial rows.
+// tensor, so workgroups each add a tile of rows into one partial row (several
+// rows in flight per lane), and the column-sum finalize kernel of the norm
+// backward folds the partial rows.
 // Every sum has a fixed order.
 //
 // Broadcast Mul (cpu_mul_forward / cpu_mul_backward, backend.py:107-146) has the
@@ -19,7 +19,10 @@
 // ("col": one factor per row) or y[0] ("scalar").  dx (+)= g * y[..] is the forward
 // kernel again; dy is a column sum, a row sum or a full sum of the product g * x,
 // each in a fixed order.
+#include <cstdlib>
+
 #include "common.hpp"
+#include "gelu_math.hpp"
 #include "launch.hpp"
 
 namespace agrad {
@@ -27,20 +30,14 @@ namespace agrad {
 namespace {
 
 constexpr int kBcastBlock = 64;
-constexpr int kColBlock = 256;
 constexpr int kColRows = 4;             // rows a lane keeps in flight
 constexpr uint32_t kColMaxBlocks = 1024;
 constexpr uint64_t kColDirectLead = 64; // up to this many leading rows a thread adds them itself
 
+// vector j (VEC elements) of a small operand that every leading row re-reads: one
+// ordinary (cached) load; the operand is 16-byte aligned when VEC > 1
 template <typename T, int VEC>
-__global__ void __launch_bounds__(kBcastBlock)
-bcast_add_kernel(const T* __restrict__ x, const T* __restrict__ y, T* __restrict__ out, uint64_t nvec, uint32_t inner_vec) {
-    const uint64_t idx = (uint64_t)blockIdx.x * kBcastBlock + threadIdx.x;
-    if (idx >= nvec) return;
-    float a[VEC], b[VEC];
-    VecIO<T, VEC>::load(x + idx * VEC, a);
-    const uint32_t j = (uint32_t)(idx % inner_vec);
-    // the small operand is re-read by every leading row: ordinary (cached) loads
+__device__ __forceinline__ void small_vec(const T* __restrict__ y, uint32_t j, float (&b)[VEC]) {
     if constexpr (VEC == 1) {
         b[0] = sizeof(T) == 2 ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(y)[j]) : reinterpret_cast<const float*>(y)[j];
     } else if constexpr (sizeof(T) == 4) {
@@ -55,6 +52,16 @@ bcast_add_kernel(const T* __restrict__ x, const T* __restrict__ y, T* __restrict
             b[2 * k + 1] = __builtin_bit_cast(float, w[k] & 0xffff0000u);
         }
     }
+}
+
+template <typename T, int VEC>
+__global__ void __launch_bounds__(kBcastBlock)
+bcast_add_kernel(const T* __restrict__ x, const T* __restrict__ y, T* __restrict__ out, uint64_t nvec, uint32_t inner_vec) {
+    const uint64_t idx = (uint64_t)blockIdx.x * kBcastBlock + threadIdx.x;
+    if (idx >= nvec) return;
+    float a[VEC], b[VEC];
+    VecIO<T, VEC>::load(x + idx * VEC, a);
+    small_vec<T, VEC>(y, (uint32_t)(idx % inner_vec), b);
 #pragma unroll
     for (int k = 0; k < VEC; ++k) a[k] = a[k] + b[k];
     VecIO<T, VEC>::store(out + idx * VEC, a);
@@ -66,34 +73,48 @@ template <typename T> __device__ __forceinline__ float small_elem(const T* y, ui
     else return reinterpret_cast<const float*>(y)[i];
 }
 
-// partial[p, :] = sum over rows p, p + P, p + 2P, ... of g[row, :] (* x2[row, :]), for P partial
-// rows.  `lanes` threads share a row (a multiple of 64 that covers the row's vectors, at most
-// the workgroup), so a workgroup of 256 takes 256 / lanes partial rows: narrow tensors
-// (C = 384: 96 vectors) keep three quarters of their lanes busy instead of three eighths.
+// partial[t % P, :] = sum over the rows of tile t of g[row, :] (* x2[row, :]).  A workgroup of
+// 256 threads is `lanes` column vectors (32 or 64) wide and 256 / lanes row groups deep; every
+// thread has kTileRows rows in flight, so a workgroup covers a tile of (256 / lanes) * kTileRows
+// rows, adds its threads' sums through LDS and writes ONE partial row.  With more tiles than
+// partial rows a workgroup walks tiles t, t + P, ...  Many short workgroups keep the loads,
+// arithmetic and stores of different tiles overlapped (a persistent grid of P workgroups with
+// strided rows ran its load / compute / store phases in step: 20.1 against 17.5 us at
+// 16384 x 384 fp32, 46 against 34 us at 16384 x 1536 bf16).
 // With dx given the kernel also writes dx[row, :] (+)= g[row, :] * y[:] -- the other gradient
 // of x * y[:], from the g it has in registers anyway.
-template <typename T, int VEC>
-__global__ void __launch_bounds__(kColBlock)
-colsum_partial_kernel(const T* __restrict__ g, const T* __restrict__ x2, const T* __restrict__ ysmall, T* dx,
-                      float* __restrict__ partial, uint64_t lead, uint32_t inner, uint32_t inner_vec, uint32_t lanes,
-                      uint32_t P, int acc_dx) {
+// STAGE kStageGeluBias is the backward of GELU(x2 + y[:]): the summed term is
+// g * GELU'(x2 + y), and dx (+)= the same term.
+constexpr int kStageSum = 0, kStageGeluBias = 1;
+constexpr int kTileBlock = 256;
+constexpr uint32_t kTileMaxPartials = 512;
+
+template <typename T, int VEC, int STAGE, int kTileRows>
+__global__ void __launch_bounds__(kTileBlock)
+colsum_tile_kernel(const T* __restrict__ g, const T* __restrict__ x2, const T* __restrict__ ysmall, T* dx,
+                   float* __restrict__ partial, uint64_t lead, uint32_t inner, uint32_t inner_vec, uint32_t lanes,
+                   uint32_t tiles, int acc_dx) {
+    __shared__ float part[kTileBlock * VEC];
     const uint32_t sub = threadIdx.x / lanes, lane = threadIdx.x - sub * lanes;
-    const uint32_t p = blockIdx.x * (blockDim.x / lanes) + sub;
-    if (p >= P) return;
-    for (uint32_t cv = lane; cv < inner_vec; cv += lanes) {
-        const uint32_t col = cv * VEC;
-        float acc[VEC], yv[VEC];
+    const uint32_t subs = kTileBlock / lanes;
+    const uint32_t tile_rows = subs * kTileRows;
+    const uint32_t cv = blockIdx.x * lanes + lane;
+    const bool live = cv < inner_vec;
+    const uint32_t col = cv * VEC;
+    float acc[VEC], yv[VEC];
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
-        if (dx != nullptr) {
+    for (int k = 0; k < VEC; ++k) { acc[k] = 0.0f; yv[k] = 0.0f; }
+    if (live && (STAGE == kStageGeluBias || dx != nullptr)) {
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) yv[k] = small_elem<T>(ysmall, col + k);
-        }
-        for (uint64_t r0 = p; r0 < lead; r0 += (uint64_t)P * kColRows) {
-            float v[kColRows][VEC], w[kColRows][VEC], o[kColRows][VEC];
+        for (int k = 0; k < VEC; ++k) yv[k] = small_elem<T>(ysmall, col + k);
+    }
+    if (live) {
+        for (uint32_t tile = blockIdx.y; tile < tiles; tile += gridDim.y) {
+            const uint64_t r0 = (uint64_t)tile * tile_rows + sub;      // rows r0, r0 + subs, ...
+            float v[kTileRows][VEC], w[kTileRows][VEC], o[kTileRows][VEC];
 #pragma unroll
-            for (int u = 0; u < kColRows; ++u) {
-                const uint64_t r = r0 + (uint64_t)u * P;
+            for (int u = 0; u < kTileRows; ++u) {
+                const uint64_t r = r0 + (uint64_t)u * subs;
                 if (r < lead) {
                     VecIO<T, VEC>::load(g + r * inner + col, v[u]);
                     if (x2 != nullptr) VecIO<T, VEC>::load(x2 + r * inner + col, w[u]);   // uniform branches
@@ -101,24 +122,45 @@ colsum_partial_kernel(const T* __restrict__ g, const T* __restrict__ x2, const T
                 }
             }
 #pragma unroll
-            for (int u = 0; u < kColRows; ++u) {
-                const uint64_t r = r0 + (uint64_t)u * P;
+            for (int u = 0; u < kTileRows; ++u) {
+                const uint64_t r = r0 + (uint64_t)u * subs;
                 if (r < lead) {
-#pragma unroll
-                    for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + (x2 != nullptr ? v[u][k] * w[u][k] : v[u][k]);
-                    if (dx != nullptr) {
+                    if constexpr (STAGE == kStageGeluBias) {
 #pragma unroll
                         for (int k = 0; k < VEC; ++k) {
-                            const float t = v[u][k] * yv[k];
+                            const float t = v[u][k] * gelu_slope(w[u][k] + yv[k]);
+                            acc[k] = acc[k] + t;
                             o[u][k] = acc_dx ? (o[u][k] + t) : t;
                         }
-                        VecIO<T, VEC>::store(dx + r * inner + col, o[u]);
+                        if (dx != nullptr) VecIO<T, VEC>::store(dx + r * inner + col, o[u]);
+                    } else {
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + (x2 != nullptr ? v[u][k] * w[u][k] : v[u][k]);
+                        if (dx != nullptr) {
+#pragma unroll
+                            for (int k = 0; k < VEC; ++k) {
+                                const float t = v[u][k] * yv[k];
+                                o[u][k] = acc_dx ? (o[u][k] + t) : t;
+                            }
+                            VecIO<T, VEC>::store(dx + r * inner + col, o[u]);
+                        }
                     }
                 }
             }
         }
+    }
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) partial[(uint64_t)p * inner + col + k] = acc[k];
+    for (int k = 0; k < VEC; ++k) part[(sub * lanes + lane) * VEC + k] = acc[k];
+    __syncthreads();
+    if (sub == 0 && live) {
+        float sum[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) sum[k] = acc[k];
+        for (uint32_t q = 1; q < subs; ++q)
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) sum[k] = sum[k] + part[(q * lanes + lane) * VEC + k];
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) partial[(uint64_t)blockIdx.y * inner + col + k] = sum[k];
     }
 }
 
@@ -305,27 +347,38 @@ namespace {
 
 // dy[j] (+)= sum_l g[l, j] (* x2[l, j]) in two stages through `workspace`; bf16 sums are
 // finished in fp32 and rounded once
-template <typename T>
+template <typename T, int STAGE = kStageSum>
 int colsum_two_stage(hipStream_t s, const T* g, const T* x2, T* dy, void* workspace, uint64_t lead, uint64_t inner,
                      int accumulate, const T* ysmall = nullptr, T* dx = nullptr, int acc_dx = 0) {
     constexpr int WIDE = WideVec<T>::value;
-    const uint32_t blocks = colsum_blocks(lead);     // partial rows
     float* partial = (float*)workspace;
     const bool wide = inner % WIDE == 0 && aligned16(g) && (!x2 || aligned16(x2)) && (!dx || aligned16(dx));
     const uint32_t iv = (uint32_t)(wide ? inner / WIDE : inner);
-    uint32_t lanes = (iv + kWave - 1) / kWave * kWave;
-    if (lanes > (uint32_t)kColBlock) lanes = kColBlock;
-    const uint32_t per_wg = kColBlock / lanes;       // partial rows per workgroup
-    const dim3 grid((blocks + per_wg - 1) / per_wg), block(lanes * per_wg);
-    if (wide) hipLaunchKernelGGL((colsum_partial_kernel<T, WIDE>), grid, block, 0, s, g, x2, ysmall, dx, partial, lead, (uint32_t)inner, iv, lanes, blocks, acc_dx);
-    else hipLaunchKernelGGL((colsum_partial_kernel<T, 1>), grid, block, 0, s, g, x2, ysmall, dx, partial, lead, (uint32_t)inner, iv, lanes, blocks, acc_dx);
+    uint32_t blocks;                                 // partial rows
+    // 32 lanes when that leaves fewer of them idle in the last column group (96 vectors:
+    // three full groups of 32, not one and a half of 64)
+    const uint32_t lanes = (iv + 31) / 32 * 32 < (iv + 63) / 64 * 64 ? 32 : 64;
+    // Four rows in flight per thread when one tile per workgroup then covers the tensor
+    // within kTileMaxPartials partial rows; else two (fewer registers, more waves
+    // resident) and a walk over several tiles.  Measured on 16384 rows, fp32 x 384 /
+    // x 768 / bf16 x 1536: 17.5 / 30.4 / 34.0 us this way, 19.1 / 30.4 / 34.0 with two
+    // everywhere, 17.4 / 33.1 / 36.6 with four and 1024 partial rows.
+    const uint32_t subs = kTileBlock / lanes;
+    const uint32_t cap = colsum_blocks(lead) < kTileMaxPartials ? colsum_blocks(lead) : kTileMaxPartials;
+    const int R = (lead + subs * 4 - 1) / (subs * 4) <= cap ? 4 : 2;
+    const uint32_t tile_rows = subs * R;
+    const uint64_t tiles = (lead + tile_rows - 1) / tile_rows;
+    blocks = (uint32_t)(tiles < cap ? tiles : cap);
+    const dim3 grid((iv + lanes - 1) / lanes, blocks), block(kTileBlock);
+#define AGRAD_TILE_LAUNCH(V, RR) hipLaunchKernelGGL((colsum_tile_kernel<T, V, STAGE, RR>), grid, block, 0, s, g, x2, ysmall, dx, partial, lead, (uint32_t)inner, iv, lanes, (uint32_t)tiles, acc_dx)
+    if (wide) { if (R == 4) AGRAD_TILE_LAUNCH(WIDE, 4); else AGRAD_TILE_LAUNCH(WIDE, 2); }
+    else { if (R == 4) AGRAD_TILE_LAUNCH(1, 4); else AGRAD_TILE_LAUNCH(1, 2); }
+#undef AGRAD_TILE_LAUNCH
     if (int rc = check_hip(hipGetLastError(), "column sum launch")) return rc;
     if constexpr (sizeof(T) == 4) {
         return launch_colsum_finalize(s, partial, nullptr, blocks, (uint32_t)inner, (float*)dy, nullptr, accumulate);
     } else {
-        float* row = partial + (uint64_t)blocks * inner;
-        if (int rc = launch_colsum_finalize(s, partial, nullptr, blocks, (uint32_t)inner, row, nullptr, 0)) return rc;
-        return launch_cast_f32_bf16(s, row, dy, inner, accumulate);
+        return launch_colsum_finalize(s, partial, nullptr, blocks, (uint32_t)inner, reinterpret_cast<float*>(dy), nullptr, accumulate, true);
     }
 }
 
@@ -501,5 +554,105 @@ int launch_mul_bwd(hipStream_t s, int dtype, int kind, const void* g, const void
     if (dtype == AGRAD_F32) return colsum_two_stage<float>(s, (const float*)g, (const float*)x, (float*)dy, workspace, lead, inner, acc_y);
     return colsum_two_stage<bf16_t>(s, (const bf16_t*)g, (const bf16_t*)x, (bf16_t*)dy, workspace, lead, inner, acc_y);
 }
+
+// ---- bias + GELU: y = GELU(h + b[:]) and its backward ---------------------------
+// The bias add of a linear layer folded into its activation: the [rows, C] tensor
+// is read once instead of written and read again (gelu_add_bias_kernel /
+// gelu_backward_bias_kernel, metal_ops.metal:3737-3773; on the CPU the composition
+// of cpu_add_forward, backend.py:74-88, and cpu_gelu_forward, backend.py:376-395).
+// The backward also owns the bias gradient -- the column sum of the very terms it
+// writes to dh -- where the reference runs bias_grad_reduce over dh afterwards.
+
+namespace {
+
+template <typename T, int VEC, bool BACKWARD>
+__global__ void __launch_bounds__(kBcastBlock)
+gelu_bias_kernel(const T* __restrict__ h, const T* __restrict__ b, const T* __restrict__ dy, T* out, uint64_t nvec,
+                 uint32_t inner_vec, FastDiv32 by_inner, int accumulate) {
+    const uint64_t idx = (uint64_t)blockIdx.x * kBcastBlock + threadIdx.x;
+    if (idx >= nvec) return;
+    float v[VEC], g[VEC], o[VEC];
+    VecIO<T, VEC>::load(h + idx * VEC, v);
+    if constexpr (BACKWARD) {
+        VecIO<T, VEC>::load(dy + idx * VEC, g);
+        if (accumulate) VecIO<T, VEC>::load(out + idx * VEC, o);
+    }
+    // the transcendental leaves no room for an emulated divide: with idx % inner_vec the
+    // forward ran at 0.66 of a copy (fp32, 16384 x 3072)
+    float bv[VEC];
+    small_vec<T, VEC>(b, nvec <= 0xffffffffull ? by_inner.mod((uint32_t)idx) : (uint32_t)(idx % inner_vec), bv);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+        const float z = v[k] + bv[k];
+        if constexpr (BACKWARD) {
+            const float t = g[k] * gelu_slope(z);
+            o[k] = accumulate ? (o[k] + t) : t;
+        } else {
+            o[k] = gelu_value(z);
+        }
+    }
+    VecIO<T, VEC>::store(out + idx * VEC, o);
+}
+
+template <typename T, bool BACKWARD>
+int gelu_bias_stream(hipStream_t s, const T* h, const T* b, const T* dy, T* out, uint64_t rows, uint64_t C, int acc) {
+    constexpr int WIDE = WideVec<T>::value;
+    const uint64_t n = rows * C;
+    const bool wide = C % WIDE == 0 && aligned16(h) && aligned16(b) && aligned16(out) && (!BACKWARD || aligned16(dy));
+    const uint64_t nvec = wide ? n / WIDE : n;
+    const uint64_t inner_vec = wide ? C / WIDE : C;
+    const uint64_t grid = (nvec + kBcastBlock - 1) / kBcastBlock;
+    if (grid > 0x7fffffffull) return set_error(AGRAD_EINVAL, "bias gelu: tensor too large");
+    const FastDiv32 by_inner((uint32_t)inner_vec);
+    if (wide) hipLaunchKernelGGL((gelu_bias_kernel<T, WIDE, BACKWARD>), dim3((uint32_t)grid), dim3(kBcastBlock), 0, s, h, b, dy, out, nvec, (uint32_t)inner_vec, by_inner, acc);
+    else hipLaunchKernelGGL((gelu_bias_kernel<T, 1, BACKWARD>), dim3((uint32_t)grid), dim3(kBcastBlock), 0, s, h, b, dy, out, nvec, (uint32_t)inner_vec, by_inner, acc);
+    return check_hip(hipGetLastError(), "bias gelu launch");
+}
+
+}  // namespace
+
+int launch_gelu_bias_fwd(hipStream_t s, int dtype, const void* h, const void* b, void* y, uint64_t rows, uint32_t C) {
+    if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "bias gelu: unknown dtype %d", dtype);
+    if (rows == 0 || C == 0) return AGRAD_OK;
+    if (h == nullptr || b == nullptr || y == nullptr) return set_error(AGRAD_EINVAL, "bias gelu: null operand");
+    if (dtype == AGRAD_F32) return gelu_bias_stream<float, false>(s, (const float*)h, (const float*)b, nullptr, (float*)y, rows, C, 0);
+    return gelu_bias_stream<bf16_t, false>(s, (const bf16_t*)h, (const bf16_t*)b, nullptr, (bf16_t*)y, rows, C, 0);
+}
+
+// partial rows, plus one fp32 row in which a bf16 bias gradient is finished before it is rounded
+uint64_t gelu_bias_backward_workspace_bytes(uint64_t rows, uint32_t C) {
+    if (rows == 0 || C == 0) return 0;
+    return ((uint64_t)colsum_blocks(rows) + 1) * C * sizeof(float);
+}
+
+int launch_gelu_bias_bwd(hipStream_t s, int dtype, const void* dy, const void* h, const void* b, void* dh, void* db,
+                         void* workspace, uint64_t workspace_bytes, uint64_t rows, uint32_t C, uint32_t flags) {
+    if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "bias gelu backward: unknown dtype %d", dtype);
+    if (C == 0) return AGRAD_OK;
+    if (rows >= 0x7fffffffull) return set_error(AGRAD_EINVAL, "bias gelu backward: tensor too large");
+    const int acc_db = (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0, acc_dh = (flags & AGRAD_ACC_INPUT_GRAD) ? 1 : 0;
+    if (rows == 0) {
+        // an empty sum: a stored bias gradient is zero, an accumulated one keeps its value
+        if (db != nullptr && !acc_db) return launch_fill(s, db, 0, (int)dtype_size(dtype), C);
+        return AGRAD_OK;
+    }
+    if (dy == nullptr || h == nullptr || b == nullptr || (dh == nullptr && db == nullptr))
+        return set_error(AGRAD_EINVAL, "bias gelu backward: null operand");
+    if (db == nullptr) {
+        if (dtype == AGRAD_F32) return gelu_bias_stream<float, true>(s, (const float*)h, (const float*)b, (const float*)dy, (float*)dh, rows, C, acc_dh);
+        return gelu_bias_stream<bf16_t, true>(s, (const bf16_t*)h, (const bf16_t*)b, (const bf16_t*)dy, (bf16_t*)dh, rows, C, acc_dh);
+    }
+    const uint64_t need = gelu_bias_backward_workspace_bytes(rows, C);
+    if (workspace == nullptr || workspace_bytes < need)
+        return set_error(AGRAD_EWORKSPACE, "bias gelu backward: workspace %llu < %llu bytes",
+                         (unsigned long long)workspace_bytes, (unsigned long long)need);
+    if (!aligned16(workspace)) return set_error(AGRAD_EINVAL, "bias gelu backward: workspace must be 16-byte aligned");
+    if (dtype == AGRAD_F32)
+        return colsum_two_stage<float, kStageGeluBias>(s, (const float*)dy, (const float*)h, (float*)db, workspace, rows, C,
+                                                       acc_db, (const float*)b, (float*)dh, acc_dh);
+    return colsum_two_stage<bf16_t, kStageGeluBias>(s, (const bf16_t*)dy, (const bf16_t*)h, (bf16_t*)db, workspace, rows, C,
+                                                    acc_db, (const bf16_t*)b, (bf16_t*)dh, acc_dh);
+}
+
 
 }  // namespace agrad

@@ -365,6 +365,27 @@ class GELUOp(Op):
         return [0]
 
 
+class BiasGELUOp(Op):
+    """y = GELU(h + b) with b the trailing [C] of h: the bias add of a linear layer folded
+    into its activation (gelu_add_bias_kernel / gelu_backward_bias_kernel,
+    metal_ops.metal:3737-3773; as a graph the reference writes Add then GELU, op.py:47-59, 241-245)"""
+    op_name = "BiasGELU"
+
+    def infer_shape(self, h, b):
+        trailing = tuple(b.shape)
+        while len(trailing) > 1 and trailing[0] == 1:
+            trailing = trailing[1:]
+        if len(h.shape) < 1 or trailing != (h.shape[-1],):
+            raise RuntimeError(f"BiasGELU: the bias must be the trailing [C] of h, got h={h.shape} b={b.shape}")
+        return h.shape
+
+    def save_for_backward(self, inputs, outputs):
+        return list(inputs)
+
+    def fully_written_inputs(self, inputs, outputs):
+        return [0, 1]
+
+
 class ReLUSquaredOp(Op):
     op_name = "ReLUSquared"
 

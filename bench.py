@@ -347,6 +347,29 @@ def _primitive_cases(ctx, cfg, pool, rng, nbytes, ids0):
         cases.append(Case("mul_row", "prim-fwd", 2 * m_n * e, m_k, mul_fwd, "bcast_mul_kernel"))
         if m_k > 1:
             cases.append(Case("mul_row", "prim-bwd", 3 * m_n * e, m_k, mul_bwd, "bcast_mul_kernel"))
+    if cfg.act == "gelu":
+        # GELU(h + b) on the MLP's hidden tensor [N, 4C]: forward reads h, writes y (2*n*e);
+        # backward reads dy and h, writes dh (3*n*e) and leaves the bias gradient beside it
+        bg_rows, bg_C = cfg.N, cfg.act_width
+        bg_n = bg_rows * bg_C
+        bg_k = n_sets(3 * bg_n * e)
+        bg_h = [pool.normal(bg_n, cfg.dtype) for _ in range(bg_k)]
+        bg_dy = [pool.normal(bg_n, cfg.dtype) for _ in range(bg_k)]
+        bg_out = [pool.empty(bg_n, cfg.dtype) for _ in range(bg_k)]
+        bg_b = pool.normal(bg_C, cfg.dtype)
+        bg_db = pool.empty(bg_C, cfg.dtype)
+        bg_ws_bytes = ctx.lib.agrad_gelu_bias_backward_workspace_bytes(bg_rows, bg_C)
+        bg_ws = pool.raw(max(bg_ws_bytes, 256))
+
+        def bias_gelu_fwd(i):
+            ctx.call("agrad_gelu_bias_forward", dt, vp(bg_h[i]), vp(bg_b), vp(bg_out[i]), bg_rows, bg_C)
+
+        def bias_gelu_bwd(i):
+            ctx.call("agrad_gelu_bias_backward", dt, vp(bg_dy[i]), vp(bg_h[i]), vp(bg_b), vp(bg_out[i]), vp(bg_db),
+                     vp(bg_ws), bg_ws_bytes, bg_rows, bg_C, 0)
+
+        cases.append(Case("bias_gelu", "prim-fwd", 2 * bg_n * e, bg_k, bias_gelu_fwd, "gelu_bias_kernel"))
+        cases.append(Case("bias_gelu", "prim-bwd", 3 * bg_n * e, bg_k, bias_gelu_bwd, "colsum_partial_kernel"))
     return cases
 
 

@@ -223,6 +223,20 @@ int agrad_norm_backward(agrad_ctx* ctx, int kind, int dtype,
 /* tanh-GELU (cpu_gelu_forward / backward, backend.py:376-414).               */
 int agrad_gelu_forward(agrad_ctx* ctx, int dtype, const void* x, void* y, uint64_t n);
 int agrad_gelu_backward(agrad_ctx* ctx, int dtype, const void* x, const void* dy, void* dx, uint64_t n, uint32_t flags);
+/* The bias add of a linear layer folded into its GELU: y[r, c] = GELU(h[r, c] + b[c])
+ * for h of shape [rows, C] (gelu_add_bias_kernel / gelu_backward_bias_kernel,
+ * metal_ops.metal:3737-3773; on the CPU cpu_add_forward, backend.py:74-88, followed
+ * by cpu_gelu_forward, backend.py:376-395).  Backward: dh (+)= dy * GELU'(h + b)
+ * (AGRAD_ACC_INPUT_GRAD accumulates) and, when db is not NULL, db[c] (+)= the sum
+ * over rows of the same terms in a fixed order (AGRAD_ACC_PARAM_GRAD accumulates;
+ * the reference runs bias_grad_reduce, metal_ops.metal:1026-1193, over dh
+ * afterwards).  Either of dh and db may be NULL, not both.  With db the call needs
+ * a 16-byte aligned workspace of agrad_gelu_bias_backward_workspace_bytes(rows, C)
+ * bytes; without, none. */
+int agrad_gelu_bias_forward(agrad_ctx* ctx, int dtype, const void* h, const void* b, void* y, uint64_t rows, uint32_t C);
+uint64_t agrad_gelu_bias_backward_workspace_bytes(uint64_t rows, uint32_t C);
+int agrad_gelu_bias_backward(agrad_ctx* ctx, int dtype, const void* dy, const void* h, const void* b, void* dh, void* db,
+                             void* workspace, uint64_t workspace_bytes, uint64_t rows, uint32_t C, uint32_t flags);
 /* ReLU^2: y = max(x,0)^2, dx = 2 max(x,0) dy.  No counterpart in the reference. */
 int agrad_relu2_forward(agrad_ctx* ctx, int dtype, const void* x, void* y, uint64_t n);
 int agrad_relu2_backward(agrad_ctx* ctx, int dtype, const void* x, const void* dy, void* dx, uint64_t n, uint32_t flags);

@@ -18,7 +18,7 @@ import numpy as np
 from autograd_amd.backend import Backend
 from autograd_amd.device import Device
 from autograd_amd.op import (AddLayerNormOp, AddOp, AddRMSNormOp, ContiguousOp, CrossEntropyLossOp, EmbeddingSumOp,
-                             ExpOp, GatherOp, GELUOp, LayerNormOp, LogOp, MulOp, PermuteOp, ReLUSquaredOp, ReshapeOp,
+                             BiasGELUOp, ExpOp, GatherOp, GELUOp, LayerNormOp, LogOp, MulOp, PermuteOp, ReLUSquaredOp, ReshapeOp,
                              RMSNormOp, RopeOp, RsqrtOp, SoftmaxOp, SwiGLUOp, TransposeOp, ViewOp)
 from autograd_amd.storage import Allocator, Storage
 from autograd_amd.utils import is_bf16, storage_dtype
@@ -208,6 +208,23 @@ cpu_gelu_forward, cpu_gelu_backward = _unary(K.gelu_forward, K.gelu_backward_int
 cpu_relu2_forward, cpu_relu2_backward = _unary(K.relu2_forward, K.relu2_backward_into)
 
 
+def cpu_bias_gelu_forward(inputs, outputs, scratch=None):
+    _put(outputs[0], K.bias_gelu_forward(_val(inputs[0]), _val(inputs[1])))
+
+
+def cpu_bias_gelu_backward(inputs, outputs, scratch=None):
+    h, b, out = inputs[0], inputs[1], outputs[0]
+    if out.grad is None:
+        return
+    g, hv, bv = _val(out.grad), _val(h), _val(b)
+    if h.requires_grad and h.grad is not None:
+        with _Acc(h.grad) as acc:
+            K.bias_gelu_backward_into(hv, bv, g, dh=acc)
+    if b.requires_grad and b.grad is not None:
+        with _Acc(b.grad) as acc:
+            K.bias_gelu_backward_into(hv, bv, g, db=acc)
+
+
 def cpu_swiglu_forward(inputs, outputs, scratch=None):
     _put(outputs[0], K.swiglu_forward(_val(inputs[0])))
 
@@ -371,7 +388,7 @@ class CPUBackend(Backend):
         self.accumulate_parameter_grads = False
         self.forward_kernels = {
             AddOp: cpu_add_forward, GatherOp: cpu_gather_forward, EmbeddingSumOp: cpu_embedding_sum_forward,
-            GELUOp: cpu_gelu_forward, ReLUSquaredOp: cpu_relu2_forward, SwiGLUOp: cpu_swiglu_forward,
+            GELUOp: cpu_gelu_forward, BiasGELUOp: cpu_bias_gelu_forward, ReLUSquaredOp: cpu_relu2_forward, SwiGLUOp: cpu_swiglu_forward,
             LayerNormOp: cpu_layernorm_forward, RMSNormOp: cpu_rmsnorm_forward,
             AddLayerNormOp: cpu_add_norm_forward, AddRMSNormOp: cpu_add_norm_forward, RopeOp: cpu_rope_forward,
             CrossEntropyLossOp: cpu_cross_entropy_forward,
@@ -382,7 +399,7 @@ class CPUBackend(Backend):
         }
         self.backward_kernels = {
             AddOp: cpu_add_backward, GatherOp: cpu_gather_backward, EmbeddingSumOp: cpu_embedding_sum_backward,
-            GELUOp: cpu_gelu_backward, ReLUSquaredOp: cpu_relu2_backward, SwiGLUOp: cpu_swiglu_backward,
+            GELUOp: cpu_gelu_backward, BiasGELUOp: cpu_bias_gelu_backward, ReLUSquaredOp: cpu_relu2_backward, SwiGLUOp: cpu_swiglu_backward,
             LayerNormOp: cpu_layernorm_backward, RMSNormOp: cpu_rmsnorm_backward,
             AddLayerNormOp: cpu_add_norm_backward, AddRMSNormOp: cpu_add_norm_backward, RopeOp: cpu_rope_backward,
             CrossEntropyLossOp: cpu_cross_entropy_backward,

@@ -24,6 +24,8 @@ Pinning (what shows these functions are the right functions; tests/test_oracle.p
   * mul / exp / log / rsqrt / softmax: float64 closed forms (scipy.special.softmax,
     the softmax Jacobian written out), explicit index loops for the broadcast sums
     of the mul gradient, finite differences, rows of a softmax sum to one.
+  * bias_gelu: the float64 closed form of GELU at h + b, finite differences in h and in b,
+    an explicit row loop for the bias gradient.
   * adamw: the textbook bias-corrected recurrence in float64 over several steps;
     the first step from zero moments moves every weight by lr * sign(g).
 Parity unpinned by the reference:
@@ -213,6 +215,23 @@ def gelu_backward_into(x, dy, dx):
     np.add(t, a, out=t)
     np.multiply(dy, t, out=a)
     np.add(dx, a, out=dx)
+
+
+def bias_gelu_forward(h, b):
+    """GELU(h + b): cpu_add_forward (backend.py:74-88) then cpu_gelu_forward (backend.py:376-395);
+    the sum is what gelu_add_bias_kernel forms per element (metal_ops.metal:3746-3747)"""
+    return gelu_forward(np.add(h, b))
+
+
+def bias_gelu_backward_into(h, b, dy, dh=None, db=None):
+    """dh += dy * GELU'(h + b) (cpu_gelu_backward, backend.py:396-414); db += the same terms
+    summed over the leading axes (cpu_add_backward's reduction, backend.py:89-105)"""
+    term = np.zeros_like(np.asarray(h, dtype=np.float32))
+    gelu_backward_into(np.add(h, b), dy, term)
+    if dh is not None:
+        np.add(dh, term, out=dh)
+    if db is not None:
+        add_backward_into(term, db)
 
 
 # --------------------------------------------------------------------------

@@ -222,3 +222,90 @@ def test_argument_errors(ctx):
     ctx.call("agrad_unary_forward", capi.UNARY_EXP, capi.F32, vp(buf), vp(buf), 0)
     ctx.synchronize()
     buf.free()
+
+
+# -- GELU(h + b) and its backward with the bias gradient ---------------------------------
+BIAS_GELU_SHAPES = [(1, 1), (3, 5), (64, 384), (65, 384), (1000, 96), (300, 1536), (2048, 1000), (5000, 130),
+                    (16384, 64)]
+
+
+@pytest.mark.parametrize("rows,Cw", BIAS_GELU_SHAPES)
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_bias_gelu_forward_and_backward(ctx, rows, Cw, dtype):
+    """agrad_gelu_bias_forward / _backward against the CPU composition Add -> GELU
+    (cpu_add_forward, cpu_gelu_forward / backward, cpu_add_backward's reduction):
+    dh stored and accumulated, db stored and accumulated, each alone and together.
+    fp32: rtol 1e-5 / atol 1e-6 for y and dh; the bias gradient is a sum of `rows`
+    terms, compared to float64 with the bound of the other column sums.  bf16
+    storage: 1e-2 relative to the fp32 restatement on the bf16-rounded inputs."""
+    rng = np.random.default_rng(SEED + rows * 7 + Cw)
+    dt = capi.BF16 if dtype == "bf16" else capi.F32
+    hs, h = _io(rng.standard_normal((rows, Cw)).astype(np.float32), dtype)
+    bs, b = _io((0.5 * rng.standard_normal(Cw)).astype(np.float32), dtype)
+    dys, dy = _io(rng.standard_normal((rows, Cw)).astype(np.float32), dtype)
+    dh0s, dh0 = _io(rng.standard_normal((rows, Cw)).astype(np.float32), dtype)
+    db0s, db0 = _io(rng.standard_normal(Cw).astype(np.float32), dtype)
+    d_h, d_b, d_dy = ctx.upload(hs), ctx.upload(bs), ctx.upload(dys)
+    d_y = ctx.empty((rows, Cw), hs.dtype)
+    ctx.call("agrad_gelu_bias_forward", dt, vp(d_h), vp(d_b), vp(d_y), rows, Cw)
+    ctx.synchronize()
+    got_y = d_y.download()
+    want_y = ref.bias_gelu_forward(h, b)
+    if dtype == "bf16":
+        assert_bf16_close(from_bf16_bits(got_y), want_y, "bias gelu forward")
+    else:
+        assert_fp32_close(got_y, want_y, "bias gelu forward")
+
+    term = np.zeros((rows, Cw), np.float32)
+    ref.bias_gelu_backward_into(h, b, dy, dh=term)
+    col = term.astype(np.float64).sum(axis=0)
+    ws_b = ctx.lib.agrad_gelu_bias_backward_workspace_bytes(rows, Cw)
+    assert ws_b >= 4 * Cw
+    ws = ctx.empty((ws_b,), np.uint8)
+    cases = [(0, True, True), (capi.ACC_INPUT_GRAD | capi.ACC_PARAM_GRAD, True, True),
+             (capi.ACC_INPUT_GRAD, True, False), (capi.ACC_PARAM_GRAD, False, True), (0, False, True)]
+    for flags, want_dh, want_db in cases:
+        d_dh = ctx.upload(dh0s) if want_dh else None
+        d_db = ctx.upload(db0s) if want_db else None
+        ctx.call("agrad_gelu_bias_backward", dt, vp(d_dy), vp(d_h), vp(d_b), vp(d_dh), vp(d_db),
+                 vp(ws) if want_db else None, ws_b if want_db else 0, rows, Cw, flags)
+        ctx.synchronize()
+        what = f"bias gelu backward flags={flags} dh={want_dh} db={want_db}"
+        if want_dh:
+            got = d_dh.download()
+            want = term + dh0 if flags & capi.ACC_INPUT_GRAD else term
+            if dtype == "bf16":
+                assert_bf16_close(from_bf16_bits(got), want, what + " dh")
+            else:
+                # beyond |h + b| = 4.5 the CPU's 1 - tanh^2 has lost its bits to cancellation
+                # and the device value is the accurate one: 3e-6 absolute, as for plain GELU
+                assert_fp32_close(got, want, what + " dh", rtol=1e-5, atol=3e-6)
+            d_dh.free()
+        if want_db:
+            got = d_db.download()
+            want = col + db0 if flags & capi.ACC_PARAM_GRAD else col
+            if dtype == "bf16":
+                scale = np.abs(term).astype(np.float64).sum(axis=0) + np.abs(db0)
+                err = np.abs(from_bf16_bits(got).astype(np.float64) - want)
+                assert (err <= 1e-2 * np.maximum(np.abs(want), 1e-2 * scale) + 1e-3).all(), what + " db"
+            else:
+                assert_fp32_close(got, want.astype(np.float32), what + " db", rtol=1e-5,
+                                  atol=max(2e-6, 1e-4 * np.sqrt(rows / 14)))
+            d_db.free()
+    for d in (d_h, d_b, d_dy, d_y, ws):
+        d.free()
+
+
+def test_bias_gelu_argument_errors(ctx):
+    h = ctx.zeros((128, 64), np.float32)
+    b = ctx.zeros((64,), np.float32)
+    with pytest.raises(capi.AgradError):         # the bias gradient needs its workspace
+        ctx.call("agrad_gelu_bias_backward", capi.F32, vp(h), vp(h), vp(b), vp(h), vp(b), None, 0, 128, 64, 0)
+    with pytest.raises(capi.AgradError):         # nothing to compute
+        ctx.call("agrad_gelu_bias_backward", capi.F32, vp(h), vp(h), vp(b), None, None, None, 0, 128, 64, 0)
+    with pytest.raises(capi.AgradError):
+        ctx.call("agrad_gelu_bias_forward", 7, vp(h), vp(b), vp(h), 128, 64)
+    ctx.call("agrad_gelu_bias_forward", capi.F32, vp(h), vp(b), vp(h), 0, 64)      # empty: no launch
+    ctx.synchronize()
+    h.free()
+    b.free()

@@ -475,6 +475,40 @@ def test_primitive_ops_in_a_graph():
     np.testing.assert_allclose(h_out[0], want, rtol=2e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("bias_grad", [True, False])
+def test_bias_gelu_in_a_graph_equals_add_then_gelu(bias_grad):
+    """x.bias_gelu(b) against (x + b).gelu() -- the way the reference writes it
+    (op.py:47-59, 241-245) -- on both devices, twice over the same arena; with the
+    bias frozen the fused backward needs no workspace"""
+    rng = np.random.default_rng(SEED + 41)
+    B, T, C = 4, 50, 192
+    x_np = rng.standard_normal((B, T, C), dtype=np.float32)
+    b_np = rng.standard_normal(C).astype(np.float32)
+    g_np = (1 + 0.1 * rng.standard_normal(C)).astype(np.float32)
+    upstream = rng.standard_normal((B, T, C), dtype=np.float32)
+
+    def build_with(fused):
+        def build(device):
+            x = make_tensor(x_np.shape, np.float32, device, True, x_np, "x")
+            b = make_tensor(b_np.shape, np.float32, device, bias_grad, b_np, "b")
+            g = make_tensor(g_np.shape, np.float32, device, True, g_np, "g")
+            h = x.rms_norm(g)                       # an activation feeds the fused op
+            out = h.bias_gelu(b) if fused else (h + b).gelu()
+            return out, {"x": x, "b": b, "g": g} if bias_grad else {"x": x, "g": g}
+        return build
+
+    (c_out, c_g), (h_out, h_g) = both(build_with(True), upstream)
+    (p_out, p_g), (q_out, q_g) = both(build_with(False), upstream)
+    assert_fp32_close(h_out[0], c_out[0], "fused forward, hip vs cpu", rtol=2e-5, atol=2e-6)
+    np.testing.assert_array_equal(c_out[0], p_out[0])         # the oracle's fused op IS the composition
+    assert_fp32_close(h_out[0], q_out[0], "fused vs add->gelu on hip", rtol=2e-5, atol=2e-6)
+    for name in c_g:
+        terms = B * T if name in ("b", "g") else 1
+        bound = 2e-5 * np.sqrt(terms) * (np.abs(c_g[name]).max() + 1.0)
+        assert np.abs(h_g[name] - c_g[name]).max() <= bound, name
+        assert np.abs(h_g[name] - q_g[name]).max() <= bound, name
+
+
 def test_captured_graph_replays_match_eager():
     """Record forward + zero_grad + upstream copy + backward of the tiny GPT-2 chain
     once, replay it several times with eager work and synchronisations in between,

@@ -55,6 +55,39 @@ def test_gelu_backward_finite_difference_and_accumulate():
     close(acc, base + dx, atol=2e-6)
 
 
+def test_bias_gelu_is_gelu_of_the_sum_and_its_bias_gradient_is_the_row_sum():
+    r = rng(23)
+    h = r.standard_normal((4, 9, 33), dtype=np.float32)
+    b = r.standard_normal(33, dtype=np.float32)
+    dy = r.standard_normal(h.shape, dtype=np.float32)
+    close(K.bias_gelu_forward(h, b), cf.gelu(h.astype(np.float64) + b))
+    dh = np.zeros_like(h)
+    db = np.zeros_like(b)
+    K.bias_gelu_backward_into(h, b, dy, dh=dh, db=db)
+    slope = cf.gelu_grad(h.astype(np.float64) + b)
+    close(dh, dy * slope, rtol=2e-5, atol=2e-6)
+    by_rows = np.zeros(33)
+    for i in range(4):                     # the bias gradient, row by row
+        for j in range(9):
+            by_rows += dy[i, j] * slope[i, j]
+    close(db, by_rows, rtol=2e-5, atol=2e-5)
+    # finite differences: in one element of h, and in one element of b (which moves a whole column)
+    loss = lambda hh, bb: float((cf.gelu(hh + bb) * dy).sum())
+    h64, b64 = h.astype(np.float64), b.astype(np.float64)
+    for idx in ((0, 0, 0), (3, 8, 32), (1, 4, 17)):
+        e = np.zeros_like(h64); e[idx] = 1e-5
+        close(dh[idx], (loss(h64 + e, b64) - loss(h64 - e, b64)) / 2e-5, rtol=1e-4, atol=1e-5)
+    for c in (0, 17, 32):
+        e = np.zeros_like(b64); e[c] = 1e-5
+        close(db[c], (loss(h64, b64 + e) - loss(h64, b64 - e)) / 2e-5, rtol=1e-4, atol=2e-5)
+    # "grad += ..." on both, and either alone
+    dh2, db2 = dh.copy(), db.copy()
+    K.bias_gelu_backward_into(h, b, dy, dh=dh2)
+    K.bias_gelu_backward_into(h, b, dy, db=db2)
+    close(dh2, 2 * dh, atol=4e-6)
+    close(db2, 2 * db, atol=4e-5)
+
+
 # ---- ReLU^2 (closed form only: the reference has none) ---------------------------
 def test_relu2():
     r = rng(11)
