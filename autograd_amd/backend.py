@@ -774,10 +774,31 @@ class HipBackend(Backend):
         return self.ctx.copy_to_host(storage.ptr.buffer_id, storage.ptr.offset, list(storage.shape),
                                      np.dtype(storage.dtype).name)
 
+    def storage_from_host(self, storage, host_np):
+        """raw host copy into a storage (the array already has the storage's dtype and size)"""
+        host = np.ascontiguousarray(host_np, dtype=np.dtype(storage.dtype))
+        if host.size != prod(storage.shape):
+            raise ValueError(f"storage_from_host: {host.shape} does not fill {storage.shape}")
+        self.ctx.copy_from_host(storage.ptr.buffer_id, storage.ptr.offset, host.reshape(-1))
+
     # -- optimizer (backend.py:5115-5140) ------------------------------------------------
     def grad_norm_sq(self, g_storage, partial, numel):
         """partial[i] = sum of squares of 256-element group i of the gradient"""
         self._launch("grad_norm_sq", [g_storage, partial], _lo_hi(int(numel)) + [_dt(g_storage)])
+
+    def adamw8bit_step(self, p, g, qm, qv, absmax_m, absmax_v, qmap_m, qmap_v,
+                       lr, lr_bc1, inv_sqrt_bc2, b1, b2, eps, weight_decay, numel, decay_numel, first_step, grad_scale=1.0):
+        """One AdamW step with 8-bit moments on one parameter; the signature and the
+        argument list of the launch are the Metal backend's (backend.py:5142-5151)."""
+        g_bf16 = np.dtype(g.dtype) == np.dtype(np.uint16)
+        if not g_bf16 and np.dtype(g.dtype) != np.dtype(np.float32):
+            raise RuntimeError(f"adamw8bit: gradient dtype {g.dtype}")
+        if int(numel) > 0xFFFFFFFF:
+            raise RuntimeError("adamw8bit: one launch takes at most 2^32 - 1 elements")
+        self._launch("adamw8bit_step", [p, g, qm, qv, absmax_m, absmax_v, qmap_m, qmap_v],
+                     [f32_bits(1.0 - float(lr) * float(weight_decay)), f32_bits(lr_bc1), f32_bits(b1), f32_bits(b2),
+                      f32_bits(eps), int(numel), int(decay_numel), int(bool(first_step)), f32_bits(inv_sqrt_bc2),
+                      int(g_bf16), f32_bits(grad_scale)])
 
     def adamw_step(self, p_storage, g_storage, m_storage, v_storage, tmp_storage,
                    lr, lr_t, b1, b2, eps, weight_decay, numel=None, decay_numel=None, grad_scale=1.0,

@@ -96,6 +96,8 @@ SIGNATURES = {
     "agrad_broadcast_add_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _u64, _u64, _u64, _u32]),
     "agrad_cross_entropy_forward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u32]),
     "agrad_cross_entropy_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _u64, _u32, _u32]),
+    "agrad_adamw8bit_step": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _u64, _u64,
+                                    _f32, _f32, _f32, _f32, _f32, _f32, _f32, _int]),
     "agrad_adamw_step": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u64] + [_f32] * 9),
     "agrad_grad_norm_groups": (_u64, [_u64]),
     "agrad_grad_norm_sq": (_int, [_ctx, _int, _ptr, _ptr, _u64]),

@@ -439,6 +439,18 @@ int h_adamw(const Call& c) {
                         f32(c.a[1]), f32(c.a[2]), f32(c.a[3]), f32(c.a[4]), f32(c.a[5]), f32(c.a[6]),
                         f32(c.a[7]), f32(c.a[8]));
 }
+// buffers p, g, qm, qv, absmax_m, absmax_v, qmap_m, qmap_v; args decay, lr_bc1, b1, b2, eps (float
+// bits), numel, decay_numel, first_step, inv_sqrt_bc2 (bits), grad_bf16, clip_coef (bits) -- the
+// reference's own list (Backend.adamw8bit_step, backend.py:5142-5151)
+int h_adamw8bit(const Call& c) {
+    const uint64_t n = c.a[5], blocks = (n + 255) / 256;
+    const int gd = c.a[9] ? AGRAD_BF16 : AGRAD_F32;
+    RESOLVE(0, n * 4, p) RESOLVE(1, n * dtype_size(gd), g) RESOLVE(2, n, qm) RESOLVE(3, n, qv)
+    RESOLVE(4, blocks * 4, am) RESOLVE(5, blocks * 4, av) RESOLVE(6, 1024, mapm) RESOLVE(7, 1024, mapv)
+    return launch_adamw8bit(c.ctx->stream, gd, (float*)p, g, (uint8_t*)qm, (uint8_t*)qv, (float*)am, (float*)av,
+                            (const float*)mapm, (const float*)mapv, n, c.a[6], f32(c.a[0]), f32(c.a[1]), f32(c.a[2]),
+                            f32(c.a[3]), f32(c.a[4]), f32(c.a[8]), f32(c.a[10]), (int)c.a[7]);
+}
 // buffers g, partial | args numel lo, hi, dtype
 int h_grad_norm(const Call& c) {
     NEED_DTYPE(c.a[2])
@@ -487,6 +499,7 @@ const Entry kTable[] = {
     {"cross_entropy_forward", 4, 5, "logits, labels, loss, lse | dtype, rows_lo, rows_hi, V, present_mask", h_ce_fwd},
     {"cross_entropy_backward", 5, 6, "logits, labels, dloss, lse, dlogits | dtype, rows_lo, rows_hi, V, flags, present_mask", h_ce_bwd},
     {"adamw_step", 4, 14, "p, g, m, v | lr_wd, b1, one_minus_b1, b2, one_minus_b2, eps, step_lr, inv_sqrt_bc2, grad_scale (float bits), n_lo, n_hi, decay_lo, decay_hi, grad_dtype", h_adamw},
+    {"adamw8bit_step", 8, 11, "p, g, qm, qv, absmax_m, absmax_v, qmap_m, qmap_v | decay, lr_bc1, b1, b2, eps (float bits), numel, decay_numel, first_step, inv_sqrt_bc2 (bits), grad_bf16, clip_coef (bits)", h_adamw8bit},
     {"grad_norm_sq", 2, 3, "g, partial | n_lo, n_hi, dtype", h_grad_norm},
 };
 constexpr int kTableSize = (int)(sizeof(kTable) / sizeof(kTable[0]));
@@ -932,6 +945,14 @@ int agrad_cross_entropy_backward(agrad_ctx* ctx, int dtype, const void* logits, 
     return launch_ce_bwd(ctx->stream, dtype, logits, labels, dloss, lse, dlogits, rows, V, flags, ctx->err_flag);
 }
 
+int agrad_adamw8bit_step(agrad_ctx* ctx, int grad_dtype, float* p, const void* g, uint8_t* qm, uint8_t* qv,
+                         float* absmax_m, float* absmax_v, const float* qmap_m, const float* qmap_v,
+                         uint64_t numel, uint64_t decay_numel, float decay, float lr_bc1, float b1, float b2,
+                         float eps, float inv_sqrt_bc2, float clip_coef, int first_step) {
+    CTX_OR_FAIL(ctx)
+    return launch_adamw8bit(ctx->stream, grad_dtype, p, g, qm, qv, absmax_m, absmax_v, qmap_m, qmap_v, numel,
+                            decay_numel, decay, lr_bc1, b1, b2, eps, inv_sqrt_bc2, clip_coef, first_step);
+}
 int agrad_adamw_step(agrad_ctx* ctx, int grad_dtype, float* p, const void* g, float* m, float* v,
                      uint64_t numel, uint64_t decay_numel, float lr_wd, float b1, float one_minus_b1,
                      float b2, float one_minus_b2, float eps, float step_lr, float inv_sqrt_bc2,

@@ -117,6 +117,10 @@ int launch_pos_embedding_bwd(hipStream_t s, int dtype, const void* dY, void* dwp
 int launch_adamw(hipStream_t s, int grad_dtype, float* p, const void* g, float* m, float* v,
                  uint64_t numel, uint64_t decay_numel, float lr_wd, float b1, float one_minus_b1,
                  float b2, float one_minus_b2, float eps, float step_lr, float inv_sqrt_bc2, float grad_scale);
+int launch_adamw8bit(hipStream_t s, int grad_dtype, float* p, const void* g, uint8_t* qm, uint8_t* qv,
+                     float* absmax_m, float* absmax_v, const float* qmap_m, const float* qmap_v,
+                     uint64_t numel, uint64_t decay_numel, float decay, float lr_bc1, float b1, float b2, float eps,
+                     float inv_sqrt_bc2, float clip_coef, int first_step);
 uint64_t grad_norm_groups(uint64_t numel);
 int launch_grad_norm_sq(hipStream_t s, int dtype, const void* g, float* partial, uint64_t numel);
 

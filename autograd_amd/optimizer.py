@@ -1,8 +1,10 @@
 """AdamW over the runtime's parameter slabs, and the gradient-norm clip
 (counterpart of the reference's optimizer.py:11-20, 54-140, 443-600).
 
-Only the fp32-state optimizer is provided (`state_mode="fp32"`); the reference's
-8-bit and "mini" state modes are outside this package.
+`state_mode="fp32"` keeps both moments in fp32; `state_mode="8bit"` keeps them as
+one byte per element plus one fp32 scale per block of 256 (optimizer.py:143-232,
+469-479) for every parameter of at least 4096 elements, fp32 below that.  The
+reference's "mini" mode is outside this package.
 
 On a device whose backend owns a native context, parameters that the runtime
 packed into one slab (matrices first, then vectors) are updated by ONE kernel
@@ -41,18 +43,49 @@ def get_lr_cosine_schedule(step, max_steps, warmup_steps, max_lr, min_lr):
     return min_lr + 0.5 * (1.0 + math.cos(math.pi * ratio)) * (max_lr - min_lr)
 
 
+def build_dynamic_map(signed, max_exponent_bits=7, total_bits=8):
+    """The sorted 256-entry code book of the 8-bit moments (optimizer.py:144-179):
+    per decade 10^-6 .. 10^0 the centres of 2^k equal bins of [0.1, 1] (k grows by one
+    per decade; the unsigned map starts one power higher and has one more value below
+    the last decade), mirrored when signed, zero-padded to 256, sorted, and scaled so
+    that the largest magnitude is exactly 1."""
+    f32 = np.float32
+    magnitude_bits = total_bits - 1 if signed else total_bits
+    runs = []
+    for decade in range(max_exponent_bits):
+        edges = np.linspace(0.1, 1.0, 2 ** (decade + magnitude_bits - max_exponent_bits) + 1, dtype=f32)
+        runs.append((edges[:-1] + edges[1:]) * f32(0.5) * f32(10.0 ** (decade - (max_exponent_bits - 1))))
+    below = 2 ** (magnitude_bits - max_exponent_bits) - 1
+    if below > 0:
+        edges = np.linspace(0.0, 0.1, below + 1, dtype=f32)
+        runs.append((edges[:-1] + edges[1:]) * f32(0.5) * f32(10.0 ** (-(max_exponent_bits - 1))))
+    # the reference collects the values as Python floats before rounding them back to fp32
+    positive = np.concatenate(runs).astype(np.float64)
+    values = np.concatenate([positive, -positive]) if signed else positive
+    size = 1 << total_bits
+    if values.size >= size:
+        raise RuntimeError(f"invalid dynamic-map size: {values.size}")
+    qmap = np.zeros(size, f32)
+    qmap[:values.size] = values.astype(f32)
+    qmap.sort()
+    qmap /= np.max(np.abs(qmap))
+    return np.ascontiguousarray(qmap, dtype=f32)
+
+
 def _span(storage, numel, dtype):
     ptr = type(storage.ptr)(storage.ptr.buffer_id, storage.ptr.offset)
     return Storage(ptr, (numel,), dtype, storage.device, numel * itemsize(dtype))
 
 
 class AdamW:
+    BLOCK_SIZE = 256          # elements per scale of the 8-bit moments (optimizer.py:50)
+
     def __init__(self, params, lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, state_mode="fp32",
                  runtime=None, bias_correction="folded"):
         if state_mode not in VALID_MODE:
             raise ValueError(f"invalid state_mode={state_mode!r}, expected one of {VALID_MODE}")
-        if state_mode != "fp32":
-            raise NotImplementedError(f"state_mode={state_mode!r}: only fp32 optimizer state is provided")
+        if state_mode == "mini":
+            raise NotImplementedError("state_mode='mini': only fp32 and 8-bit optimizer state are provided")
         if bias_correction not in ("folded", "split"):
             raise ValueError(f"bias_correction={bias_correction!r}: expected 'folded' or 'split'")
         self.params = [p for p in params if p.requires_grad]
@@ -75,7 +108,10 @@ class AdamW:
                 raise RuntimeError(f"parameter {getattr(p, 'name', '?')} has no storage yet: bind the graph first")
             if np.dtype(p.dtype) != np.dtype(np.float32):
                 raise RuntimeError("AdamW keeps fp32 master parameters; got " + str(p.dtype))
-        if hasattr(self.backend, "ctx"):
+        self.qmap_m = self.qmap_v = None
+        if state_mode == "8bit":
+            self._prepare_8bit()
+        elif hasattr(self.backend, "ctx"):
             self._prepare_merged()
         else:
             self._prepare_per_parameter()
@@ -92,6 +128,53 @@ class AdamW:
             n = prod(p.shape)
             out.append((p.storage, p.grad.storage, m, v, n, n if p.ndim > 1 else 0))
         self.dispatches = tuple(out)
+
+    # ("fp32", p, g, m, v, numel, decays) or ("q8", p, g, qm, qv, absmax_m, absmax_v, numel, decays)
+    # per parameter (optimizer.py:143-232) ------------------------------------------------
+    def _prepare_8bit(self, min_8bit_size=4096):
+        if not hasattr(self.backend, "adamw8bit_step"):
+            raise NotImplementedError("this device's backend has no 8-bit AdamW step")
+        self.qmap_m = self.allocator.empty((256,), np.float32)
+        self.qmap_v = self.allocator.empty((256,), np.float32)
+        self.backend.storage_from_host(self.qmap_m, build_dynamic_map(signed=True))
+        self.backend.storage_from_host(self.qmap_v, build_dynamic_map(signed=False))
+        self._state += [self.qmap_m, self.qmap_v]
+        out = []
+        for p in self.params:
+            n = prod(p.shape)
+            if n < min_8bit_size:                  # small state is not worth quantising
+                m = self.allocator.zeros(p.shape, np.float32)
+                v = self.allocator.zeros(p.shape, np.float32)
+                self._state += [m, v]
+                out.append(("fp32", p.storage, p.grad.storage, m, v, n, p.ndim > 1))
+            else:
+                blocks = (n + self.BLOCK_SIZE - 1) // self.BLOCK_SIZE
+                m = self.allocator.zeros((n,), np.uint8)
+                v = self.allocator.zeros((n,), np.uint8)
+                absmax_m = self.allocator.zeros((blocks,), np.float32)
+                absmax_v = self.allocator.zeros((blocks,), np.float32)
+                self._state += [m, v, absmax_m, absmax_v]
+                out.append(("q8", p.storage, p.grad.storage, m, v, absmax_m, absmax_v, n, p.ndim > 1))
+            self.m.append(m)
+            self.v.append(v)
+        self.dispatches = tuple(out)
+
+    def _step_8bit(self, grad_scale):
+        b1, b2 = self.betas
+        lr_t = self.lr * math.sqrt(1.0 - b2 ** self.t) / (1.0 - b1 ** self.t)
+        lr_bc1 = self.lr / (1.0 - b1 ** self.t)
+        inv_sqrt_bc2 = 1.0 / math.sqrt(1.0 - b2 ** self.t)
+        for item in self.dispatches:
+            if item[0] == "fp32":
+                _, p, g, m, v, n, decays = item
+                self.backend.adamw_step(p, g, m, v, None, self.lr, lr_t, b1, b2, self.eps,
+                                        self.weight_decay if decays else 0.0, numel=n, decay_numel=n if decays else 0,
+                                        grad_scale=grad_scale, lr_bc1=lr_bc1, inv_sqrt_bc2=inv_sqrt_bc2)
+            else:
+                _, p, g, qm, qv, absmax_m, absmax_v, n, decays = item
+                self.backend.adamw8bit_step(p, g, qm, qv, absmax_m, absmax_v, self.qmap_m, self.qmap_v, self.lr, lr_bc1,
+                                            inv_sqrt_bc2, b1, b2, self.eps, self.weight_decay if decays else 0.0, n,
+                                            n if decays else 0, first_step=(self.t == 1), grad_scale=grad_scale)
 
     def _prepare_merged(self):
         groups = {}
@@ -152,6 +235,10 @@ class AdamW:
             lr_bc1 = self.lr / (1.0 - b1 ** self.t)
             inv_sqrt_bc2 = 1.0 / math.sqrt(1.0 - b2 ** self.t)
         self.backend.begin_pass()
+        if self.state_mode == "8bit":
+            self._step_8bit(grad_scale)
+            self.backend.end_pass()
+            return
         for p, g, m, v, numel, decay_numel in self.dispatches:
             self.backend.adamw_step(p, g, m, v, None, self.lr, lr_t, b1, b2, self.eps, self.weight_decay,
                                     numel=numel, decay_numel=decay_numel, grad_scale=grad_scale,
@@ -167,7 +254,10 @@ class AdamW:
         """-> clip_grad_norm(max_norm, eps=1e-6) -> (grad_norm, clip_coef); the
         coefficient is handed to step(grad_scale=...) rather than applied to the
         gradients (optimizer.py:505-600)."""
-        items = [(g, int(n)) for _, g, _, _, n, _ in self.dispatches]
+        if self.state_mode == "8bit":
+            items = [(item[2], int(item[-2])) for item in self.dispatches]
+        else:
+            items = [(g, int(n)) for _, g, _, _, n, _ in self.dispatches]
         partials = [self.allocator.empty(((n + 255) // 256,), np.float32) for _, n in items]
         self._state += partials
 

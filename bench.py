@@ -450,7 +450,27 @@ def _opt_cases(ctx, cfg, pool, rng, nbytes, ids0):
     def norm(i):
         ctx.call("agrad_grad_norm_sq", gdt, vp(sets[i][1]), vp(partial), n)
 
+    # the same step with 8-bit moments: p read and written (8), g, one code byte of each
+    # moment read and written (4), one scale pair per 256 elements
+    from autograd_amd.optimizer import build_dynamic_map
+    per_elem8 = 12 + cfg.esize
+    q_n = n
+    q_k = n_sets(per_elem8 * q_n)
+    q_sets = []
+    for _ in range(q_k):
+        q_sets.append((pool.normal(q_n, "f32"), pool.normal(q_n, cfg.dtype), pool.raw(q_n), pool.raw(q_n),
+                       pool.empty(groups, "f32"), pool.empty(groups, "f32")))
+    map_m, map_v = ctx.upload(build_dynamic_map(True)), ctx.upload(build_dynamic_map(False))
+    q_first = [True] * q_k
+
+    def step8(i):
+        p8, g8, qm, qv, am, av = q_sets[i]
+        ctx.call("agrad_adamw8bit_step", gdt, vp(p8), vp(g8), vp(qm), vp(qv), vp(am), vp(av), vp(map_m), vp(map_v),
+                 q_n, q_n, 1.0 - lr * 0.01, lr, b1, b2, 1e-8, 1.0, 1.0, int(q_first[i]))
+        q_first[i] = False
+
     return [Case("adamw", "opt", per_elem * n, k, step, "adamw_vec_kernel"),
+            Case("adamw_8bit", "opt", per_elem8 * q_n + 16 * groups, q_k, step8, "adamw8bit_kernel"),
             Case("grad_norm_sq", "opt", cfg.esize * n + 4 * groups, k, norm, "grad_norm_sq_kernel")]
 
 

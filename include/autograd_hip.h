@@ -345,6 +345,26 @@ int agrad_adamw_step(agrad_ctx* ctx, int grad_dtype, float* p, const void* g, fl
                      float b2, float one_minus_b2, float eps, float step_lr, float inv_sqrt_bc2,
                      float grad_scale);
 
+/* One AdamW step with 8-bit moments (adamw8bit_step, metal_ops.metal:10229-10361;
+ * Backend.adamw8bit_step, backend.py:5142-5151; optimizer.py:143-232, 469-479).
+ * qm / qv hold one byte per element: an index into the 256-entry sorted maps qmap_m
+ * (values in [-1, 1]) and qmap_v ([0, 1]); absmax_m / absmax_v hold one fp32 scale per
+ * block of 256 elements ((numel + 255) / 256 of them).  Per element, each operation
+ * rounded once, in the Metal kernel's order:
+ *     m = absmax_m[blk] * qmap_m[qm], v = absmax_v[blk] * qmap_v[qv]     (both 0 when first_step)
+ *     g *= clip_coef;  p *= decay                     (decay on elements [0, decay_numel) only)
+ *     m += (g - m) * (1 - b1);  v += (g*g - v) * (1 - b2)
+ *     p += -(m / (sqrt(max(v, 0)) * inv_sqrt_bc2 + eps)) * lr_bc1
+ * then absmax_m[blk] = max(max |m|, 1e-30), absmax_v[blk] = max(max v, 1e-30) over the
+ * block, and qm / qv = the index of the map entry nearest to m / absmax_m and to
+ * max(v, 0) / absmax_v (bisection for the first entry not below, then the nearer of it
+ * and the entry below; a tie takes the lower).  The caller passes decay = 1 - lr *
+ * weight_decay and lr_bc1 = lr / (1 - b1^t).  The gradient is fp32 or bf16. */
+int agrad_adamw8bit_step(agrad_ctx* ctx, int grad_dtype, float* p, const void* g, uint8_t* qm, uint8_t* qv,
+                         float* absmax_m, float* absmax_v, const float* qmap_m, const float* qmap_v,
+                         uint64_t numel, uint64_t decay_numel, float decay, float lr_bc1, float b1, float b2,
+                         float eps, float inv_sqrt_bc2, float clip_coef, int first_step);
+
 /* partial[i] = sum of squares of g[256 i .. 256 i + 255] for i < agrad_grad_norm_groups(numel);
  * the caller adds the partials in double precision and takes the square root
  * (grad_norm_sq, metal_ops.metal:10103-10137; Backend.grad_norm_sq,

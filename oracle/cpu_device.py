@@ -457,6 +457,21 @@ class CPUBackend(Backend):
             K.adamw_step_split(p, g, m, v, lr * weight_decay if weight_decay > 0.0 else 0.0, b1, b2, eps,
                                lr_t if lr_bc1 is None else lr_bc1, inv_sqrt_bc2, grad_scale, dn)
 
+    def storage_from_host(self, storage, host_np):
+        storage.data.reshape(-1)[:] = np.asarray(host_np, dtype=storage.data.dtype).reshape(-1)
+
+    # the Metal backend's signature (backend.py:5142-5143) over the numpy restatement of its kernel
+    def adamw8bit_step(self, p, g, qm, qv, absmax_m, absmax_v, qmap_m, qmap_v,
+                       lr, lr_bc1, inv_sqrt_bc2, b1, b2, eps, weight_decay, numel, decay_numel, first_step, grad_scale=1.0):
+        gv = g.data
+        if gv.dtype == np.uint16:
+            gv = K.bf16_bits_to_f32(gv)
+        n = int(numel)
+        K.adamw8bit_step(p.data.reshape(-1)[:n], gv.reshape(-1)[:n], qm.data.reshape(-1)[:n], qv.data.reshape(-1)[:n],
+                         absmax_m.data.reshape(-1), absmax_v.data.reshape(-1), qmap_m.data, qmap_v.data,
+                         np.float32(1.0 - float(lr) * float(weight_decay)), lr_bc1, b1, b2, eps, int(decay_numel),
+                         bool(first_step), inv_sqrt_bc2, clip_coef=grad_scale)
+
     def grad_norm_sq(self, g_storage, partial, numel):
         g = g_storage.data
         if g.dtype == np.uint16:

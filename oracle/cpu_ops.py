@@ -26,9 +26,14 @@ Pinning (what shows these functions are the right functions; tests/test_oracle.p
     of the mul gradient, finite differences, rows of a softmax sum to one.
   * bias_gelu: the float64 closed form of GELU at h + b, finite differences in h and in b,
     an explicit row loop for the bias gradient.
+  * adamw8bit: the maps against their defining properties (256 sorted values, extremes
+    -1 / 0 / 1, seven decades), nearest_code against a brute-force argmin over all 256
+    entries, and several steps against fp32-moment AdamW within the quantisation bound.
   * adamw: the textbook bias-corrected recurrence in float64 over several steps;
     the first step from zero moments moves every weight by lr * sign(g).
 Parity unpinned by the reference:
+  * adamw8bit_step -- the reference runs it on its GPU only and keeps no vectors for
+    it; pinned by the properties above, not by reference outputs.
   * relu2_* -- the reference has no ReLU^2; pinned by its closed form only.
   * d(gamma), d(beta) at large row counts -- numpy sums rows sequentially in
     fp32 (backend.py:461,466); the value is pinned, its rounding noise (~1e-4
@@ -534,6 +539,93 @@ def adamw_step_split(p, g, m, v, lr_wd, b1, b2, eps, step_lr, inv_sqrt_bc2, grad
     np.divide(m, tmp, out=tmp)
     np.multiply(tmp, step_lr, out=tmp)
     np.subtract(p, tmp, out=p)
+
+
+# --------------------------------------------------------------------------
+# AdamW with 8-bit moments  (adamw8bit_step, metal_ops.metal:10229-10361; the
+# maps of optimizer.py:144-179).  The reference has this path on its GPU only:
+# what follows restates that kernel, one numpy call per rounded operation.
+# --------------------------------------------------------------------------
+def dynamic_map(signed, max_exponent_bits=7, total_bits=8):
+    """The 256 sorted code values of bitsandbytes' "dynamic" 8-bit format as the
+    reference builds them (optimizer.py:144-179): for each of 7 decades a linear
+    run of bin centres whose length doubles per decade, one finer run below the
+    last decade, zero, sorted and scaled so that the largest magnitude is 1."""
+    non_sign_bits = total_bits - 1 if signed else total_bits
+    additional_items = 2 ** (non_sign_bits - max_exponent_bits) - 1
+    values = []
+    for exponent in range(max_exponent_bits):
+        fraction_items = 2 ** (exponent + non_sign_bits - max_exponent_bits) + 1
+        boundaries = np.linspace(0.1, 1.0, fraction_items, dtype=F32)
+        means = (boundaries[:-1] + boundaries[1:]) * F32(0.5)
+        scaled = means * F32(10.0 ** (exponent - (max_exponent_bits - 1)))
+        values.extend(scaled.tolist())
+        if signed:
+            values.extend((-scaled).tolist())
+    if additional_items > 0:
+        boundaries = np.linspace(0.0, 0.1, additional_items + 1, dtype=F32)
+        means = (boundaries[:-1] + boundaries[1:]) * F32(0.5)
+        scaled = means * F32(10.0 ** (-(max_exponent_bits - 1)))
+        values.extend(scaled.tolist())
+        if signed:
+            values.extend((-scaled).tolist())
+    values.append(0.0)
+    while len(values) < (1 << total_bits):      # the signed map has two zero codes
+        values.append(0.0)
+    if len(values) != (1 << total_bits):
+        raise RuntimeError(f"invalid dynamic-map size: {len(values)}")
+    qmap = np.asarray(values, dtype=F32)
+    qmap.sort()
+    qmap /= np.max(np.abs(qmap))
+    return np.ascontiguousarray(qmap, dtype=F32)
+
+
+def nearest_code(qmap, x):
+    """metal_ops.metal:10326-10343: the first entry not below x (bisection over the
+    sorted map, never past the last entry), then the nearer of it and the entry below;
+    a tie takes the lower"""
+    upper = np.minimum(np.searchsorted(qmap, x, side="left"), 255)
+    lower = np.where(upper > 0, upper - 1, 0)
+    take_upper = np.abs(qmap[upper] - x) < np.abs(qmap[lower] - x)
+    return np.where(take_upper, upper, lower).astype(np.uint8)
+
+
+def adamw8bit_step(p, g, qm, qv, absmax_m, absmax_v, qmap_m, qmap_v, decay, lr_bc1, b1, b2, eps,
+                   decay_numel, first_step, inv_sqrt_bc2, clip_coef=1.0):
+    """In place on p (fp32), qm, qv (uint8), absmax_m, absmax_v (fp32, one per block
+    of 256); g (fp32 values) is read.  Scalars are rounded to fp32 first, as kernel
+    arguments are."""
+    decay, lr_bc1, b1, b2, eps, inv_sqrt_bc2, clip_coef = (F32(x) for x in (decay, lr_bc1, b1, b2, eps, inv_sqrt_bc2, clip_coef))
+    n = p.size
+    flat_p = p.reshape(-1)
+    blk = np.arange(n) // 256
+    if first_step:
+        m = np.zeros(n, F32)
+        v = np.zeros(n, F32)
+    else:
+        m = np.multiply(absmax_m[blk], qmap_m[qm.reshape(-1)], dtype=F32)
+        v = np.multiply(absmax_v[blk], qmap_v[qv.reshape(-1)], dtype=F32)
+    gv = np.multiply(np.asarray(g, F32).reshape(-1), clip_coef, dtype=F32)
+    factor = np.where(np.arange(n) < decay_numel, decay, F32(1.0)).astype(F32)
+    pv = np.multiply(flat_p, factor, dtype=F32)
+    dm = np.multiply(np.subtract(gv, m, dtype=F32), F32(1.0) - b1, dtype=F32)
+    m = np.add(m, dm, dtype=F32)
+    dv = np.multiply(np.subtract(np.multiply(gv, gv, dtype=F32), v, dtype=F32), F32(1.0) - b2, dtype=F32)
+    v = np.add(v, dv, dtype=F32)
+    denom = np.add(np.multiply(np.sqrt(np.maximum(v, F32(0.0)), dtype=F32), inv_sqrt_bc2, dtype=F32), eps, dtype=F32)
+    dp = np.multiply(np.negative(np.divide(m, denom, dtype=F32)), lr_bc1, dtype=F32)
+    flat_p[:] = np.add(pv, dp, dtype=F32)
+    nblocks = (n + 255) // 256
+    top_m = np.zeros(nblocks, F32)
+    top_v = np.zeros(nblocks, F32)
+    np.maximum.at(top_m, blk, np.abs(m))
+    np.maximum.at(top_v, blk, np.maximum(v, F32(0.0)))
+    absmax_m[:] = np.maximum(top_m, F32(1.0e-30))
+    absmax_v[:] = np.maximum(top_v, F32(1.0e-30))
+    mn = np.clip(np.divide(m, absmax_m[blk], dtype=F32), F32(-1.0), F32(1.0))
+    vn = np.clip(np.divide(np.maximum(v, F32(0.0)), absmax_v[blk], dtype=F32), F32(0.0), F32(1.0))
+    qm.reshape(-1)[:] = nearest_code(qmap_m, mn)
+    qv.reshape(-1)[:] = nearest_code(qmap_v, vn)
 
 
 def grad_norm_partials(g):

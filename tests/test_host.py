@@ -51,7 +51,7 @@ def test_header_compiles_as_plain_c(tmp_path):
 
 def test_library_reports_errors_without_gpu_or_kernel():
     lib = capi.load_library()
-    assert lib.agrad_kernel_count() == 40
+    assert lib.agrad_kernel_count() == 41
     names = [lib.agrad_kernel_name(i).decode() for i in range(lib.agrad_kernel_count())]
     for n in ("layernorm_forward", "layernorm_backward_kernel", "rmsnorm_forward", "rmsnorm_backward",
               "gelu_forward_kernel", "gelu_backward_kernel", "swiglu_forward_kernel", "rope_qk_inplace",
@@ -407,7 +407,7 @@ def test_adamw_host_logic_on_oracle_device():
     with pytest.raises(ValueError):
         AdamW([w], state_mode="4bit", runtime=rt)
     with pytest.raises(NotImplementedError):
-        AdamW([w], state_mode="8bit", runtime=rt)
+        AdamW([w], state_mode="mini", runtime=rt)
     lr, betas, eps, wd = 1e-2, (0.9, 0.95), 1e-8, 0.1
     opt = AdamW([w, g, b, ids], lr=lr, betas=betas, eps=eps, weight_decay=wd, runtime=rt)
     assert len(opt.params) == 3                       # ids needs no gradient
@@ -429,3 +429,43 @@ def test_adamw_host_logic_on_oracle_device():
     assert opt.t == 2
     opt.zero_grad()
     assert not rt.backend.copy_to_host(w.grad).any()
+
+
+def test_adamw_8bit_state_on_the_oracle_device():
+    """AdamW(state_mode="8bit") drives the oracle device through the same calls as the hip
+    one: large parameters get byte moments and per-block scales, small ones fp32 moments
+    (optimizer.py:205-222); its code books are the reference's; "mini" is refused"""
+    from autograd_amd.optimizer import AdamW, build_dynamic_map
+    from oracle import cpu_ops as K
+    for signed in (True, False):
+        np.testing.assert_array_equal(build_dynamic_map(signed), K.dynamic_map(signed))
+    rng = np.random.default_rng(21)
+    V, C = 80, 64
+    w = T((V, C), val=rng.standard_normal((V, C)).astype(np.float32))
+    g = T((C,), val=np.ones(C, np.float32))
+    ids = Tensor(shape=(2, 9), dtype=np.int32, device="cpu", requires_grad=False,
+                 init_val=rng.integers(0, V, (2, 9), dtype=np.int32))
+    out = ids.gather(w).rms_norm(g)
+    rt = Runtime(device="cpu")
+    rt.loss = out
+    rt.build_topo(out)
+    rt.bind_memory()
+    opt = AdamW([w, g], lr=1e-2, weight_decay=0.1, runtime=rt, state_mode="8bit")
+    assert [d[0] for d in opt.dispatches] == ["q8", "fp32"]
+    assert opt.m[0].data.dtype == np.uint8 and opt.m[0].data.size == V * C and opt.dispatches[0][5].data.size == V * C // 256
+    before = rt.backend.copy_to_host(w).copy()
+    up = rng.standard_normal((2, 9, C)).astype(np.float32)
+    for _ in range(2):
+        rt.forward()
+        rt.zero_grad()
+        rt.backend.copy_from_host(out.grad, up)
+        rt.backward_graph()
+        opt.step()
+    after = rt.backend.copy_to_host(w)
+    touched = np.unique(rt.backend.copy_to_host(ids))
+    moved = np.abs(after - before * np.float32(1 - 1e-2 * 0.1) ** 2).max(axis=1)
+    assert (moved[touched] > 5e-3).all()                       # rows with a gradient took Adam-sized steps
+    rest = np.setdiff1d(np.arange(V), touched)
+    assert (moved[rest] < 1e-6).all()                          # the others only decayed
+    with pytest.raises(NotImplementedError):
+        AdamW([w, g], runtime=rt, state_mode="mini")

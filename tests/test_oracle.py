@@ -410,6 +410,79 @@ def test_adamw_first_step_is_lr_times_sign_and_matches_textbook():
     assert not m.any() and not v.any()
 
 
+def test_dynamic_maps_have_the_defining_shape():
+    """optimizer.py:144-179: 256 sorted values; the signed map is symmetric with two zero
+    codes and extremes -1 / +1, the unsigned one starts at 0, ends at 1 and is strictly
+    increasing; seven decades: the smallest non-zero magnitude is a few 1e-7"""
+    sm, um = K.dynamic_map(True), K.dynamic_map(False)
+    for q in (sm, um):
+        assert q.shape == (256,) and q.dtype == np.float32 and (np.diff(q) >= 0).all()
+    assert sm[0] == -1 and sm[-1] == 1 and (sm == 0).sum() == 2
+    np.testing.assert_array_equal(sm, -sm[::-1])
+    assert um[0] == 0 and um[-1] == 1 and (np.diff(um) > 0).all()
+    assert 1e-7 < np.abs(sm[sm != 0]).min() < 1e-6 and 1e-8 < um[1] < 1e-6
+    # each decade of the signed map holds twice the codes of the decade below
+    pos = sm[sm > 0]
+    counts = [int(((pos > 10.0 ** -(k + 1)) & (pos <= 10.0 ** -k)).sum()) for k in range(6)]
+    assert all(a >= 1.6 * b for a, b in zip(counts, counts[1:])), counts
+
+
+def test_nearest_code_is_the_nearest_entry_and_ties_go_down():
+    r = rng(51)
+    for q, lo in ((K.dynamic_map(True), -1.0), (K.dynamic_map(False), 0.0)):
+        x = np.concatenate([r.uniform(lo, 1.0, 4000), r.uniform(-1, 1, 500) * 1e-4, q, [lo, 1.0, 0.0]]).astype(np.float32)
+        x = np.clip(x, lo, 1.0)
+        code = K.nearest_code(q, x)
+        brute = np.abs(q[None, :].astype(np.float64) - x[:, None].astype(np.float64)).min(axis=1)
+        got = np.abs(q[code].astype(np.float64) - x.astype(np.float64))
+        # distances are compared as the kernel forms them, in fp32
+        np.testing.assert_array_equal(np.abs(q[code] - x), np.abs(q[None, :] - x[:, None]).min(axis=1))
+        assert (got <= brute + 1e-9).all()
+        np.testing.assert_array_equal(q[K.nearest_code(q, q)], q)       # a map value is its own code's value
+    q = K.dynamic_map(False)
+    mid = ((q[200].astype(np.float64) + q[201]) / 2).astype(np.float32)
+    if np.abs(q[201] - mid) == np.abs(q[200] - mid):                      # an exact tie in fp32
+        assert K.nearest_code(q, np.array([mid]))[0] == 200
+    assert K.nearest_code(q, np.array([np.nextafter(q[255], 0, dtype=np.float32)]))[0] in (254, 255)
+
+
+def test_adamw8bit_tracks_fp32_adamw_within_the_quantisation_error():
+    """Five steps of the 8-bit update beside the same update with fp32 moments
+    (adamw_step_split with the Metal scalars): the first step is identical in p
+    (both start from zero moments), later ones differ by what quantising m and v to
+    the map costs -- a few percent of a step -- and the stored moments decode to the
+    fp32 ones within the map's resolution.  Weight decay reaches the prefix only."""
+    import math
+    lr, b1, b2, eps, wd = 1e-3, 0.9, 0.95, 1e-8, 0.1
+    n, decay_n = 1000, 600
+    r = rng(52)
+    p0 = r.standard_normal(n).astype(np.float32)
+    grads = [r.standard_normal(n).astype(np.float32) for _ in range(5)]
+    qm_map, qv_map = K.dynamic_map(True), K.dynamic_map(False)
+    p8 = p0.copy()
+    qm, qv = np.zeros(n, np.uint8), np.zeros(n, np.uint8)
+    am, av = np.zeros(4, np.float32), np.zeros(4, np.float32)
+    p32, m32, v32 = p0.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    for t, g in enumerate(grads, 1):
+        lr_bc1 = lr / (1.0 - b1 ** t)
+        inv_sqrt_bc2 = 1.0 / math.sqrt(1.0 - b2 ** t)
+        K.adamw8bit_step(p8, g, qm, qv, am, av, qm_map, qv_map, 1.0 - lr * wd, lr_bc1, b1, b2, eps, decay_n, t == 1,
+                         inv_sqrt_bc2, clip_coef=0.5)
+        K.adamw_step_split(p32, g, m32, v32, lr * wd, b1, b2, eps, lr_bc1, inv_sqrt_bc2, 0.5, decay_numel=decay_n)
+        if t == 1:
+            np.testing.assert_allclose(p8, p32, rtol=0, atol=6e-7)      # the two spell the same update differently: an ulp or two
+            # the first step moves every weight by lr * sign(g) (after the decay factor)
+            moved = p8 - p0 * np.where(np.arange(n) < decay_n, np.float32(1.0 - lr * wd), np.float32(1.0))
+            np.testing.assert_allclose(moved, -lr * np.sign(g), rtol=1e-3, atol=1e-8)
+        blk = np.arange(n) // 256
+        m_dec, v_dec = am[blk] * qm_map[qm], av[blk] * qv_map[qv]
+        assert np.abs(m_dec - m32).max() <= 0.03 * am.max() * t       # errors of earlier steps carry over, damped by b1
+        assert np.abs(v_dec - v32).max() <= 0.03 * av.max() * t
+        np.testing.assert_array_equal(am, [np.abs(m_dec[blk == b]).max() for b in range(4)])   # the block maximum is a code value 1
+    assert np.abs(p8 - p32).max() < 0.25 * 5 * lr
+    assert np.abs(p8[decay_n:] - p0[decay_n:]).max() <= 5.5 * lr       # no decay outside the prefix: only Adam-sized moves
+
+
 def test_adamw_split_form_is_the_same_update():
     import math
     lr, b1, b2, eps, wd = 3e-4, 0.9, 0.95, 1e-8, 0.05
