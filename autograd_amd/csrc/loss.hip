@@ -38,6 +38,17 @@ constexpr int kCeBwdUnroll = AGRAD_CE_BWD_UNROLL;   // backward (read + write)
 template <typename T> __device__ __forceinline__ float exp_io(float x) { return exp_compensated(x); }
 template <> __device__ __forceinline__ float exp_io<bf16_t>(float x) { return __builtin_amdgcn_exp2f(x * kLog2eHi); }
 
+// The softmax quotient e / sum by I/O type, from `scale = row_scale<T>(sum)`.  fp32
+// tensors divide, as the CPU does.  bf16 tensors multiply by the reciprocal of the sum
+// (one correctly rounded division per row): a division per element is ten instructions
+// of the twenty the bf16 kernel spent per element -- it issued vector instructions for
+// 78 % of its run time -- and the two differ by an ulp of fp32, gone in the rounding to
+// eight bits.
+template <typename T> __device__ __forceinline__ float row_scale(float sum) { return sum; }
+template <> __device__ __forceinline__ float row_scale<bf16_t>(float sum) { return 1.0f / sum; }
+template <typename T> __device__ __forceinline__ float quotient_io(float e, float scale) { return e / scale; }
+template <> __device__ __forceinline__ float quotient_io<bf16_t>(float e, float scale) { return e * scale; }
+
 // running (maximum, sum of exp(x - maximum))
 struct MaxSum {
     float m, s;
@@ -365,12 +376,13 @@ softmax_fwd_kernel(const T* __restrict__ x, T* __restrict__ y, uint32_t V) {
             const uint32_t e = threadIdx.x < sp.head ? threadIdx.x : sp.tail_start + (threadIdx.x - sp.head);
             float v[1];
             VecIO<T, 1>::load(base + e, v);
-            v[0] = exp_io<T>(v[0] - t.m) / t.s;
+            v[0] = quotient_io<T>(exp_io<T>(v[0] - t.m), row_scale<T>(t.s));
             VecIO<T, 1>::store(out + e, v);
         }
     }
     const T* body = base + sp.head;
     T* obody = out + sp.head;
+    const float scale = row_scale<T>(t.s);
     for (uint32_t i0 = threadIdx.x; i0 < sp.nvec; i0 += BLOCK * kCeBwdUnroll) {
         float v[kCeBwdUnroll][VEC];
 #pragma unroll
@@ -383,7 +395,7 @@ softmax_fwd_kernel(const T* __restrict__ x, T* __restrict__ y, uint32_t V) {
             const uint32_t i = i0 + u * BLOCK;
             if (i < sp.nvec) {
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) v[u][k] = exp_io<T>(v[u][k] - t.m) / t.s;
+                for (int k = 0; k < VEC; ++k) v[u][k] = quotient_io<T>(exp_io<T>(v[u][k] - t.m), scale);
                 VecIO<T, VEC>::store(obody + (uint64_t)i * VEC, v[u]);
             }
         }
@@ -524,12 +536,13 @@ softmax_fwd_reg_kernel(const T* __restrict__ x, T* __restrict__ y, uint32_t V, u
     }
 #pragma unroll
     for (int off = 1; off < kWave; off <<= 1) sum = sum + __shfl_xor(sum, off);
+    const float scale = row_scale<T>(sum);
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const uint32_t c = i * kWave + threadIdx.x;
         if (c < VV) {
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) v[i][k] = v[i][k] / sum;
+            for (int k = 0; k < VEC; ++k) v[i][k] = quotient_io<T>(v[i][k], scale);
             VecIO<T, VEC>::store(out + (uint64_t)c * VEC, v[i]);
         }
     }
