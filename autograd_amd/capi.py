@@ -69,6 +69,7 @@ SIGNATURES = {
     "agrad_relu2_forward": (_int, [_ctx, _int, _ptr, _ptr, _u64]),
     "agrad_relu2_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _u64, _u32]),
     "agrad_swiglu_forward": (_int, [_ctx, _int, _ptr, _ptr, _u64, _u32]),
+    "agrad_swiglu_forward_tile": (_int, [_ctx, _int, _ptr, _ptr, _u64, _u32, _u32, _u32]),
     "agrad_swiglu_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _u64, _u32, _u32]),
     "agrad_rope_qk": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u32, _u32, _u32, _u32, _u32, _int, _int]),
     "agrad_gather_forward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u32, _u32, _u32]),

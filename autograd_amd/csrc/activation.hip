@@ -54,10 +54,13 @@ template <> __device__ __forceinline__ float sigmoid_io<bf16_t>(float g) {
     return __builtin_amdgcn_rcpf(1.0f + e);
 }
 
-// gu[rows, 2H] -> h[rows, H]; a "vector" is VEC consecutive columns of one row.
+// gu[rows, 2H] -> h[rows, HV * VEC]: columns h0 ... h0 + HV * VEC - 1 of the gate and up
+// halves, written densely (the whole width when h0 = 0 and HV * VEC = H; a column tile
+// otherwise: swiglu_forward_tile_kernel, metal_ops.metal:12043-12088).  A "vector" is VEC
+// consecutive columns of one row.
 template <typename T, int VEC, int UNROLL>
 __global__ void __launch_bounds__(kEwBlock)
-swiglu_fwd_kernel(const T* __restrict__ gu, T* __restrict__ h, uint32_t H, uint32_t HV, uint32_t nvec) {
+swiglu_fwd_kernel(const T* __restrict__ gu, T* __restrict__ h, uint32_t H, uint32_t h0, uint32_t HV, uint32_t nvec) {
     const uint32_t first = blockIdx.x * (kEwBlock * UNROLL) + threadIdx.x;
     float g[UNROLL][VEC], u[UNROLL][VEC];
     uint64_t off_out[UNROLL];
@@ -67,8 +70,8 @@ swiglu_fwd_kernel(const T* __restrict__ gu, T* __restrict__ h, uint32_t H, uint3
         if (idx < nvec) {
             const uint32_t row = idx / HV;
             const uint32_t col = (idx - row * HV) * VEC;
-            const uint64_t off_in = (uint64_t)row * 2 * H + col;
-            off_out[j] = (uint64_t)row * H + col;
+            const uint64_t off_in = (uint64_t)row * 2 * H + h0 + col;
+            off_out[j] = (uint64_t)row * HV * VEC + col;
             VecIO<T, VEC>::load(gu + off_in, g[j]);
             VecIO<T, VEC>::load(gu + off_in + H, u[j]);
         }
@@ -143,9 +146,10 @@ swiglu_bwd_kernel(const T* gu, const T* __restrict__ dh, T* dgu, uint32_t H, uin
 // Rows are processed in slabs small enough for 32-bit vector indices.
 template <typename T, int VEC>
 int swiglu_typed(hipStream_t s, const T* gu, const T* dh, T* out, uint64_t rows, uint32_t H,
-                 bool backward, int acc) {
+                 bool backward, int acc, uint32_t h0 = 0, uint32_t hw = 0) {
     constexpr int UNROLL = 1;
-    const uint32_t HV = H / VEC;
+    if (hw == 0) hw = H;                       // forward only: the column tile [h0, h0 + hw)
+    const uint32_t HV = hw / VEC;
     const uint64_t max_rows = 0xf0000000ull / HV;
     for (uint64_t r0 = 0; r0 < rows; r0 += max_rows) {
         const uint64_t nr = rows - r0 < max_rows ? rows - r0 : max_rows;
@@ -154,7 +158,7 @@ int swiglu_typed(hipStream_t s, const T* gu, const T* dh, T* out, uint64_t rows,
         const uint32_t grid = (nvec + per_block - 1) / per_block;
         if (!backward) {
             hipLaunchKernelGGL((swiglu_fwd_kernel<T, VEC, UNROLL>), dim3(grid), dim3(kEwBlock), 0, s,
-                               gu + r0 * 2 * H, out + r0 * H, H, HV, nvec);
+                               gu + r0 * 2 * H, out + r0 * hw, H, h0, HV, nvec);
         } else {
             hipLaunchKernelGGL((swiglu_bwd_kernel<T, VEC, UNROLL>), dim3(grid), dim3(kEwBlock), 0, s,
                                gu + r0 * 2 * H, dh + r0 * H, out + r0 * 2 * H, H, HV, nvec, acc);
@@ -170,6 +174,14 @@ int swiglu_dispatch(hipStream_t s, const void* gu, const void* dh, void* out, ui
     const bool wide = H % VEC == 0 && aligned16(gu) && aligned16(out) && (!dh || aligned16(dh));
     if (wide) return swiglu_typed<T, VEC>(s, (const T*)gu, (const T*)dh, (T*)out, rows, H, backward, acc);
     return swiglu_typed<T, 1>(s, (const T*)gu, (const T*)dh, (T*)out, rows, H, backward, acc);
+}
+
+template <typename T>
+int swiglu_tile_dispatch(hipStream_t s, const void* gu, void* out, uint64_t rows, uint32_t H, uint32_t h0, uint32_t hw) {
+    constexpr int VEC = WideVec<T>::value;
+    const bool wide = H % VEC == 0 && h0 % VEC == 0 && hw % VEC == 0 && aligned16(gu) && aligned16(out);
+    if (wide) return swiglu_typed<T, VEC>(s, (const T*)gu, nullptr, (T*)out, rows, H, false, 0, h0, hw);
+    return swiglu_typed<T, 1>(s, (const T*)gu, nullptr, (T*)out, rows, H, false, 0, h0, hw);
 }
 
 }  // namespace
@@ -197,6 +209,16 @@ int launch_swiglu_fwd(hipStream_t s, int dtype, const void* gu, void* h, uint64_
     if (dtype == AGRAD_F32) return swiglu_dispatch<float>(s, gu, nullptr, h, rows, H, false, 0);
     if (dtype == AGRAD_BF16) return swiglu_dispatch<bf16_t>(s, gu, nullptr, h, rows, H, false, 0);
     return set_error(AGRAD_EINVAL, "swiglu forward: unknown dtype %d", dtype);
+}
+
+int launch_swiglu_fwd_tile(hipStream_t s, int dtype, const void* gu, void* tile, uint64_t rows, uint32_t H,
+                           uint32_t h0, uint32_t hw) {
+    if ((uint64_t)h0 + hw > H) return set_error(AGRAD_EINVAL, "swiglu tile: columns %u..%u of %u", h0, h0 + hw, H);
+    if (rows == 0 || hw == 0) return AGRAD_OK;
+    if (gu == nullptr || tile == nullptr) return set_error(AGRAD_EINVAL, "swiglu tile: null operand");
+    if (dtype == AGRAD_F32) return swiglu_tile_dispatch<float>(s, gu, tile, rows, H, h0, hw);
+    if (dtype == AGRAD_BF16) return swiglu_tile_dispatch<bf16_t>(s, gu, tile, rows, H, h0, hw);
+    return set_error(AGRAD_EINVAL, "swiglu tile: unknown dtype %d", dtype);
 }
 
 int launch_swiglu_bwd(hipStream_t s, int dtype, const void* gu, const void* dh, void* dgu,

@@ -333,6 +333,13 @@ int h_swiglu_fwd(const Call& c) {
     RESOLVE(0, 2 * hb, gu) RESOLVE(1, hb, h)
     return launch_swiglu_fwd(c.ctx->stream, c.a[0], gu, h, rows, c.a[2]);
 }
+// buffers gu, hidden_tile | args dtype, then the reference's N, H, h0, h (backend.py:3910-3913)
+int h_swiglu_tile(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t rows = c.a[1], es = dtype_size(c.a[0]);
+    RESOLVE(0, rows * 2 * c.a[2] * es, gu) RESOLVE(1, rows * c.a[4] * es, tile)
+    return launch_swiglu_fwd_tile(c.ctx->stream, c.a[0], gu, tile, rows, c.a[2], c.a[3], c.a[4]);
+}
 // buffers gu, dh, dgu | args dtype, rows, H, flags
 int h_swiglu_bwd(const Call& c) {
     NEED_DTYPE(c.a[0])
@@ -488,6 +495,7 @@ const Entry kTable[] = {
     {"relu2_forward_kernel", 2, 3, "x, y | dtype, n_lo, n_hi", h_act_fwd<1>},
     {"relu2_backward_kernel", 3, 4, "dy, x, dx | dtype, flags, n_lo, n_hi", h_act_bwd<1>},
     {"swiglu_forward_kernel", 2, 3, "gu, h | dtype, rows, H", h_swiglu_fwd},
+    {"swiglu_forward_tile_kernel", 2, 5, "gu, hidden_tile | dtype, rows, H, h0, h", h_swiglu_tile},
     {"swiglu_backward_kernel", 3, 4, "gu, dh, dgu | dtype, rows, H, flags", h_swiglu_bwd},
     {"rope_qk_inplace", 4, 9, "q, k, cos, sin | dtype, B, T, H, HKV, D, hf_sign, backward, present_mask", h_rope},
     {"gather_forward_kernel", 3, 4, "ids, W, out | dtype, N, C, V", h_gather_fwd},
@@ -867,6 +875,11 @@ int agrad_relu2_backward(agrad_ctx* ctx, int dtype, const void* x, const void* d
 int agrad_swiglu_forward(agrad_ctx* ctx, int dtype, const void* gu, void* h, uint64_t rows, uint32_t H) {
     CTX_OR_FAIL(ctx)
     return launch_swiglu_fwd(ctx->stream, dtype, gu, h, rows, H);
+}
+int agrad_swiglu_forward_tile(agrad_ctx* ctx, int dtype, const void* gu, void* tile, uint64_t rows, uint32_t H,
+                              uint32_t h0, uint32_t h) {
+    CTX_OR_FAIL(ctx)
+    return launch_swiglu_fwd_tile(ctx->stream, dtype, gu, tile, rows, H, h0, h);
 }
 int agrad_swiglu_backward(agrad_ctx* ctx, int dtype, const void* gu, const void* dh, void* dgu,
                           uint64_t rows, uint32_t H, uint32_t flags) {

@@ -83,6 +83,8 @@ int launch_gelu_bwd(hipStream_t s, int dtype, const void* x, const void* dy, voi
 int launch_relu2_fwd(hipStream_t s, int dtype, const void* x, void* y, uint64_t n);
 int launch_relu2_bwd(hipStream_t s, int dtype, const void* x, const void* dy, void* dx, uint64_t n, uint32_t flags);
 int launch_swiglu_fwd(hipStream_t s, int dtype, const void* gu, void* h, uint64_t rows, uint32_t H);
+int launch_swiglu_fwd_tile(hipStream_t s, int dtype, const void* gu, void* tile, uint64_t rows, uint32_t H,
+                           uint32_t h0, uint32_t hw);
 int launch_swiglu_bwd(hipStream_t s, int dtype, const void* gu, const void* dh, void* dgu,
                       uint64_t rows, uint32_t H, uint32_t flags);
 

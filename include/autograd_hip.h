@@ -245,6 +245,11 @@ int agrad_relu2_backward(agrad_ctx* ctx, int dtype, const void* x, const void* d
  * backend.py:1113-1126, 1178-1217; swiglu_forward_kernel /
  * swiglu_backward_inplace_kernel (metal_ops.metal:3808-4017). */
 int agrad_swiglu_forward(agrad_ctx* ctx, int dtype, const void* gu, void* h, uint64_t rows, uint32_t H);
+/* A column tile of the same forward: tile[r, c] = silu(gu[r, h0 + c]) * gu[r, H + h0 + c] for
+ * c < h, written densely as [rows, h] (swiglu_forward_tile_kernel, metal_ops.metal:12043-12088;
+ * the recompute of the hidden activations in column tiles, backend.py:3906-3913). */
+int agrad_swiglu_forward_tile(agrad_ctx* ctx, int dtype, const void* gu, void* tile, uint64_t rows, uint32_t H,
+                              uint32_t h0, uint32_t h);
 int agrad_swiglu_backward(agrad_ctx* ctx, int dtype, const void* gu, const void* dh, void* dgu,
                           uint64_t rows, uint32_t H, uint32_t flags);
 

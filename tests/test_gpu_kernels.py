@@ -358,6 +358,43 @@ def test_swiglu_bf16_io(ctx):
     assert_bf16_close(from_bf16_bits(G.swiglu_backward(ctx, gub, dhb)), ref.swiglu_backward(gu, dh), "bf16 swiglu bwd")
 
 
+@pytest.mark.parametrize("rows,H,h0,h", [(7, 64, 0, 64), (7, 64, 16, 32), (33, 200, 8, 100), (5, 96, 3, 50),
+                                        (2, 8960, 2048, 2048), (3, 10, 9, 1), (4, 40, 40, 0)])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_swiglu_forward_column_tile(ctx, rows, H, h0, h, dtype):
+    """agrad_swiglu_forward_tile (swiglu_forward_tile_kernel, metal_ops.metal:12043-12088):
+    columns h0 .. h0 + h of the hidden activations, dense [rows, h] -- the very bits of
+    those columns of the full forward call (aligned tiles take the 16-byte path, odd
+    offsets and widths the element-wise one), and within tolerance of the CPU kernel"""
+    import ctypes as Ct
+    rng = _rng(15 + h0)
+    gu = (2 * rng.standard_normal((rows, 2 * H))).astype(np.float32)
+    if dtype == "bf16":
+        store = to_bf16_bits(gu)
+        seen = from_bf16_bits(store)
+        dt = capi.BF16
+    else:
+        store, seen, dt = gu, gu, capi.F32
+    full = G.swiglu_forward(ctx, store)
+    d_gu = ctx.upload(store)
+    tile = ctx.upload(np.full((rows, max(h, 1)), 0x7F7F if dtype == "bf16" else 7.0, store.dtype))
+    ctx.call("agrad_swiglu_forward_tile", dt, Ct.c_void_p(d_gu.ptr), Ct.c_void_p(tile.ptr), rows, H, h0, h)
+    ctx.synchronize()
+    got = tile.download()
+    if h:
+        got = got.reshape(-1)[:rows * h].reshape(rows, h)
+        np.testing.assert_array_equal(got, full[:, h0:h0 + h])
+        want = ref.swiglu_forward(seen)[:, h0:h0 + h]
+        if dtype == "bf16":
+            assert_bf16_close(from_bf16_bits(got), want, "swiglu tile")
+        else:
+            assert_fp32_close(got, want, "swiglu tile")
+    with pytest.raises(capi.AgradError):       # the tile must lie inside the row
+        ctx.call("agrad_swiglu_forward_tile", dt, Ct.c_void_p(d_gu.ptr), Ct.c_void_p(tile.ptr), rows, H, H - 1, 2)
+    d_gu.free()
+    tile.free()
+
+
 # ---------------------------------------------------------------------------
 # RoPE
 # ---------------------------------------------------------------------------
