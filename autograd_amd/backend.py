@@ -663,10 +663,15 @@ class HipBackend(Backend):
                             second.grad if second is not None else None, op.eps, flags, scratch)
 
     # -- rotary (backend.py:1382-1417, 1755-1782, 1937-1958) ----------------------------
-    def _rope(self, q, k, cos, sin, sign, backward):
-        B, T, H, D = q.shape
-        HKV = k.shape[2] if k is not None else 0
-        self._launch("rope_qk_inplace", [q, k, cos, sin],
+    def _rope(self, q, k, cos, sin, sign, backward, layout="bthd"):
+        """q (and k, if given) rotated in place; shapes are [B,T,heads,D], or [B,heads,T,D] for layout 'bhtd'"""
+        if layout == "bhtd":
+            B, H, T, D = q.shape
+            HKV = k.shape[1] if k is not None else 0
+        else:
+            B, T, H, D = q.shape
+            HKV = k.shape[2] if k is not None else 0
+        self._launch("rope_qk_inplace_bhtd" if layout == "bhtd" else "rope_qk_inplace", [q, k, cos, sin],
                      [_dt(q), B, T, H, HKV, D, 1 if sign == 1 else 0, 1 if backward else 0, _mask(q, k)])
 
     @staticmethod
@@ -682,7 +687,7 @@ class HipBackend(Backend):
         for a, b in ((q, q2), (k, k2)):
             if not self._same_memory(a, b):
                 self._launch("copy_kernel", [a, b], _lo_hi(b.storage.nbytes))
-        self._rope(q2, k2, cos, sin, q2.op.op.rope_sign, False)
+        self._rope(q2, k2, cos, sin, q2.op.op.rope_sign, False, q2.op.op.layout)
 
     def hip_rope_backward(self, inputs, outputs, scratch=None):
         q, k, cos, sin = inputs
@@ -691,13 +696,11 @@ class HipBackend(Backend):
         gk = k2.grad if k.requires_grad else None
         if gq is None and gk is None:
             return
-        sign = q2.op.op.rope_sign
+        sign, layout = q2.op.op.rope_sign, q2.op.op.layout
         if gq is not None:
-            self._rope(gq, gk, cos, sin, sign, True)
+            self._rope(gq, gk, cos, sin, sign, True, layout)
         else:
-            B, T, H, D = gk.shape
-            self._launch("rope_qk_inplace", [gk, None, cos, sin],
-                         [_dt(gk), B, T, H, 0, D, 1 if sign == 1 else 0, 1, _mask(gk, None)])
+            self._rope(gk, None, cos, sin, sign, True, layout)      # k alone takes q's slot
         node = q2.op
         for src, g in ((q, gq), (k, gk)):
             if g is not None and src.grad is not None and not self._same_memory(src.grad, g):

@@ -72,6 +72,7 @@ SIGNATURES = {
     "agrad_swiglu_forward_tile": (_int, [_ctx, _int, _ptr, _ptr, _u64, _u32, _u32, _u32]),
     "agrad_swiglu_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _u64, _u32, _u32]),
     "agrad_rope_qk": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u32, _u32, _u32, _u32, _u32, _int, _int]),
+    "agrad_rope_qk_bhtd": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u32, _u32, _u32, _u32, _u32, _int, _int]),
     "agrad_gather_forward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u32, _u32, _u32]),
     "agrad_embedding_backward_workspace_bytes": (_u64, [_u64, _u32, _u32, _int]),
     "agrad_embedding_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u64, _u32, _u32, _u32]),

@@ -348,6 +348,7 @@ int h_swiglu_bwd(const Call& c) {
     return launch_swiglu_bwd(c.ctx->stream, c.a[0], gu, dh, dgu, rows, c.a[2], c.a[3]);
 }
 // buffers q, k, cos, sin | args dtype, B, T, H, HKV, D, hf_sign, backward, present
+template <int BHTD>
 int h_rope(const Call& c) {
     NEED_DTYPE(c.a[0])
     const uint32_t B = c.a[1], T = c.a[2], H = c.a[3], HKV = c.a[4], D = c.a[5], present = c.a[8];
@@ -356,7 +357,7 @@ int h_rope(const Call& c) {
     RESOLVE_IF(present & 2u, 1, tok * HKV * D * es, k)
     RESOLVE(2, (uint64_t)T * (D / 2) * 4, cs) RESOLVE(3, (uint64_t)T * (D / 2) * 4, sn)
     return launch_rope(c.ctx->stream, c.a[0], q, k, (const float*)cs, (const float*)sn, B, T, H, HKV, D,
-                       c.a[6] ? 1 : -1, c.a[7] != 0);
+                       c.a[6] ? 1 : -1, c.a[7] != 0, BHTD);
 }
 // buffers ids, W, out | args dtype, N, C, V
 int h_gather_fwd(const Call& c) {
@@ -497,7 +498,8 @@ const Entry kTable[] = {
     {"swiglu_forward_kernel", 2, 3, "gu, h | dtype, rows, H", h_swiglu_fwd},
     {"swiglu_forward_tile_kernel", 2, 5, "gu, hidden_tile | dtype, rows, H, h0, h", h_swiglu_tile},
     {"swiglu_backward_kernel", 3, 4, "gu, dh, dgu | dtype, rows, H, flags", h_swiglu_bwd},
-    {"rope_qk_inplace", 4, 9, "q, k, cos, sin | dtype, B, T, H, HKV, D, hf_sign, backward, present_mask", h_rope},
+    {"rope_qk_inplace", 4, 9, "q, k, cos, sin | dtype, B, T, H, HKV, D, hf_sign, backward, present_mask", h_rope<0>},
+    {"rope_qk_inplace_bhtd", 4, 9, "q, k, cos, sin | dtype, B, T, H, HKV, D, hf_sign, backward, present_mask", h_rope<1>},
     {"gather_forward_kernel", 3, 4, "ids, W, out | dtype, N, C, V", h_gather_fwd},
     {"embedding_sum_forward", 4, 5, "ids, W, wpe, out | dtype, N, T, C, V", h_embed_sum_fwd},
     {"gather_backward_kernel", 4, 7, "ids, dY, dW, workspace | dtype, N, C, V, flags, ws_lo, ws_hi", h_gather_bwd},
@@ -891,6 +893,11 @@ int agrad_rope_qk(agrad_ctx* ctx, int dtype, void* q, void* k, const float* cos_
                   uint32_t B, uint32_t T, uint32_t H, uint32_t HKV, uint32_t D, int rope_sign, int backward) {
     CTX_OR_FAIL(ctx)
     return launch_rope(ctx->stream, dtype, q, k, cos_table, sin_table, B, T, H, HKV, D, rope_sign, backward);
+}
+int agrad_rope_qk_bhtd(agrad_ctx* ctx, int dtype, void* q, void* k, const float* cos_table, const float* sin_table,
+                       uint32_t B, uint32_t T, uint32_t H, uint32_t HKV, uint32_t D, int rope_sign, int backward) {
+    CTX_OR_FAIL(ctx)
+    return launch_rope(ctx->stream, dtype, q, k, cos_table, sin_table, B, T, H, HKV, D, rope_sign, backward, 1);
 }
 
 int agrad_gather_forward(agrad_ctx* ctx, int dtype, const int32_t* ids, const void* W, const void* wpe,

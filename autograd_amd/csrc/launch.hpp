@@ -90,7 +90,7 @@ int launch_swiglu_bwd(hipStream_t s, int dtype, const void* gu, const void* dh, 
 
 // rope.hip
 int launch_rope(hipStream_t s, int dtype, void* q, void* k, const float* cos_t, const float* sin_t,
-                uint32_t B, uint32_t T, uint32_t H, uint32_t HKV, uint32_t D, int sign, int backward);
+                uint32_t B, uint32_t T, uint32_t H, uint32_t HKV, uint32_t D, int sign, int backward, int bhtd = 0);
 
 // embedding.hip
 int launch_gather_fwd(hipStream_t s, int dtype, const int32_t* ids, const void* W, const void* wpe,

@@ -1,5 +1,8 @@
 // Split-half rotary embedding on q[B,T,H,D] and k[B,T,HKV,D], in place, both
 // tensors in one launch.  Tables cos/sin are fp32 [T, D/2] and stay L2-resident.
+// The same for q[B,H,T,D] and k[B,HKV,T,D] (the layout attention works in; the
+// layout flag of rope_qk_inplace / gqa_rope_inplace, metal_ops.metal:7458-7465,
+// 11741): only the mapping from work item to position differs.
 //
 // A work item is one 128-bit vector of the low half of a head together with
 // the matching vector of the high half, so each item is two loads and two
@@ -28,6 +31,8 @@ struct RopeArgs {
     uint32_t I;      // items per token        = (H + HKV)*J
     uint32_t total;  // B*T*I
     float sgn;       // +1 or -1 (already includes the backward flip)
+    uint32_t bhtd;   // 0: [B,T,heads,D]; 1: [B,heads,T,D]
+    uint32_t q_rows; // bhtd: B*H*T rows of D elements belong to q, the rest to k
 };
 
 template <int VEC>
@@ -54,15 +59,25 @@ __global__ void __launch_bounds__(kRopeBlock) rope_kernel(const RopeArgs<T> a) {
         const uint32_t idx = first + u * kRopeBlock;
         ptr[u] = nullptr;
         if (idx < a.total) {
-            const uint32_t token = idx / a.I;
-            uint32_t r = idx - token * a.I;
-            const uint32_t t = token % a.T_len;
-            T* base;
-            uint32_t heads;
-            if (r < a.Iq) { base = a.q; heads = a.H; } else { base = a.k; heads = a.HKV; r -= a.Iq; }
-            const uint32_t head = r / a.J;
-            const uint32_t j = r - head * a.J;
-            ptr[u] = base + ((uint64_t)token * heads + head) * a.D + (uint64_t)j * VEC;
+            uint32_t t, j;
+            if (a.bhtd) {                       // uniform over the launch
+                uint32_t row = idx / a.J;       // a row is one (batch, head, position)
+                j = idx - row * a.J;
+                T* base = a.q;
+                if (row >= a.q_rows) { base = a.k; row -= a.q_rows; }
+                t = row % a.T_len;
+                ptr[u] = base + (uint64_t)row * a.D + (uint64_t)j * VEC;
+            } else {
+                const uint32_t token = idx / a.I;
+                uint32_t r = idx - token * a.I;
+                t = token % a.T_len;
+                T* base;
+                uint32_t heads;
+                if (r < a.Iq) { base = a.q; heads = a.H; } else { base = a.k; heads = a.HKV; r -= a.Iq; }
+                const uint32_t head = r / a.J;
+                j = r - head * a.J;
+                ptr[u] = base + ((uint64_t)token * heads + head) * a.D + (uint64_t)j * VEC;
+            }
             VecIO<T, VEC>::load(ptr[u], lo[u]);
             VecIO<T, VEC>::load(ptr[u] + half, hi[u]);
             const uint32_t tab = t * half + j * VEC;
@@ -99,6 +114,7 @@ int rope_typed(hipStream_t s, RopeArgs<T> a, uint32_t B) {
     const uint64_t total = (uint64_t)B * a.T_len * a.I;
     if (total >= 0xffff0000ull) return set_error(AGRAD_EINVAL, "rope: %llu work items exceed 32-bit indexing", (unsigned long long)total);
     a.total = (uint32_t)total;
+    a.q_rows = B * a.T_len * a.H;
     const uint32_t per_block = kRopeBlock * UNROLL;
     const uint32_t grid = (a.total + per_block - 1) / per_block;
     hipLaunchKernelGGL((rope_kernel<T, VEC, UNROLL>), dim3(grid), dim3(kRopeBlock), 0, s, a);
@@ -107,11 +123,11 @@ int rope_typed(hipStream_t s, RopeArgs<T> a, uint32_t B) {
 
 template <typename T>
 int rope_dispatch(hipStream_t s, void* q, void* k, const float* cos_t, const float* sin_t,
-                  uint32_t B, uint32_t T_len, uint32_t H, uint32_t HKV, uint32_t D, float sgn) {
+                  uint32_t B, uint32_t T_len, uint32_t H, uint32_t HKV, uint32_t D, float sgn, int bhtd) {
     constexpr int VEC = WideVec<T>::value;
     RopeArgs<T> a{};
     a.q = (T*)q; a.k = (T*)k; a.cos_t = cos_t; a.sin_t = sin_t;
-    a.T_len = T_len; a.H = H; a.HKV = HKV; a.D = D; a.sgn = sgn;
+    a.T_len = T_len; a.H = H; a.HKV = HKV; a.D = D; a.sgn = sgn; a.bhtd = bhtd ? 1u : 0u;
     const bool wide = (D / 2) % VEC == 0 && aligned16(q) && (!k || aligned16(k)) &&
                       aligned16(cos_t) && aligned16(sin_t);
     if (wide) return rope_typed<T, VEC>(s, a, B);
@@ -121,7 +137,7 @@ int rope_dispatch(hipStream_t s, void* q, void* k, const float* cos_t, const flo
 }  // namespace
 
 int launch_rope(hipStream_t s, int dtype, void* q, void* k, const float* cos_t, const float* sin_t,
-                uint32_t B, uint32_t T, uint32_t H, uint32_t HKV, uint32_t D, int sign, int backward) {
+                uint32_t B, uint32_t T, uint32_t H, uint32_t HKV, uint32_t D, int sign, int backward, int bhtd) {
     if (sign != 1 && sign != -1) return set_error(AGRAD_EINVAL, "rope: rope_sign must be +1 or -1, got %d", sign);
     if (D == 0 || D % 2 != 0) return set_error(AGRAD_EINVAL, "rope: head_dim %u must be even and non-zero", D);
     if (B == 0 || T == 0 || (H == 0 && (k == nullptr || HKV == 0))) return AGRAD_OK;
@@ -129,8 +145,8 @@ int launch_rope(hipStream_t s, int dtype, void* q, void* k, const float* cos_t, 
     if (H == 0) return set_error(AGRAD_EINVAL, "rope: q must have at least one head");
     if (k != nullptr && HKV == 0) k = nullptr;
     const float sgn = (float)(backward ? -sign : sign);
-    if (dtype == AGRAD_F32) return rope_dispatch<float>(s, q, k, cos_t, sin_t, B, T, H, HKV, D, sgn);
-    if (dtype == AGRAD_BF16) return rope_dispatch<bf16_t>(s, q, k, cos_t, sin_t, B, T, H, HKV, D, sgn);
+    if (dtype == AGRAD_F32) return rope_dispatch<float>(s, q, k, cos_t, sin_t, B, T, H, HKV, D, sgn, bhtd);
+    if (dtype == AGRAD_BF16) return rope_dispatch<bf16_t>(s, q, k, cos_t, sin_t, B, T, H, HKV, D, sgn, bhtd);
     return set_error(AGRAD_EINVAL, "rope: unknown dtype %d", dtype);
 }
 

@@ -552,16 +552,21 @@ class RopeOp(Op):
     op_name = "Rope"
     inplace_aliases = {0: 0, 1: 1}
 
-    def __init__(self, rope_sign=1):
+    def __init__(self, rope_sign=1, layout="bthd"):
         if rope_sign not in (1, -1):
             raise ValueError("rope_sign must be +1 or -1")
+        if layout not in ("bthd", "bhtd"):
+            raise ValueError("layout must be 'bthd' (the CPU kernels', backend.py:1383) or 'bhtd' (attention's)")
         self.rope_sign = rope_sign
+        self.layout = layout
 
     def infer_shape(self, q, k, cos, sin):
-        if q.ndim != 4 or k.ndim != 4 or q.shape[:2] != k.shape[:2] or q.shape[3] != k.shape[3]:
-            raise ValueError("Rope takes q (B,T,H,D) and k (B,T,HKV,D)")
+        t_axis, h_axis = (1, 2) if self.layout == "bthd" else (2, 1)
+        if (q.ndim != 4 or k.ndim != 4 or q.shape[0] != k.shape[0] or q.shape[t_axis] != k.shape[t_axis]
+                or q.shape[3] != k.shape[3]):
+            raise ValueError("Rope takes q (B,T,H,D) and k (B,T,HKV,D), or (B,H,T,D) and (B,HKV,T,D) with layout='bhtd'")
         D = q.shape[3]
-        if D % 2 or cos.shape != sin.shape or cos.ndim != 2 or cos.shape[1] != D // 2 or cos.shape[0] < q.shape[1]:
+        if D % 2 or cos.shape != sin.shape or cos.ndim != 2 or cos.shape[1] != D // 2 or cos.shape[0] < q.shape[t_axis]:
             raise ValueError("Rope tables must be (T_max >= T, D/2)")
         return q.shape, k.shape
 

@@ -264,6 +264,13 @@ int agrad_rope_qk(agrad_ctx* ctx, int dtype, void* q, void* k,
                   const float* cos_table, const float* sin_table,
                   uint32_t B, uint32_t T, uint32_t H, uint32_t HKV, uint32_t D,
                   int rope_sign, int backward);
+/* The same rotation for q[B,H,T,D] and k[B,HKV,T,D], the layout the attention kernels
+ * work in (the layout flag of rope_qk_inplace mode 0 / gqa_rope_inplace,
+ * metal_ops.metal:7458-7465, 11741; call sites backend.py:3764-3767, 3816-3824). */
+int agrad_rope_qk_bhtd(agrad_ctx* ctx, int dtype, void* q, void* k,
+                       const float* cos_table, const float* sin_table,
+                       uint32_t B, uint32_t T, uint32_t H, uint32_t HKV, uint32_t D,
+                       int rope_sign, int backward);
 
 /* out[n,:] = W[ids[n],:] (+ wpe[n % T,:] if wpe != NULL).
  * cpu_gather_forward (backend.py:525-529), gather_forward_kernel

@@ -359,10 +359,13 @@ def cpu_cross_entropy_backward(inputs, outputs, scratch=None):
 def cpu_rope_forward(inputs, outputs, scratch=None):
     q, k, cos, sin = inputs
     q2, k2 = outputs
-    qv, kv = _val(q).copy(), _val(k).copy()
+    bhtd = q2.op.op.layout == "bhtd"        # the CPU kernels take [B,T,H,D] (backend.py:1383): transpose around them
+    qv, kv = _val(q), _val(k)
+    qv = np.ascontiguousarray(qv.transpose(0, 2, 1, 3)) if bhtd else qv.copy()
+    kv = np.ascontiguousarray(kv.transpose(0, 2, 1, 3)) if bhtd else kv.copy()
     K.rope_signed(qv, kv, cos.storage.data, sin.storage.data, q2.op.op.rope_sign, False)
-    _put(q2, qv)
-    _put(k2, kv)
+    _put(q2, np.ascontiguousarray(qv.transpose(0, 2, 1, 3)) if bhtd else qv)
+    _put(k2, np.ascontiguousarray(kv.transpose(0, 2, 1, 3)) if bhtd else kv)
 
 
 def cpu_rope_backward(inputs, outputs, scratch=None):
@@ -372,9 +375,13 @@ def cpu_rope_backward(inputs, outputs, scratch=None):
     for src, dst in ((q, q2), (k, k2)):
         if not src.requires_grad or dst.grad is None:
             continue
-        g = _val(dst.grad).copy()
+        bhtd = q2.op.op.layout == "bhtd"
+        g = _val(dst.grad)
+        g = np.ascontiguousarray(g.transpose(0, 2, 1, 3)) if bhtd else g.copy()
         dummy = np.zeros((g.shape[0], g.shape[1], 1, g.shape[3]), np.float32)
         K.rope_signed(g, dummy, cos.storage.data, sin.storage.data, sign, True)
+        if bhtd:
+            g = np.ascontiguousarray(g.transpose(0, 2, 1, 3))
         if src.grad.storage.data is dst.grad.storage.data or np.shares_memory(src.grad.storage.data, dst.grad.storage.data):
             _put(src.grad, g)
         else:

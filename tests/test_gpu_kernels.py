@@ -428,6 +428,44 @@ def test_rope_fp32_bit_exact(ctx, B, T, H, HKV, D, theta, sign, backward):
         np.testing.assert_array_equal(gk, nk)
 
 
+@pytest.mark.parametrize("B,T,H,HKV,D,theta", ROPE_CASES)
+@pytest.mark.parametrize("sign", [1, -1])
+@pytest.mark.parametrize("backward", [False, True])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_rope_bhtd_layout(ctx, B, T, H, HKV, D, theta, sign, backward, dtype):
+    """agrad_rope_qk_bhtd on q[B,H,T,D], k[B,HKV,T,D] gives the very bits of agrad_rope_qk
+    on the transposed tensors, which is bit-exact against the CPU loops in fp32
+    (test_rope_fp32_bit_exact); also k alone and q alone"""
+    import ctypes as Ct
+    rng = _rng(17)
+    q = rng.standard_normal((B, T, H, D), dtype=np.float32)
+    k = rng.standard_normal((B, T, HKV, D), dtype=np.float32)
+    cos, sin = ref.rope_tables(T, D, theta)
+    if dtype == "bf16":
+        q, k, dt = to_bf16_bits(q), to_bf16_bits(k), capi.BF16
+    else:
+        dt = capi.F32
+    want_q, want_k = G.rope(ctx, q, k, cos, sin, sign, backward)
+    if dtype == "f32":
+        rq, rk = q.copy(), k.copy()
+        ref.rope_signed(rq, rk, cos, sin, sign, backward)
+        np.testing.assert_array_equal(want_q, rq)
+    d_c, d_s = ctx.upload(cos), ctx.upload(sin)
+    for with_q, with_k in ((True, True), (True, False)):
+        d_q = ctx.upload(np.ascontiguousarray(q.transpose(0, 2, 1, 3)))
+        d_k = ctx.upload(np.ascontiguousarray(k.transpose(0, 2, 1, 3))) if with_k else None
+        ctx.call("agrad_rope_qk_bhtd", dt, Ct.c_void_p(d_q.ptr), Ct.c_void_p(d_k.ptr) if d_k is not None else None,
+                 Ct.c_void_p(d_c.ptr), Ct.c_void_p(d_s.ptr), B, T, H, HKV if with_k else 0, D, sign, int(backward))
+        ctx.synchronize()
+        np.testing.assert_array_equal(d_q.download().transpose(0, 2, 1, 3), want_q)
+        d_q.free()
+        if d_k is not None:
+            np.testing.assert_array_equal(d_k.download().transpose(0, 2, 1, 3), want_k)
+            d_k.free()
+    d_c.free()
+    d_s.free()
+
+
 def test_rope_invariants(ctx):
     rng = _rng(16)
     B, T, H, HKV, D = 2, 64, 12, 2, 128

@@ -297,6 +297,35 @@ def test_rope_op_in_graph(sign):
     assert_fp32_close(h_g["q"], c_g["q"], "q.grad (aliased)")
 
 
+def test_rope_op_bhtd_layout_in_graph():
+    """RopeOp(layout="bhtd") on [B,H,T,D] activations equals the default layout on the
+    transposed tensors, forward and gradients, on both devices"""
+    rng = np.random.default_rng(SEED + 9)
+    B, T, H, HKV, D = 2, 12, 4, 2, 32
+    q_np = rng.standard_normal((B, H, T, D)).astype(np.float32)
+    k_np = rng.standard_normal((B, HKV, T, D)).astype(np.float32)
+    cos_np, sin_np = ref.rope_tables(16, D, 1e4)
+    up = rng.standard_normal((B, H, T, D)).astype(np.float32)
+
+    def build(device):
+        q = make_tensor(q_np.shape, np.float32, device, True, q_np)
+        k = make_tensor(k_np.shape, np.float32, device, True, k_np)
+        c = make_tensor(cos_np.shape, np.float32, device, False, cos_np)
+        s = make_tensor(sin_np.shape, np.float32, device, False, sin_np)
+        q2, k2 = RopeOp(rope_sign=1, layout="bhtd")(ReLUSquaredOp()(q), ReLUSquaredOp()(k), c, s)
+        return (AddOp()(q2, q2), k2), {"q": q, "k": k}
+
+    (c_out, c_g), (h_out, h_g) = both(build, up)
+    qa = np.maximum(q_np, 0) ** 2
+    want = np.ascontiguousarray(qa.transpose(0, 2, 1, 3))
+    ref.rope_signed(want, np.zeros((B, T, 1, D), np.float32), cos_np, sin_np, 1, False)
+    np.testing.assert_array_equal(h_out[0], 2 * want.transpose(0, 2, 1, 3))
+    np.testing.assert_array_equal(c_out[0], h_out[0])
+    assert_fp32_close(h_g["q"], c_g["q"], "q.grad, bhtd")
+    with pytest.raises(ValueError):
+        RopeOp(layout="thbd")
+
+
 def test_accumulate_parameter_grads_and_rerun():
     """Two backward passes with accumulate_parameter_grads give twice the
     parameter gradient; without it the second pass starts from zero."""
