@@ -576,6 +576,10 @@ class HipBackend(Backend):
         rows, C = prod(x_saved.shape[:-1]), x_saved.shape[-1]
         dgamma = gamma.grad if gamma is not None and gamma.requires_grad else None
         dbeta = beta.grad if beta is not None and beta.requires_grad else None
+        for name, g in (("gamma", dgamma), ("beta", dbeta)):
+            if g is not None and np.dtype(g.dtype) != np.dtype(np.float32):
+                raise RuntimeError(f"norm backward: the gradient of {name} must be fp32, got {g.dtype} "
+                                   "(norm parameters and their gradients stay fp32 in bf16-I/O graphs)")
         ws = None
         if dgamma is not None or dbeta is not None:
             if scratch is None:
