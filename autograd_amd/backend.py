@@ -459,6 +459,10 @@ class HipBackend(Backend):
         out = outputs[0]
         ws = scratch["workspace"]
         V, C = weight.shape
+        for what, g in (("dY", out.grad), ("dW", weight.grad), ("dwpe", wpe.grad if wpe is not None else None)):
+            if g is not None and _dt(g) != _dt(weight):
+                raise RuntimeError(f"embedding backward: {what} is {g.dtype} but the table is {weight.dtype}; the "
+                                   "kernels take one storage type for the table, its gradient and the activations")
         flag = self._param_flag(node, weight)
         if len(outputs) > 1:
             T = 0
