@@ -32,9 +32,9 @@ import numpy as np
 from .op import (AddLayerNormOp, AddOp, AddRMSNormOp, BiasGELUOp, ContiguousOp, CrossEntropyLossOp, EmbeddingSumOp, ExpOp,
                  GatherOp, GELUOp, LayerNormOp, LogOp, MulOp, PermuteOp, ReLUSquaredOp, ReshapeOp, RMSNormOp, RopeOp,
                  RsqrtOp, SoftmaxOp, SwiGLUOp, TransposeOp, ViewOp)
-from .scratch import single_slot
+from .scratch import equal_slots, single_slot
 from .utils import (bf16_bits, bf16_bits_to_f32_array, contiguous_strides, f32_array_to_bf16_bits, f32_bits,
-                    is_bf16, mul_bcast_kind, xavier_uniform)
+                    is_bf16, mul_bcast_kind, storage_dtype, xavier_uniform)
 
 F32, BF16 = 0, 1
 ACC_INPUT_GRAD, ACC_PARAM_GRAD, ACC_INPUT_GRAD2, ACC_PARAM_GRAD2 = 1, 2, 4, 8
@@ -244,6 +244,12 @@ class HipBackend(Backend):
                     need = max(need, self.ctx.broadcast_grad_workspace_bytes(out.numel // t.numel, t.numel))
             if need:
                 return None, single_slot("workspace", need)
+        if isinstance(op, SoftmaxOp):
+            x = node.inputs[0]
+            if x.ndim and op.axis(x) != x.ndim - 1 and x.numel:
+                dt = storage_dtype(x.dtype)
+                return (equal_slots(("moved_x", "moved_y"), (x.numel,), dt),
+                        equal_slots(("moved_y", "moved_dy", "moved_dx"), (x.numel,), dt) if x.requires_grad else None)
         if isinstance(op, BiasGELUOp):
             h, b = node.inputs
             if b.requires_grad:
@@ -371,18 +377,65 @@ class HipBackend(Backend):
         self._launch("unary_backward", [out.grad, saved, x.grad],
                      [_dt(x), UNARY_OPS[type(op)], self._grad_flag(out.op, x)] + _lo_hi(x.numel))
 
+    # Softmax over an inner axis: the axis is moved to the end through a strided copy
+    # into scratch, the row kernels run there, and a second strided copy brings the
+    # result back (two extra passes; the last axis -- what attention uses -- takes none).
+    @staticmethod
+    def _axis_last(x, axis):
+        """(dims, shape, strides) of x read with `axis` moved to the end"""
+        dims = [d for d in range(x.ndim) if d != axis] + [axis]
+        dense = contiguous_strides(x.shape)
+        return dims, [x.shape[d] for d in dims], [dense[d] for d in dims]
+
+    @staticmethod
+    def _axis_back(x, dims, moved_shape):
+        """strides with which the moved (dense) tensor is read in x's own index order"""
+        dense = contiguous_strides(moved_shape)
+        strides = [0] * x.ndim
+        for i, d in enumerate(dims):
+            strides[d] = dense[i]
+        return strides
+
     def hip_softmax_forward(self, inputs, outputs, scratch=None):
         x, out = inputs[0], outputs[0]
-        V = x.shape[-1]
-        self._launch("softmax_forward", [x, out], [_dt(x)] + _lo_hi(x.numel // max(V, 1)) + [V])
+        axis = out.op.op.axis(x)
+        if axis == x.ndim - 1:
+            V = x.shape[-1]
+            self._launch("softmax_forward", [x, out], [_dt(x)] + _lo_hi(x.numel // max(V, 1)) + [V])
+            return
+        if scratch is None:
+            raise RuntimeError("softmax over an inner axis needs its arena scratch (plan_scratch)")
+        if x.numel == 0:
+            return
+        dims, shape, strides = self._axis_last(x, axis)
+        moved, result = scratch["moved_x"], scratch["moved_y"]
+        V = x.shape[axis]
+        self._gather_strided("contiguous_forward_kernel", x, 0, moved, shape, strides, 0)
+        self._launch("softmax_forward", [moved, result], [_dt(x)] + _lo_hi(x.numel // V) + [V])
+        self._gather_strided("contiguous_forward_kernel", result, 0, out, x.shape, self._axis_back(x, dims, shape), 0)
 
     def hip_softmax_backward(self, inputs, outputs, scratch=None):
         x, out = inputs[0], outputs[0]
         if out.grad is None or not x.requires_grad:
             return
-        V = x.shape[-1]
-        self._launch("softmax_backward", [out, out.grad, x.grad],
-                     [_dt(x)] + _lo_hi(x.numel // max(V, 1)) + [V, self._grad_flag(out.op, x)])
+        axis = out.op.op.axis(x)
+        if axis == x.ndim - 1:
+            V = x.shape[-1]
+            self._launch("softmax_backward", [out, out.grad, x.grad],
+                         [_dt(x)] + _lo_hi(x.numel // max(V, 1)) + [V, self._grad_flag(out.op, x)])
+            return
+        if scratch is None:
+            raise RuntimeError("softmax over an inner axis needs its arena scratch (plan_scratch)")
+        if x.numel == 0:
+            return
+        dims, shape, strides = self._axis_last(x, axis)
+        y, dy, dx = scratch["moved_y"], scratch["moved_dy"], scratch["moved_dx"]
+        V = x.shape[axis]
+        self._gather_strided("contiguous_forward_kernel", out, 0, y, shape, strides, 0)
+        self._gather_strided("contiguous_forward_kernel", out.grad, 0, dy, shape, strides, 0)
+        self._launch("softmax_backward", [y, dy, dx], [_dt(x)] + _lo_hi(x.numel // V) + [V, 0])
+        self._gather_strided("strided_add_backward_kernel", dx, 0, x.grad, x.shape, self._axis_back(x, dims, shape),
+                             self._grad_flag(out.op, x))
 
     # -- views and layout changes (backend.py:263-318, 2754-2866) --------------------
     # View / Reshape / Permute / Transpose outputs share their input's memory, so

@@ -148,16 +148,21 @@ class RsqrtOp(_UnaryOp):
 
 
 class SoftmaxOp(_UnaryOp):
-    """softmax over `dim`; the kernels take the last axis (op.py:205-218)"""
+    """softmax over `dim` (op.py:205-218; any axis, as cpu_softmax_forward takes it,
+    backend.py:354-362).  The kernels work along the last axis; another axis is moved
+    there and back through scratch copies."""
     op_name = "Softmax"
 
     def __init__(self, dim=-1):
         self.dim = dim
 
     def infer_shape(self, x):
-        if self.dim % max(x.ndim, 1) != x.ndim - 1:
-            raise ValueError(f"Softmax: only the last axis is supported, got dim={self.dim} for {x.ndim} axes")
+        if x.ndim == 0 or not -x.ndim <= self.dim < x.ndim:
+            raise ValueError(f"Softmax: dim={self.dim} for a tensor of {x.ndim} axes")
         return x.shape
+
+    def axis(self, x):
+        return self.dim % x.ndim
 
 
 # -- views and layout changes (op.py:89-185) --------------------------------------

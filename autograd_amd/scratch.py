@@ -26,3 +26,14 @@ class ScratchViews(dict):
 def single_slot(name, nbytes):
     nbytes = int(nbytes)
     return ScratchLayout(nbytes=nbytes, slots={name: (0, (nbytes,), np.uint8)})
+
+
+def equal_slots(names, shape, dtype):
+    """several slots of one shape and storage dtype, each starting on a 256-byte boundary"""
+    dtype = np.dtype(dtype)
+    count = 1
+    for d in shape:
+        count *= int(d)
+    step = (count * dtype.itemsize + 255) // 256 * 256
+    slots = {name: (i * step, tuple(int(d) for d in shape), dtype) for i, name in enumerate(names)}
+    return ScratchLayout(nbytes=step * len(names), slots=slots)

@@ -122,8 +122,17 @@ def _cpu_unary(fwd, bwd, saves_output):
 cpu_exp_forward, cpu_exp_backward = _cpu_unary(K.exp_forward, K.exp_backward_into, True)
 cpu_log_forward, cpu_log_backward = _cpu_unary(K.log_forward, K.log_backward_into, False)
 cpu_rsqrt_forward, cpu_rsqrt_backward = _cpu_unary(K.rsqrt_forward, K.rsqrt_backward_into, True)
-cpu_softmax_forward, cpu_softmax_backward = _cpu_unary(
-    K.softmax_forward, lambda g, y, acc: K.softmax_backward_into(y, g, acc), True)
+def cpu_softmax_forward(inputs, outputs, scratch=None):
+    x, out = inputs[0], outputs[0]
+    _put(out, K.softmax_forward(_val(x), axis=out.op.op.dim))       # the op's own axis (backend.py:356)
+
+
+def cpu_softmax_backward(inputs, outputs, scratch=None):
+    x, out = inputs[0], outputs[0]
+    if out.grad is None or not x.requires_grad:
+        return
+    with _Acc(x.grad) as acc:
+        K.softmax_backward_into(_val(out), _val(out.grad), acc, axis=out.op.op.dim)
 
 
 # views share their input's memory: nothing to do going forward (backend.py:263-313)

@@ -143,18 +143,18 @@ def rsqrt_backward_into(dy, y, dx):
     np.add(dx, dy * (-0.5) * y * y * y, out=dx)
 
 
-def softmax_forward(x):
-    m = np.max(x, axis=-1, keepdims=True)
+def softmax_forward(x, axis=-1):
+    m = np.max(x, axis=axis, keepdims=True)
     e = np.subtract(x, m)
     np.exp(e, out=e)
-    s = np.sum(e, axis=-1, keepdims=True)
+    s = np.sum(e, axis=axis, keepdims=True)
     np.divide(e, s, out=e)
     return e
 
 
-def softmax_backward_into(y, g, dx):
+def softmax_backward_into(y, g, dx, axis=-1):
     t = np.multiply(g, y)
-    dot = np.sum(t, axis=-1, keepdims=True)
+    dot = np.sum(t, axis=axis, keepdims=True)
     np.subtract(g, dot, out=t)
     np.multiply(y, t, out=t)
     np.add(dx, t, out=dx)

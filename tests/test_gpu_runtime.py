@@ -297,6 +297,37 @@ def test_rope_op_in_graph(sign):
     assert_fp32_close(h_g["q"], c_g["q"], "q.grad (aliased)")
 
 
+@pytest.mark.parametrize("dim", [0, 1, 2, -1])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_softmax_over_any_axis_in_a_graph(dim, dtype):
+    """SoftmaxOp(dim) for every axis of a [B, T, C] activation on both devices
+    (cpu_softmax_forward / backward take any axis, backend.py:354-374): forward,
+    the gradient into an activation, and a second pass over the same arena"""
+    from autograd_amd.utils import BF16
+    rng = np.random.default_rng(SEED + 50 + (dim % 3))
+    B, T, C = 5, 70, 24
+    x_np = rng.standard_normal((B, T, C), dtype=np.float32)
+    g_np = (1 + 0.1 * rng.standard_normal(C)).astype(np.float32)
+    upstream = rng.standard_normal((B, T, C), dtype=np.float32)
+    dt = BF16 if dtype == "bf16" else np.float32
+
+    def build(device):
+        x = make_tensor(x_np.shape, dt, device, True, x_np, "x")
+        g = make_tensor(g_np.shape, np.float32, device, True, g_np, "g")
+        return x.rms_norm(g).softmax(dim), {"x": x}
+
+    (c_out, c_g), (h_out, h_g) = both(build, upstream)
+    if dtype == "bf16":
+        assert_bf16_close(h_out[0], c_out[0], f"softmax dim={dim}")
+        scale = float(np.abs(c_g["x"]).max())
+        assert np.abs(h_g["x"] - c_g["x"]).max() <= 3e-2 * scale
+    else:
+        assert_fp32_close(h_out[0], c_out[0], f"softmax dim={dim}", rtol=2e-5, atol=2e-6)
+        scale = float(np.abs(c_g["x"]).max())
+        assert_fp32_close(h_g["x"], c_g["x"], "x.grad", rtol=1e-4, atol=1e-5 * scale)
+        np.testing.assert_allclose(h_out[0].sum(axis=dim), 1.0, rtol=0, atol=2e-6)
+
+
 def test_rope_op_bhtd_layout_in_graph():
     """RopeOp(layout="bhtd") on [B,H,T,D] activations equals the default layout on the
     transposed tensors, forward and gradients, on both devices"""

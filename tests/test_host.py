@@ -143,7 +143,7 @@ def test_op_shapes_and_errors():
 
 
 def test_primitive_op_shapes_and_errors():
-    """Mul's broadcast kinds are the reference's (utils.py:134-143); Softmax takes the last axis"""
+    """Mul's broadcast kinds are the reference's (utils.py:134-143); Softmax takes any axis of its input"""
     from autograd_amd.utils import mul_bcast_kind
     x = T((2, 3, 8))
     assert (x * T((2, 3, 8))).shape == (2, 3, 8) and (x * T((8,))).shape == (2, 3, 8)
@@ -156,8 +156,9 @@ def test_primitive_op_shapes_and_errors():
         T((8,)) * x                    # the broadcast operand goes second
     assert x.exp().shape == x.log().shape == x.rsqrt().shape == x.shape
     assert x.softmax(-1).op.op.dim == -1 and x.softmax(2).shape == x.shape
+    assert x.softmax(1).op.op.axis(x) == 1 and x.softmax(-3).op.op.axis(x) == 0      # any axis (backend.py:356)
     with pytest.raises(ValueError):
-        x.softmax(1)
+        x.softmax(3)
     assert x.exp().op.op.save_for_backward((x,), ("y",)) == ["y"]
     assert x.log().op.op.save_for_backward((x,), ("y",)) == [x]
 

@@ -410,6 +410,24 @@ def test_adamw_first_step_is_lr_times_sign_and_matches_textbook():
     assert not m.any() and not v.any()
 
 
+def test_softmax_over_an_inner_axis_is_softmax_of_the_moved_axis():
+    import scipy.special as sp
+    r = rng(61)
+    x = r.standard_normal((3, 5, 4, 6), dtype=np.float32)
+    g = r.standard_normal(x.shape, dtype=np.float32)
+    for axis in (0, 1, 2, -3):
+        y = K.softmax_forward(x, axis=axis)
+        close(y, sp.softmax(x.astype(np.float64), axis=axis))
+        close(y.sum(axis=axis), np.ones_like(y.sum(axis=axis)), atol=1e-6)
+        dx = np.zeros_like(x)
+        K.softmax_backward_into(y, g, dx, axis=axis)
+        moved_y, moved_g = np.moveaxis(y, axis, -1), np.moveaxis(g, axis, -1)
+        want = np.zeros_like(moved_y)
+        K.softmax_backward_into(np.ascontiguousarray(moved_y), np.ascontiguousarray(moved_g), want)
+        close(dx, np.moveaxis(want, -1, axis), atol=1e-7)
+        close(dx.sum(axis=axis), np.zeros_like(dx.sum(axis=axis)), atol=1e-6)      # rows of the Jacobian sum to zero
+
+
 def test_dynamic_maps_have_the_defining_shape():
     """optimizer.py:144-179: 256 sorted values; the signed map is symmetric with two zero
     codes and extremes -1 / +1, the unsigned one starts at 0, ends at 1 and is strictly
