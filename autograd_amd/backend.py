@@ -37,7 +37,7 @@ from .utils import (bf16_bits, bf16_bits_to_f32_array, contiguous_strides, f32_a
                     is_bf16, mul_bcast_kind, storage_dtype, xavier_uniform)
 
 F32, BF16 = 0, 1
-ACC_INPUT_GRAD, ACC_PARAM_GRAD, ACC_INPUT_GRAD2, ACC_PARAM_GRAD2 = 1, 2, 4, 8
+ACC_INPUT_GRAD, ACC_PARAM_GRAD, ACC_INPUT_GRAD2, ACC_PARAM_GRAD2, PARAM_GRAD_BF16 = 1, 2, 4, 8, 16
 UNARY_OPS = {ExpOp: 0, LogOp: 1, RsqrtOp: 2}
 MUL_KINDS = {"same": 0, "row": 1, "col": 2, "scalar": 3}
 
@@ -97,7 +97,8 @@ class Backend:
 
 
 def _dt(t):
-    if is_bf16(t.dtype):
+    """dtype code of a tensor or of a storage (whose bf16 bytes are typed uint16)"""
+    if is_bf16(t.dtype) or np.dtype(t.dtype) == np.dtype(np.uint16):
         return BF16
     if np.dtype(t.dtype) == np.dtype(np.float32):
         return F32
@@ -512,11 +513,15 @@ class HipBackend(Backend):
         out = outputs[0]
         ws = scratch["workspace"]
         V, C = weight.shape
-        for what, g in (("dY", out.grad), ("dW", weight.grad), ("dwpe", wpe.grad if wpe is not None else None)):
-            if g is not None and _dt(g) != _dt(weight):
-                raise RuntimeError(f"embedding backward: {what} is {g.dtype} but the table is {weight.dtype}; the "
-                                   "kernels take one storage type for the table, its gradient and the activations")
-        flag = self._param_flag(node, weight)
+        # one storage type throughout, or bf16 table gradients under fp32 activations
+        # (the reference's bf16 gradient store, backend.py:2808-2812)
+        grads = [g for g in (weight.grad, wpe.grad if wpe is not None else None) if g is not None]
+        narrow = _dt(out.grad) == F32 and all(_dt(g) == BF16 for g in grads)
+        if _dt(out.grad) != _dt(weight) or not (narrow or all(_dt(g) == _dt(weight) for g in grads)):
+            raise RuntimeError(f"embedding backward: upstream {out.grad.dtype}, table {weight.dtype}, gradients "
+                               f"{[str(g.dtype) for g in grads]}: the kernels take one storage type throughout, or "
+                               "bf16 table gradients under fp32 activations")
+        flag = self._param_flag(node, weight) | (PARAM_GRAD_BF16 if narrow else 0)
         if len(outputs) > 1:
             T = 0
             if wpe is not None:

@@ -17,7 +17,7 @@ LIB_PATH = Path(__file__).resolve().parent / "libautograd_hip.so"
 
 F32, BF16 = 0, 1
 NORM_LAYER, NORM_RMS = 0, 1
-ACC_INPUT_GRAD, ACC_PARAM_GRAD, ACC_INPUT_GRAD2, ACC_PARAM_GRAD2 = 1, 2, 4, 8
+ACC_INPUT_GRAD, ACC_PARAM_GRAD, ACC_INPUT_GRAD2, ACC_PARAM_GRAD2, PARAM_GRAD_BF16 = 1, 2, 4, 8, 16
 UNARY_EXP, UNARY_LOG, UNARY_RSQRT = 0, 1, 2
 MUL_SAME, MUL_ROW, MUL_COL, MUL_SCALAR = 0, 1, 2, 3
 OK, EINVAL, EHIP, ENOKERNEL, EINDEX, EWORKSPACE = 0, -1, -2, -3, -4, -5

@@ -107,6 +107,24 @@ template <> struct VecIO<bf16_t, 8> {
     }
 };
 
+// four bf16 values: one 8-byte access (the bf16 gradient row of an fp32 upstream)
+template <> struct VecIO<bf16_t, 4> {
+    typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[4]) {
+        const u32x2_t t = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(p));
+        v[0] = __builtin_bit_cast(float, t.x << 16);
+        v[1] = __builtin_bit_cast(float, t.x & 0xffff0000u);
+        v[2] = __builtin_bit_cast(float, t.y << 16);
+        v[3] = __builtin_bit_cast(float, t.y & 0xffff0000u);
+    }
+    static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[4]) {
+        u32x2_t t;
+        t.x = f32_to_bf16_bits(v[0]) | (f32_to_bf16_bits(v[1]) << 16);
+        t.y = f32_to_bf16_bits(v[2]) | (f32_to_bf16_bits(v[3]) << 16);
+        __builtin_nontemporal_store(t, reinterpret_cast<u32x2_t*>(p));
+    }
+};
+
 template <> struct VecIO<bf16_t, 1> {
     static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[1]) {
         v[0] = bf16_bits_to_f32(__builtin_nontemporal_load(p));

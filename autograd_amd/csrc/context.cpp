@@ -381,7 +381,8 @@ int h_gather_bwd(const Call& c) {
     NEED_DTYPE(c.a[0])
     const uint64_t N = c.a[1], es = dtype_size(c.a[0]), ws_bytes = u64(c.a, 5);
     const uint32_t C = c.a[2], V = c.a[3];
-    RESOLVE(0, N * 4, ids) RESOLVE(1, N * C * es, dY) RESOLVE(2, (uint64_t)V * C * es, dW)
+    const uint64_t gs = (c.a[4] & AGRAD_PARAM_GRAD_BF16) ? 2 : es;      // element size of the table gradient
+    RESOLVE(0, N * 4, ids) RESOLVE(1, N * C * es, dY) RESOLVE(2, (uint64_t)V * C * gs, dW)
     RESOLVE(3, ws_bytes, ws)
     return launch_embedding_bwd(c.ctx->stream, c.a[0], (const int32_t*)ids, dY, dW, ws, ws_bytes, N, C, V,
                                 c.a[4], c.ctx->err_flag);
@@ -402,8 +403,9 @@ int h_gather_bwd_sorted(const Call& c) {
     NEED_DTYPE(c.a[0])
     const uint64_t N = c.a[1], es = dtype_size(c.a[0]), wsb = u64(c.a, 5);
     const uint32_t C = c.a[2], V = c.a[3], T = c.a[7], mask = c.a[8];
-    RESOLVE(0, N * 8, order) RESOLVE(1, N * C * es, dY) RESOLVE(2, (uint64_t)V * C * es, dW) RESOLVE(3, wsb, ws)
-    RESOLVE_IF(mask & 16u, 4, (uint64_t)T * C * es, dwpe)
+    const uint64_t gs = (c.a[4] & AGRAD_PARAM_GRAD_BF16) ? 2 : es;      // element size of the table gradients
+    RESOLVE(0, N * 8, order) RESOLVE(1, N * C * es, dY) RESOLVE(2, (uint64_t)V * C * gs, dW) RESOLVE(3, wsb, ws)
+    RESOLVE_IF(mask & 16u, 4, (uint64_t)T * C * gs, dwpe)
     return launch_embedding_bwd_sorted(c.ctx->stream, (int)c.a[0], (const uint32_t*)order, dY, dW, dwpe, ws, wsb, N, T,
                                        C, V, c.a[4]);
 }

@@ -611,12 +611,15 @@ __device__ __forceinline__ void store_grad_row(T* dW, uint64_t off, const float 
 // One workgroup per chunk of L sorted positions; thread j owns column vectors
 // j, j + blockDim, ...  Control flow depends only on the (uniform) token run
 // structure, so a workgroup never diverges except on the column mask.
-template <typename T, int VEC>
+// T is the upstream gradient's storage type, TO the table gradient's: the same, or
+// bf16 under an fp32 upstream (gather_backward_bf16_kernel, metal_ops.metal:12395-12446:
+// the row sum is finished in fp32, added to the stored bf16 value and rounded once).
+template <typename T, typename TO, int VEC>
 __global__ void __launch_bounds__(512)
 emb_segment_sum_kernel(const uint32_t* __restrict__ tok_s, const uint32_t* __restrict__ row_s,
-                       const T* __restrict__ dY, T* dW, float* __restrict__ carry_head,
+                       const T* __restrict__ dY, TO* dW, float* __restrict__ carry_head,
                        float* __restrict__ carry_tail, uint32_t N, uint32_t C, uint32_t CV,
-                       uint32_t V, uint32_t L, int accumulate, uint32_t chunks, T* dwpe, uint32_t B,
+                       uint32_t V, uint32_t L, int accumulate, uint32_t chunks, TO* dwpe, uint32_t B,
                        uint32_t T_len, int accumulate_pos) {
     if (blockIdx.x >= chunks) {
         // Workgroups past the chunks (present only when a position table wants its
@@ -634,7 +637,7 @@ emb_segment_sum_kernel(const uint32_t* __restrict__ tok_s, const uint32_t* __res
 #pragma unroll
             for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + v[k];
         }
-        store_grad_row<T, VEC>(dwpe, off, acc, accumulate_pos != 0);
+        store_grad_row<TO, VEC>(dwpe, off, acc, accumulate_pos != 0);
         return;
     }
     const ChunkEdges e = chunk_edges(tok_s, blockIdx.x, L, N);
@@ -668,7 +671,7 @@ emb_segment_sum_kernel(const uint32_t* __restrict__ tok_s, const uint32_t* __res
                             if (run_is_first && e.open_left) {
                                 store_carry<VEC>(carry_head + (uint64_t)blockIdx.x * C + col, acc);
                             } else {
-                                store_grad_row<T, VEC>(dW, (uint64_t)cur * C + col, acc, accumulate != 0);
+                                store_grad_row<TO, VEC>(dW, (uint64_t)cur * C + col, acc, accumulate != 0);
                             }
                         }
                         if (have) run_is_first = false;
@@ -687,7 +690,7 @@ emb_segment_sum_kernel(const uint32_t* __restrict__ tok_s, const uint32_t* __res
             } else if (e.open_right) {
                 store_carry<VEC>(carry_tail + (uint64_t)blockIdx.x * C + col, acc);
             } else {
-                store_grad_row<T, VEC>(dW, (uint64_t)cur * C + col, acc, accumulate != 0);
+                store_grad_row<TO, VEC>(dW, (uint64_t)cur * C + col, acc, accumulate != 0);
             }
         }
     }
@@ -761,9 +764,9 @@ constexpr uint32_t kFixLongRun = 64;
 constexpr int kFixBatch = 8;        // partial rows a lane keeps in flight
 static_assert(kFixCols * kFixLanes == kFixThreads && kFixColsLong * kFixLanesLong == kFixThreads, "carry fix layout");
 
-template <typename T, int VEC>
+template <typename TO, int VEC>
 __global__ void __launch_bounds__(kFixThreads)
-emb_carry_fix_kernel(const uint32_t* __restrict__ tok_s, T* dW, const float* __restrict__ carry_head,
+emb_carry_fix_kernel(const uint32_t* __restrict__ tok_s, TO* dW, const float* __restrict__ carry_head,
                      const float* __restrict__ carry_tail, uint32_t N, uint32_t C, uint32_t CV,
                      uint32_t V, uint32_t L, int accumulate) {
     __shared__ float part[kFixThreads * VEC];
@@ -811,7 +814,7 @@ emb_carry_fix_kernel(const uint32_t* __restrict__ tok_s, T* dW, const float* __r
 #pragma unroll
                     for (int k = 0; k < VEC; ++k) sum[k] = sum[k] + v[q][k];
                 }
-            store_grad_row<T, VEC>(dW, (uint64_t)tok * C + col, sum, accumulate != 0);
+            store_grad_row<TO, VEC>(dW, (uint64_t)tok * C + col, sum, accumulate != 0);
         }
         return;
     }
@@ -866,7 +869,7 @@ emb_carry_fix_kernel(const uint32_t* __restrict__ tok_s, T* dW, const float* __r
             for (uint32_t q = 0; q < lanes; ++q)
 #pragma unroll
                 for (int k = 0; k < VEC; ++k) sum[k] = sum[k] + part[(q * cols + colv) * VEC + k];
-            store_grad_row<T, VEC>(dW, (uint64_t)tok * C + col, sum, accumulate != 0);
+            store_grad_row<TO, VEC>(dW, (uint64_t)tok * C + col, sum, accumulate != 0);
         }
         __syncthreads();
     }
@@ -943,15 +946,16 @@ void plan_sum(uint64_t N, uint32_t C, SumPlan* p) {
 
 inline uint64_t order_bytes(uint64_t N) { return align256(N * 8); }   // tok_s[N] then row_s[N]
 
-template <typename T>
+template <typename T, typename TO = T>
 int embedding_sum_typed(hipStream_t s, const SumPlan& p, const uint32_t* tok_s, const uint32_t* row_s, const T* dY,
-                        T* dW, uint8_t* ws, uint32_t N, uint32_t C, uint32_t V, uint32_t flags, T* dwpe,
+                        TO* dW, uint8_t* ws, uint32_t N, uint32_t C, uint32_t V, uint32_t flags, TO* dwpe,
                         uint32_t B, uint32_t T_len) {
     float* head = (float*)(ws + p.off_head);
     float* tail = (float*)(ws + p.off_tail);
     const int acc = (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0;
     const int acc_pos = (flags & AGRAD_ACC_PARAM_GRAD2) ? 1 : 0;
     constexpr int WIDE = WideVec<T>::value;
+    // (a bf16 row under an fp32 upstream moves 8 bytes per vector: 8-byte alignment is implied by 16)
     const bool wide = C % WIDE == 0 && aligned16(dY) && aligned16(dW) && (!dwpe || aligned16(dwpe));
     const uint64_t TC = dwpe ? (uint64_t)T_len * C : 0;
     if (wide) {
@@ -960,18 +964,18 @@ int embedding_sum_typed(hipStream_t s, const SumPlan& p, const uint32_t* tok_s, 
         if (block > 512) block = 512;
         const uint64_t extra = (TC / WIDE + block - 1) / block;
         if (p.chunks + extra > 0x7fffffffull) return set_error(AGRAD_EINVAL, "embedding backward: position table too large");
-        hipLaunchKernelGGL((emb_segment_sum_kernel<T, WIDE>), dim3(p.chunks + (uint32_t)extra), dim3(block), 0, s, tok_s,
+        hipLaunchKernelGGL((emb_segment_sum_kernel<T, TO, WIDE>), dim3(p.chunks + (uint32_t)extra), dim3(block), 0, s, tok_s,
                            row_s, dY, dW, head, tail, N, C, CV, V, p.L, acc, p.chunks, dwpe, B, T_len, acc_pos);
-        hipLaunchKernelGGL((emb_carry_fix_kernel<T, WIDE>), dim3(p.chunks), dim3(kFixThreads), 0, s,
+        hipLaunchKernelGGL((emb_carry_fix_kernel<TO, WIDE>), dim3(p.chunks), dim3(kFixThreads), 0, s,
                            tok_s, dW, head, tail, N, C, CV, V, p.L, acc);
     } else {
         uint32_t block = ((C + 63) / 64) * 64;
         if (block > 512) block = 512;
         const uint64_t extra = (TC + block - 1) / block;
         if (p.chunks + extra > 0x7fffffffull) return set_error(AGRAD_EINVAL, "embedding backward: position table too large");
-        hipLaunchKernelGGL((emb_segment_sum_kernel<T, 1>), dim3(p.chunks + (uint32_t)extra), dim3(block), 0, s, tok_s,
+        hipLaunchKernelGGL((emb_segment_sum_kernel<T, TO, 1>), dim3(p.chunks + (uint32_t)extra), dim3(block), 0, s, tok_s,
                            row_s, dY, dW, head, tail, N, C, C, V, p.L, acc, p.chunks, dwpe, B, T_len, acc_pos);
-        hipLaunchKernelGGL((emb_carry_fix_kernel<T, 1>), dim3(p.chunks), dim3(kFixThreads), 0, s,
+        hipLaunchKernelGGL((emb_carry_fix_kernel<TO, 1>), dim3(p.chunks), dim3(kFixThreads), 0, s,
                            tok_s, dW, head, tail, N, C, C, V, p.L, acc);
     }
     return check_hip(hipGetLastError(), "embedding backward launch");
@@ -1105,6 +1109,11 @@ int launch_embedding_bwd_sorted(hipStream_t s, int dtype, const uint32_t* order,
                          (unsigned long long)workspace_bytes, (unsigned long long)p.total);
     if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
         return set_error(AGRAD_EINVAL, "embedding backward: workspace must be 256-byte aligned");
+    if (flags & AGRAD_PARAM_GRAD_BF16) {
+        if (dtype != AGRAD_F32) return set_error(AGRAD_EINVAL, "embedding backward: AGRAD_PARAM_GRAD_BF16 goes with an fp32 upstream gradient");
+        return embedding_sum_typed<float, bf16_t>(s, p, order, order + N, (const float*)dY, (bf16_t*)dW, (uint8_t*)workspace,
+                                                  (uint32_t)N, C, V, flags, (bf16_t*)dwpe, B, T);
+    }
     if (dtype == AGRAD_F32)
         return embedding_sum_typed<float>(s, p, order, order + N, (const float*)dY, (float*)dW, (uint8_t*)workspace,
                                           (uint32_t)N, C, V, flags, (float*)dwpe, B, T);

@@ -190,6 +190,7 @@ PYBIND11_MODULE(hip_ext, m) {
     m.attr("ACC_INPUT_GRAD") = (unsigned)AGRAD_ACC_INPUT_GRAD;
     m.attr("ACC_PARAM_GRAD") = (unsigned)AGRAD_ACC_PARAM_GRAD;
     m.attr("ACC_PARAM_GRAD2") = (unsigned)AGRAD_ACC_PARAM_GRAD2;
+    m.attr("PARAM_GRAD_BF16") = (unsigned)AGRAD_PARAM_GRAD_BF16;
     m.def("device_count", [] {
         int n = 0;
         agrad_device_count(&n);

@@ -45,7 +45,10 @@ enum {
     AGRAD_ACC_INPUT_GRAD = 1u, /* dx += ... (CPU semantics, backend.py:414,477-487); else dx = ... */
     AGRAD_ACC_PARAM_GRAD = 2u, /* dgamma/dbeta/dW += ...; else =                                   */
     AGRAD_ACC_INPUT_GRAD2 = 4u, /* norm backward: the same choice for the second output dx2        */
-    AGRAD_ACC_PARAM_GRAD2 = 8u  /* sorted embedding backward: the same choice for dwpe             */
+    AGRAD_ACC_PARAM_GRAD2 = 8u, /* sorted embedding backward: the same choice for dwpe             */
+    AGRAD_PARAM_GRAD_BF16 = 16u /* embedding backward with an fp32 upstream gradient: dW (and dwpe) are
+                                 * bf16; a row's sum is finished in fp32, added to the stored value and
+                                 * rounded once (gather_backward_bf16_kernel, metal_ops.metal:12395-12446) */
 };
 
 /* ---- context, memory, passes --------------------------------------------

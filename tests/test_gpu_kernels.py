@@ -943,3 +943,75 @@ def test_id_ordering_with_frequent_tokens(ctx, case):
         dW.free()
     for d in (d_ids, d_W, d_dY, out, order, sws, bws):
         d.free()
+
+
+@pytest.mark.parametrize("B,T,V,C,dist", [(4, 128, 500, 64, "uniform"), (2, 700, 90, 50, "zipf"), (8, 512, 4000, 384, "zipf"),
+                                          (3, 23000, 3000, 32, "zipf")])
+def test_embedding_gradient_stored_as_bf16_under_an_fp32_upstream(ctx, B, T, V, C, dist):
+    """AGRAD_PARAM_GRAD_BF16 (gather_backward_bf16_kernel, metal_ops.metal:12395-12446): dY is
+    fp32, dW and dwpe are bf16.  A row's sum is finished in fp32, added to the stored bf16
+    value (when accumulating) and rounded once: compared with that computation on the CPU
+    row sums to one bf16 ulp (the fp32 sums may associate differently across chunk edges);
+    rows without a token keep their bits.  Through the plain and the pre-sorted call."""
+    import ctypes as Ct
+    rng = _rng(70 + C)
+    N = B * T
+    ids = (_zipf_ids(rng, N, V) if dist == "zipf" else rng.integers(0, V, size=N, dtype=np.int32)).reshape(B, T)
+    dY = rng.standard_normal((B, T, C)).astype(np.float32)
+    old_w = to_bf16_bits((0.5 * rng.standard_normal((V, C))).astype(np.float32))
+    old_p = to_bf16_bits((0.5 * rng.standard_normal((T, C))).astype(np.float32))
+    rows = np.zeros((V, C), np.float32)
+    ref.gather_backward_into(ids, dY, rows)
+    pos = dY.astype(np.float64).sum(0)
+    touched = np.zeros(V, bool)
+    touched[ids.reshape(-1)] = True
+
+    def vp(d):
+        return Ct.c_void_p(d.ptr) if d is not None else None
+
+    def check(got_bits, sums, old_bits, accumulate, what, only=None):
+        want = (from_bf16_bits(old_bits).astype(np.float64) if accumulate else 0.0) + sums.astype(np.float64)
+        got = from_bf16_bits(got_bits).astype(np.float64)
+        ulp = np.maximum(np.abs(want), 1e-30) * 2.0 ** -7            # one bf16 ulp is at most 2^-7 of the value
+        bound = ulp + 1e-5 * np.sqrt(N / V + 1)                       # plus the fp32 sums' own re-association noise
+        bad = np.abs(got - want) > bound
+        if only is not None:
+            bad &= only[:, None]
+        assert not bad.any(), (what, int(bad.sum()), float(np.abs(got - want).max()))
+
+    d_ids, d_dY = ctx.upload(ids), ctx.upload(dY)
+    ws_b = ctx.lib.agrad_embedding_backward_workspace_bytes(N, C, V, capi.F32)
+    ws = ctx.empty((ws_b,), np.uint8)
+    for accumulate in (False, True):
+        dW = ctx.upload(old_w)
+        ctx.call("agrad_embedding_backward", capi.F32, vp(d_ids), vp(d_dY), vp(dW), vp(ws), ws_b, N, C, V,
+                 capi.PARAM_GRAD_BF16 | (capi.ACC_PARAM_GRAD if accumulate else 0))
+        ctx.synchronize()
+        got = dW.download()
+        check(got, rows, old_w, accumulate, f"plain call, accumulate={accumulate}", touched)
+        np.testing.assert_array_equal(got[~touched], old_w[~touched])
+        dW.free()
+    # pre-sorted pair with the position table in the same launch
+    d_W = ctx.upload(np.zeros((V, C), np.float32))
+    out = ctx.empty((N, C), np.float32)
+    order = ctx.empty((2 * N,), np.uint32)
+    sws_b = ctx.lib.agrad_embedding_sort_workspace_bytes(N, V)
+    bws_b = ctx.lib.agrad_embedding_backward_sorted_workspace_bytes(N, C)
+    sws, bws = ctx.empty((sws_b,), np.uint8), ctx.empty((bws_b,), np.uint8)
+    ctx.call("agrad_gather_forward_sorted", capi.F32, vp(d_ids), vp(d_W), None, vp(out), N, T, C, V, vp(order), vp(sws), sws_b)
+    for accumulate in (False, True):
+        dW, dP = ctx.upload(old_w), ctx.upload(old_p)
+        flags = capi.PARAM_GRAD_BF16 | ((capi.ACC_PARAM_GRAD | capi.ACC_PARAM_GRAD2) if accumulate else 0)
+        ctx.call("agrad_embedding_backward_sorted", capi.F32, vp(order), vp(d_dY), vp(dW), vp(dP), vp(bws), bws_b, N, T, C, V, flags)
+        ctx.synchronize()
+        got = dW.download()
+        check(got, rows, old_w, accumulate, f"sorted call, accumulate={accumulate}", touched)
+        np.testing.assert_array_equal(got[~touched], old_w[~touched])
+        check(dP.download(), pos, old_p, accumulate, f"position table, accumulate={accumulate}")
+        dW.free()
+        dP.free()
+    with pytest.raises(capi.AgradError):      # the narrow store goes with an fp32 upstream only
+        dW = ctx.upload(old_w)
+        ctx.call("agrad_embedding_backward", capi.BF16, vp(d_ids), vp(d_dY), vp(dW), vp(ws), ws_b, N, C, V, capi.PARAM_GRAD_BF16)
+    for d in (d_ids, d_dY, ws, d_W, out, order, sws, bws):
+        d.free()

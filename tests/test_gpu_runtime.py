@@ -328,6 +328,51 @@ def test_softmax_over_any_axis_in_a_graph(dim, dtype):
         np.testing.assert_allclose(h_out[0].sum(axis=dim), 1.0, rtol=0, atol=2e-6)
 
 
+def test_embedding_table_with_bf16_gradient_storage():
+    """an fp32 table whose gradient is kept in bf16 (Tensor(grad_dtype=BF16); the
+    reference's bf16 gradient store, backend.py:2808-2812): the backward pass rounds each
+    row's fp32 sum once; two passes accumulate in bf16, on both devices; AdamW then reads
+    the bf16 gradient"""
+    from autograd_amd.optimizer import AdamW
+    from autograd_amd.utils import BF16
+    rng = np.random.default_rng(SEED + 60)
+    B, T, V, C = 4, 96, 300, 64
+    ids_np = rng.integers(0, V, (B, T), dtype=np.int32)
+    w_np = (0.5 * rng.standard_normal((V, C))).astype(np.float32)
+    upstream = rng.standard_normal((B, T, C)).astype(np.float32)
+    results = {}
+    for device in ("cpu", "hip"):
+        rt = Runtime(device=device)
+        ids = Tensor(shape=(B, T), dtype=np.int32, device=device, requires_grad=False, init_val=ids_np)
+        w = Tensor(shape=(V, C), dtype=np.float32, device=device, requires_grad=True, init_val=w_np, grad_dtype=BF16)
+        out = ids.gather(w).relu2()
+        rt.loss = out
+        rt.build_topo(out)
+        rt.bind_memory()
+        rt.accumulate_parameter_grads = True
+        rt.backend.accumulate_parameter_grads = True
+        rt.zero_grad()
+        for _ in range(2):
+            rt.forward()
+            rt.backend.copy_from_host(out.grad, upstream)
+            rt.backward_graph()
+        rt.backend.synchronize()
+        assert np.dtype(w.grad.storage.dtype) == np.dtype(np.uint16)
+        grad = rt.backend.copy_to_host(w.grad).copy()
+        opt = AdamW([w], lr=1e-2, weight_decay=0.0, runtime=rt)
+        opt.step()
+        results[device] = (grad, rt.backend.copy_to_host(w).copy())
+        opt.release()
+        rt.release()
+    (c_grad, c_w), (h_grad, h_w) = results["cpu"], results["hip"]
+    x = np.maximum(w_np[ids_np], 0)
+    once = np.zeros((V, C), np.float64)
+    np.add.at(once, ids_np.reshape(-1), (2 * x * upstream).reshape(-1, C).astype(np.float64))
+    assert_bf16_close(h_grad, 2 * once, "bf16 table gradient vs float64", rel=2e-2)
+    assert_bf16_close(h_grad, c_grad, "bf16 table gradient, hip vs cpu", rel=1.6e-2)
+    assert np.abs(h_w - c_w).max() <= 2.1e-2          # a first Adam step moves by lr * sign(g): same side, or a zero gradient
+
+
 def test_rope_op_bhtd_layout_in_graph():
     """RopeOp(layout="bhtd") on [B,H,T,D] activations equals the default layout on the
     transposed tensors, forward and gradients, on both devices"""
