@@ -638,10 +638,12 @@ class HipBackend(Backend):
         rows, C = prod(x_saved.shape[:-1]), x_saved.shape[-1]
         dgamma = gamma.grad if gamma is not None and gamma.requires_grad else None
         dbeta = beta.grad if beta is not None and beta.requires_grad else None
-        for name, g in (("gamma", dgamma), ("beta", dbeta)):
-            if g is not None and np.dtype(g.dtype) != np.dtype(np.float32):
-                raise RuntimeError(f"norm backward: the gradient of {name} must be fp32, got {g.dtype} "
-                                   "(norm parameters and their gradients stay fp32 in bf16-I/O graphs)")
+        # fp32 parameter gradients, or both stored as bf16 (the reference's bf16 gradient store)
+        kinds = {_dt(g) for g in (dgamma, dbeta) if g is not None}
+        if len(kinds) > 1:
+            raise RuntimeError("norm backward: the gradients of gamma and beta must share one storage type")
+        if kinds == {BF16}:
+            flags |= PARAM_GRAD_BF16
         ws = None
         if dgamma is not None or dbeta is not None:
             if scratch is None:

@@ -279,13 +279,14 @@ int h_norm_bwd(const Call& c) {
     const uint32_t C = c.a[2], flags = c.a[4], present = c.a[5];
     const uint64_t ws_bytes = u64(c.a, 6);
     const uint64_t act = rows * C * dtype_size(c.a[0]), par = (uint64_t)C * 4;
+    const uint64_t gpar = (flags & AGRAD_PARAM_GRAD_BF16) ? (uint64_t)C * 2 : par;     // dgamma / dbeta element size
     RESOLVE(0, act, x) RESOLVE(1, act, dy)
     RESOLVE_IF(present & 4u, 2, par, gamma)
     RESOLVE_IF(present & 8u, 3, act, dres)
     RESOLVE_IF(present & 16u, 4, act, dx)
     RESOLVE_IF(present & 32u, 5, act, dx2)
-    RESOLVE_IF(present & 64u, 6, par, dgamma)
-    RESOLVE_IF(present & 128u, 7, par, dbeta)
+    RESOLVE_IF(present & 64u, 6, gpar, dgamma)
+    RESOLVE_IF(present & 128u, 7, gpar, dbeta)
     RESOLVE_IF(present & 256u, 8, ws_bytes, ws)
     return launch_norm_bwd(c.ctx->stream, KIND, c.a[0], x, dy, (const float*)gamma, dres, dx, dx2,
                            (float*)dgamma, (float*)dbeta, ws, ws ? ws_bytes : 0, rows, C, f32(c.a[3]), flags);

@@ -945,8 +945,9 @@ int launch_norm_bwd(hipStream_t s, int kind, int dtype, const void* x, const voi
     if (rows == 0) {
         // nothing to add: stored parameter grads become zero, accumulated ones stay
         if (want_params && !(flags & AGRAD_ACC_PARAM_GRAD)) {
-            if (dgamma) if (int rc = launch_fill(s, dgamma, 0, 4, C)) return rc;
-            if (dbeta) if (int rc = launch_fill(s, dbeta, 0, 4, C)) return rc;
+            const int gsize = (flags & AGRAD_PARAM_GRAD_BF16) ? 2 : 4;
+            if (dgamma) if (int rc = launch_fill(s, dgamma, 0, gsize, C)) return rc;
+            if (dbeta) if (int rc = launch_fill(s, dbeta, 0, gsize, C)) return rc;
         }
         return AGRAD_OK;
     }
@@ -973,7 +974,8 @@ int launch_norm_bwd(hipStream_t s, int kind, int dtype, const void* x, const voi
     }
     if (rc != AGRAD_OK) return rc;
     if (want_params)
-        return launch_colsum_finalize(s, pg, pb, grid, C, dgamma, dbeta, (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0);
+        return launch_colsum_finalize(s, pg, pb, grid, C, dgamma, dbeta, (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0,
+                                      (flags & AGRAD_PARAM_GRAD_BF16) != 0);
     return check_hip(hipGetLastError(), "norm backward launch");
 }
 

@@ -46,9 +46,12 @@ enum {
     AGRAD_ACC_PARAM_GRAD = 2u, /* dgamma/dbeta/dW += ...; else =                                   */
     AGRAD_ACC_INPUT_GRAD2 = 4u, /* norm backward: the same choice for the second output dx2        */
     AGRAD_ACC_PARAM_GRAD2 = 8u, /* sorted embedding backward: the same choice for dwpe             */
-    AGRAD_PARAM_GRAD_BF16 = 16u /* embedding backward with an fp32 upstream gradient: dW (and dwpe) are
-                                 * bf16; a row's sum is finished in fp32, added to the stored value and
-                                 * rounded once (gather_backward_bf16_kernel, metal_ops.metal:12395-12446) */
+    AGRAD_PARAM_GRAD_BF16 = 16u /* parameter gradients stored as bf16: the embedding backward with an fp32
+                                 * upstream gradient (dW and dwpe; gather_backward_bf16_kernel,
+                                 * metal_ops.metal:12395-12446) and the norm backward (dgamma and dbeta then
+                                 * point at bf16; the bf16 option of rmsnorm_weighted_dgamma and
+                                 * gqa_rms_dgamma_bf16, metal_ops.metal:12448-12479, 14541-14746).  A sum is
+                                 * finished in fp32, added to the stored value and rounded once */
 };
 
 /* ---- context, memory, passes --------------------------------------------

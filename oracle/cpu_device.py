@@ -11,6 +11,7 @@ bf16 tensors are stored as uint16 bits and widened around every op.
 """
 from __future__ import annotations
 
+from contextlib import ExitStack
 from math import prod
 
 import numpy as np
@@ -74,6 +75,14 @@ class _Acc:
             _put(self.t, self.work)
 
 
+def _param_grad(stack, t):
+    """fp32 working view of a parameter's gradient (None if it wants none); a bf16-stored
+    gradient is widened here and rounded back once when `stack` closes"""
+    if t is None or not t.requires_grad or t.grad is None:
+        return None
+    return stack.enter_context(_Acc(t.grad))
+
+
 def cpu_add_forward(inputs, outputs, scratch=None):
     _put(outputs[0], K.add_forward(_val(inputs[0]), _val(inputs[1])))
 
@@ -122,6 +131,8 @@ def _cpu_unary(fwd, bwd, saves_output):
 cpu_exp_forward, cpu_exp_backward = _cpu_unary(K.exp_forward, K.exp_backward_into, True)
 cpu_log_forward, cpu_log_backward = _cpu_unary(K.log_forward, K.log_backward_into, False)
 cpu_rsqrt_forward, cpu_rsqrt_backward = _cpu_unary(K.rsqrt_forward, K.rsqrt_backward_into, True)
+
+
 def cpu_softmax_forward(inputs, outputs, scratch=None):
     x, out = inputs[0], outputs[0]
     _put(out, K.softmax_forward(_val(x), axis=out.op.op.dim))       # the op's own axis (backend.py:356)
@@ -274,9 +285,9 @@ def cpu_layernorm_backward(inputs, outputs, scratch=None):
     eps = out.op.op.eps
     if x.requires_grad and x.grad.storage.data.dtype != np.uint16:
         # fp32: accumulate straight into x.grad in the reference's order (backend.py:469-487)
-        dg = gamma.grad.storage.data if gamma.requires_grad else None
-        db = beta.grad.storage.data if beta.requires_grad else None
-        K.layernorm_backward_into(_val(x), _val(gamma), _val(out.grad), eps, x.grad.storage.data, dg, db)
+        with ExitStack() as stack:
+            dg, db = _param_grad(stack, gamma), _param_grad(stack, beta)
+            K.layernorm_backward_into(_val(x), _val(gamma), _val(out.grad), eps, x.grad.storage.data, dg, db)
         return
     local = _norm_backward("layer", _val(x), gamma, beta, _val(out.grad), eps, x.requires_grad, gamma, beta)
     if x.requires_grad:
@@ -298,9 +309,9 @@ def cpu_rmsnorm_backward(inputs, outputs, scratch=None):
         return
     eps = out.op.op.eps
     if x.requires_grad and x.grad.storage.data.dtype != np.uint16:
-        dg = gamma.grad.storage.data if gamma is not None and gamma.requires_grad else None
-        K.rmsnorm_backward_into(_val(x), _val(gamma) if gamma is not None else None, _val(out.grad), eps,
-                                x.grad.storage.data, dg)
+        with ExitStack() as stack:
+            K.rmsnorm_backward_into(_val(x), _val(gamma) if gamma is not None else None, _val(out.grad), eps,
+                                    x.grad.storage.data, _param_grad(stack, gamma))
         return
     local = _norm_backward("rms", _val(x), gamma, None, _val(out.grad), eps, x.requires_grad, gamma, None)
     if x.requires_grad:
@@ -333,12 +344,12 @@ def cpu_add_norm_backward(inputs, outputs, scratch=None):
         need_dx = any(t.requires_grad for t in (x, res))
         C = h.shape[-1]
         g = _val(gamma) if gamma is not None else None
-        dg = gamma.grad.storage.data if gamma is not None and gamma.requires_grad else None
-        db = beta.grad.storage.data if beta is not None and beta.requires_grad else None
-        if is_ln:
-            K.layernorm_backward_into(_val(h), g, _val(y.grad), op.eps, total if need_dx else None, dg, db)
-        else:
-            K.rmsnorm_backward_into(_val(h), g, _val(y.grad), op.eps, total if need_dx else None, dg)
+        with ExitStack() as stack:
+            dg, db = _param_grad(stack, gamma), _param_grad(stack, beta)
+            if is_ln:
+                K.layernorm_backward_into(_val(h), g, _val(y.grad), op.eps, total if need_dx else None, dg, db)
+            else:
+                K.rmsnorm_backward_into(_val(h), g, _val(y.grad), op.eps, total if need_dx else None, dg)
     elif h.grad is None:
         return
     for t in (x, res):

@@ -1015,3 +1015,33 @@ def test_embedding_gradient_stored_as_bf16_under_an_fp32_upstream(ctx, B, T, V, 
         ctx.call("agrad_embedding_backward", capi.BF16, vp(d_ids), vp(d_dY), vp(dW), vp(ws), ws_b, N, C, V, capi.PARAM_GRAD_BF16)
     for d in (d_ids, d_dY, ws, d_W, out, order, sws, bws):
         d.free()
+
+
+@pytest.mark.parametrize("kind", [capi.NORM_LAYER, capi.NORM_RMS])
+@pytest.mark.parametrize("rows,Cw", [(37, 96), (2048, 384), (500, 1536)])
+@pytest.mark.parametrize("io", ["f32", "bf16"])
+def test_norm_parameter_gradients_stored_as_bf16(ctx, kind, rows, Cw, io):
+    """AGRAD_PARAM_GRAD_BF16 on the norm backward: dgamma / dbeta point at bf16 (the bf16
+    option of rmsnorm_weighted_dgamma, gqa_rms_dgamma_bf16).  The stored value is the fp32
+    call's sum (plus the stored bf16 value when accumulating) rounded once: the two calls
+    share the partial sums, so the comparison is exact."""
+    rng = _rng(90 + Cw)
+    x = rng.standard_normal((rows, Cw)).astype(np.float32)
+    dy = rng.standard_normal((rows, Cw)).astype(np.float32)
+    gamma = (1 + 0.1 * rng.standard_normal(Cw)).astype(np.float32)
+    if io == "bf16":
+        x, dy = to_bf16_bits(x), to_bf16_bits(dy)
+    want_beta = kind == capi.NORM_LAYER
+    wide = G.norm_backward(ctx, kind, x, gamma, dy, 1e-5, want_dbeta=want_beta)
+    old_g = to_bf16_bits(rng.standard_normal(Cw).astype(np.float32))
+    old_b = to_bf16_bits(rng.standard_normal(Cw).astype(np.float32))
+    for accumulate in (False, True):
+        flags = capi.PARAM_GRAD_BF16 | (capi.ACC_PARAM_GRAD if accumulate else 0)
+        got = G.norm_backward(ctx, kind, x, gamma, dy, 1e-5, want_dbeta=want_beta, dgamma_init=old_g,
+                              dbeta_init=old_b if want_beta else None, flags=flags)
+        np.testing.assert_array_equal(got["dx"], wide["dx"])
+        for name, old in (("dgamma", old_g), ("dbeta", old_b)):
+            if wide[name] is None:
+                continue
+            base = from_bf16_bits(old) if accumulate else np.zeros(Cw, np.float32)
+            np.testing.assert_array_equal(got[name], to_bf16_bits(base + wide[name]), err_msg=f"{name} accumulate={accumulate}")

@@ -373,6 +373,29 @@ def test_embedding_table_with_bf16_gradient_storage():
     assert np.abs(h_w - c_w).max() <= 2.1e-2          # a first Adam step moves by lr * sign(g): same side, or a zero gradient
 
 
+def test_norm_parameters_with_bf16_gradient_storage():
+    """gamma / beta with grad_dtype=BF16 under fp32 activations, on both devices"""
+    from autograd_amd.utils import BF16
+    rng = np.random.default_rng(SEED + 61)
+    B, T, C = 6, 40, 96
+    x_np = rng.standard_normal((B, T, C), dtype=np.float32)
+    g_np = (1 + 0.1 * rng.standard_normal(C)).astype(np.float32)
+    b_np = (0.1 * rng.standard_normal(C)).astype(np.float32)
+    upstream = rng.standard_normal((B, T, C), dtype=np.float32)
+
+    def build(device):
+        x = make_tensor(x_np.shape, np.float32, device, True, x_np, "x")
+        g = Tensor(shape=(C,), dtype=np.float32, device=device, requires_grad=True, init_val=g_np, grad_dtype=BF16)
+        b = Tensor(shape=(C,), dtype=np.float32, device=device, requires_grad=True, init_val=b_np, grad_dtype=BF16)
+        return x.relu2().layer_norm(g, b), {"x": x, "g": g, "b": b}
+
+    (c_out, c_g), (h_out, h_g) = both(build, upstream)
+    assert_fp32_close(h_out[0], c_out[0], "forward", rtol=2e-5, atol=2e-6)
+    assert_fp32_close(h_g["x"], c_g["x"], "x.grad", rtol=1e-4, atol=1e-5)
+    for name in ("g", "b"):
+        assert_bf16_close(h_g[name], c_g[name], f"{name}.grad stored as bf16", rel=1.6e-2)
+
+
 def test_rope_op_bhtd_layout_in_graph():
     """RopeOp(layout="bhtd") on [B,H,T,D] activations equals the default layout on the
     transposed tensors, forward and gradients, on both devices"""
