@@ -229,8 +229,27 @@ class HipBackend(Backend):
         return self._input_flag(node, t)
 
     # -- scratch -----------------------------------------------------------------
+    def _check_gradient_storage(self, node):
+        """A leaf may keep its gradient in another type than its values (fp32 values, bf16
+        gradient: the reference's bf16 gradient store).  Only the kernels that own a
+        parameter gradient can write one: the embedding tables and the norm parameters."""
+        op = node.op
+        for i, t in enumerate(node.inputs):
+            if t.op is not None or not t.requires_grad or t.grad is None or t.grad.dtype == t.dtype:
+                continue
+            if _dt(t.grad) == _dt(t):
+                continue
+            table = isinstance(op, (GatherOp, EmbeddingSumOp)) and i >= 1
+            norm_param = (isinstance(op, (LayerNormOp, RMSNormOp)) and i >= 1) or \
+                         (isinstance(op, (AddLayerNormOp, AddRMSNormOp)) and i >= 2)
+            if not (table or norm_param) or _dt(t) != F32 or _dt(t.grad) != BF16:
+                raise RuntimeError(f"{op.op_name}: input {i} ({t.name or 'unnamed'}) stores {t.dtype} values and a "
+                                   f"{t.grad.dtype} gradient; only embedding tables and norm parameters (fp32 values, "
+                                   "bf16 gradient) can keep their gradient in another type")
+
     def plan_scratch(self, node):
         op = node.op
+        self._check_gradient_storage(node)
         if isinstance(op, (LayerNormOp, RMSNormOp, AddLayerNormOp, AddRMSNormOp)):
             first_param = 2 if isinstance(op, (AddLayerNormOp, AddRMSNormOp)) else 1
             if any(p.requires_grad for p in node.inputs[first_param:]):

@@ -470,3 +470,22 @@ def test_adamw_8bit_state_on_the_oracle_device():
     assert (moved[rest] < 1e-6).all()                          # the others only decayed
     with pytest.raises(NotImplementedError):
         AdamW([w, g], runtime=rt, state_mode="mini")
+
+
+def test_hip_backend_refuses_a_gradient_type_no_kernel_can_write():
+    """fp32 values with a bf16 gradient are for embedding tables and norm parameters; a bias
+    under a broadcast Add is refused when the graph is planned, not corrupted when it runs
+    (checked on the planning hook alone: no device is needed)"""
+    from autograd_amd.backend import HipBackend
+    from autograd_amd.utils import BF16
+    backend = HipBackend.__new__(HipBackend)          # no context: plan-time checks only
+    x = Tensor(shape=(4, 8), dtype=np.float32, device="hip", requires_grad=True)
+    bias = Tensor(shape=(8,), dtype=np.float32, device="hip", requires_grad=True, grad_dtype=BF16)
+    for t in (x, bias):
+        t.grad = Tensor(shape=t.shape, dtype=t.grad_dtype, device="hip", requires_grad=False)
+    out = x + bias
+    with pytest.raises(RuntimeError, match="another type"):
+        backend._check_gradient_storage(out.op)
+    gamma = Tensor(shape=(8,), dtype=np.float32, device="hip", requires_grad=True, grad_dtype=BF16)
+    gamma.grad = Tensor(shape=(8,), dtype=BF16, device="hip", requires_grad=False)
+    backend._check_gradient_storage(x.rms_norm(gamma).op)         # a norm parameter may
