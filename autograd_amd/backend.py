@@ -232,7 +232,8 @@ class HipBackend(Backend):
     def _check_gradient_storage(self, node):
         """A leaf may keep its gradient in another type than its values (fp32 values, bf16
         gradient: the reference's bf16 gradient store).  Only the kernels that own a
-        parameter gradient can write one: the embedding tables and the norm parameters."""
+        parameter gradient can write one: the embedding tables, the norm parameters and the
+        broadcast operand of an Add (a bias, a position table)."""
         op = node.op
         for i, t in enumerate(node.inputs):
             if t.op is not None or not t.requires_grad or t.grad is None or t.grad.dtype == t.dtype:
@@ -242,10 +243,11 @@ class HipBackend(Backend):
             table = isinstance(op, (GatherOp, EmbeddingSumOp)) and i >= 1
             norm_param = (isinstance(op, (LayerNormOp, RMSNormOp)) and i >= 1) or \
                          (isinstance(op, (AddLayerNormOp, AddRMSNormOp)) and i >= 2)
-            if not (table or norm_param) or _dt(t) != F32 or _dt(t.grad) != BF16:
+            bias = isinstance(op, AddOp) and t.shape != node.outputs[0].shape and self._trailing(t.shape, node.outputs[0].shape)
+            if not (table or norm_param or bias) or _dt(t) != F32 or _dt(t.grad) != BF16:
                 raise RuntimeError(f"{op.op_name}: input {i} ({t.name or 'unnamed'}) stores {t.dtype} values and a "
-                                   f"{t.grad.dtype} gradient; only embedding tables and norm parameters (fp32 values, "
-                                   "bf16 gradient) can keep their gradient in another type")
+                                   f"{t.grad.dtype} gradient; only embedding tables, norm parameters and the broadcast "
+                                   "operand of an Add (fp32 values, bf16 gradient) can keep their gradient in another type")
 
     def plan_scratch(self, node):
         op = node.op
@@ -326,12 +328,17 @@ class HipBackend(Backend):
             if not t.requires_grad or t.grad is None:
                 continue
             if t.shape == out.shape:
+                if _dt(t.grad) != _dt(out.grad):
+                    raise RuntimeError(f"Add backward: gradient of {t.dtype} input stored as {t.grad.dtype}")
                 self._launch("add_residual_backward", [out.grad, t.grad],
                              [_dt(out), self._grad_flag(node, t)] + _lo_hi(out.numel))
-            elif self._trailing(t.shape, out.shape) and _dt(t.grad) == _dt(out.grad):
+            elif self._trailing(t.shape, out.shape) and (_dt(t.grad) == _dt(out.grad)
+                                                        or (_dt(out.grad) == F32 and _dt(t.grad) == BF16)):
                 inner = t.numel
                 lead = out.numel // max(inner, 1)
                 flag = ACC_PARAM_GRAD if self._grad_flag(node, t) else 0
+                if _dt(t.grad) != _dt(out.grad):
+                    flag |= PARAM_GRAD_BF16       # a bf16 bias gradient under fp32 activations
                 ws = scratch["workspace"] if scratch and "workspace" in scratch else None
                 self._launch("add_broadcast_backward", [out.grad, t.grad, ws],
                              [_dt(out)] + _lo_hi(lead) + _lo_hi(inner) + [flag]

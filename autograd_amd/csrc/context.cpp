@@ -166,7 +166,7 @@ int h_bcast_add(const Call& c) {
 int h_bcast_grad(const Call& c) {
     NEED_DTYPE(c.a[0])
     const uint64_t lead = u64(c.a, 1), inner = u64(c.a, 3), es = dtype_size(c.a[0]), wsb = u64(c.a, 6);
-    RESOLVE(0, lead * inner * es, g) RESOLVE(1, inner * es, dy)
+    RESOLVE(0, lead * inner * es, g) RESOLVE(1, inner * ((c.a[5] & AGRAD_PARAM_GRAD_BF16) ? 2 : es), dy)
     RESOLVE_IF(c.a[8] & 4u, 2, wsb, ws)
     return launch_broadcast_grad(c.ctx->stream, (int)c.a[0], g, dy, ws, ws ? wsb : 0, lead, inner, c.a[5]);
 }
@@ -414,7 +414,7 @@ int h_gather_bwd_sorted(const Call& c) {
 int h_pos_grad(const Call& c) {
     NEED_DTYPE(c.a[0])
     const uint64_t es = dtype_size(c.a[0]), tc = (uint64_t)c.a[2] * c.a[3] * es;
-    RESOLVE(0, tc * c.a[1], dY) RESOLVE(1, tc, dwpe)
+    RESOLVE(0, tc * c.a[1], dY) RESOLVE(1, (c.a[4] & AGRAD_PARAM_GRAD_BF16) ? tc / es * 2 : tc, dwpe)
     return launch_pos_embedding_bwd(c.ctx->stream, c.a[0], dY, dwpe, c.a[1], c.a[2], c.a[3], c.a[4]);
 }
 

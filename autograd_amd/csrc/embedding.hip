@@ -876,9 +876,9 @@ emb_carry_fix_kernel(const uint32_t* __restrict__ tok_s, TO* dW, const float* __
 }
 
 // dwpe[t, c] (+)= sum_b dY[b, t, c], b ascending
-template <typename T, int VEC>
+template <typename T, typename TO, int VEC>
 __global__ void __launch_bounds__(256)
-pos_grad_kernel(const T* __restrict__ dY, T* dwpe, uint32_t B, uint64_t TCV, uint64_t TC, int accumulate) {
+pos_grad_kernel(const T* __restrict__ dY, TO* dwpe, uint32_t B, uint64_t TCV, uint64_t TC, int accumulate) {
     const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= TCV) return;
     const uint64_t off = idx * VEC;
@@ -890,7 +890,7 @@ pos_grad_kernel(const T* __restrict__ dY, T* dwpe, uint32_t B, uint64_t TCV, uin
 #pragma unroll
         for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + v[k];
     }
-    store_grad_row<T, VEC>(dwpe, off, acc, accumulate != 0);
+    store_grad_row<TO, VEC>(dwpe, off, acc, accumulate != 0);
 }
 
 // AGRAD_EMB_GROUP_SORT=0 forces the radix-sort path (for comparison runs)
@@ -1202,12 +1202,16 @@ int launch_pos_embedding_bwd(hipStream_t s, int dtype, const void* dY, void* dwp
     const uint64_t n = wide ? TC / per16 : TC;
     const uint64_t grid = (n + 255) / 256;
     if (grid > 0x7fffffffull) return set_error(AGRAD_EINVAL, "position grad: table too large");
-    if (dtype == AGRAD_F32) {
-        if (wide) hipLaunchKernelGGL((pos_grad_kernel<float, 4>), dim3((uint32_t)grid), dim3(256), 0, s, (const float*)dY, (float*)dwpe, B, n, TC, acc);
-        else hipLaunchKernelGGL((pos_grad_kernel<float, 1>), dim3((uint32_t)grid), dim3(256), 0, s, (const float*)dY, (float*)dwpe, B, n, TC, acc);
+    if (flags & AGRAD_PARAM_GRAD_BF16) {        // fp32 rows summed into a bf16 table (bias_grad_reduce_bf16, metal_ops.metal:12101)
+        if (dtype != AGRAD_F32) return set_error(AGRAD_EINVAL, "position grad: AGRAD_PARAM_GRAD_BF16 goes with an fp32 upstream gradient");
+        if (wide) hipLaunchKernelGGL((pos_grad_kernel<float, bf16_t, 4>), dim3((uint32_t)grid), dim3(256), 0, s, (const float*)dY, (bf16_t*)dwpe, B, n, TC, acc);
+        else hipLaunchKernelGGL((pos_grad_kernel<float, bf16_t, 1>), dim3((uint32_t)grid), dim3(256), 0, s, (const float*)dY, (bf16_t*)dwpe, B, n, TC, acc);
+    } else if (dtype == AGRAD_F32) {
+        if (wide) hipLaunchKernelGGL((pos_grad_kernel<float, float, 4>), dim3((uint32_t)grid), dim3(256), 0, s, (const float*)dY, (float*)dwpe, B, n, TC, acc);
+        else hipLaunchKernelGGL((pos_grad_kernel<float, float, 1>), dim3((uint32_t)grid), dim3(256), 0, s, (const float*)dY, (float*)dwpe, B, n, TC, acc);
     } else {
-        if (wide) hipLaunchKernelGGL((pos_grad_kernel<bf16_t, 8>), dim3((uint32_t)grid), dim3(256), 0, s, (const bf16_t*)dY, (bf16_t*)dwpe, B, n, TC, acc);
-        else hipLaunchKernelGGL((pos_grad_kernel<bf16_t, 1>), dim3((uint32_t)grid), dim3(256), 0, s, (const bf16_t*)dY, (bf16_t*)dwpe, B, n, TC, acc);
+        if (wide) hipLaunchKernelGGL((pos_grad_kernel<bf16_t, bf16_t, 8>), dim3((uint32_t)grid), dim3(256), 0, s, (const bf16_t*)dY, (bf16_t*)dwpe, B, n, TC, acc);
+        else hipLaunchKernelGGL((pos_grad_kernel<bf16_t, bf16_t, 1>), dim3((uint32_t)grid), dim3(256), 0, s, (const bf16_t*)dY, (bf16_t*)dwpe, B, n, TC, acc);
     }
     return check_hip(hipGetLastError(), "position grad launch");
 }

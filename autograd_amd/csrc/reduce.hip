@@ -349,7 +349,7 @@ namespace {
 // finished in fp32 and rounded once
 template <typename T, int STAGE = kStageSum>
 int colsum_two_stage(hipStream_t s, const T* g, const T* x2, T* dy, void* workspace, uint64_t lead, uint64_t inner,
-                     int accumulate, const T* ysmall = nullptr, T* dx = nullptr, int acc_dx = 0) {
+                     int accumulate, const T* ysmall = nullptr, T* dx = nullptr, int acc_dx = 0, bool narrow_out = false) {
     constexpr int WIDE = WideVec<T>::value;
     float* partial = (float*)workspace;
     const bool wide = inner % WIDE == 0 && aligned16(g) && (!x2 || aligned16(x2)) && (!dx || aligned16(dx));
@@ -376,7 +376,8 @@ int colsum_two_stage(hipStream_t s, const T* g, const T* x2, T* dy, void* worksp
 #undef AGRAD_TILE_LAUNCH
     if (int rc = check_hip(hipGetLastError(), "column sum launch")) return rc;
     if constexpr (sizeof(T) == 4) {
-        return launch_colsum_finalize(s, partial, nullptr, blocks, (uint32_t)inner, (float*)dy, nullptr, accumulate);
+        // narrow_out: dy points at bf16 although the summed tensor is fp32
+        return launch_colsum_finalize(s, partial, nullptr, blocks, (uint32_t)inner, (float*)dy, nullptr, accumulate, narrow_out);
     } else {
         return launch_colsum_finalize(s, partial, nullptr, blocks, (uint32_t)inner, reinterpret_cast<float*>(dy), nullptr, accumulate, true);
     }
@@ -390,9 +391,12 @@ int launch_broadcast_grad(hipStream_t s, int dtype, const void* g, void* dy, voi
     if (inner == 0) return AGRAD_OK;
     if (dy == nullptr) return set_error(AGRAD_EINVAL, "broadcast gradient: null destination");
     if (inner >= 0x7fffffffull || lead >= 0x7fffffffull) return set_error(AGRAD_EINVAL, "broadcast gradient: tensor too large");
+    const bool narrow = (flags & AGRAD_PARAM_GRAD_BF16) != 0;      // fp32 rows summed into a bf16 gradient
+    if (narrow && dtype != AGRAD_F32)
+        return set_error(AGRAD_EINVAL, "broadcast gradient: AGRAD_PARAM_GRAD_BF16 goes with an fp32 upstream gradient");
     if (lead == 0) {
         // an empty sum: a stored gradient is zero, an accumulated one keeps its value
-        if (!(flags & AGRAD_ACC_PARAM_GRAD)) return launch_fill(s, dy, 0, (int)dtype_size(dtype), inner);
+        if (!(flags & AGRAD_ACC_PARAM_GRAD)) return launch_fill(s, dy, 0, narrow ? 2 : (int)dtype_size(dtype), inner);
         return AGRAD_OK;
     }
     if (g == nullptr) return set_error(AGRAD_EINVAL, "broadcast gradient: null operand");
@@ -406,7 +410,8 @@ int launch_broadcast_grad(hipStream_t s, int dtype, const void* g, void* dy, voi
                          (unsigned long long)workspace_bytes, (unsigned long long)need);
     if (!aligned16(workspace)) return set_error(AGRAD_EINVAL, "broadcast gradient: workspace must be 16-byte aligned");
     const int acc = (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0;
-    if (dtype == AGRAD_F32) return colsum_two_stage<float>(s, (const float*)g, nullptr, (float*)dy, workspace, lead, inner, acc);
+    if (dtype == AGRAD_F32)
+        return colsum_two_stage<float>(s, (const float*)g, nullptr, (float*)dy, workspace, lead, inner, acc, nullptr, nullptr, 0, narrow);
     return colsum_two_stage<bf16_t>(s, (const bf16_t*)g, nullptr, (bf16_t*)dy, workspace, lead, inner, acc);
 }
 

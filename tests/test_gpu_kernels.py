@@ -1045,3 +1045,47 @@ def test_norm_parameter_gradients_stored_as_bf16(ctx, kind, rows, Cw, io):
                 continue
             base = from_bf16_bits(old) if accumulate else np.zeros(Cw, np.float32)
             np.testing.assert_array_equal(got[name], to_bf16_bits(base + wide[name]), err_msg=f"{name} accumulate={accumulate}")
+
+
+@pytest.mark.parametrize("lead,inner", [(16, 384), (64, 130), (65, 384), (3000, 96), (16384, 768), (5, 7)])
+def test_bias_gradient_stored_as_bf16_under_an_fp32_upstream(ctx, lead, inner):
+    """AGRAD_PARAM_GRAD_BF16 on the broadcast-add gradient (bias_grad_reduce_bf16): the column
+    sum of fp32 rows lands in a bf16 vector -- the fp32 call's sum (plus the stored bf16
+    value when accumulating) rounded once; few rows take the direct kernel, many the two
+    stages.  Also through agrad_pos_embedding_backward."""
+    import ctypes as Ct
+    rng = _rng(95 + inner)
+    g = rng.standard_normal((lead, inner)).astype(np.float32)
+    old = to_bf16_bits(rng.standard_normal(inner).astype(np.float32))
+
+    def vp(d):
+        return Ct.c_void_p(d.ptr) if d is not None else None
+    d_g = ctx.upload(g)
+    ws_b = ctx.lib.agrad_broadcast_grad_workspace_bytes(lead, inner)
+    ws = ctx.empty((max(ws_b, 1),), np.uint8)
+    wide = ctx.zeros((inner,), np.float32)
+    ctx.call("agrad_broadcast_add_backward", capi.F32, vp(d_g), vp(wide), vp(ws) if ws_b else None, ws_b, lead, inner, 0)
+    ctx.synchronize()
+    sums = wide.download()
+    assert_fp32_close(sums, g.astype(np.float64).sum(0).astype(np.float32), "fp32 column sum", rtol=1e-5,
+                      atol=max(2e-6, 1e-4 * np.sqrt(lead / 14)))
+    for accumulate in (False, True):
+        for entry in ("agrad_broadcast_add_backward", "agrad_pos_embedding_backward"):
+            if entry == "agrad_pos_embedding_backward" and lead > 64:
+                continue                      # one thread per column walks the rows: the small-batch kernel
+            narrow = ctx.upload(old)
+            flags = capi.PARAM_GRAD_BF16 | (capi.ACC_PARAM_GRAD if accumulate else 0)
+            if entry == "agrad_broadcast_add_backward":
+                ctx.call(entry, capi.F32, vp(d_g), vp(narrow), vp(ws) if ws_b else None, ws_b, lead, inner, flags)
+            else:
+                ctx.call(entry, capi.F32, vp(d_g), vp(narrow), lead, 1, inner, flags)
+            ctx.synchronize()
+            base = from_bf16_bits(old) if accumulate else np.zeros(inner, np.float32)
+            np.testing.assert_array_equal(narrow.download(), to_bf16_bits(base + sums), err_msg=f"{entry} accumulate={accumulate}")
+            narrow.free()
+    with pytest.raises(capi.AgradError):
+        narrow = ctx.upload(old)
+        ctx.call("agrad_broadcast_add_backward", capi.BF16, vp(d_g), vp(narrow), vp(ws) if ws_b else None, ws_b, lead, inner,
+                 capi.PARAM_GRAD_BF16)
+    for d in (d_g, ws, wide):
+        d.free()

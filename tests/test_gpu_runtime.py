@@ -374,7 +374,8 @@ def test_embedding_table_with_bf16_gradient_storage():
 
 
 def test_norm_parameters_with_bf16_gradient_storage():
-    """gamma / beta with grad_dtype=BF16 under fp32 activations, on both devices"""
+    """gamma / beta and a bias under a broadcast Add with grad_dtype=BF16 under fp32
+    activations, on both devices"""
     from autograd_amd.utils import BF16
     rng = np.random.default_rng(SEED + 61)
     B, T, C = 6, 40, 96
@@ -387,12 +388,13 @@ def test_norm_parameters_with_bf16_gradient_storage():
         x = make_tensor(x_np.shape, np.float32, device, True, x_np, "x")
         g = Tensor(shape=(C,), dtype=np.float32, device=device, requires_grad=True, init_val=g_np, grad_dtype=BF16)
         b = Tensor(shape=(C,), dtype=np.float32, device=device, requires_grad=True, init_val=b_np, grad_dtype=BF16)
-        return x.relu2().layer_norm(g, b), {"x": x, "g": g, "b": b}
+        bias = Tensor(shape=(C,), dtype=np.float32, device=device, requires_grad=True, init_val=b_np, grad_dtype=BF16)
+        return x.relu2().layer_norm(g, b) + bias, {"x": x, "g": g, "b": b, "bias": bias}
 
     (c_out, c_g), (h_out, h_g) = both(build, upstream)
     assert_fp32_close(h_out[0], c_out[0], "forward", rtol=2e-5, atol=2e-6)
     assert_fp32_close(h_g["x"], c_g["x"], "x.grad", rtol=1e-4, atol=1e-5)
-    for name in ("g", "b"):
+    for name in ("g", "b", "bias"):
         assert_bf16_close(h_g[name], c_g[name], f"{name}.grad stored as bf16", rel=1.6e-2)
 
 

@@ -473,8 +473,8 @@ def test_adamw_8bit_state_on_the_oracle_device():
 
 
 def test_hip_backend_refuses_a_gradient_type_no_kernel_can_write():
-    """fp32 values with a bf16 gradient are for embedding tables and norm parameters; a bias
-    under a broadcast Add is refused when the graph is planned, not corrupted when it runs
+    """fp32 values with a bf16 gradient are for embedding tables, norm parameters and biases; the
+    second operand of a Mul is refused when the graph is planned, not corrupted when it runs
     (checked on the planning hook alone: no device is needed)"""
     from autograd_amd.backend import HipBackend
     from autograd_amd.utils import BF16
@@ -483,9 +483,10 @@ def test_hip_backend_refuses_a_gradient_type_no_kernel_can_write():
     bias = Tensor(shape=(8,), dtype=np.float32, device="hip", requires_grad=True, grad_dtype=BF16)
     for t in (x, bias):
         t.grad = Tensor(shape=t.shape, dtype=t.grad_dtype, device="hip", requires_grad=False)
-    out = x + bias
+    backend._check_gradient_storage((x + bias).op)                # a bias under a broadcast Add may
+    out = x * bias
     with pytest.raises(RuntimeError, match="another type"):
-        backend._check_gradient_storage(out.op)
+        backend._check_gradient_storage(out.op)                   # Mul's second operand may not
     gamma = Tensor(shape=(8,), dtype=np.float32, device="hip", requires_grad=True, grad_dtype=BF16)
     gamma.grad = Tensor(shape=(8,), dtype=BF16, device="hip", requires_grad=False)
     backend._check_gradient_storage(x.rms_norm(gamma).op)         # a norm parameter may
