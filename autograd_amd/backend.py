@@ -243,11 +243,12 @@ class HipBackend(Backend):
             table = isinstance(op, (GatherOp, EmbeddingSumOp)) and i >= 1
             norm_param = (isinstance(op, (LayerNormOp, RMSNormOp)) and i >= 1) or \
                          (isinstance(op, (AddLayerNormOp, AddRMSNormOp)) and i >= 2)
-            bias = isinstance(op, AddOp) and t.shape != node.outputs[0].shape and self._trailing(t.shape, node.outputs[0].shape)
+            bias = (isinstance(op, AddOp) and t.shape != node.outputs[0].shape
+                    and self._trailing(t.shape, node.outputs[0].shape)) or (isinstance(op, BiasGELUOp) and i == 1)
             if not (table or norm_param or bias) or _dt(t) != F32 or _dt(t.grad) != BF16:
                 raise RuntimeError(f"{op.op_name}: input {i} ({t.name or 'unnamed'}) stores {t.dtype} values and a "
-                                   f"{t.grad.dtype} gradient; only embedding tables, norm parameters and the broadcast "
-                                   "operand of an Add (fp32 values, bf16 gradient) can keep their gradient in another type")
+                                   f"{t.grad.dtype} gradient; only embedding tables, norm parameters and biases "
+                                   "(fp32 values, bf16 gradient) can keep their gradient in another type")
 
     def plan_scratch(self, node):
         op = node.op
@@ -631,6 +632,8 @@ class HipBackend(Backend):
             ws_bytes = ws.nbytes
             if self._grad_flag(node, b):
                 flags |= ACC_PARAM_GRAD
+            if _dt(db) != _dt(h):
+                flags |= PARAM_GRAD_BF16          # planning has checked that this is bf16 under fp32
         self._launch("gelu_backward_bias_kernel", [out.grad, h, b, dh, db, ws],
                      [_dt(h)] + _lo_hi(prod(h.shape[:-1])) + [h.shape[-1], flags] + _lo_hi(ws_bytes)
                      + [_mask(out.grad, h, b, dh, db, ws)])

@@ -324,7 +324,7 @@ int h_gelu_bias_bwd(const Call& c) {
     const uint64_t rows = u64(c.a, 1), es = dtype_size(c.a[0]), wsb = u64(c.a, 5);
     const uint64_t big = rows * c.a[3] * es, small = (uint64_t)c.a[3] * es;
     RESOLVE(0, big, dy) RESOLVE(1, big, h) RESOLVE(2, small, b) RESOLVE_IF(c.a[7] & 8u, 3, big, dh)
-    RESOLVE_IF(c.a[7] & 16u, 4, small, db) RESOLVE_IF(c.a[7] & 32u, 5, wsb, ws)
+    RESOLVE_IF(c.a[7] & 16u, 4, (c.a[4] & AGRAD_PARAM_GRAD_BF16) ? (uint64_t)c.a[3] * 2 : small, db) RESOLVE_IF(c.a[7] & 32u, 5, wsb, ws)
     return launch_gelu_bias_bwd(c.ctx->stream, (int)c.a[0], dy, h, b, dh, db, ws, ws ? wsb : 0, rows, c.a[3], c.a[4]);
 }
 // buffers gu, h | args dtype, rows, H

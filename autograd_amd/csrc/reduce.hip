@@ -636,9 +636,12 @@ int launch_gelu_bias_bwd(hipStream_t s, int dtype, const void* dy, const void* h
     if (C == 0) return AGRAD_OK;
     if (rows >= 0x7fffffffull) return set_error(AGRAD_EINVAL, "bias gelu backward: tensor too large");
     const int acc_db = (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0, acc_dh = (flags & AGRAD_ACC_INPUT_GRAD) ? 1 : 0;
+    const bool narrow = (flags & AGRAD_PARAM_GRAD_BF16) != 0;      // an fp32 tensor's bias gradient stored as bf16
+    if (narrow && dtype != AGRAD_F32)
+        return set_error(AGRAD_EINVAL, "bias gelu backward: AGRAD_PARAM_GRAD_BF16 goes with fp32 tensors");
     if (rows == 0) {
         // an empty sum: a stored bias gradient is zero, an accumulated one keeps its value
-        if (db != nullptr && !acc_db) return launch_fill(s, db, 0, (int)dtype_size(dtype), C);
+        if (db != nullptr && !acc_db) return launch_fill(s, db, 0, narrow ? 2 : (int)dtype_size(dtype), C);
         return AGRAD_OK;
     }
     if (dy == nullptr || h == nullptr || b == nullptr || (dh == nullptr && db == nullptr))
@@ -654,7 +657,7 @@ int launch_gelu_bias_bwd(hipStream_t s, int dtype, const void* dy, const void* h
     if (!aligned16(workspace)) return set_error(AGRAD_EINVAL, "bias gelu backward: workspace must be 16-byte aligned");
     if (dtype == AGRAD_F32)
         return colsum_two_stage<float, kStageGeluBias>(s, (const float*)dy, (const float*)h, (float*)db, workspace, rows, C,
-                                                       acc_db, (const float*)b, (float*)dh, acc_dh);
+                                                       acc_db, (const float*)b, (float*)dh, acc_dh, narrow);
     return colsum_two_stage<bf16_t, kStageGeluBias>(s, (const bf16_t*)dy, (const bf16_t*)h, (bf16_t*)db, workspace, rows, C,
                                                     acc_db, (const bf16_t*)b, (bf16_t*)dh, acc_dh);
 }

@@ -51,8 +51,8 @@ enum {
                                  * metal_ops.metal:12395-12446) and the norm backward (dgamma and dbeta then
                                  * point at bf16; the bf16 option of rmsnorm_weighted_dgamma and
                                  * gqa_rms_dgamma_bf16, metal_ops.metal:12448-12479, 14541-14746), and the column
-                                 * sums agrad_broadcast_add_backward / agrad_pos_embedding_backward
-                                 * (bias_grad_reduce_bf16, metal_ops.metal:12101).  A sum is finished in fp32,
+                                 * sums agrad_broadcast_add_backward / agrad_pos_embedding_backward / db of
+                                 * agrad_gelu_bias_backward (bias_grad_reduce_bf16, metal_ops.metal:12101).  A sum is finished in fp32,
                                  * added to the stored value and rounded once */
 };
 

@@ -292,6 +292,24 @@ def test_bias_gelu_forward_and_backward(ctx, rows, Cw, dtype):
                 assert_fp32_close(got, want.astype(np.float32), what + " db", rtol=1e-5,
                                   atol=max(2e-6, 1e-4 * np.sqrt(rows / 14)))
             d_db.free()
+    if dtype == "f32":
+        # the bias gradient stored as bf16: the fp32 call's sum (plus the stored value) rounded once
+        wide_db = ctx.zeros((Cw,), np.float32)
+        d_dh = ctx.upload(dh0s)
+        ctx.call("agrad_gelu_bias_backward", dt, vp(d_dy), vp(d_h), vp(d_b), vp(d_dh), vp(wide_db), vp(ws), ws_b, rows, Cw, 0)
+        ctx.synchronize()
+        sums = wide_db.download()
+        old_bits = to_bf16_bits(db0)
+        for accumulate in (False, True):
+            narrow = ctx.upload(old_bits)
+            ctx.call("agrad_gelu_bias_backward", dt, vp(d_dy), vp(d_h), vp(d_b), vp(d_dh), vp(narrow), vp(ws), ws_b, rows, Cw,
+                     capi.PARAM_GRAD_BF16 | (capi.ACC_PARAM_GRAD if accumulate else 0))
+            ctx.synchronize()
+            base = from_bf16_bits(old_bits) if accumulate else np.zeros(Cw, np.float32)
+            np.testing.assert_array_equal(narrow.download(), to_bf16_bits(base + sums))
+            narrow.free()
+        wide_db.free()
+        d_dh.free()
     for d in (d_h, d_b, d_dy, d_y, ws):
         d.free()
 
