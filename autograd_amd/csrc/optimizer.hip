@@ -218,9 +218,9 @@ int launch_adamw(hipStream_t s, int grad_dtype, float* p, const void* g, float* 
 //
 // The step is bound by vector instructions, not by memory: about 150 per element
 // (three correctly rounded divisions and a square root are 45 of them, the two code
-// searches 40), 35 M wave instructions for 12.6 M parameters = 57 us of issue time
-// on 1024 SIMDs, 66 us measured -- the time of the fp32-moment step on the same
-// parameters (58 us), for a quarter of its state memory.
+// searches 40), 33 M wave instructions for 12.6 M parameters = 54 us of issue time
+// on 1024 SIMDs, 62 us measured -- about the time of the fp32-moment step on the
+// same parameters (58 us), for a quarter of its state memory.
 
 constexpr uint64_t kAdamw8MaxGrid = 2048;     // workgroups (8 waves a SIMD; 1024 and 4096 were 10 % slower); each walks its share of the blocks
 
@@ -279,12 +279,33 @@ struct CodeTables {
     uint8_t down[kBuckets];      // x < 0 with |x| in bucket k (values in (-ceil_k, -floor_k]): starts at down[k]
 };
 
-// every thread of the workgroup; a barrier before and after belongs to the caller
+// Every thread of the workgroup; a barrier before and after belongs to the caller.  A
+// thread takes a run of neighbouring buckets: the first by bisection, the others by
+// walking on from it (the answers are monotone in the bucket and a step or two apart).
 __device__ __forceinline__ void build_tables(CodeTables& t, bool is_signed) {
-    for (uint32_t k = threadIdx.x; k < kBuckets; k += blockDim.x) {
-        t.up[k] = (uint8_t)first_not_below(t.map, bucket_floor(k));
-        if (is_signed)
-            t.down[k] = k + 1 < kBuckets ? (uint8_t)first_not_below(t.map, -bucket_floor(k + 1)) : (uint8_t)0;
+    const uint32_t per_thread = (kBuckets + blockDim.x - 1) / blockDim.x;
+    const uint32_t k0 = threadIdx.x * per_thread;
+    const uint32_t k1 = k0 + per_thread < kBuckets ? k0 + per_thread : kBuckets;
+    if (k0 >= k1) return;
+    uint32_t at = first_not_below(t.map, bucket_floor(k0));
+    t.up[k0] = (uint8_t)at;
+    for (uint32_t k = k0 + 1; k < k1; ++k) {                     // rising thresholds: walk up
+        const float edge = bucket_floor(k);
+        while (at < 255u && t.map[at] < edge) ++at;
+        t.up[k] = (uint8_t)at;
+    }
+    if (!is_signed) return;
+    // down[k] = first entry not below -bucket_floor(k + 1): falling thresholds, walk down
+    at = k0 + 1 < kBuckets ? first_not_below(t.map, -bucket_floor(k0 + 1)) : 0u;
+    t.down[k0] = (uint8_t)at;
+    for (uint32_t k = k0 + 1; k < k1; ++k) {
+        if (k + 1 < kBuckets) {
+            const float edge = -bucket_floor(k + 1);
+            while (at > 0u && !(t.map[at - 1] < edge)) --at;
+        } else {
+            at = 0u;
+        }
+        t.down[k] = (uint8_t)at;
     }
 }
 
