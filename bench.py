@@ -2,27 +2,31 @@
 """Benchmark of the fused layer-op path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config I]
-                    [--workload-only] [--no-cpu] [--iters N]
+                    [--workload-only] [--no-cpu] [--iters N] [--detail PATH]
 
 A step is one forward + backward pass of every op of the workload configuration
-(default --config 1: the nanochat d6 shape, fp32) over one batch of synthetic
-data already resident in HBM.  Prints ONE JSON line:
+(default --config 5: the Llama-3-8B-width shape with bf16 I/O, the largest
+configuration that fits one GPU) over one batch of synthetic data already resident
+in HBM.
+
+Output: one JSON line per configuration with its per-op table (every op and
+direction timed on its own with HIP events on the library's stream over rotating
+buffer sets, so the working set exceeds the 256 MB Infinity Cache; copy_us /
+vs_copy compare with a plain copy kernel moving the same number of bytes the same
+way), the same tables as one file (--detail, default gpurun_out/bench_per_op.json),
+and as the LAST line one compact JSON object:
 
   value / unit     whole-step algorithmic GB/s (sum of the ops' algorithmic bytes
                    / wall-clock step time, synchronised on both sides)
   tokens_per_s     B*T / step time
-  per_op           every op and direction of the workload, timed on its own with
-                   HIP events on the library's stream over rotating buffer sets
-                   (so the working set exceeds the 256 MB Infinity Cache);
-                   copy_us / vs_copy compare with a plain copy kernel moving the
-                   same number of bytes the same way
-  roofline         the dominant kernel of the step (largest share of time)
+  roofline         the dominant kernel of the step (largest share of time);
+                   traffic = HBM bytes per launch of that kernel from the committed
+                   counter summary profiles/hbm_traffic.json
   cpu_baseline     the numpy restatement of the reference's CPU kernels, timed
-                   on this host with the reference's protocol (2 warm-up + 5
-                   timed passes, timing_ops.py:76-100)
-  graph_replay     the launch-bound chain of config 0 launched op by op and
-                   replayed from a recorded device graph
-  all_configs      the same per-op table for the other configurations
+                   on this host with the reference's protocol (2 warm-up + >= 5
+                   timed passes, timing_ops.py:76-100) on a bounded number of rows
+  min_frac         per configuration, the op and direction furthest below the
+                   8 TB/s roofline and its fraction
 
 All device calls go through the C ABI (autograd_amd/capi.py).
 """
@@ -48,13 +52,10 @@ from autograd_amd.utils import f32_array_to_bf16_bits  # noqa: E402
 
 METRIC = "HBM GB/s (% of 8 TB/s) + tokens/s for fused norm/act/RoPE/embed fwd+bwd"
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of a workload's dominant kernel, from two `rocprofv3 --pmc`
+# HBM bytes per launch of each kernel, per configuration, from two `rocprofv3 --pmc`
 # runs of this file (FETCH_SIZE, then WRITE_SIZE), each scaled by what the counter
-# reads for the 64 MiB copy of spin_up(); the run and its numbers are recorded in
-# profiles/hbm_traffic_*.txt.  Keyed by config index, then "op direction".
-MEASURED_TRAFFIC_BYTES = {
-    1: {"relu2 bwd": 301.97e6},
-}
+# reads for the 64 MiB copy of spin_up(); the commands are recorded in the file.
+TRAFFIC_FILE = ROOT / "profiles" / "hbm_traffic.json"
 ROTATE_BYTES = 768 << 20      # cycle at least this much distinct memory per op
 MAX_SETS = 8
 
@@ -182,7 +183,7 @@ def _embed_cases(ctx, cfg, pool, rng, nbytes, ids0):
         def zero(i):
             ctx.call("agrad_fill", dW.ptr, 0, 0, 1, dW.nbytes)
 
-        cases.append(Case(name, "fwd", nbytes[name][0], k, fwd, "gather"))
+        cases.append(Case(name, "fwd", nbytes[name][0], k, fwd, "gather_sort_kernel"))
         cases.append(Case(name, "bwd", nbytes[name][1], k, bwd, "emb_segment_sum_kernel"))
         cases.append(Case(name + "_grad_zero_fill", "aux", cfg.V * Cw * e, 1, zero, "fill16_kernel"))
     return cases
@@ -260,8 +261,9 @@ def _act_cases(ctx, cfg, pool, rng, nbytes, ids0):
             def bwd(i):
                 ctx.call(b_name, dt, vp(x[i]), vp(y[i]), vp(dx[i]), n, 0)
 
-            cases.append(Case(cfg.act, "fwd", nbytes[cfg.act][0], k, fwd, "ew_kernel"))
-            cases.append(Case(cfg.act, "bwd", nbytes[cfg.act][1], k, bwd, "ew_kernel"))
+            functor = {"gelu": "Gelu", "relu2": "Relu2"}[cfg.act]
+            cases.append(Case(cfg.act, "fwd", nbytes[cfg.act][0], k, fwd, f"ew_kernel {functor}Fwd"))
+            cases.append(Case(cfg.act, "bwd", nbytes[cfg.act][1], k, bwd, f"ew_kernel {functor}Bwd"))
     return cases
 
 
@@ -490,7 +492,8 @@ def spin_up(ctx, seconds=0.25):
 
 def time_case(ctx, case, iters, exact=False):
     # at least `iters` launches and at least ~2 ms of GPU time (exactly `iters`
-    # launches when exact: a counter-collection run pays per dispatch)
+    # launches when exact: a counter-collection run pays per dispatch), timed as
+    # up to five back-to-back groups; the figure is the median group's average
     for i in range(min(case.nsets, 3)):
         case.launch(i)
     ctx.synchronize()
@@ -500,12 +503,17 @@ def time_case(ctx, case, iters, exact=False):
     probe_us = ctx.timer_stop() * 1e3 / 8
     if not exact:
         iters = int(max(iters, min(2000, 2000.0 / max(probe_us, 0.5))))
-    ctx.timer_start()
-    for it in range(iters):
-        case.launch(it % case.nsets)
-    ms = ctx.timer_stop()
+    groups = 1 if exact else min(5, max(1, iters // 6))
+    per = -(-iters // groups)
+    samples, it = [], 0
+    for _ in range(groups):
+        ctx.timer_start()
+        for _ in range(per):
+            case.launch(it % case.nsets)
+            it += 1
+        samples.append(ctx.timer_stop() * 1e3 / per)
     ctx.synchronize()
-    case.us = ms * 1e3 / iters
+    case.us = float(np.median(samples))
     return case.us
 
 
@@ -634,10 +642,15 @@ def cpu_baseline(cfg):
 
     if cfg.embed:
         ids = token_ids(cfg, rng, rows).reshape(B, T)
-        W = widen((0.02 * rng.standard_normal((cfg.V, Cw))).astype(np.float32))
+        # the table at its full [V, C] size as untouched zero pages, with values only in
+        # the rows these ids address: the CPU kernels touch nothing else, and drawing
+        # (or even zero-filling) V*C samples on one core takes minutes at the large shapes
+        W = np.zeros((cfg.V, Cw), np.float32)
+        uniq = np.unique(ids)
+        W[uniq] = widen((0.02 * rng.standard_normal((uniq.size, Cw), dtype=np.float32)).astype(np.float32))
         wpe = widen((0.02 * rng.standard_normal((T, Cw))).astype(np.float32)) if cfg.embed == "gather_sum" else None
         dY = rng.standard_normal((B, T, Cw), dtype=np.float32)
-        dW = np.zeros_like(W)
+        dW = np.zeros((cfg.V, Cw), np.float32)
         dwpe = np.zeros_like(wpe) if wpe is not None else None
 
         def emb():
@@ -702,10 +715,10 @@ def cpu_baseline(cfg):
     distinct = int(np.unique(ids).size) if cfg.embed else None
     total = sum(f + b for f, b in op_bytes(scaled, distinct).values())
     return {"value": round(total / sec / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"numpy restatement, fwd+bwd of every op at B={B} T={T} (rows {rows} of {cfg.N}), "
-                      f"2 warm-up + {passes} timed passes, {sec * 1e3:.1f} ms/pass; host {platform.processor() or platform.machine()}, "
+            "sample": f"numpy restatement of the CPU kernels, fwd+bwd of every op on rows {rows} of {cfg.N} "
+                      f"(B={B} T={T}), 2 warm-up + {passes} timed passes, {sec * 1e3:.1f} ms/pass; "
                       f"os.cpu_count()={os.cpu_count()}, numpy {np.__version__}",
-            "tokens_per_s": round(rows / sec, 1), "ms_per_pass": round(sec * 1e3, 2)}
+            "tokens_per_s": round(rows / sec, 1)}
 
 
 def LayerLike(cfg, B, T):
@@ -713,15 +726,40 @@ def LayerLike(cfg, B, T):
     return replace(cfg, B=B, T=T)
 
 
+def measured_traffic(cfg, case):
+    """HBM bytes per launch of the case's kernel from the committed counter summary:
+    entries of this configuration whose kernel name contains every word of
+    case.kernel; None when the summary has no such kernel (never a guess)"""
+    try:
+        table = json.loads(TRAFFIC_FILE.read_text())["configs"].get(str(cfg.index), {})
+    except (OSError, ValueError, KeyError):
+        return None, None
+    words = case.kernel.split()
+    hits = [(k, v) for k, v in table.items() if all(w in k for w in words)]
+    if len(hits) != 1:
+        return None, None
+    name, row = hits[0]
+    return name, int(round(row["read_bytes"] + row["written_bytes"]))
+
+
+def min_frac(rows):
+    """the op and direction of the step furthest below the roofline"""
+    step = [r for r in rows if r["dir"] in ("fwd", "bwd")]
+    worst = min(step, key=lambda r: r["frac_hbm"])
+    return [f"{worst['op']} {worst['dir']}", worst["frac_hbm"]]
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", type=int, default=1, help="index into autograd_amd.configs.CONFIGS")
+    ap.add_argument("--config", type=int, default=5, help="index into autograd_amd.configs.CONFIGS")
     ap.add_argument("--iters", type=int, default=30, help="launches per op in the per-op timing")
     ap.add_argument("--workload-only", action="store_true", help="skip the per-op tables of the other configs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--detail", default=str(ROOT / "gpurun_out" / "bench_per_op.json"),
+                    help="file that receives the per-op tables of every configuration")
     ap.add_argument("--exact-iters", action="store_true",
                     help="time each op over exactly --iters launches and shorten the clock spin-up "
                          "(for rocprofv3 --pmc runs, which serialise every dispatch)")
@@ -740,35 +778,51 @@ def main():
     timed = [c for c in cases if c.direction in ("fwd", "bwd")]
     dom = max(timed, key=lambda c: c.us)
     dom_gbps = dom.nbytes / (dom.us * 1e-6) / 1e9
+    dom_kernel, dom_traffic = measured_traffic(cfg, dom)
+
+    def title(c):
+        return f"configs[{c.index}] {c.name} ({c.dtype})"
+
+    tables = {title(cfg): [case_row(c) for c in cases]}
+    print(json.dumps({"per_op": title(cfg), "rows": tables[title(cfg)]}), flush=True)
+    detail = {"workload": title(cfg), "per_op": tables}
+    if not args.workload_only:
+        detail["graph_replay"] = graph_replay(ctx, CONFIGS[0])
+        print(json.dumps({"graph_replay": detail["graph_replay"]}), flush=True)
+        for other in CONFIGS:
+            if other.index != cfg.index:
+                tables[title(other)] = run_config(ctx, other, args.iters)
+                print(json.dumps({"per_op": title(other), "rows": tables[title(other)]}), flush=True)
+    ctx.synchronize()
+    ctx.close()
+    try:
+        Path(args.detail).parent.mkdir(parents=True, exist_ok=True)
+        Path(args.detail).write_text(json.dumps(detail, indent=1))
+    except OSError as err:
+        print(f"could not write {args.detail}: {err}", file=sys.stderr)
+
     result = {
         "metric": METRIC, "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": cfg.dtype, "data": "synthetic",
+        "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 I/O, fp32 arithmetic" if cfg.dtype == "bf16" else "f32", "data": "synthetic",
         "config": {"workload": f"configs[{cfg.index}] {cfg.name}: B={cfg.B} T={cfg.T} C={cfg.C} V={cfg.V}, "
                                f"ops {'/'.join(dict.fromkeys(c.op for c in timed))} fwd+bwd",
                    "step_MB": round(step_bytes / 1e6, 1)},
         "tokens_per_s": round(cfg.N * args.steps / wall, 1),
         "pct_of_hbm_peak": round(100 * gbps / HBM_PEAK_GBS, 2),
-        "roofline": {"bound": "hbm", "kernel": dom.kernel, "op": f"{dom.op} {dom.direction}",
+        "roofline": {"bound": "hbm", "kernel": dom_kernel or dom.kernel, "op": f"{dom.op} {dom.direction}",
                      "achieved": round(dom_gbps, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(dom_gbps / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(cfg.index, {}).get(f"{dom.op} {dom.direction}"),
+                     "frac": round(dom_gbps / HBM_PEAK_GBS, 4), "traffic": dom_traffic,
                      "launch_us": round(dom.us, 2), "algorithmic_bytes": dom.nbytes,
                      "same_bytes_copy_us": round(dom.copy_us, 2) if getattr(dom, "copy_us", None) else None},
-        "per_op": [case_row(c) for c in cases],
+        "min_frac": {t.split(" ")[0]: min_frac(rows) for t, rows in tables.items()},
     }
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(cfg)
-    if not args.workload_only:
-        result["graph_replay"] = graph_replay(ctx, CONFIGS[0])
-        others = {}
-        for other in CONFIGS:
-            if other.index != cfg.index:
-                others[f"configs[{other.index}] {other.name} ({other.dtype})"] = run_config(ctx, other, args.iters)
-        result["all_configs"] = others
-    ctx.synchronize()
-    ctx.close()
-    print(json.dumps(result))
+    line = json.dumps(result, separators=(",", ":"))
+    assert len(line) < 1800, len(line)
+    print(line, flush=True)
     return 0
 
 
