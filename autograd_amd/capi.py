@@ -21,6 +21,7 @@ ACC_INPUT_GRAD, ACC_PARAM_GRAD, ACC_INPUT_GRAD2, ACC_PARAM_GRAD2, PARAM_GRAD_BF1
 UNARY_EXP, UNARY_LOG, UNARY_RSQRT = 0, 1, 2
 MUL_SAME, MUL_ROW, MUL_COL, MUL_SCALAR = 0, 1, 2, 3
 OK, EINVAL, EHIP, ENOKERNEL, EINDEX, EWORKSPACE = 0, -1, -2, -3, -4, -5
+NOALLOC_SCRATCH_BYTES = 32 << 20
 
 _ctx = C.c_void_p
 _ptr = C.c_void_p
@@ -61,6 +62,8 @@ SIGNATURES = {
     "agrad_norm_backward_workspace_bytes": (_u64, [_u64, _u32, _int]),
     "agrad_norm_backward": (_int, [_ctx, _int, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
                                    _ptr, _u64, _u64, _u32, _f32, _u32]),
+    "agrad_norm_backward_noalloc": (_int, [_ctx, _int, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
+                                           _u64, _u32, _f32, _u32]),
     "agrad_gelu_forward": (_int, [_ctx, _int, _ptr, _ptr, _u64]),
     "agrad_gelu_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _u64, _u32]),
     "agrad_gelu_bias_forward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _u64, _u32]),

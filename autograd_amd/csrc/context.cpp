@@ -557,6 +557,7 @@ int agrad_ctx_create(int device, agrad_ctx** out) {
     if (int rc = check_hip(hipGetDeviceProperties(&prop, device), "hipGetDeviceProperties")) return rc;
     if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return set_error(AGRAD_EHIP, "device %d is %s; this library carries gfx950 code only", device, prop.gcnArchName);
+    if (int rc = norm_noalloc_setup(device)) return rc;   // this GPU's address of the fixed scratch array
     agrad_ctx* c = new agrad_ctx();
     c->device = device;
     c->total_mem = prop.totalGlobalMem;
@@ -847,6 +848,13 @@ int agrad_norm_backward(agrad_ctx* ctx, int kind, int dtype, const void* x, cons
     CTX_OR_FAIL(ctx)
     return launch_norm_bwd(ctx->stream, kind, dtype, x, dy, gamma, dres_in, dx, dx2, dgamma, dbeta,
                            workspace, workspace_bytes, rows, C, eps, flags);
+}
+int agrad_norm_backward_noalloc(agrad_ctx* ctx, int kind, int dtype, const void* x, const void* dy,
+                                const float* gamma, const void* dres_in, void* dx, void* dx2,
+                                float* dgamma, float* dbeta, uint64_t rows, uint32_t C, float eps, uint32_t flags) {
+    CTX_OR_FAIL(ctx)
+    return launch_norm_bwd_noalloc(ctx->stream, ctx->device, kind, dtype, x, dy, gamma, dres_in, dx, dx2,
+                                   dgamma, dbeta, rows, C, eps, flags);
 }
 
 int agrad_gelu_forward(agrad_ctx* ctx, int dtype, const void* x, void* y, uint64_t n) {

@@ -40,6 +40,12 @@ int launch_norm_bwd(hipStream_t s, int kind, int dtype, const void* x, const voi
                     const float* gamma, const void* dres_in, void* dx, void* dx2,
                     float* dgamma, float* dbeta, void* workspace, uint64_t workspace_bytes,
                     uint64_t rows, uint32_t C, float eps, uint32_t flags);
+// the same with the partial rows in a fixed per-GPU array instead of a workspace;
+// norm_noalloc_setup(device) runs once per GPU, with that GPU current, before it
+int norm_noalloc_setup(int device);
+int launch_norm_bwd_noalloc(hipStream_t s, int device, int kind, int dtype, const void* x, const void* dy,
+                            const float* gamma, const void* dres_in, void* dx, void* dx2,
+                            float* dgamma, float* dbeta, uint64_t rows, uint32_t C, float eps, uint32_t flags);
 
 // out_a[c] (+)= sum over the P rows of pa[P, C] (same for pb -> out_b; either pair may be null)
 // out_bf16: out_a / out_b point at bf16 elements (the sum is rounded once, after the optional accumulate)

@@ -27,6 +27,13 @@
 #include "launch.hpp"
 
 #include <cstdlib>
+#include <mutex>
+
+// Partial dgamma / dbeta rows of the entry point that allocates nothing
+// (agrad_norm_backward_noalloc): a fixed array in every GPU's memory, held until the
+// process ends.  In host code this name is only a handle for hipGetSymbolAddress;
+// the device address it yields (one per GPU) is what kernels are given.
+static __device__ __align__(256) unsigned char scratch[AGRAD_NOALLOC_SCRATCH_BYTES];
 
 namespace agrad {
 
@@ -977,6 +984,55 @@ int launch_norm_bwd(hipStream_t s, int kind, int dtype, const void* x, const voi
         return launch_colsum_finalize(s, pg, pb, grid, C, dgamma, dbeta, (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0,
                                       (flags & AGRAD_PARAM_GRAD_BF16) != 0);
     return check_hip(hipGetLastError(), "norm backward launch");
+}
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {};   // device address of `scratch` on each GPU
+}  // namespace
+
+// Called by agrad_ctx_create with `device` current: looks up, once per GPU, where
+// that GPU keeps its copy of `scratch`.
+int norm_noalloc_setup(int device) {
+    if (device < 0 || device >= kMaxDevices)
+        return set_error(AGRAD_EINVAL, "device %d beyond the %d the scratch table covers", device, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (g_scratch_ptr[device] != nullptr) return AGRAD_OK;
+    void* ptr = nullptr;
+    if (int rc = check_hip(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)"))
+        return rc;
+    if (ptr == nullptr) return set_error(AGRAD_EHIP, "hipGetSymbolAddress(scratch) returned no address");
+    g_scratch_ptr[device] = ptr;
+    return AGRAD_OK;
+}
+
+// launch_norm_bwd with the partial rows in this GPU's `scratch`.  Every partial row
+// the finalize kernel reads is written by the backward kernel of the same call, so
+// nothing has to be cleared between calls; two calls in flight on one GPU (two
+// streams, two contexts) would overwrite each other's rows.
+int launch_norm_bwd_noalloc(hipStream_t s, int device, int kind, int dtype, const void* x, const void* dy,
+                            const float* gamma, const void* dres_in, void* dx, void* dx2,
+                            float* dgamma, float* dbeta, uint64_t rows, uint32_t C, float eps, uint32_t flags) {
+    void* ptr = nullptr;
+    if (device >= 0 && device < kMaxDevices) {
+        std::lock_guard<std::mutex> lock(g_scratch_mu);
+        ptr = g_scratch_ptr[device];
+    }
+    if (ptr == nullptr) return set_error(AGRAD_EINVAL, "norm backward (no allocation): device %d was never set up", device);
+    if ((dgamma != nullptr || dbeta != nullptr) && rows > 0 && C > 0) {
+        if (dtype != AGRAD_F32 && dtype != AGRAD_BF16)
+            return set_error(AGRAD_EINVAL, "norm backward: unknown dtype %d", dtype);
+        const uint64_t need = norm_bwd_workspace_bytes(rows, C, dtype);
+        if (need > AGRAD_NOALLOC_SCRATCH_BYTES)
+            return set_error(AGRAD_EINVAL,
+                             "norm backward (no allocation): rows=%llu C=%u need %llu bytes of partial rows, the fixed "
+                             "scratch holds %llu; use agrad_norm_backward with a workspace",
+                             (unsigned long long)rows, C, (unsigned long long)need,
+                             (unsigned long long)AGRAD_NOALLOC_SCRATCH_BYTES);
+    }
+    return launch_norm_bwd(s, kind, dtype, x, dy, gamma, dres_in, dx, dx2, dgamma, dbeta, ptr,
+                           AGRAD_NOALLOC_SCRATCH_BYTES, rows, C, eps, flags);
 }
 
 }  // namespace agrad

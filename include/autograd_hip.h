@@ -228,6 +228,24 @@ int agrad_norm_backward(agrad_ctx* ctx, int kind, int dtype,
                         void* workspace, uint64_t workspace_bytes,
                         uint64_t rows, uint32_t C, float eps, uint32_t flags);
 
+/* agrad_norm_backward for callers that cannot allocate device memory (code under
+ * HIP graph capture, serving loops, harnesses that forbid hipMalloc): no workspace
+ * argument; the partial dgamma / dbeta rows go to a fixed array of
+ * AGRAD_NOALLOC_SCRATCH_BYTES that the library keeps in each GPU's memory for the
+ * life of the process, and the call makes no hipMalloc / hipFree.  Same kernels,
+ * same launch geometry and same results, bit for bit, as agrad_norm_backward.
+ * A problem whose partial rows (agrad_norm_backward_workspace_bytes(rows, C, dtype))
+ * exceed the array is refused with AGRAD_EINVAL; without dgamma and dbeta any size
+ * runs.  All calls on one GPU share the array: calls that overlap there (two
+ * contexts, or a replaying graph beside eager calls) race.  This entry point has no
+ * counterpart in the reference. */
+#define AGRAD_NOALLOC_SCRATCH_BYTES (32u * 1024u * 1024u)
+int agrad_norm_backward_noalloc(agrad_ctx* ctx, int kind, int dtype,
+                                const void* x, const void* dy, const float* gamma,
+                                const void* dres_in, void* dx, void* dx2,
+                                float* dgamma, float* dbeta,
+                                uint64_t rows, uint32_t C, float eps, uint32_t flags);
+
 /* tanh-GELU (cpu_gelu_forward / backward, backend.py:376-414).               */
 int agrad_gelu_forward(agrad_ctx* ctx, int dtype, const void* x, void* y, uint64_t n);
 int agrad_gelu_backward(agrad_ctx* ctx, int dtype, const void* x, const void* dy, void* dx, uint64_t n, uint32_t flags);
