@@ -250,9 +250,17 @@ class Runtime:
             for out_i, in_i in node.op.inplace_aliases.items():
                 src, dst = node.inputs[in_i], node.outputs[out_i]
                 # a view's memory belongs to its base, which others may still read
-                if src.op is not None and len(self.consumers.get(id(src), [])) == 1 and src is not self.loss \
-                        and id(src) not in self._view_of:
-                    self._alias_of[id(dst)] = src
+                if src.op is None or len(self.consumers.get(id(src), [])) != 1 or src is self.loss \
+                        or id(src) in self._view_of:
+                    continue
+                # The only other reader a single-consumer activation can have is its own
+                # producer's backward kernel (Exp, Rsqrt and Softmax keep their OUTPUT):
+                # overwriting it in place would feed that kernel the rotated values.
+                made_by = src.op
+                if not self.forward_only and any(t is src for t in
+                                                 made_by.op.save_for_backward(made_by.inputs, made_by.outputs)):
+                    continue
+                self._alias_of[id(dst)] = src
 
     def _root(self, t):
         """the tensor whose memory `t` lives in (views: same memory, own gradient)"""
@@ -318,6 +326,16 @@ class Runtime:
                             self._stored_leaf_grads.add(id(x.grad))
                     elif x.op is not None:
                         self.node_to_clear_grads[id(node)].append(x)
+                # A kernel has ONE store-or-accumulate choice for its parameter gradients
+                # (gamma and beta of a norm share a flag bit).  If only some of this node's
+                # leaf gradients are first written here -- a gamma tied to a later node, a
+                # beta of its own -- none of them may skip the zero fill, or the kernel
+                # would accumulate onto memory nobody cleared.
+                leaf_grads = {id(x.grad) for x in node.inputs
+                              if x.op is None and x.requires_grad and x.grad is not None}
+                if leaf_grads - overwrite:
+                    overwrite -= leaf_grads
+                    self._stored_leaf_grads -= leaf_grads
                 node.overwrite_grads = frozenset(overwrite)
 
         life = {}       # key object -> [first step, last step]

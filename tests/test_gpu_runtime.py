@@ -453,6 +453,71 @@ def test_accumulate_parameter_grads_and_rerun():
     rt.release()
 
 
+def test_tied_gamma_with_separate_betas_over_two_steps():
+    """Two LayerNorms share gamma and own a beta each.  gamma.grad is first written by the
+    later node, so the earlier one accumulates its parameter gradients -- including its own
+    beta's, which therefore must have been zero-filled: a second step gives the first
+    step's numbers again, and they are the CPU device's."""
+    rng = np.random.default_rng(SEED + 21)
+    x_np = rng.standard_normal((4, 16, 64)).astype(np.float32)
+    g_np = (1 + 0.1 * rng.standard_normal(64)).astype(np.float32)
+    up = rng.standard_normal(x_np.shape).astype(np.float32)
+    grads = {}
+    for device in ("cpu", "hip"):
+        x = make_tensor(x_np.shape, np.float32, device, True, x_np)
+        gamma = make_tensor((64,), np.float32, device, True, g_np)
+        beta_a = make_tensor((64,), np.float32, device, True, np.zeros(64, np.float32))
+        beta_b = make_tensor((64,), np.float32, device, True, np.zeros(64, np.float32))
+        out = LayerNormOp(eps=1e-5)(GELUOp()(LayerNormOp(eps=1e-5)(x, gamma, beta_a)), gamma, beta_b)
+        rt = Runtime(device=device)
+        rt.loss = out
+        rt.build_topo(out)
+        rt.bind_memory()
+        steps = []
+        for _ in range(2):
+            rt.forward()
+            rt.zero_grad()
+            rt.backend.copy_from_host(out.grad, up)
+            rt.backward_graph()
+            rt.backend.synchronize()
+            steps.append({k: rt.backend.copy_to_host(t.grad) for k, t in
+                          (("x", x), ("gamma", gamma), ("beta_a", beta_a), ("beta_b", beta_b))})
+        for k in steps[0]:
+            np.testing.assert_array_equal(steps[1][k], steps[0][k], err_msg=f"{device}: {k}.grad changed on step 2")
+        grads[device] = steps[1]
+        rt.release()
+    for k in grads["cpu"]:
+        assert_fp32_close(grads["hip"][k], grads["cpu"][k], f"{k}.grad", atol=4e-6)
+
+
+def test_rope_after_an_op_that_saves_its_output():
+    """q = exp(x) is read again by Exp's backward, so Rope must not rotate it in place."""
+    from autograd_amd.op import ExpOp
+    rng = np.random.default_rng(SEED + 22)
+    B, T, H, D = 2, 8, 2, 64
+    x_np = (0.5 * rng.standard_normal((B, T, H, D))).astype(np.float32)
+    k_np = rng.standard_normal((B, T, H, D)).astype(np.float32)
+    cos_np, sin_np = ref.rope_tables(T, D, 1e4)
+    up = rng.standard_normal((B, T, H, D)).astype(np.float32)
+
+    def build(device):
+        x = make_tensor(x_np.shape, np.float32, device, True, x_np)
+        k = make_tensor(k_np.shape, np.float32, device, True, k_np)
+        c = make_tensor(cos_np.shape, np.float32, device, False, cos_np)
+        s = make_tensor(sin_np.shape, np.float32, device, False, sin_np)
+        q2, k2 = RopeOp(rope_sign=1)(ExpOp()(x), GELUOp()(k), c, s)
+        return AddOp()(q2, k2), {"x": x, "k": k}
+
+    (c_out, c_g), (h_out, h_g) = both(build, up)
+    assert_fp32_close(h_out[0], c_out[0], "forward")
+    assert_fp32_close(h_g["x"], c_g["x"], "x.grad through exp", atol=2e-6)
+    assert_fp32_close(h_g["k"], c_g["k"], "k.grad through gelu", atol=3e-6)
+    # and against the formula: d/dx of rope(exp(x)) is rope^T(up) * exp(x)
+    back = up.copy()
+    ref.rope_signed(back, np.zeros_like(back), cos_np, sin_np, 1, True)
+    assert_fp32_close(h_g["x"], back * np.exp(x_np), "x.grad closed form", rtol=2e-5, atol=2e-6)
+
+
 def test_add_with_a_broadcast_operand():
     """x[B, T, C] + bias[C] and + table[T, C]: forward and both gradients through the
     runtime on both devices (the broadcasting branch of cpu_add_backward,

@@ -381,6 +381,62 @@ def test_runtime_arena_views_and_execution_on_oracle_device():
     assert h2.grad is None and y2.grad is not None
 
 
+def test_partly_first_written_parameter_grads_are_all_zero_filled():
+    """Two LayerNorms share gamma and have their own betas.  The backward kernel has one
+    store-or-accumulate choice for (dgamma, dbeta), and gamma's gradient is first written
+    by the LATER node (backward runs in reverse), so the earlier node must accumulate --
+    and then its own beta's gradient has to be zero-filled like everything else."""
+    rng = np.random.default_rng(5)
+    x_np = rng.standard_normal((4, 8, 16)).astype(np.float32)
+    g_np = (1 + 0.1 * rng.standard_normal(16)).astype(np.float32)
+    x = T(x_np.shape, val=x_np)
+    gamma = T((16,), val=g_np)
+    beta_a, beta_b = T((16,), val=np.zeros(16, np.float32)), T((16,), val=np.zeros(16, np.float32))
+    a = LayerNormOp(eps=1e-5)(x, gamma, beta_a)
+    out = LayerNormOp(eps=1e-5)(a.gelu(), gamma, beta_b)
+    rt = Runtime(device="cpu")
+    rt.fuse_grad_zeroing = True        # the first-writer analysis as the hip device runs it (planning only)
+    rt.loss = out
+    rt.build_topo(out)
+    rt.plan_memory()
+    first, last = rt.topo[0], rt.topo[-1]
+    assert first.inputs[2] is beta_a and last.inputs[2] is beta_b
+    # the last node writes gamma.grad and beta_b.grad first: both may be stored
+    assert {id(gamma.grad), id(beta_b.grad)} <= last.overwrite_grads
+    # the first node accumulates onto gamma.grad, so beta_a.grad may not skip its fill
+    assert id(gamma.grad) not in first.overwrite_grads
+    assert id(beta_a.grad) not in first.overwrite_grads
+    assert id(beta_a.grad) not in rt._stored_leaf_grads
+    assert id(x.grad) not in first.overwrite_grads        # x is a leaf of the same node: same treatment
+
+
+def test_inplace_op_leaves_a_tensor_its_producer_saved_alone():
+    """Rope rotates its input in place when nobody else reads it -- but Exp's backward
+    reads Exp's OUTPUT, so q = exp(x) must keep its values and Rope gets its own memory."""
+    rng = np.random.default_rng(6)
+    B, Tn, H, D = 1, 4, 2, 8
+    x = T((B, Tn, H, D), val=rng.standard_normal((B, Tn, H, D)).astype(np.float32))
+    k = T((B, Tn, H, D), val=rng.standard_normal((B, Tn, H, D)).astype(np.float32))
+    from oracle import cpu_ops
+    cos_np, sin_np = cpu_ops.rope_tables(Tn, D, 1e4)
+    cos, sin = T(cos_np.shape, requires_grad=False, val=cos_np), T(sin_np.shape, requires_grad=False, val=sin_np)
+    q = x.exp()
+    kk = k.gelu()                      # GELU saves its input, not kk: kk may be rotated in place
+    q2, k2 = RopeOp(rope_sign=1)(q, kk, cos, sin)
+    out = q2 + k2
+    rt = Runtime(device="cpu")
+    rt.loss = out
+    rt.build_topo(out)
+    rt._resolve_aliases()
+    assert id(q2) not in rt._alias_of
+    assert rt._alias_of.get(id(k2)) is kk
+    fwd_only = Runtime(device="cpu", forward_only=True)
+    fwd_only.loss = out
+    fwd_only.build_topo(out)
+    fwd_only._resolve_aliases()
+    assert fwd_only._alias_of.get(id(q2)) is q       # nothing is read back without a backward pass
+
+
 def test_runtime_rejects_ops_without_kernels():
     class Bare(GELUOp):
         pass
