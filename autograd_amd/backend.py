@@ -292,7 +292,7 @@ class HipBackend(Backend):
                 n = prod(ids.shape)
                 if len(node.outputs) > 1:
                     return (single_slot("sort_workspace", self.ctx.embedding_sort_workspace_bytes(n, w.shape[0])),
-                            single_slot("workspace", self.ctx.embedding_backward_sorted_workspace_bytes(n, w.shape[1])))
+                            single_slot("workspace", max(256, self.ctx.embedding_backward_sorted_workspace_bytes(n, w.shape[1]))))
                 nbytes = self.ctx.embedding_backward_workspace_bytes(n, w.shape[1], w.shape[0], _dt(w))
                 return None, single_slot("workspace", nbytes)
         return None, None

@@ -158,6 +158,19 @@ template <> struct RawVec<bf16_t, 8> {
     }
 };
 
+template <> struct RawVec<float, 1> {
+    typedef float type;
+    static __device__ __forceinline__ type load(const float* p) { return __builtin_nontemporal_load(p); }
+    static __device__ __forceinline__ type zero() { return 0.0f; }
+    static __device__ __forceinline__ void unpack(const type& r, float (&v)[1]) { v[0] = r; }
+};
+template <> struct RawVec<bf16_t, 1> {
+    typedef bf16_t type;
+    static __device__ __forceinline__ type load(const bf16_t* p) { return __builtin_nontemporal_load(p); }
+    static __device__ __forceinline__ type zero() { return 0; }
+    static __device__ __forceinline__ void unpack(const type& r, float (&v)[1]) { v[0] = bf16_bits_to_f32(r); }
+};
+
 // Widest vector a dtype supports (16 bytes).
 template <typename T> struct WideVec;
 template <> struct WideVec<float>  { static constexpr int value = 4; };

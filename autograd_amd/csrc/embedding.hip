@@ -6,20 +6,17 @@
 // Backward dW[ids[n],:] += dY[n,:] (np.add.at, backend.py:531-538) is done
 // without float atomics:
 //   1. (token, row) pairs are ordered so that each token's rows form one run,
-//      in ascending row order.  Up to 65536 rows this is ONE launch: every
-//      workgroup owns a hash group of tokens, scans all ids for its own, and
-//      orders its pairs in LDS (runs of distinct tokens then follow hash-group
-//      order, which is all the later steps need).  Larger inputs take a stable
-//      LSD radix sort by token (rocPRIM);
-//   2. the sorted order is cut into chunks of L positions, one workgroup each;
-//      a workgroup sums every run inside its chunk in order (fp32) and stores
-//      it straight to dW when the run lies wholly inside the chunk;
-//   3. a run that crosses a chunk edge leaves fp32 partial rows in a carry
-//      buffer; a second kernel adds the partial rows of such a run in a fixed
-//      order and stores the total (a hot token's many partial rows are shared
-//      out over the run's own middle chunks).
-// Every sum has a fixed order, so the result is run-to-run identical, and runs
-// inside one chunk are bit-identical to the sequential CPU sum.
+//      in ascending row order, and every row learns its place in that order.
+//      Up to 65536 rows this is ONE launch: every workgroup owns a hash group of
+//      tokens, scans all ids for its own, and orders its pairs in LDS (runs of
+//      distinct tokens then follow hash-group order, which is all the next step
+//      needs).  Larger inputs take a stable LSD radix sort by token (rocPRIM);
+//   2. one launch walks dY in row order: the first row of a token's run adds the
+//      run's rows in ascending order and stores the table row; a long run (a
+//      frequent token) is shared out by column slab among its first rows'
+//      workgroups.  Every table row is written once, by one workgroup.
+// Every sum has a fixed order, so the result is run-to-run identical, and runs of
+// up to 16 rows are bit-identical to the sequential CPU sum.
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -33,10 +30,6 @@ namespace agrad {
 namespace {
 
 constexpr int kGatherBlock = 256;
-constexpr int kBatch = 8;          // rows a thread keeps in flight in the segmented sum
-constexpr uint32_t kMaxChunks = 2048;        // chunks of the segmented sum ...
-constexpr uint32_t kMaxChunksLarge = 1024;   // ... and from kLargeRows rows on: longer chunks, fewer carry rows to fix up
-constexpr uint64_t kLargeRows = 65536;
 
 inline uint64_t align256(uint64_t v) { return (v + 255) & ~255ull; }
 
@@ -221,15 +214,35 @@ __device__ __forceinline__ void bitonic_sort_u64(unsigned long long* keys, uint3
     }
 }
 
+// What a row is told about its token's run: the token, the position in the order where
+// the run starts, the row's index within the run (rows ascend with it) and the run's length.
+struct __attribute__((aligned(16))) RunInfo { uint32_t tok, start, j, R; };
+
+// smallest index in sorted keys[0..n) whose key is not below `bound`
+__device__ __forceinline__ uint32_t first_not_below(const unsigned long long* keys, uint32_t n, unsigned long long bound) {
+    uint32_t lo = 0, hi = n;
+    while (lo < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (keys[mid] < bound) lo = mid + 1; else hi = mid;
+    }
+    return lo;
+}
+
 // the work of workgroup `g` of the grouping sort (kSortBlock threads)
 __device__ __forceinline__ void
-emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __restrict__ tok_s,
-                    uint32_t* __restrict__ row_s, unsigned long long* __restrict__ spill,
+emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __restrict__ row_s,
+                    RunInfo* __restrict__ info, unsigned long long* __restrict__ spill,
                     uint32_t N, uint32_t V, uint32_t log2G, int* err_flag) {
     __shared__ unsigned long long keys[kSortLdsEntries];
     __shared__ unsigned long long few[kRankSortMax];
     __shared__ uint32_t row_map[kRowMapWords];
     __shared__ uint32_t s_count, s_less, s_rest, s_below, s_wave_rows[kSortWaves];
+    // a pair leaves for the order: its row at position `at`, and what the row is told about
+    // its token's run (where the run starts, the row's index in it, its length)
+    auto emit = [&](uint32_t tok, uint32_t row, uint32_t at, uint32_t j, uint32_t R) {
+        row_s[at] = row;
+        info[row] = RunInfo{tok, at - j, j, R};
+    };
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & (kWave - 1);
     auto lanes_below = [&](unsigned long long mask) {     // set bits of `mask` below this lane
@@ -312,13 +325,17 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
         // smaller keys.  Each thread counts that for its own key with broadcast
         // LDS reads -- no barriers, no exchanges.
         const unsigned long long mine = tid < count ? keys[tid] : ~0ull;
-        uint32_t rank = 0;
+        const uint32_t my_tok = (uint32_t)(mine >> 32);
+        uint32_t rank = 0, same = 0, same_before = 0;       // ... and its run: the keys with its token
 #pragma unroll 8
-        for (uint32_t j = 0; j < count; ++j) rank += keys[j] < mine ? 1u : 0u;
-        if (tid < count) {
-            tok_s[offset + rank] = (uint32_t)(mine >> 32);
-            row_s[offset + rank] = (uint32_t)mine;
+        for (uint32_t j = 0; j < count; ++j) {
+            const unsigned long long k = keys[j];
+            const bool smaller = k < mine, same_tok = (uint32_t)(k >> 32) == my_tok;
+            rank += smaller ? 1u : 0u;
+            same += same_tok ? 1u : 0u;
+            same_before += same_tok && smaller ? 1u : 0u;
         }
+        if (tid < count) emit(my_tok, (uint32_t)mine, offset + rank, same_before, same);
         return;
     }
 
@@ -394,8 +411,10 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
             bitonic_sort_u64<kSortBlock>(keys, count, tid, [] { __syncthreads(); });
             for (uint32_t i = tid; i < count; i += kSortBlock) {
                 const unsigned long long key = keys[i];
-                tok_s[offset + i] = (uint32_t)(key >> 32);
-                row_s[offset + i] = (uint32_t)key;
+                const uint32_t tok = (uint32_t)(key >> 32);
+                const uint32_t lo = first_not_below(keys, count, (unsigned long long)tok << 32);
+                const uint32_t hi = first_not_below(keys, count, (unsigned long long)(tok + 1u) << 32);
+                emit(tok, (uint32_t)key, offset + i, i - lo, hi - lo);
             }
             return;
         }
@@ -414,8 +433,10 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
         bitonic_sort_u64<kSortBlock>(mine, count, tid, [] { __threadfence_block(); __syncthreads(); });
         for (uint32_t i = tid; i < count; i += kSortBlock) {
             const unsigned long long key = mine[i];
-            tok_s[offset + i] = (uint32_t)(key >> 32);
-            row_s[offset + i] = (uint32_t)key;
+            const uint32_t tok = (uint32_t)(key >> 32);
+            const uint32_t lo = first_not_below(mine, count, (unsigned long long)tok << 32);
+            const uint32_t hi = first_not_below(mine, count, (unsigned long long)(tok + 1u) << 32);
+            emit(tok, (uint32_t)key, offset + i, i - lo, hi - lo);
         }
         return;
     }
@@ -426,14 +447,16 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
     if (rest_n <= kRankSortMax) {
         const unsigned long long mine = tid < rest_n ? rest[tid] : ~0ull;
         const uint32_t tok = (uint32_t)(mine >> 32);
-        uint32_t rank = 0;
+        uint32_t rank = 0, same = 0, same_before = 0;
 #pragma unroll 8
-        for (uint32_t j = 0; j < rest_n; ++j) rank += rest[j] < mine ? 1u : 0u;
-        if (tid < rest_n) {
-            const uint32_t at = offset + rank + (tok > hot ? hot_rows : 0u);
-            tok_s[at] = tok;
-            row_s[at] = (uint32_t)mine;
+        for (uint32_t j = 0; j < rest_n; ++j) {
+            const unsigned long long k = rest[j];
+            const bool smaller = k < mine, same_tok = (uint32_t)(k >> 32) == tok;
+            rank += smaller ? 1u : 0u;
+            same += same_tok ? 1u : 0u;
+            same_before += same_tok && smaller ? 1u : 0u;
         }
+        if (tid < rest_n) emit(tok, (uint32_t)mine, offset + rank + (tok > hot ? hot_rows : 0u), same_before, same);
         below = (uint32_t)__syncthreads_count(tid < rest_n && tok < hot);
     } else {
         bitonic_sort_u64<kSortBlock>(rest, rest_n, tid, [] { __syncthreads(); });
@@ -442,9 +465,9 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
             const unsigned long long key = rest[i];
             const uint32_t tok = (uint32_t)(key >> 32);
             n_below += tok < hot ? 1u : 0u;
-            const uint32_t at = offset + i + (tok > hot ? hot_rows : 0u);
-            tok_s[at] = tok;
-            row_s[at] = (uint32_t)key;
+            const uint32_t lo = first_not_below(rest, rest_n, (unsigned long long)tok << 32);
+            const uint32_t hi = first_not_below(rest, rest_n, (unsigned long long)(tok + 1u) << 32);
+            emit(tok, (uint32_t)key, offset + i + (tok > hot ? hot_rows : 0u), i - lo, hi - lo);
         }
         if (n_below) atomicAdd(&s_below, n_below);
         __syncthreads();
@@ -483,8 +506,7 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
         const uint32_t word = upper ? word1 : word0;
         if ((word >> bit) & 1u) {
             const uint32_t to = at + (upper ? n0 : 0u) + (uint32_t)__popc(word & ((1u << bit) - 1u));
-            tok_s[to] = hot;
-            row_s[to] = (w0 + upper) * 32u + bit;
+            emit(hot, (w0 + upper) * 32u + bit, to, to - (offset + below), hot_rows);
         }
         at += n0 + (uint32_t)__popc(word1);
     }
@@ -503,10 +525,10 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
 inline uint32_t group_sort_log2g(uint32_t n) { return n > 32768 ? 9u : n > 16384 ? 8u : n > 1024 ? 7u : 4u; }
 
 __global__ void __launch_bounds__(kSortBlock)
-emb_group_sort_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ tok_s,
-                      uint32_t* __restrict__ row_s, unsigned long long* __restrict__ spill,
+emb_group_sort_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ row_s,
+                      RunInfo* __restrict__ info, unsigned long long* __restrict__ spill,
                       uint32_t N, uint32_t V, uint32_t log2G, int* err_flag) {
-    emb_group_sort_body(blockIdx.x, ids, tok_s, row_s, spill, N, V, log2G, err_flag);
+    emb_group_sort_body(blockIdx.x, ids, row_s, info, spill, N, V, log2G, err_flag);
 }
 
 // Forward gather and the ordering of the ids for the later gradient in ONE
@@ -524,11 +546,11 @@ template <typename T, int VEC, bool RAW>
 __global__ void __launch_bounds__(kSortBlock) __attribute__((amdgpu_num_sgpr(80)))
 gather_sort_kernel(const int32_t* __restrict__ ids, const T* __restrict__ W, const T* __restrict__ wpe,
                    T* __restrict__ out, uint32_t total, uint32_t CV, uint32_t C, uint32_t T_len, uint32_t V,
-                   uint32_t* __restrict__ tok_s, uint32_t* __restrict__ row_s, unsigned long long* __restrict__ spill,
+                   uint32_t* __restrict__ row_s, RunInfo* __restrict__ info, unsigned long long* __restrict__ spill,
                    uint32_t N, uint32_t log2G, int* err_flag) {
     const uint32_t groups = 1u << log2G;
     if (blockIdx.x < groups) {
-        emb_group_sort_body(blockIdx.x, ids, tok_s, row_s, spill, N, V, log2G, err_flag);
+        emb_group_sort_body(blockIdx.x, ids, row_s, info, spill, N, V, log2G, err_flag);
         return;
     }
     const uint32_t idx = (blockIdx.x - groups) * kSortBlock + threadIdx.x;
@@ -550,50 +572,6 @@ gather_sort_kernel(const int32_t* __restrict__ ids, const T* __restrict__ W, con
     }
 }
 
-struct ChunkEdges {
-    uint32_t start, end;
-    bool open_left, open_right, single;
-};
-
-__device__ __forceinline__ ChunkEdges chunk_edges(const uint32_t* tok_s, uint32_t chunk, uint32_t L, uint32_t N) {
-    ChunkEdges e;
-    e.start = chunk * L;
-    e.end = e.start + L < N ? e.start + L : N;
-    const uint32_t first_tok = tok_s[e.start];
-    const uint32_t last_tok = tok_s[e.end - 1];
-    e.open_left = e.start > 0 && tok_s[e.start - 1] == first_tok;
-    e.open_right = e.end < N && tok_s[e.end] == last_tok;
-    e.single = first_tok == last_tok;
-    return e;
-}
-
-// VEC consecutive floats of a carry row (fp32 partial sums in the workspace): as
-// 16-byte accesses when VEC is a multiple of 4 (the rows are 16-byte aligned and
-// col is a multiple of VEC then), cached -- the fix-up kernel re-reads them at once
-template <int VEC>
-__device__ __forceinline__ void load_carry(const float* __restrict__ p, float (&v)[VEC]) {
-    if constexpr (VEC % 4 == 0) {
-#pragma unroll
-        for (int k = 0; k < VEC; k += 4) {
-            const float4 t = *reinterpret_cast<const float4*>(p + k);
-            v[k] = t.x; v[k + 1] = t.y; v[k + 2] = t.z; v[k + 3] = t.w;
-        }
-    } else {
-#pragma unroll
-        for (int k = 0; k < VEC; ++k) v[k] = p[k];
-    }
-}
-template <int VEC>
-__device__ __forceinline__ void store_carry(float* __restrict__ p, const float (&v)[VEC]) {
-    if constexpr (VEC % 4 == 0) {
-#pragma unroll
-        for (int k = 0; k < VEC; k += 4) *reinterpret_cast<float4*>(p + k) = make_float4(v[k], v[k + 1], v[k + 2], v[k + 3]);
-    } else {
-#pragma unroll
-        for (int k = 0; k < VEC; ++k) p[k] = v[k];
-    }
-}
-
 template <typename T, int VEC>
 __device__ __forceinline__ void store_grad_row(T* dW, uint64_t off, const float (&acc)[VEC], bool accumulate) {
     float o[VEC];
@@ -608,271 +586,233 @@ __device__ __forceinline__ void store_grad_row(T* dW, uint64_t off, const float 
     VecIO<T, VEC>::store(dW + off, o);
 }
 
-// One workgroup per chunk of L sorted positions; thread j owns column vectors
-// j, j + blockDim, ...  Control flow depends only on the (uniform) token run
-// structure, so a workgroup never diverges except on the column mask.
-// T is the upstream gradient's storage type, TO the table gradient's: the same, or
-// bf16 under an fp32 upstream (gather_backward_bf16_kernel, metal_ops.metal:12395-12446:
-// the row sum is finished in fp32, added to the stored bf16 value and rounded once).
+// The gradient sum proper, in ROW order.  A workgroup takes kRowBatch consecutive rows of
+// dY (or, with a position table, the B rows b*T + t of one position t, a batch at a
+// time); a thread takes one column vector.  One 16-byte scalar load tells a row what it
+// is (RunInfo, written by the ordering step):
+//   * the first row of its token's run (the lowest row number) when the run has up to
+//     kSoloRun rows: it adds the run's rows in ascending order -- the very sequence of
+//     fp32 adds np.add.at makes -- and stores the table row.  Most rows are their token's
+//     only row and just move their vector; a batch keeps all of its rows in flight.
+//   * a row of a LONGER run (a frequent token: padding, "the").  S evenly spaced rows of
+//     the run are its workers; worker w sums column slab w over all of the run's rows,
+//     its threads laid out as columns x row lanes: a lane adds every lanes-th row in
+//     ascending order with kLongBatch loads in flight, and the lanes are then added in
+//     lane order.  A fixed association: the same bits on every run.
+//   * any other row: nothing to do for the table.
+// dY is read front to back, every row of dW is written once, by one workgroup: no
+// atomics, no partial sums in memory, no second launch.  With a position table the
+// workgroup also adds its B rows' vectors in ascending b, from the same loads:
+// dwpe[t, :] (+)= sum_b dY[b, t, :].
+constexpr int kRowBatch = 8;          // rows of a workgroup, all in flight together
+constexpr int kLongBatch = 8;         // rows a lane of a long run's slab keeps in flight
+constexpr uint32_t kSoloRun = 16;     // longest run its first row's workgroup sums alone
+constexpr uint32_t kMaxSlabs = 64;    // most workgroups sharing a longer run
+constexpr int kRowSumMaxBlock = 512;
+
+// Column vectors per slab of a run of R rows: at least a 64th of the row and at least a
+// row's share when the run has fewer rows than that; otherwise `min_slab` (whole cache
+// lines per access), narrowed when the run is so long that a lane would otherwise walk
+// more than a few batches of rows.
+__device__ __forceinline__ uint32_t slab_width(uint32_t R, uint32_t CV, uint32_t block, uint32_t min_slab) {
+    const uint32_t w_min = (CV + kMaxSlabs - 1) / kMaxSlabs;
+    const uint32_t w_rows = (CV + R - 1) / R;
+    uint32_t w_lat = (uint32_t)(((uint64_t)4 * kLongBatch * block) / R);
+    w_lat = w_lat ? w_lat : 1u;
+    uint32_t width = min_slab < w_lat ? min_slab : w_lat;
+    width = width > w_min ? width : w_min;
+    width = width > w_rows ? width : w_rows;
+    return width;
+}
+
+// Slab `w` of a long run: rows row_s[start .. start + R) of dY, summed for one band of
+// columns by the whole workgroup (every thread calls it with the same arguments).
 template <typename T, typename TO, int VEC>
-__global__ void __launch_bounds__(512)
-emb_segment_sum_kernel(const uint32_t* __restrict__ tok_s, const uint32_t* __restrict__ row_s,
-                       const T* __restrict__ dY, TO* dW, float* __restrict__ carry_head,
-                       float* __restrict__ carry_tail, uint32_t N, uint32_t C, uint32_t CV,
-                       uint32_t V, uint32_t L, int accumulate, uint32_t chunks, TO* dwpe, uint32_t B,
-                       uint32_t T_len, int accumulate_pos) {
-    if (blockIdx.x >= chunks) {
-        // Workgroups past the chunks (present only when a position table wants its
-        // gradient) add dY over the batch, b ascending: dwpe[t, :] (+)= sum_b dY[b, t, :].
-        // Independent of the token sums, so it rides in the same launch.
-        const uint64_t TC = (uint64_t)T_len * C;
-        const uint64_t idx = (uint64_t)(blockIdx.x - chunks) * blockDim.x + threadIdx.x;
-        if (idx * VEC >= TC) return;
-        const uint64_t off = idx * VEC;
-        float acc[VEC];
-        VecIO<T, VEC>::load(dY + off, acc);
-        for (uint32_t b = 1; b < B; ++b) {
-            float v[VEC];
-            VecIO<T, VEC>::load(dY + (uint64_t)b * TC + off, v);
-#pragma unroll
-            for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + v[k];
-        }
-        store_grad_row<TO, VEC>(dwpe, off, acc, accumulate_pos != 0);
-        return;
-    }
-    const ChunkEdges e = chunk_edges(tok_s, blockIdx.x, L, N);
-    for (uint32_t cv = threadIdx.x; cv < CV; cv += blockDim.x) {
-        const uint32_t col = cv * VEC;
-        float acc[VEC];
-        uint32_t cur = tok_s[e.start];
-        bool run_is_first = true;
-        bool have = false;
-        for (uint32_t p0 = e.start; p0 < e.end; p0 += kBatch) {
-            float v[kBatch][VEC];
-            uint32_t tk[kBatch];
-#pragma unroll
-            for (int b = 0; b < kBatch; ++b) {
-                const uint32_t p = p0 + b;
-                if (p < e.end) {
-                    tk[b] = tok_s[p];
-                    VecIO<T, VEC>::load(dY + (uint64_t)row_s[p] * C + col, v[b]);
-                }
-            }
-#pragma unroll
-            for (int b = 0; b < kBatch; ++b) {
-                const uint32_t p = p0 + b;
-                if (p < e.end) {
-                    if (have && tk[b] == cur) {
-#pragma unroll
-                        for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + v[b][k];
-                    } else {
-                        if (have && cur < V) {
-                            // the finished run cannot touch the chunk's right edge
-                            if (run_is_first && e.open_left) {
-                                store_carry<VEC>(carry_head + (uint64_t)blockIdx.x * C + col, acc);
-                            } else {
-                                store_grad_row<TO, VEC>(dW, (uint64_t)cur * C + col, acc, accumulate != 0);
-                            }
-                        }
-                        if (have) run_is_first = false;
-                        cur = tk[b];
-                        have = true;
-#pragma unroll
-                        for (int k = 0; k < VEC; ++k) acc[k] = v[b][k];
-                    }
-                }
-            }
-        }
-        // the last run ends at the chunk's right edge
-        if (have && cur < V) {
-            if (run_is_first && e.open_left) {
-                store_carry<VEC>(carry_head + (uint64_t)blockIdx.x * C + col, acc);
-            } else if (e.open_right) {
-                store_carry<VEC>(carry_tail + (uint64_t)blockIdx.x * C + col, acc);
-            } else {
-                store_grad_row<TO, VEC>(dW, (uint64_t)cur * C + col, acc, accumulate != 0);
-            }
-        }
-    }
-}
-
-// A run that crosses chunk edges starts as the tail partial of its first chunk
-// (its origin) and continues as head partials of the following chunks.  One
-// workgroup per chunk:
-//   * a run with at most kFixLanes head partials (every run of a spread-out
-//     token distribution) is finished by its origin, a thread per column;
-//   * a long run -- a hot token under a Zipf distribution spans hundreds of
-//     chunks -- is finished slab by slab (kFixCols column vectors each).  The
-//     chunks in the middle of the run have nothing else to do, so middle chunk
-//     i takes slab i and the origin takes the slabs left over.  Within a slab,
-//     kFixLanes lanes per column each add every kFixLanes-th partial in chunk
-//     order with kFixBatch loads in flight, and the lanes are then added in
-//     lane order: a fixed association, the same on every run.
-// Run ends come from binary searches on "equals this token" over the sorted
-// positions (equal tokens are contiguous whichever sorter ran).
-// One end of the run of `tok` that position `at` touches, found by the whole
-// workgroup (every thread must call it, with the same arguments).
-//   FORWARD:  tok_s[at - 1] == tok; returns the smallest p >= at with p == N or tok_s[p] != tok.
-//   backward: tok_s[at] == tok;     returns the smallest p <= at with tok_s[p..at] all == tok.
-// Each step probes blockDim.x evenly spaced positions of the bracket (the first
-// step takes the positions next to `at`, where most runs end) and counts the
-// probes that still see the token: equal tokens are contiguous, so those are the
-// probes nearest to `at`.
-template <bool FORWARD>
-__device__ __forceinline__ uint32_t run_edge(const uint32_t* __restrict__ tok_s, uint32_t tok, uint32_t at, uint32_t N) {
-    const uint32_t nt = blockDim.x;
-    // distance from `at` (0, 1, 2, ... outwards) of the first position that is not `tok`, in [lo, hi]
-    uint32_t lo = FORWARD ? 0u : 1u;
-    uint32_t hi = FORWARD ? N - at : at + 1;     // at distance hi the array ends
-    uint32_t step = 1;
-    while (lo < hi) {
-        const uint64_t d = (uint64_t)lo + (uint64_t)threadIdx.x * step;   // probes lo, lo + step, ...
-        int same = 0;
-        if (d < hi) same = tok_s[FORWARD ? at + (uint32_t)d : at - (uint32_t)d] == tok;
-        const uint32_t cnt = (uint32_t)__syncthreads_count(same);
-        // probes 0 .. cnt-1 see the token, probe cnt (if any) does not
-        const uint32_t new_lo = cnt ? lo + (cnt - 1) * step + 1 : lo;
-        const uint64_t cap = (uint64_t)lo + (uint64_t)cnt * step;
-        const uint32_t new_hi = cap < hi ? (uint32_t)cap : hi;
-        if (cnt == nt && new_lo < hi) {
-            // every probe matched: widen the stride so that the next step spans the rest
-            lo = new_lo;
-            const uint32_t span = hi - lo;
-            step = (span + nt - 1) / nt;
-        } else {
-            lo = new_lo;
-            hi = new_hi;
-            const uint32_t span = hi > lo ? hi - lo : 0;
-            step = span ? (span + nt - 1) / nt : 1;
-        }
-    }
-    return FORWARD ? at + lo : at + 1 - lo;
-}
-
-// A workgroup of the carry fix-up is kFixThreads threads laid out as columns x
-// lanes over one slab of the row: 64 column vectors x 4 partial-sum lanes for the
-// usual run of a few chunks, 16 x 16 for a run of more than kFixLongRun chunks (a
-// frequent token: four times the slabs, so four times the workgroups, and a
-// quarter of the partial rows per lane -- all rows one token, 16384 x 384 fp32:
-// backward 53 -> 25 us).
-constexpr int kFixThreads = 256;
-constexpr int kFixCols = 64;        // column vectors per slab ...
-constexpr int kFixLanes = 4;        // ... and partial-sum lanes per column
-constexpr int kFixColsLong = 16;    // the same for a long run
-constexpr int kFixLanesLong = 16;
-constexpr uint32_t kFixLongRun = 64;
-constexpr int kFixBatch = 8;        // partial rows a lane keeps in flight
-static_assert(kFixCols * kFixLanes == kFixThreads && kFixColsLong * kFixLanesLong == kFixThreads, "carry fix layout");
-
-template <typename TO, int VEC>
-__global__ void __launch_bounds__(kFixThreads)
-emb_carry_fix_kernel(const uint32_t* __restrict__ tok_s, TO* dW, const float* __restrict__ carry_head,
-                     const float* __restrict__ carry_tail, uint32_t N, uint32_t C, uint32_t CV,
-                     uint32_t V, uint32_t L, int accumulate) {
-    __shared__ float part[kFixThreads * VEC];
-    const uint32_t chunk = blockIdx.x;
-    const ChunkEdges e = chunk_edges(tok_s, chunk, L, N);
-    const bool origin = e.open_right && !(e.single && e.open_left);
-    const bool middle = e.single && e.open_left && e.open_right;
-    if (!origin && !middle) return;
-    const uint32_t tok = tok_s[e.end - 1];
-    if (tok >= V) return;
-    // Equal tokens are contiguous, but the order of distinct tokens is the
-    // sorter's business (the grouping sort orders by hash group first), so the
-    // searches test "equals tok".  The whole workgroup searches: one probe per
-    // thread and a barrier count per step, so a run of any length is bracketed in
-    // two or three memory round trips (a hot token's run spans thousands of
-    // positions; bisecting it with dependent loads took longer than the sums).
-    if (middle) {
-        // only the first `slabs` middle chunks of a run help (slabs of the long-run
-        // layout at most); one probe tells the rest
-        const uint64_t far = (uint64_t)((CV + kFixColsLong - 1) / kFixColsLong + 1) * L;
-        if (e.start >= far && tok_s[e.start - far] == tok) return;
-    }
-    const uint32_t run_end = run_edge<true>(tok_s, tok, e.end, N);        // first position after the run
-    const uint32_t c1 = (run_end - 1) / L;       // chunk holding the run's last position
-    uint32_t c0 = chunk;                         // chunk holding its first
-    if (middle) c0 = run_edge<false>(tok_s, tok, e.start, N) / L;
-    const uint32_t count = c1 - c0;              // head partials live in chunks c0+1 .. c1
-    const float* tail = carry_tail + (uint64_t)c0 * C;
-    const float* heads = carry_head + (uint64_t)(c0 + 1) * C;
-
-    if (count <= (uint32_t)kFixLanes) {
-        if (!origin) return;
-        for (uint32_t cv = threadIdx.x; cv < CV; cv += blockDim.x) {
-            const uint32_t col = cv * VEC;
-            float sum[VEC], v[kFixLanes][VEC];
-            load_carry<VEC>(tail + col, sum);
-#pragma unroll
-            for (int q = 0; q < kFixLanes; ++q)
-                if ((uint32_t)q < count) {
-                    load_carry<VEC>(heads + (uint64_t)q * C + col, v[q]);
-                }
-#pragma unroll
-            for (int q = 0; q < kFixLanes; ++q)
-                if ((uint32_t)q < count) {
-#pragma unroll
-                    for (int k = 0; k < VEC; ++k) sum[k] = sum[k] + v[q][k];
-                }
-            store_grad_row<TO, VEC>(dW, (uint64_t)tok * C + col, sum, accumulate != 0);
-        }
-        return;
-    }
-
-    const bool long_run = count > kFixLongRun;
-    const uint32_t cols = long_run ? kFixColsLong : kFixCols;
-    const uint32_t lanes = long_run ? kFixLanesLong : kFixLanes;
-    const uint32_t slabs = (CV + cols - 1) / cols;
-    const uint32_t helpers = count - 1 < slabs ? count - 1 : slabs;   // middle chunks that take a slab
-    uint32_t slab_begin, slab_end;
-    if (origin) {
-        slab_begin = helpers; slab_end = slabs;
-    } else {
-        slab_begin = chunk - c0 - 1; slab_end = slab_begin + 1;
-        if (slab_begin >= helpers) return;
-    }
-    const uint32_t colv = threadIdx.x % cols;
-    const uint32_t lane = threadIdx.x / cols;
-    for (uint32_t slab = slab_begin; slab < slab_end; ++slab) {
-        const uint32_t cv = slab * cols + colv;
-        const bool live = cv < CV;
-        const uint32_t col = cv * VEC;
+__device__ __forceinline__ void
+emb_long_run_slab(float* part, const uint32_t* __restrict__ row_s, const T* __restrict__ dY, TO* dW, uint32_t tok,
+                  uint32_t start, uint32_t R, uint32_t w, uint32_t width, uint32_t C, uint32_t CV, int accumulate) {
+    typedef RawVec<T, VEC> Raw;
+    const uint32_t slab_lo = w * width;
+    const uint32_t slab_hi = slab_lo + width < CV ? slab_lo + width : CV;
+    const uint32_t cols = width < blockDim.x ? width : blockDim.x;
+    const uint32_t lanes = blockDim.x / cols;
+    const uint32_t colv = threadIdx.x % cols, lane = threadIdx.x / cols;
+    for (uint32_t c0 = slab_lo; c0 < slab_hi; c0 += cols) {
+        const uint32_t scv = c0 + colv;
+        const bool on = lane < lanes && scv < slab_hi;
         float acc[VEC];
 #pragma unroll
         for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
-        if (live) {
-            for (uint32_t q0 = lane; q0 < count; q0 += lanes * kFixBatch) {
-                float v[kFixBatch][VEC];
+        if (on) {
+#pragma nounroll
+            for (uint32_t q0 = lane; q0 < R; q0 += lanes * kLongBatch) {
+                uint32_t rr[kLongBatch];
+                typename Raw::type v[kLongBatch];
 #pragma unroll
-                for (int b = 0; b < kFixBatch; ++b) {
-                    const uint32_t q = q0 + (uint32_t)b * lanes;
-                    if (q < count) {
-                        load_carry<VEC>(heads + (uint64_t)q * C + col, v[b]);
-                    }
+                for (int q = 0; q < kLongBatch; ++q) {
+                    const uint32_t at_q = q0 + (uint32_t)q * lanes;
+                    rr[q] = at_q < R ? row_s[start + at_q] : 0u;
                 }
 #pragma unroll
-                for (int b = 0; b < kFixBatch; ++b) {
-                    const uint32_t q = q0 + (uint32_t)b * lanes;
-                    if (q < count) {
+                for (int q = 0; q < kLongBatch; ++q) {
+                    const uint32_t at_q = q0 + (uint32_t)q * lanes;
+                    v[q] = Raw::zero();
+                    if (at_q < R) v[q] = Raw::load(dY + (uint64_t)rr[q] * C + (uint64_t)scv * VEC);
+                }
 #pragma unroll
-                        for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + v[b][k];
+                for (int q = 0; q < kLongBatch; ++q) {
+                    const uint32_t at_q = q0 + (uint32_t)q * lanes;
+                    if (at_q < R) {
+                        float x[VEC];
+                        Raw::unpack(v[q], x);
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + x[k];
                     }
                 }
             }
         }
+        __syncthreads();            // the previous pass's readers are done with `part`
+        if (lane < lanes) {
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) part[(lane * cols + colv) * VEC + k] = acc[k];
-        __syncthreads();
-        if (lane == 0 && live) {
-            float sum[VEC];
-            load_carry<VEC>(tail + col, sum);
-            for (uint32_t q = 0; q < lanes; ++q)
-#pragma unroll
-                for (int k = 0; k < VEC; ++k) sum[k] = sum[k] + part[(q * cols + colv) * VEC + k];
-            store_grad_row<TO, VEC>(dW, (uint64_t)tok * C + col, sum, accumulate != 0);
+            for (int k = 0; k < VEC; ++k) part[(lane * cols + colv) * VEC + k] = acc[k];
         }
         __syncthreads();
+        if (lane == 0 && scv < slab_hi) {
+            float sum[VEC];
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) sum[k] = part[colv * VEC + k];
+            for (uint32_t q = 1; q < lanes && q < R; ++q)
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) sum[k] = sum[k] + part[(q * cols + colv) * VEC + k];
+            store_grad_row<TO, VEC>(dW, (uint64_t)tok * C + (uint64_t)scv * VEC, sum, accumulate != 0);
+        }
     }
+}
+
+template <typename T, typename TO, int VEC, bool POS>
+__global__ void __launch_bounds__(kRowSumMaxBlock)
+emb_row_sum_kernel(const RunInfo* __restrict__ info, const uint32_t* __restrict__ row_s, const T* __restrict__ dY,
+                   TO* dW, TO* dwpe, uint32_t N, uint32_t C, uint32_t CV, uint32_t V, uint32_t T_len, uint32_t B,
+                   int accumulate, int accumulate_pos, uint32_t min_slab) {
+    __shared__ float part[kRowSumMaxBlock * VEC];
+    typedef RawVec<T, VEC> Raw;
+    const uint32_t first = POS ? blockIdx.x : blockIdx.x * kRowBatch;
+    const uint32_t row_step = POS ? T_len : 1u;
+    const uint32_t n_rows = POS ? B : (N - first < (uint32_t)kRowBatch ? N - first : (uint32_t)kRowBatch);
+
+    for (uint32_t cv0 = 0; cv0 < CV; cv0 += blockDim.x) {       // one pass unless a row is wider than the workgroup
+        const uint32_t cv = cv0 + threadIdx.x;
+        const bool live = cv < CV;
+        const uint32_t col = cv * VEC;
+        float pos_acc[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) pos_acc[k] = 0.0f;
+
+        for (uint32_t b0 = 0; b0 < n_rows; b0 += kRowBatch) {
+            // what each row of the batch is (the same in every thread: scalar loads)
+            RunInfo inf[kRowBatch];
+            bool solo[kRowBatch];
+#pragma unroll
+            for (int i = 0; i < kRowBatch; ++i) {
+                inf[i] = RunInfo{V, 0u, 1u, 1u};
+                if (b0 + i < n_rows) inf[i] = info[first + (b0 + i) * row_step];
+                solo[i] = inf[i].tok < V && inf[i].j == 0 && inf[i].R <= kSoloRun;
+            }
+            // the vectors that are certainly wanted: a run's first row (and, for the position
+            // table, every row), and the second row of a run of two
+            typename Raw::type own[kRowBatch], two[kRowBatch];
+#pragma unroll
+            for (int i = 0; i < kRowBatch; ++i) {
+                own[i] = Raw::zero();
+                const bool want = (POS && b0 + i < n_rows) || solo[i];
+                if (want && live) own[i] = Raw::load(dY + (uint64_t)(first + (b0 + i) * row_step) * C + col);
+            }
+#pragma unroll
+            for (int i = 0; i < kRowBatch; ++i) {
+                two[i] = Raw::zero();
+                if (solo[i] && inf[i].R >= 2) {
+                    const uint32_t r = row_s[inf[i].start + 1];
+                    if (live) two[i] = Raw::load(dY + (uint64_t)r * C + col);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < kRowBatch; ++i) {
+                float acc[VEC];
+                Raw::unpack(own[i], acc);
+                if constexpr (POS) {
+                    if (b0 + i < n_rows) {
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) pos_acc[k] = b0 + i == 0 ? acc[k] : pos_acc[k] + acc[k];
+                    }
+                }
+                if (solo[i]) {
+                    if (inf[i].R >= 2) {
+                        float x[VEC];
+                        Raw::unpack(two[i], x);
+#pragma unroll
+                        for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + x[k];
+                    }
+#pragma nounroll
+                    for (uint32_t r0 = 2; r0 < inf[i].R; r0 += kRowBatch) {       // rows 3 .. kSoloRun of the run
+                        typename Raw::type v[kRowBatch];
+#pragma unroll
+                        for (int q = 0; q < kRowBatch; ++q) {
+                            v[q] = Raw::zero();
+                            if (r0 + q < inf[i].R) {
+                                const uint32_t r = row_s[inf[i].start + r0 + q];
+                                if (live) v[q] = Raw::load(dY + (uint64_t)r * C + col);
+                            }
+                        }
+#pragma unroll
+                        for (int q = 0; q < kRowBatch; ++q) {
+                            if (r0 + q < inf[i].R) {
+                                float x[VEC];
+                                Raw::unpack(v[q], x);
+#pragma unroll
+                                for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + x[k];
+                            }
+                        }
+                    }
+                    if (live) store_grad_row<TO, VEC>(dW, (uint64_t)inf[i].tok * C + col, acc, accumulate != 0);
+                }
+            }
+            // longer runs: is one of these rows a worker of its run?  (first column pass only:
+            // a slab covers its columns whatever the workgroup's width)
+            if (cv0 == 0) {
+#pragma unroll
+                for (int i = 0; i < kRowBatch; ++i) {
+                    if (inf[i].tok < V && inf[i].R > kSoloRun) {
+                        const uint32_t R = inf[i].R;
+                        const uint32_t width = slab_width(R, CV, blockDim.x, min_slab);
+                        const uint32_t slabs = (CV + width - 1) / width;        // at most kMaxSlabs, at most R
+                        const uint32_t stride = R / slabs;
+                        const uint32_t w = inf[i].j / stride;
+                        if (w * stride == inf[i].j && w < slabs)
+                            emb_long_run_slab<T, TO, VEC>(part, row_s, dY, dW, inf[i].tok, inf[i].start, R, w, width, C, CV, accumulate);
+                    }
+                }
+            }
+        }
+        if constexpr (POS) {
+            if (live) store_grad_row<TO, VEC>(dwpe, (uint64_t)blockIdx.x * C + col, pos_acc, accumulate_pos != 0);
+        }
+    }
+}
+
+// The radix path's ordering is by token throughout: the run of position p is found by
+// two bisections of the sorted tokens.
+__global__ void __launch_bounds__(256)
+emb_run_info_kernel(const uint32_t* __restrict__ tok_s, const uint32_t* __restrict__ row_s, RunInfo* __restrict__ info,
+                    uint32_t N) {
+    const uint32_t p = blockIdx.x * 256 + threadIdx.x;
+    if (p >= N) return;
+    const uint32_t tok = tok_s[p];
+    uint32_t lo = 0, hi = p;                    // first position holding tok
+    while (lo < hi) { const uint32_t mid = (lo + hi) >> 1; if (tok_s[mid] < tok) lo = mid + 1; else hi = mid; }
+    const uint32_t start = lo;
+    lo = p + 1; hi = N;                         // first position after the run
+    while (lo < hi) { const uint32_t mid = (lo + hi) >> 1; if (tok_s[mid] <= tok) lo = mid + 1; else hi = mid; }
+    info[row_s[p]] = RunInfo{tok, start, p - start, lo - start};
 }
 
 // dwpe[t, c] (+)= sum_b dY[b, t, c], b ascending
@@ -905,7 +845,7 @@ bool group_sort_enabled() {
 // Scratch of the ordering step: input key / value arrays of the radix path (the
 // grouping sort uses the same bytes as N 64-bit spill slots) and rocPRIM's temp.
 struct SortPlan {
-    uint64_t off_keys_in, off_vals_in, off_temp, temp_bytes, total;
+    uint64_t off_keys_in, off_vals_in, off_keys_out, off_temp, temp_bytes, total;
 };
 
 int plan_sort(uint64_t N, uint32_t V, SortPlan* p) {
@@ -920,64 +860,45 @@ int plan_sort(uint64_t N, uint32_t V, SortPlan* p) {
     // keys_in and vals_in are adjacent: the grouping sort uses the pair as N 64-bit spill slots
     p->off_keys_in = o;  o += align256(N * 4);
     p->off_vals_in = o;  o += align256(N * 4);
+    p->off_keys_out = o; o += align256(N * 4);     // the sorted tokens (radix path)
     p->off_temp = o;     o += align256(temp);
     p->temp_bytes = temp;
     p->total = o;
     return AGRAD_OK;
 }
 
-// Scratch of the summing step: one head and one tail carry row per chunk.
-struct SumPlan {
-    uint32_t L, chunks;
-    uint64_t off_head, off_tail, total;
-};
+// The order: row_s[N] (rows, each token's run adjacent and ascending), then, from the
+// next multiple of four words on, one RunInfo per row.
+inline uint64_t order_info_word(uint64_t N) { return (N + 3) & ~3ull; }
+inline uint64_t order_bytes(uint64_t N) { return align256((order_info_word(N) + 4 * N) * 4); }
 
-void plan_sum(uint64_t N, uint32_t C, SumPlan* p) {
-    const uint64_t max_chunks = N >= kLargeRows ? kMaxChunksLarge : kMaxChunks;
-    uint32_t per = (uint32_t)((N + (uint64_t)kBatch * max_chunks - 1) / ((uint64_t)kBatch * max_chunks));
-    if (per == 0) per = 1;
-    p->L = kBatch * per;
-    p->chunks = (uint32_t)((N + p->L - 1) / p->L);
-    uint64_t o = 0;
-    p->off_head = o;     o += align256((uint64_t)p->chunks * C * 4);
-    p->off_tail = o;     o += align256((uint64_t)p->chunks * C * 4);
-    p->total = o;
-}
-
-inline uint64_t order_bytes(uint64_t N) { return align256(N * 8); }   // tok_s[N] then row_s[N]
+// A long run's column slabs are at least this many 16-byte vectors wide (two cache
+// lines per access) unless the run is long enough to want more workgroups.
+constexpr uint32_t kMinSlabVectors = 8;
 
 template <typename T, typename TO = T>
-int embedding_sum_typed(hipStream_t s, const SumPlan& p, const uint32_t* tok_s, const uint32_t* row_s, const T* dY,
-                        TO* dW, uint8_t* ws, uint32_t N, uint32_t C, uint32_t V, uint32_t flags, TO* dwpe,
-                        uint32_t B, uint32_t T_len) {
-    float* head = (float*)(ws + p.off_head);
-    float* tail = (float*)(ws + p.off_tail);
+int embedding_sum_typed(hipStream_t s, const uint32_t* order, const T* dY, TO* dW, uint32_t N, uint32_t C, uint32_t V,
+                        uint32_t flags, TO* dwpe, uint32_t B, uint32_t T_len) {
+    const uint32_t* row_s = order;
+    const RunInfo* info = reinterpret_cast<const RunInfo*>(order + order_info_word(N));
     const int acc = (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0;
     const int acc_pos = (flags & AGRAD_ACC_PARAM_GRAD2) ? 1 : 0;
     constexpr int WIDE = WideVec<T>::value;
     // (a bf16 row under an fp32 upstream moves 8 bytes per vector: 8-byte alignment is implied by 16)
     const bool wide = C % WIDE == 0 && aligned16(dY) && aligned16(dW) && (!dwpe || aligned16(dwpe));
-    const uint64_t TC = dwpe ? (uint64_t)T_len * C : 0;
+    const uint32_t CV = wide ? C / WIDE : C;
+    uint32_t block = ((CV + 63) / 64) * 64;
+    if (block > (uint32_t)kRowSumMaxBlock) block = kRowSumMaxBlock;
+    const uint32_t grid = dwpe ? T_len : (N + kRowBatch - 1) / kRowBatch;
+#define AGRAD_ROW_SUM(VEC, POS) \
+    hipLaunchKernelGGL((emb_row_sum_kernel<T, TO, VEC, POS>), dim3(grid), dim3(block), 0, s, info, row_s, dY, dW, \
+                       dwpe, N, C, CV, V, T_len, B, acc, acc_pos, kMinSlabVectors)
     if (wide) {
-        const uint32_t CV = C / WIDE;
-        uint32_t block = ((CV + 63) / 64) * 64;
-        if (block > 512) block = 512;
-        const uint64_t extra = (TC / WIDE + block - 1) / block;
-        if (p.chunks + extra > 0x7fffffffull) return set_error(AGRAD_EINVAL, "embedding backward: position table too large");
-        hipLaunchKernelGGL((emb_segment_sum_kernel<T, TO, WIDE>), dim3(p.chunks + (uint32_t)extra), dim3(block), 0, s, tok_s,
-                           row_s, dY, dW, head, tail, N, C, CV, V, p.L, acc, p.chunks, dwpe, B, T_len, acc_pos);
-        hipLaunchKernelGGL((emb_carry_fix_kernel<TO, WIDE>), dim3(p.chunks), dim3(kFixThreads), 0, s,
-                           tok_s, dW, head, tail, N, C, CV, V, p.L, acc);
+        if (dwpe) AGRAD_ROW_SUM(WIDE, true); else AGRAD_ROW_SUM(WIDE, false);
     } else {
-        uint32_t block = ((C + 63) / 64) * 64;
-        if (block > 512) block = 512;
-        const uint64_t extra = (TC + block - 1) / block;
-        if (p.chunks + extra > 0x7fffffffull) return set_error(AGRAD_EINVAL, "embedding backward: position table too large");
-        hipLaunchKernelGGL((emb_segment_sum_kernel<T, TO, 1>), dim3(p.chunks + (uint32_t)extra), dim3(block), 0, s, tok_s,
-                           row_s, dY, dW, head, tail, N, C, C, V, p.L, acc, p.chunks, dwpe, B, T_len, acc_pos);
-        hipLaunchKernelGGL((emb_carry_fix_kernel<TO, 1>), dim3(p.chunks), dim3(kFixThreads), 0, s,
-                           tok_s, dW, head, tail, N, C, C, V, p.L, acc);
+        if (dwpe) AGRAD_ROW_SUM(1, true); else AGRAD_ROW_SUM(1, false);
     }
+#undef AGRAD_ROW_SUM
     return check_hip(hipGetLastError(), "embedding backward launch");
 }
 
@@ -998,7 +919,9 @@ uint64_t embedding_sort_workspace_bytes(uint64_t N, uint32_t V) {
     return p.total;
 }
 
-// order[0 .. N) = tokens, order[N .. 2N) = rows: each token's rows adjacent, ascending
+// order[0 .. N) = rows, each token's rows adjacent and ascending; then (from the next
+// multiple of four words) four words per row: its token, where its token's run starts,
+// its index in the run and the run's length
 int launch_embedding_sort(hipStream_t s, const int32_t* ids, uint32_t* order, void* workspace,
                           uint64_t workspace_bytes, uint64_t N, uint32_t V, int* err_flag) {
     if (N == 0) return AGRAD_OK;
@@ -1011,15 +934,17 @@ int launch_embedding_sort(hipStream_t s, const int32_t* ids, uint32_t* order, vo
                          (unsigned long long)workspace_bytes, (unsigned long long)p.total);
     if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
         return set_error(AGRAD_EINVAL, "embedding sort: workspace must be 256-byte aligned");
+    if ((reinterpret_cast<uintptr_t>(order) & 15u) != 0)
+        return set_error(AGRAD_EINVAL, "embedding sort: the order buffer must be 16-byte aligned");
     uint8_t* ws = (uint8_t*)workspace;
-    uint32_t* tok_s = order;
-    uint32_t* row_s = order + N;
+    uint32_t* row_s = order;
+    RunInfo* info = reinterpret_cast<RunInfo*>(order + order_info_word(N));
     const uint32_t n = (uint32_t)N;
     if (n <= kGroupSortMaxN && group_sort_enabled()) {
         static_assert(sizeof(unsigned long long) == 2 * sizeof(uint32_t), "spill layout");
         unsigned long long* spill = reinterpret_cast<unsigned long long*>(ws + p.off_keys_in);
         const uint32_t log2G = group_sort_log2g(n);
-        hipLaunchKernelGGL(emb_group_sort_kernel, dim3(1u << log2G), dim3(kSortBlock), 0, s, ids, tok_s, row_s,
+        hipLaunchKernelGGL(emb_group_sort_kernel, dim3(1u << log2G), dim3(kSortBlock), 0, s, ids, row_s, info,
                            spill, n, V, log2G, err_flag);
         return check_hip(hipGetLastError(), "embedding sort launch");
     }
@@ -1032,9 +957,12 @@ int launch_embedding_sort(hipStream_t s, const int32_t* ids, uint32_t* order, vo
     int bits = 1;
     while ((1ull << bits) <= V) ++bits;
     size_t temp = p.temp_bytes;
+    uint32_t* tok_s = (uint32_t*)(ws + p.off_keys_out);
     hipError_t err = rocprim::radix_sort_pairs(ws + p.off_temp, temp, keys_in, tok_s, vals_in, row_s,
                                                (size_t)N, 0u, (unsigned)bits, s, false);
-    return check_hip(err, "radix sort");
+    if (int rc = check_hip(err, "radix sort")) return rc;
+    hipLaunchKernelGGL(emb_run_info_kernel, dim3((n + 255) / 256), dim3(256), 0, s, tok_s, row_s, info, n);
+    return check_hip(hipGetLastError(), "embedding order launch");
 }
 
 // out = W[ids] (+ wpe) and order = the ids' ordering for the later gradient
@@ -1068,57 +996,50 @@ int launch_gather_fwd_sorted(hipStream_t s, int dtype, const int32_t* ids, const
     const uint32_t n = (uint32_t)N, CV = C / per16, total = (uint32_t)total_vec;
     const uint32_t log2G = group_sort_log2g(n);
     const uint32_t grid = (1u << log2G) + (total + kSortBlock - 1) / kSortBlock;
-    uint32_t* tok_s = order;
-    uint32_t* row_s = order + N;
+    if ((reinterpret_cast<uintptr_t>(order) & 15u) != 0)
+        return set_error(AGRAD_EINVAL, "gather: the order buffer must be 16-byte aligned");
+    uint32_t* row_s = order;
+    RunInfo* info = reinterpret_cast<RunInfo*>(order + order_info_word(N));
     if (wpe == nullptr) {
         hipLaunchKernelGGL((gather_sort_kernel<float, 4, true>), dim3(grid), dim3(kSortBlock), 0, s, ids, (const float*)W,
-                           (const float*)nullptr, (float*)out, total, CV, C, T ? T : 1u, V, tok_s, row_s, spill, n, log2G, err_flag);
+                           (const float*)nullptr, (float*)out, total, CV, C, T ? T : 1u, V, row_s, info, spill, n, log2G, err_flag);
     } else if (dtype == AGRAD_F32) {
         hipLaunchKernelGGL((gather_sort_kernel<float, 4, false>), dim3(grid), dim3(kSortBlock), 0, s, ids, (const float*)W,
-                           (const float*)wpe, (float*)out, total, CV, C, T, V, tok_s, row_s, spill, n, log2G, err_flag);
+                           (const float*)wpe, (float*)out, total, CV, C, T, V, row_s, info, spill, n, log2G, err_flag);
     } else {
         hipLaunchKernelGGL((gather_sort_kernel<bf16_t, 8, false>), dim3(grid), dim3(kSortBlock), 0, s, ids, (const bf16_t*)W,
-                           (const bf16_t*)wpe, (bf16_t*)out, total, CV, C, T, V, tok_s, row_s, spill, n, log2G, err_flag);
+                           (const bf16_t*)wpe, (bf16_t*)out, total, CV, C, T, V, row_s, info, spill, n, log2G, err_flag);
     }
     return check_hip(hipGetLastError(), "gather launch");
 }
 
 uint64_t embedding_bwd_sorted_workspace_bytes(uint64_t N, uint32_t C) {
-    if (N == 0 || C == 0) return 0;
-    SumPlan p;
-    plan_sum(N, C, &p);
-    return p.total;
+    (void)N; (void)C;
+    return 0;       // every table row is summed and stored by one workgroup: nothing is staged
 }
 
 int launch_embedding_bwd_sorted(hipStream_t s, int dtype, const uint32_t* order, const void* dY, void* dW,
                                 void* dwpe, void* workspace, uint64_t workspace_bytes, uint64_t N, uint32_t T,
                                 uint32_t C, uint32_t V, uint32_t flags) {
+    (void)workspace; (void)workspace_bytes;
     if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "embedding backward: unknown dtype %d", dtype);
     if (N == 0 || C == 0) return AGRAD_OK;
     if (int rc = check_embedding_sizes("embedding backward", N, V)) return rc;
     if (order == nullptr || dY == nullptr || dW == nullptr) return set_error(AGRAD_EINVAL, "embedding backward: null operand");
+    if ((reinterpret_cast<uintptr_t>(order) & 15u) != 0)
+        return set_error(AGRAD_EINVAL, "embedding backward: the order buffer must be 16-byte aligned");
     uint32_t B = 0;
     if (dwpe != nullptr) {
         if (T == 0 || N % T != 0) return set_error(AGRAD_EINVAL, "embedding backward: %llu rows are not a whole number of sequences of %u", (unsigned long long)N, T);
         B = (uint32_t)(N / T);
     }
-    SumPlan p;
-    plan_sum(N, C, &p);
-    if (workspace == nullptr || workspace_bytes < p.total)
-        return set_error(AGRAD_EWORKSPACE, "embedding backward: workspace %llu < %llu bytes",
-                         (unsigned long long)workspace_bytes, (unsigned long long)p.total);
-    if ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0)
-        return set_error(AGRAD_EINVAL, "embedding backward: workspace must be 256-byte aligned");
     if (flags & AGRAD_PARAM_GRAD_BF16) {
         if (dtype != AGRAD_F32) return set_error(AGRAD_EINVAL, "embedding backward: AGRAD_PARAM_GRAD_BF16 goes with an fp32 upstream gradient");
-        return embedding_sum_typed<float, bf16_t>(s, p, order, order + N, (const float*)dY, (bf16_t*)dW, (uint8_t*)workspace,
-                                                  (uint32_t)N, C, V, flags, (bf16_t*)dwpe, B, T);
+        return embedding_sum_typed<float, bf16_t>(s, order, (const float*)dY, (bf16_t*)dW, (uint32_t)N, C, V, flags, (bf16_t*)dwpe, B, T);
     }
     if (dtype == AGRAD_F32)
-        return embedding_sum_typed<float>(s, p, order, order + N, (const float*)dY, (float*)dW, (uint8_t*)workspace,
-                                          (uint32_t)N, C, V, flags, (float*)dwpe, B, T);
-    return embedding_sum_typed<bf16_t>(s, p, order, order + N, (const bf16_t*)dY, (bf16_t*)dW, (uint8_t*)workspace,
-                                       (uint32_t)N, C, V, flags, (bf16_t*)dwpe, B, T);
+        return embedding_sum_typed<float>(s, order, (const float*)dY, (float*)dW, (uint32_t)N, C, V, flags, (float*)dwpe, B, T);
+    return embedding_sum_typed<bf16_t>(s, order, (const bf16_t*)dY, (bf16_t*)dW, (uint32_t)N, C, V, flags, (bf16_t*)dwpe, B, T);
 }
 
 int launch_gather_fwd(hipStream_t s, int dtype, const int32_t* ids, const void* W, const void* wpe,
@@ -1165,7 +1086,7 @@ int launch_gather_fwd(hipStream_t s, int dtype, const int32_t* ids, const void* 
 uint64_t embedding_bwd_workspace_bytes(uint64_t N, uint32_t C, uint32_t V, int dtype) {
     (void)dtype;
     if (N == 0 || C == 0) return 0;
-    return order_bytes(N) + embedding_sort_workspace_bytes(N, V) + embedding_bwd_sorted_workspace_bytes(N, C);
+    return order_bytes(N) + embedding_sort_workspace_bytes(N, V);
 }
 
 int launch_embedding_bwd(hipStream_t s, int dtype, const int32_t* ids, const void* dY, void* dW,
@@ -1176,8 +1097,7 @@ int launch_embedding_bwd(hipStream_t s, int dtype, const int32_t* ids, const voi
     if (ids == nullptr || dY == nullptr || dW == nullptr) return set_error(AGRAD_EINVAL, "embedding backward: null operand");
     if (int rc = check_embedding_sizes("embedding backward", N, V)) return rc;
     const uint64_t sort_bytes = embedding_sort_workspace_bytes(N, V);
-    const uint64_t sum_bytes = embedding_bwd_sorted_workspace_bytes(N, C);
-    const uint64_t need = order_bytes(N) + sort_bytes + sum_bytes;
+    const uint64_t need = order_bytes(N) + sort_bytes;
     if (workspace == nullptr || workspace_bytes < need)
         return set_error(AGRAD_EWORKSPACE, "embedding backward: workspace %llu < %llu bytes",
                          (unsigned long long)workspace_bytes, (unsigned long long)need);
@@ -1186,7 +1106,7 @@ int launch_embedding_bwd(hipStream_t s, int dtype, const int32_t* ids, const voi
     uint8_t* ws = (uint8_t*)workspace;
     uint32_t* order = (uint32_t*)ws;
     if (int rc = launch_embedding_sort(s, ids, order, ws + order_bytes(N), sort_bytes, N, V, err_flag)) return rc;
-    return launch_embedding_bwd_sorted(s, dtype, order, dY, dW, nullptr, ws + order_bytes(N) + sort_bytes, sum_bytes, N, 0, C, V, flags);
+    return launch_embedding_bwd_sorted(s, dtype, order, dY, dW, nullptr, nullptr, 0, N, 0, C, V, flags);
 }
 
 int launch_pos_embedding_bwd(hipStream_t s, int dtype, const void* dY, void* dwpe, uint32_t B,

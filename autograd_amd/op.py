@@ -288,7 +288,8 @@ class ContiguousOp(Op):
 
 def _order_output(indices, table):
     """When the table needs a gradient, the embedding ops carry a second,
-    gradient-free output: the (token, row) order of the indices, 2N uint32.  A
+    gradient-free output of 5N + 4 uint32: the rows ordered so that each token's rows are
+    adjacent and ascending, and what every row is told about its token's run.  A
     device may fill it in its forward kernel (where ordering the ids is free) and
     start its backward kernel from it; a device that has no use for it leaves it
     alone.  `__call__` still returns the embedding only."""
@@ -297,7 +298,7 @@ def _order_output(indices, table):
     n = 1
     for d in indices.shape:
         n *= d
-    return (Tensor(shape=(2 * n,), dtype=np.uint32, requires_grad=False, device=table.device),)
+    return (Tensor(shape=(5 * n + 4,), dtype=np.uint32, requires_grad=False, device=table.device),)
 
 
 class GatherOp(Op):

@@ -305,12 +305,18 @@ int agrad_gather_forward(agrad_ctx* ctx, int dtype, const int32_t* ids,
                          const void* W, const void* wpe, void* out,
                          uint64_t N, uint32_t T, uint32_t C, uint32_t V);
 
-/* Embedding gradient dW[ids[n],:] += dY[n,:], deterministic: rows are sorted by
- * token id (stable), then each token's run is summed in ascending row order
- * (cpu_gather_backward = np.add.at, backend.py:531-538; replaces the float-atomic
- * gather_backward_kernel, metal_ops.metal:406-427).
+/* Embedding gradient dW[ids[n],:] += dY[n,:], deterministic: the (token, row) pairs
+ * are ordered so that each token's rows are adjacent and ascending, and the first
+ * row of every token adds that token's rows in ascending row order -- the sequence
+ * of fp32 adds np.add.at makes (cpu_gather_backward, backend.py:531-538; replaces
+ * the float-atomic gather_backward_kernel, metal_ops.metal:406-427).  A token with
+ * more than 16 rows is summed by several workgroups, a column band each, with a
+ * fixed association of its rows.  Every table row is written once, by one workgroup:
+ * same bits on every run.
  * Without AGRAD_ACC_PARAM_GRAD the touched rows of dW are overwritten (correct on
- * a table that was just zero-filled); untouched rows are never written. */
+ * a table that was just zero-filled); untouched rows are never written.
+ * workspace: agrad_embedding_backward_workspace_bytes(N, C, V, dtype) bytes, 256-byte
+ * aligned (the order of the ids and the sort's scratch). */
 uint64_t agrad_embedding_backward_workspace_bytes(uint64_t N, uint32_t C, uint32_t V, int dtype);
 int agrad_embedding_backward(agrad_ctx* ctx, int dtype, const int32_t* ids, const void* dY, void* dW,
                              void* workspace, uint64_t workspace_bytes,
@@ -318,11 +324,15 @@ int agrad_embedding_backward(agrad_ctx* ctx, int dtype, const int32_t* ids, cons
 /* The same pair with the ordering of the ids done in the forward call, where it
  * is free: up to 65536 rows the gather and the ordering are ONE launch (the
  * ordering workgroups run beside the bandwidth-bound gather), and the backward
- * call starts at the segmented sum.  The forward call also writes order[0..N) =
- * tokens and order[N..2N) = rows (each token's rows adjacent, ascending; 2N
- * uint32).  sort_workspace (256-byte aligned, agrad_embedding_sort_workspace_bytes(N, V)
- * bytes) is free again when the call's work has run; the backward call's
- * workspace holds agrad_embedding_backward_sorted_workspace_bytes(N, C) bytes.
+ * call is one launch that reads dY front to back.  The forward call also writes
+ * `order`, 5N + 4 uint32, 16-byte aligned: order[0..N) = the rows, each token's
+ * rows adjacent and ascending; then, from the next multiple of four words on, four
+ * words for row n = 0..N-1: its token (V for an id outside the table), the place
+ * in order[] where its token's run starts, its index in the run and the run's
+ * length.  sort_workspace (256-byte aligned, agrad_embedding_sort_workspace_bytes(N, V)
+ * bytes) is free again when the call's work has run; the backward call stages
+ * nothing (agrad_embedding_backward_sorted_workspace_bytes is 0 and workspace may
+ * be NULL; both stay in the signature for callers written against it).
  * Same results, bit for bit, as agrad_gather_forward + agrad_embedding_backward.
  * (The reference orders nothing: np.add.at, backend.py:531-538, and float
  * atomics, metal_ops.metal:406-427.) */
@@ -332,8 +342,9 @@ int agrad_gather_forward_sorted(agrad_ctx* ctx, int dtype, const int32_t* ids, c
                                 uint32_t* order, void* sort_workspace, uint64_t sort_workspace_bytes);
 uint64_t agrad_embedding_backward_sorted_workspace_bytes(uint64_t N, uint32_t C);
 /* dwpe may be NULL; otherwise it is the [T, C] position table's gradient
- * dwpe[t,:] (+)= sum_b dY[b,t,:] (N = B*T rows), computed by extra workgroups of
- * the same launch; AGRAD_ACC_PARAM_GRAD2 accumulates into it. */
+ * dwpe[t,:] (+)= sum_b dY[b,t,:] (N = B*T rows, b ascending), added up from the
+ * same loads of dY that feed the table rows; AGRAD_ACC_PARAM_GRAD2 accumulates
+ * into it. */
 int agrad_embedding_backward_sorted(agrad_ctx* ctx, int dtype, const uint32_t* order, const void* dY, void* dW,
                                     void* dwpe, void* workspace, uint64_t workspace_bytes,
                                     uint64_t N, uint32_t T, uint32_t C, uint32_t V, uint32_t flags);
