@@ -395,7 +395,7 @@ int h_gather_fwd_sorted(const Call& c) {
     const uint32_t T = c.a[2], C = c.a[3], V = c.a[4], mask = c.a[7];
     RESOLVE(0, N * 4, ids) RESOLVE(1, (uint64_t)V * C * es, W)
     RESOLVE_IF(mask & 4u, 2, (uint64_t)T * C * es, wpe)
-    RESOLVE(3, N * C * es, out) RESOLVE(4, (N * 5 + 4) * 4, order) RESOLVE(5, wsb, ws)
+    RESOLVE(3, N * C * es, out) RESOLVE(4, (N * 6 + 128) * 4, order) RESOLVE(5, wsb, ws)
     return launch_gather_fwd_sorted(c.ctx->stream, (int)c.a[0], (const int32_t*)ids, W, wpe, out, N, T, C, V,
                                     (uint32_t*)order, ws, wsb, c.ctx->err_flag);
 }
@@ -405,7 +405,7 @@ int h_gather_bwd_sorted(const Call& c) {
     const uint64_t N = c.a[1], es = dtype_size(c.a[0]), wsb = u64(c.a, 5);
     const uint32_t C = c.a[2], V = c.a[3], T = c.a[7], mask = c.a[8];
     const uint64_t gs = (c.a[4] & AGRAD_PARAM_GRAD_BF16) ? 2 : es;      // element size of the table gradients
-    RESOLVE(0, (N * 5 + 4) * 4, order) RESOLVE(1, N * C * es, dY) RESOLVE(2, (uint64_t)V * C * gs, dW) RESOLVE(3, wsb, ws)
+    RESOLVE(0, (N * 6 + 128) * 4, order) RESOLVE(1, N * C * es, dY) RESOLVE(2, (uint64_t)V * C * gs, dW) RESOLVE(3, wsb, ws)
     RESOLVE_IF(mask & 16u, 4, (uint64_t)T * C * gs, dwpe)
     return launch_embedding_bwd_sorted(c.ctx->stream, (int)c.a[0], (const uint32_t*)order, dY, dW, dwpe, ws, wsb, N, T,
                                        C, V, c.a[4]);

@@ -214,9 +214,32 @@ __device__ __forceinline__ void bitonic_sort_u64(unsigned long long* keys, uint3
     }
 }
 
-// What a row is told about its token's run: the token, the position in the order where
-// the run starts, the row's index within the run (rows ascend with it) and the run's length.
-struct __attribute__((aligned(16))) RunInfo { uint32_t tok, start, j, R; };
+// What the ordering step tells row n about its token's run, one 16-byte word per row:
+//   R == 0               nothing to do for this row: a later row of a short run, or an id
+//                        outside the table;
+//   1 <= R <= kSoloRun   row n is the FIRST (lowest) row of a run of R rows, which it adds
+//                        up alone; x = the run's second row, or kNoRow when the ordering
+//                        did not have it at hand (then it is row_s[start + 1]);
+//   R > kSoloRun         row n is row number x of a long run of R rows.
+// `start` is the place in row_s[] where the run begins.
+struct __attribute__((aligned(16))) RunInfo { uint32_t tok, start, R, x; };
+
+constexpr uint32_t kSoloRun = 63;        // longest run its first row adds up alone, in np.add.at's order
+constexpr uint32_t kChunkRows = 32;      // a longer run is cut into chunks of this many rows (the last takes the rest)
+constexpr uint32_t kGroupChunks = 16;    // ... whose partial rows are added in groups of this many (the last takes the rest)
+constexpr uint32_t kTicketFold = 32;     // arrival counters per chunk group: column block kb counts on kb % kTicketFold
+constexpr uint32_t kNoRow = 0xFFFFFFFFu;
+
+// Layout of the order buffer, in 32-bit words: row_s[N] | (pad to 4) RunInfo[N] | group
+// tickets | run tickets.  The tickets are arrival counters of the gradient kernel's long
+// runs; the ordering step zeroes them and the gradient kernel leaves them zero.
+__host__ __device__ inline uint64_t order_info_word(uint64_t N) { return (N + 3) & ~3ull; }
+__host__ __device__ inline uint64_t order_ticket_word(uint64_t N) { return order_info_word(N) + 4 * N; }
+__host__ __device__ inline uint64_t order_group_tickets(uint64_t N) { return (N / (kChunkRows * 2) + 1) * kTicketFold; }
+__host__ __device__ inline uint64_t order_run_tickets(uint64_t N) { return (N / (kChunkRows * kGroupChunks * 2) + 1) * kTicketFold; }
+__host__ __device__ inline uint64_t order_words(uint64_t N) {
+    return order_ticket_word(N) + order_group_tickets(N) + order_run_tickets(N);
+}
 
 // smallest index in sorted keys[0..n) whose key is not below `bound`
 __device__ __forceinline__ uint32_t first_not_below(const unsigned long long* keys, uint32_t n, unsigned long long bound) {
@@ -228,50 +251,74 @@ __device__ __forceinline__ uint32_t first_not_below(const unsigned long long* ke
     return lo;
 }
 
+// The hash group of a token: the bits just below bit 24 of a 24-bit Fibonacci product
+// (a full-rate multiply; tokens that agree in their low 24 bits share a group, which is
+// as good a partition as any).
+__device__ __forceinline__ uint32_t token_group(uint32_t tok, uint32_t log2G) {
+    return (__umul24(tok, 0x9E3779u) >> (24u - log2G)) & ((1u << log2G) - 1u);
+}
+
 // the work of workgroup `g` of the grouping sort (kSortBlock threads)
 __device__ __forceinline__ void
-emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __restrict__ row_s,
-                    RunInfo* __restrict__ info, unsigned long long* __restrict__ spill,
-                    uint32_t N, uint32_t V, uint32_t log2G, int* err_flag) {
+emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __restrict__ order,
+                    unsigned long long* __restrict__ spill, uint32_t N, uint32_t V, uint32_t log2G, int* err_flag) {
     __shared__ unsigned long long keys[kSortLdsEntries];
-    __shared__ unsigned long long few[kRankSortMax];
+    __shared__ unsigned long long few[kRankSortMax + 1];
     __shared__ uint32_t row_map[kRowMapWords];
+    // the ranking of a short list uses `few`'s bytes (a long list's rest comes later)
+    uint32_t* tally = reinterpret_cast<uint32_t*>(few);     // per key: smaller tokens | same token << 10 | same token, lower row << 20
+    uint32_t* placed = tally + kRankSortMax;                // rows by rank, kRankSortMax + 1 of them
     __shared__ uint32_t s_count, s_less, s_rest, s_below, s_wave_rows[kSortWaves];
-    // a pair leaves for the order: its row at position `at`, and what the row is told about
-    // its token's run (where the run starts, the row's index in it, its length)
-    auto emit = [&](uint32_t tok, uint32_t row, uint32_t at, uint32_t j, uint32_t R) {
+    uint32_t* __restrict__ row_s = order;
+    RunInfo* __restrict__ info = reinterpret_cast<RunInfo*>(order + order_info_word(N));
+    // a pair leaves for the order: its row at place `at`, and what the row is told
+    auto emit = [&](uint32_t tok, uint32_t row, uint32_t at, uint32_t j, uint32_t R, uint32_t next) {
         row_s[at] = row;
-        info[row] = RunInfo{tok, at - j, j, R};
+        RunInfo ri;
+        ri.tok = tok;
+        ri.start = at - j;
+        if (tok >= V) { ri.R = 0; ri.x = 0; }
+        else if (R <= kSoloRun) { ri.R = j == 0 ? R : 0u; ri.x = next; }
+        else { ri.R = R; ri.x = j; }
+        info[row] = ri;
     };
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & (kWave - 1);
     auto lanes_below = [&](unsigned long long mask) {     // set bits of `mask` below this lane
         return (uint32_t)__builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
     };
+#ifdef AGRAD_SORT_TIMING
+#define STAMP(k) if (tid == 0) spill[g * 8 + (k)] = wall_clock64();
+#else
+#define STAMP(k)
+#endif
+    STAMP(0)
     if (tid == 0) { s_count = 0; s_less = 0; s_rest = 0; s_below = 0; }
-    for (uint32_t w = tid; w < kRowMapWords; w += kSortBlock) row_map[w] = 0;
+    tally[tid] = 0;                     // kRankSortMax == kSortBlock
+    {   // this group's share of the gradient kernel's arrival counters
+        const uint32_t groups = 1u << log2G;
+        const uint32_t words = (uint32_t)(order_group_tickets(N) + order_run_tickets(N));
+        uint32_t* tickets = order + order_ticket_word(N);
+        for (uint32_t w = g * kSortBlock + tid; w < words; w += groups * kSortBlock) tickets[w] = 0;
+    }
     __syncthreads();
 
-    auto owner_of = [&](int32_t t, uint32_t& tok) {
-        const bool bad = t < 0 || (uint32_t)t >= V;
-        tok = bad ? V : (uint32_t)t;
-        return log2G ? (tok * 0x9E3779B1u) >> (32 - log2G) : 0u;
-    };
-
-    uint32_t less = 0;
+    STAMP(1)
+    uint32_t less = 0, worst = 0;                   // `worst`: the largest id seen, as unsigned (a negative id is huge)
     constexpr int ROUND = 16;                       // id loads in flight per thread
+    constexpr int AGG = 8;
     for (uint32_t base = 0; base < N; base += kSortBlock * ROUND) {
-        int32_t t[ROUND];
+        const bool whole = base + kSortBlock * ROUND <= N;          // no row of this round lies beyond N
+        uint32_t t[ROUND];
 #pragma unroll
         for (int r = 0; r < ROUND; ++r) {
             const uint32_t i = base + r * kSortBlock + tid;
-            t[r] = i < N ? ids[i] : -1;
+            t[r] = (whole || i < N) ? (uint32_t)ids[i] : 0u;
         }
         // The pairs this group owns go into the list.  One LDS atomic per wave and
         // eight loads, not one per pair: a frequent token would otherwise queue
         // thousands of them on one address, and waiting for each one's return
         // value in turn costs the usual case a microsecond.
-        constexpr int AGG = 8;
 #pragma unroll
         for (int r0 = 0; r0 < ROUND; r0 += AGG) {
             unsigned long long owners[AGG];
@@ -279,11 +326,11 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
 #pragma unroll
             for (int a = 0; a < AGG; ++a) {
                 const uint32_t i = base + (r0 + a) * kSortBlock + tid;
-                const bool live = i < N;
-                uint32_t tok;
-                const uint32_t owner = owner_of(t[r0 + a], tok);
-                if (live && tok == V && g == 0) *err_flag = 1;
-                less += live && owner < g ? 1u : 0u;
+                const bool live = whole || i < N;
+                worst = t[r0 + a] > worst ? t[r0 + a] : worst;
+                const uint32_t tok = t[r0 + a] < V ? t[r0 + a] : V;
+                const uint32_t owner = token_group(tok, log2G);
+                less += (live && owner < g) ? 1u : 0u;
                 owners[a] = __ballot(live && owner == g);
                 wave_total += (uint32_t)__popcll(owners[a]);
             }
@@ -293,11 +340,11 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
                 first = (uint32_t)__builtin_amdgcn_readfirstlane((int)first);
 #pragma unroll
                 for (int a = 0; a < AGG; ++a) {
+                    if (owners[a] == 0) continue;
                     const uint32_t i = base + (r0 + a) * kSortBlock + tid;
                     const uint32_t slot = first + lanes_below(owners[a]);
                     if (((owners[a] >> lane) & 1ull) && slot < kSortLdsEntries) {
-                        const int32_t id = t[r0 + a];
-                        const uint32_t tok = id < 0 || (uint32_t)id >= V ? V : (uint32_t)id;
+                        const uint32_t tok = t[r0 + a] < V ? t[r0 + a] : V;
                         keys[slot] = ((unsigned long long)tok << 32) | i;
                     }
                     first += (uint32_t)__popcll(owners[a]);
@@ -305,6 +352,8 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
             }
         }
     }
+    STAMP(2)
+    if (g == 0 && worst >= V) *err_flag = 1;
     // rows owned by lower groups: exact integer wave totals, added in LDS
     {
         uint32_t v = less;
@@ -314,28 +363,50 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
         v += __builtin_amdgcn_update_dpp(0, v, kDppRowMirror, 0xf, 0xf, true);
         v += __builtin_amdgcn_ds_swizzle(v, kSwizzleXor16);
         const uint32_t total = __builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 32);
-        if (lane == 0) atomicAdd(&s_less, total);
+        if (lane == 0 && total) atomicAdd(&s_less, total);
     }
     __syncthreads();
     const uint32_t count = s_count;
     const uint32_t offset = s_less;
+    STAMP(3)
 
     if (count <= kRankSortMax) {
-        // every key is unique, so its place in the order is the number of
-        // smaller keys.  Each thread counts that for its own key with broadcast
-        // LDS reads -- no barriers, no exchanges.
-        const unsigned long long mine = tid < count ? keys[tid] : ~0ull;
-        const uint32_t my_tok = (uint32_t)(mine >> 32);
-        uint32_t rank = 0, same = 0, same_before = 0;       // ... and its run: the keys with its token
+        // Every key is unique, so its place in the order is the number of smaller keys.
+        // The threads share the counting: `parts` threads per key, each comparing the key
+        // with its slice of the list (broadcast LDS reads), their tallies added in LDS.
+        uint32_t span = 1;                       // count rounded up to a power of two
+        while (span < count) span <<= 1;
+        const uint32_t parts = kSortBlock / span;
+        const uint32_t k = tid & (span - 1), part = tid / span;
+        const uint32_t j_lo = (part * count) / parts, j_hi = ((part + 1) * count) / parts;
+        const unsigned long long mine = k < count ? keys[k] : ~0ull;
+        const uint32_t my_tok = (uint32_t)(mine >> 32), my_row = (uint32_t)mine;
+        uint32_t smaller_tok = 0, same = 0, same_before = 0;
 #pragma unroll 8
-        for (uint32_t j = 0; j < count; ++j) {
-            const unsigned long long k = keys[j];
-            const bool smaller = k < mine, same_tok = (uint32_t)(k >> 32) == my_tok;
-            rank += smaller ? 1u : 0u;
-            same += same_tok ? 1u : 0u;
-            same_before += same_tok && smaller ? 1u : 0u;
+        for (uint32_t j = j_lo; j < j_hi; ++j) {
+            const unsigned long long other = keys[j];
+            const uint32_t tok = (uint32_t)(other >> 32), row = (uint32_t)other;
+            smaller_tok += tok < my_tok ? 1u : 0u;
+            same += tok == my_tok ? 1u : 0u;
+            same_before += (tok == my_tok && row < my_row) ? 1u : 0u;
         }
-        if (tid < count) emit(my_tok, (uint32_t)mine, offset + rank, same_before, same);
+        if (k < count) atomicAdd(&tally[k], smaller_tok | (same << 10) | (same_before << 20));
+        __syncthreads();
+        uint32_t rank = 0, run = 0, j = 0;
+        if (tid < count) {
+            const uint32_t packed = tally[tid];
+            j = packed >> 20;
+            run = (packed >> 10) & 1023u;
+            rank = (packed & 1023u) + j;
+            placed[rank] = (uint32_t)keys[tid];
+        }
+        __syncthreads();
+        STAMP(4)
+        if (tid < count) {
+            const uint32_t next = j + 1 < run ? placed[rank + 1] : kNoRow;
+            emit((uint32_t)(keys[tid] >> 32), (uint32_t)keys[tid], offset + rank, j, run, next);
+        }
+        STAMP(5)
         return;
     }
 
@@ -356,7 +427,8 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
             if (votes > best_votes) { best_votes = votes; hot = candidate; }
         }
     }
-    if (reread) __syncthreads();         // `keys` is about to be overwritten
+    for (uint32_t w = tid; w < kRowMapWords; w += kSortBlock) row_map[w] = 0;
+    __syncthreads();         // the map is clear, and `keys` may be overwritten
 
     // its rows go into the row map, every other pair into `rest`.  A list that
     // fits LDS is split from LDS and stays intact; a longer one is read again
@@ -370,6 +442,10 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
             const uint32_t slot = atomicAdd(&s_rest, 1u);
             if (slot < rest_cap) rest[slot] = ((unsigned long long)tok << 32) | row;
         }
+    };
+    auto owner_of = [&](int32_t t, uint32_t& tok) {
+        tok = (uint32_t)t < V ? (uint32_t)t : V;
+        return token_group(tok, log2G);
     };
     if (!reread) {
         for (uint32_t i = tid; i < count; i += kSortBlock) {
@@ -405,17 +481,20 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
     __syncthreads();
     const uint32_t rest_n = s_rest;
 
+    // pairs of a sorted list: a pair's run is found by bisection, its successor is its neighbour
+    auto emit_sorted = [&](const unsigned long long* sorted, uint32_t n, uint32_t i, uint32_t shift) {
+        const unsigned long long key = sorted[i];
+        const uint32_t tok = (uint32_t)(key >> 32);
+        const uint32_t lo = first_not_below(sorted, n, (unsigned long long)tok << 32);
+        const uint32_t hi = first_not_below(sorted, n, (unsigned long long)(tok + 1u) << 32);
+        emit(tok, (uint32_t)key, offset + i + shift, i - lo, hi - lo, i + 1 < hi ? (uint32_t)sorted[i + 1] : kNoRow);
+    };
+
     if (rest_n > rest_cap) {
         if (!reread) {
             // no single frequent token: the network over the whole list
             bitonic_sort_u64<kSortBlock>(keys, count, tid, [] { __syncthreads(); });
-            for (uint32_t i = tid; i < count; i += kSortBlock) {
-                const unsigned long long key = keys[i];
-                const uint32_t tok = (uint32_t)(key >> 32);
-                const uint32_t lo = first_not_below(keys, count, (unsigned long long)tok << 32);
-                const uint32_t hi = first_not_below(keys, count, (unsigned long long)(tok + 1u) << 32);
-                emit(tok, (uint32_t)key, offset + i, i - lo, hi - lo);
-            }
+            for (uint32_t i = tid; i < count; i += kSortBlock) emit_sorted(keys, count, i, 0u);
             return;
         }
         // gather the group's pairs into its slice of `spill` (slices are
@@ -431,48 +510,22 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
         __threadfence_block();
         __syncthreads();
         bitonic_sort_u64<kSortBlock>(mine, count, tid, [] { __threadfence_block(); __syncthreads(); });
-        for (uint32_t i = tid; i < count; i += kSortBlock) {
-            const unsigned long long key = mine[i];
-            const uint32_t tok = (uint32_t)(key >> 32);
-            const uint32_t lo = first_not_below(mine, count, (unsigned long long)tok << 32);
-            const uint32_t hi = first_not_below(mine, count, (unsigned long long)(tok + 1u) << 32);
-            emit(tok, (uint32_t)key, offset + i, i - lo, hi - lo);
-        }
+        for (uint32_t i = tid; i < count; i += kSortBlock) emit_sorted(mine, count, i, 0u);
         return;
     }
 
     // -- the rest, in order; pairs above the frequent token leave room for its rows
     const uint32_t hot_rows = count - rest_n;
-    uint32_t below;                                // pairs of the rest that sort before the frequent token
-    if (rest_n <= kRankSortMax) {
-        const unsigned long long mine = tid < rest_n ? rest[tid] : ~0ull;
-        const uint32_t tok = (uint32_t)(mine >> 32);
-        uint32_t rank = 0, same = 0, same_before = 0;
-#pragma unroll 8
-        for (uint32_t j = 0; j < rest_n; ++j) {
-            const unsigned long long k = rest[j];
-            const bool smaller = k < mine, same_tok = (uint32_t)(k >> 32) == tok;
-            rank += smaller ? 1u : 0u;
-            same += same_tok ? 1u : 0u;
-            same_before += same_tok && smaller ? 1u : 0u;
-        }
-        if (tid < rest_n) emit(tok, (uint32_t)mine, offset + rank + (tok > hot ? hot_rows : 0u), same_before, same);
-        below = (uint32_t)__syncthreads_count(tid < rest_n && tok < hot);
-    } else {
-        bitonic_sort_u64<kSortBlock>(rest, rest_n, tid, [] { __syncthreads(); });
-        uint32_t n_below = 0;
-        for (uint32_t i = tid; i < rest_n; i += kSortBlock) {
-            const unsigned long long key = rest[i];
-            const uint32_t tok = (uint32_t)(key >> 32);
-            n_below += tok < hot ? 1u : 0u;
-            const uint32_t lo = first_not_below(rest, rest_n, (unsigned long long)tok << 32);
-            const uint32_t hi = first_not_below(rest, rest_n, (unsigned long long)(tok + 1u) << 32);
-            emit(tok, (uint32_t)key, offset + i + (tok > hot ? hot_rows : 0u), i - lo, hi - lo);
-        }
-        if (n_below) atomicAdd(&s_below, n_below);
-        __syncthreads();
-        below = s_below;
+    bitonic_sort_u64<kSortBlock>(rest, rest_n, tid, [] { __syncthreads(); });
+    uint32_t n_below = 0;                          // pairs of the rest that sort before the frequent token
+    for (uint32_t i = tid; i < rest_n; i += kSortBlock) {
+        const uint32_t tok = (uint32_t)(rest[i] >> 32);
+        n_below += tok < hot ? 1u : 0u;
+        emit_sorted(rest, rest_n, i, tok > hot ? hot_rows : 0u);
     }
+    if (n_below) atomicAdd(&s_below, n_below);
+    __syncthreads();
+    const uint32_t below = s_below;
 
     // -- the frequent token's rows.  Word w of the map holds rows 32 w ... 32 w + 31.
     // The waves share the words that rows below N can mark, an even number each;
@@ -506,7 +559,7 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
         const uint32_t word = upper ? word1 : word0;
         if ((word >> bit) & 1u) {
             const uint32_t to = at + (upper ? n0 : 0u) + (uint32_t)__popc(word & ((1u << bit) - 1u));
-            emit(hot, (w0 + upper) * 32u + bit, to, to - (offset + below), hot_rows);
+            emit(hot, (w0 + upper) * 32u + bit, to, to - (offset + below), hot_rows, kNoRow);
         }
         at += n0 + (uint32_t)__popc(word1);
     }
@@ -525,10 +578,9 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
 inline uint32_t group_sort_log2g(uint32_t n) { return n > 32768 ? 9u : n > 16384 ? 8u : n > 1024 ? 7u : 4u; }
 
 __global__ void __launch_bounds__(kSortBlock)
-emb_group_sort_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ row_s,
-                      RunInfo* __restrict__ info, unsigned long long* __restrict__ spill,
-                      uint32_t N, uint32_t V, uint32_t log2G, int* err_flag) {
-    emb_group_sort_body(blockIdx.x, ids, row_s, info, spill, N, V, log2G, err_flag);
+emb_group_sort_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ order,
+                      unsigned long long* __restrict__ spill, uint32_t N, uint32_t V, uint32_t log2G, int* err_flag) {
+    emb_group_sort_body(blockIdx.x, ids, order, spill, N, V, log2G, err_flag);
 }
 
 // Forward gather and the ordering of the ids for the later gradient in ONE
@@ -546,11 +598,11 @@ template <typename T, int VEC, bool RAW>
 __global__ void __launch_bounds__(kSortBlock) __attribute__((amdgpu_num_sgpr(80)))
 gather_sort_kernel(const int32_t* __restrict__ ids, const T* __restrict__ W, const T* __restrict__ wpe,
                    T* __restrict__ out, uint32_t total, uint32_t CV, uint32_t C, uint32_t T_len, uint32_t V,
-                   uint32_t* __restrict__ row_s, RunInfo* __restrict__ info, unsigned long long* __restrict__ spill,
+                   uint32_t* __restrict__ order, unsigned long long* __restrict__ spill,
                    uint32_t N, uint32_t log2G, int* err_flag) {
     const uint32_t groups = 1u << log2G;
     if (blockIdx.x < groups) {
-        emb_group_sort_body(blockIdx.x, ids, row_s, info, spill, N, V, log2G, err_flag);
+        emb_group_sort_body(blockIdx.x, ids, order, spill, N, V, log2G, err_flag);
         return;
     }
     const uint32_t idx = (blockIdx.x - groups) * kSortBlock + threadIdx.x;
@@ -586,233 +638,282 @@ __device__ __forceinline__ void store_grad_row(T* dW, uint64_t off, const float 
     VecIO<T, VEC>::store(dW + off, o);
 }
 
-// The gradient sum proper, in ROW order.  A workgroup takes kRowBatch consecutive rows of
-// dY (or, with a position table, the B rows b*T + t of one position t, a batch at a
-// time); a thread takes one column vector.  One 16-byte scalar load tells a row what it
-// is (RunInfo, written by the ordering step):
-//   * the first row of its token's run (the lowest row number) when the run has up to
-//     kSoloRun rows: it adds the run's rows in ascending order -- the very sequence of
-//     fp32 adds np.add.at makes -- and stores the table row.  Most rows are their token's
-//     only row and just move their vector; a batch keeps all of its rows in flight.
-//   * a row of a LONGER run (a frequent token: padding, "the").  S evenly spaced rows of
-//     the run are its workers; worker w sums column slab w over all of the run's rows,
-//     its threads laid out as columns x row lanes: a lane adds every lanes-th row in
-//     ascending order with kLongBatch loads in flight, and the lanes are then added in
-//     lane order.  A fixed association: the same bits on every run.
+// The gradient sum proper, in ROW order, one launch.  A wave takes one row of dY and one
+// block of 64 column vectors (with a position table: the B rows b*T + t of one position t,
+// a batch at a time, whose vectors it also adds in ascending b: dwpe[t, :] (+)= sum_b
+// dY[b, t, :]).  One 16-byte scalar load tells it what the row is (RunInfo):
+//   * the first row of its token's run when the run has up to kSoloRun rows: it adds the
+//     run's rows in ascending order -- the very sequence of fp32 adds np.add.at makes --
+//     and stores the table row.  Most rows are their token's only row and just move
+//     their vector;
+//   * a row of a LONGER run (a frequent token: padding, "the").  Every kChunkRows-th row
+//     of the run adds up the chunk of rows that starts with it (whole rows, read once,
+//     eight in flight) and leaves the partial row in the workspace.  The wave that
+//     completes a group of kGroupChunks chunks -- it learns that from an arrival counter
+//     -- adds the group's partial rows in chunk order, and the wave that completes the
+//     run's last group adds the groups in order and stores the table row.  Which wave
+//     does the adding varies from run to run, what it adds in which order does not: the
+//     same bits every time.  The counters are zero before and after the call;
 //   * any other row: nothing to do for the table.
-// dY is read front to back, every row of dW is written once, by one workgroup: no
-// atomics, no partial sums in memory, no second launch.  With a position table the
-// workgroup also adds its B rows' vectors in ascending b, from the same loads:
-// dwpe[t, :] (+)= sum_b dY[b, t, :].
-constexpr int kRowBatch = 8;          // rows of a workgroup, all in flight together
-constexpr int kLongBatch = 8;         // rows a lane of a long run's slab keeps in flight
-constexpr uint32_t kSoloRun = 16;     // longest run its first row's workgroup sums alone
-constexpr uint32_t kMaxSlabs = 64;    // most workgroups sharing a longer run
-constexpr int kRowSumMaxBlock = 512;
+// dY is read once, every row of dW is written once: no float atomics, no second launch.
+constexpr int kRowBatch = 8;          // rows a wave keeps in flight
+constexpr int kRowSumBlock = 256;
+constexpr uint32_t kRowSumWaves = kRowSumBlock / kWave;
 
-// Column vectors per slab of a run of R rows: at least a 64th of the row and at least a
-// row's share when the run has fewer rows than that; otherwise `min_slab` (whole cache
-// lines per access), narrowed when the run is so long that a lane would otherwise walk
-// more than a few batches of rows.
-__device__ __forceinline__ uint32_t slab_width(uint32_t R, uint32_t CV, uint32_t block, uint32_t min_slab) {
-    const uint32_t w_min = (CV + kMaxSlabs - 1) / kMaxSlabs;
-    const uint32_t w_rows = (CV + R - 1) / R;
-    uint32_t w_lat = (uint32_t)(((uint64_t)4 * kLongBatch * block) / R);
-    w_lat = w_lat ? w_lat : 1u;
-    uint32_t width = min_slab < w_lat ? min_slab : w_lat;
-    width = width > w_min ? width : w_min;
-    width = width > w_rows ? width : w_rows;
-    return width;
+// Partial rows travel between waves of one launch, which may sit on different L2 caches:
+// they are written and read with device-scope accesses (which go past the L2 to where
+// all of the GPU's caches agree), two floats at a time, so that the arrival counters
+// need no cache write-back or invalidation.
+template <int VEC>
+__device__ __forceinline__ void store_partial(float* p, const float (&acc)[VEC]) {
+    if constexpr (VEC % 2 == 0) {
+#pragma unroll
+        for (int k = 0; k < VEC; k += 2) {
+            const unsigned long long w = (unsigned long long)__float_as_uint(acc[k]) | ((unsigned long long)__float_as_uint(acc[k + 1]) << 32);
+            __hip_atomic_store(reinterpret_cast<unsigned long long*>(p + k), w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) __hip_atomic_store(p + k, acc[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 }
 
-// Slab `w` of a long run: rows row_s[start .. start + R) of dY, summed for one band of
-// columns by the whole workgroup (every thread calls it with the same arguments).
-template <typename T, typename TO, int VEC>
-__device__ __forceinline__ void
-emb_long_run_slab(float* part, const uint32_t* __restrict__ row_s, const T* __restrict__ dY, TO* dW, uint32_t tok,
-                  uint32_t start, uint32_t R, uint32_t w, uint32_t width, uint32_t C, uint32_t CV, int accumulate) {
+template <int VEC>
+__device__ __forceinline__ void load_partial(const float* p, float (&v)[VEC]) {
+    if constexpr (VEC % 2 == 0) {
+#pragma unroll
+        for (int k = 0; k < VEC; k += 2) {
+            const unsigned long long w = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p + k), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            v[k] = __uint_as_float((uint32_t)w);
+            v[k + 1] = __uint_as_float((uint32_t)(w >> 32));
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) v[k] = __hip_atomic_load(p + k, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+// acc += dY[row_s[p], col ...] for p = from .. to-1, ascending (p is the same in every lane)
+template <typename T, int VEC>
+__device__ __forceinline__ void add_listed_rows(float (&acc)[VEC], const uint32_t* __restrict__ row_s, uint32_t from,
+                                                uint32_t to, const T* __restrict__ dY, uint32_t C, uint32_t col, bool live) {
     typedef RawVec<T, VEC> Raw;
-    const uint32_t slab_lo = w * width;
-    const uint32_t slab_hi = slab_lo + width < CV ? slab_lo + width : CV;
-    const uint32_t cols = width < blockDim.x ? width : blockDim.x;
-    const uint32_t lanes = blockDim.x / cols;
-    const uint32_t colv = threadIdx.x % cols, lane = threadIdx.x / cols;
-    for (uint32_t c0 = slab_lo; c0 < slab_hi; c0 += cols) {
-        const uint32_t scv = c0 + colv;
-        const bool on = lane < lanes && scv < slab_hi;
-        float acc[VEC];
-#pragma unroll
-        for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
-        if (on) {
 #pragma nounroll
-            for (uint32_t q0 = lane; q0 < R; q0 += lanes * kLongBatch) {
-                uint32_t rr[kLongBatch];
-                typename Raw::type v[kLongBatch];
+    for (uint32_t p = from; p < to; p += kRowBatch) {
+        uint32_t rr[kRowBatch];
+        typename Raw::type v[kRowBatch];
 #pragma unroll
-                for (int q = 0; q < kLongBatch; ++q) {
-                    const uint32_t at_q = q0 + (uint32_t)q * lanes;
-                    rr[q] = at_q < R ? row_s[start + at_q] : 0u;
-                }
+        for (int q = 0; q < kRowBatch; ++q) rr[q] = p + q < to ? row_s[p + q] : 0u;
 #pragma unroll
-                for (int q = 0; q < kLongBatch; ++q) {
-                    const uint32_t at_q = q0 + (uint32_t)q * lanes;
-                    v[q] = Raw::zero();
-                    if (at_q < R) v[q] = Raw::load(dY + (uint64_t)rr[q] * C + (uint64_t)scv * VEC);
-                }
+        for (int q = 0; q < kRowBatch; ++q) {
+            v[q] = Raw::zero();
+            if (p + q < to && live) v[q] = Raw::load(dY + (uint64_t)rr[q] * C + col);
+        }
 #pragma unroll
-                for (int q = 0; q < kLongBatch; ++q) {
-                    const uint32_t at_q = q0 + (uint32_t)q * lanes;
-                    if (at_q < R) {
-                        float x[VEC];
-                        Raw::unpack(v[q], x);
+        for (int q = 0; q < kRowBatch; ++q) {
+            if (p + q < to) {
+                float x[VEC];
+                Raw::unpack(v[q], x);
 #pragma unroll
-                        for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + x[k];
-                    }
-                }
+                for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + x[k];
             }
         }
-        __syncthreads();            // the previous pass's readers are done with `part`
-        if (lane < lanes) {
+    }
+}
+
+// sum = slots[first], slots[first + step], ... (n of them), added in that order; the
+// partial rows were written by other waves of this launch
+template <int VEC>
+__device__ __forceinline__ void add_partial_rows(float (&sum)[VEC], const float* slots, uint64_t first, uint64_t step,
+                                                 uint32_t n, uint32_t C, uint32_t col, bool live) {
+    constexpr int BATCH = VEC >= 8 ? 4 : 8;         // partial rows in flight
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) part[(lane * cols + colv) * VEC + k] = acc[k];
+    for (int k = 0; k < VEC; ++k) sum[k] = 0.0f;
+#pragma nounroll
+    for (uint32_t i0 = 0; i0 < n; i0 += BATCH) {
+        float v[BATCH][VEC];
+#pragma unroll
+        for (int q = 0; q < BATCH; ++q) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) v[q][k] = 0.0f;
+            if (i0 + q < n && live) load_partial<VEC>(slots + (first + (uint64_t)(i0 + q) * step) * C + col, v[q]);
         }
-        __syncthreads();
-        if (lane == 0 && scv < slab_hi) {
-            float sum[VEC];
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) sum[k] = part[colv * VEC + k];
-            for (uint32_t q = 1; q < lanes && q < R; ++q)
+        for (int q = 0; q < BATCH; ++q) {
+            if (i0 + q < n) {
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) sum[k] = sum[k] + part[(q * cols + colv) * VEC + k];
-            store_grad_row<TO, VEC>(dW, (uint64_t)tok * C + (uint64_t)scv * VEC, sum, accumulate != 0);
+                for (int k = 0; k < VEC; ++k) sum[k] = (i0 + q == 0) ? v[q][k] : sum[k] + v[q][k];
+            }
         }
     }
+}
+
+// One arrival at a counter; true for the wave whose arrival is number `expected` (it also
+// puts the counter back to zero).  A wave arrives after its partial rows have been
+// written (its device-scope stores have completed before the counter moves), so the wave
+// that arrives last finds all of them.
+__device__ __forceinline__ bool arrive_last(uint32_t* ticket, uint32_t expected, uint32_t lane) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");          // wait for this wave's stores
+    uint32_t old = 0;
+    if (lane == 0) old = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    old = (uint32_t)__builtin_amdgcn_readfirstlane((int)old);
+    if (old + 1u != expected) return false;
+    if (lane == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    return true;
 }
 
 template <typename T, typename TO, int VEC, bool POS>
-__global__ void __launch_bounds__(kRowSumMaxBlock)
-emb_row_sum_kernel(const RunInfo* __restrict__ info, const uint32_t* __restrict__ row_s, const T* __restrict__ dY,
-                   TO* dW, TO* dwpe, uint32_t N, uint32_t C, uint32_t CV, uint32_t V, uint32_t T_len, uint32_t B,
-                   int accumulate, int accumulate_pos, uint32_t min_slab) {
-    __shared__ float part[kRowSumMaxBlock * VEC];
+__global__ void __launch_bounds__(kRowSumBlock)
+emb_row_sum_kernel(const uint32_t* __restrict__ order, uint32_t* group_tickets, const T* __restrict__ dY, TO* dW,
+                   TO* dwpe, float* part, uint32_t N, uint32_t C, uint32_t CV, uint32_t CB, uint32_t V, uint32_t T_len, uint32_t B,
+                   int accumulate, int accumulate_pos) {
     typedef RawVec<T, VEC> Raw;
-    const uint32_t first = POS ? blockIdx.x : blockIdx.x * kRowBatch;
-    const uint32_t row_step = POS ? T_len : 1u;
-    const uint32_t n_rows = POS ? B : (N - first < (uint32_t)kRowBatch ? N - first : (uint32_t)kRowBatch);
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t unit = (uint32_t)__builtin_amdgcn_readfirstlane((int)(blockIdx.x * kRowSumWaves + threadIdx.x / kWave));
+    const uint32_t units = (POS ? T_len : N) * CB;
+    if (unit >= units) return;
+    const uint32_t first = unit / CB, kb = unit - first * CB;
+    const uint32_t cv = kb * kWave + lane;
+    const bool live = cv < CV;
+    const uint32_t col = cv * VEC;
+    const uint32_t* __restrict__ row_s = order;
+    const RunInfo* __restrict__ info = reinterpret_cast<const RunInfo*>(order + order_info_word(N));
+    uint32_t* run_tickets = group_tickets + order_group_tickets(N);     // (the counters follow the RunInfo words of `order`)
+    float* part2 = part + (uint64_t)(N / kChunkRows + 1) * C;          // the groups' partial rows
 
-    for (uint32_t cv0 = 0; cv0 < CV; cv0 += blockDim.x) {       // one pass unless a row is wider than the workgroup
-        const uint32_t cv = cv0 + threadIdx.x;
-        const bool live = cv < CV;
-        const uint32_t col = cv * VEC;
+    // row `n` of a long run (the wave's column block only)
+    auto long_run_row = [&](const RunInfo& ri) {
+        const uint32_t R = ri.R, j = ri.x, start = ri.start;
+        const uint32_t n1 = R / kChunkRows;                             // chunks (at least 2)
+        if (j % kChunkRows != 0 || j / kChunkRows >= n1) return;
+        const uint32_t c = j / kChunkRows;
+        const uint32_t lo = start + c * kChunkRows, hi = c + 1 == n1 ? start + R : lo + kChunkRows;
+        float acc[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
+        add_listed_rows<T, VEC>(acc, row_s, lo, hi, dY, C, col, live);
+        if (live) store_partial<VEC>(part + (uint64_t)(lo / kChunkRows) * C + col, acc);
+        // the group of chunks this one belongs to, and its counter
+        const uint32_t n2 = n1 / kGroupChunks ? n1 / kGroupChunks : 1u;   // groups
+        const uint32_t q = c / kGroupChunks < n2 ? c / kGroupChunks : n2 - 1;
+        const uint32_t c_lo = q * kGroupChunks, c_hi = q + 1 == n2 ? n1 : c_lo + kGroupChunks;
+        const uint32_t g_at = start + c_lo * kChunkRows;                  // where the group starts
+        const uint32_t fold = kb % kTicketFold, n_fold = (CB - 1 - fold) / kTicketFold + 1;
+        if (!arrive_last(group_tickets + (g_at / (kChunkRows * 2)) * kTicketFold + fold, (c_hi - c_lo) * n_fold, lane)) return;
+        for (uint32_t kb2 = fold; kb2 < CB; kb2 += kTicketFold) {
+            const uint32_t cv2 = kb2 * kWave + lane, col2 = cv2 * VEC;
+            const bool live2 = cv2 < CV;
+            float sum[VEC];
+            add_partial_rows<VEC>(sum, part, g_at / kChunkRows, 1, c_hi - c_lo, C, col2, live2);
+            if (!live2) continue;
+            if (n2 == 1) store_grad_row<TO, VEC>(dW, (uint64_t)ri.tok * C + col2, sum, accumulate != 0);
+            else store_partial<VEC>(part2 + (uint64_t)(g_at / (kChunkRows * kGroupChunks)) * C + col2, sum);
+        }
+        if (n2 == 1) return;
+        if (!arrive_last(run_tickets + (start / (kChunkRows * kGroupChunks * 2)) * kTicketFold + fold, n2, lane)) return;
+        for (uint32_t kb2 = fold; kb2 < CB; kb2 += kTicketFold) {
+            const uint32_t cv2 = kb2 * kWave + lane, col2 = cv2 * VEC;
+            const bool live2 = cv2 < CV;
+            float sum[VEC];
+            // group q' starts at start + q' * 512: its slot is (start + q' * 512) / 512
+            add_partial_rows<VEC>(sum, part2, start / (kChunkRows * kGroupChunks), 1, n2, C, col2, live2);
+            if (live2) store_grad_row<TO, VEC>(dW, (uint64_t)ri.tok * C + col2, sum, accumulate != 0);
+        }
+    };
+
+    // the first row of a short run: `own` is its vector, `second` the run's second row's
+    auto short_run_head = [&](const RunInfo& ri, const typename Raw::type& own, const typename Raw::type& second) {
+        float acc[VEC];
+        Raw::unpack(own, acc);
+        if (ri.R >= 2) {
+            float x[VEC];
+            Raw::unpack(second, x);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + x[k];
+            if (ri.R > 2) add_listed_rows<T, VEC>(acc, row_s, ri.start + 2, ri.start + ri.R, dY, C, col, live);
+        }
+        if (live) store_grad_row<TO, VEC>(dW, (uint64_t)ri.tok * C + col, acc, accumulate != 0);
+    };
+    auto load_second = [&](const RunInfo& ri) {
+        typename Raw::type second = Raw::zero();
+        if (ri.R >= 2 && ri.R <= kSoloRun) {
+            const uint32_t r1 = ri.x != kNoRow ? ri.x : row_s[ri.start + 1];
+            if (live) second = Raw::load(dY + (uint64_t)r1 * C + col);
+        }
+        return second;
+    };
+
+    if constexpr (!POS) {
+        const RunInfo ri = info[first];
+        if (ri.R == 0) return;
+        if (ri.R > kSoloRun) { long_run_row(ri); return; }
+        typename Raw::type own = Raw::zero();
+        if (live) own = Raw::load(dY + (uint64_t)first * C + col);
+        short_run_head(ri, own, load_second(ri));
+    } else {
         float pos_acc[VEC];
 #pragma unroll
         for (int k = 0; k < VEC; ++k) pos_acc[k] = 0.0f;
-
-        for (uint32_t b0 = 0; b0 < n_rows; b0 += kRowBatch) {
-            // what each row of the batch is (the same in every thread: scalar loads)
-            RunInfo inf[kRowBatch];
-            bool solo[kRowBatch];
-#pragma unroll
-            for (int i = 0; i < kRowBatch; ++i) {
-                inf[i] = RunInfo{V, 0u, 1u, 1u};
-                if (b0 + i < n_rows) inf[i] = info[first + (b0 + i) * row_step];
-                solo[i] = inf[i].tok < V && inf[i].j == 0 && inf[i].R <= kSoloRun;
-            }
-            // the vectors that are certainly wanted: a run's first row (and, for the position
-            // table, every row), and the second row of a run of two
-            typename Raw::type own[kRowBatch], two[kRowBatch];
-#pragma unroll
-            for (int i = 0; i < kRowBatch; ++i) {
-                own[i] = Raw::zero();
-                const bool want = (POS && b0 + i < n_rows) || solo[i];
-                if (want && live) own[i] = Raw::load(dY + (uint64_t)(first + (b0 + i) * row_step) * C + col);
-            }
-#pragma unroll
-            for (int i = 0; i < kRowBatch; ++i) {
-                two[i] = Raw::zero();
-                if (solo[i] && inf[i].R >= 2) {
-                    const uint32_t r = row_s[inf[i].start + 1];
-                    if (live) two[i] = Raw::load(dY + (uint64_t)r * C + col);
-                }
-            }
-#pragma unroll
-            for (int i = 0; i < kRowBatch; ++i) {
-                float acc[VEC];
-                Raw::unpack(own[i], acc);
-                if constexpr (POS) {
-                    if (b0 + i < n_rows) {
-#pragma unroll
-                        for (int k = 0; k < VEC; ++k) pos_acc[k] = b0 + i == 0 ? acc[k] : pos_acc[k] + acc[k];
-                    }
-                }
-                if (solo[i]) {
-                    if (inf[i].R >= 2) {
-                        float x[VEC];
-                        Raw::unpack(two[i], x);
-#pragma unroll
-                        for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + x[k];
-                    }
 #pragma nounroll
-                    for (uint32_t r0 = 2; r0 < inf[i].R; r0 += kRowBatch) {       // rows 3 .. kSoloRun of the run
-                        typename Raw::type v[kRowBatch];
+        for (uint32_t b0 = 0; b0 < B; b0 += kRowBatch) {
+            RunInfo ri[kRowBatch];
+            typename Raw::type own[kRowBatch], second[kRowBatch];
 #pragma unroll
-                        for (int q = 0; q < kRowBatch; ++q) {
-                            v[q] = Raw::zero();
-                            if (r0 + q < inf[i].R) {
-                                const uint32_t r = row_s[inf[i].start + r0 + q];
-                                if (live) v[q] = Raw::load(dY + (uint64_t)r * C + col);
-                            }
-                        }
-#pragma unroll
-                        for (int q = 0; q < kRowBatch; ++q) {
-                            if (r0 + q < inf[i].R) {
-                                float x[VEC];
-                                Raw::unpack(v[q], x);
-#pragma unroll
-                                for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + x[k];
-                            }
-                        }
-                    }
-                    if (live) store_grad_row<TO, VEC>(dW, (uint64_t)inf[i].tok * C + col, acc, accumulate != 0);
+            for (int i = 0; i < kRowBatch; ++i) {
+                ri[i] = RunInfo{V, 0u, 0u, 0u};
+                own[i] = Raw::zero();
+                if (b0 + i < B) {
+                    const uint32_t n = (b0 + i) * T_len + first;
+                    ri[i] = info[n];
+                    if (live) own[i] = Raw::load(dY + (uint64_t)n * C + col);
                 }
             }
-            // longer runs: is one of these rows a worker of its run?  (first column pass only:
-            // a slab covers its columns whatever the workgroup's width)
-            if (cv0 == 0) {
 #pragma unroll
-                for (int i = 0; i < kRowBatch; ++i) {
-                    if (inf[i].tok < V && inf[i].R > kSoloRun) {
-                        const uint32_t R = inf[i].R;
-                        const uint32_t width = slab_width(R, CV, blockDim.x, min_slab);
-                        const uint32_t slabs = (CV + width - 1) / width;        // at most kMaxSlabs, at most R
-                        const uint32_t stride = R / slabs;
-                        const uint32_t w = inf[i].j / stride;
-                        if (w * stride == inf[i].j && w < slabs)
-                            emb_long_run_slab<T, TO, VEC>(part, row_s, dY, dW, inf[i].tok, inf[i].start, R, w, width, C, CV, accumulate);
-                    }
-                }
+            for (int i = 0; i < kRowBatch; ++i) second[i] = load_second(ri[i]);
+#pragma unroll
+            for (int i = 0; i < kRowBatch; ++i) {
+                if (b0 + i >= B) continue;
+                float x[VEC];
+                Raw::unpack(own[i], x);
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) pos_acc[k] = b0 + i == 0 ? x[k] : pos_acc[k] + x[k];
+                if (ri[i].R == 0) continue;
+                if (ri[i].R > kSoloRun) long_run_row(ri[i]);
+                else short_run_head(ri[i], own[i], second[i]);
             }
         }
-        if constexpr (POS) {
-            if (live) store_grad_row<TO, VEC>(dwpe, (uint64_t)blockIdx.x * C + col, pos_acc, accumulate_pos != 0);
-        }
+        if (live) store_grad_row<TO, VEC>(dwpe, (uint64_t)first * C + col, pos_acc, accumulate_pos != 0);
     }
 }
 
-// The radix path's ordering is by token throughout: the run of position p is found by
-// two bisections of the sorted tokens.
+// The radix path's ordering is by token throughout: the run of place p is found by two
+// bisections of the sorted tokens.  Also zeroes the gradient kernel's arrival counters.
 __global__ void __launch_bounds__(256)
-emb_run_info_kernel(const uint32_t* __restrict__ tok_s, const uint32_t* __restrict__ row_s, RunInfo* __restrict__ info,
-                    uint32_t N) {
+emb_run_info_kernel(const uint32_t* __restrict__ tok_s, uint32_t* __restrict__ order, uint32_t N, uint32_t V) {
     const uint32_t p = blockIdx.x * 256 + threadIdx.x;
+    {
+        const uint32_t words = (uint32_t)(order_group_tickets(N) + order_run_tickets(N));
+        uint32_t* tickets = order + order_ticket_word(N);
+        for (uint32_t w = p; w < words; w += gridDim.x * 256) tickets[w] = 0;
+    }
     if (p >= N) return;
+    const uint32_t* row_s = order;
+    RunInfo* info = reinterpret_cast<RunInfo*>(order + order_info_word(N));
     const uint32_t tok = tok_s[p];
-    uint32_t lo = 0, hi = p;                    // first position holding tok
+    uint32_t lo = 0, hi = p;                    // first place holding tok
     while (lo < hi) { const uint32_t mid = (lo + hi) >> 1; if (tok_s[mid] < tok) lo = mid + 1; else hi = mid; }
     const uint32_t start = lo;
-    lo = p + 1; hi = N;                         // first position after the run
+    lo = p + 1; hi = N;                         // first place after the run
     while (lo < hi) { const uint32_t mid = (lo + hi) >> 1; if (tok_s[mid] <= tok) lo = mid + 1; else hi = mid; }
-    info[row_s[p]] = RunInfo{tok, start, p - start, lo - start};
+    const uint32_t R = lo - start, j = p - start;
+    RunInfo ri;
+    ri.tok = tok;
+    ri.start = start;
+    if (tok >= V) { ri.R = 0; ri.x = 0; }
+    else if (R <= kSoloRun) { ri.R = j == 0 ? R : 0u; ri.x = j + 1 < R ? row_s[p + 1] : kNoRow; }
+    else { ri.R = R; ri.x = j; }
+    info[row_s[p]] = ri;
 }
 
 // dwpe[t, c] (+)= sum_b dY[b, t, c], b ascending
@@ -867,32 +968,28 @@ int plan_sort(uint64_t N, uint32_t V, SortPlan* p) {
     return AGRAD_OK;
 }
 
-// The order: row_s[N] (rows, each token's run adjacent and ascending), then, from the
-// next multiple of four words on, one RunInfo per row.
-inline uint64_t order_info_word(uint64_t N) { return (N + 3) & ~3ull; }
-inline uint64_t order_bytes(uint64_t N) { return align256((order_info_word(N) + 4 * N) * 4); }
+// bytes of the order buffer (see order_words)
+inline uint64_t order_bytes(uint64_t N) { return align256(order_words(N) * 4); }
 
-// A long run's column slabs are at least this many 16-byte vectors wide (two cache
-// lines per access) unless the run is long enough to want more workgroups.
-constexpr uint32_t kMinSlabVectors = 8;
+// fp32 partial rows of the long runs: one per chunk, one per group of chunks
+inline uint64_t partial_rows(uint64_t N) { return N / kChunkRows + 1 + N / (kChunkRows * kGroupChunks) + 1; }
 
 template <typename T, typename TO = T>
-int embedding_sum_typed(hipStream_t s, const uint32_t* order, const T* dY, TO* dW, uint32_t N, uint32_t C, uint32_t V,
-                        uint32_t flags, TO* dwpe, uint32_t B, uint32_t T_len) {
-    const uint32_t* row_s = order;
-    const RunInfo* info = reinterpret_cast<const RunInfo*>(order + order_info_word(N));
+int embedding_sum_typed(hipStream_t s, const uint32_t* order, const T* dY, TO* dW, float* part, uint32_t N, uint32_t C,
+                        uint32_t V, uint32_t flags, TO* dwpe, uint32_t B, uint32_t T_len) {
     const int acc = (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0;
     const int acc_pos = (flags & AGRAD_ACC_PARAM_GRAD2) ? 1 : 0;
     constexpr int WIDE = WideVec<T>::value;
     // (a bf16 row under an fp32 upstream moves 8 bytes per vector: 8-byte alignment is implied by 16)
     const bool wide = C % WIDE == 0 && aligned16(dY) && aligned16(dW) && (!dwpe || aligned16(dwpe));
     const uint32_t CV = wide ? C / WIDE : C;
-    uint32_t block = ((CV + 63) / 64) * 64;
-    if (block > (uint32_t)kRowSumMaxBlock) block = kRowSumMaxBlock;
-    const uint32_t grid = dwpe ? T_len : (N + kRowBatch - 1) / kRowBatch;
+    const uint32_t CB = (CV + kWave - 1) / kWave;               // column blocks: a wave's worth of vectors each
+    const uint64_t units = (uint64_t)(dwpe ? T_len : N) * CB;
+    if (units >= 0xffffff00ull) return set_error(AGRAD_EINVAL, "embedding backward: %u rows of %u columns are too many", N, C);
+    const uint32_t grid = (uint32_t)((units + kRowSumWaves - 1) / kRowSumWaves);
 #define AGRAD_ROW_SUM(VEC, POS) \
-    hipLaunchKernelGGL((emb_row_sum_kernel<T, TO, VEC, POS>), dim3(grid), dim3(block), 0, s, info, row_s, dY, dW, \
-                       dwpe, N, C, CV, V, T_len, B, acc, acc_pos, kMinSlabVectors)
+    hipLaunchKernelGGL((emb_row_sum_kernel<T, TO, VEC, POS>), dim3(grid), dim3(kRowSumBlock), 0, s, order, \
+                       const_cast<uint32_t*>(order) + order_ticket_word(N), dY, dW, dwpe, part, N, C, CV, CB, V, T_len, B, acc, acc_pos)
     if (wide) {
         if (dwpe) AGRAD_ROW_SUM(WIDE, true); else AGRAD_ROW_SUM(WIDE, false);
     } else {
@@ -937,14 +1034,12 @@ int launch_embedding_sort(hipStream_t s, const int32_t* ids, uint32_t* order, vo
     if ((reinterpret_cast<uintptr_t>(order) & 15u) != 0)
         return set_error(AGRAD_EINVAL, "embedding sort: the order buffer must be 16-byte aligned");
     uint8_t* ws = (uint8_t*)workspace;
-    uint32_t* row_s = order;
-    RunInfo* info = reinterpret_cast<RunInfo*>(order + order_info_word(N));
     const uint32_t n = (uint32_t)N;
     if (n <= kGroupSortMaxN && group_sort_enabled()) {
         static_assert(sizeof(unsigned long long) == 2 * sizeof(uint32_t), "spill layout");
         unsigned long long* spill = reinterpret_cast<unsigned long long*>(ws + p.off_keys_in);
         const uint32_t log2G = group_sort_log2g(n);
-        hipLaunchKernelGGL(emb_group_sort_kernel, dim3(1u << log2G), dim3(kSortBlock), 0, s, ids, row_s, info,
+        hipLaunchKernelGGL(emb_group_sort_kernel, dim3(1u << log2G), dim3(kSortBlock), 0, s, ids, order,
                            spill, n, V, log2G, err_flag);
         return check_hip(hipGetLastError(), "embedding sort launch");
     }
@@ -958,10 +1053,10 @@ int launch_embedding_sort(hipStream_t s, const int32_t* ids, uint32_t* order, vo
     while ((1ull << bits) <= V) ++bits;
     size_t temp = p.temp_bytes;
     uint32_t* tok_s = (uint32_t*)(ws + p.off_keys_out);
-    hipError_t err = rocprim::radix_sort_pairs(ws + p.off_temp, temp, keys_in, tok_s, vals_in, row_s,
+    hipError_t err = rocprim::radix_sort_pairs(ws + p.off_temp, temp, keys_in, tok_s, vals_in, order,
                                                (size_t)N, 0u, (unsigned)bits, s, false);
     if (int rc = check_hip(err, "radix sort")) return rc;
-    hipLaunchKernelGGL(emb_run_info_kernel, dim3((n + 255) / 256), dim3(256), 0, s, tok_s, row_s, info, n);
+    hipLaunchKernelGGL(emb_run_info_kernel, dim3((n + 255) / 256), dim3(256), 0, s, tok_s, order, n, V);
     return check_hip(hipGetLastError(), "embedding order launch");
 }
 
@@ -998,34 +1093,38 @@ int launch_gather_fwd_sorted(hipStream_t s, int dtype, const int32_t* ids, const
     const uint32_t grid = (1u << log2G) + (total + kSortBlock - 1) / kSortBlock;
     if ((reinterpret_cast<uintptr_t>(order) & 15u) != 0)
         return set_error(AGRAD_EINVAL, "gather: the order buffer must be 16-byte aligned");
-    uint32_t* row_s = order;
-    RunInfo* info = reinterpret_cast<RunInfo*>(order + order_info_word(N));
     if (wpe == nullptr) {
         hipLaunchKernelGGL((gather_sort_kernel<float, 4, true>), dim3(grid), dim3(kSortBlock), 0, s, ids, (const float*)W,
-                           (const float*)nullptr, (float*)out, total, CV, C, T ? T : 1u, V, row_s, info, spill, n, log2G, err_flag);
+                           (const float*)nullptr, (float*)out, total, CV, C, T ? T : 1u, V, order, spill, n, log2G, err_flag);
     } else if (dtype == AGRAD_F32) {
         hipLaunchKernelGGL((gather_sort_kernel<float, 4, false>), dim3(grid), dim3(kSortBlock), 0, s, ids, (const float*)W,
-                           (const float*)wpe, (float*)out, total, CV, C, T, V, row_s, info, spill, n, log2G, err_flag);
+                           (const float*)wpe, (float*)out, total, CV, C, T, V, order, spill, n, log2G, err_flag);
     } else {
         hipLaunchKernelGGL((gather_sort_kernel<bf16_t, 8, false>), dim3(grid), dim3(kSortBlock), 0, s, ids, (const bf16_t*)W,
-                           (const bf16_t*)wpe, (bf16_t*)out, total, CV, C, T, V, row_s, info, spill, n, log2G, err_flag);
+                           (const bf16_t*)wpe, (bf16_t*)out, total, CV, C, T, V, order, spill, n, log2G, err_flag);
     }
     return check_hip(hipGetLastError(), "gather launch");
 }
 
 uint64_t embedding_bwd_sorted_workspace_bytes(uint64_t N, uint32_t C) {
-    (void)N; (void)C;
-    return 0;       // every table row is summed and stored by one workgroup: nothing is staged
+    if (N == 0 || C == 0) return 0;
+    return align256(partial_rows(N) * C * 4);       // the long runs' partial rows
 }
 
 int launch_embedding_bwd_sorted(hipStream_t s, int dtype, const uint32_t* order, const void* dY, void* dW,
                                 void* dwpe, void* workspace, uint64_t workspace_bytes, uint64_t N, uint32_t T,
                                 uint32_t C, uint32_t V, uint32_t flags) {
-    (void)workspace; (void)workspace_bytes;
     if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "embedding backward: unknown dtype %d", dtype);
     if (N == 0 || C == 0) return AGRAD_OK;
     if (int rc = check_embedding_sizes("embedding backward", N, V)) return rc;
     if (order == nullptr || dY == nullptr || dW == nullptr) return set_error(AGRAD_EINVAL, "embedding backward: null operand");
+    const uint64_t need = embedding_bwd_sorted_workspace_bytes(N, C);
+    if (workspace == nullptr || workspace_bytes < need)
+        return set_error(AGRAD_EWORKSPACE, "embedding backward: workspace %llu < %llu bytes",
+                         (unsigned long long)workspace_bytes, (unsigned long long)need);
+    if ((reinterpret_cast<uintptr_t>(workspace) & 15u) != 0)
+        return set_error(AGRAD_EINVAL, "embedding backward: workspace must be 16-byte aligned");
+    float* part = (float*)workspace;
     if ((reinterpret_cast<uintptr_t>(order) & 15u) != 0)
         return set_error(AGRAD_EINVAL, "embedding backward: the order buffer must be 16-byte aligned");
     uint32_t B = 0;
@@ -1035,11 +1134,11 @@ int launch_embedding_bwd_sorted(hipStream_t s, int dtype, const uint32_t* order,
     }
     if (flags & AGRAD_PARAM_GRAD_BF16) {
         if (dtype != AGRAD_F32) return set_error(AGRAD_EINVAL, "embedding backward: AGRAD_PARAM_GRAD_BF16 goes with an fp32 upstream gradient");
-        return embedding_sum_typed<float, bf16_t>(s, order, (const float*)dY, (bf16_t*)dW, (uint32_t)N, C, V, flags, (bf16_t*)dwpe, B, T);
+        return embedding_sum_typed<float, bf16_t>(s, order, (const float*)dY, (bf16_t*)dW, part, (uint32_t)N, C, V, flags, (bf16_t*)dwpe, B, T);
     }
     if (dtype == AGRAD_F32)
-        return embedding_sum_typed<float>(s, order, (const float*)dY, (float*)dW, (uint32_t)N, C, V, flags, (float*)dwpe, B, T);
-    return embedding_sum_typed<bf16_t>(s, order, (const bf16_t*)dY, (bf16_t*)dW, (uint32_t)N, C, V, flags, (bf16_t*)dwpe, B, T);
+        return embedding_sum_typed<float>(s, order, (const float*)dY, (float*)dW, part, (uint32_t)N, C, V, flags, (float*)dwpe, B, T);
+    return embedding_sum_typed<bf16_t>(s, order, (const bf16_t*)dY, (bf16_t*)dW, part, (uint32_t)N, C, V, flags, (bf16_t*)dwpe, B, T);
 }
 
 int launch_gather_fwd(hipStream_t s, int dtype, const int32_t* ids, const void* W, const void* wpe,
@@ -1082,11 +1181,11 @@ int launch_gather_fwd(hipStream_t s, int dtype, const int32_t* ids, const void* 
     return check_hip(hipGetLastError(), "gather launch");
 }
 
-// one workspace for the unsorted entry point: [order | sort scratch | carry rows]
+// one workspace for the unsorted entry point: [order | sort scratch | partial rows]
 uint64_t embedding_bwd_workspace_bytes(uint64_t N, uint32_t C, uint32_t V, int dtype) {
     (void)dtype;
     if (N == 0 || C == 0) return 0;
-    return order_bytes(N) + embedding_sort_workspace_bytes(N, V);
+    return order_bytes(N) + embedding_sort_workspace_bytes(N, V) + embedding_bwd_sorted_workspace_bytes(N, C);
 }
 
 int launch_embedding_bwd(hipStream_t s, int dtype, const int32_t* ids, const void* dY, void* dW,
@@ -1097,7 +1196,8 @@ int launch_embedding_bwd(hipStream_t s, int dtype, const int32_t* ids, const voi
     if (ids == nullptr || dY == nullptr || dW == nullptr) return set_error(AGRAD_EINVAL, "embedding backward: null operand");
     if (int rc = check_embedding_sizes("embedding backward", N, V)) return rc;
     const uint64_t sort_bytes = embedding_sort_workspace_bytes(N, V);
-    const uint64_t need = order_bytes(N) + sort_bytes;
+    const uint64_t part_bytes = embedding_bwd_sorted_workspace_bytes(N, C);
+    const uint64_t need = order_bytes(N) + sort_bytes + part_bytes;
     if (workspace == nullptr || workspace_bytes < need)
         return set_error(AGRAD_EWORKSPACE, "embedding backward: workspace %llu < %llu bytes",
                          (unsigned long long)workspace_bytes, (unsigned long long)need);
@@ -1106,7 +1206,8 @@ int launch_embedding_bwd(hipStream_t s, int dtype, const int32_t* ids, const voi
     uint8_t* ws = (uint8_t*)workspace;
     uint32_t* order = (uint32_t*)ws;
     if (int rc = launch_embedding_sort(s, ids, order, ws + order_bytes(N), sort_bytes, N, V, err_flag)) return rc;
-    return launch_embedding_bwd_sorted(s, dtype, order, dY, dW, nullptr, nullptr, 0, N, 0, C, V, flags);
+    return launch_embedding_bwd_sorted(s, dtype, order, dY, dW, nullptr, ws + order_bytes(N) + sort_bytes, part_bytes, N, 0,
+                                       C, V, flags);
 }
 
 int launch_pos_embedding_bwd(hipStream_t s, int dtype, const void* dY, void* dwpe, uint32_t B,

@@ -288,8 +288,9 @@ class ContiguousOp(Op):
 
 def _order_output(indices, table):
     """When the table needs a gradient, the embedding ops carry a second,
-    gradient-free output of 5N + 4 uint32: the rows ordered so that each token's rows are
-    adjacent and ascending, and what every row is told about its token's run.  A
+    gradient-free output of 6N + 128 uint32: the rows ordered so that each token's rows are
+    adjacent and ascending, what every row is told about its token's run, and the
+    gradient kernel's arrival counters.  A
     device may fill it in its forward kernel (where ordering the ids is free) and
     start its backward kernel from it; a device that has no use for it leaves it
     alone.  `__call__` still returns the embedding only."""
@@ -298,7 +299,7 @@ def _order_output(indices, table):
     n = 1
     for d in indices.shape:
         n *= d
-    return (Tensor(shape=(5 * n + 4,), dtype=np.uint32, requires_grad=False, device=table.device),)
+    return (Tensor(shape=(6 * n + 128,), dtype=np.uint32, requires_grad=False, device=table.device),)
 
 
 class GatherOp(Op):

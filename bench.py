@@ -161,7 +161,7 @@ def _embed_cases(ctx, cfg, pool, rng, nbytes, ids0):
         # the forward call also orders the ids (one launch: the ordering runs beside the
         # bandwidth-bound gather); the backward call consumes that order.  Same results
         # as agrad_gather_forward + agrad_embedding_backward.
-        order = [pool.raw(4 * (5 * N + 4)) for _ in range(k)]
+        order = [pool.raw(4 * (6 * N + 128)) for _ in range(k)]
         sort_ws_bytes = ctx.lib.agrad_embedding_sort_workspace_bytes(N, cfg.V)
         sort_ws = pool.raw(sort_ws_bytes)
         ws_bytes = ctx.lib.agrad_embedding_backward_sorted_workspace_bytes(N, Cw)

@@ -822,7 +822,7 @@ def test_presorted_embedding_pair_matches_the_plain_pair(ctx, B, T, V, C, dist, 
     d_ids, d_W, d_dY = ctx.upload(ids), ctx.upload(W), ctx.upload(dY)
     d_wpe = ctx.upload(wpe) if wpe is not None else None
     out = ctx.empty((N, C), W.dtype)
-    order = ctx.empty((5 * N + 4,), np.uint32)
+    order = ctx.empty((6 * N + 128,), np.uint32)
     sws_b = ctx.lib.agrad_embedding_sort_workspace_bytes(N, V)
     bws_b = ctx.lib.agrad_embedding_backward_sorted_workspace_bytes(N, C)
     sws, bws = ctx.empty((sws_b,), np.uint8), ctx.empty((bws_b,), np.uint8)
@@ -838,7 +838,7 @@ def test_presorted_embedding_pair_matches_the_plain_pair(ctx, B, T, V, C, dist, 
         np.testing.assert_array_equal(out.download().reshape(B, T, C), want_out)
         np.testing.assert_array_equal(dW.download(), want_dW)
         got = order.download()
-        rows, toks = _check_order(got, N, ids.reshape(-1))
+        rows, toks = _check_order(got, N, ids.reshape(-1), V)
         # each token's rows are adjacent and ascending
         d_tok = np.diff(toks.astype(np.int64))
         assert len(np.unique(toks)) == int((d_tok != 0).sum()) + 1
@@ -851,29 +851,50 @@ def test_presorted_embedding_pair_matches_the_plain_pair(ctx, B, T, V, C, dist, 
             d.free()
 
 
-def _check_order(order, N, tokens):
+def _check_order(order, N, tokens, V):
     """The order buffer of the pre-sorted embedding pair: rows[N] (each token's rows adjacent
-    and ascending), then, from the next multiple of four words, (token, run start, index in
-    the run, run length) for every row.  Returns the rows and their tokens."""
-    rows = order[:N]
-    info = order[(N + 3) // 4 * 4:][:4 * N].reshape(N, 4)
+    and ascending), then, from the next multiple of four words, four words for every row:
+    its token, where its token's run starts, and (R, x): R = 0 for a later row of a run of
+    up to 63 rows and for an id outside the table; the run's length for the first row of
+    such a run, with x = the run's second row (or 0xFFFFFFFF: not given); for a longer run
+    its length and x = the row's index in it.  Then the gradient kernel's arrival counters,
+    all zero.  Returns the rows and their tokens."""
+    rows = order[:N].astype(np.int64)
+    at = (N + 3) // 4 * 4
+    info = order[at:at + 4 * N].reshape(N, 4).astype(np.int64)
+    tickets = order[at + 4 * N:at + 4 * N + (N // 64 + 1) * 32 + (N // 1024 + 1) * 32]
+    assert not tickets.any()
     np.testing.assert_array_equal(np.sort(rows), np.arange(N))
-    toks = tokens[rows]
-    tok, start, j, R = (info[rows, k].astype(np.int64) for k in range(4))
+    toks = tokens[rows].astype(np.int64)
+    run = np.bincount(tokens, minlength=int(tokens.max()) + 1)[toks]
+    change = np.flatnonzero(np.diff(toks) != 0) + 1
+    starts = np.concatenate([[0], change])
+    start = np.repeat(starts, np.diff(np.concatenate([starts, [N]])))
+    j = np.arange(N) - start
+    tok, got_start, R, x = (info[rows, k] for k in range(4))
     np.testing.assert_array_equal(tok, toks)
-    np.testing.assert_array_equal(start + j, np.arange(N))          # every row knows where it stands
-    np.testing.assert_array_equal(R, np.bincount(tokens, minlength=int(tokens.max()) + 1)[toks])
-    assert (j < R).all()
+    np.testing.assert_array_equal(got_start, start)
+    valid = toks < V
+    short = valid & (run <= 63)
+    np.testing.assert_array_equal(R[~valid], 0)
+    np.testing.assert_array_equal(R[short], np.where(j == 0, run, 0)[short])
+    second = short & (j == 0) & (run >= 2)
+    given = second & (x != 0xFFFFFFFF)
+    np.testing.assert_array_equal(x[given], rows[np.flatnonzero(given) + 1])
+    np.testing.assert_array_equal(x[short & (j == 0) & (run == 1)], 0xFFFFFFFF)
+    np.testing.assert_array_equal(R[valid & ~short], run[valid & ~short])
+    np.testing.assert_array_equal(x[valid & ~short], j[valid & ~short])
     return rows, toks
 
 
 def _same_group_tokens(V, how_many, N):
-    """tokens below V that the grouping sort hands to one workgroup (its hash:
-    the top log2g bits of token * 0x9E3779B1 mod 2^32; 128, 256 or 512 groups
-    by the number of rows)"""
-    log2g = 9 if N > 32768 else 8 if N > 16384 else 7
+    """tokens below V that the grouping sort hands to one workgroup (its hash: the log2g
+    bits below bit 24 of (token mod 2^24) * 0x9E3779; 128, 256 or 512 groups by the number
+    of rows)"""
+    log2g = 9 if N > 32768 else 8 if N > 16384 else 7 if N > 1024 else 4
     toks = np.arange(V, dtype=np.uint64)
-    group = ((toks * np.uint64(0x9E3779B1)) & np.uint64(0xFFFFFFFF)) >> np.uint64(32 - log2g)
+    prod = ((toks & np.uint64(0xFFFFFF)) * np.uint64(0x9E3779)) & np.uint64(0xFFFFFFFF)
+    group = (prod >> np.uint64(24 - log2g)) & np.uint64((1 << log2g) - 1)
     best = np.bincount(group.astype(np.int64)).argmax()
     found = toks[group == best][:how_many].astype(np.int32)
     assert len(found) == how_many
@@ -928,7 +949,7 @@ def test_id_ordering_with_frequent_tokens(ctx, case):
         return Ct.c_void_p(d.ptr)
     d_ids, d_W, d_dY = ctx.upload(ids), ctx.upload(W), ctx.upload(dY)
     out = ctx.empty((N, C), np.float32)
-    order = ctx.empty((5 * N + 4,), np.uint32)
+    order = ctx.empty((6 * N + 128,), np.uint32)
     sws_b = ctx.lib.agrad_embedding_sort_workspace_bytes(N, V)
     bws_b = ctx.lib.agrad_embedding_backward_sorted_workspace_bytes(N, C)
     sws, bws = ctx.empty((sws_b,), np.uint8), ctx.empty((bws_b,), np.uint8)
@@ -945,7 +966,7 @@ def test_id_ordering_with_frequent_tokens(ctx, case):
                 ctx.synchronize()
         ctx.synchronize()
         got = order.download()
-        rows, toks = _check_order(got, N, np.where(valid, ids, V))
+        rows, toks = _check_order(got, N, np.where(valid, ids, V), V)
         d_tok = np.diff(toks.astype(np.int64))
         assert len(np.unique(toks)) == int((d_tok != 0).sum()) + 1
         assert (np.diff(rows.astype(np.int64))[d_tok == 0] > 0).all()
@@ -1008,7 +1029,7 @@ def test_embedding_gradient_stored_as_bf16_under_an_fp32_upstream(ctx, B, T, V, 
     # pre-sorted pair with the position table in the same launch
     d_W = ctx.upload(np.zeros((V, C), np.float32))
     out = ctx.empty((N, C), np.float32)
-    order = ctx.empty((5 * N + 4,), np.uint32)
+    order = ctx.empty((6 * N + 128,), np.uint32)
     sws_b = ctx.lib.agrad_embedding_sort_workspace_bytes(N, V)
     bws_b = ctx.lib.agrad_embedding_backward_sorted_workspace_bytes(N, C)
     sws, bws = ctx.empty((sws_b,), np.uint8), ctx.empty((bws_b,), np.uint8)
