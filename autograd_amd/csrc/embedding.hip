@@ -13,10 +13,11 @@
 //      needs).  Larger inputs take a stable LSD radix sort by token (rocPRIM);
 //   2. one launch walks dY in row order: the first row of a token's run adds the
 //      run's rows in ascending order and stores the table row; a long run (a
-//      frequent token) is shared out by column slab among its first rows'
-//      workgroups.  Every table row is written once, by one workgroup.
+//      frequent token) is cut into chunks of rows whose sums pass through the
+//      workspace and are added in chunk order by the wave that an arrival counter
+//      names the last of its group.  Every table row is written once.
 // Every sum has a fixed order, so the result is run-to-run identical, and runs of
-// up to 16 rows are bit-identical to the sequential CPU sum.
+// up to 127 rows are bit-identical to the sequential CPU sum.
 #include "common.hpp"
 #include "launch.hpp"
 
@@ -224,8 +225,8 @@ __device__ __forceinline__ void bitonic_sort_u64(unsigned long long* keys, uint3
 // `start` is the place in row_s[] where the run begins.
 struct __attribute__((aligned(16))) RunInfo { uint32_t tok, start, R, x; };
 
-constexpr uint32_t kSoloRun = 63;        // longest run its first row adds up alone, in np.add.at's order
-constexpr uint32_t kChunkRows = 32;      // a longer run is cut into chunks of this many rows (the last takes the rest)
+constexpr uint32_t kChunkRows = 64;      // a long run is cut into chunks of this many rows (the last takes the rest)
+constexpr uint32_t kSoloRun = 2 * kChunkRows - 1;   // longest run its first row adds up alone, in np.add.at's order
 constexpr uint32_t kGroupChunks = 16;    // ... whose partial rows are added in groups of this many (the last takes the rest)
 constexpr uint32_t kTicketFold = 32;     // arrival counters per chunk group: column block kb counts on kb % kTicketFold
 constexpr uint32_t kNoRow = 0xFFFFFFFFu;
@@ -287,12 +288,6 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
     auto lanes_below = [&](unsigned long long mask) {     // set bits of `mask` below this lane
         return (uint32_t)__builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
     };
-#ifdef AGRAD_SORT_TIMING
-#define STAMP(k) if (tid == 0) spill[g * 8 + (k)] = wall_clock64();
-#else
-#define STAMP(k)
-#endif
-    STAMP(0)
     if (tid == 0) { s_count = 0; s_less = 0; s_rest = 0; s_below = 0; }
     tally[tid] = 0;                     // kRankSortMax == kSortBlock
     {   // this group's share of the gradient kernel's arrival counters
@@ -303,20 +298,27 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
     }
     __syncthreads();
 
-    STAMP(1)
     uint32_t less = 0, worst = 0;                   // `worst`: the largest id seen, as unsigned (a negative id is huge)
-    constexpr int ROUND = 16;                       // id loads in flight per thread
-    constexpr int AGG = 8;
+    // A thread reads four consecutive ids with one 16-byte load and keeps kScanLoads of
+    // them in flight: one round covers 8192 rows.
+    constexpr int kScanLoads = 4, ROUND = 4 * kScanLoads, AGG = 8;
+    const bool wide_ids = (reinterpret_cast<uintptr_t>(ids) & 15u) == 0;
     for (uint32_t base = 0; base < N; base += kSortBlock * ROUND) {
         const bool whole = base + kSortBlock * ROUND <= N;          // no row of this round lies beyond N
         uint32_t t[ROUND];
+        auto row_of = [&](int r) { return base + ((uint32_t)(r >> 2) * kSortBlock + tid) * 4u + (uint32_t)(r & 3); };
+        if (whole && wide_ids) {
 #pragma unroll
-        for (int r = 0; r < ROUND; ++r) {
-            const uint32_t i = base + r * kSortBlock + tid;
-            t[r] = (whole || i < N) ? (uint32_t)ids[i] : 0u;
+            for (int r = 0; r < ROUND; r += 4) {
+                const u32x4 q = *reinterpret_cast<const u32x4*>(ids + row_of(r));
+                t[r] = q.x; t[r + 1] = q.y; t[r + 2] = q.z; t[r + 3] = q.w;
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < ROUND; ++r) t[r] = row_of(r) < N ? (uint32_t)ids[row_of(r)] : 0u;
         }
         // The pairs this group owns go into the list.  One LDS atomic per wave and
-        // eight loads, not one per pair: a frequent token would otherwise queue
+        // eight ids, not one per pair: a frequent token would otherwise queue
         // thousands of them on one address, and waiting for each one's return
         // value in turn costs the usual case a microsecond.
 #pragma unroll
@@ -325,13 +327,12 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
             uint32_t wave_total = 0;
 #pragma unroll
             for (int a = 0; a < AGG; ++a) {
-                const uint32_t i = base + (r0 + a) * kSortBlock + tid;
-                const bool live = whole || i < N;
+                const bool live = whole || row_of(r0 + a) < N;
                 worst = t[r0 + a] > worst ? t[r0 + a] : worst;
                 const uint32_t tok = t[r0 + a] < V ? t[r0 + a] : V;
                 const uint32_t owner = token_group(tok, log2G);
                 less += (live && owner < g) ? 1u : 0u;
-                owners[a] = __ballot(live && owner == g);
+                owners[a] = __builtin_amdgcn_ballot_w64(live && owner == g);
                 wave_total += (uint32_t)__popcll(owners[a]);
             }
             if (wave_total) {
@@ -341,18 +342,16 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
 #pragma unroll
                 for (int a = 0; a < AGG; ++a) {
                     if (owners[a] == 0) continue;
-                    const uint32_t i = base + (r0 + a) * kSortBlock + tid;
                     const uint32_t slot = first + lanes_below(owners[a]);
                     if (((owners[a] >> lane) & 1ull) && slot < kSortLdsEntries) {
                         const uint32_t tok = t[r0 + a] < V ? t[r0 + a] : V;
-                        keys[slot] = ((unsigned long long)tok << 32) | i;
+                        keys[slot] = ((unsigned long long)tok << 32) | row_of(r0 + a);
                     }
                     first += (uint32_t)__popcll(owners[a]);
                 }
             }
         }
     }
-    STAMP(2)
     if (g == 0 && worst >= V) *err_flag = 1;
     // rows owned by lower groups: exact integer wave totals, added in LDS
     {
@@ -368,17 +367,14 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
     __syncthreads();
     const uint32_t count = s_count;
     const uint32_t offset = s_less;
-    STAMP(3)
 
     if (count <= kRankSortMax) {
         // Every key is unique, so its place in the order is the number of smaller keys.
         // The threads share the counting: `parts` threads per key, each comparing the key
         // with its slice of the list (broadcast LDS reads), their tallies added in LDS.
-        uint32_t span = 1;                       // count rounded up to a power of two
-        while (span < count) span <<= 1;
-        const uint32_t parts = kSortBlock / span;
-        const uint32_t k = tid & (span - 1), part = tid / span;
-        const uint32_t j_lo = (part * count) / parts, j_hi = ((part + 1) * count) / parts;
+        const uint32_t parts = count ? kSortBlock / count : 1u;     // threads per key
+        const uint32_t part = count ? tid / count : 0u, k = part < parts ? tid - part * count : count;
+        const uint32_t j_lo = (part * count) / parts, j_hi = k < count ? ((part + 1) * count) / parts : j_lo;
         const unsigned long long mine = k < count ? keys[k] : ~0ull;
         const uint32_t my_tok = (uint32_t)(mine >> 32), my_row = (uint32_t)mine;
         uint32_t smaller_tok = 0, same = 0, same_before = 0;
@@ -401,12 +397,10 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
             placed[rank] = (uint32_t)keys[tid];
         }
         __syncthreads();
-        STAMP(4)
         if (tid < count) {
             const uint32_t next = j + 1 < run ? placed[rank + 1] : kNoRow;
             emit((uint32_t)(keys[tid] >> 32), (uint32_t)keys[tid], offset + rank, j, run, next);
         }
-        STAMP(5)
         return;
     }
 
@@ -594,6 +588,8 @@ emb_group_sort_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ or
 // rows are added in fp32.  Held to 80 scalar registers: compiled to 86 or more
 // (the ordering code's appetite, the gather needs a dozen) the gather ran 5 %
 // slower -- 38.2 against 36.2 us at 16384 x 1536 fp32.
+constexpr int kGatherPerThread = 2;
+
 template <typename T, int VEC, bool RAW>
 __global__ void __launch_bounds__(kSortBlock) __attribute__((amdgpu_num_sgpr(80)))
 gather_sort_kernel(const int32_t* __restrict__ ids, const T* __restrict__ W, const T* __restrict__ wpe,
@@ -605,22 +601,44 @@ gather_sort_kernel(const int32_t* __restrict__ ids, const T* __restrict__ W, con
         emb_group_sort_body(blockIdx.x, ids, order, spill, N, V, log2G, err_flag);
         return;
     }
-    const uint32_t idx = (blockIdx.x - groups) * kSortBlock + threadIdx.x;
-    if (idx >= total) return;
-    const uint32_t row = idx / CV;
-    const uint32_t cv = idx - row * CV;
-    const int32_t tok = ids[row];
-    if (tok < 0 || (uint32_t)tok >= V) return;      // the ordering workgroups report bad ids
-    if constexpr (RAW) {
-        const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(W) + (uint64_t)tok * CV + cv);
-        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(out) + idx);
-    } else {
-        float v[VEC], p[VEC];
-        VecIO<T, VEC>::load(W + (uint64_t)tok * C + cv * VEC, v);
-        VecIO<T, VEC>::load(wpe + (uint64_t)(row % T_len) * C + cv * VEC, p);
+    // the gather proper: kGatherPerThread vectors per thread, all in flight together (the
+    // ordering code sets this kernel's register and LDS footprint, so fewer waves fit a
+    // CU than in a plain copy: each has to keep more bytes in flight)
+    const uint32_t first = (blockIdx.x - groups) * (kSortBlock * kGatherPerThread) + threadIdx.x;
+    uint32_t row[kGatherPerThread], cv[kGatherPerThread];
+    int32_t tok[kGatherPerThread];
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) v[k] = v[k] + p[k];
-        VecIO<T, VEC>::store(out + (uint64_t)row * C + cv * VEC, v);
+    for (int u = 0; u < kGatherPerThread; ++u) {
+        const uint32_t idx = first + u * kSortBlock;
+        row[u] = idx / CV;
+        cv[u] = idx - row[u] * CV;
+        tok[u] = idx < total ? ids[row[u]] : -1;      // (the ordering workgroups report bad ids)
+    }
+    if constexpr (RAW) {
+        u32x4 v[kGatherPerThread];
+#pragma unroll
+        for (int u = 0; u < kGatherPerThread; ++u)
+            if ((uint32_t)tok[u] < V) v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(W) + (uint64_t)tok[u] * CV + cv[u]);
+#pragma unroll
+        for (int u = 0; u < kGatherPerThread; ++u)
+            if ((uint32_t)tok[u] < V) __builtin_nontemporal_store(v[u], reinterpret_cast<u32x4*>(out) + first + u * kSortBlock);
+    } else {
+        float v[kGatherPerThread][VEC], p[kGatherPerThread][VEC];
+#pragma unroll
+        for (int u = 0; u < kGatherPerThread; ++u) {
+            if ((uint32_t)tok[u] < V) {
+                VecIO<T, VEC>::load(W + (uint64_t)tok[u] * C + cv[u] * VEC, v[u]);
+                VecIO<T, VEC>::load(wpe + (uint64_t)(row[u] % T_len) * C + cv[u] * VEC, p[u]);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kGatherPerThread; ++u) {
+            if ((uint32_t)tok[u] < V) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) v[u][k] = v[u][k] + p[u][k];
+                VecIO<T, VEC>::store(out + (uint64_t)row[u] * C + cv[u] * VEC, v[u]);
+            }
+        }
     }
 }
 
@@ -693,38 +711,53 @@ __device__ __forceinline__ void load_partial(const float* p, float (&v)[VEC]) {
     }
 }
 
-// acc += dY[row_s[p], col ...] for p = from .. to-1, ascending (p is the same in every lane)
-template <typename T, int VEC>
-__device__ __forceinline__ void add_listed_rows(float (&acc)[VEC], const uint32_t* __restrict__ row_s, uint32_t from,
-                                                uint32_t to, const T* __restrict__ dY, uint32_t C, uint32_t col, bool live) {
+// The column vectors of one wave: KW blocks of 64 vectors, block w at columns col[w] (a
+// lane is `live` in a block while its vector lies inside the row).
+template <int KW>
+struct WaveCols {
+    uint32_t col[KW];
+    bool live[KW];
+};
+
+// acc += dY[row_s[p], ...] for p = from .. to-1, ascending (p is the same in every lane)
+template <typename T, int VEC, int KW>
+__device__ __forceinline__ void add_listed_rows(float (&acc)[KW][VEC], const uint32_t* __restrict__ row_s, uint32_t from,
+                                                uint32_t to, const T* __restrict__ dY, uint32_t C, const WaveCols<KW>& wc) {
     typedef RawVec<T, VEC> Raw;
+    constexpr int ROWS = kRowBatch / KW;            // rows in flight: kRowBatch loads per lane
 #pragma nounroll
-    for (uint32_t p = from; p < to; p += kRowBatch) {
-        uint32_t rr[kRowBatch];
-        typename Raw::type v[kRowBatch];
+    for (uint32_t p = from; p < to; p += ROWS) {
+        uint32_t rr[ROWS];
+        typename Raw::type v[ROWS][KW];
 #pragma unroll
-        for (int q = 0; q < kRowBatch; ++q) rr[q] = p + q < to ? row_s[p + q] : 0u;
+        for (int q = 0; q < ROWS; ++q) rr[q] = p + q < to ? row_s[p + q] : 0u;
 #pragma unroll
-        for (int q = 0; q < kRowBatch; ++q) {
-            v[q] = Raw::zero();
-            if (p + q < to && live) v[q] = Raw::load(dY + (uint64_t)rr[q] * C + col);
+        for (int q = 0; q < ROWS; ++q) {
+#pragma unroll
+            for (int w = 0; w < KW; ++w) {
+                v[q][w] = Raw::zero();
+                if (p + q < to && wc.live[w]) v[q][w] = Raw::load(dY + (uint64_t)rr[q] * C + wc.col[w]);
+            }
         }
 #pragma unroll
-        for (int q = 0; q < kRowBatch; ++q) {
+        for (int q = 0; q < ROWS; ++q) {
             if (p + q < to) {
-                float x[VEC];
-                Raw::unpack(v[q], x);
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + x[k];
+                for (int w = 0; w < KW; ++w) {
+                    float x[VEC];
+                    Raw::unpack(v[q][w], x);
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) acc[w][k] = acc[w][k] + x[k];
+                }
             }
         }
     }
 }
 
-// sum = slots[first], slots[first + step], ... (n of them), added in that order; the
+// sum = slots[first], slots[first + 1], ... (n of them), added in that order; the
 // partial rows were written by other waves of this launch
 template <int VEC>
-__device__ __forceinline__ void add_partial_rows(float (&sum)[VEC], const float* slots, uint64_t first, uint64_t step,
+__device__ __forceinline__ void add_partial_rows(float (&sum)[VEC], const float* slots, uint64_t first,
                                                  uint32_t n, uint32_t C, uint32_t col, bool live) {
     constexpr int BATCH = VEC >= 8 ? 4 : 8;         // partial rows in flight
 #pragma unroll
@@ -736,7 +769,7 @@ __device__ __forceinline__ void add_partial_rows(float (&sum)[VEC], const float*
         for (int q = 0; q < BATCH; ++q) {
 #pragma unroll
             for (int k = 0; k < VEC; ++k) v[q][k] = 0.0f;
-            if (i0 + q < n && live) load_partial<VEC>(slots + (first + (uint64_t)(i0 + q) * step) * C + col, v[q]);
+            if (i0 + q < n && live) load_partial<VEC>(slots + (first + i0 + q) * C + col, v[q]);
         }
 #pragma unroll
         for (int q = 0; q < BATCH; ++q) {
@@ -763,95 +796,136 @@ __device__ __forceinline__ bool arrive_last(uint32_t* ticket, uint32_t expected,
     return true;
 }
 
-template <typename T, typename TO, int VEC, bool POS>
+// POS: a wave takes the B rows of one position (one column block); otherwise one row and
+// KW neighbouring column blocks.
+template <typename T, typename TO, int VEC, int KW, bool POS>
 __global__ void __launch_bounds__(kRowSumBlock)
 emb_row_sum_kernel(const uint32_t* __restrict__ order, uint32_t* group_tickets, const T* __restrict__ dY, TO* dW,
-                   TO* dwpe, float* part, uint32_t N, uint32_t C, uint32_t CV, uint32_t CB, uint32_t V, uint32_t T_len, uint32_t B,
-                   int accumulate, int accumulate_pos) {
+                   TO* dwpe, float* part, uint32_t N, uint32_t C, uint32_t CV, uint32_t CB, uint32_t V, uint32_t T_len,
+                   uint32_t B, int accumulate, int accumulate_pos) {
+    static_assert(!POS || KW == 1, "a position's rows go one column block at a time");
     typedef RawVec<T, VEC> Raw;
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const uint32_t unit = (uint32_t)__builtin_amdgcn_readfirstlane((int)(blockIdx.x * kRowSumWaves + threadIdx.x / kWave));
-    const uint32_t units = (POS ? T_len : N) * CB;
-    if (unit >= units) return;
-    const uint32_t first = unit / CB, kb = unit - first * CB;
-    const uint32_t cv = kb * kWave + lane;
-    const bool live = cv < CV;
-    const uint32_t col = cv * VEC;
+    const uint32_t CG = (CB + KW - 1) / KW;                     // groups of KW column blocks in a row
+    if (unit >= (POS ? T_len : N) * CG) return;
+    const uint32_t first = unit / CG, kg = unit - first * CG;
+    WaveCols<KW> wc;
+#pragma unroll
+    for (int w = 0; w < KW; ++w) {
+        const uint32_t cv = (kg * KW + w) * kWave + lane;
+        wc.live[w] = cv < CV;
+        wc.col[w] = cv * VEC;
+    }
     const uint32_t* __restrict__ row_s = order;
     const RunInfo* __restrict__ info = reinterpret_cast<const RunInfo*>(order + order_info_word(N));
     uint32_t* run_tickets = group_tickets + order_group_tickets(N);     // (the counters follow the RunInfo words of `order`)
     float* part2 = part + (uint64_t)(N / kChunkRows + 1) * C;          // the groups' partial rows
 
-    // row `n` of a long run (the wave's column block only)
+    // the columns of wave-unit `g` (this wave's own, or those it adds partial rows for)
+    auto cols_of = [&](uint32_t g) {
+        WaveCols<KW> c;
+#pragma unroll
+        for (int w = 0; w < KW; ++w) {
+            const uint32_t cv = (g * KW + w) * kWave + lane;
+            c.live[w] = cv < CV;
+            c.col[w] = cv * VEC;
+        }
+        return c;
+    };
+
+    // a row of a long run
     auto long_run_row = [&](const RunInfo& ri) {
         const uint32_t R = ri.R, j = ri.x, start = ri.start;
         const uint32_t n1 = R / kChunkRows;                             // chunks (at least 2)
         if (j % kChunkRows != 0 || j / kChunkRows >= n1) return;
         const uint32_t c = j / kChunkRows;
         const uint32_t lo = start + c * kChunkRows, hi = c + 1 == n1 ? start + R : lo + kChunkRows;
-        float acc[VEC];
+        float acc[KW][VEC];
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
-        add_listed_rows<T, VEC>(acc, row_s, lo, hi, dY, C, col, live);
-        if (live) store_partial<VEC>(part + (uint64_t)(lo / kChunkRows) * C + col, acc);
+        for (int w = 0; w < KW; ++w)
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) acc[w][k] = 0.0f;
+        add_listed_rows<T, VEC, KW>(acc, row_s, lo, hi, dY, C, wc);
+#pragma unroll
+        for (int w = 0; w < KW; ++w)
+            if (wc.live[w]) store_partial<VEC>(part + (uint64_t)(lo / kChunkRows) * C + wc.col[w], acc[w]);
         // the group of chunks this one belongs to, and its counter
         const uint32_t n2 = n1 / kGroupChunks ? n1 / kGroupChunks : 1u;   // groups
         const uint32_t q = c / kGroupChunks < n2 ? c / kGroupChunks : n2 - 1;
         const uint32_t c_lo = q * kGroupChunks, c_hi = q + 1 == n2 ? n1 : c_lo + kGroupChunks;
         const uint32_t g_at = start + c_lo * kChunkRows;                  // where the group starts
-        const uint32_t fold = kb % kTicketFold, n_fold = (CB - 1 - fold) / kTicketFold + 1;
+        const uint32_t fold = kg % kTicketFold, n_fold = (CG - 1 - fold) / kTicketFold + 1;
         if (!arrive_last(group_tickets + (g_at / (kChunkRows * 2)) * kTicketFold + fold, (c_hi - c_lo) * n_fold, lane)) return;
-        for (uint32_t kb2 = fold; kb2 < CB; kb2 += kTicketFold) {
-            const uint32_t cv2 = kb2 * kWave + lane, col2 = cv2 * VEC;
-            const bool live2 = cv2 < CV;
-            float sum[VEC];
-            add_partial_rows<VEC>(sum, part, g_at / kChunkRows, 1, c_hi - c_lo, C, col2, live2);
-            if (!live2) continue;
-            if (n2 == 1) store_grad_row<TO, VEC>(dW, (uint64_t)ri.tok * C + col2, sum, accumulate != 0);
-            else store_partial<VEC>(part2 + (uint64_t)(g_at / (kChunkRows * kGroupChunks)) * C + col2, sum);
+        for (uint32_t g2 = fold; g2 < CG; g2 += kTicketFold) {
+            const WaveCols<KW> c2 = cols_of(g2);
+#pragma unroll
+            for (int w = 0; w < KW; ++w) {
+                float sum[VEC];
+                add_partial_rows<VEC>(sum, part, g_at / kChunkRows, c_hi - c_lo, C, c2.col[w], c2.live[w]);
+                if (!c2.live[w]) continue;
+                if (n2 == 1) store_grad_row<TO, VEC>(dW, (uint64_t)ri.tok * C + c2.col[w], sum, accumulate != 0);
+                else store_partial<VEC>(part2 + (uint64_t)(g_at / (kChunkRows * kGroupChunks)) * C + c2.col[w], sum);
+            }
         }
         if (n2 == 1) return;
         if (!arrive_last(run_tickets + (start / (kChunkRows * kGroupChunks * 2)) * kTicketFold + fold, n2, lane)) return;
-        for (uint32_t kb2 = fold; kb2 < CB; kb2 += kTicketFold) {
-            const uint32_t cv2 = kb2 * kWave + lane, col2 = cv2 * VEC;
-            const bool live2 = cv2 < CV;
-            float sum[VEC];
-            // group q' starts at start + q' * 512: its slot is (start + q' * 512) / 512
-            add_partial_rows<VEC>(sum, part2, start / (kChunkRows * kGroupChunks), 1, n2, C, col2, live2);
-            if (live2) store_grad_row<TO, VEC>(dW, (uint64_t)ri.tok * C + col2, sum, accumulate != 0);
+        for (uint32_t g2 = fold; g2 < CG; g2 += kTicketFold) {
+            const WaveCols<KW> c2 = cols_of(g2);
+#pragma unroll
+            for (int w = 0; w < KW; ++w) {
+                float sum[VEC];
+                // group q' starts kChunkRows * kGroupChunks places after group q' - 1: its slot is the next
+                add_partial_rows<VEC>(sum, part2, start / (kChunkRows * kGroupChunks), n2, C, c2.col[w], c2.live[w]);
+                if (c2.live[w]) store_grad_row<TO, VEC>(dW, (uint64_t)ri.tok * C + c2.col[w], sum, accumulate != 0);
+            }
         }
     };
 
-    // the first row of a short run: `own` is its vector, `second` the run's second row's
-    auto short_run_head = [&](const RunInfo& ri, const typename Raw::type& own, const typename Raw::type& second) {
-        float acc[VEC];
-        Raw::unpack(own, acc);
-        if (ri.R >= 2) {
-            float x[VEC];
-            Raw::unpack(second, x);
+    // the first row `n` of a short run
+    auto short_run_head = [&](const RunInfo& ri, uint32_t n) {
+        typename Raw::type own[KW], second[KW];
+        uint32_t r1 = n;
+        if (ri.R >= 2) r1 = ri.x != kNoRow ? ri.x : row_s[ri.start + 1];
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + x[k];
-            if (ri.R > 2) add_listed_rows<T, VEC>(acc, row_s, ri.start + 2, ri.start + ri.R, dY, C, col, live);
+        for (int w = 0; w < KW; ++w) {
+            own[w] = Raw::zero();
+            second[w] = Raw::zero();
+            if (wc.live[w]) {
+                own[w] = Raw::load(dY + (uint64_t)n * C + wc.col[w]);
+                if (ri.R >= 2) second[w] = Raw::load(dY + (uint64_t)r1 * C + wc.col[w]);
+            }
         }
-        if (live) store_grad_row<TO, VEC>(dW, (uint64_t)ri.tok * C + col, acc, accumulate != 0);
-    };
-    auto load_second = [&](const RunInfo& ri) {
-        typename Raw::type second = Raw::zero();
-        if (ri.R >= 2 && ri.R <= kSoloRun) {
-            const uint32_t r1 = ri.x != kNoRow ? ri.x : row_s[ri.start + 1];
-            if (live) second = Raw::load(dY + (uint64_t)r1 * C + col);
+        float acc[KW][VEC];
+#pragma unroll
+        for (int w = 0; w < KW; ++w) {
+            Raw::unpack(own[w], acc[w]);
+            if (ri.R >= 2) {
+                float x[VEC];
+                Raw::unpack(second[w], x);
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) acc[w][k] = acc[w][k] + x[k];
+            }
         }
-        return second;
+        if (ri.R > 2) add_listed_rows<T, VEC, KW>(acc, row_s, ri.start + 2, ri.start + ri.R, dY, C, wc);
+#pragma unroll
+        for (int w = 0; w < KW; ++w)
+            if (wc.live[w]) store_grad_row<TO, VEC>(dW, (uint64_t)ri.tok * C + wc.col[w], acc[w], accumulate != 0);
     };
 
     if constexpr (!POS) {
         const RunInfo ri = info[first];
         if (ri.R == 0) return;
-        if (ri.R > kSoloRun) { long_run_row(ri); return; }
-        typename Raw::type own = Raw::zero();
-        if (live) own = Raw::load(dY + (uint64_t)first * C + col);
-        short_run_head(ri, own, load_second(ri));
+        if (ri.R > kSoloRun) long_run_row(ri);
+        else short_run_head(ri, first);
     } else {
+        // All B rows of one position, a batch at a time.  The loads of a batch are issued
+        // without branches, so that all are in flight together: a lane beyond the row's last
+        // vector reads the last vector, and where a run's second row is not wanted the
+        // load reads row 0 (a cache hit after the first time).
+        const bool live = wc.live[0];
+        const uint32_t col = wc.col[0];
+        const uint32_t col_in = (live ? col : (CV - 1) * VEC);
         float pos_acc[VEC];
 #pragma unroll
         for (int k = 0; k < VEC; ++k) pos_acc[k] = 0.0f;
@@ -861,26 +935,44 @@ emb_row_sum_kernel(const uint32_t* __restrict__ order, uint32_t* group_tickets, 
             typename Raw::type own[kRowBatch], second[kRowBatch];
 #pragma unroll
             for (int i = 0; i < kRowBatch; ++i) {
-                ri[i] = RunInfo{V, 0u, 0u, 0u};
-                own[i] = Raw::zero();
-                if (b0 + i < B) {
-                    const uint32_t n = (b0 + i) * T_len + first;
-                    ri[i] = info[n];
-                    if (live) own[i] = Raw::load(dY + (uint64_t)n * C + col);
-                }
+                ri[i] = info[b0 + i < B ? first + (b0 + i) * T_len : first];
+                if (b0 + i >= B) ri[i].R = 0;
             }
 #pragma unroll
-            for (int i = 0; i < kRowBatch; ++i) second[i] = load_second(ri[i]);
+            for (int i = 0; i < kRowBatch; ++i)
+                own[i] = Raw::load(dY + (b0 + i < B ? (uint64_t)(first + (b0 + i) * T_len) * C : 0ull) + col_in);
 #pragma unroll
             for (int i = 0; i < kRowBatch; ++i) {
-                if (b0 + i >= B) continue;
-                float x[VEC];
-                Raw::unpack(own[i], x);
+                const bool wanted = ri[i].R == 2 && ri[i].x != kNoRow;
+                second[i] = Raw::load(dY + (wanted ? (uint64_t)ri[i].x * C : 0ull) + col_in);
+            }
+            uint32_t later = 0;                 // rows of longer runs: one at a time, below
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) pos_acc[k] = b0 + i == 0 ? x[k] : pos_acc[k] + x[k];
+            for (int i = 0; i < kRowBatch; ++i) {
+                float acc[VEC];
+                Raw::unpack(own[i], acc);
+                if (b0 + i < B) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) pos_acc[k] = b0 + i == 0 ? acc[k] : pos_acc[k] + acc[k];
+                }
                 if (ri[i].R == 0) continue;
-                if (ri[i].R > kSoloRun) long_run_row(ri[i]);
-                else short_run_head(ri[i], own[i], second[i]);
+                if (ri[i].R > 2 || (ri[i].R == 2 && ri[i].x == kNoRow)) { later |= 1u << i; continue; }
+                if (ri[i].R == 2) {
+                    float x[VEC];
+                    Raw::unpack(second[i], x);
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + x[k];
+                }
+                if (live) store_grad_row<TO, VEC>(dW, (uint64_t)ri[i].tok * C + col, acc, accumulate != 0);
+            }
+#pragma nounroll
+            while (later) {
+                const uint32_t i = (uint32_t)__builtin_ctz(later);
+                later &= later - 1u;
+                const uint32_t n = first + (b0 + i) * T_len;
+                const RunInfo r = info[n];
+                if (r.R > kSoloRun) long_run_row(r);
+                else short_run_head(r, n);
             }
         }
         if (live) store_grad_row<TO, VEC>(dwpe, (uint64_t)first * C + col, pos_acc, accumulate_pos != 0);
@@ -934,15 +1026,6 @@ pos_grad_kernel(const T* __restrict__ dY, TO* dwpe, uint32_t B, uint64_t TCV, ui
     store_grad_row<TO, VEC>(dwpe, off, acc, accumulate != 0);
 }
 
-// AGRAD_EMB_GROUP_SORT=0 forces the radix-sort path (for comparison runs)
-bool group_sort_enabled() {
-    static const bool on = [] {
-        const char* e = std::getenv("AGRAD_EMB_GROUP_SORT");
-        return !(e && e[0] == '0');
-    }();
-    return on;
-}
-
 // Scratch of the ordering step: input key / value arrays of the radix path (the
 // grouping sort uses the same bytes as N 64-bit spill slots) and rocPRIM's temp.
 struct SortPlan {
@@ -984,12 +1067,16 @@ int embedding_sum_typed(hipStream_t s, const uint32_t* order, const T* dY, TO* d
     const bool wide = C % WIDE == 0 && aligned16(dY) && aligned16(dW) && (!dwpe || aligned16(dwpe));
     const uint32_t CV = wide ? C / WIDE : C;
     const uint32_t CB = (CV + kWave - 1) / kWave;               // column blocks: a wave's worth of vectors each
+    // (KW = 4 column blocks per wave was measured too: it saves most of the 30 us that starting
+    // half a million waves costs at 65536 x 4096 bf16 and gains 4 % on runs of 4..32 rows, but
+    // a long run's chunks then take four times as long each, and Zipf ids lose 20 %.)
     const uint64_t units = (uint64_t)(dwpe ? T_len : N) * CB;
     if (units >= 0xffffff00ull) return set_error(AGRAD_EINVAL, "embedding backward: %u rows of %u columns are too many", N, C);
     const uint32_t grid = (uint32_t)((units + kRowSumWaves - 1) / kRowSumWaves);
 #define AGRAD_ROW_SUM(VEC, POS) \
-    hipLaunchKernelGGL((emb_row_sum_kernel<T, TO, VEC, POS>), dim3(grid), dim3(kRowSumBlock), 0, s, order, \
-                       const_cast<uint32_t*>(order) + order_ticket_word(N), dY, dW, dwpe, part, N, C, CV, CB, V, T_len, B, acc, acc_pos)
+    hipLaunchKernelGGL((emb_row_sum_kernel<T, TO, VEC, 1, POS>), dim3(grid), dim3(kRowSumBlock), 0, s, order, \
+                       const_cast<uint32_t*>(order) + order_ticket_word(N), dY, dW, dwpe, part, N, C, CV, CB, V, T_len, B, \
+                       acc, acc_pos)
     if (wide) {
         if (dwpe) AGRAD_ROW_SUM(WIDE, true); else AGRAD_ROW_SUM(WIDE, false);
     } else {
@@ -1035,7 +1122,7 @@ int launch_embedding_sort(hipStream_t s, const int32_t* ids, uint32_t* order, vo
         return set_error(AGRAD_EINVAL, "embedding sort: the order buffer must be 16-byte aligned");
     uint8_t* ws = (uint8_t*)workspace;
     const uint32_t n = (uint32_t)N;
-    if (n <= kGroupSortMaxN && group_sort_enabled()) {
+    if (n <= kGroupSortMaxN) {
         static_assert(sizeof(unsigned long long) == 2 * sizeof(uint32_t), "spill layout");
         unsigned long long* spill = reinterpret_cast<unsigned long long*>(ws + p.off_keys_in);
         const uint32_t log2G = group_sort_log2g(n);
@@ -1072,7 +1159,7 @@ int launch_gather_fwd_sorted(hipStream_t s, int dtype, const int32_t* ids, const
     const bool wide = C > 0 && C % per16 == 0 && W != nullptr && out != nullptr && aligned16(W) && aligned16(out) &&
                       (!wpe || aligned16(wpe));
     const uint64_t total_vec = wide ? N * (C / per16) : 0;
-    const bool fused = wide && N <= kGroupSortMaxN && group_sort_enabled() && total_vec < 0xff000000ull &&
+    const bool fused = wide && N <= kGroupSortMaxN && total_vec < 0xff000000ull &&
                        ids != nullptr && (wpe == nullptr || T > 0);
     if (!fused) {
         if (int rc = launch_embedding_sort(s, ids, order, sort_workspace, sort_workspace_bytes, N, V, err_flag)) return rc;
@@ -1090,7 +1177,7 @@ int launch_gather_fwd_sorted(hipStream_t s, int dtype, const int32_t* ids, const
     unsigned long long* spill = reinterpret_cast<unsigned long long*>((uint8_t*)sort_workspace + p.off_keys_in);
     const uint32_t n = (uint32_t)N, CV = C / per16, total = (uint32_t)total_vec;
     const uint32_t log2G = group_sort_log2g(n);
-    const uint32_t grid = (1u << log2G) + (total + kSortBlock - 1) / kSortBlock;
+    const uint32_t grid = (1u << log2G) + (total + kSortBlock * kGatherPerThread - 1) / (kSortBlock * kGatherPerThread);
     if ((reinterpret_cast<uintptr_t>(order) & 15u) != 0)
         return set_error(AGRAD_EINVAL, "gather: the order buffer must be 16-byte aligned");
     if (wpe == nullptr) {

@@ -184,7 +184,7 @@ def _embed_cases(ctx, cfg, pool, rng, nbytes, ids0):
             ctx.call("agrad_fill", dW.ptr, 0, 0, 1, dW.nbytes)
 
         cases.append(Case(name, "fwd", nbytes[name][0], k, fwd, "gather_sort_kernel"))
-        cases.append(Case(name, "bwd", nbytes[name][1], k, bwd, "emb_segment_sum_kernel"))
+        cases.append(Case(name, "bwd", nbytes[name][1], k, bwd, "emb_row_sum_kernel"))
         cases.append(Case(name + "_grad_zero_fill", "aux", cfg.V * Cw * e, 1, zero, "fill16_kernel"))
     return cases
 

@@ -307,11 +307,11 @@ int agrad_gather_forward(agrad_ctx* ctx, int dtype, const int32_t* ids,
 
 /* Embedding gradient dW[ids[n],:] += dY[n,:], deterministic: the rows are ordered
  * so that each token's rows are adjacent and ascending, and one launch then walks dY
- * in row order.  The first row of a token with up to 63 rows adds that token's rows
+ * in row order.  The first row of a token with up to 127 rows adds that token's rows
  * in ascending row order -- the sequence of fp32 adds np.add.at makes
  * (cpu_gather_backward, backend.py:531-538; replaces the float-atomic
  * gather_backward_kernel, metal_ops.metal:406-427).  A token with more rows is cut
- * into chunks of 32 rows, summed in row order each; the chunk sums are added in
+ * into chunks of 64 rows, summed in row order each; the chunk sums are added in
  * chunk order in groups of 16, the groups in group order.  No float atomics; every
  * table row is written once, with the same bits on every run.
  * Without AGRAD_ACC_PARAM_GRAD the touched rows of dW are overwritten (correct on
@@ -330,15 +330,15 @@ int agrad_embedding_backward(agrad_ctx* ctx, int dtype, const int32_t* ids, cons
  * rows adjacent and ascending; then, from the next multiple of four words on, four
  * words for row n = 0..N-1: its token (V for an id outside the table), the place
  * in order[] where its token's run starts, and (R, x): R = 0 for a row with
- * nothing to do (a later row of a run of up to 63 rows, an id outside the table);
- * 1..63 for the first row of such a run, x = the run's second row or 0xFFFFFFFF
+ * nothing to do (a later row of a run of up to 127 rows, an id outside the table);
+ * 1..127 for the first row of such a run, x = the run's second row or 0xFFFFFFFF
  * (not given: it is order[start + 1]); for a longer run its length, x = the row's
  * index in the run.  The words after that are arrival counters of the backward
  * call's long runs: zero after the forward call and after every backward call.
  * sort_workspace (256-byte aligned, agrad_embedding_sort_workspace_bytes(N, V)
  * bytes) is free again when the forward call's work has run; the backward call's
  * workspace (16-byte aligned, agrad_embedding_backward_sorted_workspace_bytes(N, C)
- * bytes) holds the fp32 partial rows of runs longer than 63 rows.  Backward calls
+ * bytes) holds the fp32 partial rows of runs longer than 127 rows.  Backward calls
  * that share one order buffer must not overlap in time.
  * Same results, bit for bit, as agrad_gather_forward + agrad_embedding_backward.
  * (The reference orders nothing: np.add.at, backend.py:531-538, and float

@@ -855,14 +855,14 @@ def _check_order(order, N, tokens, V):
     """The order buffer of the pre-sorted embedding pair: rows[N] (each token's rows adjacent
     and ascending), then, from the next multiple of four words, four words for every row:
     its token, where its token's run starts, and (R, x): R = 0 for a later row of a run of
-    up to 63 rows and for an id outside the table; the run's length for the first row of
+    up to 127 rows and for an id outside the table; the run's length for the first row of
     such a run, with x = the run's second row (or 0xFFFFFFFF: not given); for a longer run
     its length and x = the row's index in it.  Then the gradient kernel's arrival counters,
     all zero.  Returns the rows and their tokens."""
     rows = order[:N].astype(np.int64)
     at = (N + 3) // 4 * 4
     info = order[at:at + 4 * N].reshape(N, 4).astype(np.int64)
-    tickets = order[at + 4 * N:at + 4 * N + (N // 64 + 1) * 32 + (N // 1024 + 1) * 32]
+    tickets = order[at + 4 * N:at + 4 * N + (N // 128 + 1) * 32 + (N // 2048 + 1) * 32]
     assert not tickets.any()
     np.testing.assert_array_equal(np.sort(rows), np.arange(N))
     toks = tokens[rows].astype(np.int64)
@@ -875,7 +875,7 @@ def _check_order(order, N, tokens, V):
     np.testing.assert_array_equal(tok, toks)
     np.testing.assert_array_equal(got_start, start)
     valid = toks < V
-    short = valid & (run <= 63)
+    short = valid & (run <= 127)
     np.testing.assert_array_equal(R[~valid], 0)
     np.testing.assert_array_equal(R[short], np.where(j == 0, run, 0)[short])
     second = short & (j == 0) & (run >= 2)
