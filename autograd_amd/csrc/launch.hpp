@@ -21,7 +21,6 @@ inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 
 inline uint32_t dtype_size(int dtype) { return dtype == AGRAD_BF16 ? 2u : 4u; }
 
 // Upper bound on the number of row-partials the norm backward keeps per column.
-uint32_t norm_bwd_max_blocks();
 
 // memops.hip
 int launch_fill(hipStream_t s, void* dst, uint32_t bits, int itemsize, uint64_t n);

@@ -341,7 +341,8 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
     // requested (as raw bits) before the current row is worked on, so a wave
     // always has a row of loads in flight while it computes.
     typedef RawVec<T, VEC> Raw;
-    typename Raw::type nx[NV], ng[NV];
+    typename Raw::type nx[NV], ng[NV], nr[NV];       // nr: the incoming residual gradient, when there is one
+    const bool has_res = a.dres != nullptr && a.dx != nullptr;
     const uint64_t stride = (uint64_t)gridDim.x * RPB;
     uint64_t row = (uint64_t)blockIdx.x * RPB + sub;
     if (row < a.rows) {
@@ -350,15 +351,18 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
             const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
             nx[i] = on[i] ? Raw::load(a.x + row * C + col) : Raw::zero();
             ng[i] = on[i] ? Raw::load(a.dy + row * C + col) : Raw::zero();
+            nr[i] = on[i] && has_res ? Raw::load(a.dres + row * C + col) : Raw::zero();
         }
     }
     for (; row < a.rows; row += stride) {
         const uint64_t base = row * C;
         float xv[NV][VEC], g[NV][VEC];
+        typename Raw::type rv[NV];
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             Raw::unpack(nx[i], xv[i]);
             Raw::unpack(ng[i], g[i]);
+            rv[i] = nr[i];
         }
         if (row + stride < a.rows) {
             const uint64_t nbase = (row + stride) * C;
@@ -368,6 +372,7 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
                 if (on[i]) {
                     nx[i] = Raw::load(a.x + nbase + col);
                     ng[i] = Raw::load(a.dy + nbase + col);
+                    if (has_res) nr[i] = Raw::load(a.dres + nbase + col);
                 }
             }
         }
@@ -439,9 +444,9 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
                         for (int k = 0; k < VEC; ++k)
                             t[k] = mad<T>(-xv[i][k], c2, g[i][k]) * scale;
                     }
-                    if (a.dres != nullptr) {
+                    if (has_res) {
                         float r[VEC];
-                        VecIO<T, VEC>::load(a.dres + base + col, r);
+                        Raw::unpack(rv[i], r);
 #pragma unroll
                         for (int k = 0; k < VEC; ++k) t[k] = r[k] + t[k];
                     }
@@ -672,13 +677,9 @@ struct NormPlan {
 // Elements of a row a thread may hold.  Forward keeps one array; backward keeps
 // x, dy, gamma, the two column accumulators and the prefetched next row, so it
 // gets fewer -- except bf16, whose prefetched rows stay packed (half the
-// registers).  Measured on MI355X over the benchmark shapes; the environment
-// variables override for sweeps.
+// registers).  Measured on MI355X over the benchmark shapes.
 int norm_max_ept(bool backward, int dtype) {
-    static const int fwd = [] { const char* e = std::getenv("AGRAD_NORM_EPT_FWD"); int v = e ? std::atoi(e) : 0; return v >= 4 && v <= kMaxEPT ? v : 0; }();
-    static const int bwd = [] { const char* e = std::getenv("AGRAD_NORM_EPT_BWD"); int v = e ? std::atoi(e) : 0; return v >= 4 && v <= kMaxEPT ? v : 0; }();
-    if (!backward) return fwd ? fwd : 24;
-    if (bwd) return bwd;
+    if (!backward) return 24;
     return dtype == AGRAD_BF16 ? 24 : 16;
 }
 
@@ -713,8 +714,7 @@ constexpr uint32_t kMaxBwdBlocks = 1024;
 
 uint32_t bwd_blocks(const NormPlan& p, uint64_t rows, uint32_t resident) {
     const uint64_t want = (rows + p.rpb - 1) / p.rpb;
-    uint64_t cap = norm_bwd_max_blocks();
-    if (cap == 0) cap = resident && resident < kMaxBwdBlocks ? resident : kMaxBwdBlocks;
+    const uint64_t cap = resident && resident < kMaxBwdBlocks ? resident : kMaxBwdBlocks;
     return (uint32_t)(want < cap ? (want ? want : 1) : cap);
 }
 
@@ -734,14 +734,8 @@ inline size_t bwd_dyn_lds(const NormPlan& p, uint32_t C) {
     return p.rpb > 1 ? (size_t)(BLOCK / kWave - 1) * C * sizeof(float) : 0;
 }
 
-// request gamma before the row?  (AGRAD_NORM_FWD_EARLY=0/1 overrides, for comparison runs)
-inline bool fwd_params_early(int tpr) {
-    static const int forced = [] {
-        const char* e = std::getenv("AGRAD_NORM_FWD_EARLY");
-        return e ? (e[0] == '0' ? 0 : 1) : -1;
-    }();
-    return forced >= 0 ? forced != 0 : tpr >= kWave;
-}
+// request gamma before the row?
+inline bool fwd_params_early(int tpr) { return tpr >= kWave; }
 
 template <typename T, int VEC, int NV, int TPR>
 void fwd_launch(hipStream_t s, const NormFwdArgs<T>& a, uint32_t grid, bool early) {
@@ -883,15 +877,6 @@ int launch_colsum_finalize(hipStream_t s, const float* pa, const float* pb, uint
         hipLaunchKernelGGL((colsum_finalize_kernel<1>), dim3((C + 7) / 8, 2), dim3(1024), 0, s, pa, pb, P, C,
                            out_a, out_b, accumulate, out_bf16 ? 1 : 0);
     return check_hip(hipGetLastError(), "column-sum finalize launch");
-}
-
-uint32_t norm_bwd_max_blocks() {
-    static const uint32_t value = [] {
-        const char* e = std::getenv("AGRAD_NORM_BWD_BLOCKS");
-        long v = e ? std::atol(e) : 0;
-        return (uint32_t)(v > 0 && v <= 4096 ? v : 0);   // 0: choose from the row count
-    }();
-    return value;
 }
 
 uint64_t norm_bwd_workspace_bytes(uint64_t rows, uint32_t C, int dtype) {

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 from autograd_amd import capi
-from tests.helpers import assert_fp32_close
+from tests.helpers import assert_fp32_close, assert_fp32_parity
 
 GOLDEN = Path(__file__).parent / "golden" / "layer_ops_small.npz"
 
@@ -34,24 +34,28 @@ def test_restatement_reproduces_the_frozen_vectors(vec):
 
 @pytest.mark.gpu
 def test_kernels_reproduce_the_frozen_vectors(ctx, vec):
+    from oracle import closed_form as cf
     from tests import gpu_ops as G
     v = vec
     y, _ = G.norm_forward(ctx, capi.NORM_LAYER, v["x"], v["gamma"], v["beta"], 1e-5)
     assert_fp32_close(y, v["ln_y"], "layernorm y")
     out = G.norm_backward(ctx, capi.NORM_LAYER, v["x"], v["gamma"], v["dy"], 1e-5)
     assert_fp32_close(out["dx"], v["ln_dx"], "layernorm dx")
-    assert_fp32_close(out["dgamma"], v["ln_dgamma"], "layernorm dgamma", atol=6e-6)
-    assert_fp32_close(out["dbeta"], v["ln_dbeta"], "layernorm dbeta", atol=6e-6)
+    _, dg64, db64 = cf.layernorm_grads(v["x"], v["gamma"], v["dy"], 1e-5)
+    assert_fp32_parity(out["dgamma"], v["ln_dgamma"], dg64.reshape(v["ln_dgamma"].shape), "layernorm dgamma")
+    assert_fp32_parity(out["dbeta"], v["ln_dbeta"], db64.reshape(v["ln_dbeta"].shape), "layernorm dbeta")
     y, _ = G.norm_forward(ctx, capi.NORM_RMS, v["x"], v["gamma"], None, 1e-6)
     assert_fp32_close(y, v["rms_y"], "rmsnorm y")
     out = G.norm_backward(ctx, capi.NORM_RMS, v["x"], v["gamma"], v["dy"], 1e-6, want_dbeta=False)
     assert_fp32_close(out["dx"], v["rms_dx"], "rmsnorm dx")
-    assert_fp32_close(out["dgamma"], v["rms_dgamma"], "rmsnorm dgamma", atol=6e-6)
+    assert_fp32_parity(out["dgamma"], v["rms_dgamma"], cf.rmsnorm_grads(v["x"], v["gamma"], v["dy"], 1e-6)[1].reshape(v["rms_dgamma"].shape),
+                       "rmsnorm dgamma")
     y, h = G.norm_forward(ctx, capi.NORM_LAYER, v["x"], v["gamma"], v["beta"], 1e-5, residual=v["res"], want_h=True)
     np.testing.assert_array_equal(h, v["addln_h"])
     assert_fp32_close(y, v["addln_y"], "add+layernorm y")
     assert_fp32_close(G.unary(ctx, "agrad_gelu_forward", v["act_x"]), v["gelu_y"], "gelu y")
-    assert_fp32_close(G.unary_backward(ctx, "agrad_gelu_backward", v["act_x"], v["act_dy"]), v["gelu_dx"], "gelu dx", atol=3e-6)
+    assert_fp32_parity(G.unary_backward(ctx, "agrad_gelu_backward", v["act_x"], v["act_dy"]), v["gelu_dx"],
+                       cf.gelu_grad(v["act_x"]) * v["act_dy"].astype(np.float64), "gelu dx")
     np.testing.assert_array_equal(G.unary(ctx, "agrad_relu2_forward", v["act_x"]), v["relu2_y"])
     np.testing.assert_array_equal(G.unary_backward(ctx, "agrad_relu2_backward", v["act_x"], v["act_dy"]), v["relu2_dx"])
     assert_fp32_close(G.swiglu_forward(ctx, v["gu"]), v["swiglu_h"], "swiglu h")

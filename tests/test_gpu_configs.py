@@ -26,7 +26,7 @@ from autograd_amd.configs import CONFIGS
 from oracle import closed_form as cf
 from oracle import cpu_ops as K
 
-from tests.helpers import assert_bf16_close, assert_fp32_close, from_bf16_bits, to_bf16_bits
+from tests.helpers import assert_bf16_close, assert_fp32_close, assert_fp32_parity, from_bf16_bits, to_bf16_bits
 
 pytestmark = pytest.mark.gpu
 
@@ -251,8 +251,8 @@ def test_activation_full_shape(ctx, cfg):
                     # far tails the CPU form loses bits, so hold both to float64 there
                     core = np.abs(xv) <= 4.5
                     assert_fp32_close(got[core], dx_ref[core], "gelu dx core")
-                    assert_fp32_close(got, dx_ref, "gelu dx", atol=3e-6)
                     ref64 = cf.gelu_grad(xv) * dyv.astype(np.float64)
+                    assert_fp32_parity(got, dx_ref, ref64, "gelu dx")
                     assert (np.abs(got - ref64) <= 1e-6 + 1e-6 * np.abs(ref64)).all()
                 else:
                     d.close_enough(got, dx_ref, f"{cfg.name} {cfg.act} dx block {blk}")
