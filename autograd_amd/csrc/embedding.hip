@@ -232,15 +232,18 @@ constexpr uint32_t kTicketFold = 32;     // arrival counters per chunk group: co
 constexpr uint32_t kNoRow = 0xFFFFFFFFu;
 
 // Layout of the order buffer, in 32-bit words: row_s[N] | (pad to 4) RunInfo[N] | group
-// tickets | run tickets.  The tickets are arrival counters of the gradient kernel's long
+// tickets | run tickets | chunk heads.  The tickets are arrival counters of the gradient kernel's long
 // runs; the ordering step zeroes them and the gradient kernel leaves them zero.
 __host__ __device__ inline uint64_t order_info_word(uint64_t N) { return (N + 3) & ~3ull; }
 __host__ __device__ inline uint64_t order_ticket_word(uint64_t N) { return order_info_word(N) + 4 * N; }
 __host__ __device__ inline uint64_t order_group_tickets(uint64_t N) { return (N / (kChunkRows * 2) + 1) * kTicketFold; }
 __host__ __device__ inline uint64_t order_run_tickets(uint64_t N) { return (N / (kChunkRows * kGroupChunks * 2) + 1) * kTicketFold; }
-__host__ __device__ inline uint64_t order_words(uint64_t N) {
-    return order_ticket_word(N) + order_group_tickets(N) + order_run_tickets(N);
-}
+// ... | chunk heads: for every chunk of a long run, at word (place of the chunk's first row) / kChunkRows,
+// the row that starts it.  Words that hold no chunk keep whatever they held: a reader checks
+// what the row's RunInfo says against the word's index.
+__host__ __device__ inline uint64_t order_task_word(uint64_t N) { return order_ticket_word(N) + order_group_tickets(N) + order_run_tickets(N); }
+__host__ __device__ inline uint64_t order_tasks(uint64_t N) { return N / kChunkRows + 1; }
+__host__ __device__ inline uint64_t order_words(uint64_t N) { return order_task_word(N) + order_tasks(N); }
 
 // smallest index in sorted keys[0..n) whose key is not below `bound`
 __device__ __forceinline__ uint32_t first_not_below(const unsigned long long* keys, uint32_t n, unsigned long long bound) {
@@ -280,7 +283,11 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
         ri.start = at - j;
         if (tok >= V) { ri.R = 0; ri.x = 0; }
         else if (R <= kSoloRun) { ri.R = j == 0 ? R : 0u; ri.x = next; }
-        else { ri.R = R; ri.x = j; }
+        else {
+            ri.R = R;
+            ri.x = j;
+            if (j % kChunkRows == 0 && j / kChunkRows < R / kChunkRows) order[order_task_word(N) + at / kChunkRows] = row;
+        }
         info[row] = ri;
     };
     const uint32_t tid = threadIdx.x;
@@ -809,8 +816,13 @@ emb_row_sum_kernel(const uint32_t* __restrict__ order, uint32_t* group_tickets, 
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const uint32_t unit = (uint32_t)__builtin_amdgcn_readfirstlane((int)(blockIdx.x * kRowSumWaves + threadIdx.x / kWave));
     const uint32_t CG = (CB + KW - 1) / KW;                     // groups of KW column blocks in a row
-    if (unit >= (POS ? T_len : N) * CG) return;
-    const uint32_t first = unit / CG, kg = unit - first * CG;
+    // The chunks of the long runs come first in the grid, so that their sums and the adding
+    // up of those are under way while the rest of the grid walks the rows.
+    const uint32_t chunk_units = (uint32_t)order_tasks(N) * CG;
+    const bool chunk_unit = unit < chunk_units;
+    const uint32_t row_unit = chunk_unit ? unit : unit - chunk_units;
+    if (!chunk_unit && row_unit >= (POS ? T_len : N) * CG) return;
+    const uint32_t first = row_unit / CG, kg = row_unit - first * CG;
     WaveCols<KW> wc;
 #pragma unroll
     for (int w = 0; w < KW; ++w) {
@@ -914,11 +926,19 @@ emb_row_sum_kernel(const uint32_t* __restrict__ order, uint32_t* group_tickets, 
             if (wc.live[w]) store_grad_row<TO, VEC>(dW, (uint64_t)ri.tok * C + wc.col[w], acc[w], accumulate != 0);
     };
 
+    if (chunk_unit) {
+        // `first` is a word of the chunk heads: take the row it names if that row's RunInfo
+        // agrees that it starts the chunk at this place
+        const uint32_t row = order[order_task_word(N) + first];
+        if (row >= N) return;
+        const RunInfo ri = info[row];
+        if (ri.R > kSoloRun && ri.x % kChunkRows == 0 && (ri.start + ri.x) / kChunkRows == first) long_run_row(ri);
+        return;
+    }
     if constexpr (!POS) {
         const RunInfo ri = info[first];
-        if (ri.R == 0) return;
-        if (ri.R > kSoloRun) long_run_row(ri);
-        else short_run_head(ri, first);
+        if (ri.R == 0 || ri.R > kSoloRun) return;            // (a long run's rows are summed by the chunk units)
+        short_run_head(ri, first);
     } else {
         // All B rows of one position, a batch at a time.  The loads of a batch are issued
         // without branches, so that all are in flight together: a lane beyond the row's last
@@ -956,7 +976,7 @@ emb_row_sum_kernel(const uint32_t* __restrict__ order, uint32_t* group_tickets, 
 #pragma unroll
                     for (int k = 0; k < VEC; ++k) pos_acc[k] = b0 + i == 0 ? acc[k] : pos_acc[k] + acc[k];
                 }
-                if (ri[i].R == 0) continue;
+                if (ri[i].R == 0 || ri[i].R > kSoloRun) continue;
                 if (ri[i].R > 2 || (ri[i].R == 2 && ri[i].x == kNoRow)) { later |= 1u << i; continue; }
                 if (ri[i].R == 2) {
                     float x[VEC];
@@ -971,9 +991,7 @@ emb_row_sum_kernel(const uint32_t* __restrict__ order, uint32_t* group_tickets, 
                 const uint32_t i = (uint32_t)__builtin_ctz(later);
                 later &= later - 1u;
                 const uint32_t n = first + (b0 + i) * T_len;
-                const RunInfo r = info[n];
-                if (r.R > kSoloRun) long_run_row(r);
-                else short_run_head(r, n);
+                short_run_head(info[n], n);
             }
         }
         if (live) store_grad_row<TO, VEC>(dwpe, (uint64_t)first * C + col, pos_acc, accumulate_pos != 0);
@@ -1005,7 +1023,11 @@ emb_run_info_kernel(const uint32_t* __restrict__ tok_s, uint32_t* __restrict__ o
     ri.start = start;
     if (tok >= V) { ri.R = 0; ri.x = 0; }
     else if (R <= kSoloRun) { ri.R = j == 0 ? R : 0u; ri.x = j + 1 < R ? row_s[p + 1] : kNoRow; }
-    else { ri.R = R; ri.x = j; }
+    else {
+        ri.R = R;
+        ri.x = j;
+        if (j % kChunkRows == 0 && j / kChunkRows < R / kChunkRows) order[order_task_word(N) + p / kChunkRows] = row_s[p];
+    }
     info[row_s[p]] = ri;
 }
 
@@ -1071,7 +1093,7 @@ int embedding_sum_typed(hipStream_t s, const uint32_t* order, const T* dY, TO* d
     // (KW = 4 column blocks per wave was measured too: it saves most of the 30 us that starting
     // half a million waves costs at 65536 x 4096 bf16 and gains 4 % on runs of 4..32 rows, but
     // a long run's chunks then take four times as long each, and Zipf ids lose 20 %.)
-    const uint64_t units = (uint64_t)(dwpe ? T_len : N) * CB;
+    const uint64_t units = ((uint64_t)(dwpe ? T_len : N) + order_tasks(N)) * CB;
     if (units >= 0xffffff00ull) return set_error(AGRAD_EINVAL, "embedding backward: %u rows of %u columns are too many", N, C);
     const uint32_t grid = (uint32_t)((units + kRowSumWaves - 1) / kRowSumWaves);
 #define AGRAD_ROW_SUM(VEC, POS) \

@@ -341,8 +341,7 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
     // requested (as raw bits) before the current row is worked on, so a wave
     // always has a row of loads in flight while it computes.
     typedef RawVec<T, VEC> Raw;
-    typename Raw::type nx[NV], ng[NV], nr[NV];       // nr: the incoming residual gradient, when there is one
-    const bool has_res = a.dres != nullptr && a.dx != nullptr;
+    typename Raw::type nx[NV], ng[NV];
     const uint64_t stride = (uint64_t)gridDim.x * RPB;
     uint64_t row = (uint64_t)blockIdx.x * RPB + sub;
     if (row < a.rows) {
@@ -351,18 +350,15 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
             const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
             nx[i] = on[i] ? Raw::load(a.x + row * C + col) : Raw::zero();
             ng[i] = on[i] ? Raw::load(a.dy + row * C + col) : Raw::zero();
-            nr[i] = on[i] && has_res ? Raw::load(a.dres + row * C + col) : Raw::zero();
         }
     }
     for (; row < a.rows; row += stride) {
         const uint64_t base = row * C;
         float xv[NV][VEC], g[NV][VEC];
-        typename Raw::type rv[NV];
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             Raw::unpack(nx[i], xv[i]);
             Raw::unpack(ng[i], g[i]);
-            rv[i] = nr[i];
         }
         if (row + stride < a.rows) {
             const uint64_t nbase = (row + stride) * C;
@@ -372,7 +368,6 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
                 if (on[i]) {
                     nx[i] = Raw::load(a.x + nbase + col);
                     ng[i] = Raw::load(a.dy + nbase + col);
-                    if (has_res) nr[i] = Raw::load(a.dres + nbase + col);
                 }
             }
         }
@@ -444,9 +439,11 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
                         for (int k = 0; k < VEC; ++k)
                             t[k] = mad<T>(-xv[i][k], c2, g[i][k]) * scale;
                     }
-                    if (has_res) {
+                    if (a.dres != nullptr) {
+                        // (requesting these with the row, an iteration ahead, was measured: no gain at
+                        // C = 384 ... 1536, and 8 % slower at C = 4096 bf16, where it costs a wave per SIMD)
                         float r[VEC];
-                        Raw::unpack(rv[i], r);
+                        VecIO<T, VEC>::load(a.dres + base + col, r);
 #pragma unroll
                         for (int k = 0; k < VEC; ++k) t[k] = r[k] + t[k];
                     }
