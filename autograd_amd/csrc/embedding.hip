@@ -682,7 +682,8 @@ __device__ __forceinline__ void store_grad_row(T* dW, uint64_t off, const float 
 //   * any other row: nothing to do for the table.
 // dY is read once, every row of dW is written once: no float atomics, no second launch.
 constexpr int kRowBatch = 8;          // rows a wave keeps in flight
-constexpr int kPosBatch = 8;          // ... of one position (16 was measured no faster at 1024 positions x 16 rows x 768 fp32)
+constexpr int kPosWaves = 4;          // most waves that share the rows of one position
+constexpr int kPosRows = 1;           // rows a wave takes in one pass (4, all in flight, was measured 5 % slower)
 constexpr int kRowSumBlock = 256;
 constexpr uint32_t kRowSumWaves = kRowSumBlock / kWave;
 
@@ -807,21 +808,26 @@ __device__ __forceinline__ bool arrive_last(uint32_t* ticket, uint32_t expected,
 // POS: a wave takes the B rows of one position (one column block); otherwise one row and
 // KW neighbouring column blocks.
 template <typename T, typename TO, int VEC, int KW, bool POS>
-__global__ void __launch_bounds__(kRowSumBlock)
+__global__ void __launch_bounds__(POS ? kPosWaves * kWave : kRowSumBlock)
 emb_row_sum_kernel(const uint32_t* __restrict__ order, uint32_t* group_tickets, const T* __restrict__ dY, TO* dW,
                    TO* dwpe, float* part, uint32_t N, uint32_t C, uint32_t CV, uint32_t CB, uint32_t V, uint32_t T_len,
                    uint32_t B, int accumulate, int accumulate_pos) {
     static_assert(!POS || KW == 1, "a position's rows go one column block at a time");
     typedef RawVec<T, VEC> Raw;
     const uint32_t lane = threadIdx.x & (kWave - 1);
-    const uint32_t unit = (uint32_t)__builtin_amdgcn_readfirstlane((int)(blockIdx.x * kRowSumWaves + threadIdx.x / kWave));
+    const uint32_t waves = blockDim.x / kWave;                  // waves of a workgroup
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
     const uint32_t CG = (CB + KW - 1) / KW;                     // groups of KW column blocks in a row
-    // The chunks of the long runs come first in the grid, so that their sums and the adding
-    // up of those are under way while the rest of the grid walks the rows.
+    // The chunks of the long runs come first in the grid (whole workgroups of them), so that
+    // their sums and the adding up of those are under way while the rest of the grid walks
+    // the rows.
     const uint32_t chunk_units = (uint32_t)order_tasks(N) * CG;
-    const bool chunk_unit = unit < chunk_units;
-    const uint32_t row_unit = chunk_unit ? unit : unit - chunk_units;
-    if (!chunk_unit && row_unit >= (POS ? T_len : N) * CG) return;
+    const uint32_t chunk_wgs = (chunk_units + waves - 1) / waves;
+    const bool chunk_unit = blockIdx.x < chunk_wgs;
+    // a wave's unit: a chunk; a row and a column group; with a position table the workgroup
+    // is a position and a column group, and its waves share the position's rows
+    const uint32_t row_unit = chunk_unit ? blockIdx.x * waves + wave : POS ? blockIdx.x - chunk_wgs : (blockIdx.x - chunk_wgs) * waves + wave;
+    if (chunk_unit ? row_unit >= chunk_units : row_unit >= (POS ? T_len : N) * CG) return;
     const uint32_t first = row_unit / CG, kg = row_unit - first * CG;
     WaveCols<KW> wc;
 #pragma unroll
@@ -895,19 +901,15 @@ emb_row_sum_kernel(const uint32_t* __restrict__ order, uint32_t* group_tickets, 
         }
     };
 
-    // the first row `n` of a short run
-    auto short_run_head = [&](const RunInfo& ri, uint32_t n) {
-        typename Raw::type own[KW], second[KW];
+    // the first row `n` of a short run; `own` are its vectors
+    auto short_run_head = [&](const RunInfo& ri, uint32_t n, const typename Raw::type (&own)[KW]) {
+        typename Raw::type second[KW];
         uint32_t r1 = n;
         if (ri.R >= 2) r1 = ri.x != kNoRow ? ri.x : row_s[ri.start + 1];
 #pragma unroll
         for (int w = 0; w < KW; ++w) {
-            own[w] = Raw::zero();
             second[w] = Raw::zero();
-            if (wc.live[w]) {
-                own[w] = Raw::load(dY + (uint64_t)n * C + wc.col[w]);
-                if (ri.R >= 2) second[w] = Raw::load(dY + (uint64_t)r1 * C + wc.col[w]);
-            }
+            if (wc.live[w] && ri.R >= 2) second[w] = Raw::load(dY + (uint64_t)r1 * C + wc.col[w]);
         }
         float acc[KW][VEC];
 #pragma unroll
@@ -935,66 +937,68 @@ emb_row_sum_kernel(const uint32_t* __restrict__ order, uint32_t* group_tickets, 
         if (ri.R > kSoloRun && ri.x % kChunkRows == 0 && (ri.start + ri.x) / kChunkRows == first) long_run_row(ri);
         return;
     }
+    auto load_row = [&](uint32_t n, typename Raw::type (&own)[KW]) {
+#pragma unroll
+        for (int w = 0; w < KW; ++w) {
+            own[w] = Raw::zero();
+            if (wc.live[w]) own[w] = Raw::load(dY + (uint64_t)n * C + wc.col[w]);
+        }
+    };
+
     if constexpr (!POS) {
         const RunInfo ri = info[first];
         if (ri.R == 0 || ri.R > kSoloRun) return;            // (a long run's rows are summed by the chunk units)
-        short_run_head(ri, first);
+        typename Raw::type own[KW];
+        load_row(first, own);
+        short_run_head(ri, first, own);
     } else {
-        // All B rows of one position, a batch at a time.  The loads of a batch are issued
-        // without branches, so that all are in flight together: a lane beyond the row's last
-        // vector reads the last vector, and where a run's second row is not wanted the
-        // load reads row 0 (a cache hit after the first time).
-        const bool live = wc.live[0];
-        const uint32_t col = wc.col[0];
-        const uint32_t col_in = (live ? col : (CV - 1) * VEC);
+        // The workgroup has position `first`; wave w takes the rows b = w, w + waves, ... of the
+        // batch, each like a row of its own, and leaves the row's vector in LDS, where wave 0
+        // adds the batch's vectors in ascending b: dwpe[t, :] (+)= sum_b dY[b, t, :].
+        __shared__ float shared_rows[kPosWaves * kPosRows][kWave * VEC];
+        const uint32_t pass_rows = waves * kPosRows;            // rows of a pass: kPosRows per wave, all in flight
         float pos_acc[VEC];
 #pragma unroll
         for (int k = 0; k < VEC; ++k) pos_acc[k] = 0.0f;
 #pragma nounroll
-        for (uint32_t b0 = 0; b0 < B; b0 += kPosBatch) {
-            RunInfo ri[kPosBatch];
-            typename Raw::type own[kPosBatch], second[kPosBatch];
+        for (uint32_t b0 = 0; b0 < B; b0 += pass_rows) {
+            RunInfo ri[kPosRows];
+            typename Raw::type own[kPosRows][1];
 #pragma unroll
-            for (int i = 0; i < kPosBatch; ++i) {
-                ri[i] = info[b0 + i < B ? first + (b0 + i) * T_len : first];
-                if (b0 + i >= B) ri[i].R = 0;
-            }
-#pragma unroll
-            for (int i = 0; i < kPosBatch; ++i)
-                own[i] = Raw::load(dY + (b0 + i < B ? (uint64_t)(first + (b0 + i) * T_len) * C : 0ull) + col_in);
-#pragma unroll
-            for (int i = 0; i < kPosBatch; ++i) {
-                const bool wanted = ri[i].R == 2 && ri[i].x != kNoRow;
-                second[i] = Raw::load(dY + (wanted ? (uint64_t)ri[i].x * C : 0ull) + col_in);
-            }
-            uint32_t later = 0;                 // rows of longer runs: one at a time, below
-#pragma unroll
-            for (int i = 0; i < kPosBatch; ++i) {
-                float acc[VEC];
-                Raw::unpack(own[i], acc);
-                if (b0 + i < B) {
-#pragma unroll
-                    for (int k = 0; k < VEC; ++k) pos_acc[k] = b0 + i == 0 ? acc[k] : pos_acc[k] + acc[k];
+            for (int j = 0; j < kPosRows; ++j) {
+                const uint32_t b = b0 + j * waves + wave;
+                ri[j] = RunInfo{V, 0u, 0u, 0u};
+                own[j][0] = Raw::zero();
+                if (b < B) {
+                    ri[j] = info[b * T_len + first];
+                    load_row(b * T_len + first, own[j]);
                 }
-                if (ri[i].R == 0 || ri[i].R > kSoloRun) continue;
-                if (ri[i].R > 2 || (ri[i].R == 2 && ri[i].x == kNoRow)) { later |= 1u << i; continue; }
-                if (ri[i].R == 2) {
+            }
+#pragma unroll
+            for (int j = 0; j < kPosRows; ++j) {
+                const uint32_t b = b0 + j * waves + wave;
+                if (b < B) {
                     float x[VEC];
-                    Raw::unpack(second[i], x);
+                    Raw::unpack(own[j][0], x);
 #pragma unroll
-                    for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + x[k];
+                    for (int k = 0; k < VEC; ++k) shared_rows[j * waves + wave][lane * VEC + k] = x[k];
+                    if (ri[j].R != 0 && ri[j].R <= kSoloRun) short_run_head(ri[j], b * T_len + first, own[j]);
                 }
-                if (live) store_grad_row<TO, VEC>(dW, (uint64_t)ri[i].tok * C + col, acc, accumulate != 0);
             }
-#pragma nounroll
-            while (later) {
-                const uint32_t i = (uint32_t)__builtin_ctz(later);
-                later &= later - 1u;
-                const uint32_t n = first + (b0 + i) * T_len;
-                short_run_head(info[n], n);
+            __syncthreads();
+            if (wave == 0) {
+                const uint32_t rows = B - b0 < pass_rows ? B - b0 : pass_rows;
+                for (uint32_t r = 0; r < rows; ++r) {           // (row b0 + r sits in slot r: r = j * waves + w)
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) {
+                        const float v = shared_rows[r][lane * VEC + k];
+                        pos_acc[k] = b0 + r == 0 ? v : pos_acc[k] + v;
+                    }
+                }
             }
+            __syncthreads();
         }
-        if (live) store_grad_row<TO, VEC>(dwpe, (uint64_t)first * C + col, pos_acc, accumulate_pos != 0);
+        if (wave == 0 && wc.live[0]) store_grad_row<TO, VEC>(dwpe, (uint64_t)first * C + wc.col[0], pos_acc, accumulate_pos != 0);
     }
 }
 
@@ -1093,11 +1097,17 @@ int embedding_sum_typed(hipStream_t s, const uint32_t* order, const T* dY, TO* d
     // (KW = 4 column blocks per wave was measured too: it saves most of the 30 us that starting
     // half a million waves costs at 65536 x 4096 bf16 and gains 4 % on runs of 4..32 rows, but
     // a long run's chunks then take four times as long each, and Zipf ids lose 20 %.)
-    const uint64_t units = ((uint64_t)(dwpe ? T_len : N) + order_tasks(N)) * CB;
-    if (units >= 0xffffff00ull) return set_error(AGRAD_EINVAL, "embedding backward: %u rows of %u columns are too many", N, C);
-    const uint32_t grid = (uint32_t)((units + kRowSumWaves - 1) / kRowSumWaves);
+    // workgroups: the chunks of long runs, packed; then four rows each -- or, with a position
+    // table, one position and column block each, with a wave per row of the batch
+    const uint32_t waves = dwpe ? (B < (uint32_t)kPosWaves ? B : (uint32_t)kPosWaves) : kRowSumWaves;
+    const uint64_t chunk_wgs = (order_tasks(N) * CB + waves - 1) / waves;
+    const uint64_t row_wgs = dwpe ? (uint64_t)T_len * CB : ((uint64_t)N * CB + waves - 1) / waves;
+    if (chunk_wgs + row_wgs >= 0x7fffffffull || (uint64_t)N * CB >= 0xffffff00ull)
+        return set_error(AGRAD_EINVAL, "embedding backward: %u rows of %u columns are too many", N, C);
+    const uint32_t grid = (uint32_t)(chunk_wgs + row_wgs);
+    const uint32_t block = waves * kWave;
 #define AGRAD_ROW_SUM(VEC, POS) \
-    hipLaunchKernelGGL((emb_row_sum_kernel<T, TO, VEC, 1, POS>), dim3(grid), dim3(kRowSumBlock), 0, s, order, \
+    hipLaunchKernelGGL((emb_row_sum_kernel<T, TO, VEC, 1, POS>), dim3(grid), dim3(block), 0, s, order, \
                        const_cast<uint32_t*>(order) + order_ticket_word(N), dY, dW, dwpe, part, N, C, CV, CB, V, T_len, B, \
                        acc, acc_pos)
     if (wide) {
