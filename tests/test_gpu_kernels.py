@@ -673,6 +673,33 @@ def test_embedding_backward_beyond_the_one_launch_ordering(ctx, dist):
         d.free()
 
 
+@pytest.mark.parametrize("N,C,tokens", [(4096, 10240, 1), (2000, 8196, 3), (65536, 8, 1), (40000, 72, 2)])
+def test_embedding_backward_long_runs_wide_rows_and_deep_trees(ctx, N, C, tokens):
+    """Long runs at the corners of their hand-off scheme: rows of more than 32 column blocks
+    (several blocks then share one arrival counter), a scalar-column width, a run long
+    enough for the second level of adding-up (more than 2048 rows), and two such runs side
+    by side.  Against the float64 row loop and the sequential fp32 loop, twice (the
+    counters must be back at zero), and through the accumulate flag."""
+    rng = _rng(33)
+    V = 50
+    ids = rng.integers(0, tokens, size=N, dtype=np.int32).reshape(1, N) * 7 + 3
+    dY = rng.standard_normal((1, N, C), dtype=np.float32)
+    got = G.embedding_backward(ctx, ids, dY, V)
+    rows = np.flatnonzero(np.bincount(ids.ravel(), minlength=V))
+    d64 = np.zeros((V, C))
+    seq = np.zeros((V, C), np.float32)
+    for t in rows:
+        sel = dY[0][ids[0] == t]
+        d64[t] = sel.astype(np.float64).sum(0)
+        seq[t] = np.add.accumulate(sel, axis=0, dtype=np.float32)[-1]          # np.add.at's order
+    assert_fp32_parity(got, seq, d64, f"dW {N}x{C}, {tokens} tokens")
+    assert not np.delete(got, rows, axis=0).any()
+    np.testing.assert_array_equal(got, G.embedding_backward(ctx, ids, dY, V))
+    base = rng.standard_normal((V, C), dtype=np.float32)
+    acc = G.embedding_backward(ctx, ids, dY, V, dW_init=base, flags=capi.ACC_PARAM_GRAD)
+    np.testing.assert_array_equal(acc, base + got)
+
+
 def test_embedding_backward_short_runs_bit_exact(ctx):
     """Runs of up to 127 rows are summed by their first row in ascending row order: the
     same sequence of fp32 adds as np.add.at."""
