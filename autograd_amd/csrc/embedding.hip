@@ -664,26 +664,29 @@ __device__ __forceinline__ void store_grad_row(T* dW, uint64_t off, const float 
 }
 
 // The gradient sum proper, in ROW order, one launch.  A wave takes one row of dY and one
-// block of 64 column vectors (with a position table: the B rows b*T + t of one position t,
-// a batch at a time, whose vectors it also adds in ascending b: dwpe[t, :] (+)= sum_b
-// dY[b, t, :]).  One 16-byte scalar load tells it what the row is (RunInfo):
+// block of 64 column vectors; one 16-byte scalar load tells it what the row is (RunInfo):
 //   * the first row of its token's run when the run has up to kSoloRun rows: it adds the
 //     run's rows in ascending order -- the very sequence of fp32 adds np.add.at makes --
 //     and stores the table row.  Most rows are their token's only row and just move
 //     their vector;
-//   * a row of a LONGER run (a frequent token: padding, "the").  Every kChunkRows-th row
-//     of the run adds up the chunk of rows that starts with it (whole rows, read once,
-//     eight in flight) and leaves the partial row in the workspace.  The wave that
-//     completes a group of kGroupChunks chunks -- it learns that from an arrival counter
-//     -- adds the group's partial rows in chunk order, and the wave that completes the
-//     run's last group adds the groups in order and stores the table row.  Which wave
-//     does the adding varies from run to run, what it adds in which order does not: the
-//     same bits every time.  The counters are zero before and after the call;
 //   * any other row: nothing to do for the table.
+// With a position table a workgroup takes one position t and column block, its waves the
+// rows b*T + t of the batch; besides the above they leave their vectors in LDS, where
+// wave 0 adds them in ascending b: dwpe[t, :] (+)= sum_b dY[b, t, :].
+// LONGER runs (a frequent token: padding, "the") are cut into chunks of kChunkRows rows.
+// The waves at the FRONT of the grid take one chunk each (the order buffer names the row
+// that starts it): a wave adds up its chunk's rows (whole rows, read once, eight in
+// flight) and leaves the partial row in the workspace.  The wave that completes a group of
+// kGroupChunks chunks -- it learns that from an arrival counter -- adds the group's
+// partial rows in chunk order, and the wave that completes the run's last group adds the
+// groups in order and stores the table row.  Which wave does the adding varies from run
+// to run, what it adds in which order does not: the same bits every time.  The counters
+// are zero before and after the call.
 // dY is read once, every row of dW is written once: no float atomics, no second launch.
 constexpr int kRowBatch = 8;          // rows a wave keeps in flight
 constexpr int kPosWaves = 4;          // most waves that share the rows of one position
-constexpr int kPosRows = 1;           // rows a wave takes in one pass (4, all in flight, was measured 5 % slower)
+constexpr int kPosRows = 1;           // rows a wave takes in one pass (4, all in flight, was measured 5 % slower; 16
+                                      // waves of one row each 50 % slower: large workgroups start and end slowly)
 constexpr int kRowSumBlock = 256;
 constexpr uint32_t kRowSumWaves = kRowSumBlock / kWave;
 

@@ -75,11 +75,14 @@ struct NormBwdArgs {
 // agent-scope atomic stores, a 16-ary tree) was measured 3 to 11 us slower per
 // call on MI355X than this second launch, and device-wide fences slower still
 // (each one writes back a whole L2), so the second launch stayed.
+constexpr int kFinalizeCols = 8;     // column vectors of a finalize workgroup (2, in 256-thread workgroups, was measured 1.5-3.5 us slower)
+constexpr int kFinalizeLanes = 128;  // row lanes per column vector
+
 template <int W>   // W = 4: float4 columns, W = 1: scalar columns
-__global__ void __launch_bounds__(1024)
+__global__ void __launch_bounds__(kFinalizeCols * kFinalizeLanes)
 colsum_finalize_kernel(const float* __restrict__ pg, const float* __restrict__ pb, uint32_t P, uint32_t C,
                        float* __restrict__ dgamma, float* __restrict__ dbeta, int accumulate, int out_bf16) {
-    constexpr int COLS = 8, LANES = 128, BATCH = 8;
+    constexpr int COLS = kFinalizeCols, LANES = kFinalizeLanes, BATCH = 8;
     __shared__ float tile[LANES][COLS * W];
     __shared__ float tile2[LANES / 16][COLS * W];
     const float* src = blockIdx.y == 0 ? pg : pb;
@@ -868,10 +871,10 @@ int launch_colsum_finalize(hipStream_t s, const float* pa, const float* pb, uint
     const bool vec4 = C % 4 == 0 && (!out_a || aligned16(out_a)) && (!out_b || aligned16(out_b)) &&
                       (!pa || aligned16(pa)) && (!pb || aligned16(pb));
     if (vec4)
-        hipLaunchKernelGGL((colsum_finalize_kernel<4>), dim3((C / 4 + 7) / 8, 2), dim3(1024), 0, s, pa, pb, P, C,
+        hipLaunchKernelGGL((colsum_finalize_kernel<4>), dim3((C / 4 + kFinalizeCols - 1) / kFinalizeCols, 2), dim3(kFinalizeCols * kFinalizeLanes), 0, s, pa, pb, P, C,
                            out_a, out_b, accumulate, out_bf16 ? 1 : 0);
     else
-        hipLaunchKernelGGL((colsum_finalize_kernel<1>), dim3((C + 7) / 8, 2), dim3(1024), 0, s, pa, pb, P, C,
+        hipLaunchKernelGGL((colsum_finalize_kernel<1>), dim3((C + kFinalizeCols - 1) / kFinalizeCols, 2), dim3(kFinalizeCols * kFinalizeLanes), 0, s, pa, pb, P, C,
                            out_a, out_b, accumulate, out_bf16 ? 1 : 0);
     return check_hip(hipGetLastError(), "column-sum finalize launch");
 }
