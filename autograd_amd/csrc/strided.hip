@@ -15,7 +15,8 @@
 //   * tiles: the unit-stride source dimension is another one (a true transpose):
 //     256-byte-square tiles (64x64 fp32, 128x128 bf16) go through LDS so that both the reads (along the source's
 //     contiguous dimension) and the writes (along the destination's) are
-//     coalesced 16-byte accesses; the other dimensions enumerate tiles.
+//     coalesced 16-byte accesses; the other dimensions enumerate tiles.  2-byte
+//     elements travel through LDS as 32-bit words of two destination neighbours;
 // A source with no unit-stride dimension, or extents that do not divide into
 // vectors, takes the same kernels with one element per access.
 //
@@ -31,6 +32,7 @@ namespace {
 constexpr int kMaxDims = AGRAD_MAX_DIMS;
 constexpr int kRowsBlock = 64;
 constexpr int kTileBlock = 256;
+constexpr uint32_t kXcds = 8;           // accelerator dies of the GPU; workgroups are dealt to them round-robin
 // tile edge in elements: 256 bytes along either contiguous dimension
 template <int ES> struct TileOf { static constexpr int value = 256 / ES; };
 
@@ -112,6 +114,7 @@ strided_rows_kernel(const typename Elem<ES>::type* __restrict__ src, typename El
 // source strides; bstride_dst holds their dense destination strides.
 struct TileGeom {
     uint32_t ni, nj, tiles_i, tiles_j;
+    uint32_t tiles, per_xcd;      // all tiles; tiles per XCD (the grid is 8 * per_xcd workgroups)
     uint64_t si;                  // source stride of I
     uint64_t dj;                  // destination stride of J
     uint64_t bstride_dst[kMaxDims];
@@ -127,7 +130,11 @@ strided_tile_kernel(const typename Elem<ES>::type* __restrict__ src, typename El
     constexpr int kPitch = kTile + (ES == 4 ? 1 : 2);
     __shared__ E tile[kTile][kPitch];
 
-    uint32_t rem = blockIdx.x;
+    // Workgroups go to the eight XCDs in turn, each with an L2 of its own: workgroup b takes
+    // tile (b % 8) * per_xcd + b / 8, so that the tiles one L2 sees one after the other are
+    // neighbours in the destination and their 256-byte pieces of a row leave it together.
+    uint32_t rem = (blockIdx.x % kXcds) * g.per_xcd + blockIdx.x / kXcds;
+    if (rem >= g.tiles) return;
     const uint32_t ti = rem % g.tiles_i; rem /= g.tiles_i;
     const uint32_t tj = rem % g.tiles_j; rem /= g.tiles_j;
     uint64_t src_base = 0, dst_base = 0;
@@ -189,6 +196,82 @@ strided_tile_kernel(const typename Elem<ES>::type* __restrict__ src, typename El
                 if (accumulate) v = add_vec<ES>(__builtin_nontemporal_load(out), v);
                 __builtin_nontemporal_store(v, out);
             }
+        }
+    }
+}
+
+// 2-byte elements, vector path: the same 128 x 128 tile moved as 32-bit WORDS.  A thread
+// reads the same eight columns of two neighbouring source rows i, i + 1 and pairs them up
+// column by column (one byte-permute each), so that a word already holds two elements
+// that are neighbours in the DESTINATION; the tile is stored transposed, word (j, i/2), and
+// phase 2 reads four words (eight elements along I) with one 16-byte LDS access.  Ten LDS
+// accesses per pair of vectors where the element-wise tile takes thirty-two.  Groups of
+// four words are XOR-swizzled with the tile row (j / 8), which spreads both phases over
+// all 64 banks without padding (32 KB a tile).
+__global__ void __launch_bounds__(kTileBlock)
+transpose_pairs16_kernel(const uint16_t* __restrict__ src, uint16_t* dst, Dims d, TileGeom g, int accumulate) {
+    constexpr int kTile = 128, kWords = kTile / 2;          // words along I in a tile row
+    __shared__ __attribute__((aligned(16))) uint32_t tile[kTile][kWords];
+
+    // Workgroups go to the eight XCDs in turn, each with an L2 of its own: workgroup b takes
+    // tile (b % 8) * per_xcd + b / 8, so that the tiles one L2 sees one after the other are
+    // neighbours in the destination and their 256-byte pieces of a row leave it together.
+    uint32_t rem = (blockIdx.x % kXcds) * g.per_xcd + blockIdx.x / kXcds;
+    if (rem >= g.tiles) return;
+    const uint32_t ti = rem % g.tiles_i; rem /= g.tiles_i;
+    const uint32_t tj = rem % g.tiles_j; rem /= g.tiles_j;
+    uint64_t src_base = 0, dst_base = 0;
+#pragma unroll
+    for (int i = kMaxDims - 1; i >= 0; --i) {
+        if (i < (int)d.n) {
+            const uint32_t q = rem / d.size[i];
+            const uint32_t c = rem - q * d.size[i];
+            src_base += (uint64_t)c * d.stride[i];
+            dst_base += (uint64_t)c * g.bstride_dst[i];
+            rem = q;
+        }
+    }
+    const uint32_t i0 = ti * kTile, j0 = tj * kTile;
+    const uint32_t lane = threadIdx.x % 16;                 // which vector of a 128-element row
+    const uint32_t row = threadIdx.x / 16;                  // 16 rows (row pairs) per pass
+
+    // phase 1: rows i, i + 1 of the source, eight columns each
+    u32x4 lo[4], hi[4];
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        const uint32_t i = (pass * 16 + row) * 2, j = lane * 8;
+        lo[pass] = u32x4{0u, 0u, 0u, 0u};
+        hi[pass] = u32x4{0u, 0u, 0u, 0u};
+        if (i0 + i < g.ni && j0 + j < g.nj) {               // (extents are multiples of 8: row i + 1 exists)
+            const uint16_t* p = src + src_base + (uint64_t)(i0 + i) * g.si + (j0 + j);
+            lo[pass] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+            hi[pass] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + g.si));
+        }
+    }
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        const uint32_t ip = pass * 16 + row;                // the row pair: word column of the transposed tile
+        const uint32_t a[4] = {lo[pass].x, lo[pass].y, lo[pass].z, lo[pass].w};
+        const uint32_t b[4] = {hi[pass].x, hi[pass].y, hi[pass].z, hi[pass].w};
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            // element k of row i in the low half, of row i + 1 in the high half
+            const uint32_t word = (k & 1) ? __builtin_amdgcn_perm(b[k / 2], a[k / 2], 0x07060302u)
+                                          : __builtin_amdgcn_perm(b[k / 2], a[k / 2], 0x05040100u);
+            const uint32_t jj = lane * 8 + k;
+            tile[jj][(((ip >> 2) ^ (jj >> 3)) & 15u) * 4u + (ip & 3u)] = word;
+        }
+    }
+    __syncthreads();
+    // phase 2: a destination row j, eight elements along I per thread
+#pragma unroll
+    for (int pass = 0; pass < 8; ++pass) {
+        const uint32_t j = pass * 16 + row, i = lane * 8;
+        if (j0 + j < g.nj && i0 + i < g.ni) {
+            u32x4 v = *reinterpret_cast<const u32x4*>(&tile[j][((lane ^ (j >> 3)) & 15u) * 4u]);
+            u32x4* out = reinterpret_cast<u32x4*>(dst + dst_base + (uint64_t)(j0 + j) * g.dj + (i0 + i));
+            if (accumulate) v = add_vec<2>(__builtin_nontemporal_load(out), v);
+            __builtin_nontemporal_store(v, out);
         }
     }
 }
@@ -261,7 +344,17 @@ int strided_typed(hipStream_t st, const void* src_v, void* dst_v, const Simplifi
                 ++d.n;
             }
             for (int i = d.n; i < kMaxDims; ++i) { d.size[i] = 1; d.stride[i] = 0; g.bstride_dst[i] = 0; }
-            if (blocks > 0x7fffffffull) return set_error(AGRAD_EINVAL, "strided copy: too many tiles");
+            if (blocks > 0x7ffffff0ull) return set_error(AGRAD_EINVAL, "strided copy: too many tiles");
+            g.tiles = (uint32_t)blocks;
+            g.per_xcd = (uint32_t)((blocks + kXcds - 1) / kXcds);
+            blocks = (uint64_t)g.per_xcd * kXcds;
+            if constexpr (ES == 2) {
+                if (vec) {
+                    hipLaunchKernelGGL(transpose_pairs16_kernel, dim3((uint32_t)blocks), dim3(kTileBlock), 0, st,
+                                       src, dst, d, g, acc);
+                    return check_hip(hipGetLastError(), "strided copy launch");
+                }
+            }
             if (vec)
                 hipLaunchKernelGGL((strided_tile_kernel<ES, WIDE>), dim3((uint32_t)blocks), dim3(kTileBlock), 0, st,
                                    src, dst, d, g, acc);
