@@ -218,32 +218,81 @@ __device__ __forceinline__ void bitonic_sort_u64(unsigned long long* keys, uint3
 // What the ordering step tells row n about its token's run, one 16-byte word per row:
 //   R == 0               nothing to do for this row: a later row of a short run, or an id
 //                        outside the table;
-//   1 <= R <= kSoloRun   row n is the FIRST (lowest) row of a run of R rows, which it adds
-//                        up alone; x = the run's second row, or kNoRow when the ordering
-//                        did not have it at hand (then it is row_s[start + 1]);
+//   1 <= R <= kSoloRun   row n is the FIRST (lowest) row of a run of R rows, which one wave adds
+//                        up in ascending order; x = the run's second row, or kNoRow when the
+//                        ordering did not have it at hand (then it is row_s[start + 1]);
 //   R > kSoloRun         row n is row number x of a long run of R rows.
 // `start` is the place in row_s[] where the run begins.
 struct __attribute__((aligned(16))) RunInfo { uint32_t tok, start, R, x; };
 
 constexpr uint32_t kChunkRows = 64;      // a long run is cut into chunks of this many rows (the last takes the rest)
-constexpr uint32_t kSoloRun = 2 * kChunkRows - 1;   // longest run its first row adds up alone, in np.add.at's order
+constexpr uint32_t kSoloRun = 2 * kChunkRows - 1;   // longest run that one wave adds up alone, in np.add.at's order
 constexpr uint32_t kGroupChunks = 16;    // ... whose partial rows are added in groups of this many (the last takes the rest)
 constexpr uint32_t kTicketFold = 32;     // arrival counters per chunk group: column block kb counts on kb % kTicketFold
 constexpr uint32_t kNoRow = 0xFFFFFFFFu;
+// row_s[] holds a row in its low 30 bits.  The top bit marks a TASK of the gradient kernel:
+// the first row of a run of 2 .. kSoloRun rows, or the first row of a chunk of a long run.
+// (A row that is its token's only row is no task: the row itself moves its vector.)  The
+// bit below it marks the tasks of more than kRowRunMax rows: where a row's wave can add up
+// a few rows itself (rows of few column blocks), only these are tasks.
+constexpr uint32_t kTaskFlag = 0x80000000u;
+constexpr uint32_t kBigTaskFlag = 0x40000000u;
+constexpr uint32_t kRowMask = 0x3FFFFFFFu;
+constexpr uint32_t kRowRunMax = 10;      // (the partner and one batch of rows)
+// places of row_s[] that one wave of the gradient kernel searches for tasks: few where every run is a
+// task, so that many waves share them; a wave's worth where only the runs of more than kRowRunMax rows are
+constexpr uint32_t kTaskSpan = 16, kBigTaskSpan = 64;
 
 // Layout of the order buffer, in 32-bit words: row_s[N] | (pad to 4) RunInfo[N] | group
-// tickets | run tickets | chunk heads.  The tickets are arrival counters of the gradient kernel's long
+// tickets | run tickets.  The tickets are arrival counters of the gradient kernel's long
 // runs; the ordering step zeroes them and the gradient kernel leaves them zero.
 __host__ __device__ inline uint64_t order_info_word(uint64_t N) { return (N + 3) & ~3ull; }
 __host__ __device__ inline uint64_t order_ticket_word(uint64_t N) { return order_info_word(N) + 4 * N; }
 __host__ __device__ inline uint64_t order_group_tickets(uint64_t N) { return (N / (kChunkRows * 2) + 1) * kTicketFold; }
 __host__ __device__ inline uint64_t order_run_tickets(uint64_t N) { return (N / (kChunkRows * kGroupChunks * 2) + 1) * kTicketFold; }
-// ... | chunk heads: for every chunk of a long run, at word (place of the chunk's first row) / kChunkRows,
-// the row that starts it.  Words that hold no chunk keep whatever they held: a reader checks
-// what the row's RunInfo says against the word's index.
-__host__ __device__ inline uint64_t order_task_word(uint64_t N) { return order_ticket_word(N) + order_group_tickets(N) + order_run_tickets(N); }
-__host__ __device__ inline uint64_t order_tasks(uint64_t N) { return N / kChunkRows + 1; }
-__host__ __device__ inline uint64_t order_words(uint64_t N) { return order_task_word(N) + order_tasks(N); }
+__host__ __device__ inline uint64_t order_words(uint64_t N) { return order_ticket_word(N) + order_group_tickets(N) + order_run_tickets(N); }
+
+// the task marks of row number j of a run of R rows (of a token inside the table)
+__host__ __device__ inline uint32_t task_marks(uint32_t j, uint32_t R) {
+    if (R <= kSoloRun) return j != 0 || R < 2 ? 0u : R > kRowRunMax ? kTaskFlag | kBigTaskFlag : kTaskFlag;
+    return j % kChunkRows == 0 && j / kChunkRows < R / kChunkRows ? kTaskFlag | kBigTaskFlag : 0u;
+}
+
+// How the gradient kernel's task workgroups (of `waves` waves) share the work: a wave has a
+// span of `span` places of row_s[] and ONE column block, and takes that block of every
+// task that starts in the span.  A workgroup holds `spans` spans x `blocks` column blocks
+// (blocks: a power of two); rows with more column blocks take `sets` workgroups per span.
+struct TaskGrid {
+    uint32_t blocks, spans, sets, wgs;
+    uint32_t cg, cg_magic;      // (the row part) column groups of a row; ceil(2^32 / cg) where that divides exactly, or 0
+};
+// u / g.cg for u below rows x g.cg
+__device__ __forceinline__ uint32_t row_of_unit(uint32_t u, const TaskGrid& g) {
+    return g.cg == 1 ? u : g.cg_magic != 0 ? __umulhi(u, g.cg_magic) : u / g.cg;
+}
+inline TaskGrid task_grid(uint32_t N, uint32_t CB, uint32_t waves, uint32_t span, uint32_t cg) {
+    TaskGrid g;
+    g.cg = cg;
+    // floor(u * ceil(2^32 / cg) / 2^32) = u / cg for u < 2^32 / cg, which holds for every u < N * cg then
+    g.cg_magic = cg > 1 && (uint64_t)N * cg * cg < (1ull << 32) ? (uint32_t)(((1ull << 32) + cg - 1) / cg) : 0u;
+    g.blocks = 1;
+    while (g.blocks < CB && g.blocks * 2 <= waves) g.blocks *= 2;
+    g.spans = waves / g.blocks;
+    g.sets = (CB + g.blocks - 1) / g.blocks;
+    const uint32_t places = g.spans * span;
+    g.wgs = (((N + places - 1) / places) * g.sets + 7u) & ~7u;
+    return g;
+}
+// Workgroups go to the GPU's eight XCDs in turn.  The chunks of a long run start every
+// kChunkRows places, so the workgroups with that work would be every 2nd, 4th or 8th one --
+// a fraction of the XCDs.  Workgroup b therefore takes piece task_piece(b) of the work: b with
+// its low three bits XOR-ed by all its higher three-bit groups, a permutation within every
+// eight consecutive numbers under which any such regular subset lands on all XCDs alike.
+__host__ __device__ inline uint32_t task_piece(uint32_t b) {
+    uint32_t fold = 0;
+    for (uint32_t x = b >> 3; x != 0; x >>= 3) fold ^= x;
+    return b ^ (fold & 7u);
+}
 
 // smallest index in sorted keys[0..n) whose key is not below `bound`
 __device__ __forceinline__ uint32_t first_not_below(const unsigned long long* keys, uint32_t n, unsigned long long bound) {
@@ -277,17 +326,13 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
     RunInfo* __restrict__ info = reinterpret_cast<RunInfo*>(order + order_info_word(N));
     // a pair leaves for the order: its row at place `at`, and what the row is told
     auto emit = [&](uint32_t tok, uint32_t row, uint32_t at, uint32_t j, uint32_t R, uint32_t next) {
-        row_s[at] = row;
         RunInfo ri;
         ri.tok = tok;
         ri.start = at - j;
         if (tok >= V) { ri.R = 0; ri.x = 0; }
         else if (R <= kSoloRun) { ri.R = j == 0 ? R : 0u; ri.x = next; }
-        else {
-            ri.R = R;
-            ri.x = j;
-            if (j % kChunkRows == 0 && j / kChunkRows < R / kChunkRows) order[order_task_word(N) + at / kChunkRows] = row;
-        }
+        else { ri.R = R; ri.x = j; }
+        row_s[at] = tok < V ? row | task_marks(j, R) : row;
         info[row] = ri;
     };
     const uint32_t tid = threadIdx.x;
@@ -663,32 +708,42 @@ __device__ __forceinline__ void store_grad_row(T* dW, uint64_t off, const float 
     VecIO<T, VEC>::store(dW + off, o);
 }
 
-// The gradient sum proper, in ROW order, one launch.  A wave takes one row of dY and one
-// block of 64 column vectors; one 16-byte scalar load tells it what the row is (RunInfo):
-//   * the first row of its token's run when the run has up to kSoloRun rows: it adds the
-//     run's rows in ascending order -- the very sequence of fp32 adds np.add.at makes --
-//     and stores the table row.  Most rows are their token's only row and just move
-//     their vector;
-//   * any other row: nothing to do for the table.
-// With a position table a workgroup takes one position t and column block, its waves the
-// rows b*T + t of the batch; besides the above they leave their vectors in LDS, where
-// wave 0 adds them in ascending b: dwpe[t, :] (+)= sum_b dY[b, t, :].
-// LONGER runs (a frequent token: padding, "the") are cut into chunks of kChunkRows rows.
-// The waves at the FRONT of the grid take one chunk each (the order buffer names the row
-// that starts it): a wave adds up its chunk's rows (whole rows, read once, eight in
-// flight) and leaves the partial row in the workspace.  The wave that completes a group of
-// kGroupChunks chunks -- it learns that from an arrival counter -- adds the group's
-// partial rows in chunk order, and the wave that completes the run's last group adds the
-// groups in order and stores the table row.  Which wave does the adding varies from run
-// to run, what it adds in which order does not: the same bits every time.  The counters
-// are zero before and after the call.
-// dY is read once, every row of dW is written once: no float atomics, no second launch.
+// The gradient sum proper, one launch, no float atomics.  dY is read once and every row of
+// dW is written once.  The grid has two parts.
+//
+// ROWS.  A wave takes one row of dY and KW neighbouring blocks of 64 column vectors (the
+// whole row when it has up to KW blocks); one 16-byte scalar load tells it what the row is
+// (RunInfo).  A row that is its token's only row moves its vectors to the table -- most rows
+// do -- and every other row ends there.  With a position table a workgroup takes one
+// position t and column block, its waves the rows b*T + t of the batch; besides the above
+// they leave their vectors in LDS, where wave 0 adds them in ascending b:
+// dwpe[t, :] (+)= sum_b dY[b, t, :].
+//
+// TASKS, at the FRONT of the grid so that they are under way while the rest walks the rows.
+// A wave searches kTaskSpan places of row_s[] for marked rows and takes ONE column block of
+// every one found (TaskGrid):
+//   * the first row of a run of 2 .. kSoloRun rows: the wave adds the run's rows in
+//     ascending order -- the very sequence of fp32 adds np.add.at makes -- and stores the
+//     table row;
+//   * the first row of a chunk of a LONGER run (a frequent token: padding, "the"), which is
+//     cut into chunks of kChunkRows rows: the wave adds up its chunk's rows (eight in
+//     flight) and leaves the partial row in the workspace.  The wave that completes a group
+//     of kGroupChunks chunks -- it learns that from an arrival counter -- adds the group's
+//     partial rows in chunk order, and the wave that completes the run's last group adds
+//     the groups in order and stores the table row.  Which wave does the adding varies from
+//     call to call, what it adds in which order does not: the same bits every time.  The
+//     counters are zero before and after the call.
+// (One wave per row and column block, runs included, started half a million waves at
+// 65536 rows of 4096 bf16 columns, most of them with nothing to do, behind the waves that
+// had: 30 to 45 us of the call.)
 constexpr int kRowBatch = 8;          // rows a wave keeps in flight
+                                      // (16 for the chunks of long runs take the kernel from 60 to 90 registers: fewer waves
+                                      // per CU, and single rows move 3 to 10 % slower for 4 % on Zipf ids)
 constexpr int kPosWaves = 4;          // most waves that share the rows of one position
-constexpr int kPosRows = 1;           // rows a wave takes in one pass (4, all in flight, was measured 5 % slower; 16
-                                      // waves of one row each 50 % slower: large workgroups start and end slowly)
 constexpr int kRowSumBlock = 256;
 constexpr uint32_t kRowSumWaves = kRowSumBlock / kWave;
+constexpr int kRowBlocksMax = 8;      // most column blocks of a row that one wave moves
+constexpr uint64_t kRowWavesEasy = 131072;
 
 // Partial rows travel between waves of one launch, which may sit on different L2 caches:
 // they are written and read with device-scope accesses (which go past the L2 to where
@@ -723,46 +778,44 @@ __device__ __forceinline__ void load_partial(const float* p, float (&v)[VEC]) {
     }
 }
 
-// The column vectors of one wave: KW blocks of 64 vectors, block w at columns col[w] (a
-// lane is `live` in a block while its vector lies inside the row).
-template <int KW>
-struct WaveCols {
-    uint32_t col[KW];
-    bool live[KW];
-};
-
-// acc += dY[row_s[p], ...] for p = from .. to-1, ascending (p is the same in every lane)
-template <typename T, int VEC, int KW>
-__device__ __forceinline__ void add_listed_rows(float (&acc)[KW][VEC], const uint32_t* __restrict__ row_s, uint32_t from,
-                                                uint32_t to, const T* __restrict__ dY, uint32_t C, const WaveCols<KW>& wc) {
+// acc += dY[r, col ...] for the rows r that lanes 0 .. cnt-1 hold in `mine`, in lane order
+template <typename T, int VEC>
+__device__ __forceinline__ void add_lane_rows(float (&acc)[VEC], uint32_t mine, uint32_t cnt, const T* __restrict__ dY,
+                                              uint32_t C, uint32_t col, bool live) {
     typedef RawVec<T, VEC> Raw;
-    constexpr int ROWS = kRowBatch / KW;            // rows in flight: kRowBatch loads per lane
 #pragma nounroll
-    for (uint32_t p = from; p < to; p += ROWS) {
-        uint32_t rr[ROWS];
-        typename Raw::type v[ROWS][KW];
+    for (uint32_t q0 = 0; q0 < cnt; q0 += kRowBatch) {
+        typename Raw::type v[kRowBatch];
 #pragma unroll
-        for (int q = 0; q < ROWS; ++q) rr[q] = p + q < to ? row_s[p + q] : 0u;
-#pragma unroll
-        for (int q = 0; q < ROWS; ++q) {
-#pragma unroll
-            for (int w = 0; w < KW; ++w) {
-                v[q][w] = Raw::zero();
-                if (p + q < to && wc.live[w]) v[q][w] = Raw::load(dY + (uint64_t)rr[q] * C + wc.col[w]);
-            }
+        for (int q = 0; q < kRowBatch; ++q) {
+            const uint32_t r = (uint32_t)__builtin_amdgcn_readlane((int)mine, (int)(q0 + q));
+            v[q] = Raw::zero();
+            if (q0 + q < cnt && live) v[q] = Raw::load(dY + (uint64_t)r * C + col);
         }
 #pragma unroll
-        for (int q = 0; q < ROWS; ++q) {
-            if (p + q < to) {
+        for (int q = 0; q < kRowBatch; ++q) {
+            if (q0 + q < cnt) {
+                float x[VEC];
+                Raw::unpack(v[q], x);
 #pragma unroll
-                for (int w = 0; w < KW; ++w) {
-                    float x[VEC];
-                    Raw::unpack(v[q][w], x);
-#pragma unroll
-                    for (int k = 0; k < VEC; ++k) acc[w][k] = acc[w][k] + x[k];
-                }
+                for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + x[k];
             }
         }
+    }
+}
+
+// acc += dY[row_s[p], col ...] for p = from .. to-1, ascending (p is the same in every lane).
+// The wave fetches 64 places of row_s[] with one load, a place per lane, and hands the rows
+// round from there.
+template <typename T, int VEC>
+__device__ __forceinline__ void add_listed_rows(float (&acc)[VEC], const uint32_t* __restrict__ row_s, uint32_t from,
+                                                uint32_t to, const T* __restrict__ dY, uint32_t C, uint32_t col, bool live,
+                                                uint32_t lane) {
+#pragma nounroll
+    for (uint32_t base = from; base < to; base += kWave) {
+        const uint32_t cnt = to - base < kWave ? to - base : kWave;
+        const uint32_t mine = lane < cnt ? row_s[base + lane] & kRowMask : 0u;
+        add_lane_rows<T, VEC>(acc, mine, cnt, dY, C, col, live);
     }
 }
 
@@ -808,190 +861,203 @@ __device__ __forceinline__ bool arrive_last(uint32_t* ticket, uint32_t expected,
     return true;
 }
 
-// POS: a wave takes the B rows of one position (one column block); otherwise one row and
-// KW neighbouring column blocks.
+// What the tasks of the gradient kernel work on.
+template <typename T, typename TO>
+struct RowSumArgs {
+    const uint32_t* __restrict__ row_s;
+    uint32_t* group_tickets;
+    uint32_t* run_tickets;
+    const T* __restrict__ dY;
+    TO* dW;
+    float* part;            // a partial row per chunk of a long run ...
+    float* part2;           // ... and per group of chunks
+    uint32_t C, CV, CB;
+    bool accumulate;
+};
+
+// Column block kb of the run of 1 .. kSoloRun rows that row `n` starts.  The row's own vector,
+// its partner's and the list of the rows after those are asked for together: every lane
+// loads from a valid place (a lane outside the row from the row's start), with no branch
+// between the loads for the compiler to put a wait into.
+template <typename T, typename TO, int VEC>
+__device__ __forceinline__ void sum_short_run(const RowSumArgs<T, TO>& a, const RunInfo& ri, uint32_t n, uint32_t kb, uint32_t lane) {
+    typedef RawVec<T, VEC> Raw;
+    const uint32_t cv = kb * kWave + lane, col = cv * VEC;
+    const bool live = cv < a.CV;
+    const uint32_t col_ld = live ? col : 0u;
+    float acc[VEC];
+    if (ri.R == 1) {
+        const typename Raw::type own = Raw::load(a.dY + (uint64_t)n * a.C + col_ld);
+        Raw::unpack(own, acc);
+    } else {
+        const uint32_t rest = ri.R - 2, cnt = rest < kWave ? rest : kWave;
+        uint32_t mine = a.row_s[ri.start + 1 + (lane < cnt ? lane + 1 : 0u)];       // (asked for first: needed first)
+        const uint32_t r1 = ri.x != kNoRow ? ri.x : a.row_s[ri.start + 1] & kRowMask;
+        const typename Raw::type first = Raw::load(a.dY + (uint64_t)n * a.C + col_ld);
+        const typename Raw::type second = Raw::load(a.dY + (uint64_t)r1 * a.C + col_ld);
+        mine &= kRowMask;
+        float x[VEC];
+        Raw::unpack(first, acc);
+        Raw::unpack(second, x);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + x[k];
+        if (cnt != 0) add_lane_rows<T, VEC>(acc, mine, cnt, a.dY, a.C, col, live);
+        if (rest > kWave) add_listed_rows<T, VEC>(acc, a.row_s, ri.start + 2 + kWave, ri.start + ri.R, a.dY, a.C, col, live, lane);
+    }
+    if (live) store_grad_row<TO, VEC>(a.dW, (uint64_t)ri.tok * a.C + col, acc, a.accumulate);
+}
+
+// Column block kb of the chunk of a long run that starts with row number ri.x of the run.
+template <typename T, typename TO, int VEC>
+__device__ __forceinline__ void sum_chunk(const RowSumArgs<T, TO>& a, const RunInfo& ri, uint32_t kb, uint32_t lane) {
+    const uint32_t R = ri.R, start = ri.start, CB = a.CB, C = a.C;
+    const uint32_t n1 = R / kChunkRows;                             // chunks (at least 2)
+    const uint32_t c = ri.x / kChunkRows;
+    const uint32_t lo = start + c * kChunkRows, hi = c + 1 == n1 ? start + R : lo + kChunkRows;
+    auto col_of = [&](uint32_t b) { return (b * kWave + lane) * VEC; };
+    auto live_in = [&](uint32_t b) { return b * kWave + lane < a.CV; };
+    float acc[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
+    add_listed_rows<T, VEC>(acc, a.row_s, lo, hi, a.dY, C, col_of(kb), live_in(kb), lane);
+    if (live_in(kb)) store_partial<VEC>(a.part + (uint64_t)(lo / kChunkRows) * C + col_of(kb), acc);
+    // the group of chunks this one belongs to, and its counter
+    const uint32_t n2 = n1 / kGroupChunks ? n1 / kGroupChunks : 1u;   // groups
+    const uint32_t q = c / kGroupChunks < n2 ? c / kGroupChunks : n2 - 1;
+    const uint32_t c_lo = q * kGroupChunks, c_hi = q + 1 == n2 ? n1 : c_lo + kGroupChunks;
+    const uint32_t g_at = start + c_lo * kChunkRows;                  // where the group starts
+    const uint32_t fold = kb % kTicketFold, n_fold = (CB - 1 - fold) / kTicketFold + 1;
+    if (!arrive_last(a.group_tickets + (g_at / (kChunkRows * 2)) * kTicketFold + fold, (c_hi - c_lo) * n_fold, lane)) return;
+    for (uint32_t b = fold; b < CB; b += kTicketFold) {
+        float sum[VEC];
+        add_partial_rows<VEC>(sum, a.part, g_at / kChunkRows, c_hi - c_lo, C, col_of(b), live_in(b));
+        if (!live_in(b)) continue;
+        if (n2 == 1) store_grad_row<TO, VEC>(a.dW, (uint64_t)ri.tok * C + col_of(b), sum, a.accumulate);
+        else store_partial<VEC>(a.part2 + (uint64_t)(g_at / (kChunkRows * kGroupChunks)) * C + col_of(b), sum);
+    }
+    if (n2 == 1) return;
+    if (!arrive_last(a.run_tickets + (start / (kChunkRows * kGroupChunks * 2)) * kTicketFold + fold, n2, lane)) return;
+    for (uint32_t b = fold; b < CB; b += kTicketFold) {
+        float sum[VEC];
+        // group q' starts kChunkRows * kGroupChunks places after group q' - 1: its slot is the next
+        add_partial_rows<VEC>(sum, a.part2, start / (kChunkRows * kGroupChunks), n2, C, col_of(b), live_in(b));
+        if (live_in(b)) store_grad_row<TO, VEC>(a.dW, (uint64_t)ri.tok * C + col_of(b), sum, a.accumulate);
+    }
+}
+
+// POS: a workgroup takes the B rows of one position (one column block); otherwise a wave
+// takes one row and KW neighbouring column blocks.
 template <typename T, typename TO, int VEC, int KW, bool POS>
 __global__ void __launch_bounds__(POS ? kPosWaves * kWave : kRowSumBlock)
 emb_row_sum_kernel(const uint32_t* __restrict__ order, uint32_t* group_tickets, const T* __restrict__ dY, TO* dW,
                    TO* dwpe, float* part, uint32_t N, uint32_t C, uint32_t CV, uint32_t CB, uint32_t V, uint32_t T_len,
-                   uint32_t B, int accumulate, int accumulate_pos) {
+                   uint32_t B, int accumulate, int accumulate_pos, TaskGrid tg) {
     static_assert(!POS || KW == 1, "a position's rows go one column block at a time");
     typedef RawVec<T, VEC> Raw;
     const uint32_t lane = threadIdx.x & (kWave - 1);
-    const uint32_t waves = blockDim.x / kWave;                  // waves of a workgroup
+    const uint32_t waves = POS ? blockDim.x / kWave : kRowSumWaves;     // waves of a workgroup
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x / kWave));
-    const uint32_t CG = (CB + KW - 1) / KW;                     // groups of KW column blocks in a row
-    // The chunks of the long runs come first in the grid (whole workgroups of them), so that
-    // their sums and the adding up of those are under way while the rest of the grid walks
-    // the rows.
-    const uint32_t chunk_units = (uint32_t)order_tasks(N) * CG;
-    const uint32_t chunk_wgs = (chunk_units + waves - 1) / waves;
-    const bool chunk_unit = blockIdx.x < chunk_wgs;
-    // a wave's unit: a chunk; a row and a column group; with a position table the workgroup
-    // is a position and a column group, and its waves share the position's rows
-    const uint32_t row_unit = chunk_unit ? blockIdx.x * waves + wave : POS ? blockIdx.x - chunk_wgs : (blockIdx.x - chunk_wgs) * waves + wave;
-    if (chunk_unit ? row_unit >= chunk_units : row_unit >= (POS ? T_len : N) * CG) return;
-    const uint32_t first = row_unit / CG, kg = row_unit - first * CG;
-    WaveCols<KW> wc;
-#pragma unroll
-    for (int w = 0; w < KW; ++w) {
-        const uint32_t cv = (kg * KW + w) * kWave + lane;
-        wc.live[w] = cv < CV;
-        wc.col[w] = cv * VEC;
-    }
     const uint32_t* __restrict__ row_s = order;
     const RunInfo* __restrict__ info = reinterpret_cast<const RunInfo*>(order + order_info_word(N));
-    uint32_t* run_tickets = group_tickets + order_group_tickets(N);     // (the counters follow the RunInfo words of `order`)
-    float* part2 = part + (uint64_t)(N / kChunkRows + 1) * C;          // the groups' partial rows
+    constexpr uint32_t kSpan = KW == 1 ? kBigTaskSpan : kTaskSpan;       // (tg: the host's task_grid() for this span)
+    const uint32_t task_wgs = tg.wgs;
+    RowSumArgs<T, TO> a;
+    a.row_s = row_s;
+    a.group_tickets = group_tickets;
+    a.run_tickets = group_tickets + order_group_tickets(N);     // (the counters follow the RunInfo words of `order`)
+    a.dY = dY;
+    a.dW = dW;
+    a.part = part;
+    a.part2 = part + (uint64_t)(N / kChunkRows + 1) * C;
+    a.C = C; a.CV = CV; a.CB = CB;
+    a.accumulate = accumulate != 0;
+    // runs that a row wave adds up itself when it takes one column block (a task's way to the
+    // rows is one round trip to memory longer, and these are most of the runs of ids that
+    // rarely repeat); wider row waves leave every run to the tasks
+    constexpr uint32_t kRowRun = KW == 1 ? kRowRunMax : 1;
+    static_assert(kRowRunMax == kRowBatch + 2, "the partner and one batch of rows");
 
-    // the columns of wave-unit `g` (this wave's own, or those it adds partial rows for)
-    auto cols_of = [&](uint32_t g) {
-        WaveCols<KW> c;
-#pragma unroll
-        for (int w = 0; w < KW; ++w) {
-            const uint32_t cv = (g * KW + w) * kWave + lane;
-            c.live[w] = cv < CV;
-            c.col[w] = cv * VEC;
+    if (blockIdx.x < task_wgs) {
+        const uint32_t piece = task_piece(blockIdx.x);
+        const uint32_t group = piece / tg.sets, set = piece - group * tg.sets;
+        if (wave >= tg.spans * tg.blocks) return;
+        const uint32_t span = group * tg.spans + wave / tg.blocks;
+        const uint32_t kb = set * tg.blocks + wave % tg.blocks;                 // this wave's column block
+        if (kb >= CB || span * kSpan >= N) return;
+        static_assert(kSpan <= kWave, "a lane per place of the span");
+        const uint32_t p = span * kSpan + lane;
+        const uint32_t word = lane < kSpan && p < N ? row_s[p] : 0u;
+        unsigned long long marked = __builtin_amdgcn_ballot_w64((word & (KW == 1 ? kBigTaskFlag : kTaskFlag)) != 0);
+        while (marked != 0) {
+            const uint32_t at = (uint32_t)__builtin_ctzll(marked);
+            marked &= marked - 1;
+            const uint32_t row = (uint32_t)__builtin_amdgcn_readlane((int)word, (int)at) & kRowMask;
+            const RunInfo ri = info[row];
+            if (ri.R <= kRowRun) continue;                      // (the row itself adds its few partners)
+            if (ri.R <= kSoloRun) sum_short_run<T, TO, VEC>(a, ri, row, kb, lane);
+            else sum_chunk<T, TO, VEC>(a, ri, kb, lane);
         }
-        return c;
-    };
-
-    // a row of a long run
-    auto long_run_row = [&](const RunInfo& ri) {
-        const uint32_t R = ri.R, j = ri.x, start = ri.start;
-        const uint32_t n1 = R / kChunkRows;                             // chunks (at least 2)
-        if (j % kChunkRows != 0 || j / kChunkRows >= n1) return;
-        const uint32_t c = j / kChunkRows;
-        const uint32_t lo = start + c * kChunkRows, hi = c + 1 == n1 ? start + R : lo + kChunkRows;
-        float acc[KW][VEC];
-#pragma unroll
-        for (int w = 0; w < KW; ++w)
-#pragma unroll
-            for (int k = 0; k < VEC; ++k) acc[w][k] = 0.0f;
-        add_listed_rows<T, VEC, KW>(acc, row_s, lo, hi, dY, C, wc);
-#pragma unroll
-        for (int w = 0; w < KW; ++w)
-            if (wc.live[w]) store_partial<VEC>(part + (uint64_t)(lo / kChunkRows) * C + wc.col[w], acc[w]);
-        // the group of chunks this one belongs to, and its counter
-        const uint32_t n2 = n1 / kGroupChunks ? n1 / kGroupChunks : 1u;   // groups
-        const uint32_t q = c / kGroupChunks < n2 ? c / kGroupChunks : n2 - 1;
-        const uint32_t c_lo = q * kGroupChunks, c_hi = q + 1 == n2 ? n1 : c_lo + kGroupChunks;
-        const uint32_t g_at = start + c_lo * kChunkRows;                  // where the group starts
-        const uint32_t fold = kg % kTicketFold, n_fold = (CG - 1 - fold) / kTicketFold + 1;
-        if (!arrive_last(group_tickets + (g_at / (kChunkRows * 2)) * kTicketFold + fold, (c_hi - c_lo) * n_fold, lane)) return;
-        for (uint32_t g2 = fold; g2 < CG; g2 += kTicketFold) {
-            const WaveCols<KW> c2 = cols_of(g2);
-#pragma unroll
-            for (int w = 0; w < KW; ++w) {
-                float sum[VEC];
-                add_partial_rows<VEC>(sum, part, g_at / kChunkRows, c_hi - c_lo, C, c2.col[w], c2.live[w]);
-                if (!c2.live[w]) continue;
-                if (n2 == 1) store_grad_row<TO, VEC>(dW, (uint64_t)ri.tok * C + c2.col[w], sum, accumulate != 0);
-                else store_partial<VEC>(part2 + (uint64_t)(g_at / (kChunkRows * kGroupChunks)) * C + c2.col[w], sum);
-            }
-        }
-        if (n2 == 1) return;
-        if (!arrive_last(run_tickets + (start / (kChunkRows * kGroupChunks * 2)) * kTicketFold + fold, n2, lane)) return;
-        for (uint32_t g2 = fold; g2 < CG; g2 += kTicketFold) {
-            const WaveCols<KW> c2 = cols_of(g2);
-#pragma unroll
-            for (int w = 0; w < KW; ++w) {
-                float sum[VEC];
-                // group q' starts kChunkRows * kGroupChunks places after group q' - 1: its slot is the next
-                add_partial_rows<VEC>(sum, part2, start / (kChunkRows * kGroupChunks), n2, C, c2.col[w], c2.live[w]);
-                if (c2.live[w]) store_grad_row<TO, VEC>(dW, (uint64_t)ri.tok * C + c2.col[w], sum, accumulate != 0);
-            }
-        }
-    };
-
-    // the first row `n` of a short run; `own` are its vectors
-    auto short_run_head = [&](const RunInfo& ri, uint32_t n, const typename Raw::type (&own)[KW]) {
-        typename Raw::type second[KW];
-        uint32_t r1 = n;
-        if (ri.R >= 2) r1 = ri.x != kNoRow ? ri.x : row_s[ri.start + 1];
-#pragma unroll
-        for (int w = 0; w < KW; ++w) {
-            second[w] = Raw::zero();
-            if (wc.live[w] && ri.R >= 2) second[w] = Raw::load(dY + (uint64_t)r1 * C + wc.col[w]);
-        }
-        float acc[KW][VEC];
-#pragma unroll
-        for (int w = 0; w < KW; ++w) {
-            Raw::unpack(own[w], acc[w]);
-            if (ri.R >= 2) {
-                float x[VEC];
-                Raw::unpack(second[w], x);
-#pragma unroll
-                for (int k = 0; k < VEC; ++k) acc[w][k] = acc[w][k] + x[k];
-            }
-        }
-        if (ri.R > 2) add_listed_rows<T, VEC, KW>(acc, row_s, ri.start + 2, ri.start + ri.R, dY, C, wc);
-#pragma unroll
-        for (int w = 0; w < KW; ++w)
-            if (wc.live[w]) store_grad_row<TO, VEC>(dW, (uint64_t)ri.tok * C + wc.col[w], acc[w], accumulate != 0);
-    };
-
-    if (chunk_unit) {
-        // `first` is a word of the chunk heads: take the row it names if that row's RunInfo
-        // agrees that it starts the chunk at this place
-        const uint32_t row = order[order_task_word(N) + first];
-        if (row >= N) return;
-        const RunInfo ri = info[row];
-        if (ri.R > kSoloRun && ri.x % kChunkRows == 0 && (ri.start + ri.x) / kChunkRows == first) long_run_row(ri);
         return;
     }
-    auto load_row = [&](uint32_t n, typename Raw::type (&own)[KW]) {
-#pragma unroll
-        for (int w = 0; w < KW; ++w) {
-            own[w] = Raw::zero();
-            if (wc.live[w]) own[w] = Raw::load(dY + (uint64_t)n * C + wc.col[w]);
-        }
-    };
 
     if constexpr (!POS) {
-        const RunInfo ri = info[first];
-        if (ri.R == 0 || ri.R > kSoloRun) return;            // (a long run's rows are summed by the chunk units)
-        typename Raw::type own[KW];
-        load_row(first, own);
-        short_run_head(ri, first, own);
+        const uint32_t CG = tg.cg;                              // groups of KW column blocks in a row
+        const uint32_t unit = (blockIdx.x - task_wgs) * waves + wave;
+        if (unit >= N * CG) return;
+        const uint32_t n = row_of_unit(unit, tg), kg = unit - n * CG;
+        const RunInfo ri = info[n];
+        if constexpr (KW == 1) {
+            if (ri.R == 0 || ri.R > kRowRun) return;
+            sum_short_run<T, TO, VEC>(a, ri, n, kg, lane);
+        } else {
+            if (ri.R != 1) return;                              // (runs are summed by the tasks)
+            typename Raw::type own[KW];
+#pragma unroll
+            for (int w = 0; w < KW; ++w) {
+                const uint32_t cv = (kg * KW + w) * kWave + lane;
+                own[w] = Raw::zero();
+                if (cv < CV) own[w] = Raw::load(dY + (uint64_t)n * C + cv * VEC);
+            }
+#pragma unroll
+            for (int w = 0; w < KW; ++w) {
+                const uint32_t cv = (kg * KW + w) * kWave + lane;
+                float x[VEC];
+                Raw::unpack(own[w], x);
+                if (cv < CV) store_grad_row<TO, VEC>(dW, (uint64_t)ri.tok * C + cv * VEC, x, accumulate != 0);
+            }
+        }
     } else {
-        // The workgroup has position `first`; wave w takes the rows b = w, w + waves, ... of the
-        // batch, each like a row of its own, and leaves the row's vector in LDS, where wave 0
-        // adds the batch's vectors in ascending b: dwpe[t, :] (+)= sum_b dY[b, t, :].
-        __shared__ float shared_rows[kPosWaves * kPosRows][kWave * VEC];
-        const uint32_t pass_rows = waves * kPosRows;            // rows of a pass: kPosRows per wave, all in flight
+        // The workgroup has position t and one column block; wave w takes the rows b = w,
+        // w + waves, ... of the batch, each like a row of its own, and leaves the row's vector in
+        // LDS, where wave 0 adds the batch's vectors in ascending b.
+        __shared__ float shared_rows[kPosWaves][kWave * VEC];
+        const uint32_t unit = blockIdx.x - task_wgs;
+        if (unit >= T_len * CB) return;
+        const uint32_t t = row_of_unit(unit, tg), kb = unit - t * CB;     // (tg.cg == CB here)
+        const uint32_t cv = kb * kWave + lane, col = cv * VEC;
+        const bool live = cv < CV;
         float pos_acc[VEC];
 #pragma unroll
         for (int k = 0; k < VEC; ++k) pos_acc[k] = 0.0f;
 #pragma nounroll
-        for (uint32_t b0 = 0; b0 < B; b0 += pass_rows) {
-            RunInfo ri[kPosRows];
-            typename Raw::type own[kPosRows][1];
+        for (uint32_t b0 = 0; b0 < B; b0 += waves) {
+            const uint32_t b = b0 + wave;
+            if (b < B) {
+                const uint32_t n = b * T_len + t;
+                const RunInfo ri = info[n];
+                typename Raw::type own = Raw::zero();
+                if (live) own = Raw::load(dY + (uint64_t)n * C + col);
+                float x[VEC];
+                Raw::unpack(own, x);
 #pragma unroll
-            for (int j = 0; j < kPosRows; ++j) {
-                const uint32_t b = b0 + j * waves + wave;
-                ri[j] = RunInfo{V, 0u, 0u, 0u};
-                own[j][0] = Raw::zero();
-                if (b < B) {
-                    ri[j] = info[b * T_len + first];
-                    load_row(b * T_len + first, own[j]);
-                }
-            }
-#pragma unroll
-            for (int j = 0; j < kPosRows; ++j) {
-                const uint32_t b = b0 + j * waves + wave;
-                if (b < B) {
-                    float x[VEC];
-                    Raw::unpack(own[j][0], x);
-#pragma unroll
-                    for (int k = 0; k < VEC; ++k) shared_rows[j * waves + wave][lane * VEC + k] = x[k];
-                    if (ri[j].R != 0 && ri[j].R <= kSoloRun) short_run_head(ri[j], b * T_len + first, own[j]);
-                }
+                for (int k = 0; k < VEC; ++k) shared_rows[wave][lane * VEC + k] = x[k];
+                if (ri.R == 1 && live) store_grad_row<TO, VEC>(dW, (uint64_t)ri.tok * C + col, x, accumulate != 0);
+                else if (ri.R >= 2 && ri.R <= kRowRun) sum_short_run<T, TO, VEC>(a, ri, n, kb, lane);
             }
             __syncthreads();
             if (wave == 0) {
-                const uint32_t rows = B - b0 < pass_rows ? B - b0 : pass_rows;
-                for (uint32_t r = 0; r < rows; ++r) {           // (row b0 + r sits in slot r: r = j * waves + w)
+                const uint32_t rows = B - b0 < waves ? B - b0 : waves;
+                for (uint32_t r = 0; r < rows; ++r) {
 #pragma unroll
                     for (int k = 0; k < VEC; ++k) {
                         const float v = shared_rows[r][lane * VEC + k];
@@ -1001,14 +1067,14 @@ emb_row_sum_kernel(const uint32_t* __restrict__ order, uint32_t* group_tickets, 
             }
             __syncthreads();
         }
-        if (wave == 0 && wc.live[0]) store_grad_row<TO, VEC>(dwpe, (uint64_t)first * C + wc.col[0], pos_acc, accumulate_pos != 0);
+        if (wave == 0 && live) store_grad_row<TO, VEC>(dwpe, (uint64_t)t * C + col, pos_acc, accumulate_pos != 0);
     }
 }
 
 // The radix path's ordering is by token throughout: the run of place p is found by two
 // bisections of the sorted tokens.  Also zeroes the gradient kernel's arrival counters.
 __global__ void __launch_bounds__(256)
-emb_run_info_kernel(const uint32_t* __restrict__ tok_s, uint32_t* __restrict__ order, uint32_t N, uint32_t V) {
+emb_run_info_kernel(const uint32_t* __restrict__ tok_s, uint32_t* order, uint32_t N, uint32_t V) {
     const uint32_t p = blockIdx.x * 256 + threadIdx.x;
     {
         const uint32_t words = (uint32_t)(order_group_tickets(N) + order_run_tickets(N));
@@ -1016,7 +1082,7 @@ emb_run_info_kernel(const uint32_t* __restrict__ tok_s, uint32_t* __restrict__ o
         for (uint32_t w = p; w < words; w += gridDim.x * 256) tickets[w] = 0;
     }
     if (p >= N) return;
-    const uint32_t* row_s = order;
+    const volatile uint32_t* row_s = order;
     RunInfo* info = reinterpret_cast<RunInfo*>(order + order_info_word(N));
     const uint32_t tok = tok_s[p];
     uint32_t lo = 0, hi = p;                    // first place holding tok
@@ -1025,17 +1091,16 @@ emb_run_info_kernel(const uint32_t* __restrict__ tok_s, uint32_t* __restrict__ o
     lo = p + 1; hi = N;                         // first place after the run
     while (lo < hi) { const uint32_t mid = (lo + hi) >> 1; if (tok_s[mid] <= tok) lo = mid + 1; else hi = mid; }
     const uint32_t R = lo - start, j = p - start;
+    // (the neighbour's word may already carry its task mark: only the row bits are read)
+    const uint32_t row = row_s[p] & kRowMask;
     RunInfo ri;
     ri.tok = tok;
     ri.start = start;
     if (tok >= V) { ri.R = 0; ri.x = 0; }
-    else if (R <= kSoloRun) { ri.R = j == 0 ? R : 0u; ri.x = j + 1 < R ? row_s[p + 1] : kNoRow; }
-    else {
-        ri.R = R;
-        ri.x = j;
-        if (j % kChunkRows == 0 && j / kChunkRows < R / kChunkRows) order[order_task_word(N) + p / kChunkRows] = row_s[p];
-    }
-    info[row_s[p]] = ri;
+    else if (R <= kSoloRun) { ri.R = j == 0 ? R : 0u; ri.x = j + 1 < R ? row_s[p + 1] & kRowMask : kNoRow; }
+    else { ri.R = R; ri.x = j; }
+    if (tok < V && task_marks(j, R) != 0) order[p] = row | task_marks(j, R);
+    info[row] = ri;
 }
 
 // dwpe[t, c] (+)= sum_b dY[b, t, c], b ascending
@@ -1097,33 +1162,46 @@ int embedding_sum_typed(hipStream_t s, const uint32_t* order, const T* dY, TO* d
     const bool wide = C % WIDE == 0 && aligned16(dY) && aligned16(dW) && (!dwpe || aligned16(dwpe));
     const uint32_t CV = wide ? C / WIDE : C;
     const uint32_t CB = (CV + kWave - 1) / kWave;               // column blocks: a wave's worth of vectors each
-    // (KW = 4 column blocks per wave was measured too: it saves most of the 30 us that starting
-    // half a million waves costs at 65536 x 4096 bf16 and gains 4 % on runs of 4..32 rows, but
-    // a long run's chunks then take four times as long each, and Zipf ids lose 20 %.)
-    // workgroups: the chunks of long runs, packed; then four rows each -- or, with a position
+    // workgroups: the tasks' (a span of row_s[] each); then four rows each -- or, with a position
     // table, one position and column block each, with a wave per row of the batch
     const uint32_t waves = dwpe ? (B < (uint32_t)kPosWaves ? B : (uint32_t)kPosWaves) : kRowSumWaves;
-    const uint64_t chunk_wgs = (order_tasks(N) * CB + waves - 1) / waves;
-    const uint64_t row_wgs = dwpe ? (uint64_t)T_len * CB : ((uint64_t)N * CB + waves - 1) / waves;
-    if (chunk_wgs + row_wgs >= 0x7fffffffull || (uint64_t)N * CB >= 0xffffff00ull)
+    // Column blocks of a row per wave: one, while that starts no more than kRowWavesEasy waves
+    // (a wave that takes a whole wide row alone moves single rows 3 to 10 % slower); beyond, as
+    // many as bring the count down to that -- a wave with nothing to do costs about 0.08 ns
+    // of the call, and they run after the waves that have.
+    int KW = 1;
+    if (wide && !dwpe)
+        while (KW < kRowBlocksMax && KW < (int)CB && (uint64_t)N * ((CB + KW - 1) / KW) > kRowWavesEasy) KW *= 2;
+    const uint32_t CG = (CB + KW - 1) / KW;
+    const TaskGrid tg = task_grid(N, CB, waves, KW == 1 ? kBigTaskSpan : kTaskSpan, CG);
+    const uint64_t task_wgs = tg.wgs;
+    const uint64_t row_wgs = dwpe ? (uint64_t)T_len * CB : ((uint64_t)N * CG + waves - 1) / waves;
+    if (task_wgs + row_wgs >= 0x7fffffffull || (uint64_t)N * CB >= 0xffffff00ull)
         return set_error(AGRAD_EINVAL, "embedding backward: %u rows of %u columns are too many", N, C);
-    const uint32_t grid = (uint32_t)(chunk_wgs + row_wgs);
+    const uint32_t grid = (uint32_t)(task_wgs + row_wgs);
     const uint32_t block = waves * kWave;
-#define AGRAD_ROW_SUM(VEC, POS) \
-    hipLaunchKernelGGL((emb_row_sum_kernel<T, TO, VEC, 1, POS>), dim3(grid), dim3(block), 0, s, order, \
+#define AGRAD_ROW_SUM(VEC, KW, POS) \
+    hipLaunchKernelGGL((emb_row_sum_kernel<T, TO, VEC, KW, POS>), dim3(grid), dim3(block), 0, s, order, \
                        const_cast<uint32_t*>(order) + order_ticket_word(N), dY, dW, dwpe, part, N, C, CV, CB, V, T_len, B, \
-                       acc, acc_pos)
-    if (wide) {
-        if (dwpe) AGRAD_ROW_SUM(WIDE, true); else AGRAD_ROW_SUM(WIDE, false);
+                       acc, acc_pos, tg)
+    if (dwpe) {
+        if (wide) AGRAD_ROW_SUM(WIDE, 1, true); else AGRAD_ROW_SUM(1, 1, true);
+    } else if (!wide) {
+        AGRAD_ROW_SUM(1, 1, false);
     } else {
-        if (dwpe) AGRAD_ROW_SUM(1, true); else AGRAD_ROW_SUM(1, false);
+        switch (KW) {
+            case 1: AGRAD_ROW_SUM(WIDE, 1, false); break;
+            case 2: AGRAD_ROW_SUM(WIDE, 2, false); break;
+            case 4: AGRAD_ROW_SUM(WIDE, 4, false); break;
+            default: AGRAD_ROW_SUM(WIDE, kRowBlocksMax, false); break;
+        }
     }
 #undef AGRAD_ROW_SUM
     return check_hip(hipGetLastError(), "embedding backward launch");
 }
 
 int check_embedding_sizes(const char* what, uint64_t N, uint32_t V) {
-    if (N >= 0x7fffffffull) return set_error(AGRAD_EINVAL, "%s: too many rows", what);
+    if (N >= 0x40000000ull) return set_error(AGRAD_EINVAL, "%s: too many rows", what);
     if (V == 0 || V >= 0x7fffffffu) return set_error(AGRAD_EINVAL, "%s: bad vocabulary size %u", what, V);
     return AGRAD_OK;
 }

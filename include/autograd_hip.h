@@ -306,9 +306,9 @@ int agrad_gather_forward(agrad_ctx* ctx, int dtype, const int32_t* ids,
                          uint64_t N, uint32_t T, uint32_t C, uint32_t V);
 
 /* Embedding gradient dW[ids[n],:] += dY[n,:], deterministic: the rows are ordered
- * so that each token's rows are adjacent and ascending, and one launch then walks dY
- * in row order.  The first row of a token with up to 127 rows adds that token's rows
- * in ascending row order -- the sequence of fp32 adds np.add.at makes
+ * so that each token's rows are adjacent and ascending, and one launch then reads dY
+ * once.  One wave adds the rows of a token with up to 127 rows in ascending row
+ * order -- the sequence of fp32 adds np.add.at makes
  * (cpu_gather_backward, backend.py:531-538; replaces the float-atomic
  * gather_backward_kernel, metal_ops.metal:406-427).  A token with more rows is cut
  * into chunks of 64 rows, summed in row order each; the chunk sums are added in
@@ -326,8 +326,11 @@ int agrad_embedding_backward(agrad_ctx* ctx, int dtype, const int32_t* ids, cons
  * is free: up to 65536 rows the gather and the ordering are ONE launch (the
  * ordering workgroups run beside the bandwidth-bound gather), and the backward
  * call is one launch that reads dY front to back.  The forward call also writes
- * `order`, 6N + 128 uint32, 16-byte aligned: order[0..N) = the rows, each token's
- * rows adjacent and ascending; then, from the next multiple of four words on, four
+ * `order`, 6N + 128 uint32, 16-byte aligned: order[0..N) = the rows (in the low 30
+ * bits: N < 2^30), each token's rows adjacent and ascending; bit 31 marks the first
+ * row of a run of 2..127 rows and the first row of each 64-row chunk of a longer run
+ * (the run's last chunk takes the rest), bit 30 those of them that start more than
+ * 10 rows: what the backward call hands out as tasks.  Then, from the next multiple of four words on, four
  * words for row n = 0..N-1: its token (V for an id outside the table), the place
  * in order[] where its token's run starts, and (R, x): R = 0 for a row with
  * nothing to do (a later row of a run of up to 127 rows, an id outside the table);

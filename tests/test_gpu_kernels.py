@@ -945,13 +945,17 @@ def test_presorted_embedding_pair_matches_the_plain_pair(ctx, B, T, V, C, dist, 
 
 def _check_order(order, N, tokens, V):
     """The order buffer of the pre-sorted embedding pair: rows[N] (each token's rows adjacent
-    and ascending), then, from the next multiple of four words, four words for every row:
-    its token, where its token's run starts, and (R, x): R = 0 for a later row of a run of
-    up to 127 rows and for an id outside the table; the run's length for the first row of
+    and ascending; the top bit of a word marks a task of the gradient kernel: the first row
+    of a run of 2 to 127 rows, or the first row of a 64-row chunk of a longer run, whose last
+    chunk takes the rest; the bit below marks the tasks of more than 10 rows), then, from the next multiple of four words, four words for every
+    row: its token, where its token's run starts, and (R, x): R = 0 for a later row of a run
+    of up to 127 rows and for an id outside the table; the run's length for the first row of
     such a run, with x = the run's second row (or 0xFFFFFFFF: not given); for a longer run
     its length and x = the row's index in it.  Then the gradient kernel's arrival counters,
     all zero.  Returns the rows and their tokens."""
-    rows = order[:N].astype(np.int64)
+    rows = (order[:N] & 0x3FFFFFFF).astype(np.int64)
+    marked = (order[:N] >> 31).astype(bool)
+    marked_big = ((order[:N] >> 30) & 1).astype(bool)
     at = (N + 3) // 4 * 4
     info = order[at:at + 4 * N].reshape(N, 4).astype(np.int64)
     tickets = order[at + 4 * N:at + 4 * N + (N // 128 + 1) * 32 + (N // 2048 + 1) * 32]
@@ -976,6 +980,9 @@ def _check_order(order, N, tokens, V):
     np.testing.assert_array_equal(x[short & (j == 0) & (run == 1)], 0xFFFFFFFF)
     np.testing.assert_array_equal(R[valid & ~short], run[valid & ~short])
     np.testing.assert_array_equal(x[valid & ~short], j[valid & ~short])
+    chunk_head = valid & ~short & (j % 64 == 0) & (j // 64 < run // 64)
+    np.testing.assert_array_equal(marked, second | chunk_head)
+    np.testing.assert_array_equal(marked_big, (second & (run > 10)) | chunk_head)
     return rows, toks
 
 
