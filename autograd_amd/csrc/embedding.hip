@@ -740,6 +740,7 @@ constexpr int kRowBatch = 8;          // rows a wave keeps in flight
                                       // (16 for the chunks of long runs take the kernel from 60 to 90 registers: fewer waves
                                       // per CU, and single rows move 3 to 10 % slower for 4 % on Zipf ids)
 constexpr int kPosWaves = 4;          // most waves that share the rows of one position
+constexpr int kPosRows = 4;           // rows that each of them has in flight
 constexpr int kRowSumBlock = 256;
 constexpr uint32_t kRowSumWaves = kRowSumBlock / kWave;
 constexpr int kRowBlocksMax = 8;      // most column blocks of a row that one wave moves
@@ -1027,43 +1028,60 @@ emb_row_sum_kernel(const uint32_t* __restrict__ order, uint32_t* group_tickets, 
             }
         }
     } else {
-        // The workgroup has position t and one column block; wave w takes the rows b = w,
-        // w + waves, ... of the batch, each like a row of its own, and leaves the row's vector in
-        // LDS, where wave 0 adds the batch's vectors in ascending b.
-        __shared__ float shared_rows[kPosWaves][kWave * VEC];
+        // The workgroup has position t and one column block.  In a pass its waves read
+        // waves x kPosRows rows of the batch -- wave w the rows b0 + w, b0 + waves + w, ..., all in
+        // flight, each with what the row is -- and leave the vectors in LDS, where wave 0 adds them
+        // in ascending b; the other waves meanwhile add up the short runs that their rows start.
+        // (A batch's last rows are read again where B is no multiple of a pass: every load has a
+        // valid address and no branch around it.)
+        __shared__ typename Raw::type shared_rows[kPosWaves * kPosRows][kWave];
         const uint32_t unit = blockIdx.x - task_wgs;
         if (unit >= T_len * CB) return;
         const uint32_t t = row_of_unit(unit, tg), kb = unit - t * CB;     // (tg.cg == CB here)
         const uint32_t cv = kb * kWave + lane, col = cv * VEC;
         const bool live = cv < CV;
+        const uint32_t col_ld = live ? col : 0u;
+        const uint32_t pass_rows = waves * kPosRows;
         float pos_acc[VEC];
 #pragma unroll
         for (int k = 0; k < VEC; ++k) pos_acc[k] = 0.0f;
 #pragma nounroll
-        for (uint32_t b0 = 0; b0 < B; b0 += waves) {
-            const uint32_t b = b0 + wave;
-            if (b < B) {
-                const uint32_t n = b * T_len + t;
-                const RunInfo ri = info[n];
-                typename Raw::type own = Raw::zero();
-                if (live) own = Raw::load(dY + (uint64_t)n * C + col);
-                float x[VEC];
-                Raw::unpack(own, x);
+        for (uint32_t b0 = 0; b0 < B; b0 += pass_rows) {
+            RunInfo ri[kPosRows];
+            typename Raw::type v[kPosRows];
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) shared_rows[wave][lane * VEC + k] = x[k];
-                if (ri.R == 1 && live) store_grad_row<TO, VEC>(dW, (uint64_t)ri.tok * C + col, x, accumulate != 0);
-                else if (ri.R >= 2 && ri.R <= kRowRun) sum_short_run<T, TO, VEC>(a, ri, n, kb, lane);
+            for (int j = 0; j < kPosRows; ++j) {
+                const uint32_t b = b0 + j * waves + wave;
+                const uint32_t n = (b < B ? b : B - 1) * T_len + t;
+                ri[j] = info[n];
+                v[j] = Raw::load(dY + (uint64_t)n * C + col_ld);
+            }
+#pragma unroll
+            for (int j = 0; j < kPosRows; ++j) {
+                const uint32_t b = b0 + j * waves + wave;
+                if (b < B) {
+                    shared_rows[j * waves + wave][lane] = v[j];
+                    if (ri[j].R == 1 && live) {
+                        float x[VEC];
+                        Raw::unpack(v[j], x);
+                        store_grad_row<TO, VEC>(dW, (uint64_t)ri[j].tok * C + col, x, accumulate != 0);
+                    }
+                }
             }
             __syncthreads();
             if (wave == 0) {
-                const uint32_t rows = B - b0 < waves ? B - b0 : waves;
-                for (uint32_t r = 0; r < rows; ++r) {
+                const uint32_t rows = B - b0 < pass_rows ? B - b0 : pass_rows;
+                for (uint32_t r = 0; r < rows; ++r) {           // (row b0 + r sits in slot r = j * waves + w)
+                    float x[VEC];
+                    Raw::unpack(shared_rows[r][lane], x);
 #pragma unroll
-                    for (int k = 0; k < VEC; ++k) {
-                        const float v = shared_rows[r][lane * VEC + k];
-                        pos_acc[k] = b0 + r == 0 ? v : pos_acc[k] + v;
-                    }
+                    for (int k = 0; k < VEC; ++k) pos_acc[k] = b0 + r == 0 ? x[k] : pos_acc[k] + x[k];
                 }
+            }
+#pragma unroll
+            for (int j = 0; j < kPosRows; ++j) {
+                const uint32_t b = b0 + j * waves + wave;
+                if (b < B && ri[j].R >= 2 && ri[j].R <= kRowRun) sum_short_run<T, TO, VEC>(a, ri[j], b * T_len + t, kb, lane);
             }
             __syncthreads();
         }
