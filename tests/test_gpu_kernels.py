@@ -700,6 +700,80 @@ def test_embedding_backward_long_runs_wide_rows_and_deep_trees(ctx, N, C, tokens
     np.testing.assert_array_equal(acc, base + got)
 
 
+def _sums_in_row_order(ids, dY, V):
+    """dW[t] = ((dY[r0] + dY[r1]) + dY[r2]) + ... over the rows of token t in ascending order, in
+    fp32: what np.add.at does to a zero table, written with one vector add per position in
+    the run instead of one numpy call per row (cpu_ops.gather_backward_into takes 20 s
+    where this takes a fraction of one; the test below checks the two against each other on
+    a slice)"""
+    N, C = dY.shape
+    rows = np.argsort(ids, kind="stable")
+    toks = ids[rows]
+    starts = np.flatnonzero(np.concatenate([[True], toks[1:] != toks[:-1]]))
+    lens = np.diff(np.concatenate([starts, [N]]))
+    dW = np.zeros((V, C), np.float32)
+    for L in np.unique(lens):
+        first = starts[lens == L]
+        acc = dY[rows[first]].copy()
+        for j in range(1, L):
+            acc += dY[rows[first + j]]
+        dW[toks[first]] = acc
+    return dW
+
+
+def _ids_with_runs(rng, lengths, V):
+    """a shuffled id list in which token k occurs lengths[k] times"""
+    toks = rng.choice(V, size=len(lengths), replace=False).astype(np.int32)
+    return rng.permutation(np.repeat(toks, lengths))
+
+
+@pytest.mark.parametrize("C,io", [(96, "f32"), (1024, "f32"), (2048, "bf16")])
+def test_embedding_backward_every_run_length(ctx, C, io):
+    """Runs of every length around the places where the gradient kernel changes its way of
+    adding a run up: a token's only row (moved by the row's own wave); 2 to 10 rows (added by
+    the first row's wave when a wave takes one column block -- narrow rows -- and by a task
+    wave when it takes several: the wide shapes here start more than 131072 waves); 11 to
+    127 rows (a task wave, ascending row order: np.add.at's own bits); 128 rows and more
+    (64-row chunks, the last taking the rest, in groups of 16).  Twice (the arrival counters
+    must be back at zero) and through the accumulate flag."""
+    rng = _rng(C + 5)
+    lengths = np.array(list(range(1, 14)) * 40 + [1] * 20000 + [2] * 3000 + [3] * 500
+                       + [62, 63, 64, 65, 66, 126, 127, 128, 129, 130, 191, 192, 193, 255, 256, 257, 1023, 1024, 1025, 1100, 2049, 2500])
+    V = 26000
+    ids = _ids_with_runs(rng, lengths, V)
+    N = ids.size
+    if io == "bf16":
+        dY = to_bf16_bits(rng.random((1, N, C), dtype=np.float32) - 0.5)
+        dY32 = from_bf16_bits(dY)
+    else:
+        dY = dY32 = rng.random((1, N, C), dtype=np.float32) - 0.5
+    ids2 = ids.reshape(1, N)
+    got = G.embedding_backward(ctx, ids2, dY, V)
+    seq = _sums_in_row_order(ids, dY32[0], V)                          # np.add.at: ascending rows
+    part = np.zeros((V, 16), np.float32)
+    ref.gather_backward_into(ids2, np.ascontiguousarray(dY32[:, :, :16]), part)
+    np.testing.assert_array_equal(seq[:, :16], part)
+    run = np.bincount(ids, minlength=V)
+    if io == "bf16":
+        got32 = from_bf16_bits(got)
+        short = (run >= 1) & (run <= 127)
+        np.testing.assert_array_equal(got[short], to_bf16_bits(seq[short]))       # the same fp32 sum, rounded once
+        assert_bf16_close(got32, seq, "bf16 embedding backward, every run length")
+        assert not got32[run == 0].any()
+    else:
+        short = run <= 127
+        np.testing.assert_array_equal(got[short], seq[short])
+        d64 = np.zeros((V, C))
+        for t in np.flatnonzero(run > 127):
+            d64[t] = dY32[0][ids == t].astype(np.float64).sum(0)
+        long_rows = run > 127
+        assert_fp32_parity(got[long_rows], seq[long_rows], d64[long_rows], f"dW of the long runs, C = {C}")
+        base = rng.standard_normal((V, C), dtype=np.float32)
+        acc = G.embedding_backward(ctx, ids2, dY, V, dW_init=base, flags=capi.ACC_PARAM_GRAD)
+        np.testing.assert_array_equal(acc, base + got)
+    np.testing.assert_array_equal(got, G.embedding_backward(ctx, ids2, dY, V))
+
+
 def test_embedding_backward_short_runs_bit_exact(ctx):
     """Runs of up to 127 rows are summed by their first row in ascending row order: the
     same sequence of fp32 adds as np.add.at."""
