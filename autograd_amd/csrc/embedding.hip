@@ -264,6 +264,7 @@ __host__ __device__ inline uint32_t task_marks(uint32_t j, uint32_t R) {
 // (blocks: a power of two); rows with more column blocks take `sets` workgroups per span.
 struct TaskGrid {
     uint32_t blocks, spans, sets, wgs;
+    uint32_t big_wgs;           // workgroups in front of those that take only the tasks of more than kRowRunMax rows, or 0
     uint32_t cg, cg_magic;      // (the row part) column groups of a row; ceil(2^32 / cg) where that divides exactly, or 0
 };
 // u / g.cg for u below rows x g.cg
@@ -281,6 +282,10 @@ inline TaskGrid task_grid(uint32_t N, uint32_t CB, uint32_t waves, uint32_t span
     g.sets = (CB + g.blocks - 1) / g.blocks;
     const uint32_t places = g.spans * span;
     g.wgs = (((N + places - 1) / places) * g.sets + 7u) & ~7u;
+    // Where every run is a task, the big ones (the chunks of long runs above all: their sums
+    // have two hand-offs still to go through) get workgroups of their own, in front of all others.
+    const uint32_t big_places = g.spans * kBigTaskSpan;
+    g.big_wgs = span == kBigTaskSpan ? 0u : (((N + big_places - 1) / big_places) * g.sets + 7u) & ~7u;
     return g;
 }
 // Workgroups go to the GPU's eight XCDs in turn.  The chunks of a long run start every
@@ -780,21 +785,21 @@ __device__ __forceinline__ void load_partial(const float* p, float (&v)[VEC]) {
 }
 
 // acc += dY[r, col ...] for the rows r that lanes 0 .. cnt-1 hold in `mine`, in lane order
-template <typename T, int VEC>
+template <typename T, int VEC, int BATCH = kRowBatch>
 __device__ __forceinline__ void add_lane_rows(float (&acc)[VEC], uint32_t mine, uint32_t cnt, const T* __restrict__ dY,
                                               uint32_t C, uint32_t col, bool live) {
     typedef RawVec<T, VEC> Raw;
 #pragma nounroll
-    for (uint32_t q0 = 0; q0 < cnt; q0 += kRowBatch) {
-        typename Raw::type v[kRowBatch];
+    for (uint32_t q0 = 0; q0 < cnt; q0 += BATCH) {
+        typename Raw::type v[BATCH];
 #pragma unroll
-        for (int q = 0; q < kRowBatch; ++q) {
+        for (int q = 0; q < BATCH; ++q) {
             const uint32_t r = (uint32_t)__builtin_amdgcn_readlane((int)mine, (int)(q0 + q));
             v[q] = Raw::zero();
             if (q0 + q < cnt && live) v[q] = Raw::load(dY + (uint64_t)r * C + col);
         }
 #pragma unroll
-        for (int q = 0; q < kRowBatch; ++q) {
+        for (int q = 0; q < BATCH; ++q) {
             if (q0 + q < cnt) {
                 float x[VEC];
                 Raw::unpack(v[q], x);
@@ -808,7 +813,7 @@ __device__ __forceinline__ void add_lane_rows(float (&acc)[VEC], uint32_t mine, 
 // acc += dY[row_s[p], col ...] for p = from .. to-1, ascending (p is the same in every lane).
 // The wave fetches 64 places of row_s[] with one load, a place per lane, and hands the rows
 // round from there.
-template <typename T, int VEC>
+template <typename T, int VEC, int BATCH = kRowBatch>
 __device__ __forceinline__ void add_listed_rows(float (&acc)[VEC], const uint32_t* __restrict__ row_s, uint32_t from,
                                                 uint32_t to, const T* __restrict__ dY, uint32_t C, uint32_t col, bool live,
                                                 uint32_t lane) {
@@ -816,7 +821,7 @@ __device__ __forceinline__ void add_listed_rows(float (&acc)[VEC], const uint32_
     for (uint32_t base = from; base < to; base += kWave) {
         const uint32_t cnt = to - base < kWave ? to - base : kWave;
         const uint32_t mine = lane < cnt ? row_s[base + lane] & kRowMask : 0u;
-        add_lane_rows<T, VEC>(acc, mine, cnt, dY, C, col, live);
+        add_lane_rows<T, VEC, BATCH>(acc, mine, cnt, dY, C, col, live);
     }
 }
 
@@ -961,7 +966,7 @@ emb_row_sum_kernel(const uint32_t* __restrict__ order, uint32_t* group_tickets, 
     const uint32_t* __restrict__ row_s = order;
     const RunInfo* __restrict__ info = reinterpret_cast<const RunInfo*>(order + order_info_word(N));
     constexpr uint32_t kSpan = KW == 1 ? kBigTaskSpan : kTaskSpan;       // (tg: the host's task_grid() for this span)
-    const uint32_t task_wgs = tg.wgs;
+    const uint32_t task_wgs = tg.big_wgs + tg.wgs;
     RowSumArgs<T, TO> a;
     a.row_s = row_s;
     a.group_tickets = group_tickets;
@@ -979,16 +984,22 @@ emb_row_sum_kernel(const uint32_t* __restrict__ order, uint32_t* group_tickets, 
     static_assert(kRowRunMax == kRowBatch + 2, "the partner and one batch of rows");
 
     if (blockIdx.x < task_wgs) {
-        const uint32_t piece = task_piece(blockIdx.x);
+        // in front: the workgroups of the big tasks alone (where there are such); then those of
+        // every other task -- or, where the rows add short runs themselves, of the big tasks only
+        const bool big_pass = blockIdx.x < tg.big_wgs;
+        const uint32_t piece = task_piece(big_pass ? blockIdx.x : blockIdx.x - tg.big_wgs);
         const uint32_t group = piece / tg.sets, set = piece - group * tg.sets;
         if (wave >= tg.spans * tg.blocks) return;
         const uint32_t span = group * tg.spans + wave / tg.blocks;
         const uint32_t kb = set * tg.blocks + wave % tg.blocks;                 // this wave's column block
-        if (kb >= CB || span * kSpan >= N) return;
-        static_assert(kSpan <= kWave, "a lane per place of the span");
-        const uint32_t p = span * kSpan + lane;
-        const uint32_t word = lane < kSpan && p < N ? row_s[p] : 0u;
-        unsigned long long marked = __builtin_amdgcn_ballot_w64((word & (KW == 1 ? kBigTaskFlag : kTaskFlag)) != 0);
+        const uint32_t places = big_pass ? kBigTaskSpan : kSpan;
+        if (kb >= CB || span * places >= N) return;
+        static_assert(kSpan <= kWave && kBigTaskSpan <= kWave, "a lane per place of the span");
+        const uint32_t p = span * places + lane;
+        const uint32_t word = lane < places && p < N ? row_s[p] : 0u;
+        const uint32_t marks = word & (kTaskFlag | kBigTaskFlag);
+        const bool wanted = KW == 1 || big_pass ? (marks & kBigTaskFlag) != 0 : marks == kTaskFlag;
+        unsigned long long marked = __builtin_amdgcn_ballot_w64(wanted);
         while (marked != 0) {
             const uint32_t at = (uint32_t)__builtin_ctzll(marked);
             marked &= marked - 1;
@@ -1192,7 +1203,7 @@ int embedding_sum_typed(hipStream_t s, const uint32_t* order, const T* dY, TO* d
         while (KW < kRowBlocksMax && KW < (int)CB && (uint64_t)N * ((CB + KW - 1) / KW) > kRowWavesEasy) KW *= 2;
     const uint32_t CG = (CB + KW - 1) / KW;
     const TaskGrid tg = task_grid(N, CB, waves, KW == 1 ? kBigTaskSpan : kTaskSpan, CG);
-    const uint64_t task_wgs = tg.wgs;
+    const uint64_t task_wgs = (uint64_t)tg.big_wgs + tg.wgs;
     const uint64_t row_wgs = dwpe ? (uint64_t)T_len * CB : ((uint64_t)N * CG + waves - 1) / waves;
     if (task_wgs + row_wgs >= 0x7fffffffull || (uint64_t)N * CB >= 0xffffff00ull)
         return set_error(AGRAD_EINVAL, "embedding backward: %u rows of %u columns are too many", N, C);
