@@ -1139,13 +1139,26 @@ pos_grad_kernel(const T* __restrict__ dY, TO* dwpe, uint32_t B, uint64_t TCV, ui
     const uint64_t idx = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= TCV) return;
     const uint64_t off = idx * VEC;
+    // eight rows of the batch in flight (the adds stay in ascending b); the rows past the last
+    // are read from the last one, so that no load sits behind a branch
+    typedef RawVec<T, VEC> Raw;
     float acc[VEC];
-    VecIO<T, VEC>::load(dY + off, acc);
-    for (uint32_t b = 1; b < B; ++b) {
-        float v[VEC];
-        VecIO<T, VEC>::load(dY + (uint64_t)b * TC + off, v);
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) acc[k] = acc[k] + v[k];
+    for (int k = 0; k < VEC; ++k) acc[k] = 0.0f;
+#pragma nounroll
+    for (uint32_t b0 = 0; b0 < B; b0 += kRowBatch) {
+        typename Raw::type v[kRowBatch];
+#pragma unroll
+        for (int q = 0; q < kRowBatch; ++q) v[q] = Raw::load(dY + (uint64_t)(b0 + q < B ? b0 + q : B - 1) * TC + off);
+#pragma unroll
+        for (int q = 0; q < kRowBatch; ++q) {
+            if (b0 + q < B) {
+                float x[VEC];
+                Raw::unpack(v[q], x);
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) acc[k] = b0 + q == 0 ? x[k] : acc[k] + x[k];
+            }
+        }
     }
     store_grad_row<TO, VEC>(dwpe, off, acc, accumulate != 0);
 }
