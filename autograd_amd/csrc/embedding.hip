@@ -1094,7 +1094,7 @@ emb_row_sum_kernel(const uint32_t* __restrict__ order, uint32_t* group_tickets, 
                 const uint32_t b = b0 + j * waves + wave;
                 if (b < B && ri[j].R >= 2 && ri[j].R <= kRowRun) sum_short_run<T, TO, VEC>(a, ri[j], b * T_len + t, kb, lane);
             }
-            __syncthreads();
+            if (b0 + pass_rows < B) __syncthreads();            // (LDS is written again only if a pass follows)
         }
         if (wave == 0 && live) store_grad_row<TO, VEC>(dwpe, (uint64_t)t * C + col, pos_acc, accumulate_pos != 0);
     }

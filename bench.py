@@ -13,7 +13,7 @@ Output: one JSON line per configuration with its per-op table (every op and
 direction timed on its own with HIP events on the library's stream over rotating
 buffer sets, so the working set exceeds the 256 MB Infinity Cache; copy_us /
 vs_copy compare with a plain copy kernel moving the same number of bytes the same
-way), the same tables as one file (--detail, default gpurun_out/bench_per_op.json),
+way), the same tables as one file (--detail; by default bench_per_op.json in the run's output folder),
 and as the LAST line one compact JSON object:
 
   value / unit     whole-step algorithmic GB/s (sum of the ops' algorithmic bytes

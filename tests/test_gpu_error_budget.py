@@ -14,7 +14,7 @@ error no more than 1.25 x the restatement's largest, root-mean-square error no m
 evaluations over millions of elements) -- and in every case the device differs from the
 restatement by no more than the two distances from float64 together.
 
-The table goes to gpurun_out/error_budget.md when that directory can be written.
+The table is also written as error_budget.md into the run's output folder, when that can be written.
 """
 import os
 from pathlib import Path
