@@ -9,6 +9,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include "fastdiv.hpp"
 
 namespace agrad {
 

@@ -33,6 +33,7 @@ struct RopeArgs {
     float sgn;       // +1 or -1 (already includes the backward flip)
     uint32_t bhtd;   // 0: [B,T,heads,D]; 1: [B,heads,T,D]
     uint32_t q_rows; // bhtd: B*H*T rows of D elements belong to q, the rest to k
+    FastDiv by_J, by_I, by_T;   // exact division by J, I and T_len
 };
 
 template <int VEC>
@@ -61,21 +62,19 @@ __global__ void __launch_bounds__(kRopeBlock) rope_kernel(const RopeArgs<T> a) {
         if (idx < a.total) {
             uint32_t t, j;
             if (a.bhtd) {                       // uniform over the launch
-                uint32_t row = idx / a.J;       // a row is one (batch, head, position)
-                j = idx - row * a.J;
+                uint32_t row = a.by_J.divmod(idx, j);       // a row is one (batch, head, position)
                 T* base = a.q;
                 if (row >= a.q_rows) { base = a.k; row -= a.q_rows; }
-                t = row % a.T_len;
+                a.by_T.divmod(row, t);
                 ptr[u] = base + (uint64_t)row * a.D + (uint64_t)j * VEC;
             } else {
-                const uint32_t token = idx / a.I;
-                uint32_t r = idx - token * a.I;
-                t = token % a.T_len;
+                uint32_t r;
+                const uint32_t token = a.by_I.divmod(idx, r);
+                a.by_T.divmod(token, t);
                 T* base;
                 uint32_t heads;
                 if (r < a.Iq) { base = a.q; heads = a.H; } else { base = a.k; heads = a.HKV; r -= a.Iq; }
-                const uint32_t head = r / a.J;
-                j = r - head * a.J;
+                const uint32_t head = a.by_J.divmod(r, j);
                 ptr[u] = base + ((uint64_t)token * heads + head) * a.D + (uint64_t)j * VEC;
             }
             VecIO<T, VEC>::load(ptr[u], lo[u]);
@@ -115,6 +114,9 @@ int rope_typed(hipStream_t s, RopeArgs<T> a, uint32_t B) {
     if (total >= 0xffff0000ull) return set_error(AGRAD_EINVAL, "rope: %llu work items exceed 32-bit indexing", (unsigned long long)total);
     a.total = (uint32_t)total;
     a.q_rows = B * a.T_len * a.H;
+    a.by_J = FastDiv(a.J);
+    a.by_I = FastDiv(a.I);
+    a.by_T = FastDiv(a.T_len);
     const uint32_t per_block = kRopeBlock * UNROLL;
     const uint32_t grid = (a.total + per_block - 1) / per_block;
     hipLaunchKernelGGL((rope_kernel<T, VEC, UNROLL>), dim3(grid), dim3(kRopeBlock), 0, s, a);

@@ -49,6 +49,19 @@ def test_header_compiles_as_plain_c(tmp_path):
     assert len(names) >= len(capi.SIGNATURES)
 
 
+def test_index_divider_matches_the_machines_division(tmp_path):
+    """The kernels split a flat index into (row, column) with a multiply-high divider prepared
+    on the host (csrc/fastdiv.hpp); tests/c_abi/fastdiv_check.cpp, compiled here with g++,
+    compares it with / and % over strides of all 32-bit dividends, edges and random pairs."""
+    import subprocess
+    exe = tmp_path / "fastdiv_check"
+    proc = subprocess.run(["g++", "-O2", "-std=c++17", f"-I{ROOT / 'autograd_amd' / 'csrc'}",
+                           str(ROOT / "tests" / "c_abi" / "fastdiv_check.cpp"), "-o", str(exe)], capture_output=True, text=True)
+    assert proc.returncode == 0, proc.stderr
+    proc = subprocess.run([str(exe)], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stdout + proc.stderr
+
+
 def test_library_reports_errors_without_gpu_or_kernel():
     lib = capi.load_library()
     assert lib.agrad_kernel_count() == 43
