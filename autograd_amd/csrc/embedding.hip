@@ -188,7 +188,8 @@ emb_prepare_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ keys,
 constexpr int kSortBlock = 512;
 constexpr uint32_t kGroupSortMaxN = 65536;
 constexpr uint32_t kSortLdsEntries = 3072;   // (token, row) pairs a workgroup keeps in LDS
-constexpr uint32_t kRankSortMax = kSortBlock;  // lists up to one key per thread are placed by rank
+constexpr uint32_t kRankSortMax = kSortBlock;  // lists up to one key per thread can be placed by rank ...
+constexpr uint32_t kRankDirect = kSortBlock / 2;    // ... and are, up to this many (two threads or more share a key's comparisons)
 constexpr uint32_t kRowMapWords = kGroupSortMaxN / 32;
 constexpr uint32_t kSortWaves = kSortBlock / kWave;
 static_assert(kRowMapWords % (2 * kSortWaves) == 0, "the waves share the row map in whole pairs of words");
@@ -425,14 +426,16 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
     const uint32_t count = s_count;
     const uint32_t offset = s_less;
 
-    if (count <= kRankSortMax) {
-        // Every key is unique, so its place in the order is the number of smaller keys.
-        // The threads share the counting: `parts` threads per key, each comparing the key
-        // with its slice of the list (broadcast LDS reads), their tallies added in LDS.
-        const uint32_t parts = count ? kSortBlock / count : 1u;     // threads per key
-        const uint32_t part = count ? tid / count : 0u, k = part < parts ? tid - part * count : count;
-        const uint32_t j_lo = (part * count) / parts, j_hi = k < count ? ((part + 1) * count) / parts : j_lo;
-        const unsigned long long mine = k < count ? keys[k] : ~0ull;
+    // The n <= kRankSortMax pairs of keys[], ranked by counting: every key is unique, so its
+    // place in the order is the number of smaller keys.  The threads share the counting:
+    // `parts` threads per key, each comparing the key with its slice of the list (broadcast
+    // LDS reads), their tallies added in LDS.  A pair of token t leaves for place
+    // offset + rank + shift(t).  (tally[] is zero on entry.)
+    auto rank_and_emit = [&](uint32_t n, auto shift) {
+        const uint32_t parts = n ? kSortBlock / n : 1u;             // threads per key
+        const uint32_t part = n ? tid / n : 0u, k = part < parts ? tid - part * n : n;
+        const uint32_t j_lo = (part * n) / parts, j_hi = k < n ? ((part + 1) * n) / parts : j_lo;
+        const unsigned long long mine = k < n ? keys[k] : ~0ull;
         const uint32_t my_tok = (uint32_t)(mine >> 32), my_row = (uint32_t)mine;
         uint32_t smaller_tok = 0, same = 0, same_before = 0;
 #pragma unroll 8
@@ -443,10 +446,10 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
             same += tok == my_tok ? 1u : 0u;
             same_before += (tok == my_tok && row < my_row) ? 1u : 0u;
         }
-        if (k < count) atomicAdd(&tally[k], smaller_tok | (same << 10) | (same_before << 20));
+        if (k < n) atomicAdd(&tally[k], smaller_tok | (same << 10) | (same_before << 20));
         __syncthreads();
         uint32_t rank = 0, run = 0, j = 0;
-        if (tid < count) {
+        if (tid < n) {
             const uint32_t packed = tally[tid];
             j = packed >> 20;
             run = (packed >> 10) & 1023u;
@@ -454,10 +457,16 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
             placed[rank] = (uint32_t)keys[tid];
         }
         __syncthreads();
-        if (tid < count) {
+        if (tid < n) {
             const uint32_t next = j + 1 < run ? placed[rank + 1] : kNoRow;
-            emit((uint32_t)(keys[tid] >> 32), (uint32_t)keys[tid], offset + rank, j, run, next);
+            const uint32_t tok = (uint32_t)(keys[tid] >> 32);
+            emit(tok, (uint32_t)keys[tid], offset + rank + shift(tok), j, run, next);
         }
+    };
+    // (up to kRankDirect pairs: beyond, a thread has hundreds of comparisons to make, and what
+    // makes a list that long is a frequent token, which the path below takes out first)
+    if (count <= kRankDirect) {
+        rank_and_emit(count, [](uint32_t) { return 0u; });
         return;
     }
 
@@ -504,28 +513,34 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
             split((uint32_t)(key >> 32), (uint32_t)key);
         }
     } else {
-        // a wave looks at 64 consecutive rows: two whole words of the map, stored
-        // once each, no atomics
-        constexpr int AGAIN = 8;
-        for (uint32_t base = 0; base < N; base += kSortBlock * AGAIN) {
-            int32_t t[AGAIN];
+        // four consecutive ids per 16-byte load, four loads in flight per thread; a thread ORs
+        // the marks of its four rows into the map's word (the rows of one load lie in one word)
+        constexpr int AGAIN = 4;
+        for (uint32_t base = 0; base < N; base += kSortBlock * AGAIN * 4) {
+            uint32_t t[AGAIN][4];
 #pragma unroll
             for (int r = 0; r < AGAIN; ++r) {
-                const uint32_t i = base + r * kSortBlock + tid;
-                t[r] = i < N ? ids[i] : -1;
+                const uint32_t row0 = base + ((uint32_t)r * kSortBlock + tid) * 4u;
+                if (wide_ids && row0 + 4 <= N) {
+                    const u32x4 q = *reinterpret_cast<const u32x4*>(ids + row0);
+                    t[r][0] = q.x; t[r][1] = q.y; t[r][2] = q.z; t[r][3] = q.w;
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) t[r][c] = row0 + c < N ? (uint32_t)ids[row0 + c] : 0u;
+                }
             }
 #pragma unroll
             for (int r = 0; r < AGAIN; ++r) {
-                const uint32_t i = base + r * kSortBlock + tid;      // below kGroupSortMaxN, also when >= N
-                uint32_t tok;
-                const bool own = owner_of(t[r], tok) == g && i < N;
-                const bool is_hot = own && tok == hot;
-                const unsigned long long marks = __ballot(is_hot);
-                if (i < kGroupSortMaxN) {
-                    if (lane == 0) row_map[i >> 5] = (uint32_t)marks;
-                    if (lane == 32) row_map[i >> 5] = (uint32_t)(marks >> 32);
+                const uint32_t row0 = base + ((uint32_t)r * kSortBlock + tid) * 4u;
+                uint32_t marks = 0;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    uint32_t tok;
+                    const bool own = row0 + c < N && owner_of((int32_t)t[r][c], tok) == g;
+                    if (own && tok == hot) marks |= 1u << c;
+                    else if (own) split(tok, row0 + c);
                 }
-                if (own && !is_hot) split(tok, i);
+                if (marks) atomicOr(&row_map[row0 >> 5], marks << (row0 & 31u));
             }
         }
     }
@@ -567,22 +582,34 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
 
     // -- the rest, in order; pairs above the frequent token leave room for its rows
     const uint32_t hot_rows = count - rest_n;
-    bitonic_sort_u64<kSortBlock>(rest, rest_n, tid, [] { __syncthreads(); });
     uint32_t n_below = 0;                          // pairs of the rest that sort before the frequent token
-    for (uint32_t i = tid; i < rest_n; i += kSortBlock) {
-        const uint32_t tok = (uint32_t)(rest[i] >> 32);
-        n_below += tok < hot ? 1u : 0u;
-        emit_sorted(rest, rest_n, i, tok > hot ? hot_rows : 0u);
+    if (rest_n <= kRankDirect) {
+        // a short rest: ranked by counting, as a short list is.  That wants the rest in keys[]
+        // and zero tallies: a rest split off the list in LDS sits in the tallies' bytes and
+        // moves over first (the list itself is not needed any more).
+        if (!reread) {
+            const unsigned long long pair = tid < rest_n ? few[tid] : 0ull;
+            __syncthreads();
+            if (tid < rest_n) keys[tid] = pair;
+            tally[tid] = 0;
+            __syncthreads();
+        }
+        if (tid < rest_n) n_below = (uint32_t)(keys[tid] >> 32) < hot ? 1u : 0u;
+        rank_and_emit(rest_n, [&](uint32_t tok) { return tok > hot ? hot_rows : 0u; });
+    } else {
+        bitonic_sort_u64<kSortBlock>(rest, rest_n, tid, [] { __syncthreads(); });
+        for (uint32_t i = tid; i < rest_n; i += kSortBlock) {
+            const uint32_t tok = (uint32_t)(rest[i] >> 32);
+            n_below += tok < hot ? 1u : 0u;
+            emit_sorted(rest, rest_n, i, tok > hot ? hot_rows : 0u);
+        }
     }
     if (n_below) atomicAdd(&s_below, n_below);
     __syncthreads();
     const uint32_t below = s_below;
 
     // -- the frequent token's rows.  Word w of the map holds rows 32 w ... 32 w + 31.
-    // The waves share the words that rows below N can mark, an even number each;
-    // a wave takes its words two at a time: each half-wave gives one word's 32
-    // rows a lane each, and a marked row's place is the count of marks before it,
-    // so a store instruction writes up to 64 neighbouring entries.
+    // The waves share the words that rows below N can mark, an even number each.
     const uint32_t wave = tid / kWave;
     const uint32_t words = (N + 31) / 32;
     const uint32_t per_wave = ((words + kSortWaves - 1) / kSortWaves + 1) & ~1u;     // at most kRowMapWords / kSortWaves
@@ -601,18 +628,51 @@ emb_group_sort_body(uint32_t g, const int32_t* __restrict__ ids, uint32_t* __res
     __syncthreads();
     uint32_t at = offset + below;
     for (uint32_t w = 0; w < wave; ++w) at += s_wave_rows[w];
-    if (s_wave_rows[wave] == 0) return;
-    const uint32_t upper = lane >> 5, bit = lane & 31u;
+    const uint32_t mine_rows = s_wave_rows[wave];
+    if (mine_rows == 0) return;
+    if (mine_rows * 4u >= per_wave * 32u) {
+        // Many marks (a quarter of the wave's rows or more): the wave takes its words two at a
+        // time, each half-wave gives one word's 32 rows a lane each, and a marked row's place
+        // is the count of marks before it, so a store instruction writes up to 64
+        // neighbouring entries.
+        const uint32_t upper = lane >> 5, bit = lane & 31u;
 #pragma nounroll
-    for (uint32_t w0 = w_begin; w0 < w_begin + per_wave; w0 += 2) {
-        const uint32_t word0 = row_map[w0], word1 = row_map[w0 + 1];
-        const uint32_t n0 = (uint32_t)__popc(word0);
-        const uint32_t word = upper ? word1 : word0;
-        if ((word >> bit) & 1u) {
-            const uint32_t to = at + (upper ? n0 : 0u) + (uint32_t)__popc(word & ((1u << bit) - 1u));
-            emit(hot, (w0 + upper) * 32u + bit, to, to - (offset + below), hot_rows, kNoRow);
+        for (uint32_t w0 = w_begin; w0 < w_begin + per_wave; w0 += 2) {
+            const uint32_t word0 = row_map[w0], word1 = row_map[w0 + 1];
+            const uint32_t n0 = (uint32_t)__popc(word0);
+            const uint32_t word = upper ? word1 : word0;
+            if ((word >> bit) & 1u) {
+                const uint32_t to = at + (upper ? n0 : 0u) + (uint32_t)__popc(word & ((1u << bit) - 1u));
+                emit(hot, (w0 + upper) * 32u + bit, to, to - (offset + below), hot_rows, kNoRow);
+            }
+            at += n0 + (uint32_t)__popc(word1);
         }
-        at += n0 + (uint32_t)__popc(word1);
+        return;
+    }
+    // Few marks: a pass over all the wave's rows would mostly find nothing (two thousand rows
+    // of a token among 65536 are four marks a word).  The wave takes 64 words at a time, a
+    // lane each; the lanes' mark counts are summed up across the wave (with every lane
+    // active), and each lane then walks the marks of its own word.
+#pragma nounroll
+    for (uint32_t w0 = w_begin; w0 < w_begin + per_wave; w0 += kWave) {
+        const uint32_t w = w0 + lane;
+        uint32_t word = w < w_begin + per_wave ? row_map[w] : 0u;
+        const uint32_t n = (uint32_t)__popc(word);
+        uint32_t upto = n;                                  // marks in this lane's word and the lanes' before it
+#pragma unroll
+        for (int d = 1; d < kWave; d *= 2) {
+            const uint32_t other = (uint32_t)__shfl_up((int)upto, d, kWave);
+            if (lane >= (uint32_t)d) upto += other;
+        }
+        const uint32_t total = (uint32_t)__builtin_amdgcn_readlane((int)upto, kWave - 1);
+        uint32_t to = at + upto - n;
+        while (word != 0) {
+            const uint32_t bit = (uint32_t)__builtin_ctz(word);
+            word &= word - 1u;
+            emit(hot, w * 32u + bit, to, to - (offset + below), hot_rows, kNoRow);
+            ++to;
+        }
+        at += total;
     }
 }
 
