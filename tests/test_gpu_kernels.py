@@ -1075,19 +1075,25 @@ def _same_group_tokens(V, how_many, N):
 
 
 _SKEWED = {
-    # name: (N, [(rows of a token, how many such tokens)...] all within one hash group, rest of N uniform)
+    # name: (N, [(rows of a token, how many such tokens)...] all within one hash group, rest of N uniform:
+    # about 125 more pairs in the group at 16384 rows, 64 at 8192)
     "all_rows_one_token": (16384, [(16384, 1)]),
-    "padding_third": (16384, [(5500, 1)]),
+    "padding_third": (16384, [(5500, 1)]),                    # ids read again; dense map: two words a wave and step
     "two_tokens_split": (16384, [(8192, 2)]),                 # what is left after the frequent one exceeds LDS
-    "frequent_plus_few": (16384, [(5000, 1), (3, 100)]),      # ids read again, the rest placed by rank
+    "frequent_plus_few": (16384, [(5000, 1), (2, 50)]),       # ids read again, the rest (under 257 pairs) placed by rank
+    "frequent_plus_some": (16384, [(5000, 1), (3, 100)]),     # ids read again, the rest (257 .. 3072) through the network
     "frequent_plus_many": (16384, [(5000, 1), (20, 100)]),    # ids read again, the rest through the network
-    "listed_frequent_plus_few": (8192, [(1500, 1), (2, 100)]),   # list fits LDS, the rest placed by rank
+    "listed_frequent_plus_few": (8192, [(1500, 1), (2, 60)]),    # list fits LDS, the rest moves over and is placed by rank
+    "listed_frequent_plus_some": (8192, [(1500, 1), (2, 150)]),  # list fits LDS, the rest (257 .. 512) through the network
     "listed_no_frequent": (8192, [(400, 3)]),                 # list fits LDS, no single frequent token
+    "list_of_300_pairs": (16384, [(200, 1)]),                 # 257 .. 512 pairs: the frequent-token way, a sparse map
+    "medium_token": (16384, [(900, 1)]),                      # a sparse map: each lane walks the marks of its own word
+    "frequent_in_one_stretch": (16384, [(2048, 1)]),          # its rows are rows 0 .. 2047: one wave's words dense, the others' empty
     "short_input": (1500, [(1400, 1)]),                       # fewer rows than the row map has bits
     "most_rows_one_token_64k": (65536, [(60000, 1)]),         # 512 groups, every word of the row map
     "padding_40k": (40001, [(15000, 1), (3, 40)]),            # 512 groups, a ragged last word
     "padding_20k": (20001, [(7000, 1), (3, 80)]),             # 256 groups
-    "two_frequent_one_group_64k": (65536, [(9000, 1), (1500, 1), (2, 50)]),
+    "two_frequent_one_group_64k": (65536, [(9000, 1), (1500, 1), (2, 50)]),     # a sparse map of 2048 words
     "bad_ids_frequent": (4096, [(0, 1)]),                     # out-of-range ids (one sentinel token) dominate
 }
 
@@ -1108,7 +1114,7 @@ def test_id_ordering_with_frequent_tokens(ctx, case):
         ids[rng.permutation(N)[:3000]] = -5
     else:
         same = _same_group_tokens(V, sum(k for _, k in spec), N)
-        slots = rng.permutation(N)
+        slots = np.arange(N) if case == "frequent_in_one_stretch" else rng.permutation(N)
         at = t = 0
         for rows, k in spec:
             for _ in range(k):
