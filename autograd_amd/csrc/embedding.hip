@@ -11,11 +11,12 @@
 //      tokens, scans all ids for its own, and orders its pairs in LDS (runs of
 //      distinct tokens then follow hash-group order, which is all the next step
 //      needs).  Larger inputs take a stable LSD radix sort by token (rocPRIM);
-//   2. one launch walks dY in row order: the first row of a token's run adds the
-//      run's rows in ascending order and stores the table row; a long run (a
-//      frequent token) is cut into chunks of rows whose sums pass through the
-//      workspace and are added in chunk order by the wave that an arrival counter
-//      names the last of its group.  Every table row is written once.
+//   2. one launch reads dY once: a token's only row is moved by a wave of its own; the
+//      rows of a run are added in ascending order by one wave per column block (the
+//      ordering marks where runs start, and waves at the front of the grid look for
+//      the marks); a long run (a frequent token) is cut into chunks of rows whose sums
+//      pass through the workspace and are added in chunk order by the wave that an
+//      arrival counter names the last of its group.  Every table row is written once.
 // Every sum has a fixed order, so the result is run-to-run identical, and runs of
 // up to 127 rows are bit-identical to the sequential CPU sum.
 #include "common.hpp"
