@@ -1320,9 +1320,9 @@ uint64_t embedding_sort_workspace_bytes(uint64_t N, uint32_t V) {
     return p.total;
 }
 
-// order[0 .. N) = rows, each token's rows adjacent and ascending; then (from the next
-// multiple of four words) four words per row: its token, where its token's run starts,
-// its index in the run and the run's length
+// order[0 .. N) = rows (with the task marks in their top two bits), each token's rows
+// adjacent and ascending; then (from the next multiple of four words) a RunInfo per row;
+// then the gradient kernel's arrival counters, zeroed
 int launch_embedding_sort(hipStream_t s, const int32_t* ids, uint32_t* order, void* workspace,
                           uint64_t workspace_bytes, uint64_t N, uint32_t V, int* err_flag) {
     if (N == 0) return AGRAD_OK;
