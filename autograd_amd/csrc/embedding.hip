@@ -741,13 +741,14 @@ gather_sort_kernel(const int32_t* __restrict__ ids, const T* __restrict__ W, con
         for (int u = 0; u < kGatherPerThread; ++u)
             if ((uint32_t)tok[u] < V) __builtin_nontemporal_store(v[u], reinterpret_cast<u32x4*>(out) + first + u * kSortBlock);
     } else {
+        // (the position rows do not wait for the ids: asked for first, from a valid row whatever the id)
         float v[kGatherPerThread][VEC], p[kGatherPerThread][VEC];
 #pragma unroll
+        for (int u = 0; u < kGatherPerThread; ++u)
+            VecIO<T, VEC>::load(wpe + (uint64_t)(row[u] % T_len) * C + cv[u] * VEC, p[u]);
+#pragma unroll
         for (int u = 0; u < kGatherPerThread; ++u) {
-            if ((uint32_t)tok[u] < V) {
-                VecIO<T, VEC>::load(W + (uint64_t)tok[u] * C + cv[u] * VEC, v[u]);
-                VecIO<T, VEC>::load(wpe + (uint64_t)(row[u] % T_len) * C + cv[u] * VEC, p[u]);
-            }
+            if ((uint32_t)tok[u] < V) VecIO<T, VEC>::load(W + (uint64_t)tok[u] * C + cv[u] * VEC, v[u]);
         }
 #pragma unroll
         for (int u = 0; u < kGatherPerThread; ++u) {
