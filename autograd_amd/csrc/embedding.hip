@@ -51,7 +51,7 @@ gather_fwd_kernel(const int32_t* __restrict__ ids, const T* __restrict__ W, cons
         const uint32_t idx = first + u * kGatherBlock;
         tok[u] = -1;
         rows[u] = 0;
-        col[u] = 1;
+        col[u] = 0;
         if (idx < total) {
             rows[u] = idx / CV;
             col[u] = (idx - rows[u] * CV) * VEC;
@@ -60,13 +60,17 @@ gather_fwd_kernel(const int32_t* __restrict__ ids, const T* __restrict__ W, cons
     }
     float v[UNROLL][VEC], p[UNROLL][VEC];
     bool ok[UNROLL];
+    // (the position rows do not wait for the ids: asked for first, from a valid row whatever the id)
+    if (wpe != nullptr) {
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) VecIO<T, VEC>::load(wpe + (uint64_t)(rows[u] % T_len) * C + col[u], p[u]);
+    }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
         const uint32_t idx = first + u * kGatherBlock;
         ok[u] = idx < total && tok[u] >= 0 && (uint32_t)tok[u] < V;
         if (ok[u]) {
             VecIO<T, VEC>::load(W + (uint64_t)tok[u] * C + col[u], v[u]);
-            if (wpe != nullptr) VecIO<T, VEC>::load(wpe + (uint64_t)(rows[u] % T_len) * C + col[u], p[u]);
         } else if (idx < total && col[u] == 0) {
             *err_flag = 1;
         }
