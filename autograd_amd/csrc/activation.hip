@@ -143,6 +143,16 @@ swiglu_bwd_kernel(const T* gu, const T* __restrict__ dh, T* dgu, uint32_t H, uin
     }
 }
 
+// The backward kernel has five streams (gate, up and dh in; dgate and dup out), and with
+// every wave slot of the GPU filled they reach 0.91 of what a two-stream copy reaches: the
+// more loads and stores of five streams are in flight at once, the more DRAM pages they keep
+// open against each other.  Dynamic LDS that the kernel never touches caps the workgroups
+// (one wave each) of a CU at sixteen instead of thirty-two: 65536 x 14336 bf16 1513 -> 1400
+// us, 16384 x 8960 fp32 469 -> 451 us, bf16 225 -> 220 us.  (Eight: 20 % slower -- the
+// sigmoid needs waves to hide behind.  The forward kernel, three streams, gains nothing, and
+// the two- and three-stream elementwise kernels lose from any cap.)
+constexpr unsigned kSwigluBwdIdleLds = 10 * 1024;
+
 // Rows are processed in slabs small enough for 32-bit vector indices.
 template <typename T, int VEC>
 int swiglu_typed(hipStream_t s, const T* gu, const T* dh, T* out, uint64_t rows, uint32_t H,
@@ -160,7 +170,7 @@ int swiglu_typed(hipStream_t s, const T* gu, const T* dh, T* out, uint64_t rows,
             hipLaunchKernelGGL((swiglu_fwd_kernel<T, VEC, UNROLL>), dim3(grid), dim3(kEwBlock), 0, s,
                                gu + r0 * 2 * H, out + r0 * hw, H, h0, HV, nvec);
         } else {
-            hipLaunchKernelGGL((swiglu_bwd_kernel<T, VEC, UNROLL>), dim3(grid), dim3(kEwBlock), 0, s,
+            hipLaunchKernelGGL((swiglu_bwd_kernel<T, VEC, UNROLL>), dim3(grid), dim3(kEwBlock), VEC > 1 ? kSwigluBwdIdleLds : 0u, s,
                                gu + r0 * 2 * H, dh + r0 * H, out + r0 * 2 * H, H, HV, nvec, acc);
         }
     }
