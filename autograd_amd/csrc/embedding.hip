@@ -785,14 +785,16 @@ __device__ __forceinline__ void store_grad_row(T* dW, uint64_t off, const float 
 // ROWS.  A wave takes one row of dY and KW neighbouring blocks of 64 column vectors (the
 // whole row when it has up to KW blocks); one 16-byte scalar load tells it what the row is
 // (RunInfo).  A row that is its token's only row moves its vectors to the table -- most rows
-// do -- and every other row ends there.  With a position table a workgroup takes one
-// position t and column block, its waves the rows b*T + t of the batch; besides the above
-// they leave their vectors in LDS, where wave 0 adds them in ascending b:
-// dwpe[t, :] (+)= sum_b dY[b, t, :].
+// do; where a wave takes one column block (KW = 1), the first row of a run of up to
+// kRowRunMax rows also adds that run itself; every other row ends there.  With a position
+// table a workgroup takes one position t and column block, its waves the rows b*T + t of
+// the batch; besides the above they leave their vectors in LDS, where wave 0 adds them in
+// ascending b: dwpe[t, :] (+)= sum_b dY[b, t, :].
 //
 // TASKS, at the FRONT of the grid so that they are under way while the rest walks the rows.
-// A wave searches kTaskSpan places of row_s[] for marked rows and takes ONE column block of
-// every one found (TaskGrid):
+// A wave searches kTaskSpan or kBigTaskSpan places of row_s[] for marked rows and takes ONE
+// column block of every one found (TaskGrid; the tasks of more than kRowRunMax rows carry a
+// second mark and, where the rows leave all runs to the tasks, go first):
 //   * the first row of a run of 2 .. kSoloRun rows: the wave adds the run's rows in
 //     ascending order -- the very sequence of fp32 adds np.add.at makes -- and stores the
 //     table row;
