@@ -305,10 +305,14 @@ norm_fwd_kernel(const NormFwdArgs<T> a) {
 // ----------------------------------------------------------------------------
 // backward, register-resident row, dgamma / dbeta partials per workgroup
 // ----------------------------------------------------------------------------
+// Threads of a backward workgroup whose rows take a wave or less each (512 and 1024, with a
+// half and a quarter of the partial rows, were measured: within 1 us either way at 16384 rows).
+constexpr int kBwdGroupBlock = 256;
+
 template <typename T, int VEC, int NV, int TPR>
-__global__ void __launch_bounds__(TPR >= 128 ? TPR : 256)
+__global__ void __launch_bounds__(TPR >= 128 ? TPR : kBwdGroupBlock)
 norm_bwd_kernel(const NormBwdArgs<T> a) {
-    constexpr int BLOCK = TPR >= 128 ? TPR : 256;
+    constexpr int BLOCK = TPR >= 128 ? TPR : kBwdGroupBlock;
     constexpr int RPB = BLOCK / TPR;
     constexpr int NWAVES = BLOCK / kWave;
     __shared__ float lds[3 * kRowSumSlot * (TPR > kWave ? TPR / kWave : 1)];
@@ -696,7 +700,7 @@ NormPlan plan_norm(uint32_t C, int dtype, bool aligned, bool backward) {
             p.generic = false;
             p.tpr = t;
             p.nv = (int)nv;
-            p.rpb = t >= 128 ? 1 : (backward ? 256 : kFwdGroupBlock) / t;
+            p.rpb = t >= 128 ? 1 : (backward ? kBwdGroupBlock : kFwdGroupBlock) / t;
             return p;
         }
     }
@@ -730,7 +734,7 @@ uint32_t cu_count() {
 
 template <int TPR>
 inline size_t bwd_dyn_lds(const NormPlan& p, uint32_t C) {
-    constexpr int BLOCK = TPR >= 128 ? TPR : 256;
+    constexpr int BLOCK = TPR >= 128 ? TPR : kBwdGroupBlock;
     return p.rpb > 1 ? (size_t)(BLOCK / kWave - 1) * C * sizeof(float) : 0;
 }
 
@@ -775,7 +779,7 @@ int fwd_pick_nv(hipStream_t s, const NormPlan& p, const NormFwdArgs<T>& a) {
 
 template <typename T, int VEC, int TPR>
 int bwd_pick_nv(hipStream_t s, const NormPlan& p, const NormBwdArgs<T>& a, uint32_t grid) {
-    constexpr int BLOCK = TPR >= 128 ? TPR : 256;
+    constexpr int BLOCK = TPR >= 128 ? TPR : kBwdGroupBlock;
     const size_t dyn = bwd_dyn_lds<TPR>(p, a.C);
     switch (p.nv) {
 #define AGRAD_CASE(N)                                                                  \
@@ -794,7 +798,7 @@ int bwd_pick_nv(hipStream_t s, const NormPlan& p, const NormBwdArgs<T>& a, uint3
 // workgroups of the chosen backward instantiation the GPU holds at once (0: unknown)
 template <typename T, int VEC, int TPR>
 uint32_t bwd_resident_nv(const NormPlan& p, uint32_t C) {
-    constexpr int BLOCK = TPR >= 128 ? TPR : 256;
+    constexpr int BLOCK = TPR >= 128 ? TPR : kBwdGroupBlock;
     const size_t dyn = bwd_dyn_lds<TPR>(p, C);
     int per_cu = 0;
     switch (p.nv) {
