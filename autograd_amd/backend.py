@@ -37,7 +37,7 @@ from .utils import (bf16_bits, bf16_bits_to_f32_array, contiguous_strides, f32_a
                     is_bf16, mul_bcast_kind, storage_dtype, xavier_uniform)
 
 F32, BF16 = 0, 1
-ACC_INPUT_GRAD, ACC_PARAM_GRAD, ACC_INPUT_GRAD2, ACC_PARAM_GRAD2, PARAM_GRAD_BF16 = 1, 2, 4, 8, 16
+ACC_INPUT_GRAD, ACC_PARAM_GRAD, ACC_INPUT_GRAD2, ACC_PARAM_GRAD2, PARAM_GRAD_BF16, DEFER_PARAM_GRAD = 1, 2, 4, 8, 16, 32
 UNARY_OPS = {ExpOp: 0, LogOp: 1, RsqrtOp: 2}
 MUL_KINDS = {"same": 0, "row": 1, "col": 2, "scalar": 3}
 
@@ -132,6 +132,7 @@ def _mask(*present):
 
 class HipBackend(Backend):
     supports_grad_store = True   # kernels take a store / accumulate flag per gradient
+    supports_deferred_param_grads = True    # column sums of a pass can be folded in one launch at its end
 
     def __init__(self, ctx=None):
         if ctx is None:
@@ -227,6 +228,32 @@ class HipBackend(Backend):
         if t.op is None:
             return ACC_INPUT_GRAD if self._param_flag(node, t) else 0
         return self._input_flag(node, t)
+
+    # -- column sums folded at the end of the pass ---------------------------------------
+    def can_defer_param_grads(self, node):
+        """True if this node's backward kernel ends in a column-sum fold whose results
+        only parameters receive (nobody reads a parameter gradient before the pass ends)"""
+        op = node.op
+        if isinstance(op, (LayerNormOp, RMSNormOp, AddLayerNormOp, AddRMSNormOp)):
+            first = 2 if isinstance(op, (AddLayerNormOp, AddRMSNormOp)) else 1
+            params = [p for p in node.inputs[first:] if p.requires_grad]
+            return bool(params) and all(p.op is None for p in params)
+        if isinstance(op, BiasGELUOp):
+            b = node.inputs[1]
+            return b.requires_grad and b.op is None
+        if isinstance(op, AddOp):
+            out = node.outputs[0]
+            small = [t for t in node.inputs[:2] if t.requires_grad and t.shape != out.shape]
+            return bool(small) and all(t.op is None for t in small)
+        return False
+
+    @staticmethod
+    def _defer_flag(node):
+        return DEFER_PARAM_GRAD if getattr(node, "defer_param_grads", False) else 0
+
+    def finalize_param_grads(self):
+        """fold every column sum the backward kernels of this pass left pending (one launch)"""
+        self.ctx.finalize_param_grads()
 
     # -- scratch -----------------------------------------------------------------
     def _check_gradient_storage(self, node):
@@ -337,7 +364,7 @@ class HipBackend(Backend):
                                                         or (_dt(out.grad) == F32 and _dt(t.grad) == BF16)):
                 inner = t.numel
                 lead = out.numel // max(inner, 1)
-                flag = ACC_PARAM_GRAD if self._grad_flag(node, t) else 0
+                flag = (ACC_PARAM_GRAD if self._grad_flag(node, t) else 0) | self._defer_flag(node)
                 if _dt(t.grad) != _dt(out.grad):
                     flag |= PARAM_GRAD_BF16       # a bf16 bias gradient under fp32 activations
                 ws = scratch["workspace"] if scratch and "workspace" in scratch else None
@@ -632,6 +659,7 @@ class HipBackend(Backend):
             ws_bytes = ws.nbytes
             if self._grad_flag(node, b):
                 flags |= ACC_PARAM_GRAD
+            flags |= self._defer_flag(node)
             if _dt(db) != _dt(h):
                 flags |= PARAM_GRAD_BF16          # planning has checked that this is bf16 under fp32
         self._launch("gelu_backward_bias_kernel", [out.grad, h, b, dh, db, ws],
@@ -675,6 +703,7 @@ class HipBackend(Backend):
             flags |= PARAM_GRAD_BF16
         ws = None
         if dgamma is not None or dbeta is not None:
+            flags |= self._defer_flag(node)
             if scratch is None:
                 raise RuntimeError("norm backward needs its arena workspace (plan_scratch)")
             ws = scratch["workspace"]

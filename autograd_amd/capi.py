@@ -17,11 +17,17 @@ LIB_PATH = Path(__file__).resolve().parent / "libautograd_hip.so"
 
 F32, BF16 = 0, 1
 NORM_LAYER, NORM_RMS = 0, 1
-ACC_INPUT_GRAD, ACC_PARAM_GRAD, ACC_INPUT_GRAD2, ACC_PARAM_GRAD2, PARAM_GRAD_BF16 = 1, 2, 4, 8, 16
+ACC_INPUT_GRAD, ACC_PARAM_GRAD, ACC_INPUT_GRAD2, ACC_PARAM_GRAD2, PARAM_GRAD_BF16, DEFER_PARAM_GRAD = 1, 2, 4, 8, 16, 32
 UNARY_EXP, UNARY_LOG, UNARY_RSQRT = 0, 1, 2
 MUL_SAME, MUL_ROW, MUL_COL, MUL_SCALAR = 0, 1, 2, 3
 OK, EINVAL, EHIP, ENOKERNEL, EINDEX, EWORKSPACE = 0, -1, -2, -3, -4, -5
 NOALLOC_SCRATCH_BYTES = 32 << 20
+
+class ColsumJob(C.Structure):
+    """agrad_colsum_job: one column sum that is still to be folded"""
+    _fields_ = [("partial_a", C.c_void_p), ("partial_b", C.c_void_p), ("out_a", C.c_void_p), ("out_b", C.c_void_p),
+                ("partial_rows", C.c_uint32), ("C", C.c_uint32), ("flags", C.c_uint32), ("reserved", C.c_uint32)]
+
 
 _ctx = C.c_void_p
 _ptr = C.c_void_p
@@ -64,6 +70,11 @@ SIGNATURES = {
                                    _ptr, _u64, _u64, _u32, _f32, _u32]),
     "agrad_norm_backward_noalloc": (_int, [_ctx, _int, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
                                            _u64, _u32, _f32, _u32]),
+    "agrad_pending_param_grads": (_int, [_ctx, C.POINTER(_u32)]),
+    "agrad_finalize_param_grads": (_int, [_ctx]),
+    "agrad_colsum_finalize_many": (_int, [_ctx, _ptr, _u32]),
+    "agrad_norm_backward_partial": (_int, [_ctx, _int, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr,
+                                           _ptr, _u64, _u64, _u32, _f32, _u32, _ptr]),
     "agrad_gelu_forward": (_int, [_ctx, _int, _ptr, _ptr, _u64]),
     "agrad_gelu_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _u64, _u32]),
     "agrad_gelu_bias_forward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _u64, _u32]),

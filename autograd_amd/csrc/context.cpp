@@ -24,6 +24,9 @@ struct agrad_ctx {
     bool capturing = false;                // between agrad_graph_begin and agrad_graph_end
     std::map<uint64_t, hipGraphExec_t> graphs;
     uint64_t next_graph = 1;
+    // column sums (dgamma / dbeta, bias gradients) that backward calls with AGRAD_DEFER_PARAM_GRAD
+    // left unfolded: their partial rows wait in the callers' workspaces for agrad_finalize_param_grads
+    std::vector<agrad::ColsumJob> pending;
 };
 
 namespace agrad {
@@ -82,8 +85,23 @@ int no_capture(agrad_ctx* ctx, const char* what) {
     return AGRAD_OK;
 }
 
+// folds every pending column sum (one launch per kFinalizeManyJobs of them)
+int flush_pending(agrad_ctx* ctx) {
+    if (ctx->pending.empty()) return AGRAD_OK;
+    const int rc = launch_colsum_finalize_many(ctx->stream, ctx->pending.data(), ctx->pending.size());
+    ctx->pending.clear();
+    return rc;
+}
+
+// a backward entry point's scope: with AGRAD_DEFER_PARAM_GRAD in its flags, the finalize
+// launches it would make are appended to the context's pending list instead
+struct DeferScope : ColsumDefer {
+    DeferScope(agrad_ctx* ctx, uint32_t flags) : ColsumDefer((flags & AGRAD_DEFER_PARAM_GRAD) ? &ctx->pending : nullptr) {}
+};
+
 int finish_stream(agrad_ctx* ctx) {
     if (int rc = no_capture(ctx, "synchronize / end_pass")) return rc;
+    if (int rc = flush_pending(ctx)) return rc;      // nothing a caller waits for stays unfolded
     if (int rc = check_hip(hipStreamSynchronize(ctx->stream), "stream synchronize")) return rc;
     int flag = 0;
     if (int rc = check_hip(hipMemcpy(&flag, ctx->err_flag, sizeof(int), hipMemcpyDeviceToHost), "error flag read")) return rc;
@@ -168,6 +186,7 @@ int h_bcast_grad(const Call& c) {
     const uint64_t lead = u64(c.a, 1), inner = u64(c.a, 3), es = dtype_size(c.a[0]), wsb = u64(c.a, 6);
     RESOLVE(0, lead * inner * es, g) RESOLVE(1, inner * ((c.a[5] & AGRAD_PARAM_GRAD_BF16) ? 2 : es), dy)
     RESOLVE_IF(c.a[8] & 4u, 2, wsb, ws)
+    DeferScope defer(c.ctx, c.a[5]);
     return launch_broadcast_grad(c.ctx->stream, (int)c.a[0], g, dy, ws, ws ? wsb : 0, lead, inner, c.a[5]);
 }
 // buffers x, y | args dtype, op, n lo, hi
@@ -206,6 +225,7 @@ int h_mul_bwd(const Call& c) {
     RESOLVE_IF(mask & 2u, 1, big, x) RESOLVE_IF(mask & 4u, 2, small, y)
     RESOLVE_IF(mask & 8u, 3, big, dx) RESOLVE_IF(mask & 16u, 4, small, dy)
     RESOLVE_IF(mask & 32u, 5, wsb, ws)
+    DeferScope defer(c.ctx, c.a[6]);
     return launch_mul_bwd(c.ctx->stream, (int)c.a[0], (int)c.a[1], g, x, y, dx, dy, ws, ws ? wsb : 0, lead, inner, c.a[6]);
 }
 // buffers x, y | args dtype, rows lo, hi, V
@@ -288,6 +308,7 @@ int h_norm_bwd(const Call& c) {
     RESOLVE_IF(present & 64u, 6, gpar, dgamma)
     RESOLVE_IF(present & 128u, 7, gpar, dbeta)
     RESOLVE_IF(present & 256u, 8, ws_bytes, ws)
+    DeferScope defer(c.ctx, flags);
     return launch_norm_bwd(c.ctx->stream, KIND, c.a[0], x, dy, (const float*)gamma, dres, dx, dx2,
                            (float*)dgamma, (float*)dbeta, ws, ws ? ws_bytes : 0, rows, C, f32(c.a[3]), flags);
 }
@@ -325,6 +346,7 @@ int h_gelu_bias_bwd(const Call& c) {
     const uint64_t big = rows * c.a[3] * es, small = (uint64_t)c.a[3] * es;
     RESOLVE(0, big, dy) RESOLVE(1, big, h) RESOLVE(2, small, b) RESOLVE_IF(c.a[7] & 8u, 3, big, dh)
     RESOLVE_IF(c.a[7] & 16u, 4, (c.a[4] & AGRAD_PARAM_GRAD_BF16) ? (uint64_t)c.a[3] * 2 : small, db) RESOLVE_IF(c.a[7] & 32u, 5, wsb, ws)
+    DeferScope defer(c.ctx, c.a[4]);
     return launch_gelu_bias_bwd(c.ctx->stream, (int)c.a[0], dy, h, b, dh, db, ws, ws ? wsb : 0, rows, c.a[3], c.a[4]);
 }
 // buffers gu, h | args dtype, rows, H
@@ -692,6 +714,7 @@ int agrad_timer_stop(agrad_ctx* ctx, float* elapsed_ms) {
 int agrad_graph_begin(agrad_ctx* ctx) {
     CTX_OR_FAIL(ctx)
     if (ctx->capturing) return set_error(AGRAD_EINVAL, "graph capture is already open");
+    if (int rc = flush_pending(ctx)) return rc;     // what was left pending before the recording is not part of it
     // relaxed mode: allocations and queries made by other code meanwhile stay legal
     if (int rc = check_hip(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed), "hipStreamBeginCapture")) return rc;
     ctx->capturing = true;
@@ -704,10 +727,12 @@ int agrad_graph_end(agrad_ctx* ctx, uint64_t* graph_id) {
     if (graph_id == nullptr) return set_error(AGRAD_EINVAL, "null out pointer");
     *graph_id = 0;
     if (!ctx->capturing) return set_error(AGRAD_EINVAL, "no graph capture is open");
+    const int flush_rc = flush_pending(ctx);       // column sums left pending inside the recording are folded inside it
     ctx->capturing = false;
     set_capturing(false);
     hipGraph_t graph = nullptr;
     if (int rc = check_hip(hipStreamEndCapture(ctx->stream, &graph), "hipStreamEndCapture")) return rc;
+    if (flush_rc != AGRAD_OK) { if (graph) (void)hipGraphDestroy(graph); return flush_rc; }
     if (graph == nullptr) return set_error(AGRAD_EHIP, "graph capture was invalidated");
     hipGraphExec_t exec = nullptr;
     const hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
@@ -806,6 +831,7 @@ int agrad_mul_backward(agrad_ctx* ctx, int dtype, int kind, const void* g, const
                        void* dy, void* workspace, uint64_t workspace_bytes, uint64_t lead, uint64_t inner,
                        uint32_t flags) {
     CTX_OR_FAIL(ctx)
+    DeferScope defer(ctx, flags);
     return launch_mul_bwd(ctx->stream, dtype, kind, g, x, y, dx, dy, workspace, workspace_bytes, lead, inner, flags);
 }
 int agrad_softmax_forward(agrad_ctx* ctx, int dtype, const void* x, void* y, uint64_t rows, uint32_t V) {
@@ -846,6 +872,7 @@ int agrad_norm_backward(agrad_ctx* ctx, int kind, int dtype, const void* x, cons
                         float* dgamma, float* dbeta, void* workspace, uint64_t workspace_bytes,
                         uint64_t rows, uint32_t C, float eps, uint32_t flags) {
     CTX_OR_FAIL(ctx)
+    DeferScope defer(ctx, flags);
     return launch_norm_bwd(ctx->stream, kind, dtype, x, dy, gamma, dres_in, dx, dx2, dgamma, dbeta,
                            workspace, workspace_bytes, rows, C, eps, flags);
 }
@@ -853,8 +880,59 @@ int agrad_norm_backward_noalloc(agrad_ctx* ctx, int kind, int dtype, const void*
                                 const float* gamma, const void* dres_in, void* dx, void* dx2,
                                 float* dgamma, float* dbeta, uint64_t rows, uint32_t C, float eps, uint32_t flags) {
     CTX_OR_FAIL(ctx)
+    if (flags & AGRAD_DEFER_PARAM_GRAD)
+        return set_error(AGRAD_EINVAL, "norm backward (no allocation): the partial rows share one fixed array, so the "
+                                       "column sums cannot be left pending (AGRAD_DEFER_PARAM_GRAD)");
     return launch_norm_bwd_noalloc(ctx->stream, ctx->device, kind, dtype, x, dy, gamma, dres_in, dx, dx2,
                                    dgamma, dbeta, rows, C, eps, flags);
+}
+
+int agrad_pending_param_grads(agrad_ctx* ctx, uint32_t* count) {
+    CTX_OR_FAIL(ctx)
+    if (count == nullptr) return set_error(AGRAD_EINVAL, "null out pointer");
+    *count = (uint32_t)ctx->pending.size();
+    return AGRAD_OK;
+}
+int agrad_finalize_param_grads(agrad_ctx* ctx) {
+    CTX_OR_FAIL(ctx)
+    return flush_pending(ctx);
+}
+int agrad_colsum_finalize_many(agrad_ctx* ctx, const agrad_colsum_job* jobs, uint32_t n_jobs) {
+    CTX_OR_FAIL(ctx)
+    if (n_jobs == 0) return AGRAD_OK;
+    if (jobs == nullptr) return set_error(AGRAD_EINVAL, "column-sum finalize: null job list");
+    std::vector<ColsumJob> list(n_jobs);
+    for (uint32_t i = 0; i < n_jobs; ++i) {
+        const agrad_colsum_job& j = jobs[i];
+        if ((j.partial_a != nullptr) != (j.out_a != nullptr) || (j.partial_b != nullptr) != (j.out_b != nullptr))
+            return set_error(AGRAD_EINVAL, "column-sum finalize: job %u has partial rows without a destination or the reverse", i);
+        if (j.flags & ~(uint32_t)(AGRAD_ACC_PARAM_GRAD | AGRAD_PARAM_GRAD_BF16))
+            return set_error(AGRAD_EINVAL, "column-sum finalize: job %u has unknown flag bits 0x%x", i, j.flags);
+        list[i] = ColsumJob{j.partial_a, j.partial_b, j.out_a, j.out_b, j.partial_rows, j.C,
+                            (j.flags & AGRAD_ACC_PARAM_GRAD) ? 1u : 0u, (j.flags & AGRAD_PARAM_GRAD_BF16) ? 1u : 0u};
+    }
+    return launch_colsum_finalize_many(ctx->stream, list.data(), list.size());
+}
+int agrad_norm_backward_partial(agrad_ctx* ctx, int kind, int dtype, const void* x, const void* dy,
+                                const float* gamma, const void* dres_in, void* dx, void* dx2,
+                                float* dgamma, float* dbeta, void* workspace, uint64_t workspace_bytes,
+                                uint64_t rows, uint32_t C, float eps, uint32_t flags, agrad_colsum_job* job) {
+    CTX_OR_FAIL(ctx)
+    if (job == nullptr) return set_error(AGRAD_EINVAL, "norm backward (partial): null job pointer");
+    std::memset(job, 0, sizeof(*job));
+    std::vector<ColsumJob> sink;
+    int rc;
+    {
+        ColsumDefer defer(&sink);
+        rc = launch_norm_bwd(ctx->stream, kind, dtype, x, dy, gamma, dres_in, dx, dx2, dgamma, dbeta,
+                             workspace, workspace_bytes, rows, C, eps, flags);
+    }
+    if (rc != AGRAD_OK || sink.empty()) return rc;        // (no dgamma / dbeta, or no rows: nothing is left to fold)
+    const ColsumJob& j = sink[0];
+    job->partial_a = j.pa; job->partial_b = j.pb; job->out_a = j.out_a; job->out_b = j.out_b;
+    job->partial_rows = j.P; job->C = j.C;
+    job->flags = (j.accumulate ? AGRAD_ACC_PARAM_GRAD : 0u) | (j.out_bf16 ? AGRAD_PARAM_GRAD_BF16 : 0u);
+    return AGRAD_OK;
 }
 
 int agrad_gelu_forward(agrad_ctx* ctx, int dtype, const void* x, void* y, uint64_t n) {
@@ -871,6 +949,7 @@ uint64_t agrad_gelu_bias_backward_workspace_bytes(uint64_t rows, uint32_t C) {
 int agrad_gelu_bias_backward(agrad_ctx* ctx, int dtype, const void* dy, const void* h, const void* b, void* dh, void* db,
                              void* workspace, uint64_t workspace_bytes, uint64_t rows, uint32_t C, uint32_t flags) {
     CTX_OR_FAIL(ctx)
+    DeferScope defer(ctx, flags);
     return launch_gelu_bias_bwd(ctx->stream, dtype, dy, h, b, dh, db, workspace, workspace_bytes, rows, C, flags);
 }
 int agrad_gelu_backward(agrad_ctx* ctx, int dtype, const void* x, const void* dy, void* dx, uint64_t n, uint32_t flags) {
@@ -961,6 +1040,7 @@ uint64_t agrad_broadcast_grad_workspace_bytes(uint64_t lead, uint64_t inner) {
 int agrad_broadcast_add_backward(agrad_ctx* ctx, int dtype, const void* g, void* dy, void* workspace,
                                  uint64_t workspace_bytes, uint64_t lead, uint64_t inner, uint32_t flags) {
     CTX_OR_FAIL(ctx)
+    DeferScope defer(ctx, flags);
     return launch_broadcast_grad(ctx->stream, dtype, g, dy, workspace, workspace_bytes, lead, inner, flags);
 }
 

@@ -922,10 +922,16 @@ __device__ __forceinline__ void add_partial_rows(float (&sum)[VEC], const float*
 
 // One arrival at a counter; true for the wave whose arrival is number `expected` (it also
 // puts the counter back to zero).  A wave arrives after its partial rows have been
-// written (its device-scope stores have completed before the counter moves), so the wave
-// that arrives last finds all of them.
+// written, so the wave that arrives last finds all of them.  What makes that true: the
+// partial rows are device-scope (sc1) stores, which are acknowledged only once they are
+// past the L2, and the explicit s_waitcnt vmcnt(0) below holds the wave until every one of
+// its stores has been acknowledged -- only then does the counter move.  The workgroup-scope
+// release fence beside it is a compiler barrier only: on gfx950 it emits no vmcnt wait
+// (a workgroup shares its L1), so the explicit wait is what orders stores and counter
+// across workgroups, without the L2 write-back an agent-scope release would cost.
 __device__ __forceinline__ bool arrive_last(uint32_t* ticket, uint32_t expected, uint32_t lane) {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");          // wait for this wave's stores
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");          // keeps the compiler from moving stores down
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                // every store of this wave has been acknowledged
     uint32_t old = 0;
     if (lane == 0) old = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     old = (uint32_t)__builtin_amdgcn_readfirstlane((int)old);

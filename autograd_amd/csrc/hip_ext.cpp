@@ -61,6 +61,13 @@ public:
     }
     // record the launches between graph_begin and graph_end, replay them with graph_launch
     void graph_begin() { raise_for(agrad_graph_begin(ctx_)); }
+    // column sums that backward launches with DEFER_PARAM_GRAD left unfolded: fold them all / count them
+    void finalize_param_grads() { raise_for(agrad_finalize_param_grads(ctx_)); }
+    uint32_t pending_param_grads() {
+        uint32_t n = 0;
+        raise_for(agrad_pending_param_grads(ctx_, &n));
+        return n;
+    }
     uint64_t graph_end() {
         uint64_t id = 0;
         raise_for(agrad_graph_end(ctx_, &id));
@@ -190,6 +197,7 @@ PYBIND11_MODULE(hip_ext, m) {
     m.attr("ACC_INPUT_GRAD") = (unsigned)AGRAD_ACC_INPUT_GRAD;
     m.attr("ACC_PARAM_GRAD") = (unsigned)AGRAD_ACC_PARAM_GRAD;
     m.attr("ACC_PARAM_GRAD2") = (unsigned)AGRAD_ACC_PARAM_GRAD2;
+    m.attr("DEFER_PARAM_GRAD") = (unsigned)AGRAD_DEFER_PARAM_GRAD;
     m.attr("PARAM_GRAD_BF16") = (unsigned)AGRAD_PARAM_GRAD_BF16;
     m.def("device_count", [] {
         int n = 0;
@@ -228,6 +236,8 @@ PYBIND11_MODULE(hip_ext, m) {
         .def("kernel_names", &HipContext::kernel_names)
         .def("kernel_signature", &HipContext::kernel_signature)
         .def("handle", &HipContext::handle)
+        .def("finalize_param_grads", &HipContext::finalize_param_grads)
+        .def("pending_param_grads", &HipContext::pending_param_grads)
         .def("graph_begin", &HipContext::graph_begin)
         .def("graph_end", &HipContext::graph_end)
         .def("graph_launch", &HipContext::graph_launch)

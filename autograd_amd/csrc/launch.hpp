@@ -6,6 +6,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <vector>
+
 #include "../../include/autograd_hip.h"
 
 namespace agrad {
@@ -50,6 +52,29 @@ int launch_norm_bwd_noalloc(hipStream_t s, int device, int kind, int dtype, cons
 // out_bf16: out_a / out_b point at bf16 elements (the sum is rounded once, after the optional accumulate)
 int launch_colsum_finalize(hipStream_t s, const float* pa, const float* pb, uint32_t P, uint32_t C,
                            float* out_a, float* out_b, int accumulate, bool out_bf16 = false);
+
+// One column sum left to fold: out_a[c] (+)= sum of the P rows of pa[P, C], the same for pb -> out_b.
+struct ColsumJob {
+    const float* pa; const float* pb;
+    void* out_a; void* out_b;            // fp32, or bf16 when out_bf16
+    uint32_t P, C, accumulate, out_bf16;
+};
+constexpr int kFinalizeManyJobs = 32;    // jobs one batched finalize launch takes (they travel as kernel arguments)
+// While one of these lives on the calling thread (with a non-null sink), every
+// launch_colsum_finalize on that thread -- the second launch of the norm backward, of the
+// bias gradients and of Mul's row-operand gradient -- is appended to `sink` instead of
+// launched; the partial rows it names must stay untouched until the sink has been folded.
+class ColsumDefer {
+public:
+    explicit ColsumDefer(std::vector<ColsumJob>* sink);
+    ~ColsumDefer();
+    ColsumDefer(const ColsumDefer&) = delete;
+    ColsumDefer& operator=(const ColsumDefer&) = delete;
+private:
+    std::vector<ColsumJob>* prev_;
+};
+// folds `n` pending column sums in as few launches as possible: the same bits as n launch_colsum_finalize calls
+int launch_colsum_finalize_many(hipStream_t s, const ColsumJob* jobs, size_t n);
 
 // reduce.hip
 int launch_broadcast_add(hipStream_t s, int dtype, const void* x, const void* y, void* out, uint64_t lead, uint64_t inner);

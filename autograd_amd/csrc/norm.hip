@@ -28,6 +28,7 @@
 
 #include <cstdlib>
 #include <mutex>
+#include <vector>
 
 // Partial dgamma / dbeta rows of the entry point that allocates nothing
 // (agrad_norm_backward_noalloc): a fixed array in every GPU's memory, held until the
@@ -78,18 +79,15 @@ struct NormBwdArgs {
 constexpr int kFinalizeCols = 8;     // column vectors of a finalize workgroup (2, in 256-thread workgroups, was measured 1.5-3.5 us slower)
 constexpr int kFinalizeLanes = 128;  // row lanes per column vector
 
+// One finalize workgroup: column block `col_block` of out[c] (+)= sum over the P rows of src.
 template <int W>   // W = 4: float4 columns, W = 1: scalar columns
-__global__ void __launch_bounds__(kFinalizeCols * kFinalizeLanes)
-colsum_finalize_kernel(const float* __restrict__ pg, const float* __restrict__ pb, uint32_t P, uint32_t C,
-                       float* __restrict__ dgamma, float* __restrict__ dbeta, int accumulate, int out_bf16) {
+__device__ __forceinline__ void colsum_finalize_block(const float* __restrict__ src, float* __restrict__ dst, uint32_t P,
+                                                      uint32_t C, int accumulate, int out_bf16, uint32_t col_block) {
     constexpr int COLS = kFinalizeCols, LANES = kFinalizeLanes, BATCH = 8;
     __shared__ float tile[LANES][COLS * W];
     __shared__ float tile2[LANES / 16][COLS * W];
-    const float* src = blockIdx.y == 0 ? pg : pb;
-    float* dst = blockIdx.y == 0 ? dgamma : dbeta;
-    if (src == nullptr) return;                      // uniform over the workgroup
     const uint32_t cl = threadIdx.x % COLS, rl = threadIdx.x / COLS;
-    const uint32_t c = (blockIdx.x * COLS + cl) * W;
+    const uint32_t c = (col_block * COLS + cl) * W;
     float s[W];
 #pragma unroll
     for (int k = 0; k < W; ++k) s[k] = 0.0f;
@@ -148,6 +146,35 @@ colsum_finalize_kernel(const float* __restrict__ pg, const float* __restrict__ p
             }
         }
     }
+}
+
+template <int W>
+__global__ void __launch_bounds__(kFinalizeCols * kFinalizeLanes)
+colsum_finalize_kernel(const float* __restrict__ pg, const float* __restrict__ pb, uint32_t P, uint32_t C,
+                       float* __restrict__ dgamma, float* __restrict__ dbeta, int accumulate, int out_bf16) {
+    const float* src = blockIdx.y == 0 ? pg : pb;
+    float* dst = blockIdx.y == 0 ? dgamma : dbeta;
+    if (src == nullptr) return;                      // uniform over the workgroup
+    colsum_finalize_block<W>(src, dst, P, C, accumulate, out_bf16, blockIdx.x);
+}
+
+// The same fold for up to kFinalizeManyJobs column sums that were left pending, in ONE
+// launch: blockIdx.z names the job, and a job runs exactly the workgroups, loads and adds
+// that colsum_finalize_kernel would run for it, so the results are the same bits.  What it
+// saves is the launches: a finalize is a few microseconds of launch floor around a few
+// hundred nanoseconds of work, paid once per norm of a network when every backward call
+// folds its own partial rows.
+struct ColsumJobs { ColsumJob job[kFinalizeManyJobs]; };
+
+template <int W>
+__global__ void __launch_bounds__(kFinalizeCols * kFinalizeLanes)
+colsum_finalize_many_kernel(const ColsumJobs jobs) {
+    const ColsumJob& j = jobs.job[blockIdx.z];
+    const float* src = blockIdx.y == 0 ? j.pa : j.pb;
+    float* dst = reinterpret_cast<float*>(blockIdx.y == 0 ? j.out_a : j.out_b);
+    if (src == nullptr || dst == nullptr) return;    // uniform over the workgroup
+    if (blockIdx.x * (kFinalizeCols * W) >= j.C) return;     // (the grid is as wide as the widest job)
+    colsum_finalize_block<W>(src, dst, j.P, j.C, (int)j.accumulate, (int)j.out_bf16, blockIdx.x);
 }
 
 // gamma / beta are fp32 whatever the activation type: VEC of them is one or two
@@ -870,17 +897,75 @@ int norm_bwd_typed(hipStream_t s, const NormPlan& p, const NormBwdArgs<T>& a, ui
 
 }  // namespace
 
+// Where finalize launches go while a caller collects them (see ColsumDefer in launch.hpp).
+static thread_local std::vector<ColsumJob>* g_colsum_sink = nullptr;
+ColsumDefer::ColsumDefer(std::vector<ColsumJob>* sink) : prev_(g_colsum_sink) { if (sink) g_colsum_sink = sink; }
+ColsumDefer::~ColsumDefer() { g_colsum_sink = prev_; }
+
+static bool colsum_job_vec4(const ColsumJob& j) {
+    return j.C % 4 == 0 && (!j.out_a || aligned16(j.out_a)) && (!j.out_b || aligned16(j.out_b)) &&
+           (!j.pa || aligned16(j.pa)) && (!j.pb || aligned16(j.pb));
+}
+
 int launch_colsum_finalize(hipStream_t s, const float* pa, const float* pb, uint32_t P, uint32_t C,
                            float* out_a, float* out_b, int accumulate, bool out_bf16) {
-    const bool vec4 = C % 4 == 0 && (!out_a || aligned16(out_a)) && (!out_b || aligned16(out_b)) &&
-                      (!pa || aligned16(pa)) && (!pb || aligned16(pb));
-    if (vec4)
+    if (g_colsum_sink != nullptr) {
+        // left pending: the caller folds it later, together with others (launch_colsum_finalize_many)
+        g_colsum_sink->push_back(ColsumJob{pa, pb, out_a, out_b, P, C, accumulate ? 1u : 0u, out_bf16 ? 1u : 0u});
+        return AGRAD_OK;
+    }
+    const ColsumJob j{pa, pb, out_a, out_b, P, C, 0, 0};
+    if (colsum_job_vec4(j))
         hipLaunchKernelGGL((colsum_finalize_kernel<4>), dim3((C / 4 + kFinalizeCols - 1) / kFinalizeCols, 2), dim3(kFinalizeCols * kFinalizeLanes), 0, s, pa, pb, P, C,
                            out_a, out_b, accumulate, out_bf16 ? 1 : 0);
     else
         hipLaunchKernelGGL((colsum_finalize_kernel<1>), dim3((C + kFinalizeCols - 1) / kFinalizeCols, 2), dim3(kFinalizeCols * kFinalizeLanes), 0, s, pa, pb, P, C,
                            out_a, out_b, accumulate, out_bf16 ? 1 : 0);
     return check_hip(hipGetLastError(), "column-sum finalize launch");
+}
+
+// do the destination rows a (of job ja) and b (of job jb) share bytes?
+static bool outputs_overlap(const void* a, const ColsumJob& ja, const void* b, const ColsumJob& jb) {
+    if (a == nullptr || b == nullptr) return false;
+    const uintptr_t a0 = reinterpret_cast<uintptr_t>(a), b0 = reinterpret_cast<uintptr_t>(b);
+    const uintptr_t an = (uintptr_t)ja.C * (ja.out_bf16 ? 2u : 4u), bn = (uintptr_t)jb.C * (jb.out_bf16 ? 2u : 4u);
+    return a0 < b0 + bn && b0 < a0 + an;
+}
+
+int launch_colsum_finalize_many(hipStream_t s, const ColsumJob* jobs, size_t n) {
+    // The jobs are taken in order and share a launch while they can: up to kFinalizeManyJobs of
+    // one column width (float4 or scalar) whose destinations are all different.  A job that
+    // writes where an earlier job of the batch writes (a gamma tied between two norms: one stores,
+    // the other adds) starts a new launch, so that the two happen in the callers' order.
+    ColsumJobs batch;
+    uint32_t count = 0, widest = 0;
+    int batch_vec4 = 1;
+    auto flush = [&]() -> int {
+        if (count == 0) return AGRAD_OK;
+        const uint32_t w = batch_vec4 ? 4u : 1u;
+        const dim3 grid(((widest + w - 1) / w + kFinalizeCols - 1) / kFinalizeCols, 2, count);
+        if (batch_vec4) hipLaunchKernelGGL((colsum_finalize_many_kernel<4>), grid, dim3(kFinalizeCols * kFinalizeLanes), 0, s, batch);
+        else hipLaunchKernelGGL((colsum_finalize_many_kernel<1>), grid, dim3(kFinalizeCols * kFinalizeLanes), 0, s, batch);
+        count = 0;
+        widest = 0;
+        return check_hip(hipGetLastError(), "batched column-sum finalize launch");
+    };
+    for (size_t i = 0; i < n; ++i) {
+        const ColsumJob& j = jobs[i];
+        if (j.C == 0 || j.P == 0 || (j.pa == nullptr && j.pb == nullptr)) continue;
+        const int vec4 = colsum_job_vec4(j) ? 1 : 0;
+        bool clash = count == (uint32_t)kFinalizeManyJobs || (count != 0 && vec4 != batch_vec4);
+        for (uint32_t k = 0; k < count && !clash; ++k) {
+            const ColsumJob& o = batch.job[k];
+            clash = outputs_overlap(j.out_a, j, o.out_a, o) || outputs_overlap(j.out_a, j, o.out_b, o) ||
+                    outputs_overlap(j.out_b, j, o.out_a, o) || outputs_overlap(j.out_b, j, o.out_b, o);
+        }
+        if (clash) if (int rc = flush()) return rc;
+        batch_vec4 = vec4;
+        batch.job[count++] = j;
+        widest = j.C > widest ? j.C : widest;
+    }
+    return flush();
 }
 
 uint64_t norm_bwd_workspace_bytes(uint64_t rows, uint32_t C, int dtype) {

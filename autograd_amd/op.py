@@ -23,7 +23,7 @@ from .utils import broadcast_shape, mul_bcast_kind
 
 class OpNode:
     __slots__ = ("op", "inputs", "outputs", "forward", "backward", "scratch_fwd_layout",
-                 "scratch_bwd_layout", "name", "overwrite_grads")
+                 "scratch_bwd_layout", "name", "overwrite_grads", "defer_param_grads")
 
     def __init__(self, op, inputs, outputs, name=""):
         self.op = op
@@ -37,6 +37,10 @@ class OpNode:
         # ids of gradient tensors this node is the first to write in a backward
         # pass: its kernel may store instead of accumulate (set by the runtime)
         self.overwrite_grads = frozenset()
+        # the backward kernel leaves its parameter-gradient column sums (dgamma / dbeta, a bias
+        # gradient) unfolded and the runtime folds all of a pass's sums in one launch at the
+        # end of the pass (set by the runtime; the node's backward scratch then lives that long)
+        self.defer_param_grads = False
 
 
 class Op(ABC):

@@ -98,7 +98,7 @@ class Runtime:
         return cls._default_runtime
 
     def __init__(self, device="hip", forward_only=False, owns_params=True, use_fp16_gemm=False,
-                 fuse_grad_zeroing=True):
+                 fuse_grad_zeroing=True, defer_param_grad_sums=True):
         self.loss = None
         self.topo = []
         self.forward_only = forward_only
@@ -114,6 +114,13 @@ class Runtime:
         self.backend.use_fp16_gemm = use_fp16_gemm
         # only a backend whose kernels honour OpNode.overwrite_grads can skip the fills
         self.fuse_grad_zeroing = bool(fuse_grad_zeroing and getattr(self.backend, "supports_grad_store", False))
+        # The column sums of parameter gradients (dgamma / dbeta of every norm, bias gradients)
+        # end in a second, tiny launch that costs its launch floor -- a fifth of a norm backward
+        # at 16384 x 384 -- and nothing reads a parameter gradient before the pass ends: with this
+        # on, the backward kernels leave their partial rows in their scratch and ONE launch at
+        # the end of backward_graph folds them all (same bits as folding each on its own).
+        self.defer_param_grad_sums = bool(defer_param_grad_sums
+                                          and getattr(self.backend, "supports_deferred_param_grads", False))
         self.arena_bytes = 0
         self._owns_arena = False       # release() frees only an arena this runtime allocated
         self.memory_plan = None        # key -> arena offset, set by plan_memory()
@@ -197,6 +204,8 @@ class Runtime:
                 raise RuntimeError(f"device {self.allocator.device!r} has no kernel for {type(node.op).__name__}")
             fwd, bwd = self.backend.plan_scratch(node)
             node.scratch_fwd_layout, node.scratch_bwd_layout = fwd, (None if self.forward_only else bwd)
+            node.defer_param_grads = bool(self.defer_param_grad_sums and node.scratch_bwd_layout is not None
+                                          and self.backend.can_defer_param_grads(node))
 
         self._resolve_aliases()
 
@@ -366,7 +375,10 @@ class Runtime:
                         g = self._grad_root(t).grad
                         touch(g if g is not None else t.grad, step)
                 if node.scratch_bwd_layout is not None:
-                    touch(_Scratch(node.scratch_bwd_layout.nbytes, node, 1), step)
+                    block = _Scratch(node.scratch_bwd_layout.nbytes, node, 1)
+                    touch(block, step)
+                    if node.defer_param_grads:
+                        touch(block, len(steps) - 1)     # its partial rows wait for the fold that ends the pass
         if self.loss is not None and self.loss.op is not None:
             touch(self._root(self.loss), len(steps))
             if self.loss.grad is not None:
@@ -499,6 +511,8 @@ class Runtime:
                 if t.grad is not None:
                     self.backend.fill(t.grad, 0)
             node.backward(node.inputs, node.outputs)
+        if self.defer_param_grad_sums:
+            self.backend.finalize_param_grads()
         self.backend.end_pass()
 
     def capture(self, fn):

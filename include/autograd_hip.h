@@ -46,7 +46,7 @@ enum {
     AGRAD_ACC_PARAM_GRAD = 2u, /* dgamma/dbeta/dW += ...; else =                                   */
     AGRAD_ACC_INPUT_GRAD2 = 4u, /* norm backward: the same choice for the second output dx2        */
     AGRAD_ACC_PARAM_GRAD2 = 8u, /* sorted embedding backward: the same choice for dwpe             */
-    AGRAD_PARAM_GRAD_BF16 = 16u /* parameter gradients stored as bf16: the embedding backward with an fp32
+    AGRAD_PARAM_GRAD_BF16 = 16u, /* parameter gradients stored as bf16: the embedding backward with an fp32
                                  * upstream gradient (dW and dwpe; gather_backward_bf16_kernel,
                                  * metal_ops.metal:12395-12446) and the norm backward (dgamma and dbeta then
                                  * point at bf16; the bf16 option of rmsnorm_weighted_dgamma and
@@ -54,6 +54,12 @@ enum {
                                  * sums agrad_broadcast_add_backward / agrad_pos_embedding_backward / db of
                                  * agrad_gelu_bias_backward (bias_grad_reduce_bf16, metal_ops.metal:12101).  A sum is finished in fp32,
                                  * added to the stored value and rounded once */
+    AGRAD_DEFER_PARAM_GRAD = 32u /* agrad_norm_backward, agrad_broadcast_add_backward, agrad_gelu_bias_backward and
+                                 * agrad_mul_backward (row operand): the column sum over rows is left UNFOLDED -- the
+                                 * partial rows stay in the call's workspace, the context remembers the job, and
+                                 * agrad_finalize_param_grads folds all remembered jobs in one launch (see there).
+                                 * The reference splits dgamma off the same way (rmsnorm_weighted_dgamma,
+                                 * metal_ops.metal:14541-14746) */
 };
 
 /* ---- context, memory, passes --------------------------------------------
@@ -227,6 +233,48 @@ int agrad_norm_backward(agrad_ctx* ctx, int kind, int dtype,
                         float* dgamma, float* dbeta,
                         void* workspace, uint64_t workspace_bytes,
                         uint64_t rows, uint32_t C, float eps, uint32_t flags);
+
+/* One column sum that is still to be folded: out_a[c] (+)= sum over partial_rows rows of
+ * partial_a[partial_rows, C], and the same for partial_b -> out_b (either pair may be NULL).
+ * flags: AGRAD_ACC_PARAM_GRAD (add to what out_* holds), AGRAD_PARAM_GRAD_BF16 (out_* are bf16). */
+typedef struct agrad_colsum_job {
+    const float* partial_a;
+    const float* partial_b;
+    void* out_a;
+    void* out_b;
+    uint32_t partial_rows, C, flags, reserved;
+} agrad_colsum_job;
+
+/* The second launch of a column sum, amortised.  Every backward kernel that reduces over rows
+ * (dgamma / dbeta of the norms, bias gradients) leaves one partial row per workgroup and folds
+ * them with a second, tiny launch, which on this GPU costs about 4 us of launch floor whatever
+ * its size: a fifth of a norm backward at 16384 x 384.  A network has dozens of such sums
+ * per backward pass and needs none of them before the pass ends, so:
+ *   - a backward call with AGRAD_DEFER_PARAM_GRAD in its flags runs its main kernel only and
+ *     leaves the job with the context.  Its workspace must stay untouched, and may not be
+ *     shared with another deferred call, until the jobs have been folded;
+ *   - agrad_finalize_param_grads folds every job the context holds, 32 to a launch
+ *     (blockIdx.z = job), each with exactly the workgroups, loads and additions of its own
+ *     second launch: the same bits.  Jobs are folded in the order they were left; two jobs that
+ *     write the same gradient (a gamma tied between two norms: one call stores, the next adds)
+ *     go into separate launches, one after the other.  agrad_end_pass, agrad_synchronize, agrad_graph_begin and
+ *     agrad_graph_end fold what is pending first, so nothing a caller waits for stays unfolded;
+ *   - agrad_pending_param_grads reports how many jobs wait.
+ * agrad_norm_backward_partial / agrad_colsum_finalize_many are the same two halves for callers
+ * that keep the job list themselves.  The reference's closest precedent is its separate dgamma
+ * kernel (rmsnorm_weighted_dgamma, metal_ops.metal:14541-14746; backend.py:4053-4068). */
+int agrad_pending_param_grads(agrad_ctx* ctx, uint32_t* count);
+int agrad_finalize_param_grads(agrad_ctx* ctx);
+int agrad_colsum_finalize_many(agrad_ctx* ctx, const agrad_colsum_job* jobs, uint32_t n_jobs);
+/* agrad_norm_backward without the fold of dgamma / dbeta: *job receives what is left to do
+ * (partial_rows == 0 when nothing is: no dgamma and dbeta asked for, or no rows). */
+int agrad_norm_backward_partial(agrad_ctx* ctx, int kind, int dtype,
+                                const void* x, const void* dy, const float* gamma,
+                                const void* dres_in, void* dx, void* dx2,
+                                float* dgamma, float* dbeta,
+                                void* workspace, uint64_t workspace_bytes,
+                                uint64_t rows, uint32_t C, float eps, uint32_t flags,
+                                agrad_colsum_job* job);
 
 /* agrad_norm_backward for callers that cannot allocate device memory (code under
  * HIP graph capture, serving loops, harnesses that forbid hipMalloc): no workspace
