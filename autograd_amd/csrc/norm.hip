@@ -27,6 +27,7 @@
 #include "launch.hpp"
 
 #include <cstdlib>
+#include <map>
 #include <mutex>
 #include <vector>
 
@@ -213,21 +214,28 @@ template <> __device__ __forceinline__ float round_through<bf16_t>(float v) {
 // wave) gives the dispatcher the most freedom.
 constexpr int kFwdGroupBlock = 64;
 
-// EARLY (RMSNorm with gamma, fp32 rows that fill a wave or more): gamma is requested
-// before the row, so that it arrives while the row is in flight instead of costing
-// a cache round trip between the row sums and the stores (C = 1536: 36.4 -> 34.0
-// us).  It costs NV * VEC registers: with beta as well the kernel drops from 8 to 5
-// waves per SIMD and loses more than it gains; bf16 rows (8 elements per vector)
-// lose too; and when several short rows share a wave the late loads are free.
-//
-// The flavour (KIND), the fused residual (RES) and EARLY are compile-time: with them
-// as run-time branches the fp32 kernel at C = 1536 held more values live and took
-// 36.5 us where the specialised one takes 33.3 us (a plain copy: 31.3 us).
-template <typename T, int VEC, int NV, int TPR, int KIND, bool RES, bool EARLY>
+// The flavour (KIND), the fused residual (RES) and which parameters there are (PARAMS: 0 none,
+// 1 gamma, 2 gamma and beta) are compile-time: with them as run-time branches the fp32 kernel
+// at C = 1536 held more values live and took 36.5 us where the specialised one takes 33.3 us
+// (a plain copy: 31.3 us), and a parameter load behind a branch waits for itself alone -- NV
+// cache round trips one after the other between the row sums and the stores.  Here the NV
+// vectors of gamma (and beta) are requested together: before the row where params_early()
+// says so (they arrive while the row is in flight, at the price of NV * VEC registers each),
+// else right after the row sums.  A PARAMS == 2 launch may still lack one of the two (a
+// LayerNorm without bias): the missing one is read from kNoParam and ignored.
+__device__ const float kNoParam[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+
+template <typename T>
+constexpr bool params_early(int tpr, int kind, int params) {
+    return tpr >= 32 && tpr <= 128;
+}
+
+template <typename T, int VEC, int NV, int TPR, int KIND, bool RES, int PARAMS>
 __global__ void __launch_bounds__(TPR >= 128 ? TPR : kFwdGroupBlock)
 norm_fwd_kernel(const NormFwdArgs<T> a) {
     constexpr int BLOCK = TPR >= 128 ? TPR : kFwdGroupBlock;
     constexpr int RPB = BLOCK / TPR;
+    constexpr bool EARLY = params_early<T>(TPR, KIND, PARAMS);
     __shared__ float lds[3 * kRowSumSlot * (TPR > kWave ? TPR / kWave : 1)];
 
     const int sub = threadIdx.x / TPR;
@@ -237,38 +245,59 @@ norm_fwd_kernel(const NormFwdArgs<T> a) {
     const uint32_t C = a.C;
     const uint64_t base = row * C;
 
+    // Every load of the row is issued before anything waits for one.  A load behind a
+    // branch gets a full wait of its own (its value meets the zeros of the lanes that skip
+    // it), which puts the NV vectors of a row one memory latency after the other; so a lane
+    // past the end of the row loads the row's first vector instead (a valid address, one
+    // cache line for all such lanes) and its values are zeroed afterwards.
+    typedef RawVec<T, VEC> Raw;
     float v[NV][VEC];
-    float gam[EARLY ? NV : 1][VEC];
+    float gam[PARAMS >= 1 ? NV : 1][VEC], bet[PARAMS >= 2 ? NV : 1][VEC];
     bool on[NV];
-    if constexpr (EARLY) {
-#pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
-            if (col < C) load_param<VEC>(a.gamma + col, gam[i]);
-        }
-    }
+    uint32_t col_ld[NV];
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
         on[i] = col < C;
-        if (on[i]) {
-            VecIO<T, VEC>::load(a.x + base + col, v[i]);
-        } else {
+        col_ld[i] = on[i] ? col : 0u;
+    }
+    const bool has_gamma = PARAMS == 1 || a.gamma != nullptr, has_beta = a.beta != nullptr;
+    auto load_params = [&]() {
+        if constexpr (PARAMS >= 1) {
+            const float* gp = has_gamma ? a.gamma : kNoParam;
+            const uint32_t gmask = has_gamma ? ~0u : 0u;
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) v[i][k] = 0.0f;
+            for (int i = 0; i < NV; ++i) load_param<VEC>(gp + (col_ld[i] & gmask), gam[i]);
         }
+        if constexpr (PARAMS >= 2) {
+            const float* bp = has_beta ? a.beta : kNoParam;
+            const uint32_t bmask = has_beta ? ~0u : 0u;
+#pragma unroll
+            for (int i = 0; i < NV; ++i) load_param<VEC>(bp + (col_ld[i] & bmask), bet[i]);
+        }
+    };
+    if constexpr (EARLY) load_params();
+    typename Raw::type rx[NV], rr[RES ? NV : 1];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) rx[i] = Raw::load(a.x + base + col_ld[i]);
+    if constexpr (RES) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) rr[i] = Raw::load(a.res + base + col_ld[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        Raw::unpack(rx[i], v[i]);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) v[i][k] = on[i] ? v[i][k] : 0.0f;
     }
     if constexpr (RES) {
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            if (on[i]) {
-                const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
-                float r[VEC];
-                VecIO<T, VEC>::load(a.res + base + col, r);
+            float r[VEC];
+            Raw::unpack(rr[i], r);
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) v[i][k] = round_through<T>(v[i][k] + r[k]);
-                if (a.h != nullptr) VecIO<T, VEC>::store(a.h + base + col, v[i]);
-            }
+            for (int k = 0; k < VEC; ++k) v[i][k] = on[i] ? round_through<T>(v[i][k] + r[k]) : 0.0f;
+            if (on[i] && a.h != nullptr) VecIO<T, VEC>::store(a.h + base + col_ld[i], v[i]);
         }
     }
 
@@ -302,30 +331,21 @@ norm_fwd_kernel(const NormFwdArgs<T> a) {
         scale = 1.0f / sqrtf(ms + a.eps);
     }
 
+    if constexpr (!EARLY) load_params();
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-        if (on[i]) {
-            const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
-            float o[VEC];
+        float o[VEC];
 #pragma unroll
-            for (int k = 0; k < VEC; ++k) o[k] = v[i][k] * scale;
-            if constexpr (EARLY) {
+        for (int k = 0; k < VEC; ++k) o[k] = v[i][k] * scale;
+        if constexpr (PARAMS >= 1) {
 #pragma unroll
-                for (int k = 0; k < VEC; ++k) o[k] = o[k] * gam[i][k];
-            } else if (a.gamma != nullptr) {
-                float w[VEC];
-                load_param<VEC>(a.gamma + col, w);
-#pragma unroll
-                for (int k = 0; k < VEC; ++k) o[k] = o[k] * w[k];
-            }
-            if (a.beta != nullptr) {
-                float w[VEC];
-                load_param<VEC>(a.beta + col, w);
-#pragma unroll
-                for (int k = 0; k < VEC; ++k) o[k] = o[k] + w[k];
-            }
-            VecIO<T, VEC>::store(a.y + base + col, o);
+            for (int k = 0; k < VEC; ++k) o[k] = has_gamma ? o[k] * gam[i][k] : o[k];
         }
+        if constexpr (PARAMS >= 2) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) o[k] = has_beta ? o[k] + bet[i][k] : o[k];
+        }
+        if (on[i]) VecIO<T, VEC>::store(a.y + base + col_ld[i], o);
     }
 }
 
@@ -335,13 +355,23 @@ norm_fwd_kernel(const NormFwdArgs<T> a) {
 // Threads of a backward workgroup whose rows take a wave or less each (512 and 1024, with a
 // half and a quarter of the partial rows, were measured: within 1 us either way at 16384 rows).
 constexpr int kBwdGroupBlock = 256;
+// The residual gradient of a row is requested (all its vectors together) with the next row's
+// prefetch, or only once the row's own sums are under way.
+constexpr bool kDresEarly = false;
 
-template <typename T, int VEC, int NV, int TPR>
+// Compile-time: the flavour (KIND), which column sums are kept (SUMS: 0 none, 1 dgamma, 2 dgamma
+// and dbeta -- their accumulators are NV * VEC registers each, and an RMSNorm has no beta) and
+// whether a residual gradient comes in (DRES).  As run-time branches these cost registers (the
+// bf16 kernel at C = 1536 held 207 and ran two waves per SIMD) and put every load that sat
+// behind one of them a memory latency of its own away from the next.
+template <typename T, int VEC, int NV, int TPR, int KIND, int SUMS, bool DRES>
 __global__ void __launch_bounds__(TPR >= 128 ? TPR : kBwdGroupBlock)
 norm_bwd_kernel(const NormBwdArgs<T> a) {
     constexpr int BLOCK = TPR >= 128 ? TPR : kBwdGroupBlock;
     constexpr int RPB = BLOCK / TPR;
     constexpr int NWAVES = BLOCK / kWave;
+    constexpr bool is_ln = KIND == AGRAD_NORM_LAYER;
+    constexpr bool want_pg = SUMS >= 1, want_pb = SUMS >= 2;
     __shared__ float lds[3 * kRowSumSlot * (TPR > kWave ? TPR / kWave : 1)];
     extern __shared__ float comb[];  // (NWAVES - 1) * C floats when RPB > 1
 
@@ -349,41 +379,56 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
     const int lane = threadIdx.x % TPR;
     const uint32_t C = a.C;
     const float fC = (float)C;
-    const bool is_ln = a.kind == AGRAD_NORM_LAYER;
-    const bool want_pg = a.pgamma != nullptr;
-    const bool want_pb = a.pbeta != nullptr;
     const bool acc = (a.flags & AGRAD_ACC_INPUT_GRAD) != 0;
     const bool acc2 = (a.flags & AGRAD_ACC_INPUT_GRAD2) != 0;
 
+    // A lane with nothing to load (past the end of the row, no next row, no gamma) loads
+    // from a valid address that every such lane shares and never uses the value: a load
+    // behind a branch gets a wait of its own, which would put a row's vectors one memory
+    // latency after the other.
     bool on[NV];
-    float gam[NV][VEC], pg[NV][VEC], pb[NV][VEC];
-#pragma unroll
-    for (int i = 0; i < NV; ++i) {
-        const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
-        on[i] = col < C;
-#pragma unroll
-        for (int k = 0; k < VEC; ++k) {
-            gam[i][k] = 1.0f;
-            pg[i][k] = 0.0f;
-            pb[i][k] = 0.0f;
-        }
-        if (on[i] && a.gamma != nullptr) load_param<VEC>(a.gamma + col, gam[i]);
-    }
-    SlotRing ring;
-
-    // Rows are software-pipelined: the x and dy vectors of the NEXT row are
-    // requested (as raw bits) before the current row is worked on, so a wave
-    // always has a row of loads in flight while it computes.
-    typedef RawVec<T, VEC> Raw;
-    typename Raw::type nx[NV], ng[NV];
-    const uint64_t stride = (uint64_t)gridDim.x * RPB;
-    uint64_t row = (uint64_t)blockIdx.x * RPB + sub;
-    if (row < a.rows) {
+    uint32_t col_ld[NV];
+    float gam[NV][VEC], pg[want_pg ? NV : 1][VEC], pb[want_pb ? NV : 1][VEC];
+    const bool has_gamma = a.gamma != nullptr;
+    {
+        const float* gp = has_gamma ? a.gamma : kNoParam;
+        const uint32_t gmask = has_gamma ? ~0u : 0u;
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
-            nx[i] = on[i] ? Raw::load(a.x + row * C + col) : Raw::zero();
-            ng[i] = on[i] ? Raw::load(a.dy + row * C + col) : Raw::zero();
+            on[i] = col < C;
+            col_ld[i] = on[i] ? col : 0u;
+            load_param<VEC>(gp + (col_ld[i] & gmask), gam[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) gam[i][k] = has_gamma ? gam[i][k] : 1.0f;
+    }
+#pragma unroll
+    for (int i = 0; i < (want_pg ? NV : 1); ++i)
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) pg[i][k] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < (want_pb ? NV : 1); ++i)
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) pb[i][k] = 0.0f;
+    SlotRing ring;
+
+    // Rows are software-pipelined: the x and dy vectors of the NEXT row are requested (as
+    // raw bits) before the current row is worked on, so a wave always has a row of loads in
+    // flight while it computes; the current row's residual gradient is requested with them.
+    typedef RawVec<T, VEC> Raw;
+    typename Raw::type nx[NV], ng[NV], rd[DRES ? NV : 1];
+    const uint64_t stride = (uint64_t)gridDim.x * RPB;
+    uint64_t row = (uint64_t)blockIdx.x * RPB + sub;
+    {
+        const bool live = row < a.rows;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const uint64_t off = live ? row * C + col_ld[i] : 0ull;
+            nx[i] = Raw::load(a.x + off);
+            ng[i] = Raw::load(a.dy + off);
         }
     }
     for (; row < a.rows; row += stride) {
@@ -393,24 +438,31 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
         for (int i = 0; i < NV; ++i) {
             Raw::unpack(nx[i], xv[i]);
             Raw::unpack(ng[i], g[i]);
+            if (!on[i]) {
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) { xv[i][k] = 0.0f; g[i][k] = 0.0f; }
+            }
         }
-        if (row + stride < a.rows) {
+        {
+            const bool live = row + stride < a.rows;
             const uint64_t nbase = (row + stride) * C;
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
-                const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
-                if (on[i]) {
-                    nx[i] = Raw::load(a.x + nbase + col);
-                    ng[i] = Raw::load(a.dy + nbase + col);
-                }
+                const uint64_t off = live ? nbase + col_ld[i] : 0ull;
+                nx[i] = Raw::load(a.x + off);
+                ng[i] = Raw::load(a.dy + off);
             }
+        }
+        if constexpr (DRES && kDresEarly) {
+#pragma unroll
+            for (int i = 0; i < NV; ++i) rd[i] = Raw::load(a.dres + base + col_ld[i]);
         }
 
         // Row statistics and the two row sums of the dx formula in ONE reduction
         // phase (after the mean, for LayerNorm).  With d = x - mean (or x):
         //   q = sum d^2,   s1 = sum dy*gamma,   s2r = sum dy*gamma*d,
         // and sum dy*gamma*x_hat = s2r * scale.  xv becomes d, then x_hat.
-        if (is_ln) {
+        if constexpr (is_ln) {
             float s = 0.0f;
 #pragma unroll
             for (int i = 0; i < NV; ++i)
@@ -433,6 +485,10 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
                 s1 = s1 + dyg;
                 s2 = mad<T>(dyg, d, s2);
             }
+        if constexpr (DRES && !kDresEarly) {
+#pragma unroll
+            for (int i = 0; i < NV; ++i) rd[i] = Raw::load(a.dres + base + col_ld[i]);
+        }
         if (a.dx != nullptr) row_sum3<TPR>(q, s1, s2, lds, ring.next());
         else q = row_sum<TPR>(q, lds, ring.next());
         const float scale = 1.0f / sqrtf(q / fC + a.eps);
@@ -444,14 +500,14 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
             for (int k = 0; k < VEC; ++k) {
                 const float xh = xv[i][k] * scale;
                 xv[i][k] = xh;
-                if (want_pg) pg[i][k] = mad<T>(g[i][k], xh, pg[i][k]);
-                if (want_pb) pb[i][k] = pb[i][k] + g[i][k];
+                if constexpr (want_pg) pg[i][k] = mad<T>(g[i][k], xh, pg[i][k]);
+                if constexpr (want_pb) pb[i][k] = pb[i][k] + g[i][k];
                 g[i][k] = g[i][k] * gam[i][k];
             }
 
         if (a.dx != nullptr) {
             float c1 = 0.0f, c2;
-            if (is_ln) {
+            if constexpr (is_ln) {
                 c1 = (s1 / fC) * scale;
                 c2 = (s2 / fC) * scale;
             } else {
@@ -459,28 +515,26 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
             }
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
+                float t[VEC];
+                if constexpr (is_ln) {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) {
+                        const float u = mad<T>(g[i][k], scale, -c1);
+                        t[k] = mad<T>(-xv[i][k], c2, u);
+                    }
+                } else {
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k)
+                        t[k] = mad<T>(-xv[i][k], c2, g[i][k]) * scale;
+                }
+                if constexpr (DRES) {
+                    float r[VEC];
+                    Raw::unpack(rd[i], r);
+#pragma unroll
+                    for (int k = 0; k < VEC; ++k) t[k] = r[k] + t[k];
+                }
                 if (on[i]) {
-                    const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
-                    float t[VEC];
-                    if (is_ln) {
-#pragma unroll
-                        for (int k = 0; k < VEC; ++k) {
-                            const float u = mad<T>(g[i][k], scale, -c1);
-                            t[k] = mad<T>(-xv[i][k], c2, u);
-                        }
-                    } else {
-#pragma unroll
-                        for (int k = 0; k < VEC; ++k)
-                            t[k] = mad<T>(-xv[i][k], c2, g[i][k]) * scale;
-                    }
-                    if (a.dres != nullptr) {
-                        // (requesting these with the row, an iteration ahead, was measured: no gain at
-                        // C = 384 ... 1536, and 8 % slower at C = 4096 bf16, where it costs a wave per SIMD)
-                        float r[VEC];
-                        VecIO<T, VEC>::load(a.dres + base + col, r);
-#pragma unroll
-                        for (int k = 0; k < VEC; ++k) t[k] = r[k] + t[k];
-                    }
+                    const uint32_t col = col_ld[i];
                     if (a.dx2 != nullptr) {
                         float t2[VEC];
                         if (acc2) {
@@ -506,7 +560,7 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
     }
 
     // one partial row per workgroup
-    if (want_pg || want_pb) {
+    if constexpr (want_pg) {
         if constexpr (RPB > 1) {
             // lane groups of one wave first (fixed order), then the waves through LDS
             if constexpr (TPR < kWave) {
@@ -516,26 +570,24 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
                     for (int k = 0; k < VEC; ++k) {
                         if constexpr (TPR == 16) {
                             pg[i][k] = pg[i][k] + __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, pg[i][k]), kSwizzleXor16));
-                            pb[i][k] = pb[i][k] + __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, pb[i][k]), kSwizzleXor16));
+                            if constexpr (want_pb) pb[i][k] = pb[i][k] + __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, pb[i][k]), kSwizzleXor16));
                         }
                         pg[i][k] = pg[i][k] + __shfl_xor(pg[i][k], 32);
-                        pb[i][k] = pb[i][k] + __shfl_xor(pb[i][k], 32);
+                        if constexpr (want_pb) pb[i][k] = pb[i][k] + __shfl_xor(pb[i][k], 32);
                     }
             }
             const int wave = threadIdx.x / kWave;
             const bool owner = (threadIdx.x % kWave) < TPR;   // one lane group per wave speaks for it
-#pragma unroll 1
-            for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+            for (int pass = 0; pass < SUMS; ++pass) {
                 float* out = pass == 0 ? a.pgamma : a.pbeta;
-                if (out == nullptr) continue;  // uniform over the workgroup
                 if (wave > 0 && owner) {
 #pragma unroll
                     for (int i = 0; i < NV; ++i)
                         if (on[i]) {
-                            const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
 #pragma unroll
                             for (int k = 0; k < VEC; ++k)
-                                comb[(uint32_t)(wave - 1) * C + col + k] = pass == 0 ? pg[i][k] : pb[i][k];
+                                comb[(uint32_t)(wave - 1) * C + col_ld[i] + k] = pass == 0 ? pg[i][k] : pb[want_pb ? i : 0][k];
                         }
                 }
                 __syncthreads();
@@ -543,16 +595,15 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
 #pragma unroll
                     for (int i = 0; i < NV; ++i)
                         if (on[i]) {
-                            const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
                             float t[VEC];
 #pragma unroll
                             for (int k = 0; k < VEC; ++k) {
-                                t[k] = pass == 0 ? pg[i][k] : pb[i][k];
-                                for (int w = 0; w < NWAVES - 1; ++w) t[k] = t[k] + comb[(uint32_t)w * C + col + k];
+                                t[k] = pass == 0 ? pg[i][k] : pb[want_pb ? i : 0][k];
+                                for (int w = 0; w < NWAVES - 1; ++w) t[k] = t[k] + comb[(uint32_t)w * C + col_ld[i] + k];
                             }
 #pragma unroll
                             for (int k = 0; k < VEC; k += 2)
-                                { out[(uint64_t)blockIdx.x * C + col + k] = t[k]; out[(uint64_t)blockIdx.x * C + col + k + 1] = t[k + 1]; }
+                                { out[(uint64_t)blockIdx.x * C + col_ld[i] + k] = t[k]; out[(uint64_t)blockIdx.x * C + col_ld[i] + k + 1] = t[k + 1]; }
                         }
                 }
                 __syncthreads();
@@ -561,11 +612,10 @@ norm_bwd_kernel(const NormBwdArgs<T> a) {
 #pragma unroll
             for (int i = 0; i < NV; ++i)
                 if (on[i]) {
-                    const uint32_t col = (uint32_t)(i * TPR + lane) * VEC;
 #pragma unroll
                     for (int k = 0; k < VEC; k += 2) {
-                        if (want_pg) { a.pgamma[(uint64_t)blockIdx.x * C + col + k] = pg[i][k]; a.pgamma[(uint64_t)blockIdx.x * C + col + k + 1] = pg[i][k + 1]; }
-                        if (want_pb) { a.pbeta[(uint64_t)blockIdx.x * C + col + k] = pb[i][k]; a.pbeta[(uint64_t)blockIdx.x * C + col + k + 1] = pb[i][k + 1]; }
+                        { a.pgamma[(uint64_t)blockIdx.x * C + col_ld[i] + k] = pg[i][k]; a.pgamma[(uint64_t)blockIdx.x * C + col_ld[i] + k + 1] = pg[i][k + 1]; }
+                        if constexpr (want_pb) { a.pbeta[(uint64_t)blockIdx.x * C + col_ld[i] + k] = pb[i][k]; a.pbeta[(uint64_t)blockIdx.x * C + col_ld[i] + k + 1] = pb[i][k + 1]; }
                     }
                 }
         }
@@ -765,36 +815,41 @@ inline size_t bwd_dyn_lds(const NormPlan& p, uint32_t C) {
     return p.rpb > 1 ? (size_t)(BLOCK / kWave - 1) * C * sizeof(float) : 0;
 }
 
-// request gamma before the row?
-inline bool fwd_params_early(int tpr) { return tpr >= kWave; }
-
 template <typename T, int VEC, int NV, int TPR>
-void fwd_launch(hipStream_t s, const NormFwdArgs<T>& a, uint32_t grid, bool early) {
+void fwd_launch(hipStream_t s, const NormFwdArgs<T>& a, uint32_t grid) {
     constexpr int BLOCK = TPR >= 128 ? TPR : kFwdGroupBlock;
     const bool res = a.res != nullptr;
-#define AGRAD_FWD(KIND, RES, EARLY) \
-    hipLaunchKernelGGL((norm_fwd_kernel<T, VEC, NV, TPR, KIND, RES, EARLY>), dim3(grid), dim3(BLOCK), 0, s, a)
-    if (a.kind == AGRAD_NORM_LAYER) {
-        if (res) AGRAD_FWD(AGRAD_NORM_LAYER, true, false); else AGRAD_FWD(AGRAD_NORM_LAYER, false, false);
-    } else if (early && sizeof(T) == 4) {
-        if constexpr (sizeof(T) == 4) {      // bf16 rows never take it: no instantiation
-            if (res) AGRAD_FWD(AGRAD_NORM_RMS, true, true); else AGRAD_FWD(AGRAD_NORM_RMS, false, true);
-        }
-    } else {
-        if (res) AGRAD_FWD(AGRAD_NORM_RMS, true, false); else AGRAD_FWD(AGRAD_NORM_RMS, false, false);
+    // which parameters: none, gamma alone, or the two-parameter kernel (which also takes beta alone)
+    const int params = a.gamma == nullptr && a.beta == nullptr ? 0 : a.beta == nullptr ? 1 : 2;
+#define AGRAD_FWD(KIND, RES, PARAMS) \
+    hipLaunchKernelGGL((norm_fwd_kernel<T, VEC, NV, TPR, KIND, RES, PARAMS>), dim3(grid), dim3(BLOCK), 0, s, a)
+#define AGRAD_FWD_KIND(KIND)                                                                          \
+    switch (params) {                                                                                 \
+        case 0: if (res) AGRAD_FWD(KIND, true, 0); else AGRAD_FWD(KIND, false, 0); break;             \
+        case 1: if (res) AGRAD_FWD(KIND, true, 1); else AGRAD_FWD(KIND, false, 1); break;             \
+        default: if (res) AGRAD_FWD(KIND, true, 2); else AGRAD_FWD(KIND, false, 2); break;            \
     }
+    if (a.kind == AGRAD_NORM_LAYER) { AGRAD_FWD_KIND(AGRAD_NORM_LAYER) } else { AGRAD_FWD_KIND(AGRAD_NORM_RMS) }
+#undef AGRAD_FWD_KIND
 #undef AGRAD_FWD
+}
+
+// Which (lanes per row, vectors per lane) pairs plan_norm can choose: it takes the fewest
+// lanes whose share fits, so a wider group is only ever chosen with more than half of the
+// largest share (a narrower group would have fitted otherwise) -- except the narrowest and
+// the widest group, which take what is left below and above.
+constexpr bool norm_shape_reachable(int tpr, int nv, int max_nv) {
+    return nv <= max_nv && (tpr == 16 || tpr == 1024 || 2 * nv > max_nv);
 }
 
 template <typename T, int VEC, int TPR>
 int fwd_pick_nv(hipStream_t s, const NormPlan& p, const NormFwdArgs<T>& a) {
     const uint32_t grid = (uint32_t)((a.rows + p.rpb - 1) / p.rpb);
-    const bool early = a.kind == AGRAD_NORM_RMS && a.gamma != nullptr && a.beta == nullptr && fwd_params_early(TPR);
     switch (p.nv) {
 #define AGRAD_CASE(N)                                                                  \
     case N:                                                                            \
-        if constexpr (N * VEC <= kMaxEPT) {                                            \
-            fwd_launch<T, VEC, N, TPR>(s, a, grid, early);                             \
+        if constexpr (norm_shape_reachable(TPR, N, kMaxEPT / VEC)) {                   \
+            fwd_launch<T, VEC, N, TPR>(s, a, grid);                                    \
             return AGRAD_OK;                                                           \
         }                                                                              \
         break;
@@ -804,61 +859,66 @@ int fwd_pick_nv(hipStream_t s, const NormPlan& p, const NormFwdArgs<T>& a) {
     return set_error(AGRAD_EINVAL, "norm forward: no kernel for nv=%d", p.nv);
 }
 
-template <typename T, int VEC, int TPR>
-int bwd_pick_nv(hipStream_t s, const NormPlan& p, const NormBwdArgs<T>& a, uint32_t grid) {
-    constexpr int BLOCK = TPR >= 128 ? TPR : kBwdGroupBlock;
-    const size_t dyn = bwd_dyn_lds<TPR>(p, a.C);
-    switch (p.nv) {
-#define AGRAD_CASE(N)                                                                  \
-    case N:                                                                            \
-        if constexpr (N * VEC <= kMaxEPT) {                                            \
-            hipLaunchKernelGGL((norm_bwd_kernel<T, VEC, N, TPR>), dim3(grid), dim3(BLOCK), dyn, s, a); \
-            return AGRAD_OK;                                                           \
-        }                                                                              \
-        break;
-        AGRAD_CASE(1) AGRAD_CASE(2) AGRAD_CASE(3) AGRAD_CASE(4) AGRAD_CASE(5) AGRAD_CASE(6)
-#undef AGRAD_CASE
-    }
-    return set_error(AGRAD_EINVAL, "norm backward: no kernel for nv=%d", p.nv);
+// Which backward kernel: the flavour, the column sums it keeps and whether a residual
+// gradient comes in.  LayerNorm keeps both sums or none (a frozen gamma or beta gets its
+// partial rows written and not folded); RMSNorm keeps dgamma or none.
+struct BwdVariant { int kind, sums; bool dres; };
+
+// fn(kernel) for the instantiation that (T, VEC, NV, TPR, v) names
+template <typename T, int VEC, int NV, int TPR, typename Fn>
+void with_bwd_kernel(const BwdVariant& v, Fn&& fn) {
+#define AGRAD_BWD(KIND, SUMS) \
+    do { if (v.dres) fn(norm_bwd_kernel<T, VEC, NV, TPR, KIND, SUMS, true>); else fn(norm_bwd_kernel<T, VEC, NV, TPR, KIND, SUMS, false>); } while (0)
+    if (v.kind == AGRAD_NORM_LAYER) { if (v.sums) AGRAD_BWD(AGRAD_NORM_LAYER, 2); else AGRAD_BWD(AGRAD_NORM_LAYER, 0); }
+    else { if (v.sums) AGRAD_BWD(AGRAD_NORM_RMS, 1); else AGRAD_BWD(AGRAD_NORM_RMS, 0); }
+#undef AGRAD_BWD
 }
 
-// workgroups of the chosen backward instantiation the GPU holds at once (0: unknown)
-template <typename T, int VEC, int TPR>
-uint32_t bwd_resident_nv(const NormPlan& p, uint32_t C) {
-    constexpr int BLOCK = TPR >= 128 ? TPR : kBwdGroupBlock;
-    const size_t dyn = bwd_dyn_lds<TPR>(p, C);
-    int per_cu = 0;
-    switch (p.nv) {
-#define AGRAD_CASE(N)                                                                  \
-    case N:                                                                            \
-        if constexpr (N * VEC <= kMaxEPT) {                                            \
-            if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, norm_bwd_kernel<T, VEC, N, TPR>, BLOCK, dyn) != hipSuccess) \
-                per_cu = 0;                                                            \
-        }                                                                              \
-        break;
-        AGRAD_CASE(1) AGRAD_CASE(2) AGRAD_CASE(3) AGRAD_CASE(4) AGRAD_CASE(5) AGRAD_CASE(6)
-#undef AGRAD_CASE
-    }
-    if (per_cu <= 0) { (void)hipGetLastError(); return 0; }
-    return (uint32_t)per_cu * cu_count();
-}
-
-template <typename T>
-uint32_t bwd_resident_typed(const NormPlan& p, uint32_t C) {
+// fn(kernel, workgroup size, dynamic LDS bytes) for the kernel that (T, plan, v) names; false if there is none
+template <typename T, typename Fn>
+bool with_planned_bwd_kernel(const NormPlan& p, uint32_t C, const BwdVariant& v, Fn&& fn) {
     constexpr int VEC = WideVec<T>::value;
-    if (p.generic) return 0;
-    switch (p.tpr) {
-        case 16: return bwd_resident_nv<T, VEC, 16>(p, C);
-        case 32: return bwd_resident_nv<T, VEC, 32>(p, C);
-        case 64: return bwd_resident_nv<T, VEC, 64>(p, C);
-        case 128: return bwd_resident_nv<T, VEC, 128>(p, C);
-        case 256: return bwd_resident_nv<T, VEC, 256>(p, C);
-        default: return bwd_resident_nv<T, VEC, 1024>(p, C);
+    constexpr int MAXNV = (sizeof(T) == 2 ? 24 : 16) / VEC;      // norm_max_ept(backward) / VEC
+    bool found = false;
+#define AGRAD_CASE(TPR, N)                                                                              \
+    if constexpr (norm_shape_reachable(TPR, N, MAXNV)) {                                                \
+        if (p.tpr == TPR && p.nv == N) {                                                                \
+            constexpr int BLOCK = TPR >= 128 ? TPR : kBwdGroupBlock;                                    \
+            with_bwd_kernel<T, VEC, N, TPR>(v, [&](auto kernel) { fn(kernel, BLOCK, bwd_dyn_lds<TPR>(p, C)); }); \
+            found = true;                                                                               \
+        }                                                                                               \
     }
+#define AGRAD_TPR(TPR) AGRAD_CASE(TPR, 1) AGRAD_CASE(TPR, 2) AGRAD_CASE(TPR, 3) AGRAD_CASE(TPR, 4)
+    AGRAD_TPR(16) AGRAD_TPR(32) AGRAD_TPR(64) AGRAD_TPR(128) AGRAD_TPR(256) AGRAD_TPR(1024)
+#undef AGRAD_TPR
+#undef AGRAD_CASE
+    return found;
 }
 
-uint32_t bwd_resident(const NormPlan& p, uint32_t C, int dtype) {
-    return dtype == AGRAD_BF16 ? bwd_resident_typed<bf16_t>(p, C) : bwd_resident_typed<float>(p, C);
+// workgroups of the chosen backward instantiation the GPU holds at once (0: unknown).
+// Asked of the runtime once per instantiation and remembered.
+uint32_t bwd_resident(const NormPlan& p, uint32_t C, int dtype, const BwdVariant& v) {
+    if (p.generic) return 0;
+    static std::mutex mu;
+    static std::map<uint64_t, uint32_t> known;
+    // (the dynamic LDS of the sub-wave geometries grows with C: part of the key)
+    const uint64_t key = ((uint64_t)C << 32) | ((uint64_t)dtype << 24) | ((uint64_t)p.tpr << 8) | ((uint64_t)p.nv << 4) |
+                         ((uint64_t)v.kind << 3) | ((uint64_t)v.sums << 1) | (v.dres ? 1u : 0u);
+    {
+        std::lock_guard<std::mutex> lock(mu);
+        auto it = known.find(key);
+        if (it != known.end()) return it->second;
+    }
+    int per_cu = 0;
+    auto ask = [&](auto kernel, int block, size_t dyn) {
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, block, dyn) != hipSuccess) per_cu = 0;
+    };
+    const bool found = dtype == AGRAD_BF16 ? with_planned_bwd_kernel<bf16_t>(p, C, v, ask) : with_planned_bwd_kernel<float>(p, C, v, ask);
+    if (!found || per_cu <= 0) { (void)hipGetLastError(); per_cu = 0; }
+    const uint32_t resident = (uint32_t)per_cu * cu_count();
+    std::lock_guard<std::mutex> lock(mu);
+    known[key] = resident;
+    return resident;
 }
 
 template <typename T>
@@ -879,20 +939,16 @@ int norm_fwd_typed(hipStream_t s, const NormPlan& p, const NormFwdArgs<T>& a) {
 }
 
 template <typename T>
-int norm_bwd_typed(hipStream_t s, const NormPlan& p, const NormBwdArgs<T>& a, uint32_t grid) {
-    constexpr int VEC = WideVec<T>::value;
+int norm_bwd_typed(hipStream_t s, const NormPlan& p, const NormBwdArgs<T>& a, uint32_t grid, const BwdVariant& v) {
     if (p.generic) {
         hipLaunchKernelGGL((norm_bwd_generic_kernel<T>), dim3(grid), dim3(256), 0, s, a);
         return AGRAD_OK;
     }
-    switch (p.tpr) {
-        case 16: return bwd_pick_nv<T, VEC, 16>(s, p, a, grid);
-        case 32: return bwd_pick_nv<T, VEC, 32>(s, p, a, grid);
-        case 64: return bwd_pick_nv<T, VEC, 64>(s, p, a, grid);
-        case 128: return bwd_pick_nv<T, VEC, 128>(s, p, a, grid);
-        case 256: return bwd_pick_nv<T, VEC, 256>(s, p, a, grid);
-        default: return bwd_pick_nv<T, VEC, 1024>(s, p, a, grid);
-    }
+    const bool found = with_planned_bwd_kernel<T>(p, a.C, v, [&](auto kernel, int block, size_t dyn) {
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(block), dyn, s, a);
+    });
+    if (!found) return set_error(AGRAD_EINVAL, "norm backward: no kernel for %d lanes x %d vectors", p.tpr, p.nv);
+    return AGRAD_OK;
 }
 
 }  // namespace
@@ -969,13 +1025,18 @@ int launch_colsum_finalize_many(hipStream_t s, const ColsumJob* jobs, size_t n) 
 }
 
 uint64_t norm_bwd_workspace_bytes(uint64_t rows, uint32_t C, int dtype) {
-    // sized for the larger of the vector and the scalar geometry
+    // sized for the largest grid any kernel of this shape runs with: the scalar geometry, and
+    // the register-resident one in each of its flavours that keeps column sums
     NormPlan vecp = plan_norm(C, dtype, true, true);
     NormPlan genp{true, 256, 0, 1};
     uint64_t blocks = bwd_blocks(genp, rows, 0);
     if (!vecp.generic) {
-        const uint64_t b = bwd_blocks(vecp, rows, bwd_resident(vecp, C, dtype));
-        if (b > blocks) blocks = b;
+        for (int kind : {AGRAD_NORM_LAYER, AGRAD_NORM_RMS})
+            for (int dres = 0; dres < 2; ++dres) {
+                const BwdVariant v{kind, kind == AGRAD_NORM_LAYER ? 2 : 1, dres != 0};
+                const uint64_t b = bwd_blocks(vecp, rows, bwd_resident(vecp, C, dtype, v));
+                if (b > blocks) blocks = b;
+            }
     }
     return 2ull * blocks * C * sizeof(float);
 }
@@ -1020,9 +1081,12 @@ int launch_norm_bwd(hipStream_t s, int kind, int dtype, const void* x, const voi
     const bool aligned = aligned16(x) && aligned16(dy) && (!dres_in || aligned16(dres_in)) &&
                          (!dx || aligned16(dx)) && (!dx2 || aligned16(dx2)) &&
                          (!gamma || aligned16(gamma));
-    const NormPlan p = plan_norm(C, dtype, aligned, true);
-    const uint32_t grid = bwd_blocks(p, rows, bwd_resident(p, C, dtype));
+    NormPlan p = plan_norm(C, dtype, aligned, true);
     const bool want_params = dgamma != nullptr || dbeta != nullptr;
+    // an RMSNorm has no beta: a caller that asks for sum(dy) under one takes the scalar kernel
+    if (kind == AGRAD_NORM_RMS && dbeta != nullptr) p = NormPlan{true, 256, 0, 1};
+    const BwdVariant variant{kind, !want_params ? 0 : kind == AGRAD_NORM_LAYER ? 2 : 1, dres_in != nullptr};
+    const uint32_t grid = bwd_blocks(p, rows, bwd_resident(p, C, dtype, variant));
     if (rows == 0) {
         // nothing to add: stored parameter grads become zero, accumulated ones stay
         if (want_params && !(flags & AGRAD_ACC_PARAM_GRAD)) {
@@ -1040,23 +1104,25 @@ int launch_norm_bwd(hipStream_t s, int kind, int dtype, const void* x, const voi
                              (unsigned long long)workspace_bytes, (unsigned long long)need);
         if (!aligned16(workspace)) return set_error(AGRAD_EINVAL, "norm backward: workspace must be 16-byte aligned");
         float* w = (float*)workspace;
-        if (dgamma) pg = w;
-        if (dbeta) pb = w + (uint64_t)grid * C;
+        // the register-resident LayerNorm kernel keeps both sums whichever are asked for (the
+        // other's partial rows are written and not folded); the scalar kernel keeps what it is given
+        if (dgamma || (!p.generic && variant.sums == 2)) pg = w;
+        if (dbeta || (!p.generic && variant.sums == 2)) pb = w + (uint64_t)grid * C;
     }
     int rc;
     if (dtype == AGRAD_F32) {
         NormBwdArgs<float> a{(const float*)x, (const float*)dy, gamma, (const float*)dres_in,
                              (float*)dx, (float*)dx2, pg, pb, rows, C, eps, kind, flags};
-        rc = norm_bwd_typed<float>(s, p, a, grid);
+        rc = norm_bwd_typed<float>(s, p, a, grid, variant);
     } else {
         NormBwdArgs<bf16_t> a{(const bf16_t*)x, (const bf16_t*)dy, gamma, (const bf16_t*)dres_in,
                               (bf16_t*)dx, (bf16_t*)dx2, pg, pb, rows, C, eps, kind, flags};
-        rc = norm_bwd_typed<bf16_t>(s, p, a, grid);
+        rc = norm_bwd_typed<bf16_t>(s, p, a, grid, variant);
     }
     if (rc != AGRAD_OK) return rc;
     if (want_params)
-        return launch_colsum_finalize(s, pg, pb, grid, C, dgamma, dbeta, (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0,
-                                      (flags & AGRAD_PARAM_GRAD_BF16) != 0);
+        return launch_colsum_finalize(s, dgamma ? pg : nullptr, dbeta ? pb : nullptr, grid, C, dgamma, dbeta,
+                                      (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0, (flags & AGRAD_PARAM_GRAD_BF16) != 0);
     return check_hip(hipGetLastError(), "norm backward launch");
 }
 
