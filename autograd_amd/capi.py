@@ -112,6 +112,7 @@ SIGNATURES = {
     "agrad_broadcast_add_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _u64, _u64, _u64, _u32]),
     "agrad_cross_entropy_forward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u32]),
     "agrad_cross_entropy_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _u64, _u32, _u32]),
+    "agrad_cross_entropy_fused": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _u64, _u32, _u64, _f32, _u32]),
     "agrad_adamw8bit_step": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _ptr, _u64, _u64,
                                     _f32, _f32, _f32, _f32, _f32, _f32, _f32, _int]),
     "agrad_adamw_step": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u64] + [_f32] * 9),

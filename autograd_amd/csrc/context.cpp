@@ -462,6 +462,21 @@ int h_ce_bwd(const Call& c) {
     return launch_ce_bwd(c.ctx->stream, (int)c.a[0], logits, (const int32_t*)labels, (const float*)dloss,
                          (const float*)lse, dlogits, rows, V, c.a[4], c.ctx->err_flag);
 }
+// buffers logits, targets, row_loss, lse_out (the reference's order, metal_ops.metal:8808-8817), then row_scale when ROW_SCALED
+// args rows, V, row_base, scale_bits (ROW_SCALED: total_rows, unused), write_grad, dtype, present_mask
+template <bool ROW_SCALED>
+int h_ce_fused(const Call& c) {
+    NEED_DTYPE(c.a[5])
+    const uint64_t rows = c.a[0], row_base = c.a[2];
+    const uint32_t V = c.a[1], mask = c.a[6];
+    const uint64_t upto = (row_base + rows) * 4;
+    RESOLVE(0, rows * V * dtype_size(c.a[5]), logits) RESOLVE(1, upto, targets)
+    RESOLVE_IF(mask & 4u, 2, upto, row_loss) RESOLVE_IF(mask & 8u, 3, upto, lse)
+    void* row_scale = nullptr;
+    if (ROW_SCALED) { if (int rc_ = resolve(c.ctx, c.ids[4], c.offs[4], upto, "row_scale", &row_scale)) return rc_; }
+    return launch_ce_fused(c.ctx->stream, (int)c.a[5], logits, (const int32_t*)targets, (float*)row_loss, (float*)lse,
+                           (const float*)row_scale, rows, V, row_base, ROW_SCALED ? 1.0f : f32(c.a[3]), c.a[4]);
+}
 // buffers p, g, m, v | args (float bits) lr_wd, b1, 1-b1, b2, 1-b2, eps, step_lr, inv_sqrt_bc2, grad_scale,
 //                       then numel lo, hi, decay_numel lo, hi, grad dtype
 int h_adamw(const Call& c) {
@@ -533,6 +548,8 @@ const Entry kTable[] = {
     {"pos_emb_grad", 2, 5, "dY, dwpe | dtype, B, T, C, flags", h_pos_grad},
     {"cross_entropy_forward", 4, 5, "logits, labels, loss, lse | dtype, rows_lo, rows_hi, V, present_mask", h_ce_fwd},
     {"cross_entropy_backward", 5, 6, "logits, labels, dloss, lse, dlogits | dtype, rows_lo, rows_hi, V, flags, present_mask", h_ce_bwd},
+    {"fused_linear_ce_logits_to_dlogits", 4, 7, "logits (in place), targets, row_loss, lse_out | rows, V, row_base, scale_bits, write_grad, dtype, present_mask", h_ce_fused<false>},
+    {"fused_linear_ce_logits_to_dlogits_row_scaled", 5, 7, "logits (in place), targets, row_loss, lse_out, row_scale | rows, V, row_base, total_rows, write_grad, dtype, present_mask", h_ce_fused<true>},
     {"adamw_step", 4, 14, "p, g, m, v | lr_wd, b1, one_minus_b1, b2, one_minus_b2, eps, step_lr, inv_sqrt_bc2, grad_scale (float bits), n_lo, n_hi, decay_lo, decay_hi, grad_dtype", h_adamw},
     {"adamw8bit_step", 8, 11, "p, g, qm, qv, absmax_m, absmax_v, qmap_m, qmap_v | decay, lr_bc1, b1, b2, eps (float bits), numel, decay_numel, first_step, inv_sqrt_bc2 (bits), grad_bf16, clip_coef (bits)", h_adamw8bit},
     {"grad_norm_sq", 2, 3, "g, partial | n_lo, n_hi, dtype", h_grad_norm},
@@ -1048,6 +1065,12 @@ int agrad_cross_entropy_forward(agrad_ctx* ctx, int dtype, const void* logits, c
                                 float* loss, float* lse_out, uint64_t rows, uint32_t V) {
     CTX_OR_FAIL(ctx)
     return launch_ce_fwd(ctx->stream, dtype, logits, labels, loss, lse_out, rows, V, ctx->err_flag);
+}
+int agrad_cross_entropy_fused(agrad_ctx* ctx, int dtype, void* logits, const int32_t* targets, float* row_loss,
+                              float* lse, const float* row_scale, uint64_t rows, uint32_t V, uint64_t row_base,
+                              float scale, uint32_t write_grad) {
+    CTX_OR_FAIL(ctx)
+    return launch_ce_fused(ctx->stream, dtype, logits, targets, row_loss, lse, row_scale, rows, V, row_base, scale, write_grad);
 }
 int agrad_cross_entropy_backward(agrad_ctx* ctx, int dtype, const void* logits, const int32_t* labels,
                                  const float* dloss, const float* lse, void* dlogits,

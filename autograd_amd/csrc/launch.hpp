@@ -161,5 +161,10 @@ int launch_ce_fwd(hipStream_t s, int dtype, const void* logits, const int32_t* l
                   float* lse_out, uint64_t rows, uint32_t V, int* err_flag);
 int launch_ce_bwd(hipStream_t s, int dtype, const void* logits, const int32_t* labels, const float* dloss,
                   const float* lse, void* dlogits, uint64_t rows, uint32_t V, uint32_t flags, int* err_flag);
+// loss and gradient in one launch, in place: logits[r, :] becomes (softmax - onehot) * scale (row_scale[row_base + r]
+// when given), row_loss / lse [row_base + r] are written; a target outside [0, V) gives a zero row
+int launch_ce_fused(hipStream_t s, int dtype, void* logits, const int32_t* targets, float* row_loss, float* lse,
+                    const float* row_scale, uint64_t rows, uint32_t V, uint64_t row_base, float scale,
+                    uint32_t write_grad);
 
 }  // namespace agrad

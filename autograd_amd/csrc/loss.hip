@@ -30,10 +30,7 @@ namespace {
 
 constexpr int kCeBlock = 256;
 constexpr int kCeUnroll = 4;      // forward (read-only): vectors a lane keeps in flight
-#ifndef AGRAD_CE_BWD_UNROLL
-#define AGRAD_CE_BWD_UNROLL 2
-#endif
-constexpr int kCeBwdUnroll = AGRAD_CE_BWD_UNROLL;   // backward (read + write)
+constexpr int kCeBwdUnroll = 2;   // backward (read + write)
 
 template <typename T> __device__ __forceinline__ float exp_io(float x) { return exp_compensated(x); }
 template <> __device__ __forceinline__ float exp_io<bf16_t>(float x) { return __builtin_amdgcn_exp2f(x * kLog2eHi); }
@@ -354,6 +351,260 @@ int ce_typed(hipStream_t s, bool backward, const T* x, const int32_t* labels, fl
 }
 
 // ---------------------------------------------------------------------------
+// Loss and gradient in ONE launch, in place: the row of logits becomes the row of
+// (softmax - onehot) * scale, and row_loss / lse are written on the way -- the form the
+// reference uses behind its output projection (fused_linear_ce_logits_to_dlogits and its
+// per-row-scaled variant, metal_ops.metal:8808-9152; the chunk's rows are numbered from
+// row_base in targets / row_loss / lse / row_scale).  A target outside [0, V) -- an ignored
+// position -- or a row with no finite logit gives loss 0, lse 0 and a zero row, as there.
+//
+// The separate forward and backward kernels above move 3 * V * e bytes per row (the
+// logits read twice).  Here a workgroup holds its row IN REGISTERS between the statistics
+// and the rewrite -- the sixteen waves a CU gives 128 registers each are a third of a
+// megabyte -- so a row is read from memory once and written once: 2 * V * e bytes.  All of a
+// thread's loads are issued before the first wait (a thread past the end of the row loads
+// the row's first vector and ignores it: no load sits behind a branch).  fp32 rows keep
+// exp(x - max) in the registers the logits came in and the rewrite is a multiplication;
+// bf16 rows stay packed (half the registers) and take the hardware exp2 a second time.
+// Rows too long for the registers (fp32 beyond 81920 classes) take ce_fused_mem_kernel: the
+// same arithmetic with the second pass reading memory again.
+constexpr int kCeRowBlock = 1024;
+
+template <int BLOCK> __device__ __forceinline__ float block_sum(float v, float* lds);
+
+template <int BLOCK>
+__device__ __forceinline__ float block_max(float v, float* lds) {
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) v = fmaxf(v, __shfl_xor(v, off));
+    if (threadIdx.x % kWave == 0) lds[threadIdx.x / kWave] = v;
+    __syncthreads();
+    float t = lds[0];
+#pragma unroll
+    for (int w = 1; w < BLOCK / kWave; ++w) t = fmaxf(t, lds[w]);
+    __syncthreads();
+    return t;
+}
+
+// Tells the compiler that a packed vector may have changed: what it unpacked from it before is
+// unpacked again where it is next needed, instead of being kept in twice the registers.
+__device__ __forceinline__ void forget_unpacked(u32x4& r) {
+    asm volatile("" : "+v"(r.x), "+v"(r.y), "+v"(r.z), "+v"(r.w));
+}
+__device__ __forceinline__ void forget_unpacked(f32x4&) {}
+
+struct CeFusedArgs {
+    const int32_t* targets; float* row_loss; float* lse; const float* row_scale;
+    uint32_t V, row_base; float scale; uint32_t write_grad;
+};
+
+// what thread 0 leaves for the row
+__device__ __forceinline__ void ce_fused_row_results(const CeFusedArgs& a, uint32_t grow, bool valid, float lse,
+                                                     float target_logit) {
+    if (threadIdx.x == 0) {
+        if (a.row_loss != nullptr) a.row_loss[grow] = valid ? lse - target_logit : 0.0f;
+        if (a.lse != nullptr) a.lse[grow] = valid ? lse : 0.0f;
+    }
+}
+
+template <typename T, int VEC, int NV, int BLOCK>
+__global__ void __launch_bounds__(BLOCK)
+ce_fused_reg_kernel(T* x, const CeFusedArgs a) {
+    __shared__ float lds[BLOCK / kWave];
+    typedef RawVec<T, VEC> Raw;
+    const uint32_t V = a.V, tid = threadIdx.x;
+    T* base = x + (uint64_t)blockIdx.x * V;
+    const uint32_t grow = a.row_base + blockIdx.x;
+    const RowSplit<T, VEC> sp(base, V);
+    T* body = base + sp.head;
+    // every load of the row, then the few elements before and after the aligned body, then the target's logit
+    typename Raw::type raw[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint32_t idx = (uint32_t)i * BLOCK + tid;
+        raw[i] = Raw::load(body + (uint64_t)(idx < sp.nvec ? idx : 0u) * VEC);
+    }
+    const uint32_t extra = sp.head + (V - sp.tail_start);         // fewer than 2 * VEC elements
+    const uint32_t e_at = tid < sp.head ? tid : sp.tail_start + (tid - sp.head);
+    float xe = -INFINITY;
+    {
+        float t1[1];
+        VecIO<T, 1>::load(base + (tid < extra ? e_at : 0u), t1);
+        if (tid < extra) xe = t1[0];
+    }
+    const int32_t target = a.targets[grow];
+    const bool in_range = target >= 0 && (uint32_t)target < V;
+    float target_logit;
+    {
+        float t1[1];
+        VecIO<T, 1>::load(base + (in_range ? (uint32_t)target : 0u), t1);
+        target_logit = t1[0];
+    }
+
+    float m = xe;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint32_t idx = (uint32_t)i * BLOCK + tid;
+        float v[VEC];
+        Raw::unpack(raw[i], v);
+        if (idx < sp.nvec) {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) m = fmaxf(m, v[k]);
+        }
+    }
+    m = block_max<BLOCK>(m, lds);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) forget_unpacked(raw[i]);
+    const bool finite = m > -INFINITY;          // (uniform) a row of -inf has no softmax
+    const float shift = finite ? m : 0.0f;
+
+    float sum = tid < extra ? exp_io<T>(xe - shift) : 0.0f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint32_t idx = (uint32_t)i * BLOCK + tid;
+        float v[VEC];
+        Raw::unpack(raw[i], v);
+        float part = 0.0f;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            v[k] = exp_io<T>(v[k] - shift);
+            part = part + v[k];
+        }
+        if (idx < sp.nvec) sum = sum + part;
+        if constexpr (sizeof(T) == 4) raw[i] = typename Raw::type{v[0], v[1], v[2], v[3]};      // keeps exp(x - max)
+    }
+    sum = block_sum<BLOCK>(sum, lds);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) forget_unpacked(raw[i]);
+
+    const bool valid = in_range && finite && sum > 0.0f;
+    const float lse = shift + logf(sum);
+    ce_fused_row_results(a, grow, valid, lse, target_logit);
+    if ((a.write_grad & 1u) == 0u) return;
+
+    const float scale = a.row_scale != nullptr ? a.row_scale[grow] : a.scale;
+    const float inv = valid ? 1.0f / sum : 0.0f;
+    const float mul = valid ? scale : 0.0f;
+    const uint32_t hit = valid ? (uint32_t)target : 0xffffffffu;          // matches no element when the row is ignored
+    if (tid < extra) {
+        float d[1];
+        d[0] = exp_io<T>(xe - shift) * inv;
+        if (e_at == hit) d[0] = d[0] - 1.0f;
+        d[0] = d[0] * mul;
+        VecIO<T, 1>::store(base + e_at, d);
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const uint32_t idx = (uint32_t)i * BLOCK + tid;
+        float v[VEC];
+        Raw::unpack(raw[i], v);
+        const uint32_t first = sp.head + idx * VEC;
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+            float p;
+            if constexpr (sizeof(T) == 4) p = v[k] * inv;
+            else p = exp_io<T>(v[k] - shift) * inv;
+            if (first + k == hit) p = p - 1.0f;
+            v[k] = p * mul;
+        }
+        if (idx < sp.nvec) VecIO<T, VEC>::store(body + (uint64_t)idx * VEC, v);
+    }
+}
+
+// the same for rows of any length and alignment: statistics from one pass over memory, the
+// rewrite from a second (VEC == 1: element by element)
+template <typename T, int VEC>
+__global__ void __launch_bounds__(kCeRowBlock)
+ce_fused_mem_kernel(T* x, const CeFusedArgs a) {
+    __shared__ MaxSum lds[kCeRowBlock / kWave];
+    const uint32_t V = a.V, tid = threadIdx.x;
+    T* base = x + (uint64_t)blockIdx.x * V;
+    const uint32_t grow = a.row_base + blockIdx.x;
+    const int32_t target = a.targets[grow];
+    const bool in_range = target >= 0 && (uint32_t)target < V;
+    float target_logit;
+    {
+        float t1[1];
+        VecIO<T, 1>::load(base + (in_range ? (uint32_t)target : 0u), t1);
+        target_logit = t1[0];
+    }
+    const MaxSum t = row_max_sum<T, VEC, kCeRowBlock>(base, V, lds);      // (ends with a barrier: the target's logit is in)
+    const bool valid = in_range && t.m > -INFINITY && t.s > 0.0f;
+    const float lse = t.m + logf(t.s);
+    ce_fused_row_results(a, grow, valid, lse, target_logit);
+    if ((a.write_grad & 1u) == 0u) return;
+
+    const float scale = a.row_scale != nullptr ? a.row_scale[grow] : a.scale;
+    const float inv = valid ? 1.0f / t.s : 0.0f;
+    const float mul = valid ? scale : 0.0f;
+    const float shift = valid ? t.m : 0.0f;
+    const uint32_t hit = valid ? (uint32_t)target : 0xffffffffu;
+    const RowSplit<T, VEC> sp(base, V);
+    if constexpr (VEC > 1) {
+        const uint32_t extra = sp.head + (V - sp.tail_start);
+        if (tid < extra) {
+            const uint32_t e = tid < sp.head ? tid : sp.tail_start + (tid - sp.head);
+            float d[1];
+            VecIO<T, 1>::load(base + e, d);
+            d[0] = exp_io<T>(d[0] - shift) * inv;
+            if (e == hit) d[0] = d[0] - 1.0f;
+            d[0] = d[0] * mul;
+            VecIO<T, 1>::store(base + e, d);
+        }
+    }
+    T* body = base + sp.head;
+    for (uint32_t i0 = tid; i0 < sp.nvec; i0 += kCeRowBlock * kCeBwdUnroll) {
+        float v[kCeBwdUnroll][VEC];
+#pragma unroll
+        for (int u = 0; u < kCeBwdUnroll; ++u) {
+            const uint32_t i = i0 + u * kCeRowBlock;
+            VecIO<T, VEC>::load(body + (uint64_t)(i < sp.nvec ? i : 0u) * VEC, v[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < kCeBwdUnroll; ++u) {
+            const uint32_t i = i0 + u * kCeRowBlock;
+            const uint32_t first = sp.head + i * VEC;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) {
+                float p = exp_io<T>(v[u][k] - shift) * inv;
+                if (first + k == hit) p = p - 1.0f;
+                v[u][k] = p * mul;
+            }
+            if (i < sp.nvec) VecIO<T, VEC>::store(body + (uint64_t)i * VEC, v[u]);
+        }
+    }
+}
+
+// Geometry of the register-resident kernel.  Two workgroups of 512 threads share a CU when a
+// thread's share of the row leaves the kernel within 128 registers (kCeHalfMaxNV vectors: fp32
+// rows up to 40960 classes, bf16 up to 81920): one workgroup's exponentials and stores then
+// overlap the other's loads, which a lone workgroup per CU cannot do -- it reads, computes and
+// writes in turn.  Longer rows take one workgroup of 1024 threads per CU (up to kCeFullMaxNV
+// vectors a thread), and beyond that the two-pass kernel.
+constexpr int kCeHalfBlock = 512, kCeHalfMaxNV = 20, kCeFullMaxNV = 20;
+
+template <typename T>
+int ce_fused_typed(hipStream_t s, T* x, const CeFusedArgs& a, uint64_t rows) {
+    constexpr int WIDE = WideVec<T>::value;
+    const dim3 grid((uint32_t)rows);
+    // the element-wise head realigns every row to 16 bytes, which needs the element size to divide the misalignment
+    const bool wide = a.V >= 4 * WIDE && (reinterpret_cast<uintptr_t>(x) % sizeof(T)) == 0;
+    if (!wide) {
+        hipLaunchKernelGGL((ce_fused_mem_kernel<T, 1>), grid, dim3(kCeRowBlock), 0, s, x, a);
+        return check_hip(hipGetLastError(), "fused cross-entropy launch");
+    }
+    const uint32_t vectors = a.V / WIDE;                          // aligned vectors of a row, at most
+#define AGRAD_CE_REG(N, BLOCK) \
+    if (vectors <= (uint32_t)(N) * BLOCK) { hipLaunchKernelGGL((ce_fused_reg_kernel<T, WIDE, N, BLOCK>), grid, dim3(BLOCK), 0, s, x, a); return check_hip(hipGetLastError(), "fused cross-entropy launch"); }
+    AGRAD_CE_REG(4, kCeHalfBlock) AGRAD_CE_REG(8, kCeHalfBlock) AGRAD_CE_REG(12, kCeHalfBlock) AGRAD_CE_REG(16, kCeHalfBlock)
+    AGRAD_CE_REG(20, kCeHalfBlock)
+    AGRAD_CE_REG(12, kCeRowBlock) AGRAD_CE_REG(16, kCeRowBlock) AGRAD_CE_REG(20, kCeRowBlock)
+#undef AGRAD_CE_REG
+    static_assert(kCeHalfMaxNV == 20 && kCeFullMaxNV == 20, "the instantiations above");
+    hipLaunchKernelGGL((ce_fused_mem_kernel<T, WIDE>), grid, dim3(kCeRowBlock), 0, s, x, a);
+    return check_hip(hipGetLastError(), "fused cross-entropy launch");
+}
+
+// ---------------------------------------------------------------------------
 // Softmax over the last axis (cpu_softmax_forward / backward, backend.py:354-374):
 //   forward   y = exp(x - max) / sum(exp(x - max))          (a division, as on the CPU)
 //   backward  dx (+)= y * (dy - sum(dy * y))
@@ -661,6 +912,19 @@ int launch_ce_bwd(hipStream_t s, int dtype, const void* logits, const int32_t* l
     if (dtype == AGRAD_F32)
         return ce_typed<float>(s, true, (const float*)logits, labels, nullptr, nullptr, dloss, lse, (float*)dlogits, rows, V, acc, err_flag);
     return ce_typed<bf16_t>(s, true, (const bf16_t*)logits, labels, nullptr, nullptr, dloss, lse, (bf16_t*)dlogits, rows, V, acc, err_flag);
+}
+
+int launch_ce_fused(hipStream_t s, int dtype, void* logits, const int32_t* targets, float* row_loss, float* lse,
+                    const float* row_scale, uint64_t rows, uint32_t V, uint64_t row_base, float scale,
+                    uint32_t write_grad) {
+    if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "fused cross-entropy: unknown dtype %d", dtype);
+    if (rows == 0 || V == 0) return AGRAD_OK;
+    if (logits == nullptr || targets == nullptr) return set_error(AGRAD_EINVAL, "fused cross-entropy: null logits or targets");
+    if (write_grad > 1u) return set_error(AGRAD_EINVAL, "fused cross-entropy: write_grad is 0 or 1 (the fp16 gradient store of the reference is not built)");
+    if (rows > 0x7fffffffull || row_base + rows > 0xffffffffull) return set_error(AGRAD_EINVAL, "fused cross-entropy: too many rows");
+    const CeFusedArgs a{targets, row_loss, lse, row_scale, V, (uint32_t)row_base, scale, write_grad};
+    if (dtype == AGRAD_F32) return ce_fused_typed<float>(s, (float*)logits, a, rows);
+    return ce_fused_typed<bf16_t>(s, (bf16_t*)logits, a, rows);
 }
 
 int launch_softmax_fwd(hipStream_t s, int dtype, const void* x, void* y, uint64_t rows, uint32_t V) {

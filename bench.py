@@ -58,6 +58,7 @@ HBM_PEAK_GBS = 8000.0
 TRAFFIC_FILE = ROOT / "profiles" / "hbm_traffic.json"
 ROTATE_BYTES = 768 << 20      # cycle at least this much distinct memory per op
 MAX_SETS = 8
+FOLD_EVERY = 24               # norm backward calls whose column sums one batched fold takes (a 12-layer network has 25)
 
 
 def vp(d, off=0):
@@ -221,8 +222,26 @@ def _norm_cases(ctx, cfg, pool, rng, nbytes, ids0):
             ctx.call("agrad_norm_backward", kind, dt, vp(a[i]), vp(c[i]), vp(gamma), vp(b[i]) if res else None,
                      vp(d[i]), None, vp(dgamma), vp(dbeta), vp(ws), ws_bytes, N, Cw, cfg.norm_eps, 0)
 
+        # The same backward call with its dgamma / dbeta fold left pending (AGRAD_DEFER_PARAM_GRAD) and ONE
+        # launch folding FOLD_EVERY calls' sums, the way Runtime.backward_graph ends a pass over a network
+        # with that many norms; every pending call has its own workspace and gradient rows.
+        d_ws = [pool.raw(ws_bytes) for _ in range(FOLD_EVERY)]
+        d_dgamma = [pool.empty(Cw, "f32") for _ in range(FOLD_EVERY)]
+        d_dbeta = [pool.empty(Cw, "f32") if beta is not None else None for _ in range(FOLD_EVERY)]
+        calls = [0]
+
+        def bwd_deferred(i):
+            j = calls[0] % FOLD_EVERY
+            ctx.call("agrad_norm_backward", kind, dt, vp(a[i]), vp(c[i]), vp(gamma), vp(b[i]) if res else None,
+                     vp(d[i]), None, vp(d_dgamma[j]), vp(d_dbeta[j]), vp(d_ws[j]), ws_bytes, N, Cw, cfg.norm_eps,
+                     capi.DEFER_PARAM_GRAD)
+            calls[0] += 1
+            if calls[0] % FOLD_EVERY == 0:
+                ctx.call("agrad_finalize_param_grads")
+
         cases.append(Case(name, "fwd", nbytes[name][0], k, fwd, "norm_fwd_kernel"))
         cases.append(Case(name, "bwd", nbytes[name][1], k, bwd, "norm_bwd_kernel"))
+        cases.append(Case(name, f"bwd-fold/{FOLD_EVERY}", nbytes[name][1], k, bwd_deferred, "norm_bwd_kernel"))
     return cases
 
 
@@ -420,9 +439,15 @@ def _loss_cases(ctx, cfg, pool, rng, nbytes, ids0):
     def bwd(i):
         ctx.call("agrad_cross_entropy_backward", dt, vp(logits[i]), vp(labels), vp(dloss), vp(lse), vp(dlogits[i]), N, V, 0)
 
+    def fused(i):
+        # loss and gradient in one launch, in place: reads the row once, writes it once (the gradient a
+        # call leaves is the next call's logits: any finite values time alike)
+        ctx.call("agrad_cross_entropy_fused", dt, vp(logits[i]), vp(labels), vp(loss), vp(lse), None, N, V, 0, 1.0 / N, 1)
+
     fwd(0)   # lse for the backward timing
     return [Case("cross_entropy", "loss-fwd", N * V * e + 12 * N, k, fwd, "ce_fwd_kernel"),
-            Case("cross_entropy", "loss-bwd", 2 * N * V * e + 12 * N, k, bwd, "ce_bwd_kernel")]
+            Case("cross_entropy", "loss-bwd", 2 * N * V * e + 12 * N, k, bwd, "ce_bwd_kernel"),
+            Case("cross_entropy_fused", "loss-both", 2 * N * V * e + 12 * N, k, fused, "ce_fused_")]
 
 
 def _opt_cases(ctx, cfg, pool, rng, nbytes, ids0):

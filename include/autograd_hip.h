@@ -429,6 +429,21 @@ int agrad_cross_entropy_backward(agrad_ctx* ctx, int dtype, const void* logits, 
                                  const float* dloss, const float* lse, void* dlogits,
                                  uint64_t rows, uint32_t V, uint32_t flags);
 
+/* Loss and gradient of a chunk of rows in ONE launch, in place
+ * (fused_linear_ce_logits_to_dlogits and ..._row_scaled, metal_ops.metal:8808-9152; called behind the
+ * output projection, backend.py:3175-3179, 3337-3342).  For local row r of logits[rows, V] and
+ * g = row_base + r:  row_loss[g] = lse - x[r, targets[g]],  lse[g] = max + log(sum exp(x - max)), and -- when
+ * write_grad is 1 -- logits[r, :] is REPLACED by (softmax(x[r, :]) - onehot(targets[g])) * s, with
+ * s = row_scale[g] when row_scale is given, else `scale`.  A target outside [0, V) (an ignored position)
+ * or a row without a finite logit gives loss 0, lse 0 and a zero row, as in the reference; no index
+ * error is raised.  row_loss and lse may be NULL.  The row is read from memory once (a 1024-thread
+ * workgroup holds it in registers between the statistics and the rewrite) while it has at most 81920
+ * fp32 or 163840 bf16 classes, twice beyond.  The fp16 gradient store of the reference (write_grad
+ * bit 1, which feeds its fp16 GEMM) is not built. */
+int agrad_cross_entropy_fused(agrad_ctx* ctx, int dtype, void* logits, const int32_t* targets,
+                              float* row_loss, float* lse, const float* row_scale,
+                              uint64_t rows, uint32_t V, uint64_t row_base, float scale, uint32_t write_grad);
+
 /* ---- optimizer step over the parameter slab (the consumer of the gradients above) ---- */
 
 /* One AdamW step on numel fp32 parameters with fp32 moments, in place; the

@@ -488,6 +488,33 @@ def cross_entropy_backward_into(x, labels, dloss, dx):
     np.add(dx, f, out=dx)
 
 
+def cross_entropy_fused(x, targets, scale, row_scale=None, write_grad=True):
+    """The one-kernel form behind the reference's output projection
+    (fused_linear_ce_logits_to_dlogits, metal_ops.metal:8808-8996; row-scaled :8997-9152): returns
+    (row_loss, lse, dlogits) for logits x [rows, V] and int targets [rows].  A row whose target lies
+    outside [0, V) (an ignored position, metal_ops.metal:8919-8926) or that has no finite logit has
+    loss 0, lse 0 and a zero gradient row; every other row is the composition of
+    cross_entropy_forward and cross_entropy_backward_into with dloss = scale (or row_scale[r])."""
+    x = np.asarray(x, np.float32)
+    rows, V = x.shape
+    t = np.asarray(targets).astype(np.int64)
+    ok = (t >= 0) & (t < V) & np.isfinite(np.max(x, axis=-1))
+    safe = np.where(ok, t, 0)
+    xs = np.where(ok[:, None], x, np.float32(0.0)).astype(np.float32)
+    loss = cross_entropy_forward(xs, safe)
+    m = np.max(xs, axis=-1)
+    lse = (m + np.log(np.sum(np.exp(xs - m[:, None]), axis=-1, dtype=np.float32))).astype(np.float32)
+    loss = np.where(ok, loss, np.float32(0.0)).astype(np.float32)
+    lse = np.where(ok, lse, np.float32(0.0)).astype(np.float32)
+    if not write_grad:
+        return loss, lse, None
+    dl = (np.full(rows, scale, np.float32) if row_scale is None else np.asarray(row_scale, np.float32))
+    dx = np.zeros_like(xs)
+    cross_entropy_backward_into(xs, safe, dl, dx)
+    dx[~ok] = 0.0
+    return loss, lse, dx
+
+
 # --------------------------------------------------------------------------
 # AdamW  (cpu_adamw_step, backend.py:2013-2038; the step size lr_t comes from
 # optimizer.py:445)

@@ -146,3 +146,125 @@ def test_cross_entropy_through_the_runtime():
         rt.release()
     assert_fp32_close(results["hip"][0], results["cpu"][0], "loss")
     assert_fp32_close(results["hip"][1], results["cpu"][1], "dlogits")
+
+
+# ---- loss and gradient in one launch, in place (fused_linear_ce_logits_to_dlogits) ---------------
+def run_fused(ctx, x_store, targets, dtype, scale=1.0, row_scale=None, row_base=0, write_grad=1, offset_elems=0,
+              want_loss=True, want_lse=True):
+    rows, V = x_store.shape
+    esz = x_store.dtype.itemsize
+    pad = np.zeros(offset_elems, x_store.dtype)
+    d_x = ctx.upload(np.concatenate([pad, x_store.reshape(-1)]))
+    total = row_base + rows
+    tg = np.full(total, -5, np.int32)
+    tg[row_base:] = targets
+    d_t = ctx.upload(tg)
+    loss = ctx.upload(np.full(total, -7.0, np.float32))
+    lse = ctx.upload(np.full(total, -7.0, np.float32))
+    d_rs = None
+    if row_scale is not None:
+        full = np.zeros(total, np.float32)
+        full[row_base:] = row_scale
+        d_rs = ctx.upload(full)
+    ctx.call("agrad_cross_entropy_fused", dtype, vp(d_x, offset_elems * esz), vp(d_t), vp(loss) if want_loss else None,
+             vp(lse) if want_lse else None, vp(d_rs), rows, V, row_base, float(scale), write_grad)
+    ctx.synchronize()
+    out = loss.download(), lse.download(), d_x.download()[offset_elems:].reshape(x_store.shape)
+    for d in (d_x, d_t, loss, lse, d_rs):
+        if d is not None:
+            d.free()
+    return out
+
+
+# every register geometry (4 ... 20 vectors a thread), the second pass from memory (fp32 beyond 81920 classes),
+# odd row lengths (rows start at any alignment), tiny rows (element by element)
+FUSED_SHAPES = [(1, 1), (3, 7), (5, 64), (4, 1000), (6, 4099), (3, 32768), (2, 50257), (2, 65536), (2, 81920), (1, 128256),
+                (2, 151936)]
+
+
+@pytest.mark.parametrize("rows,V", FUSED_SHAPES)
+def test_fused_cross_entropy_fp32(ctx, rows, V):
+    rng = np.random.default_rng(190 + V)
+    x = (4.0 * rng.standard_normal((rows, V))).astype(np.float32)
+    t = rng.integers(0, V, rows, dtype=np.int32)
+    if rows >= 3:
+        t[1] = -1                       # an ignored position
+    scale = 1.0 / 16384
+    loss, lse, dx = run_fused(ctx, x, t, capi.F32, scale=scale, row_base=5)
+    w_loss, w_lse, w_dx = K.cross_entropy_fused(x, t, np.float32(scale))
+    assert_fp32_close(loss[5:], w_loss, "loss")
+    assert_fp32_close(lse[5:], w_lse, "lse")
+    np.testing.assert_array_equal(loss[:5], np.full(5, -7.0, np.float32))      # rows before row_base are not touched
+    # the gradient against the restatement at the scale's size (values are p * 6e-5), and against float64
+    assert_fp32_close(dx / np.float32(scale), w_dx / np.float32(scale), "dlogits")
+    ok = t >= 0
+    if ok.any():
+        assert np.abs(dx[ok] / scale - cf.cross_entropy_grad(x[ok], t[ok], np.ones(int(ok.sum()), np.float32))).max() <= 2e-6
+    assert not dx[~ok].any()
+
+
+@pytest.mark.parametrize("rows,V", [(5, 64), (4, 1000), (3, 32768), (2, 50257), (2, 128256), (2, 151936)])
+def test_fused_cross_entropy_bf16(ctx, rows, V):
+    rng = np.random.default_rng(290 + V)
+    x = from_bf16_bits(to_bf16_bits((4.0 * rng.standard_normal((rows, V))).astype(np.float32)))
+    t = rng.integers(0, V, rows, dtype=np.int32)
+    rs = rng.standard_normal(rows).astype(np.float32)
+    loss, lse, dx = run_fused(ctx, to_bf16_bits(x), t, capi.BF16, row_scale=rs)
+    w_loss, w_lse, w_dx = K.cross_entropy_fused(x, t, 1.0, row_scale=rs)
+    np.testing.assert_allclose(loss, w_loss, rtol=2e-5, atol=2e-5)
+    np.testing.assert_allclose(lse, w_lse, rtol=2e-5, atol=2e-5)
+    assert_bf16_close(from_bf16_bits(dx), w_dx, "dlogits (bf16)")
+
+
+def test_fused_cross_entropy_masks_unaligned_and_loss_only(ctx):
+    rng = np.random.default_rng(391)
+    rows, V = 6, 1537
+    x = (3.0 * rng.standard_normal((rows, V))).astype(np.float32)
+    x[2, 10:40] = -np.inf               # masked classes
+    x[4, :] = -np.inf                   # a row with no finite logit: zero row, loss 0
+    t = rng.integers(0, V, rows, dtype=np.int32)
+    t[5] = V                            # out of range above
+    for off in (0, 1, 3):               # the tensor itself starts 0, 4 or 12 bytes past a 16-byte boundary
+        loss, lse, dx = run_fused(ctx, x, t, capi.F32, scale=0.5, offset_elems=off)
+        w_loss, w_lse, w_dx = K.cross_entropy_fused(x, t, np.float32(0.5))
+        assert_fp32_close(loss, w_loss, f"loss off={off}")
+        assert_fp32_close(lse, w_lse, f"lse off={off}")
+        assert_fp32_close(dx, w_dx, f"dlogits off={off}")
+        assert not dx[4].any() and not dx[5].any() and not np.isnan(dx).any()
+    # write_grad = 0: the logits stay as they were
+    loss, lse, same = run_fused(ctx, x, t, capi.F32, write_grad=0)
+    np.testing.assert_array_equal(same, x)
+    assert_fp32_close(loss, w_loss, "loss only")
+    # NULL loss / lse outputs are allowed
+    _, _, dx = run_fused(ctx, x, t, capi.F32, scale=0.5, want_loss=False, want_lse=False)
+    assert_fp32_close(dx, w_dx, "dlogits without loss outputs")
+    with pytest.raises(capi.AgradError):
+        run_fused(ctx, x, t, capi.F32, write_grad=2)
+
+
+def test_fused_cross_entropy_through_the_name_dispatch(ctx):
+    """the reference's kernel names and argument order (backend.py:3175-3179)"""
+    import ctypes as C
+    from autograd_amd.utils import f32_bits
+    rng = np.random.default_rng(392)
+    rows, V = 7, 2048
+    x = (2.0 * rng.standard_normal((rows, V))).astype(np.float32)
+    t = rng.integers(0, V, rows, dtype=np.int32)
+    rs = rng.standard_normal(rows).astype(np.float32)
+    for scaled in (False, True):
+        d_x, d_t = ctx.upload(x), ctx.upload(t)
+        loss, lse = ctx.upload(np.zeros(rows, np.float32)), ctx.upload(np.zeros(rows, np.float32))
+        d_rs = ctx.upload(rs)
+        bufs = [d_x, d_t, loss, lse] + ([d_rs] if scaled else [])
+        ids = (C.c_uint64 * len(bufs))(*[b.ptr for b in bufs])
+        offs = (C.c_uint64 * len(bufs))(*([0] * len(bufs)))
+        args = [rows, V, 0, rows if scaled else f32_bits(0.25), 1, capi.F32, 0b1111]
+        a = (C.c_uint32 * len(args))(*args)
+        name = b"fused_linear_ce_logits_to_dlogits_row_scaled" if scaled else b"fused_linear_ce_logits_to_dlogits"
+        ctx.call("agrad_dispatch", name, ids, offs, len(bufs), a, len(args), 0, 0, 0, 0)
+        ctx.synchronize()
+        w_loss, w_lse, w_dx = K.cross_entropy_fused(x, t, np.float32(0.25), row_scale=rs if scaled else None)
+        assert_fp32_close(loss.download(), w_loss, "loss")
+        assert_fp32_close(d_x.download(), w_dx, "dlogits")
+        for b in bufs + ([] if scaled else [d_rs]):
+            b.free()

@@ -572,6 +572,39 @@ def test_cross_entropy_closed_form_fd_and_invariants():
         assert abs(val - dx.reshape(-1)[i]) < 2e-3 * max(1.0, abs(val))
 
 
+def test_cross_entropy_fused_is_the_pair_with_ignored_rows_zeroed():
+    """the one-kernel form (metal_ops.metal:8808-8996): scipy's logsumexp / softmax in float64 for
+    the valid rows; an out-of-range target or a row of -inf gives loss 0, lse 0 and a zero row"""
+    from scipy.special import logsumexp, softmax
+    r = rng(51)
+    rows, V = 9, 53
+    x = (3.0 * r.standard_normal((rows, V))).astype(np.float32)
+    t = r.integers(0, V, rows).astype(np.int32)
+    t[2], t[5] = -1, V           # ignored positions
+    x[7, :] = -np.inf            # no finite logit
+    x[8, 3] = -np.inf            # a masked class in an ordinary row
+    scale = np.float32(0.37)
+    loss, lse, dx = K.cross_entropy_fused(x, t, scale)
+    ok = np.array([i not in (2, 5, 7) for i in range(rows)])
+    x64 = x.astype(np.float64)
+    want_lse = logsumexp(x64[ok], axis=-1)
+    close(lse[ok], want_lse)
+    close(loss[ok], want_lse - x64[ok, t[ok]])
+    p = softmax(x64[ok], axis=-1)
+    p[np.arange(ok.sum()), t[ok]] -= 1.0
+    close(dx[ok], p * float(scale))
+    assert not loss[~ok].any() and not lse[~ok].any() and not dx[~ok].any()
+    assert dx[8, 3] == 0.0
+    # per-row scales, and the loss-only call
+    rs = r.standard_normal(rows).astype(np.float32)
+    _, _, dx2 = K.cross_entropy_fused(x, t, 1.0, row_scale=rs)
+    close(dx2[ok], p * rs[ok, None].astype(np.float64))
+    l3, s3, none = K.cross_entropy_fused(x, t, scale, write_grad=False)
+    assert none is None
+    np.testing.assert_array_equal(l3, loss)
+    np.testing.assert_array_equal(s3, lse)
+
+
 # ---------------------------------------------------------------------------
 # strided views and the permute / transpose gradients: an explicit loop over every
 # dense index with the index arithmetic written out
