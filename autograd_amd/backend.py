@@ -133,6 +133,7 @@ def _mask(*present):
 class HipBackend(Backend):
     supports_grad_store = True   # kernels take a store / accumulate flag per gradient
     supports_deferred_param_grads = True    # column sums of a pass can be folded in one launch at its end
+    single_pass_execute = True   # Runtime.execute runs zero_grad + forward + backward as ONE pass (one wait)
 
     def __init__(self, ctx=None):
         if ctx is None:

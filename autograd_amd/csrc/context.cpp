@@ -17,7 +17,11 @@ struct agrad_ctx {
     int device = 0;
     hipStream_t stream = nullptr;
     hipEvent_t ev_start = nullptr, ev_stop = nullptr;
-    int* err_flag = nullptr;               // device word set by kernels that see a bad token id
+    // The word kernels set when they see a token id or a class label out of range.  It lives in
+    // pinned host memory that the GPU writes directly: the pass boundary reads it without a copy
+    // (a blocking device-to-host copy per end_pass was a tenth of a small training step).
+    int* err_flag = nullptr;               // the GPU's address of the word
+    volatile int* err_host = nullptr;      // the host's address of the same word
     uint64_t total_mem = 0;
     std::mutex mu;
     std::map<uint64_t, uint64_t> allocs;   // base address -> bytes
@@ -103,10 +107,8 @@ int finish_stream(agrad_ctx* ctx) {
     if (int rc = no_capture(ctx, "synchronize / end_pass")) return rc;
     if (int rc = flush_pending(ctx)) return rc;      // nothing a caller waits for stays unfolded
     if (int rc = check_hip(hipStreamSynchronize(ctx->stream), "stream synchronize")) return rc;
-    int flag = 0;
-    if (int rc = check_hip(hipMemcpy(&flag, ctx->err_flag, sizeof(int), hipMemcpyDeviceToHost), "error flag read")) return rc;
-    if (flag != 0) {
-        (void)hipMemset(ctx->err_flag, 0, sizeof(int));
+    if (*ctx->err_host != 0) {                 // (the stream has drained: every kernel's write has landed)
+        *ctx->err_host = 0;
         return set_error(AGRAD_EINDEX, "index out of range on the device (a token id or a class label)");
     }
     return AGRAD_OK;
@@ -603,8 +605,13 @@ int agrad_ctx_create(int device, agrad_ctx** out) {
     hipError_t e = hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking);
     if (e == hipSuccess) e = hipEventCreate(&c->ev_start);
     if (e == hipSuccess) e = hipEventCreate(&c->ev_stop);
-    if (e == hipSuccess) e = hipMalloc((void**)&c->err_flag, 256);
-    if (e == hipSuccess) e = hipMemset(c->err_flag, 0, 256);
+    void* pinned = nullptr;
+    if (e == hipSuccess) e = hipHostMalloc(&pinned, 256, hipHostMallocMapped);
+    if (e == hipSuccess) {
+        std::memset(pinned, 0, 256);
+        c->err_host = static_cast<volatile int*>(pinned);
+        e = hipHostGetDevicePointer((void**)&c->err_flag, pinned, 0);
+    }
     if (e != hipSuccess) {
         agrad_ctx_destroy(c);
         return check_hip(e, "context setup");
@@ -619,7 +626,7 @@ int agrad_ctx_destroy(agrad_ctx* ctx) {
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     for (auto& kv : ctx->graphs) (void)hipGraphExecDestroy(kv.second);
     for (auto& kv : ctx->allocs) (void)hipFree(reinterpret_cast<void*>(kv.first));
-    if (ctx->err_flag) (void)hipFree(ctx->err_flag);
+    if (ctx->err_host) (void)hipHostFree(const_cast<int*>(ctx->err_host));
     if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
     if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
     if (ctx->stream) (void)hipStreamDestroy(ctx->stream);

@@ -462,6 +462,20 @@ class Runtime:
         if self.forward_only:
             self.forward()
             return
+        if getattr(self.backend, "single_pass_execute", False):
+            # one pass, one wait at its end, as the reference runs its GPU device
+            # (runtime.py:818-826): a pass boundary drains the GPU, and two of them per
+            # step (forward, then backward) are a tenth of a small step
+            self._require_bound()
+            self._sync_backend()
+            self.backend.begin_pass()
+            if not self.accumulate_parameter_grads:
+                self.zero_grad()
+            self._forward_nodes()
+            self.backend.fill(self.loss.grad, self.grad_scale)
+            self._backward_nodes()
+            self.backend.end_pass()
+            return
         if not self.accumulate_parameter_grads:
             self.zero_grad()
         self.forward()
@@ -494,18 +508,11 @@ class Runtime:
         if self.memory_plan is not None and self.arena_bytes and self.unified_arena is None:
             raise RuntimeError("this runtime's memory is planned but not bound: call bind_memory_new / bind_to first")
 
-    def forward(self):
-        self._require_bound()
-        self._sync_backend()
-        self.backend.begin_pass()
+    def _forward_nodes(self):
         for node in self.topo:
             node.forward(node.inputs, node.outputs)
-        self.backend.end_pass()
 
-    def backward_graph(self):
-        self._require_bound()
-        self._sync_backend()
-        self.backend.begin_pass()
+    def _backward_nodes(self):
         for node in reversed(self.topo):
             for t in self.node_to_clear_grads.get(id(node), ()):
                 if t.grad is not None:
@@ -513,6 +520,19 @@ class Runtime:
             node.backward(node.inputs, node.outputs)
         if self.defer_param_grad_sums:
             self.backend.finalize_param_grads()
+
+    def forward(self):
+        self._require_bound()
+        self._sync_backend()
+        self.backend.begin_pass()
+        self._forward_nodes()
+        self.backend.end_pass()
+
+    def backward_graph(self):
+        self._require_bound()
+        self._sync_backend()
+        self.backend.begin_pass()
+        self._backward_nodes()
         self.backend.end_pass()
 
     def capture(self, fn):
