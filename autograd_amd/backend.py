@@ -545,11 +545,26 @@ class HipBackend(Backend):
     # When the table needs a gradient the op carries an `order` output: the forward
     # kernel then also orders the ids (one launch, beside the gather) and the
     # backward kernel starts at the segmented sum.
+    def zero_grad_and_order(self, node, table):
+        """table.grad = 0 and the order of the node's ids for its backward kernel, in one launch
+        (the ordering workgroups ride at the front of the fill's grid); the node's forward
+        kernel is then the plain gather.  False when this node cannot take it."""
+        indices = node.inputs[0]
+        scratch = getattr(node.forward, "keywords", {}).get("scratch")
+        if len(node.outputs) < 2 or indices.op is not None or table.grad is None or scratch is None \
+                or "sort_workspace" not in scratch:
+            return False
+        ws, g = scratch["sort_workspace"], table.grad.storage
+        self._launch("embedding_order", [indices, node.outputs[1], ws, g],
+                     [prod(indices.shape), table.shape[0]] + _lo_hi(ws.nbytes) + _lo_hi(g.nbytes) + [0b1111])
+        node.order_ready = True
+        return True
+
     def _embedding_forward(self, indices, table, wpe, outputs, scratch):
         out = outputs[0]
         V, C = table.shape
         B, T = indices.shape
-        if len(outputs) > 1:
+        if len(outputs) > 1 and not out.op.order_ready:
             if scratch is None:
                 raise RuntimeError("embedding forward needs its arena workspace (plan_scratch)")
             ws = scratch["sort_workspace"]
@@ -587,6 +602,7 @@ class HipBackend(Backend):
             self._launch("gather_backward_sorted", [outputs[1], out.grad, weight.grad, ws, dwpe],
                          [_dt(weight), prod(indices.shape), C, V, flag] + _lo_hi(ws.nbytes)
                          + [T, _mask(outputs[1], out.grad, weight.grad, ws, dwpe)])
+            node.order_ready = False        # the next forward pass orders its own ids unless told otherwise
             return wpe is not None
         else:
             self._launch("gather_backward_kernel", [indices, out.grad, weight.grad, ws],

@@ -431,7 +431,7 @@ int h_gather_bwd_sorted(const Call& c) {
     const uint64_t gs = (c.a[4] & AGRAD_PARAM_GRAD_BF16) ? 2 : es;      // element size of the table gradients
     RESOLVE(0, (N * 6 + 128) * 4, order) RESOLVE(1, N * C * es, dY) RESOLVE(2, (uint64_t)V * C * gs, dW) RESOLVE(3, wsb, ws)
     RESOLVE_IF(mask & 16u, 4, (uint64_t)T * C * gs, dwpe)
-    return launch_embedding_bwd_sorted(c.ctx->stream, (int)c.a[0], (const uint32_t*)order, dY, dW, dwpe, ws, wsb, N, T,
+    return launch_embedding_bwd_sorted(c.ctx->stream, (int)c.a[0], (uint32_t*)order, dY, dW, dwpe, ws, wsb, N, T,
                                        C, V, c.a[4]);
 }
 // buffers dY, dwpe | args dtype, B, T, C, flags
@@ -478,6 +478,14 @@ int h_ce_fused(const Call& c) {
     if (ROW_SCALED) { if (int rc_ = resolve(c.ctx, c.ids[4], c.offs[4], upto, "row_scale", &row_scale)) return rc_; }
     return launch_ce_fused(c.ctx->stream, (int)c.a[5], logits, (const int32_t*)targets, (float*)row_loss, (float*)lse,
                            (const float*)row_scale, rows, V, row_base, ROW_SCALED ? 1.0f : f32(c.a[3]), c.a[4]);
+}
+// buffers ids, order, sort_workspace, zero_dst | args N, V, ws_lo, ws_hi, zero_lo, zero_hi, present_mask
+int h_emb_order(const Call& c) {
+    const uint64_t N = c.a[0], wsb = u64(c.a, 2), zb = u64(c.a, 4);
+    RESOLVE(0, N * 4, ids) RESOLVE(1, embedding_order_bytes(N), order) RESOLVE(2, wsb, ws)
+    RESOLVE_IF(c.a[6] & 8u, 3, zb, zero_dst)
+    return launch_embedding_order(c.ctx->stream, (const int32_t*)ids, (uint32_t*)order, ws, wsb, N, c.a[1], zero_dst,
+                                  zero_dst ? zb : 0, c.ctx->err_flag);
 }
 // buffers p, g, m, v | args (float bits) lr_wd, b1, 1-b1, b2, 1-b2, eps, step_lr, inv_sqrt_bc2, grad_scale,
 //                       then numel lo, hi, decay_numel lo, hi, grad dtype
@@ -552,6 +560,7 @@ const Entry kTable[] = {
     {"cross_entropy_backward", 5, 6, "logits, labels, dloss, lse, dlogits | dtype, rows_lo, rows_hi, V, flags, present_mask", h_ce_bwd},
     {"fused_linear_ce_logits_to_dlogits", 4, 7, "logits (in place), targets, row_loss, lse_out | rows, V, row_base, scale_bits, write_grad, dtype, present_mask", h_ce_fused<false>},
     {"fused_linear_ce_logits_to_dlogits_row_scaled", 5, 7, "logits (in place), targets, row_loss, lse_out, row_scale | rows, V, row_base, total_rows, write_grad, dtype, present_mask", h_ce_fused<true>},
+    {"embedding_order", 4, 7, "ids, order, sort_workspace, zero_dst | N, V, ws_lo, ws_hi, zero_lo, zero_hi, present_mask", h_emb_order},
     {"adamw_step", 4, 14, "p, g, m, v | lr_wd, b1, one_minus_b1, b2, one_minus_b2, eps, step_lr, inv_sqrt_bc2, grad_scale (float bits), n_lo, n_hi, decay_lo, decay_hi, grad_dtype", h_adamw},
     {"adamw8bit_step", 8, 11, "p, g, qm, qv, absmax_m, absmax_v, qmap_m, qmap_v | decay, lr_bc1, b1, b2, eps (float bits), numel, decay_numel, first_step, inv_sqrt_bc2 (bits), grad_bf16, clip_coef (bits)", h_adamw8bit},
     {"grad_norm_sq", 2, 3, "g, partial | n_lo, n_hi, dtype", h_grad_norm},
@@ -1037,10 +1046,16 @@ int agrad_gather_forward_sorted(agrad_ctx* ctx, int dtype, const int32_t* ids, c
     return launch_gather_fwd_sorted(ctx->stream, dtype, ids, W, wpe, out, N, T, C, V, order, sort_workspace,
                                     sort_workspace_bytes, ctx->err_flag);
 }
+int agrad_embedding_order(agrad_ctx* ctx, const int32_t* ids, uint64_t N, uint32_t V, uint32_t* order,
+                          void* sort_workspace, uint64_t sort_workspace_bytes, void* zero_dst, uint64_t zero_bytes) {
+    CTX_OR_FAIL(ctx)
+    return launch_embedding_order(ctx->stream, ids, order, sort_workspace, sort_workspace_bytes, N, V, zero_dst, zero_bytes,
+                                  ctx->err_flag);
+}
 uint64_t agrad_embedding_backward_sorted_workspace_bytes(uint64_t N, uint32_t C) {
     return embedding_bwd_sorted_workspace_bytes(N, C);
 }
-int agrad_embedding_backward_sorted(agrad_ctx* ctx, int dtype, const uint32_t* order, const void* dY, void* dW,
+int agrad_embedding_backward_sorted(agrad_ctx* ctx, int dtype, uint32_t* order, const void* dY, void* dW,
                                     void* dwpe, void* workspace, uint64_t workspace_bytes, uint64_t N, uint32_t T,
                                     uint32_t C, uint32_t V, uint32_t flags) {
     CTX_OR_FAIL(ctx)

@@ -765,6 +765,28 @@ gather_sort_kernel(const int32_t* __restrict__ ids, const T* __restrict__ W, con
     }
 }
 
+// The ordering of the ids at the front of the zero fill of the table's gradient: one launch for
+// a caller that clears dW and orders the ids before its forward pass and then gathers with the
+// plain kernel.  Measured on MI355X it is the worse of the two hosts: the fill alone runs best
+// with few waves on a CU, this kernel's 512-thread workgroups (the ordering's shape) fill at full
+// occupancy (a tenth slower), and the launch takes 3 us (50 MB table) to 25 us (1 GB) longer than
+// the plain fill where the same ordering workgroups cost the forward gather 1 to 3 us -- which is
+// why the forward call keeps them.  It still beats a fill and an ordering launched one after the
+// other (8 us more at 16384 ids, 44 us at 65536).
+constexpr uint32_t kFillOrderIdleLds = 0;      // dynamic LDS that nothing touches (an occupancy cap): none pays here
+
+__global__ void __launch_bounds__(kSortBlock) __attribute__((amdgpu_num_sgpr(80)))
+fill_order_kernel(const int32_t* __restrict__ ids, uint32_t* __restrict__ order, unsigned long long* __restrict__ spill,
+                  uint32_t N, uint32_t V, uint32_t log2G, int* err_flag, u32x4* __restrict__ dst, uint64_t vectors) {
+    const uint32_t groups = 1u << log2G;
+    if (blockIdx.x < groups) {
+        emb_group_sort_body(blockIdx.x, ids, order, spill, N, V, log2G, err_flag);
+        return;
+    }
+    const uint64_t i = (uint64_t)(blockIdx.x - groups) * kSortBlock + threadIdx.x;
+    if (i < vectors) __builtin_nontemporal_store(u32x4{0u, 0u, 0u, 0u}, dst + i);
+}
+
 template <typename T, int VEC>
 __device__ __forceinline__ void store_grad_row(T* dW, uint64_t off, const float (&acc)[VEC], bool accumulate) {
     float o[VEC];
@@ -1269,7 +1291,7 @@ inline uint64_t order_bytes(uint64_t N) { return align256(order_words(N) * 4); }
 inline uint64_t partial_rows(uint64_t N) { return N / kChunkRows + 1 + N / (kChunkRows * kGroupChunks) + 1; }
 
 template <typename T, typename TO = T>
-int embedding_sum_typed(hipStream_t s, const uint32_t* order, const T* dY, TO* dW, float* part, uint32_t N, uint32_t C,
+int embedding_sum_typed(hipStream_t s, uint32_t* order, const T* dY, TO* dW, float* part, uint32_t N, uint32_t C,
                         uint32_t V, uint32_t flags, TO* dwpe, uint32_t B, uint32_t T_len) {
     const int acc = (flags & AGRAD_ACC_PARAM_GRAD) ? 1 : 0;
     const int acc_pos = (flags & AGRAD_ACC_PARAM_GRAD2) ? 1 : 0;
@@ -1298,7 +1320,7 @@ int embedding_sum_typed(hipStream_t s, const uint32_t* order, const T* dY, TO* d
     const uint32_t block = waves * kWave;
 #define AGRAD_ROW_SUM(VEC, KW, POS) \
     hipLaunchKernelGGL((emb_row_sum_kernel<T, TO, VEC, KW, POS>), dim3(grid), dim3(block), 0, s, order, \
-                       const_cast<uint32_t*>(order) + order_ticket_word(N), dY, dW, dwpe, part, N, C, CV, CB, V, T_len, B, \
+                       order + order_ticket_word(N), dY, dW, dwpe, part, N, C, CV, CB, V, T_len, B, \
                        acc, acc_pos, tg)
     if (dwpe) {
         if (wide) AGRAD_ROW_SUM(WIDE, 1, true); else AGRAD_ROW_SUM(1, 1, true);
@@ -1377,6 +1399,38 @@ int launch_embedding_sort(hipStream_t s, const int32_t* ids, uint32_t* order, vo
     return check_hip(hipGetLastError(), "embedding order launch");
 }
 
+// order = the ids' ordering for the later gradient and, in the same launch where the shapes
+// allow, zero_dst[0 .. zero_bytes) = 0 (the table's gradient, cleared before the backward pass)
+int launch_embedding_order(hipStream_t s, const int32_t* ids, uint32_t* order, void* sort_workspace,
+                           uint64_t sort_workspace_bytes, uint64_t N, uint32_t V, void* zero_dst, uint64_t zero_bytes,
+                           int* err_flag) {
+    if (zero_dst == nullptr) zero_bytes = 0;
+    const uint64_t vectors = zero_bytes / 16;
+    const bool fused = N > 0 && N <= kGroupSortMaxN && zero_bytes > 0 && zero_bytes % 16 == 0 && aligned16(zero_dst) &&
+                       vectors / kSortBlock < 0x7ff00000ull;
+    if (!fused) {
+        if (zero_bytes) if (int rc = launch_fill(s, zero_dst, 0, 1, zero_bytes)) return rc;
+        return launch_embedding_sort(s, ids, order, sort_workspace, sort_workspace_bytes, N, V, err_flag);
+    }
+    if (int rc = check_embedding_sizes("embedding order", N, V)) return rc;
+    if (ids == nullptr || order == nullptr) return set_error(AGRAD_EINVAL, "embedding order: null operand");
+    SortPlan p;
+    if (int rc = plan_sort(N, V, &p)) return rc;
+    if (sort_workspace == nullptr || sort_workspace_bytes < p.total)
+        return set_error(AGRAD_EWORKSPACE, "embedding order: workspace %llu < %llu bytes",
+                         (unsigned long long)sort_workspace_bytes, (unsigned long long)p.total);
+    if ((reinterpret_cast<uintptr_t>(sort_workspace) & 255u) != 0)
+        return set_error(AGRAD_EINVAL, "embedding order: workspace must be 256-byte aligned");
+    if ((reinterpret_cast<uintptr_t>(order) & 15u) != 0)
+        return set_error(AGRAD_EINVAL, "embedding order: the order buffer must be 16-byte aligned");
+    unsigned long long* spill = reinterpret_cast<unsigned long long*>((uint8_t*)sort_workspace + p.off_keys_in);
+    const uint32_t n = (uint32_t)N, log2G = group_sort_log2g(n);
+    const uint32_t grid = (1u << log2G) + (uint32_t)((vectors + kSortBlock - 1) / kSortBlock);
+    hipLaunchKernelGGL(fill_order_kernel, dim3(grid), dim3(kSortBlock), kFillOrderIdleLds, s, ids, order, spill, n, V, log2G,
+                       err_flag, reinterpret_cast<u32x4*>(zero_dst), vectors);
+    return check_hip(hipGetLastError(), "embedding order launch");
+}
+
 // out = W[ids] (+ wpe) and order = the ids' ordering for the later gradient
 int launch_gather_fwd_sorted(hipStream_t s, int dtype, const int32_t* ids, const void* W, const void* wpe,
                              void* out, uint64_t N, uint32_t T, uint32_t C, uint32_t V, uint32_t* order,
@@ -1428,7 +1482,7 @@ uint64_t embedding_bwd_sorted_workspace_bytes(uint64_t N, uint32_t C) {
     return align256(partial_rows(N) * C * 4);       // the long runs' partial rows
 }
 
-int launch_embedding_bwd_sorted(hipStream_t s, int dtype, const uint32_t* order, const void* dY, void* dW,
+int launch_embedding_bwd_sorted(hipStream_t s, int dtype, uint32_t* order, const void* dY, void* dW,
                                 void* dwpe, void* workspace, uint64_t workspace_bytes, uint64_t N, uint32_t T,
                                 uint32_t C, uint32_t V, uint32_t flags) {
     if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "embedding backward: unknown dtype %d", dtype);

@@ -23,7 +23,7 @@ from .utils import broadcast_shape, mul_bcast_kind
 
 class OpNode:
     __slots__ = ("op", "inputs", "outputs", "forward", "backward", "scratch_fwd_layout",
-                 "scratch_bwd_layout", "name", "overwrite_grads", "defer_param_grads")
+                 "scratch_bwd_layout", "name", "overwrite_grads", "defer_param_grads", "order_ready")
 
     def __init__(self, op, inputs, outputs, name=""):
         self.op = op
@@ -41,11 +41,19 @@ class OpNode:
         # gradient) unfolded and the runtime folds all of a pass's sums in one launch at the
         # end of the pass (set by the runtime; the node's backward scratch then lives that long)
         self.defer_param_grads = False
+        # an embedding node whose ids have already been ordered for this step's gradient (the
+        # ordering rode with the zero fill of the table's gradient): its forward kernel is then
+        # the plain gather.  Set by Runtime.execute, cleared by the node's backward kernel.
+        self.order_ready = False
 
 
 class Op(ABC):
     op_name = "Op"
     recompute_output = False
+    # indices of outputs that may be written before the forward pass starts (the id order of
+    # an embedding, written together with the gradient's zero fill): they hold their arena
+    # bytes from the first step on
+    early_outputs = ()
     # indices (output i aliases input j): the kernel works in place, the
     # runtime gives output and input (and their grads) the same memory
     inplace_aliases: dict = {}
@@ -309,6 +317,7 @@ def _order_output(indices, table):
 class GatherOp(Op):
     """out[b, t, :] = weight[indices[b, t], :]"""
     op_name = "Gather"
+    early_outputs = (1,)
 
     def infer_shape(self, indices, weight):
         if indices.ndim != 2:
@@ -336,6 +345,7 @@ class EmbeddingSumOp(Op):
     embedding tok_emb(ids) + pos_emb(arange(T)) as one op
     (check_tiny_gpt2_kernel.py:282,301)."""
     op_name = "EmbeddingSum"
+    early_outputs = (1,)
 
     def infer_shape(self, indices, wte, wpe):
         if indices.ndim != 2 or wte.ndim != 2 or wpe.ndim != 2:

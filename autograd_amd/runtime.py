@@ -366,6 +366,9 @@ class Runtime:
                         touch(self._root(t), step)
                 if node.scratch_fwd_layout is not None:
                     touch(_Scratch(node.scratch_fwd_layout.nbytes, node, 0), step)
+                for i in node.op.early_outputs:
+                    if i < len(node.outputs):
+                        touch(self._root(node.outputs[i]), 0)      # may be written before the first node runs
             else:
                 for t in node.op.save_for_backward(node.inputs, node.outputs):
                     if self._root(t).op is not None:
@@ -489,9 +492,15 @@ class Runtime:
         self.backend.grad_scale = self.grad_scale
         self.backend.use_fp16_gemm = self.use_fp16_gemm
 
-    def zero_grad(self):
+    def zero_grad(self, order_ids=False):
         """zero the parameter gradients, except those whose first backward kernel
-        stores the whole tensor anyway"""
+        stores the whole tensor anyway.  order_ids: the zero fill of an embedding table's
+        gradient also orders that embedding's ids for the backward pass, in the same launch,
+        and the node's next forward kernel is the plain gather -- the caller vouches that the
+        ids are already what that forward pass will read.  Off by default, because it does not
+        pay on this GPU: the fill runs best with few waves on a CU, and with the 512-thread ordering
+        workgroups in its grid it takes 3 us (a 50 MB table) to 25 us (1 GB) longer, where they cost
+        the forward gather, whose grid they ride in otherwise, 1 to 3 us."""
         self._sync_backend()
         seen = set()
         for node in self.topo:
@@ -501,6 +510,9 @@ class Runtime:
                 seen.add(id(t))
                 if t.grad is not None and t.op is None:
                     if id(t.grad) in self._stored_leaf_grads and not self.accumulate_parameter_grads:
+                        continue
+                    if order_ids and node.op.early_outputs and len(node.inputs) > 1 and node.inputs[1] is t \
+                            and hasattr(self.backend, "zero_grad_and_order") and self.backend.zero_grad_and_order(node, t):
                         continue
                     self.backend.fill(t.grad, 0)
 

@@ -112,10 +112,12 @@ class Pool:
 
 
 class Case:
-    def __init__(self, op, direction, nbytes, nsets, launch, kernel):
+    def __init__(self, op, direction, nbytes, nsets, launch, kernel, in_step=None):
         self.op, self.direction, self.nbytes, self.nsets = op, direction, nbytes, nsets
         self.launch, self.kernel = launch, kernel
         self.us = None
+        # part of the wall-clock step?  by default every forward and backward row is
+        self.in_step = direction in ("fwd", "bwd") if in_step is None else in_step
 
 
 def n_sets(working_bytes):
@@ -184,9 +186,27 @@ def _embed_cases(ctx, cfg, pool, rng, nbytes, ids0):
         def zero(i):
             ctx.call("agrad_fill", dW.ptr, 0, 0, 1, dW.nbytes)
 
+        # Where the id ordering rides.  It is needed by the backward call only, and takes 8 us alone at
+        # 16384 ids (latency, not bytes).  "fwd" is the one launch that gathers and orders (what the
+        # step and Runtime use); "fwd-plain" the gather without it; "id_ordering" the ordering alone;
+        # "..._grad_zero_fill+order" the ordering at the front of the gradient table's zero fill instead
+        # (agrad_embedding_order), beside the plain fill: the fill runs best with few waves on a CU and
+        # is the worse host of the two.
+        def fwd_plain(i):
+            ctx.call("agrad_gather_forward", dt, vp(ids[i]), vp(W), vp(wpe), vp(out[i]), N, cfg.T, Cw, cfg.V)
+
+        def order_alone(i):
+            ctx.call("agrad_embedding_order", vp(ids[i]), N, cfg.V, vp(order[i]), vp(sort_ws), sort_ws_bytes, None, 0)
+
+        def zero_and_order(i):
+            ctx.call("agrad_embedding_order", vp(ids[i]), N, cfg.V, vp(order[i]), vp(sort_ws), sort_ws_bytes, vp(dW), dW.nbytes)
+
         cases.append(Case(name, "fwd", nbytes[name][0], k, fwd, "gather_sort_kernel"))
+        cases.append(Case(name, "fwd-plain", nbytes[name][0], k, fwd_plain, "gather_", in_step=False))
         cases.append(Case(name, "bwd", nbytes[name][1], k, bwd, "emb_row_sum_kernel"))
+        cases.append(Case("id_ordering", "aux", 4 * N + 4 * (6 * N + 128), k, order_alone, "emb_group_sort_kernel"))
         cases.append(Case(name + "_grad_zero_fill", "aux", cfg.V * Cw * e, 1, zero, "fill16_kernel"))
+        cases.append(Case(name + "_grad_zero_fill+order", "aux", cfg.V * Cw * e, k, zero_and_order, "fill_order_kernel"))
     return cases
 
 
@@ -588,7 +608,8 @@ def run_workload(ctx, cfg, steps, warmup, iters, exact=False):
     pool = Pool(ctx, cfg.seed)
     try:
         cases = build_cases(ctx, cfg, pool)
-        step_cases = [c for c in cases if c.direction == "fwd"] + [c for c in reversed(cases) if c.direction == "bwd"]
+        step_cases = [c for c in cases if c.in_step and c.direction.startswith("fwd")] + \
+                     [c for c in reversed(cases) if c.in_step and c.direction == "bwd"]
         step_bytes = sum(c.nbytes for c in step_cases)
 
         def step(s):
@@ -617,8 +638,8 @@ def graph_replay(ctx, cfg, iters=200):
     backward, launched one by one and replayed from a recorded graph."""
     pool = Pool(ctx, cfg.seed)
     try:
-        cases = [c for c in build_cases(ctx, cfg, pool) if c.direction in ("fwd", "bwd")]
-        chain = [c for c in cases if c.direction == "fwd"] + [c for c in reversed(cases) if c.direction == "bwd"]
+        cases = [c for c in build_cases(ctx, cfg, pool) if c.in_step]
+        chain = [c for c in cases if c.direction.startswith("fwd")] + [c for c in reversed(cases) if c.direction == "bwd"]
 
         def step():
             for c in chain:
@@ -660,7 +681,8 @@ def runtime_path(cfg, per_op_rows, steps=20, ctx=None):
     (Rotary is left out: its two outputs have no common consumer without the attention GEMMs.)
     A step is the reference's timing protocol (timing_ops.py:76-100): zero_grad, forward, fill
     the upstream gradient, backward_graph, with the pass synchronisations those calls make.
-    Returns eager and replayed microseconds per step and the C-ABI kernels' sum beside them."""
+    Returns microseconds per step -- eager by that protocol, through Runtime.execute (one pass), and
+    execute replayed from a recorded graph -- and the sum of the same kernels' C-ABI times beside them."""
     from autograd_amd import op as O
     from autograd_amd.runtime import Runtime
     from autograd_amd.tensor import Tensor
@@ -734,7 +756,11 @@ def runtime_path(cfg, per_op_rows, steps=20, ctx=None):
                 rt.execute()
         backend.synchronize()
         execute_us = (time.perf_counter() - t0) * 1e6 / steps
-        graph = rts[0].capture(step)
+        def execute_all():
+            for rt in rts:
+                rt.execute()
+
+        graph = rts[0].capture(execute_all)
         for _ in range(3):
             graph.launch()
         backend.synchronize()
@@ -747,12 +773,14 @@ def runtime_path(cfg, per_op_rows, steps=20, ctx=None):
     finally:
         for rt in rts:
             rt.release()
+    # the kernels Runtime.execute launches for these graphs, from the per-op table
     names = set()
     if cfg.embed and cfg.norm:
-        names |= {cfg.embed, ("add+" if cfg.norm_residual else "") + cfg.norm + "norm", cfg.embed + "_grad_zero_fill"}
+        names |= {cfg.embed, ("add+" if cfg.norm_residual else "") + cfg.norm + "norm"}
     if cfg.act:
         names.add(cfg.act)
-    kernels = [r for r in per_op_rows if r["op"] in names and r["dir"] in ("fwd", "bwd", "aux")]
+    kernels = [r for r in per_op_rows if (r["op"] in names and r["dir"] in ("fwd", "bwd"))
+               or r["op"] == cfg.embed + "_grad_zero_fill"]
     c_abi_us = sum(r["us"] for r in kernels)
     # the protocol's own fills, through the C ABI as well: the upstream gradient of each graph's output
     fill_us = 0.0
@@ -923,7 +951,7 @@ def main():
     cases, step_bytes, wall = run_workload(ctx, cfg, args.steps, args.warmup, args.iters, args.exact_iters)
     ms_per_step = wall * 1e3 / args.steps
     gbps = step_bytes * args.steps / wall / 1e9
-    timed = [c for c in cases if c.direction in ("fwd", "bwd")]
+    timed = [c for c in cases if c.in_step]
     dom = max(timed, key=lambda c: c.us)
     dom_gbps = dom.nbytes / (dom.us * 1e-6) / 1e9
     dom_kernel, dom_traffic = measured_traffic(cfg, dom)

@@ -398,12 +398,29 @@ uint64_t agrad_embedding_sort_workspace_bytes(uint64_t N, uint32_t V);
 int agrad_gather_forward_sorted(agrad_ctx* ctx, int dtype, const int32_t* ids, const void* W, const void* wpe,
                                 void* out, uint64_t N, uint32_t T, uint32_t C, uint32_t V,
                                 uint32_t* order, void* sort_workspace, uint64_t sort_workspace_bytes);
+/* The ordering alone: writes `order` (same layout, same bits as the forward call above
+ * leaves) from the ids, and -- when zero_dst is not NULL -- clears zero_dst[0 .. zero_bytes)
+ * in the same launch, for a caller that zero-fills the table's gradient and orders the ids
+ * before its forward pass and then calls the plain agrad_gather_forward.  One launch when
+ * N <= 65536 and zero_dst / zero_bytes are multiples of 16; otherwise a fill and the ordering
+ * one after the other.  The ids must already be what the forward pass will read.  Measured on
+ * MI355X the forward gather is the better host for the ordering workgroups (they cost it 1 to
+ * 3 us; the fill, which runs best with few waves on a CU, 3 to 25 us), so
+ * agrad_gather_forward_sorted stays the default; this call is for callers whose forward pass
+ * must be the plain gather.  The reference clears the table inside its forward gather
+ * (metal_gather_forward, backend.py:2781-2785) and orders nothing. */
+int agrad_embedding_order(agrad_ctx* ctx, const int32_t* ids, uint64_t N, uint32_t V, uint32_t* order,
+                          void* sort_workspace, uint64_t sort_workspace_bytes,
+                          void* zero_dst, uint64_t zero_bytes);
 uint64_t agrad_embedding_backward_sorted_workspace_bytes(uint64_t N, uint32_t C);
-/* dwpe may be NULL; otherwise it is the [T, C] position table's gradient
+/* `order` is read AND written: the call counts arrivals in the counters at its end and leaves
+ * them zero again; they must be zero on entry, which the calls that write an order guarantee
+ * and an interrupted backward call does not (write the order again after one).
+ * dwpe may be NULL; otherwise it is the [T, C] position table's gradient
  * dwpe[t,:] (+)= sum_b dY[b,t,:] (N = B*T rows, b ascending), added up from the
  * same loads of dY that feed the table rows; AGRAD_ACC_PARAM_GRAD2 accumulates
  * into it. */
-int agrad_embedding_backward_sorted(agrad_ctx* ctx, int dtype, const uint32_t* order, const void* dY, void* dW,
+int agrad_embedding_backward_sorted(agrad_ctx* ctx, int dtype, uint32_t* order, const void* dY, void* dW,
                                     void* dwpe, void* workspace, uint64_t workspace_bytes,
                                     uint64_t N, uint32_t T, uint32_t C, uint32_t V, uint32_t flags);
 /* dwpe[t,:] (+)= sum_b dY[b,t,:], b ascending (pos_emb_grad, metal_ops.metal:220-234;

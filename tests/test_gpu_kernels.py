@@ -1017,6 +1017,65 @@ def test_presorted_embedding_pair_matches_the_plain_pair(ctx, B, T, V, C, dist, 
             d.free()
 
 
+@pytest.mark.parametrize("B,T,V,C,dist", [(32, 512, 32768, 384, "uniform"), (2, 700, 300, 48, "zipf"),
+                                          (5, 14000, 3000, 32, "zipf"), (3, 50, 77, 10, "uniform")])
+def test_ordering_with_the_zero_fill_matches_the_forward_call(ctx, B, T, V, C, dist):
+    """agrad_embedding_order writes the order buffer agrad_gather_forward_sorted writes, word for
+    word, and clears the gradient table in the same launch; the plain gather plus the sorted
+    backward call then give the bits of the plain pair.  (5, 14000) takes the radix path with a
+    fill of its own, C = 10 a fill whose size is no multiple of 16."""
+    import ctypes as Ct
+    rng = _rng(160 + C)
+    N = B * T
+    if dist == "zipf":
+        p = np.arange(1, V + 1, dtype=np.float64) ** -1.1
+        ids = rng.choice(V, size=(B, T), p=p / p.sum()).astype(np.int32)
+    else:
+        ids = rng.integers(0, V, (B, T), dtype=np.int32)
+    W = (0.02 * rng.standard_normal((V, C))).astype(np.float32)
+    dY = rng.standard_normal((B, T, C)).astype(np.float32)
+    want_out = G.gather_forward(ctx, ids, W, None)
+    want_dW = G.embedding_backward(ctx, ids, dY, V)
+
+    def vp(d, off=0):
+        return Ct.c_void_p(d.ptr + off) if d is not None else None
+    d_ids, d_W, d_dY = ctx.upload(ids), ctx.upload(W), ctx.upload(dY)
+    out = ctx.empty((N, C), np.float32)
+    order_a, order_b = ctx.empty((6 * N + 128,), np.uint32), ctx.empty((6 * N + 128,), np.uint32)
+    sws_b = ctx.lib.agrad_embedding_sort_workspace_bytes(N, V)
+    bws_b = ctx.lib.agrad_embedding_backward_sorted_workspace_bytes(N, C)
+    sws, bws = ctx.empty((sws_b,), np.uint8), ctx.empty((bws_b,), np.uint8)
+    ctx.call("agrad_gather_forward_sorted", capi.F32, vp(d_ids), vp(d_W), None, vp(out), N, T, C, V, vp(order_a), vp(sws), sws_b)
+    ctx.synchronize()
+    # words of the buffer that an ordering writes: rows, four words of run info per row, arrival counters
+    info_at = (N + 3) & ~3                  # (words N .. info_at are padding nobody writes)
+    used = info_at + 4 * N + (N // 128 + 1) * 32 + (N // 2048 + 1) * 32
+
+    def written(order):
+        words = order.download()
+        return np.concatenate([words[:N], words[info_at:used]])
+    # the gradient table sits between two guard rows that must survive the fill
+    dW = ctx.upload(np.full((V + 2, C), 7.0, np.float32))
+    ctx.call("agrad_embedding_order", vp(d_ids), N, V, vp(order_b), vp(sws), sws_b, vp(dW, C * 4), V * C * 4)
+    ctx.call("agrad_gather_forward", capi.F32, vp(d_ids), vp(d_W), None, vp(out), N, T, C, V)
+    ctx.synchronize()
+    np.testing.assert_array_equal(written(order_b), written(order_a))
+    table = dW.download()
+    assert not table[1:-1].any() and (table[0] == 7.0).all() and (table[-1] == 7.0).all()
+    ctx.call("agrad_embedding_backward_sorted", capi.F32, vp(order_b), vp(d_dY), vp(dW, C * 4), None, vp(bws), bws_b, N, T,
+             C, V, capi.ACC_PARAM_GRAD)
+    ctx.synchronize()
+    np.testing.assert_array_equal(out.download().reshape(B, T, C), want_out)
+    np.testing.assert_array_equal(dW.download()[1:-1], want_dW)
+    # without a table to clear it is the ordering alone
+    ctx.call("agrad_fill", order_b.ptr, 0, 0xFFFFFFFF, 4, 6 * N + 128)
+    ctx.call("agrad_embedding_order", vp(d_ids), N, V, vp(order_b), vp(sws), sws_b, None, 0)
+    ctx.synchronize()
+    np.testing.assert_array_equal(written(order_b), written(order_a))
+    for d in (d_ids, d_W, d_dY, out, order_a, order_b, sws, bws, dW):
+        d.free()
+
+
 def _check_order(order, N, tokens, V):
     """The order buffer of the pre-sorted embedding pair: rows[N] (each token's rows adjacent
     and ascending; the top bit of a word marks a task of the gradient kernel: the first row

@@ -762,3 +762,47 @@ def test_captured_graph_replays_match_eager():
     with pytest.raises(RuntimeError):
         graph.launch()
     rt.release()
+
+
+@pytest.mark.parametrize("with_wpe", [False, True])
+def test_ids_ordered_with_the_zero_fill(with_wpe):
+    """zero_grad(order_ids=True) lets the id ordering ride with the zero fill of the table's gradient,
+    and the forward pass then gathers with the plain kernel; without it the forward call orders the
+    ids.  Same outputs and the same gradient bits either way, step after step with new ids."""
+    rng = np.random.default_rng(SEED + 90)
+    B, T, C, V = 8, 256, 96, 1000
+    dev = "hip"
+    results = {}
+    for mode in ("execute", "protocol"):
+        r2 = np.random.default_rng(SEED + 91)
+        ids = make_tensor((B, T), np.int32, dev, False, r2.integers(0, V, (B, T), dtype=np.int32))
+        wte = make_tensor((V, C), np.float32, dev, True, (0.5 * r2.standard_normal((V, C))).astype(np.float32))
+        g = make_tensor((C,), np.float32, dev, True, np.ones(C, np.float32))
+        if with_wpe:
+            wpe = make_tensor((T, C), np.float32, dev, True, (0.5 * r2.standard_normal((T, C))).astype(np.float32))
+            x0 = EmbeddingSumOp()(ids, wte, wpe)
+        else:
+            x0 = GatherOp()(ids, wte)
+        out = RMSNormOp(eps=1e-6)(x0, g)
+        rt = Runtime(device=dev)
+        rt.loss = out
+        rt.build_topo(out)
+        rt.bind_memory()
+        emb = x0.op
+        steps = []
+        for step in range(3):
+            rt.backend.copy_from_host(ids, np.random.default_rng(SEED + 92 + step).integers(0, V, (B, T), dtype=np.int32))
+            rt.zero_grad(order_ids=(mode == "execute"))
+            assert emb.order_ready == (mode == "execute")
+            rt.forward()
+            rt.backend.fill(out.grad, 0.5)
+            rt.backward_graph()
+            rt.backend.synchronize()
+            assert not emb.order_ready          # consumed by the backward kernel
+            steps.append([rt.backend.copy_to_host(t).copy() for t in (out, wte.grad, g.grad)]
+                         + ([rt.backend.copy_to_host(wpe.grad).copy()] if with_wpe else []))
+        results[mode] = steps
+        rt.release()
+    for a, b in zip(results["execute"], results["protocol"]):
+        for x, y in zip(a, b):
+            np.testing.assert_array_equal(x, y)
