@@ -151,7 +151,8 @@ swiglu_bwd_kernel(const T* gu, const T* __restrict__ dh, T* dgu, uint32_t H, uin
 // us, 16384 x 8960 fp32 469 -> 451 us, bf16 225 -> 220 us.  (Eight: 20 % slower -- the
 // sigmoid needs waves to hide behind.  The forward kernel, three streams, gains nothing, and
 // the two- and three-stream elementwise kernels lose from any cap.)
-constexpr unsigned kSwigluBwdIdleLds = 10 * 1024;
+constexpr int kSwigluBwdPerCu = 16;
+static_assert(kEwBlock == kWave, "the occupancy cap counts one-wave workgroups");
 
 // Rows are processed in slabs small enough for 32-bit vector indices.
 template <typename T, int VEC>
@@ -170,7 +171,7 @@ int swiglu_typed(hipStream_t s, const T* gu, const T* dh, T* out, uint64_t rows,
             hipLaunchKernelGGL((swiglu_fwd_kernel<T, VEC, UNROLL>), dim3(grid), dim3(kEwBlock), 0, s,
                                gu + r0 * 2 * H, out + r0 * hw, H, h0, HV, nvec);
         } else {
-            hipLaunchKernelGGL((swiglu_bwd_kernel<T, VEC, UNROLL>), dim3(grid), dim3(kEwBlock), VEC > 1 ? kSwigluBwdIdleLds : 0u, s,
+            hipLaunchKernelGGL((swiglu_bwd_kernel<T, VEC, UNROLL>), dim3(grid), dim3(kEwBlock), VEC > 1 ? idle_lds_for(kSwigluBwdPerCu) : 0u, s,
                                gu + r0 * 2 * H, dh + r0 * H, out + r0 * 2 * H, H, HV, nvec, acc);
         }
     }

@@ -24,6 +24,12 @@ inline uint32_t dtype_size(int dtype) { return dtype == AGRAD_BF16 ? 2u : 4u; }
 
 // Upper bound on the number of row-partials the norm backward keeps per column.
 
+// Bytes of dynamic LDS that a kernel of ONE-WAVE workgroups asks for and never touches, so that at
+// most `per_cu` of its workgroups share a CU (streams of stores, or of many operands, run faster
+// with fewer waves in flight): this GPU's LDS per CU divided by the count, in whole 512-byte
+// granules, so the cap keeps its meaning on a part with another LDS size.  0 if the size is unknown.
+uint32_t idle_lds_for(int per_cu);
+
 // memops.hip
 int launch_fill(hipStream_t s, void* dst, uint32_t bits, int itemsize, uint64_t n);
 int launch_copy(hipStream_t s, const void* src, void* dst, uint64_t nbytes);

@@ -1130,6 +1130,8 @@ namespace {
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mu;
 void* g_scratch_ptr[kMaxDevices] = {};   // device address of `scratch` on each GPU
+hipStream_t g_scratch_stream[kMaxDevices] = {};   // the stream whose call used it last
+bool g_scratch_used[kMaxDevices] = {};
 }  // namespace
 
 // Called by agrad_ctx_create with `device` current: looks up, once per GPU, where
@@ -1158,6 +1160,19 @@ int launch_norm_bwd_noalloc(hipStream_t s, int device, int kind, int dtype, cons
     if (device >= 0 && device < kMaxDevices) {
         std::lock_guard<std::mutex> lock(g_scratch_mu);
         ptr = g_scratch_ptr[device];
+        // Calls on one stream follow one another; a call from ANOTHER stream (another context)
+        // while the last user's work may still be running would overwrite its partial rows.
+        if (ptr != nullptr && (dgamma != nullptr || dbeta != nullptr)) {
+            if (g_scratch_used[device] && g_scratch_stream[device] != s && !is_capturing()) {
+                const hipError_t busy = hipStreamQuery(g_scratch_stream[device]);
+                if (busy == hipErrorNotReady)
+                    return set_error(AGRAD_EINVAL, "norm backward (no allocation): the fixed scratch of device %d is still in "
+                                     "use by work on another stream; synchronise that stream first", device);
+                (void)hipGetLastError();        // (a stream that no longer exists has nothing in flight)
+            }
+            g_scratch_used[device] = true;
+            g_scratch_stream[device] = s;
+        }
     }
     if (ptr == nullptr) return set_error(AGRAD_EINVAL, "norm backward (no allocation): device %d was never set up", device);
     if ((dgamma != nullptr || dbeta != nullptr) && rows > 0 && C > 0) {

@@ -23,7 +23,8 @@ namespace agrad {
 namespace {
 
 constexpr int kOptBlock = 64;
-constexpr unsigned kAdamwIdleLds = 13 * 1024;
+constexpr int kAdamwPerCu = 12;        // one-wave workgroups of the AdamW step that share a CU (seven streams: 5 to 7 % faster than 32)
+static_assert(kOptBlock == kWave, "the occupancy cap counts one-wave workgroups");
 
 struct AdamwArgs {
     float* p; const void* g; float* m; float* v;
@@ -174,7 +175,7 @@ int adamw_typed(hipStream_t s, AdamwArgs a, uint64_t numel) {
         b.n = nvec;
         // (seven streams -- p, g, m, v in; p, m, v out: idle dynamic LDS caps a CU at twelve of
         // these one-wave workgroups, 3 to 4 % faster than with all thirty-two: see the SwiGLU backward)
-        hipLaunchKernelGGL((adamw_vec_kernel<G>), dim3((uint32_t)grid), dim3(kOptBlock), kAdamwIdleLds, s, b);
+        hipLaunchKernelGGL((adamw_vec_kernel<G>), dim3((uint32_t)grid), dim3(kOptBlock), idle_lds_for(kAdamwPerCu), s, b);
     }
     const uint64_t done = nvec * 4;
     if (done < numel) {

@@ -50,6 +50,9 @@ class OpNode:
 class Op(ABC):
     op_name = "Op"
     recompute_output = False
+    # One store-or-accumulate choice covers all of this op's parameter gradients (gamma and beta of a
+    # norm share a flag bit of the kernel).  False where every parameter has a flag of its own.
+    shared_param_grad_flag = True
     # indices of outputs that may be written before the forward pass starts (the id order of
     # an embedding, written together with the gradient's zero fill): they hold their arena
     # bytes from the first step on
@@ -346,6 +349,7 @@ class EmbeddingSumOp(Op):
     (check_tiny_gpt2_kernel.py:282,301)."""
     op_name = "EmbeddingSum"
     early_outputs = (1,)
+    shared_param_grad_flag = False      # the token table and the position table have a flag each
 
     def infer_shape(self, indices, wte, wpe):
         if indices.ndim != 2 or wte.ndim != 2 or wpe.ndim != 2:

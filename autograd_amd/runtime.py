@@ -335,14 +335,14 @@ class Runtime:
                             self._stored_leaf_grads.add(id(x.grad))
                     elif x.op is not None:
                         self.node_to_clear_grads[id(node)].append(x)
-                # A kernel has ONE store-or-accumulate choice for its parameter gradients
-                # (gamma and beta of a norm share a flag bit).  If only some of this node's
+                # Most kernels have ONE store-or-accumulate choice for their parameter gradients
+                # (gamma and beta of a norm share a flag bit; Op.shared_param_grad_flag).  If only some of this node's
                 # leaf gradients are first written here -- a gamma tied to a later node, a
                 # beta of its own -- none of them may skip the zero fill, or the kernel
                 # would accumulate onto memory nobody cleared.
                 leaf_grads = {id(x.grad) for x in node.inputs
                               if x.op is None and x.requires_grad and x.grad is not None}
-                if leaf_grads - overwrite:
+                if node.op.shared_param_grad_flag and leaf_grads - overwrite:
                     overwrite -= leaf_grads
                     self._stored_leaf_grads -= leaf_grads
                 node.overwrite_grads = frozenset(overwrite)

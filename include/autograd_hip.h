@@ -284,9 +284,10 @@ int agrad_norm_backward_partial(agrad_ctx* ctx, int kind, int dtype,
  * same launch geometry and same results, bit for bit, as agrad_norm_backward.
  * A problem whose partial rows (agrad_norm_backward_workspace_bytes(rows, C, dtype))
  * exceed the array is refused with AGRAD_EINVAL; without dgamma and dbeta any size
- * runs.  All calls on one GPU share the array: calls that overlap there (two
- * contexts, or a replaying graph beside eager calls) race.  This entry point has no
- * counterpart in the reference. */
+ * runs.  All calls on one GPU share the array: calls that overlap there race.  A call from
+ * another stream (another context) than the last one's, while that stream still has work in
+ * flight, is refused with AGRAD_EINVAL; a replaying graph beside eager calls is the caller's
+ * to keep apart.  This entry point has no counterpart in the reference. */
 #define AGRAD_NOALLOC_SCRATCH_BYTES (32u * 1024u * 1024u)
 int agrad_norm_backward_noalloc(agrad_ctx* ctx, int kind, int dtype,
                                 const void* x, const void* dy, const float* gamma,

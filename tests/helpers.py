@@ -38,6 +38,19 @@ def assert_fp32_parity(got, cpu, exact, what=""):
         f"rms {rms_d:.3e} vs {rms_c:.3e}")
 
 
+def assert_chain_close(got, ref, what, kernels, sum_rows=1):
+    """Whole-graph fp32 comparisons.  The kernel tests hold every kernel to rtol 1e-5 / atol 1e-6 of its
+    own output; `kernels` of them in a chain (forward and backward kernels between the inputs and the
+    compared value both count) compound to at most `kernels` times that at the end of the chain, on the
+    scale of the values compared; a gradient summed over `sum_rows` rows (gamma, beta, a bias, a table
+    row that many ids hit) adds what the two devices' different summation orders may differ by,
+    1e-6 sqrt(sum_rows) of that scale."""
+    ref64 = np.asarray(ref, dtype=np.float64)
+    scale = max(1.0, float(np.abs(ref64).max()) if ref64.size else 1.0)
+    atol = FP32_ATOL * kernels * scale + (FP32_ATOL * float(np.sqrt(sum_rows)) * scale if sum_rows > 1 else 0.0)
+    assert_fp32_close(got, ref, what, rtol=FP32_RTOL * kernels, atol=atol)
+
+
 def bf16_rel_error(got, ref):
     """max relative error over elements with |ref| > 1e-3 max|ref|, and max abs error."""
     got = np.asarray(got, dtype=np.float64)
