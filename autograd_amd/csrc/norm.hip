@@ -789,9 +789,12 @@ NormPlan plan_norm(uint32_t C, int dtype, bool aligned, bool backward) {
 // MI355X over the benchmark shapes: a grid larger than what the GPU holds at
 // once (`resident`, from the occupancy query -- register use differs a lot
 // between instantiations) loses to one round, because the stragglers of the
-// second round run on a mostly idle chip; and beyond 1024 workgroups more
-// waves only add loads in flight that the memory system does not need.
-constexpr uint32_t kMaxBwdBlocks = 1024;
+// second round run on a mostly idle chip; and beyond 768 workgroups (three to a
+// CU) more waves only add loads in flight that the memory system does not need
+// -- every load of a row is in flight at once here: 65536 x 4096 bf16 without
+// column sums 386 us with 1024 workgroups, 376 us with 768; 256 or 512 lose
+// 10 to 90 % at every shape.
+constexpr uint32_t kMaxBwdBlocks = 768;
 
 uint32_t bwd_blocks(const NormPlan& p, uint64_t rows, uint32_t resident) {
     const uint64_t want = (rows + p.rpb - 1) / p.rpb;

@@ -92,7 +92,7 @@ def test_noalloc_against_cpu_restatement(ctx):
 
 
 def test_noalloc_refuses_what_the_array_cannot_hold(ctx):
-    rows, Cw = 4096, 8192          # 1024 partial rows x 2 x 8192 x 4 B = 64 MiB
+    rows, Cw = 4096, 8192          # 768 partial rows x 2 x 8192 x 4 B = 48 MiB
     assert ctx.lib.agrad_norm_backward_workspace_bytes(rows, Cw, capi.F32) > capi.NOALLOC_SCRATCH_BYTES
     x = ctx.zeros((rows, Cw), np.float32)
     dy = ctx.zeros((rows, Cw), np.float32)
