@@ -134,6 +134,7 @@ class HipBackend(Backend):
     supports_grad_store = True   # kernels take a store / accumulate flag per gradient
     supports_deferred_param_grads = True    # column sums of a pass can be folded in one launch at its end
     single_pass_execute = True   # Runtime.execute runs zero_grad + forward + backward as ONE pass (one wait)
+    supports_row_reset = True    # an embedding table's gradient is cleared by rows (clear_table_grad)
 
     def __init__(self, ctx=None):
         if ctx is None:
@@ -217,6 +218,9 @@ class HipBackend(Backend):
         return 0 if id(t.grad) in node.overwrite_grads else ACC_INPUT_GRAD
 
     def _param_flag(self, node, *params):
+        for p in params:                            # about to be written: no longer known to be all zero
+            if p is not None and p.grad is not None:
+                p.grad.dirty_rows = None
         if self.accumulate_parameter_grads:
             return ACC_PARAM_GRAD
         live = [p for p in params if p is not None and p.requires_grad and p.grad is not None]
@@ -557,6 +561,7 @@ class HipBackend(Backend):
         ws, g = scratch["sort_workspace"], table.grad.storage
         self._launch("embedding_order", [indices, node.outputs[1], ws, g],
                      [prod(indices.shape), table.shape[0]] + _lo_hi(ws.nbytes) + _lo_hi(g.nbytes) + [0b1111])
+        table.grad.dirty_rows = []
         node.order_ready = True
         return True
 
@@ -568,8 +573,14 @@ class HipBackend(Backend):
             if scratch is None:
                 raise RuntimeError("embedding forward needs its arena workspace (plan_scratch)")
             ws = scratch["sort_workspace"]
-            self._launch("gather_forward_sorted", [indices, table, wpe, out, outputs[1], ws],
-                         [_dt(table), B * T, T, C, V] + _lo_hi(ws.nbytes) + [_mask(indices, table, wpe, out, outputs[1], ws)])
+            kept = out.op.kept_ids
+            if kept is not None and table.grad is not None and table.grad.dirty_rows \
+                    and any(k is kept for k in table.grad.dirty_rows):
+                table.grad.dirty_rows = None        # the list of an earlier pass is about to be overwritten
+            self._launch("gather_forward_sorted", [indices, table, wpe, out, outputs[1], ws, kept],
+                         [_dt(table), B * T, T, C, V] + _lo_hi(ws.nbytes)
+                         + [_mask(indices, table, wpe, out, outputs[1], ws, kept)])
+            out.op.kept_fresh = kept is not None
         elif wpe is None:
             self._launch("gather_forward_kernel", [indices, table, out], [_dt(table), B * T, C, V])
         else:
@@ -591,6 +602,7 @@ class HipBackend(Backend):
             raise RuntimeError(f"embedding backward: upstream {out.grad.dtype}, table {weight.dtype}, gradients "
                                f"{[str(g.dtype) for g in grads]}: the kernels take one storage type throughout, or "
                                "bf16 table gradients under fp32 activations")
+        clean_but = weight.grad.dirty_rows          # (every gradient writer forgets it: _param_flag)
         flag = self._param_flag(node, weight) | (PARAM_GRAD_BF16 if narrow else 0)
         if len(outputs) > 1:
             T = 0
@@ -603,6 +615,11 @@ class HipBackend(Backend):
                          [_dt(weight), prod(indices.shape), C, V, flag] + _lo_hi(ws.nbytes)
                          + [T, _mask(outputs[1], out.grad, weight.grad, ws, dwpe)])
             node.order_ready = False        # the next forward pass orders its own ids unless told otherwise
+            # the rows this call stored are the rows of the ids the forward kernel kept -- if it
+            # kept them, and this is the first backward pass over that copy
+            if clean_but is not None and node.kept_fresh and not any(k is node.kept_ids for k in clean_but):
+                weight.grad.dirty_rows = clean_but + [node.kept_ids]
+            node.kept_fresh = False
             return wpe is not None
         else:
             self._launch("gather_backward_kernel", [indices, out.grad, weight.grad, ws],
@@ -892,7 +909,26 @@ class HipBackend(Backend):
         self.ctx.fill_scalar2("fill_scalar_kernel2", [storage.ptr.buffer_id], [storage.ptr.offset],
                               bits, dt.itemsize, prod(storage.shape))
 
+    def fill(self, tensor, value):
+        super().fill(tensor, value)
+        tensor.dirty_rows = [] if float(value) == 0.0 else None
+
+    def clear_table_grad(self, table):
+        """table.grad = 0.  When all that is not zero in it are the rows of id lists the forward
+        kernels kept (the backward passes since the last clear were embedding nodes' only), those
+        rows are cleared -- N*C items a list where the fill writes V*C; otherwise the fill."""
+        g = table.grad
+        lists = g.dirty_rows
+        if lists is None or len(table.shape) != 2:
+            self.fill(g, 0)
+            return
+        V, C = table.shape
+        for kept in lists:
+            self._launch("embedding_grad_reset", [kept, g], [_dt(g), prod(kept.shape), C, V])
+        g.dirty_rows = []
+
     def copy_from_host(self, tensor, host_np):
+        tensor.dirty_rows = None
         st = tensor.storage
         dt = np.dtype(st.dtype)
         host = np.asarray(host_np)

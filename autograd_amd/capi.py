@@ -92,7 +92,9 @@ SIGNATURES = {
     "agrad_embedding_backward": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u64, _u32, _u32, _u32]),
     "agrad_embedding_sort_workspace_bytes": (_u64, [_u64, _u32]),
     "agrad_gather_forward_sorted": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u32, _u32, _u32, _ptr, _ptr, _u64]),
+    "agrad_gather_forward_sorted_kept": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u32, _u32, _u32, _ptr, _ptr, _u64, _ptr]),
     "agrad_embedding_order": (_int, [_ctx, _ptr, _u64, _u32, _ptr, _ptr, _u64, _ptr, _u64]),
+    "agrad_embedding_grad_reset": (_int, [_ctx, _int, _ptr, _u64, _ptr, _u32, _u32]),
     "agrad_unary_forward": (_int, [_ctx, _int, _int, _ptr, _ptr, _u64]),
     "agrad_unary_backward": (_int, [_ctx, _int, _int, _ptr, _ptr, _ptr, _u64, _u32]),
     "agrad_mul_forward": (_int, [_ctx, _int, _int, _ptr, _ptr, _ptr, _u64, _u64]),

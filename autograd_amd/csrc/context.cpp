@@ -412,7 +412,7 @@ int h_gather_bwd(const Call& c) {
     return launch_embedding_bwd(c.ctx->stream, c.a[0], (const int32_t*)ids, dY, dW, ws, ws_bytes, N, C, V,
                                 c.a[4], c.ctx->err_flag);
 }
-// buffers ids, W, wpe, out, order, sort_ws | args dtype, N, T, C, V, ws lo, hi, present_mask
+// buffers ids, W, wpe, out, order, sort_ws, kept_ids | args dtype, N, T, C, V, ws lo, hi, present_mask
 int h_gather_fwd_sorted(const Call& c) {
     NEED_DTYPE(c.a[0])
     const uint64_t N = c.a[1], es = dtype_size(c.a[0]), wsb = u64(c.a, 5);
@@ -420,8 +420,9 @@ int h_gather_fwd_sorted(const Call& c) {
     RESOLVE(0, N * 4, ids) RESOLVE(1, (uint64_t)V * C * es, W)
     RESOLVE_IF(mask & 4u, 2, (uint64_t)T * C * es, wpe)
     RESOLVE(3, N * C * es, out) RESOLVE(4, (N * 6 + 128) * 4, order) RESOLVE(5, wsb, ws)
+    RESOLVE_IF(mask & 64u, 6, N * 4, kept)
     return launch_gather_fwd_sorted(c.ctx->stream, (int)c.a[0], (const int32_t*)ids, W, wpe, out, N, T, C, V,
-                                    (uint32_t*)order, ws, wsb, c.ctx->err_flag);
+                                    (uint32_t*)order, ws, wsb, c.ctx->err_flag, (int32_t*)kept);
 }
 // buffers order, dY, dW, workspace, dwpe | args dtype, N, C, V, flags, ws lo, hi, T, present mask
 int h_gather_bwd_sorted(const Call& c) {
@@ -486,6 +487,13 @@ int h_emb_order(const Call& c) {
     RESOLVE_IF(c.a[6] & 8u, 3, zb, zero_dst)
     return launch_embedding_order(c.ctx->stream, (const int32_t*)ids, (uint32_t*)order, ws, wsb, N, c.a[1], zero_dst,
                                   zero_dst ? zb : 0, c.ctx->err_flag);
+}
+// buffers rows, dW | args dtype, N, C, V
+int h_emb_grad_reset(const Call& c) {
+    NEED_DTYPE(c.a[0])
+    const uint64_t N = c.a[1];
+    RESOLVE(0, N * 4, rows) RESOLVE(1, (uint64_t)c.a[2] * c.a[3] * dtype_size(c.a[0]), dW)
+    return launch_embedding_grad_reset(c.ctx->stream, (int)c.a[0], (const int32_t*)rows, N, dW, c.a[2], c.a[3]);
 }
 // buffers p, g, m, v | args (float bits) lr_wd, b1, 1-b1, b2, 1-b2, eps, step_lr, inv_sqrt_bc2, grad_scale,
 //                       then numel lo, hi, decay_numel lo, hi, grad dtype
@@ -553,7 +561,7 @@ const Entry kTable[] = {
     {"gather_forward_kernel", 3, 4, "ids, W, out | dtype, N, C, V", h_gather_fwd},
     {"embedding_sum_forward", 4, 5, "ids, W, wpe, out | dtype, N, T, C, V", h_embed_sum_fwd},
     {"gather_backward_kernel", 4, 7, "ids, dY, dW, workspace | dtype, N, C, V, flags, ws_lo, ws_hi", h_gather_bwd},
-    {"gather_forward_sorted", 6, 8, "ids, W, wpe, out, order, sort_workspace | dtype, N, T, C, V, ws_lo, ws_hi, present_mask", h_gather_fwd_sorted},
+    {"gather_forward_sorted", 7, 8, "ids, W, wpe, out, order, sort_workspace, kept_ids | dtype, N, T, C, V, ws_lo, ws_hi, present_mask", h_gather_fwd_sorted},
     {"gather_backward_sorted", 5, 9, "order, dY, dW, workspace, dwpe | dtype, N, C, V, flags, ws_lo, ws_hi, T, present_mask", h_gather_bwd_sorted},
     {"pos_emb_grad", 2, 5, "dY, dwpe | dtype, B, T, C, flags", h_pos_grad},
     {"cross_entropy_forward", 4, 5, "logits, labels, loss, lse | dtype, rows_lo, rows_hi, V, present_mask", h_ce_fwd},
@@ -561,6 +569,7 @@ const Entry kTable[] = {
     {"fused_linear_ce_logits_to_dlogits", 4, 7, "logits (in place), targets, row_loss, lse_out | rows, V, row_base, scale_bits, write_grad, dtype, present_mask", h_ce_fused<false>},
     {"fused_linear_ce_logits_to_dlogits_row_scaled", 5, 7, "logits (in place), targets, row_loss, lse_out, row_scale | rows, V, row_base, total_rows, write_grad, dtype, present_mask", h_ce_fused<true>},
     {"embedding_order", 4, 7, "ids, order, sort_workspace, zero_dst | N, V, ws_lo, ws_hi, zero_lo, zero_hi, present_mask", h_emb_order},
+    {"embedding_grad_reset", 2, 4, "rows, dW | dtype, N, C, V", h_emb_grad_reset},
     {"adamw_step", 4, 14, "p, g, m, v | lr_wd, b1, one_minus_b1, b2, one_minus_b2, eps, step_lr, inv_sqrt_bc2, grad_scale (float bits), n_lo, n_hi, decay_lo, decay_hi, grad_dtype", h_adamw},
     {"adamw8bit_step", 8, 11, "p, g, qm, qv, absmax_m, absmax_v, qmap_m, qmap_v | decay, lr_bc1, b1, b2, eps (float bits), numel, decay_numel, first_step, inv_sqrt_bc2 (bits), grad_bf16, clip_coef (bits)", h_adamw8bit},
     {"grad_norm_sq", 2, 3, "g, partial | n_lo, n_hi, dtype", h_grad_norm},
@@ -1046,11 +1055,24 @@ int agrad_gather_forward_sorted(agrad_ctx* ctx, int dtype, const int32_t* ids, c
     return launch_gather_fwd_sorted(ctx->stream, dtype, ids, W, wpe, out, N, T, C, V, order, sort_workspace,
                                     sort_workspace_bytes, ctx->err_flag);
 }
+int agrad_gather_forward_sorted_kept(agrad_ctx* ctx, int dtype, const int32_t* ids, const void* W, const void* wpe,
+                                     void* out, uint64_t N, uint32_t T, uint32_t C, uint32_t V, uint32_t* order,
+                                     void* sort_workspace, uint64_t sort_workspace_bytes, int32_t* ids_kept) {
+    CTX_OR_FAIL(ctx)
+    if (ids_kept == nullptr) return set_error(AGRAD_EINVAL, "gather: null buffer for the kept ids");
+    return launch_gather_fwd_sorted(ctx->stream, dtype, ids, W, wpe, out, N, T, C, V, order, sort_workspace,
+                                    sort_workspace_bytes, ctx->err_flag, ids_kept);
+}
 int agrad_embedding_order(agrad_ctx* ctx, const int32_t* ids, uint64_t N, uint32_t V, uint32_t* order,
                           void* sort_workspace, uint64_t sort_workspace_bytes, void* zero_dst, uint64_t zero_bytes) {
     CTX_OR_FAIL(ctx)
     return launch_embedding_order(ctx->stream, ids, order, sort_workspace, sort_workspace_bytes, N, V, zero_dst, zero_bytes,
                                   ctx->err_flag);
+}
+int agrad_embedding_grad_reset(agrad_ctx* ctx, int dtype, const int32_t* rows, uint64_t N, void* dW, uint32_t C,
+                               uint32_t V) {
+    CTX_OR_FAIL(ctx)
+    return launch_embedding_grad_reset(ctx->stream, dtype, rows, N, dW, C, V);
 }
 uint64_t agrad_embedding_backward_sorted_workspace_bytes(uint64_t N, uint32_t C) {
     return embedding_bwd_sorted_workspace_bytes(N, C);

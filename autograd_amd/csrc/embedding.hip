@@ -125,6 +125,37 @@ gather_rows16_kernel(const int32_t* __restrict__ ids, const u32x4* __restrict__ 
     }
 }
 
+// Zeroes the table rows that a list of token ids names, 16 bytes to a thread.  The gradient
+// of an embedding table is zero outside the rows its backward pass stored, so clearing the
+// rows the last backward pass touched restores an all-zero table for N*C items written
+// where the full fill writes V*C.  Ids outside [0, V) name no row (the backward pass stored
+// none for them) and are skipped; a row listed twice is cleared twice.
+__global__ void __launch_bounds__(kGatherBlock)
+zero_rows16_kernel(const int32_t* __restrict__ rows, u32x4* __restrict__ table, uint32_t total,
+                   uint32_t CV, uint32_t V) {
+    const uint32_t idx = blockIdx.x * kGatherBlock + threadIdx.x;
+    if (idx >= total) return;
+    const uint32_t row = idx / CV;
+    const uint32_t cv = idx - row * CV;
+    const int32_t tok = rows[row];
+    if (tok < 0 || (uint32_t)tok >= V) return;
+    __builtin_nontemporal_store(u32x4{0u, 0u, 0u, 0u}, table + (uint64_t)tok * CV + cv);
+}
+
+// any C, any alignment
+template <typename U>
+__global__ void __launch_bounds__(kGatherBlock)
+zero_rows_scalar_kernel(const int32_t* __restrict__ rows, U* __restrict__ table, uint64_t total,
+                        uint32_t C, uint32_t V) {
+    const uint64_t idx = (uint64_t)blockIdx.x * kGatherBlock + threadIdx.x;
+    if (idx >= total) return;
+    const uint64_t row = idx / C;
+    const uint32_t c = (uint32_t)(idx - row * C);
+    const int32_t tok = rows[row];
+    if (tok < 0 || (uint32_t)tok >= V) return;
+    table[(uint64_t)tok * C + c] = (U)0;
+}
+
 // scalar raw-bits gather (any C, any alignment)
 template <typename U>
 __global__ void __launch_bounds__(kGatherBlock)
@@ -717,7 +748,7 @@ __global__ void __launch_bounds__(kSortBlock) __attribute__((amdgpu_num_sgpr(80)
 gather_sort_kernel(const int32_t* __restrict__ ids, const T* __restrict__ W, const T* __restrict__ wpe,
                    T* __restrict__ out, uint32_t total, uint32_t CV, uint32_t C, uint32_t T_len, uint32_t V,
                    uint32_t* __restrict__ order, unsigned long long* __restrict__ spill,
-                   uint32_t N, uint32_t log2G, int* err_flag) {
+                   uint32_t N, uint32_t log2G, int* err_flag, int32_t* __restrict__ kept) {
     const uint32_t groups = 1u << log2G;
     if (blockIdx.x < groups) {
         emb_group_sort_body(blockIdx.x, ids, order, spill, N, V, log2G, err_flag);
@@ -762,6 +793,13 @@ gather_sort_kernel(const int32_t* __restrict__ ids, const T* __restrict__ W, con
                 VecIO<T, VEC>::store(out + (uint64_t)row[u] * C + cv[u] * VEC, v[u]);
             }
         }
+    }
+    // a copy of the ids this pass read, for the caller that later clears exactly the rows
+    // of the table's gradient that the backward pass of these ids stores
+    if (kept != nullptr) {
+#pragma unroll
+        for (int u = 0; u < kGatherPerThread; ++u)
+            if (cv[u] == 0 && first + u * kSortBlock < total) kept[row[u]] = tok[u];
     }
 }
 
@@ -1434,10 +1472,11 @@ int launch_embedding_order(hipStream_t s, const int32_t* ids, uint32_t* order, v
 // out = W[ids] (+ wpe) and order = the ids' ordering for the later gradient
 int launch_gather_fwd_sorted(hipStream_t s, int dtype, const int32_t* ids, const void* W, const void* wpe,
                              void* out, uint64_t N, uint32_t T, uint32_t C, uint32_t V, uint32_t* order,
-                             void* sort_workspace, uint64_t sort_workspace_bytes, int* err_flag) {
+                             void* sort_workspace, uint64_t sort_workspace_bytes, int* err_flag, int32_t* kept) {
     if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "gather: unknown dtype %d", dtype);
     if (N == 0) return AGRAD_OK;
     if (order == nullptr) return set_error(AGRAD_EINVAL, "gather: null order buffer");
+    if (kept != nullptr && (const int32_t*)kept == ids) return set_error(AGRAD_EINVAL, "gather: the kept ids may not be the ids");
     const uint32_t esz = dtype_size(dtype);
     const uint32_t per16 = 16 / esz;
     const bool wide = C > 0 && C % per16 == 0 && W != nullptr && out != nullptr && aligned16(W) && aligned16(out) &&
@@ -1447,6 +1486,10 @@ int launch_gather_fwd_sorted(hipStream_t s, int dtype, const int32_t* ids, const
                        ids != nullptr && (wpe == nullptr || T > 0);
     if (!fused) {
         if (int rc = launch_embedding_sort(s, ids, order, sort_workspace, sort_workspace_bytes, N, V, err_flag)) return rc;
+        if (kept != nullptr) {
+            if (ids == nullptr) return set_error(AGRAD_EINVAL, "gather: null ids");
+            if (int rc = launch_copy(s, ids, kept, N * 4)) return rc;
+        }
         if (C == 0) return AGRAD_OK;
         return launch_gather_fwd(s, dtype, ids, W, wpe, out, N, T, C, V, err_flag);
     }
@@ -1466,13 +1509,13 @@ int launch_gather_fwd_sorted(hipStream_t s, int dtype, const int32_t* ids, const
         return set_error(AGRAD_EINVAL, "gather: the order buffer must be 16-byte aligned");
     if (wpe == nullptr) {
         hipLaunchKernelGGL((gather_sort_kernel<float, 4, true>), dim3(grid), dim3(kSortBlock), 0, s, ids, (const float*)W,
-                           (const float*)nullptr, (float*)out, total, CV, C, T ? T : 1u, V, order, spill, n, log2G, err_flag);
+                           (const float*)nullptr, (float*)out, total, CV, C, T ? T : 1u, V, order, spill, n, log2G, err_flag, kept);
     } else if (dtype == AGRAD_F32) {
         hipLaunchKernelGGL((gather_sort_kernel<float, 4, false>), dim3(grid), dim3(kSortBlock), 0, s, ids, (const float*)W,
-                           (const float*)wpe, (float*)out, total, CV, C, T, V, order, spill, n, log2G, err_flag);
+                           (const float*)wpe, (float*)out, total, CV, C, T, V, order, spill, n, log2G, err_flag, kept);
     } else {
         hipLaunchKernelGGL((gather_sort_kernel<bf16_t, 8, false>), dim3(grid), dim3(kSortBlock), 0, s, ids, (const bf16_t*)W,
-                           (const bf16_t*)wpe, (bf16_t*)out, total, CV, C, T, V, order, spill, n, log2G, err_flag);
+                           (const bf16_t*)wpe, (bf16_t*)out, total, CV, C, T, V, order, spill, n, log2G, err_flag, kept);
     }
     return check_hip(hipGetLastError(), "gather launch");
 }
@@ -1550,6 +1593,34 @@ int launch_gather_fwd(hipStream_t s, int dtype, const int32_t* ids, const void* 
                                (const bf16_t*)W, (const bf16_t*)wpe, (bf16_t*)out, total, C, T, V, err_flag);
     }
     return check_hip(hipGetLastError(), "gather launch");
+}
+
+int launch_embedding_grad_reset(hipStream_t s, int dtype, const int32_t* rows, uint64_t N, void* dW,
+                                uint32_t C, uint32_t V) {
+    if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "embedding grad reset: unknown dtype %d", dtype);
+    if (N == 0 || C == 0 || V == 0) return AGRAD_OK;
+    if (rows == nullptr || dW == nullptr) return set_error(AGRAD_EINVAL, "embedding grad reset: null operand");
+    const uint32_t esz = dtype_size(dtype);
+    const uint32_t per16 = 16 / esz;
+    const bool wide = C % per16 == 0 && aligned16(dW);
+    const uint64_t total_vec = wide ? N * (C / per16) : 0;
+    if (wide && total_vec < 0xffff0000ull) {
+        const uint32_t total = (uint32_t)total_vec;
+        const uint32_t grid = (total + kGatherBlock - 1) / kGatherBlock;
+        hipLaunchKernelGGL(zero_rows16_kernel, dim3(grid), dim3(kGatherBlock), 0, s, rows, (u32x4*)dW, total,
+                           C / per16, V);
+    } else {
+        const uint64_t total = N * C;
+        const uint64_t grid = (total + kGatherBlock - 1) / kGatherBlock;
+        if (grid > 0x7fffffffull) return set_error(AGRAD_EINVAL, "embedding grad reset: too many items");
+        if (dtype == AGRAD_F32)
+            hipLaunchKernelGGL((zero_rows_scalar_kernel<uint32_t>), dim3((uint32_t)grid), dim3(kGatherBlock), 0, s,
+                               rows, (uint32_t*)dW, total, C, V);
+        else
+            hipLaunchKernelGGL((zero_rows_scalar_kernel<uint16_t>), dim3((uint32_t)grid), dim3(kGatherBlock), 0, s,
+                               rows, (uint16_t*)dW, total, C, V);
+    }
+    return check_hip(hipGetLastError(), "embedding grad reset launch");
 }
 
 // one workspace for the unsorted entry point: [order | sort scratch | partial rows]

@@ -141,9 +141,11 @@ int launch_embedding_sort(hipStream_t s, const int32_t* ids, uint32_t* order, vo
 int launch_embedding_order(hipStream_t s, const int32_t* ids, uint32_t* order, void* sort_workspace,
                            uint64_t sort_workspace_bytes, uint64_t N, uint32_t V, void* zero_dst, uint64_t zero_bytes,
                            int* err_flag);
+int launch_embedding_grad_reset(hipStream_t s, int dtype, const int32_t* rows, uint64_t N, void* dW,
+                                uint32_t C, uint32_t V);
 int launch_gather_fwd_sorted(hipStream_t s, int dtype, const int32_t* ids, const void* W, const void* wpe,
                              void* out, uint64_t N, uint32_t T, uint32_t C, uint32_t V, uint32_t* order,
-                             void* sort_workspace, uint64_t sort_workspace_bytes, int* err_flag);
+                             void* sort_workspace, uint64_t sort_workspace_bytes, int* err_flag, int32_t* kept = nullptr);
 uint64_t embedding_bwd_sorted_workspace_bytes(uint64_t N, uint32_t C);
 // dwpe (optional, [T, C]): the position table's gradient sum_b dY[b, t, :] rides in the same launch
 int launch_embedding_bwd_sorted(hipStream_t s, int dtype, uint32_t* order, const void* dY, void* dW,

@@ -23,7 +23,7 @@ from .utils import broadcast_shape, mul_bcast_kind
 
 class OpNode:
     __slots__ = ("op", "inputs", "outputs", "forward", "backward", "scratch_fwd_layout",
-                 "scratch_bwd_layout", "name", "overwrite_grads", "defer_param_grads", "order_ready")
+                 "scratch_bwd_layout", "name", "overwrite_grads", "defer_param_grads", "order_ready", "kept_ids", "kept_fresh")
 
     def __init__(self, op, inputs, outputs, name=""):
         self.op = op
@@ -45,6 +45,12 @@ class OpNode:
         # ordering rode with the zero fill of the table's gradient): its forward kernel is then
         # the plain gather.  Set by Runtime.execute, cleared by the node's backward kernel.
         self.order_ready = False
+        # an embedding node whose table has a gradient: a buffer outside the arena in which the
+        # forward kernel leaves a copy of the ids it read (set by the runtime), and whether that
+        # copy is of the forward pass the next backward pass belongs to.  The table's gradient is
+        # then cleared row by row (those ids' rows) instead of as a whole.
+        self.kept_ids = None
+        self.kept_fresh = False
 
 
 class Op(ABC):

@@ -98,7 +98,7 @@ class Runtime:
         return cls._default_runtime
 
     def __init__(self, device="hip", forward_only=False, owns_params=True, use_fp16_gemm=False,
-                 fuse_grad_zeroing=True, defer_param_grad_sums=True):
+                 fuse_grad_zeroing=True, defer_param_grad_sums=True, row_reset=True):
         self.loss = None
         self.topo = []
         self.forward_only = forward_only
@@ -121,6 +121,11 @@ class Runtime:
         # the end of backward_graph folds them all (same bits as folding each on its own).
         self.defer_param_grad_sums = bool(defer_param_grad_sums
                                           and getattr(self.backend, "supports_deferred_param_grads", False))
+        # The gradient of an embedding table is zero outside the rows of the last pass's ids:
+        # zero_grad clears those rows (N*C items) instead of filling the table (V*C items; 1 GB
+        # at V = 151936, C = 1536 fp32, where the rows are 100 MB).  The forward kernel keeps the
+        # copy of the ids that names them.
+        self.row_reset = bool(row_reset and getattr(self.backend, "supports_row_reset", False))
         self.arena_bytes = 0
         self._owns_arena = False       # release() frees only an arena this runtime allocated
         self.memory_plan = None        # key -> arena offset, set by plan_memory()
@@ -206,6 +211,12 @@ class Runtime:
             node.scratch_fwd_layout, node.scratch_bwd_layout = fwd, (None if self.forward_only else bwd)
             node.defer_param_grads = bool(self.defer_param_grad_sums and node.scratch_bwd_layout is not None
                                           and self.backend.can_defer_param_grads(node))
+            # an embedding whose table takes a gradient keeps a copy of each pass's ids outside
+            # the arena: the rows to clear in that gradient before the next pass
+            if self.row_reset and not self.forward_only and node.op.early_outputs and len(node.outputs) > 1 \
+                    and node.inputs[1].grad is not None and node.kept_ids is None:
+                node.kept_ids = self.allocator.alloc((prod(node.inputs[0].shape),), np.int32)
+                self._slabs.append(node.kept_ids)
 
         self._resolve_aliases()
 
@@ -514,7 +525,10 @@ class Runtime:
                     if order_ids and node.op.early_outputs and len(node.inputs) > 1 and node.inputs[1] is t \
                             and hasattr(self.backend, "zero_grad_and_order") and self.backend.zero_grad_and_order(node, t):
                         continue
-                    self.backend.fill(t.grad, 0)
+                    if self.row_reset and t.grad.dirty_rows is not None:
+                        self.backend.clear_table_grad(t)
+                    else:
+                        self.backend.fill(t.grad, 0)
 
     def _require_bound(self):
         if self.memory_plan is not None and self.arena_bytes and self.unified_arena is None:

@@ -201,11 +201,18 @@ def _embed_cases(ctx, cfg, pool, rng, nbytes, ids0):
         def zero_and_order(i):
             ctx.call("agrad_embedding_order", vp(ids[i]), N, cfg.V, vp(order[i]), vp(sort_ws), sort_ws_bytes, vp(dW), dW.nbytes)
 
+        # "..._grad_row_reset": the table gradient brought back to zero by clearing the rows of the last
+        # pass's ids (agrad_embedding_grad_reset, what Runtime.zero_grad does after the first step) --
+        # N*C items written instead of the fill's V*C.
+        def row_reset(i):
+            ctx.call("agrad_embedding_grad_reset", dt, vp(ids[i]), N, vp(dW), Cw, cfg.V)
+
         cases.append(Case(name, "fwd", nbytes[name][0], k, fwd, "gather_sort_kernel"))
         cases.append(Case(name, "fwd-plain", nbytes[name][0], k, fwd_plain, "gather_", in_step=False))
         cases.append(Case(name, "bwd", nbytes[name][1], k, bwd, "emb_row_sum_kernel"))
         cases.append(Case("id_ordering", "aux", 4 * N + 4 * (6 * N + 128), k, order_alone, "emb_group_sort_kernel"))
         cases.append(Case(name + "_grad_zero_fill", "aux", cfg.V * Cw * e, 1, zero, "fill16_kernel"))
+        cases.append(Case(name + "_grad_row_reset", "aux", N * Cw * e, k, row_reset, "zero_rows16_kernel"))
         cases.append(Case(name + "_grad_zero_fill+order", "aux", cfg.V * Cw * e, k, zero_and_order, "fill_order_kernel"))
     return cases
 
@@ -780,7 +787,7 @@ def runtime_path(cfg, per_op_rows, steps=20, ctx=None):
     if cfg.act:
         names.add(cfg.act)
     kernels = [r for r in per_op_rows if (r["op"] in names and r["dir"] in ("fwd", "bwd"))
-               or r["op"] == cfg.embed + "_grad_zero_fill"]
+               or r["op"] == cfg.embed + "_grad_row_reset"]     # (what zero_grad launches after the first step)
     c_abi_us = sum(r["us"] for r in kernels)
     # the protocol's own fills, through the C ABI as well: the upstream gradient of each graph's output
     fill_us = 0.0

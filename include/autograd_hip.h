@@ -399,6 +399,13 @@ uint64_t agrad_embedding_sort_workspace_bytes(uint64_t N, uint32_t V);
 int agrad_gather_forward_sorted(agrad_ctx* ctx, int dtype, const int32_t* ids, const void* W, const void* wpe,
                                 void* out, uint64_t N, uint32_t T, uint32_t C, uint32_t V,
                                 uint32_t* order, void* sort_workspace, uint64_t sort_workspace_bytes);
+/* The same call, which also leaves a copy of the N ids it read in ids_kept (not the ids'
+ * own buffer): the list agrad_embedding_grad_reset needs after the backward call of this
+ * order, in memory the caller's next batch of ids does not overwrite. */
+int agrad_gather_forward_sorted_kept(agrad_ctx* ctx, int dtype, const int32_t* ids, const void* W, const void* wpe,
+                                     void* out, uint64_t N, uint32_t T, uint32_t C, uint32_t V,
+                                     uint32_t* order, void* sort_workspace, uint64_t sort_workspace_bytes,
+                                     int32_t* ids_kept);
 /* The ordering alone: writes `order` (same layout, same bits as the forward call above
  * leaves) from the ids, and -- when zero_dst is not NULL -- clears zero_dst[0 .. zero_bytes)
  * in the same launch, for a caller that zero-fills the table's gradient and orders the ids
@@ -413,6 +420,16 @@ int agrad_gather_forward_sorted(agrad_ctx* ctx, int dtype, const int32_t* ids, c
 int agrad_embedding_order(agrad_ctx* ctx, const int32_t* ids, uint64_t N, uint32_t V, uint32_t* order,
                           void* sort_workspace, uint64_t sort_workspace_bytes,
                           void* zero_dst, uint64_t zero_bytes);
+/* Clears the rows of dW[V, C] that `rows[0 .. N)` names (ids outside [0, V) are skipped):
+ * N*C items written where a fill of the table writes V*C.  An embedding table's gradient
+ * is zero outside the rows its backward call stored, so a caller that keeps the ids of
+ * the last backward call can bring the table back to all-zero with this call instead of
+ * agrad_fill once the optimizer has read it -- 1/3 to 1/50 of the fill's bytes at the
+ * benchmark shapes.  The caller answers for the list: rows a backward call wrote that it
+ * does not name stay as they are.  The reference clears the whole table on every forward
+ * gather (metal_gather_forward, backend.py:2781-2785). */
+int agrad_embedding_grad_reset(agrad_ctx* ctx, int dtype, const int32_t* rows, uint64_t N, void* dW,
+                               uint32_t C, uint32_t V);
 uint64_t agrad_embedding_backward_sorted_workspace_bytes(uint64_t N, uint32_t C);
 /* `order` is read AND written: the call counts arrivals in the counters at its end and leaves
  * them zero again; they must be zero on entry, which the calls that write an order guarantee

@@ -1017,6 +1017,85 @@ def test_presorted_embedding_pair_matches_the_plain_pair(ctx, B, T, V, C, dist, 
             d.free()
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("B,T,V,C,dist", [(32, 512, 32768, 384, "uniform"), (2, 700, 300, 48, "zipf"),
+                                          (5, 14000, 3000, 32, "zipf"), (3, 50, 77, 10, "uniform")])
+def test_table_gradient_cleared_by_rows(ctx, dtype, B, T, V, C, dist):
+    """agrad_gather_forward_sorted_kept is the sorted forward call and leaves a copy of its ids;
+    after the backward call of that order agrad_embedding_grad_reset with the copy brings the
+    gradient table back to all zero, touching nothing outside the listed rows (the rows of other
+    ids and the guard rows around the table keep their values).  (5, 14000) takes the forward
+    call's two-launch path, C = 10 the reset's scalar kernel; ids outside the table are skipped."""
+    import ctypes as Ct
+    rng = _rng(170 + C)
+    N = B * T
+    dt = capi.BF16 if dtype == "bf16" else capi.F32
+    if dist == "zipf":
+        p = np.arange(1, V + 1, dtype=np.float64) ** -1.1
+        ids = rng.choice(V, size=(B, T), p=p / p.sum()).astype(np.int32)
+    else:
+        ids = rng.integers(0, V, (B, T), dtype=np.int32)
+    up = (lambda a: ctx.upload(to_bf16_bits(a))) if dtype == "bf16" else ctx.upload
+    np_t = np.uint16 if dtype == "bf16" else np.float32
+    W = (0.02 * rng.standard_normal((V, C))).astype(np.float32)
+    dY = rng.standard_normal((B, T, C)).astype(np.float32)
+
+    def vp(d, off=0):
+        return Ct.c_void_p(d.ptr + off) if d is not None else None
+    d_ids, d_W, d_dY = ctx.upload(ids), up(W), up(dY)
+    out_a, out_b = ctx.empty((N, C), np_t), ctx.empty((N, C), np_t)
+    order_a, order_b = ctx.empty((6 * N + 128,), np.uint32), ctx.empty((6 * N + 128,), np.uint32)
+    kept = ctx.upload(np.full(N + 2, -5, np.int32))          # one guard word either side
+    sws_b = ctx.lib.agrad_embedding_sort_workspace_bytes(N, V)
+    bws_b = ctx.lib.agrad_embedding_backward_sorted_workspace_bytes(N, C)
+    sws, bws = ctx.empty((sws_b,), np.uint8), ctx.empty((bws_b,), np.uint8)
+    ctx.call("agrad_gather_forward_sorted", dt, vp(d_ids), vp(d_W), None, vp(out_a), N, T, C, V, vp(order_a), vp(sws), sws_b)
+    ctx.call("agrad_gather_forward_sorted_kept", dt, vp(d_ids), vp(d_W), None, vp(out_b), N, T, C, V, vp(order_b), vp(sws),
+             sws_b, vp(kept, 4))
+    ctx.synchronize()
+    np.testing.assert_array_equal(out_b.download(), out_a.download())
+    info_at = (N + 3) & ~3
+    used = info_at + 4 * N + (N // 128 + 1) * 32 + (N // 2048 + 1) * 32
+    wa, wb = order_a.download(), order_b.download()
+    np.testing.assert_array_equal(np.concatenate([wb[:N], wb[info_at:used]]), np.concatenate([wa[:N], wa[info_at:used]]))
+    got_kept = kept.download()
+    np.testing.assert_array_equal(got_kept[1:-1], ids.reshape(-1))
+    assert got_kept[0] == -5 and got_kept[-1] == -5
+    # a table of sevens between two guard rows: the backward call stores the rows of the ids
+    e = 2 if dtype == "bf16" else 4
+    seven = np.full((V + 2, C), 7.0, np.float32)
+    dW = up(seven)
+    seven_bits = dW.download().copy()
+    ctx.call("agrad_embedding_backward_sorted", dt, vp(order_b), vp(d_dY), vp(dW, C * e), None, vp(bws), bws_b, N, T, C, V, 0)
+    ctx.call("agrad_embedding_grad_reset", dt, vp(kept, 4), N, vp(dW, C * e), C, V)
+    ctx.synchronize()
+    table = dW.download().reshape(V + 2, C)
+    present = np.zeros(V + 2, bool)
+    present[ids.reshape(-1) + 1] = True
+    assert not table[present].any()
+    np.testing.assert_array_equal(table[~present], seven_bits.reshape(V + 2, C)[~present])
+    # ids outside the table name no row
+    bad = ids.reshape(-1).copy()
+    bad[::3] = V + 5
+    bad[1::7] = -1
+    d_bad = ctx.upload(bad)
+    dW2 = up(seven)
+    ctx.call("agrad_embedding_grad_reset", dt, vp(d_bad), N, vp(dW2, C * e), C, V)
+    ctx.synchronize()
+    table = dW2.download().reshape(V + 2, C)
+    ok = bad[(bad >= 0) & (bad < V)]
+    present = np.zeros(V + 2, bool)
+    present[ok + 1] = True
+    assert not table[present].any()
+    np.testing.assert_array_equal(table[~present], seven_bits.reshape(V + 2, C)[~present])
+    # the copy may not be the ids' own buffer
+    with pytest.raises(capi.AgradError):
+        ctx.call("agrad_gather_forward_sorted_kept", dt, vp(d_ids), vp(d_W), None, vp(out_b), N, T, C, V, vp(order_b),
+                 vp(sws), sws_b, vp(d_ids))
+    for d in (d_ids, d_W, d_dY, out_a, out_b, order_a, order_b, kept, sws, bws, dW, dW2, d_bad):
+        d.free()
+
+
 @pytest.mark.parametrize("B,T,V,C,dist", [(32, 512, 32768, 384, "uniform"), (2, 700, 300, 48, "zipf"),
                                           (5, 14000, 3000, 32, "zipf"), (3, 50, 77, 10, "uniform")])
 def test_ordering_with_the_zero_fill_matches_the_forward_call(ctx, B, T, V, C, dist):

@@ -807,3 +807,158 @@ def test_ids_ordered_with_the_zero_fill(with_wpe):
     for a, b in zip(results["execute"], results["protocol"]):
         for x, y in zip(a, b):
             np.testing.assert_array_equal(x, y)
+
+
+def _launch_log(rt):
+    """records the kernel names the runtime's backend launches from now on"""
+    names = []
+    plain = rt.backend._launch
+
+    def logged(name, tensors, args):
+        names.append(name)
+        plain(name, tensors, args)
+    rt.backend._launch = logged
+    return names, lambda: setattr(rt.backend, "_launch", plain)
+
+
+@pytest.mark.parametrize("with_wpe", [False, True])
+@pytest.mark.parametrize("protocol", ["execute", "manual", "graph"])
+def test_table_gradient_cleared_by_rows_over_steps(with_wpe, protocol):
+    """From the second step on zero_grad clears the rows of the last pass's ids in the table's
+    gradient instead of filling the table; the gradients are those of a runtime that fills, bit
+    for bit, step after step with new ids -- through execute, through the reference's manual
+    protocol with the ids changed between zero_grad and forward, and through replays of a
+    recorded execute."""
+    B, T, C, V = 8, 256, 96, 1000
+    dev = "hip"
+    results = {}
+    for row_reset in (True, False):
+        r2 = np.random.default_rng(SEED + 101)
+        ids = make_tensor((B, T), np.int32, dev, False, r2.integers(0, V, (B, T), dtype=np.int32))
+        wte = make_tensor((V, C), np.float32, dev, True, (0.5 * r2.standard_normal((V, C))).astype(np.float32))
+        g = make_tensor((C,), np.float32, dev, True, np.ones(C, np.float32))
+        if with_wpe:
+            wpe = make_tensor((T, C), np.float32, dev, True, (0.5 * r2.standard_normal((T, C))).astype(np.float32))
+            x0 = EmbeddingSumOp()(ids, wte, wpe)
+        else:
+            x0 = GatherOp()(ids, wte)
+        out = RMSNormOp(eps=1e-6)(x0, g)
+        rt = Runtime(device=dev, row_reset=row_reset)
+        rt.loss = out
+        rt.grad_scale = 0.5
+        rt.build_topo(out)
+        rt.bind_memory()
+        assert (x0.op.kept_ids is not None) == row_reset
+        names, restore = _launch_log(rt)
+        graph = None
+        steps = []
+        for step in range(4):
+            new_ids = np.random.default_rng(SEED + 102 + step).integers(0, V, (B, T), dtype=np.int32)
+            del names[:]
+            if protocol == "manual":
+                rt.zero_grad()
+                rt.backend.copy_from_host(ids, new_ids)
+                rt.forward()
+                rt.backend.fill(out.grad, 0.5)
+                rt.backward_graph()
+            elif protocol == "graph" and step >= 2:
+                rt.backend.copy_from_host(ids, new_ids)
+                if graph is None:
+                    graph = rt.capture(rt.execute)
+                    assert ("embedding_grad_reset" in names) == row_reset
+                graph.launch()
+            else:
+                rt.backend.copy_from_host(ids, new_ids)
+                rt.execute()
+            rt.backend.synchronize()
+            if graph is None:
+                assert ("embedding_grad_reset" in names) == (row_reset and step > 0), names
+            dW = rt.backend.copy_to_host(wte.grad).copy()
+            absent = np.ones(V, bool)
+            absent[new_ids.reshape(-1)] = False
+            assert not dW[absent].any(), f"step {step}: rows of ids that are not in this pass"
+            steps.append([rt.backend.copy_to_host(t).copy() for t in (out, g.grad)] + [dW]
+                         + ([rt.backend.copy_to_host(wpe.grad).copy()] if with_wpe else []))
+        results[row_reset] = steps
+        restore()
+        if graph is not None:
+            graph.destroy()
+        rt.release()
+    for a, b in zip(results[True], results[False]):
+        for x, y in zip(a, b):
+            np.testing.assert_array_equal(x, y)
+
+
+def test_row_reset_falls_back_to_the_fill():
+    """The rows to clear are known only while embedding nodes' backward passes are all that wrote the
+    table's gradient since it was last zero: two micro-steps that accumulate or a host write into
+    the gradient end in the plain fill.  A table that two embeddings share is cleared by both
+    lists."""
+    B, T, C, V = 4, 128, 64, 500
+    dev = "hip"
+    r2 = np.random.default_rng(SEED + 111)
+    ids_a = make_tensor((B, T), np.int32, dev, False, r2.integers(0, V, (B, T), dtype=np.int32))
+    ids_b = make_tensor((B, T), np.int32, dev, False, r2.integers(0, V, (B, T), dtype=np.int32))
+    wte = make_tensor((V, C), np.float32, dev, True, (0.5 * r2.standard_normal((V, C))).astype(np.float32))
+    g = make_tensor((C,), np.float32, dev, True, np.ones(C, np.float32))
+    xa, xb = GatherOp()(ids_a, wte), GatherOp()(ids_b, wte)
+    out = RMSNormOp(eps=1e-6)(AddOp()(xa, xb), g)
+    rt = Runtime(device=dev)
+    rt.loss = out
+    rt.grad_scale = 0.25
+    rt.build_topo(out)
+    rt.bind_memory()
+    names, restore = _launch_log(rt)
+
+    def run(a, b):
+        rt.backend.copy_from_host(ids_a, a)
+        rt.backend.copy_from_host(ids_b, b)
+        del names[:]
+        rt.execute()
+        rt.backend.synchronize()
+        return rt.backend.copy_to_host(wte.grad).copy()
+
+    def new_ids(k):
+        r = np.random.default_rng(SEED + 112 + k)
+        return r.integers(0, V, (B, T), dtype=np.int32), r.integers(0, V, (B, T), dtype=np.int32)
+
+    def rows_of(*id_arrays):
+        m = np.zeros(V, bool)
+        for a in id_arrays:
+            m[a.reshape(-1)] = True
+        return m
+    a0, b0 = new_ids(0)
+    run(a0, b0)
+    assert "embedding_grad_reset" not in names
+    a1, b1 = new_ids(1)
+    dW = run(a1, b1)
+    assert names.count("embedding_grad_reset") == 2          # one list per embedding
+    assert not dW[~rows_of(a1, b1)].any() and dW[rows_of(a1, b1)].any()
+    # two micro-steps that accumulate: the union of their rows is in no list
+    rt.accumulate_parameter_grads = True
+    rt.zero_grad()
+    a2, b2 = new_ids(2)
+    run(a2, b2)
+    a3, b3 = new_ids(3)
+    dW = run(a3, b3)
+    assert dW[rows_of(a2, b2) & ~rows_of(a3, b3)].any()      # rows of the first micro-step are still there
+    del names[:]
+    rt.zero_grad()
+    rt.backend.synchronize()
+    assert "embedding_grad_reset" not in names
+    assert not rt.backend.copy_to_host(wte.grad).any()
+    rt.accumulate_parameter_grads = False
+    # a host write into the gradient
+    a4, b4 = new_ids(4)
+    run(a4, b4)
+    rt.backend.copy_from_host(wte.grad, np.full((V, C), 3.0, np.float32))
+    a5, b5 = new_ids(5)
+    dW = run(a5, b5)
+    assert "embedding_grad_reset" not in names
+    assert not dW[~rows_of(a5, b5)].any()
+    a6, b6 = new_ids(6)
+    dW = run(a6, b6)
+    assert names.count("embedding_grad_reset") == 2
+    assert not dW[~rows_of(a6, b6)].any()
+    restore()
+    rt.release()
