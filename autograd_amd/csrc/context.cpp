@@ -31,6 +31,8 @@ struct agrad_ctx {
     // column sums (dgamma / dbeta, bias gradients) that backward calls with AGRAD_DEFER_PARAM_GRAD
     // left unfolded: their partial rows wait in the callers' workspaces for agrad_finalize_param_grads
     std::vector<agrad::ColsumJob> pending;
+    // counters and (max, sum) pairs of the workgroup teams of the fused cross-entropy (long rows)
+    void* ce_scratch = nullptr;
 };
 
 namespace agrad {
@@ -107,7 +109,12 @@ int finish_stream(agrad_ctx* ctx) {
     if (int rc = no_capture(ctx, "synchronize / end_pass")) return rc;
     if (int rc = flush_pending(ctx)) return rc;      // nothing a caller waits for stays unfolded
     if (int rc = check_hip(hipStreamSynchronize(ctx->stream), "stream synchronize")) return rc;
-    if (*ctx->err_host != 0) {                 // (the stream has drained: every kernel's write has landed)
+    if (ctx->err_host[1] != 0) {               // (the stream has drained: every kernel's write has landed)
+        ctx->err_host[0] = ctx->err_host[1] = 0;
+        return set_error(AGRAD_EHIP, "fused cross-entropy: a team of workgroups did not assemble in time; the gradient "
+                                     "it left is not valid");
+    }
+    if (*ctx->err_host != 0) {
         *ctx->err_host = 0;
         return set_error(AGRAD_EINDEX, "index out of range on the device (a token id or a class label)");
     }
@@ -478,7 +485,7 @@ int h_ce_fused(const Call& c) {
     void* row_scale = nullptr;
     if (ROW_SCALED) { if (int rc_ = resolve(c.ctx, c.ids[4], c.offs[4], upto, "row_scale", &row_scale)) return rc_; }
     return launch_ce_fused(c.ctx->stream, (int)c.a[5], logits, (const int32_t*)targets, (float*)row_loss, (float*)lse,
-                           (const float*)row_scale, rows, V, row_base, ROW_SCALED ? 1.0f : f32(c.a[3]), c.a[4]);
+                           (const float*)row_scale, rows, V, row_base, ROW_SCALED ? 1.0f : f32(c.a[3]), c.a[4], c.ctx->ce_scratch, c.ctx->err_flag);
 }
 // buffers ids, order, sort_workspace, zero_dst | args N, V, ws_lo, ws_hi, zero_lo, zero_hi, present_mask
 int h_emb_order(const Call& c) {
@@ -630,6 +637,7 @@ int agrad_ctx_create(int device, agrad_ctx** out) {
         c->err_host = static_cast<volatile int*>(pinned);
         e = hipHostGetDevicePointer((void**)&c->err_flag, pinned, 0);
     }
+    if (e == hipSuccess) e = hipMalloc(&c->ce_scratch, ce_fused_scratch_bytes());
     if (e != hipSuccess) {
         agrad_ctx_destroy(c);
         return check_hip(e, "context setup");
@@ -644,6 +652,7 @@ int agrad_ctx_destroy(agrad_ctx* ctx) {
     if (ctx->stream) (void)hipStreamSynchronize(ctx->stream);
     for (auto& kv : ctx->graphs) (void)hipGraphExecDestroy(kv.second);
     for (auto& kv : ctx->allocs) (void)hipFree(reinterpret_cast<void*>(kv.first));
+    if (ctx->ce_scratch) (void)hipFree(ctx->ce_scratch);
     if (ctx->err_host) (void)hipHostFree(const_cast<int*>(ctx->err_host));
     if (ctx->ev_start) (void)hipEventDestroy(ctx->ev_start);
     if (ctx->ev_stop) (void)hipEventDestroy(ctx->ev_stop);
@@ -1114,7 +1123,8 @@ int agrad_cross_entropy_fused(agrad_ctx* ctx, int dtype, void* logits, const int
                               float* lse, const float* row_scale, uint64_t rows, uint32_t V, uint64_t row_base,
                               float scale, uint32_t write_grad) {
     CTX_OR_FAIL(ctx)
-    return launch_ce_fused(ctx->stream, dtype, logits, targets, row_loss, lse, row_scale, rows, V, row_base, scale, write_grad);
+    return launch_ce_fused(ctx->stream, dtype, logits, targets, row_loss, lse, row_scale, rows, V, row_base, scale, write_grad,
+                           ctx->ce_scratch, ctx->err_flag);
 }
 int agrad_cross_entropy_backward(agrad_ctx* ctx, int dtype, const void* logits, const int32_t* labels,
                                  const float* dloss, const float* lse, void* dlogits,

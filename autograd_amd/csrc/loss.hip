@@ -397,6 +397,30 @@ struct CeFusedArgs {
     uint32_t V, row_base; float scale; uint32_t write_grad;
 };
 
+// exp(x - shift) in the fused kernels.  bf16 rows fold the subtraction into the argument of
+// the hardware exp2 (one fma: `bias` = -shift * log2 e); the kernel that holds a long bf16 row
+// issues vector instructions for most of its run time, and this is one of its ten an element.
+template <typename T> __device__ __forceinline__ float exp_shifted(float x, float shift, float) { return exp_io<T>(x - shift); }
+template <> __device__ __forceinline__ float exp_shifted<bf16_t>(float x, float, float bias) {
+    return __builtin_amdgcn_exp2f(__builtin_fmaf(x, kLog2eHi, bias));
+}
+
+// One vector of the rewrite: v[k] = (e[k] * inv - [first + k == hit]) * mul.  The target is
+// looked for once a vector, not once an element (a compare, a select and an add of the
+// five instructions an element otherwise costs here).
+template <int VEC>
+__device__ __forceinline__ void ce_rewrite(float (&v)[VEC], float inv, float mul, uint32_t first, uint32_t hit) {
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) v[k] = v[k] * inv;
+    if (hit - first < (uint32_t)VEC) {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k)
+            if (first + k == hit) v[k] = v[k] - 1.0f;
+    }
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) v[k] = v[k] * mul;
+}
+
 // what thread 0 leaves for the row
 __device__ __forceinline__ void ce_fused_row_results(const CeFusedArgs& a, uint32_t grow, bool valid, float lse,
                                                      float target_logit) {
@@ -574,6 +598,214 @@ ce_fused_mem_kernel(T* x, const CeFusedArgs a) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// The same, with a row shared by a TEAM of workgroups.  A row that one workgroup holds in
+// registers makes that workgroup read, compute and write in turn, and at most two such
+// workgroups fit a CU: measured, the pattern alone (load all, barrier, store all) moves
+// 0.88 of what a streaming copy moves, and rows beyond 80 K classes do not fit at all.  Here
+// G workgroups of 256 threads take a slice of the row each -- a few vectors a thread, so
+// many workgroups share a CU and their phases interleave like a stream's -- and exchange
+// one (max, sum) pair per slice through memory:
+//   slice:  m_j = max x,  s_j = sum exp(x - m_j)        (the slice stays in registers)
+//   post:   two 64-bit device-scope stores, {m_j, tag} and {s_j, tag}: each word says by
+//           its tag which row of the launch it belongs to, so no store has to wait for
+//           another and no counter is needed
+//   next:   the loads of the team's next row, into a second set of registers
+//   wait:   lane j of the first wave polls member j's two words (device-scope loads)
+//           until both carry this row's tag; the other waves sit at the workgroup barrier
+//   row:    M = max m_j,  S = sum_j s_j exp(m_j - M), j ascending: the same in every
+//           member, which then rewrites its slice as (exp(x - M) / S - onehot) * scale
+// The grid is what is resident at once (the occupancy the runtime reports, times the
+// CUs), teams are neighbours in it, and a team walks rows team, team + teams, ...: every
+// member of a team is on the GPU while the others wait for it.  The wait is bounded all
+// the same: a member that is not joined within kTeamSpinBudget polls sets the second
+// error word, stops waiting for the rest of the launch and finishes (with wrong numbers;
+// the pass boundary reports the error) -- no wave waits for ever.
+// Tags are the team's row count + 1; a fill in front of the launch clears the words.  The
+// words alternate between two sets by the parity of the row count, so a fast member's next
+// post cannot land on a pair that a slow one has yet to read (it posts row r + 2 only after
+// everyone has posted r + 1, which each does after reading the pairs of r).
+// ---------------------------------------------------------------------------
+constexpr int kTeamBlock = 256;
+constexpr uint32_t kTeamMaxMembers = 32, kTeamMaxTeams = 2048;
+constexpr uint32_t kTeamSpinBudget = 1u << 20;         // polls of ~1 us
+constexpr uint64_t kTeamWordsPerTeam = 2ull * kTeamMaxMembers * 2;      // two sets of {m, tag}, {s, tag} per member
+constexpr uint64_t kTeamScratchBytes = (uint64_t)kTeamMaxTeams * kTeamWordsPerTeam * 8;
+
+// what a row needs besides its vectors: the element before / after the aligned part that
+// this thread owns (member 0), the target and the target's logit
+struct CeRowExtras {
+    float xe, target_logit;
+    int32_t target;
+};
+
+template <typename T, int VEC, int NV>
+__global__ void __launch_bounds__(kTeamBlock)
+ce_fused_team_kernel(T* x, const CeFusedArgs a, uint32_t rows, uint32_t G, uint32_t teams,
+                     unsigned long long* words, int* err_words) {
+    constexpr int BLOCK = kTeamBlock;
+    __shared__ float lds[BLOCK / kWave];
+    __shared__ float team_m[kTeamMaxMembers], team_s[kTeamMaxMembers];
+    __shared__ uint32_t alone;                  // this workgroup has stopped waiting for its team
+    typedef RawVec<T, VEC> Raw;
+    const uint32_t V = a.V, tid = threadIdx.x;
+    const uint32_t team = blockIdx.x / G, member = blockIdx.x - team * G;
+    unsigned long long* slots = words + (uint64_t)team * kTeamWordsPerTeam;
+    if (tid == 0) alone = 0;
+    __syncthreads();
+
+    // the slice of `member` in a row, and the requests for it
+    struct Slice { T* base; T* body; uint32_t head, tail_start, lo, hi; };
+    auto slice_of = [&](uint32_t row) {
+        Slice c;
+        c.base = x + (uint64_t)row * V;
+        const RowSplit<T, VEC> sp(c.base, V);
+        c.body = c.base + sp.head;
+        c.head = sp.head;
+        c.tail_start = sp.tail_start;
+        const uint32_t per = (sp.nvec + G - 1) / G;                     // vectors of a slice (at most NV * BLOCK)
+        c.lo = member * per < sp.nvec ? member * per : sp.nvec;
+        c.hi = c.lo + per < sp.nvec ? c.lo + per : sp.nvec;
+        return c;
+    };
+    auto ask = [&](const Slice& c, uint32_t grow, typename Raw::type (&raw)[NV], CeRowExtras& ex) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const uint32_t idx = c.lo + (uint32_t)i * BLOCK + tid;
+            raw[i] = Raw::load(c.body + (uint64_t)(idx < c.hi ? idx : 0u) * VEC);   // (past the slice: the row's first vector)
+        }
+        const uint32_t extra = member == 0 ? c.head + (V - c.tail_start) : 0u;
+        const uint32_t e_at = tid < c.head ? tid : c.tail_start + (tid - c.head);
+        float t1[1];
+        VecIO<T, 1>::load(c.base + (tid < extra ? e_at : 0u), t1);
+        ex.xe = t1[0];
+        ex.target = a.targets[grow];
+        VecIO<T, 1>::load(c.base + (ex.target >= 0 && (uint32_t)ex.target < V ? (uint32_t)ex.target : 0u), t1);
+        ex.target_logit = t1[0];
+    };
+
+    typename Raw::type raw[NV], ahead[NV];
+    CeRowExtras ex, ex_ahead;
+    uint32_t row = team;
+    if (row >= rows) return;
+    Slice c = slice_of(row);
+    ask(c, a.row_base + row, raw, ex);
+    for (uint32_t it = 0;; ++it) {
+        const uint32_t grow = a.row_base + row;
+        const uint32_t next = row + teams;
+        const bool more = next < rows;                                  // (uniform)
+        const uint32_t extra = member == 0 ? c.head + (V - c.tail_start) : 0u;
+        const uint32_t e_at = tid < c.head ? tid : c.tail_start + (tid - c.head);
+        const float xe = tid < extra ? ex.xe : -INFINITY;
+        const int32_t target = ex.target;
+        const bool in_range = target >= 0 && (uint32_t)target < V;
+        const float target_logit = ex.target_logit;
+
+        float m = xe;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const uint32_t idx = c.lo + (uint32_t)i * BLOCK + tid;
+            float v[VEC];
+            Raw::unpack(raw[i], v);
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) m = fmaxf(m, idx < c.hi ? v[k] : -INFINITY);
+        }
+        m = block_max<BLOCK>(m, lds);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) forget_unpacked(raw[i]);
+        const float own_shift = m > -INFINITY ? m : 0.0f;
+        const float own_bias = -own_shift * kLog2eHi;
+        float sum = tid < extra ? exp_io<T>(xe - own_shift) : 0.0f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const uint32_t idx = c.lo + (uint32_t)i * BLOCK + tid;
+            float v[VEC];
+            Raw::unpack(raw[i], v);
+            float part = 0.0f;
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) part = part + exp_shifted<T>(v[k], own_shift, own_bias);
+            sum = sum + (idx < c.hi ? part : 0.0f);
+        }
+        sum = block_sum<BLOCK>(sum, lds);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) forget_unpacked(raw[i]);
+
+        // post this slice's pair
+        const uint32_t tag = it + 1u;
+        unsigned long long* now = slots + (uint64_t)(it & 1u) * kTeamMaxMembers * 2;
+        if (tid == 0) {
+            const unsigned long long up = (unsigned long long)tag << 32;
+            __hip_atomic_store(now + member * 2, up | __float_as_uint(m), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(now + member * 2 + 1, up | __float_as_uint(sum), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        // the next row is on its way while the team assembles
+        const Slice c_next = slice_of(more ? next : row);
+        if (more) ask(c_next, a.row_base + next, ahead, ex_ahead);
+        // wait for the team's pairs
+        if (tid < G) {
+            unsigned long long w0 = 0, w1 = 0;
+            uint32_t budget = alone == 0 ? kTeamSpinBudget : 1u;
+            for (;;) {
+                w0 = __hip_atomic_load(now + tid * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                w1 = __hip_atomic_load(now + tid * 2 + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if ((uint32_t)(w0 >> 32) == tag && (uint32_t)(w1 >> 32) == tag) break;
+                if (--budget == 0) {
+                    alone = 1;
+                    err_words[1] = 1;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+            team_m[tid] = __uint_as_float((uint32_t)w0);
+            team_s[tid] = __uint_as_float((uint32_t)w1);
+        }
+        __syncthreads();
+        float M = -INFINITY;
+        for (uint32_t j = 0; j < G; ++j) M = fmaxf(M, team_m[j]);
+        const bool finite = M > -INFINITY;          // (uniform) a row of -inf has no softmax
+        const float shift = finite ? M : 0.0f;
+        const float bias = -shift * kLog2eHi;
+        float total = 0.0f;
+        for (uint32_t j = 0; j < G; ++j)
+            if (team_m[j] > -INFINITY) total = total + team_s[j] * exp_io<T>(team_m[j] - shift);
+
+        const bool valid = in_range && finite && total > 0.0f;
+        const float lse = shift + logf(total);
+        if (member == 0) ce_fused_row_results(a, grow, valid, lse, target_logit);
+        if ((a.write_grad & 1u) != 0u) {
+            const float scale = a.row_scale != nullptr ? a.row_scale[grow] : a.scale;
+            const float inv = valid ? 1.0f / total : 0.0f;
+            const float mul = valid ? scale : 0.0f;
+            const uint32_t hit = valid ? (uint32_t)target : 0xffffffffu;      // matches no element when the row is ignored
+            if (tid < extra) {
+                float d[1];
+                d[0] = exp_io<T>(xe - shift) * inv;
+                if (e_at == hit) d[0] = d[0] - 1.0f;
+                d[0] = d[0] * mul;
+                VecIO<T, 1>::store(c.base + e_at, d);
+            }
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const uint32_t idx = c.lo + (uint32_t)i * BLOCK + tid;
+                float v[VEC];
+                Raw::unpack(raw[i], v);
+                const uint32_t first = c.head + idx * VEC;
+#pragma unroll
+                for (int k = 0; k < VEC; ++k) v[k] = exp_shifted<T>(v[k], shift, bias);
+                ce_rewrite<VEC>(v, inv, mul, first, hit);
+                if (idx < c.hi) VecIO<T, VEC>::store(c.body + (uint64_t)idx * VEC, v);
+            }
+        }
+        if (!more) break;
+        __syncthreads();                             // (team_m / team_s are written again)
+#pragma unroll
+        for (int i = 0; i < NV; ++i) raw[i] = ahead[i];
+        ex = ex_ahead;
+        row = next;
+        c = c_next;
+    }
+}
+
 // Geometry of the register-resident kernel.  Two workgroups of 512 threads share a CU when a
 // thread's share of the row leaves the kernel within 128 registers (kCeHalfMaxNV vectors: fp32
 // rows up to 40960 classes, bf16 up to 81920): one workgroup's exponentials and stores then
@@ -582,8 +814,41 @@ ce_fused_mem_kernel(T* x, const CeFusedArgs a) {
 // vectors a thread), and beyond that the two-pass kernel.
 constexpr int kCeHalfBlock = 512, kCeHalfMaxNV = 20, kCeFullMaxNV = 20;
 
+// workgroups of a kernel that share a CU, times the CUs: what is on the GPU at once
+uint32_t resident_workgroups(const void* kernel, int block) {
+    int dev = 0, cus = 0, per_cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, block, 0) != hipSuccess || cus < 1 || per_cu < 1) {
+        (void)hipGetLastError();
+        return 0;
+    }
+    return (uint32_t)cus * (uint32_t)per_cu;
+}
+
+// the team kernel for a row of `vectors` aligned vectors at most; false if no geometry fits
+template <typename T, int NV>
+bool ce_fused_team_launch(hipStream_t s, T* x, const CeFusedArgs& a, uint64_t rows, uint32_t vectors, void* scratch,
+                          int* err_words, int* rc) {
+    constexpr int WIDE = WideVec<T>::value;
+    const uint32_t G = (vectors + NV * kTeamBlock - 1) / (NV * kTeamBlock);
+    if (G < 2 || G > kTeamMaxMembers) return false;
+    static const uint32_t resident = resident_workgroups((const void*)ce_fused_team_kernel<T, WIDE, NV>, kTeamBlock);
+    uint32_t teams = resident / G;
+    if (teams > kTeamMaxTeams) teams = kTeamMaxTeams;
+    if (teams > rows) teams = (uint32_t)rows;
+    if (teams == 0) return false;                  // (a team would not be on the GPU all at once)
+    unsigned long long* words = reinterpret_cast<unsigned long long*>(scratch);
+    *rc = launch_fill(s, words, 0u, 4, (uint64_t)teams * kTeamWordsPerTeam * 2);
+    if (*rc != AGRAD_OK) return true;
+    hipLaunchKernelGGL((ce_fused_team_kernel<T, WIDE, NV>), dim3(teams * G), dim3(kTeamBlock), 0, s, x, a, (uint32_t)rows, G,
+                       teams, words, err_words);
+    *rc = check_hip(hipGetLastError(), "fused cross-entropy launch");
+    return true;
+}
+
 template <typename T>
-int ce_fused_typed(hipStream_t s, T* x, const CeFusedArgs& a, uint64_t rows) {
+int ce_fused_typed(hipStream_t s, T* x, const CeFusedArgs& a, uint64_t rows, void* team_scratch, int* err_words) {
     constexpr int WIDE = WideVec<T>::value;
     const dim3 grid((uint32_t)rows);
     // the element-wise head realigns every row to 16 bytes, which needs the element size to divide the misalignment
@@ -600,6 +865,13 @@ int ce_fused_typed(hipStream_t s, T* x, const CeFusedArgs& a, uint64_t rows) {
     AGRAD_CE_REG(12, kCeRowBlock) AGRAD_CE_REG(16, kCeRowBlock) AGRAD_CE_REG(20, kCeRowBlock)
 #undef AGRAD_CE_REG
     static_assert(kCeHalfMaxNV == 20 && kCeFullMaxNV == 20, "the instantiations above");
+    if (team_scratch != nullptr && err_words != nullptr) {
+        // a row that no workgroup can hold: a team of workgroups holds it, a slice each
+        int rc = AGRAD_OK;
+        if (ce_fused_team_launch<T, 4>(s, x, a, rows, vectors, team_scratch, err_words, &rc)) return rc;
+        if (ce_fused_team_launch<T, 8>(s, x, a, rows, vectors, team_scratch, err_words, &rc)) return rc;
+        if (ce_fused_team_launch<T, 16>(s, x, a, rows, vectors, team_scratch, err_words, &rc)) return rc;
+    }
     hipLaunchKernelGGL((ce_fused_mem_kernel<T, WIDE>), grid, dim3(kCeRowBlock), 0, s, x, a);
     return check_hip(hipGetLastError(), "fused cross-entropy launch");
 }
@@ -914,17 +1186,19 @@ int launch_ce_bwd(hipStream_t s, int dtype, const void* logits, const int32_t* l
     return ce_typed<bf16_t>(s, true, (const bf16_t*)logits, labels, nullptr, nullptr, dloss, lse, (bf16_t*)dlogits, rows, V, acc, err_flag);
 }
 
+uint64_t ce_fused_scratch_bytes() { return kTeamScratchBytes; }
+
 int launch_ce_fused(hipStream_t s, int dtype, void* logits, const int32_t* targets, float* row_loss, float* lse,
                     const float* row_scale, uint64_t rows, uint32_t V, uint64_t row_base, float scale,
-                    uint32_t write_grad) {
+                    uint32_t write_grad, void* team_scratch, int* err_words) {
     if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "fused cross-entropy: unknown dtype %d", dtype);
     if (rows == 0 || V == 0) return AGRAD_OK;
     if (logits == nullptr || targets == nullptr) return set_error(AGRAD_EINVAL, "fused cross-entropy: null logits or targets");
     if (write_grad > 1u) return set_error(AGRAD_EINVAL, "fused cross-entropy: write_grad is 0 or 1 (the fp16 gradient store of the reference is not built)");
     if (rows > 0x7fffffffull || row_base + rows > 0xffffffffull) return set_error(AGRAD_EINVAL, "fused cross-entropy: too many rows");
     const CeFusedArgs a{targets, row_loss, lse, row_scale, V, (uint32_t)row_base, scale, write_grad};
-    if (dtype == AGRAD_F32) return ce_fused_typed<float>(s, (float*)logits, a, rows);
-    return ce_fused_typed<bf16_t>(s, (bf16_t*)logits, a, rows);
+    if (dtype == AGRAD_F32) return ce_fused_typed<float>(s, (float*)logits, a, rows, team_scratch, err_words);
+    return ce_fused_typed<bf16_t>(s, (bf16_t*)logits, a, rows, team_scratch, err_words);
 }
 
 int launch_softmax_fwd(hipStream_t s, int dtype, const void* x, void* y, uint64_t rows, uint32_t V) {

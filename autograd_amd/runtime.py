@@ -567,6 +567,12 @@ class Runtime:
         submission, which removes the per-launch cost that dominates chains of small
         ops.  `fn` must already have run once eagerly (kernels load on first use), may
         not read results back, and the replay uses the tensors as they are bound now.
+        Choices the host made while recording are part of the recording: a recorded
+        zero_grad that cleared an embedding table's gradient by rows (row_reset) clears
+        the rows of the ids of the pass before it on every replay, which is right as
+        long as the replays and nothing else write that gradient between them -- write
+        it from the host or from another runtime and the next step must run eagerly
+        (or be recorded again).
         Requires a backend with capture_begin / capture_end (the "hip" device)."""
         if not hasattr(self.backend, "capture_begin"):
             raise RuntimeError(f"device {self.allocator.device!r} cannot record graphs")

@@ -242,6 +242,54 @@ def test_fused_cross_entropy_masks_unaligned_and_loss_only(ctx):
         run_fused(ctx, x, t, capi.F32, write_grad=2)
 
 
+@pytest.mark.parametrize("dtype,rows,V", [("f32", 300, 90001), ("f32", 37, 151936), ("bf16", 150, 170001)])
+def test_fused_cross_entropy_rows_shared_by_a_team_of_workgroups(ctx, dtype, rows, V):
+    """Rows too long for one workgroup's registers (fp32 beyond 81920 classes, bf16 beyond 163840)
+    are held by a team of workgroups, a slice each, which exchange their (max, sum) pairs through
+    memory.  More rows than teams, so that every team takes several rows in turn (the pairs
+    alternate between two sets of slots); an odd row length, so that rows start at every
+    alignment; a slice that is all -inf, a row that is, an ignored and an out-of-range target;
+    per-row scales, a row base, the loss-only form."""
+    rng = np.random.default_rng(490 + V)
+    x = (4.0 * rng.standard_normal((rows, V))).astype(np.float32)
+    if dtype == "bf16":
+        x = from_bf16_bits(to_bf16_bits(x))
+    x[2, :9000] = -np.inf               # one member's whole slice
+    x[3, V // 2:] = -np.inf
+    x[4, :] = -np.inf                   # no finite logit: zero row, loss 0
+    x[6, 5] = 60.0                      # one class takes all the mass
+    t = rng.integers(0, V, rows, dtype=np.int32)
+    t[1] = -1
+    t[5] = V
+    t[7] = V - 1
+    t[8] = 0
+    rs = rng.standard_normal(rows).astype(np.float32)
+    store = to_bf16_bits(x) if dtype == "bf16" else x
+    dt = capi.BF16 if dtype == "bf16" else capi.F32
+    loss, lse, dx = run_fused(ctx, store, t, dt, row_scale=rs, row_base=3)
+    w_loss, w_lse, w_dx = K.cross_entropy_fused(x, t, 1.0, row_scale=rs)
+    if dtype == "bf16":
+        np.testing.assert_allclose(loss[3:], w_loss, rtol=2e-5, atol=2e-5)
+        np.testing.assert_allclose(lse[3:], w_lse, rtol=2e-5, atol=2e-5)
+        assert_bf16_close(from_bf16_bits(dx), w_dx, "dlogits (bf16, team)")
+        dx = from_bf16_bits(dx)
+    else:
+        assert_fp32_close(loss[3:], w_loss, "loss (team)")
+        assert_fp32_close(lse[3:], w_lse, "lse (team)")
+        assert_fp32_close(dx, w_dx, "dlogits (team)")
+    np.testing.assert_array_equal(loss[:3], np.full(3, -7.0, np.float32))
+    assert not dx[1].any() and not dx[4].any() and not dx[5].any() and not np.isnan(dx).any()
+    # twice in a row: the words of the first call's rows are cleared in front of the second
+    loss2, lse2, dx2 = run_fused(ctx, store, t, dt, row_scale=rs, row_base=3)
+    np.testing.assert_array_equal(loss2, loss)
+    np.testing.assert_array_equal(lse2, lse)
+    np.testing.assert_array_equal(from_bf16_bits(dx2) if dtype == "bf16" else dx2, dx)
+    # the loss alone leaves the logits as they were
+    loss3, _, same = run_fused(ctx, store, t, dt, row_base=3, write_grad=0)
+    np.testing.assert_array_equal(same, store)
+    np.testing.assert_array_equal(loss3, loss)
+
+
 def test_fused_cross_entropy_through_the_name_dispatch(ctx):
     """the reference's kernel names and argument order (backend.py:3175-3179)"""
     import ctypes as C
