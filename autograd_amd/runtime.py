@@ -472,7 +472,12 @@ class Runtime:
                     self.backend.init(t)
 
     # -- execution (runtime.py:802-854) ---------------------------------------------
-    def execute(self):
+    def execute(self, wait=True):
+        """zero_grad + forward + backward.  wait=False (backends that run a step as one pass)
+        returns once the step is queued: the stream is in order, so the next step, an optimizer
+        step or a read-back (which waits by itself) may follow at once, and an index error of this
+        step is raised at the next call that waits.  A step's wait leaves the GPU idle while the
+        host queues the first kernels of the next: a tenth of a 0.2 ms step."""
         if self.forward_only:
             self.forward()
             return
@@ -488,7 +493,8 @@ class Runtime:
             self._forward_nodes()
             self.backend.fill(self.loss.grad, self.grad_scale)
             self._backward_nodes()
-            self.backend.end_pass()
+            if wait:
+                self.backend.end_pass()
             return
         if not self.accumulate_parameter_grads:
             self.zero_grad()

@@ -763,6 +763,13 @@ def runtime_path(cfg, per_op_rows, steps=20, ctx=None):
                 rt.execute()
         backend.synchronize()
         execute_us = (time.perf_counter() - t0) * 1e6 / steps
+        # ... and without the wait at the end of each step (one wait after the last)
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            for rt in rts:
+                rt.execute(wait=False)
+        backend.synchronize()
+        nowait_us = (time.perf_counter() - t0) * 1e6 / steps
         def execute_all():
             for rt in rts:
                 rt.execute()
@@ -801,7 +808,7 @@ def runtime_path(cfg, per_op_rows, steps=20, ctx=None):
     c_abi_us += fill_us
     return {"workload": f"configs[{cfg.index}] {cfg.name}: embedding -> norm chain and the activation, forward + backward "
                         f"through Runtime(device='hip'), {len(rts)} graphs",
-            "eager_us": round(eager_us, 1), "execute_us": round(execute_us, 1), "replay_us": round(replay_us, 1), "c_abi_kernels_us": round(c_abi_us, 1),
+            "eager_us": round(eager_us, 1), "execute_us": round(execute_us, 1), "execute_nowait_us": round(nowait_us, 1), "replay_us": round(replay_us, 1), "c_abi_kernels_us": round(c_abi_us, 1),
             "eager_vs_c_abi": round(eager_us / c_abi_us, 3) if c_abi_us else None,
             "replay_vs_c_abi": round(replay_us / c_abi_us, 3) if c_abi_us else None,
             "c_abi_rows": [f"{r['op']} {r['dir']}" for r in kernels] + [f"upstream fills {fill_us:.1f} us"]}

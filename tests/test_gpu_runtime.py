@@ -822,13 +822,13 @@ def _launch_log(rt):
 
 
 @pytest.mark.parametrize("with_wpe", [False, True])
-@pytest.mark.parametrize("protocol", ["execute", "manual", "graph"])
+@pytest.mark.parametrize("protocol", ["execute", "nowait", "manual", "graph"])
 def test_table_gradient_cleared_by_rows_over_steps(with_wpe, protocol):
     """From the second step on zero_grad clears the rows of the last pass's ids in the table's
     gradient instead of filling the table; the gradients are those of a runtime that fills, bit
-    for bit, step after step with new ids -- through execute, through the reference's manual
-    protocol with the ids changed between zero_grad and forward, and through replays of a
-    recorded execute."""
+    for bit, step after step with new ids -- through execute (with and without the wait at the
+    step's end), through the reference's manual protocol with the ids changed between zero_grad
+    and forward, and through replays of a recorded execute."""
     B, T, C, V = 8, 256, 96, 1000
     dev = "hip"
     results = {}
@@ -869,7 +869,7 @@ def test_table_gradient_cleared_by_rows_over_steps(with_wpe, protocol):
                 graph.launch()
             else:
                 rt.backend.copy_from_host(ids, new_ids)
-                rt.execute()
+                rt.execute(wait=(protocol != "nowait"))
             rt.backend.synchronize()
             if graph is None:
                 assert ("embedding_grad_reset" in names) == (row_reset and step > 0), names
