@@ -810,6 +810,7 @@ def runtime_path(cfg, per_op_rows, steps=20, ctx=None):
                         f"through Runtime(device='hip'), {len(rts)} graphs",
             "eager_us": round(eager_us, 1), "execute_us": round(execute_us, 1), "execute_nowait_us": round(nowait_us, 1), "replay_us": round(replay_us, 1), "c_abi_kernels_us": round(c_abi_us, 1),
             "eager_vs_c_abi": round(eager_us / c_abi_us, 3) if c_abi_us else None,
+            "nowait_vs_c_abi": round(nowait_us / c_abi_us, 3) if c_abi_us else None,
             "replay_vs_c_abi": round(replay_us / c_abi_us, 3) if c_abi_us else None,
             "c_abi_rows": [f"{r['op']} {r['dir']}" for r in kernels] + [f"upstream fills {fill_us:.1f} us"]}
 
