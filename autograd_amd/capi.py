@@ -93,6 +93,7 @@ SIGNATURES = {
     "agrad_embedding_sort_workspace_bytes": (_u64, [_u64, _u32]),
     "agrad_gather_forward_sorted": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u32, _u32, _u32, _ptr, _ptr, _u64]),
     "agrad_gather_forward_sorted_kept": (_int, [_ctx, _int, _ptr, _ptr, _ptr, _ptr, _u64, _u32, _u32, _u32, _ptr, _ptr, _u64, _ptr]),
+    "agrad_set_team_wait_polls": (_int, [_ctx, _u32]),
     "agrad_embedding_order": (_int, [_ctx, _ptr, _u64, _u32, _ptr, _ptr, _u64, _ptr, _u64]),
     "agrad_embedding_grad_reset": (_int, [_ctx, _int, _ptr, _u64, _ptr, _u32, _u32]),
     "agrad_unary_forward": (_int, [_ctx, _int, _int, _ptr, _ptr, _u64]),

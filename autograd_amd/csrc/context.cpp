@@ -33,6 +33,7 @@ struct agrad_ctx {
     std::vector<agrad::ColsumJob> pending;
     // counters and (max, sum) pairs of the workgroup teams of the fused cross-entropy (long rows)
     void* ce_scratch = nullptr;
+    uint32_t team_polls = 0;               // 0: the kernels' own bound on a team member's wait
 };
 
 namespace agrad {
@@ -485,7 +486,7 @@ int h_ce_fused(const Call& c) {
     void* row_scale = nullptr;
     if (ROW_SCALED) { if (int rc_ = resolve(c.ctx, c.ids[4], c.offs[4], upto, "row_scale", &row_scale)) return rc_; }
     return launch_ce_fused(c.ctx->stream, (int)c.a[5], logits, (const int32_t*)targets, (float*)row_loss, (float*)lse,
-                           (const float*)row_scale, rows, V, row_base, ROW_SCALED ? 1.0f : f32(c.a[3]), c.a[4], c.ctx->ce_scratch, c.ctx->err_flag);
+                           (const float*)row_scale, rows, V, row_base, ROW_SCALED ? 1.0f : f32(c.a[3]), c.a[4], c.ctx->ce_scratch, c.ctx->err_flag, c.ctx->team_polls);
 }
 // buffers ids, order, sort_workspace, zero_dst | args N, V, ws_lo, ws_hi, zero_lo, zero_hi, present_mask
 int h_emb_order(const Call& c) {
@@ -1124,7 +1125,12 @@ int agrad_cross_entropy_fused(agrad_ctx* ctx, int dtype, void* logits, const int
                               float scale, uint32_t write_grad) {
     CTX_OR_FAIL(ctx)
     return launch_ce_fused(ctx->stream, dtype, logits, targets, row_loss, lse, row_scale, rows, V, row_base, scale, write_grad,
-                           ctx->ce_scratch, ctx->err_flag);
+                           ctx->ce_scratch, ctx->err_flag, ctx->team_polls);
+}
+int agrad_set_team_wait_polls(agrad_ctx* ctx, uint32_t polls) {
+    CTX_OR_FAIL(ctx)
+    ctx->team_polls = polls;
+    return AGRAD_OK;
 }
 int agrad_cross_entropy_backward(agrad_ctx* ctx, int dtype, const void* logits, const int32_t* labels,
                                  const float* dloss, const float* lse, void* dlogits,

@@ -177,7 +177,7 @@ int launch_ce_bwd(hipStream_t s, int dtype, const void* logits, const int32_t* l
 // when given), row_loss / lse [row_base + r] are written; a target outside [0, V) gives a zero row
 int launch_ce_fused(hipStream_t s, int dtype, void* logits, const int32_t* targets, float* row_loss, float* lse,
                     const float* row_scale, uint64_t rows, uint32_t V, uint64_t row_base, float scale,
-                    uint32_t write_grad, void* team_scratch, int* err_words);
+                    uint32_t write_grad, void* team_scratch, int* err_words, uint32_t team_polls = 0);
 // bytes of team_scratch: arrival counters and (max, sum) pairs of the workgroup teams that share long rows
 uint64_t ce_fused_scratch_bytes();
 

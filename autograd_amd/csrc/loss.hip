@@ -618,7 +618,7 @@ ce_fused_mem_kernel(T* x, const CeFusedArgs a) {
 // The grid is what is resident at once (the occupancy the runtime reports, times the
 // CUs), teams are neighbours in it, and a team walks rows team, team + teams, ...: every
 // member of a team is on the GPU while the others wait for it.  The wait is bounded all
-// the same: a member that is not joined within kTeamSpinBudget polls sets the second
+// the same: a member that is not joined within its budget of polls (kTeamSpinBudget unless the host says otherwise) sets the second
 // error word, stops waiting for the rest of the launch and finishes (with wrong numbers;
 // the pass boundary reports the error) -- no wave waits for ever.
 // Tags are the team's row count + 1; a fill in front of the launch clears the words.  The
@@ -642,7 +642,7 @@ struct CeRowExtras {
 template <typename T, int VEC, int NV>
 __global__ void __launch_bounds__(kTeamBlock)
 ce_fused_team_kernel(T* x, const CeFusedArgs a, uint32_t rows, uint32_t G, uint32_t teams,
-                     unsigned long long* words, int* err_words) {
+                     unsigned long long* words, int* err_words, uint32_t spin_budget) {
     constexpr int BLOCK = kTeamBlock;
     __shared__ float lds[BLOCK / kWave];
     __shared__ float team_m[kTeamMaxMembers], team_s[kTeamMaxMembers];
@@ -744,7 +744,7 @@ ce_fused_team_kernel(T* x, const CeFusedArgs a, uint32_t rows, uint32_t G, uint3
         // wait for the team's pairs
         if (tid < G) {
             unsigned long long w0 = 0, w1 = 0;
-            uint32_t budget = alone == 0 ? kTeamSpinBudget : 1u;
+            uint32_t budget = alone == 0 ? spin_budget : 1u;
             for (;;) {
                 w0 = __hip_atomic_load(now + tid * 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 w1 = __hip_atomic_load(now + tid * 2 + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -829,7 +829,7 @@ uint32_t resident_workgroups(const void* kernel, int block) {
 // the team kernel for a row of `vectors` aligned vectors at most; false if no geometry fits
 template <typename T, int NV>
 bool ce_fused_team_launch(hipStream_t s, T* x, const CeFusedArgs& a, uint64_t rows, uint32_t vectors, void* scratch,
-                          int* err_words, int* rc) {
+                          int* err_words, uint32_t polls, int* rc) {
     constexpr int WIDE = WideVec<T>::value;
     const uint32_t G = (vectors + NV * kTeamBlock - 1) / (NV * kTeamBlock);
     if (G < 2 || G > kTeamMaxMembers) return false;
@@ -842,13 +842,14 @@ bool ce_fused_team_launch(hipStream_t s, T* x, const CeFusedArgs& a, uint64_t ro
     *rc = launch_fill(s, words, 0u, 4, (uint64_t)teams * kTeamWordsPerTeam * 2);
     if (*rc != AGRAD_OK) return true;
     hipLaunchKernelGGL((ce_fused_team_kernel<T, WIDE, NV>), dim3(teams * G), dim3(kTeamBlock), 0, s, x, a, (uint32_t)rows, G,
-                       teams, words, err_words);
+                       teams, words, err_words, polls ? polls : kTeamSpinBudget);
     *rc = check_hip(hipGetLastError(), "fused cross-entropy launch");
     return true;
 }
 
 template <typename T>
-int ce_fused_typed(hipStream_t s, T* x, const CeFusedArgs& a, uint64_t rows, void* team_scratch, int* err_words) {
+int ce_fused_typed(hipStream_t s, T* x, const CeFusedArgs& a, uint64_t rows, void* team_scratch, int* err_words,
+                   uint32_t team_polls) {
     constexpr int WIDE = WideVec<T>::value;
     const dim3 grid((uint32_t)rows);
     // the element-wise head realigns every row to 16 bytes, which needs the element size to divide the misalignment
@@ -868,9 +869,9 @@ int ce_fused_typed(hipStream_t s, T* x, const CeFusedArgs& a, uint64_t rows, voi
     if (team_scratch != nullptr && err_words != nullptr) {
         // a row that no workgroup can hold: a team of workgroups holds it, a slice each
         int rc = AGRAD_OK;
-        if (ce_fused_team_launch<T, 4>(s, x, a, rows, vectors, team_scratch, err_words, &rc)) return rc;
-        if (ce_fused_team_launch<T, 8>(s, x, a, rows, vectors, team_scratch, err_words, &rc)) return rc;
-        if (ce_fused_team_launch<T, 16>(s, x, a, rows, vectors, team_scratch, err_words, &rc)) return rc;
+        if (ce_fused_team_launch<T, 4>(s, x, a, rows, vectors, team_scratch, err_words, team_polls, &rc)) return rc;
+        if (ce_fused_team_launch<T, 8>(s, x, a, rows, vectors, team_scratch, err_words, team_polls, &rc)) return rc;
+        if (ce_fused_team_launch<T, 16>(s, x, a, rows, vectors, team_scratch, err_words, team_polls, &rc)) return rc;
     }
     hipLaunchKernelGGL((ce_fused_mem_kernel<T, WIDE>), grid, dim3(kCeRowBlock), 0, s, x, a);
     return check_hip(hipGetLastError(), "fused cross-entropy launch");
@@ -1190,15 +1191,15 @@ uint64_t ce_fused_scratch_bytes() { return kTeamScratchBytes; }
 
 int launch_ce_fused(hipStream_t s, int dtype, void* logits, const int32_t* targets, float* row_loss, float* lse,
                     const float* row_scale, uint64_t rows, uint32_t V, uint64_t row_base, float scale,
-                    uint32_t write_grad, void* team_scratch, int* err_words) {
+                    uint32_t write_grad, void* team_scratch, int* err_words, uint32_t team_polls) {
     if (dtype != AGRAD_F32 && dtype != AGRAD_BF16) return set_error(AGRAD_EINVAL, "fused cross-entropy: unknown dtype %d", dtype);
     if (rows == 0 || V == 0) return AGRAD_OK;
     if (logits == nullptr || targets == nullptr) return set_error(AGRAD_EINVAL, "fused cross-entropy: null logits or targets");
     if (write_grad > 1u) return set_error(AGRAD_EINVAL, "fused cross-entropy: write_grad is 0 or 1 (the fp16 gradient store of the reference is not built)");
     if (rows > 0x7fffffffull || row_base + rows > 0xffffffffull) return set_error(AGRAD_EINVAL, "fused cross-entropy: too many rows");
     const CeFusedArgs a{targets, row_loss, lse, row_scale, V, (uint32_t)row_base, scale, write_grad};
-    if (dtype == AGRAD_F32) return ce_fused_typed<float>(s, (float*)logits, a, rows, team_scratch, err_words);
-    return ce_fused_typed<bf16_t>(s, (bf16_t*)logits, a, rows, team_scratch, err_words);
+    if (dtype == AGRAD_F32) return ce_fused_typed<float>(s, (float*)logits, a, rows, team_scratch, err_words, team_polls);
+    return ce_fused_typed<bf16_t>(s, (bf16_t*)logits, a, rows, team_scratch, err_words, team_polls);
 }
 
 int launch_softmax_fwd(hipStream_t s, int dtype, const void* x, void* y, uint64_t rows, uint32_t V) {

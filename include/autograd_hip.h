@@ -471,13 +471,21 @@ int agrad_cross_entropy_backward(agrad_ctx* ctx, int dtype, const void* logits, 
  * write_grad is 1 -- logits[r, :] is REPLACED by (softmax(x[r, :]) - onehot(targets[g])) * s, with
  * s = row_scale[g] when row_scale is given, else `scale`.  A target outside [0, V) (an ignored position)
  * or a row without a finite logit gives loss 0, lse 0 and a zero row, as in the reference; no index
- * error is raised.  row_loss and lse may be NULL.  The row is read from memory once (a 1024-thread
- * workgroup holds it in registers between the statistics and the rewrite) while it has at most 81920
- * fp32 or 163840 bf16 classes, twice beyond.  The fp16 gradient store of the reference (write_grad
- * bit 1, which feeds its fp16 GEMM) is not built. */
+ * error is raised.  row_loss and lse may be NULL.  The row is read from memory once: a workgroup holds
+ * it in registers between the statistics and the rewrite while it has at most 81920 fp32 or 163840
+ * bf16 classes, and a team of up to 32 workgroups holds a slice each beyond that (the members exchange
+ * one (max, sum) pair per slice through memory that the context owns, and wait for each other a
+ * bounded number of polls: if a team does not assemble in time the call still ends, the gradient it
+ * left is not valid, and the next agrad_end_pass / agrad_synchronize returns AGRAD_EHIP).  Rows that
+ * start at odd addresses or have fewer than 16 bytes of classes are read twice.  The fp16 gradient
+ * store of the reference (write_grad bit 1, which feeds its fp16 GEMM) is not built. */
 int agrad_cross_entropy_fused(agrad_ctx* ctx, int dtype, void* logits, const int32_t* targets,
                               float* row_loss, float* lse, const float* row_scale,
                               uint64_t rows, uint32_t V, uint64_t row_base, float scale, uint32_t write_grad);
+/* How many times a member of such a team looks for the others' pairs before it gives up
+ * (0 = the default, about a second).  No counterpart in the reference; for callers that want a
+ * tighter bound on a launch's worst case, and for the test of the give-up path. */
+int agrad_set_team_wait_polls(agrad_ctx* ctx, uint32_t polls);
 
 /* ---- optimizer step over the parameter slab (the consumer of the gradients above) ---- */
 

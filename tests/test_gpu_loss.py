@@ -290,6 +290,32 @@ def test_fused_cross_entropy_rows_shared_by_a_team_of_workgroups(ctx, dtype, row
     np.testing.assert_array_equal(loss3, loss)
 
 
+def test_fused_cross_entropy_team_wait_is_bounded(ctx):
+    """A member of a team waits for the others a bounded number of polls.  With the bound set to
+    one poll from the host, members give up at once: the launch still ends, the pass boundary
+    says that the gradient is not valid (or, if every pair happened to be there in time, the
+    numbers are right), and with the default bound back the same call is right again."""
+    rng = np.random.default_rng(591)
+    rows, V = 96, 151936
+    x = (4.0 * rng.standard_normal((rows, V))).astype(np.float32)
+    t = rng.integers(0, V, rows, dtype=np.int32)
+    w_loss, w_lse, w_dx = K.cross_entropy_fused(x, t, np.float32(1.0))
+    ctx.call("agrad_set_team_wait_polls", 1)
+    try:
+        try:
+            loss, lse, dx = run_fused(ctx, x, t, capi.F32)
+        except capi.AgradError as e:
+            assert "team" in str(e)
+        else:
+            assert_fp32_close(dx, w_dx, "dlogits (every pair in time)")
+    finally:
+        ctx.call("agrad_set_team_wait_polls", 0)
+    ctx.synchronize()                       # the error has been reported once and is gone
+    loss, lse, dx = run_fused(ctx, x, t, capi.F32)
+    assert_fp32_close(loss, w_loss, "loss")
+    assert_fp32_close(dx, w_dx, "dlogits")
+
+
 def test_fused_cross_entropy_through_the_name_dispatch(ctx):
     """the reference's kernel names and argument order (backend.py:3175-3179)"""
     import ctypes as C
