@@ -606,6 +606,13 @@ class Runtime:
         for slab in self._slabs:
             rel(slab)
         self._slabs = []
+        # the kept-id buffers were among the slabs: nothing may name them any more
+        for node in self.topo:
+            if node.kept_ids is not None:
+                node.kept_ids = None
+                node.kept_fresh = False
+                if len(node.inputs) > 1 and node.inputs[1].grad is not None:
+                    node.inputs[1].grad.dirty_rows = None
 
 
 # -- execution plans (runtime.py:857-947) -------------------------------------------
