@@ -421,6 +421,24 @@ __device__ __forceinline__ void ce_rewrite(float (&v)[VEC], float inv, float mul
     for (int k = 0; k < VEC; ++k) v[k] = v[k] * mul;
 }
 
+// A vector of the gradient to memory.  bf16: the hardware's pair conversion alone -- a NaN
+// comes out as the hardware's quiet NaN instead of with the payload bits the integer rule
+// keeps; a softmax that meets a NaN is NaN throughout, and the two compares a pair cost are
+// a tenth of this kernel's instructions.
+template <typename T, int VEC>
+__device__ __forceinline__ void ce_store_grad(T* p, const float (&v)[VEC]) { VecIO<T, VEC>::store(p, v); }
+template <>
+__device__ __forceinline__ void ce_store_grad<bf16_t, 8>(bf16_t* p, const float (&v)[8]) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const f32x2_hw pair = {v[2 * i], v[2 * i + 1]};
+        w[i] = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2_hw));
+    }
+    u32x4 t; t.x = w[0]; t.y = w[1]; t.z = w[2]; t.w = w[3];
+    __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
+}
+
 // what thread 0 leaves for the row
 __device__ __forceinline__ void ce_fused_row_results(const CeFusedArgs& a, uint32_t grow, bool valid, float lse,
                                                      float target_logit) {
@@ -435,7 +453,11 @@ __global__ void __launch_bounds__(BLOCK)
 ce_fused_reg_kernel(T* x, const CeFusedArgs a) {
     __shared__ float lds[BLOCK / kWave];
     typedef RawVec<T, VEC> Raw;
-    const uint32_t V = a.V, tid = threadIdx.x;
+    const uint32_t V = a.V;
+    // (the thread's number is read anew before the last pass over the registers: what the
+    // compiler would otherwise derive from it once and keep -- an index and an address per
+    // vector -- costs the longest rows their last registers)
+    uint32_t tid = threadIdx.x;
     T* base = x + (uint64_t)blockIdx.x * V;
     const uint32_t grow = a.row_base + blockIdx.x;
     const RowSplit<T, VEC> sp(base, V);
@@ -480,6 +502,7 @@ ce_fused_reg_kernel(T* x, const CeFusedArgs a) {
     for (int i = 0; i < NV; ++i) forget_unpacked(raw[i]);
     const bool finite = m > -INFINITY;          // (uniform) a row of -inf has no softmax
     const float shift = finite ? m : 0.0f;
+    const float bias = -shift * kLog2eHi;
 
     float sum = tid < extra ? exp_io<T>(xe - shift) : 0.0f;
 #pragma unroll
@@ -490,7 +513,7 @@ ce_fused_reg_kernel(T* x, const CeFusedArgs a) {
         float part = 0.0f;
 #pragma unroll
         for (int k = 0; k < VEC; ++k) {
-            v[k] = exp_io<T>(v[k] - shift);
+            v[k] = exp_shifted<T>(v[k], shift, bias);
             part = part + v[k];
         }
         if (idx < sp.nvec) sum = sum + part;
@@ -505,9 +528,11 @@ ce_fused_reg_kernel(T* x, const CeFusedArgs a) {
     ce_fused_row_results(a, grow, valid, lse, target_logit);
     if ((a.write_grad & 1u) == 0u) return;
 
+    asm volatile("" : "+v"(tid));
     const float scale = a.row_scale != nullptr ? a.row_scale[grow] : a.scale;
     const float inv = valid ? 1.0f / sum : 0.0f;
     const float mul = valid ? scale : 0.0f;
+    const float both = inv * mul;
     const uint32_t hit = valid ? (uint32_t)target : 0xffffffffu;          // matches no element when the row is ignored
     if (tid < extra) {
         float d[1];
@@ -522,15 +547,30 @@ ce_fused_reg_kernel(T* x, const CeFusedArgs a) {
         float v[VEC];
         Raw::unpack(raw[i], v);
         const uint32_t first = sp.head + idx * VEC;
+        if constexpr (sizeof(T) == 4) {
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) {
-            float p;
-            if constexpr (sizeof(T) == 4) p = v[k] * inv;
-            else p = exp_io<T>(v[k] - shift) * inv;
-            if (first + k == hit) p = p - 1.0f;
-            v[k] = p * mul;
+            for (int k = 0; k < VEC; ++k) {
+                float p = v[k] * inv;
+                if (first + k == hit) p = p - 1.0f;
+                v[k] = p * mul;
+            }
+        } else {
+            // bf16 rows: nothing per element but the exponential and one product (the kernel
+            // issues vector instructions for most of its run time); the target's element is
+            // put right below, by the thread that stores its vector
+#pragma unroll
+            for (int k = 0; k < VEC; ++k) v[k] = exp_shifted<T>(v[k], shift, bias) * both;
         }
-        if (idx < sp.nvec) VecIO<T, VEC>::store(body + (uint64_t)idx * VEC, v);
+        if (idx < sp.nvec) ce_store_grad<T, VEC>(body + (uint64_t)idx * VEC, v);
+    }
+    if constexpr (sizeof(T) != 4) {
+        // (a later store of the same thread to the same place: in order)
+        const uint32_t hv = (hit - sp.head) / VEC;
+        if (hit >= sp.head && hit < sp.tail_start && tid == hv % BLOCK) {
+            float d[1];
+            d[0] = (exp_io<T>(target_logit - shift) * inv - 1.0f) * mul;
+            VecIO<T, 1>::store(base + hit, d);
+        }
     }
 }
 
