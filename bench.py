@@ -984,8 +984,8 @@ def main():
             if other.index != cfg.index:
                 tables[title(other)] = run_config(ctx, other, args.iters)
                 print(json.dumps({"per_op": title(other), "rows": tables[title(other)]}), flush=True)
-        # the host path beside the C ABI, at a small, a middle and the largest configuration
-        detail["runtime_path"] = [runtime_path(CONFIGS[i], tables[title(CONFIGS[i])], ctx=ctx) for i in (1, 4, 5)]
+        # the host path beside the C ABI, at two small, a middle and the largest configuration
+        detail["runtime_path"] = [runtime_path(CONFIGS[i], tables[title(CONFIGS[i])], ctx=ctx) for i in (1, 2, 4, 5)]
         print(json.dumps({"runtime_path": detail["runtime_path"]}), flush=True)
     ctx.synchronize()
     ctx.close()
