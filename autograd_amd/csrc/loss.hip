@@ -448,8 +448,12 @@ __device__ __forceinline__ void ce_fused_row_results(const CeFusedArgs& a, uint3
     }
 }
 
+// (Sixteen vectors a thread compile to 86 registers, which is five waves a SIMD and two
+// 512-thread workgroups a CU; held to six waves -- 80 registers, 22 of them spilled -- three
+// workgroups share a CU and 16384 rows of 32768 fp32 classes take 780 us instead of 810: a
+// third workgroup in another phase is worth more than the spills cost.)
 template <typename T, int VEC, int NV, int BLOCK>
-__global__ void __launch_bounds__(BLOCK)
+__global__ void __launch_bounds__(BLOCK, (BLOCK == 512 && NV == 16) ? 6 : 1)
 ce_fused_reg_kernel(T* x, const CeFusedArgs a) {
     __shared__ float lds[BLOCK / kWave];
     typedef RawVec<T, VEC> Raw;

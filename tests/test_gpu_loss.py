@@ -203,7 +203,7 @@ def test_fused_cross_entropy_fp32(ctx, rows, V):
     assert not dx[~ok].any()
 
 
-@pytest.mark.parametrize("rows,V", [(5, 64), (4, 1000), (3, 32768), (2, 50257), (2, 128256), (2, 151936)])
+@pytest.mark.parametrize("rows,V", [(5, 64), (4, 1000), (3, 32768), (2, 50257), (3, 65536), (2, 128256), (2, 151936)])
 def test_fused_cross_entropy_bf16(ctx, rows, V):
     rng = np.random.default_rng(290 + V)
     x = from_bf16_bits(to_bf16_bits((4.0 * rng.standard_normal((rows, V))).astype(np.float32)))
